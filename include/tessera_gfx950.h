@@ -1,0 +1,246 @@
+/*
+ * tessera_gfx950.h — C ABI of libtessera_gfx950.so, the MI355X (gfx950 / CDNA4)
+ * execution lane for Tessera's dense ops: GEMM (f16 / bf16 / int8 / fp8-e4m3),
+ * flash-attention forward (causal, GQA, LSE) and the MoE grouped-GEMM block
+ * (routing metadata, dispatch, grouped GEMM, fused SwiGLU, combine).
+ *
+ * Conventions follow the reference's shipped ROCm libraries
+ * (src/compiler/codegen/Tessera_ROCM_Backend/runtime/hip/tessera_rocm_gemm.cpp:843-856,
+ *  .../tessera_rocm_flash_attn.cpp:259-278, python/tessera/runtime.py:1987-1988):
+ *
+ *   - symbols are  tessera_<backend>_<op>_<dtype>  with C linkage;
+ *   - every array is contiguous row-major; dims are C int;
+ *   - the return code is 0 ok / 1 bad shape or argument (checked before the
+ *     device is touched) / 2 no usable gfx950 device / 3 a device operation
+ *     failed;
+ *   - no C++ exception crosses the boundary.
+ *
+ * Two families of entry points:
+ *
+ *   host-pointer  (no suffix)   pointers are HOST memory owned by the caller; the
+ *                               library allocates device memory, copies in, runs,
+ *                               copies out and frees — the reference's convention,
+ *                               a drop-in for its ctypes bindings.
+ *   device-pointer (_dev)       pointers are DEVICE memory, the trailing
+ *                               `void* stream` is a hipStream_t (NULL = default
+ *                               stream); the call enqueues and returns without
+ *                               synchronising.  This is the resident-buffer form
+ *                               used for chained ops and for timing.
+ */
+#ifndef TESSERA_GFX950_H
+#define TESSERA_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TESSERA_GFX950_OK 0
+#define TESSERA_GFX950_BAD_SHAPE 1
+#define TESSERA_GFX950_NO_DEVICE 2
+#define TESSERA_GFX950_DEVICE_FAILED 3
+
+/* ---- lane / device management ------------------------------------------- */
+
+/* ABI version of this header (bumped on incompatible change). */
+int tessera_gfx950_abi_version(void);
+/* 0 iff device 0 exists and is a gfx950 part; else 2.  The cached host probe the
+ * reference's lanes expose through their 16x16x16 zero-GEMM
+ * (python/tessera/runtime.py:1992-2033). */
+int tessera_gfx950_probe(void);
+/* Writes the gcnArchName / marketing name (NUL-terminated, truncated). */
+int tessera_gfx950_device_name(char* buf, int buflen);
+int tessera_gfx950_device_cus(int* cus);
+
+/* Raw device buffers for callers without their own allocator (the Python host
+ * side is ctypes-only, as Tessera never imports PyTorch).  Mirrors the buffer
+ * half of the tsr* runtime ABI (src/runtime/include/tessera/tessera_runtime.h:14-148). */
+int tessera_gfx950_malloc(void** dptr, size_t bytes);
+int tessera_gfx950_free(void* dptr);
+int tessera_gfx950_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int tessera_gfx950_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int tessera_gfx950_memset(void* dst, int value, size_t bytes);
+int tessera_gfx950_synchronize(void);
+
+/* Device-event timer on a stream (NULL = default stream): the timing clock the
+ * reference's bench ABI uses (tessera_rocm_gemm.cpp:567-667). */
+int tessera_gfx950_timer_create(void** timer);
+int tessera_gfx950_timer_start(void* timer, void* stream);
+int tessera_gfx950_timer_stop(void* timer, void* stream);
+/* Blocks until the stop event completed; *ms = elapsed device time. */
+int tessera_gfx950_timer_elapsed_ms(void* timer, float* ms);
+int tessera_gfx950_timer_destroy(void* timer);
+
+/* ---- GEMM  D[M,N] = A[M,K] . B[K,N]  ------------------------------------- */
+
+/* Call-compatible with tessera_rocm_wmma_gemm_{f16,bf16}
+ * (tessera_rocm_gemm.cpp:843-856): 16-bit storage, f32 accumulate, f32 D. */
+int tessera_gfx950_gemm_f16(const void* A, const void* B, void* D, int M, int N, int K);
+int tessera_gfx950_gemm_bf16(const void* A, const void* B, void* D, int M, int N, int K);
+/* Result stored back in the operand storage dtype (RNE) — the ops.gemm rule
+ * for reduced-precision operands (python/tessera/__init__.py:5824-5855). */
+int tessera_gfx950_gemm_f16_f16(const void* A, const void* B, void* D, int M, int N, int K);
+int tessera_gfx950_gemm_bf16_bf16(const void* A, const void* B, void* D, int M, int N, int K);
+/* ops.batched_gemm (python/tessera/__init__.py:250-254): `batch` independent
+ * products, operands densely stacked; f32 D. */
+int tessera_gfx950_batched_gemm_f16(const void* A, const void* B, void* D, int batch, int M, int N, int K);
+int tessera_gfx950_batched_gemm_bf16(const void* A, const void* B, void* D, int batch, int M, int N, int K);
+
+/* int8 x int8 -> int32, bit-exact (the int8 contract of the compiled ROCm
+ * GEMM executor, python/tessera/runtime.py:6500-6513; integer reference
+ * avx512_vnni_gemm_int8.cpp:5-18 / amx_gemm_int8.cpp:34-100). */
+int tessera_gfx950_gemm_i8_i32(const void* A, const void* B, void* C, int M, int N, int K);
+/* W8A8 direct-consume GEMM (python/tessera/compiler/smoothquant.py:115-124):
+ * D[m,n] = f32(acc[m,n]) * row_scale[m] * col_scale[n], two f32 multiplies in
+ * that order.  acc_out (int32[M,N]) may be NULL. */
+int tessera_gfx950_gemm_w8a8_f32(const void* A, const void* B, const float* row_scale,
+                                 const float* col_scale, void* D, void* acc_out,
+                                 int M, int N, int K);
+/* fp8 e4m3fn (OCP) codes, per-tensor scales: D = f32acc(A.B) * scale_a * scale_b
+ * (python/tessera/__init__.py:3340-3374 defines the codes; GEMM over raw fp8
+ * bytes as tessera_nvidia_mma_gemm_e4m3, tessera_nvidia_gemm.cpp:555-556). */
+int tessera_gfx950_gemm_e4m3_bf16(const void* A, const void* B, float scale_a, float scale_b,
+                                  void* D, int M, int N, int K);
+int tessera_gfx950_gemm_e4m3_f32(const void* A, const void* B, float scale_a, float scale_b,
+                                 void* D, int M, int N, int K);
+
+int tessera_gfx950_gemm_f16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream);
+int tessera_gfx950_gemm_bf16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream);
+int tessera_gfx950_gemm_f16_f16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream);
+int tessera_gfx950_gemm_bf16_bf16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream);
+int tessera_gfx950_batched_gemm_f16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K, void* stream);
+int tessera_gfx950_batched_gemm_bf16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K, void* stream);
+int tessera_gfx950_gemm_i8_i32_dev(const void* A, const void* B, void* C, int M, int N, int K, void* stream);
+int tessera_gfx950_gemm_w8a8_f32_dev(const void* A, const void* B, const float* row_scale,
+                                     const float* col_scale, void* D, void* acc_out,
+                                     int M, int N, int K, void* stream);
+int tessera_gfx950_gemm_e4m3_bf16_dev(const void* A, const void* B, float scale_a, float scale_b,
+                                      void* D, int M, int N, int K, void* stream);
+int tessera_gfx950_gemm_e4m3_f32_dev(const void* A, const void* B, float scale_a, float scale_b,
+                                     void* D, int M, int N, int K, void* stream);
+
+/* Kernel-only benchmark with resident, library-owned buffers: warm-up, `iters`
+ * launches between HIP events, cross-checked against wall clock
+ * (tessera_rocm_gemm.cpp:551-667).  *avg_ms = mean per-launch ms. */
+int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_ms);
+/* 0 = device events, 1 = host wall clock, -1 = no measurement yet
+ * (tessera_rocm_bench_last_timer_source, tessera_rocm_gemm.cpp:567-580). */
+int tessera_gfx950_bench_last_timer_source(void);
+
+/* ---- quantisers ------------------------------------------------------------ */
+
+/* ops.quantize_fp8(format="e4m3") (python/tessera/__init__.py:3340-3374; grid as
+ * scalar_fpquant(v,448,3,-6), avx512_fpquant_f32.cpp:28-41): codes[i] = e4m3fn
+ * byte of clip(x[i]/scale, +-448) rounded RNE.  scale <= 0 means "compute
+ * max(amax/448, 1e-12)"; the scale used is written to *scale_out. */
+int tessera_gfx950_quantize_e4m3_f32(const float* x, int64_t n, float scale, void* codes, float* scale_out);
+/* _quantize_int8_per_channel (python/tessera/compiler/smoothquant.py:79-84):
+ * axis=1 -> one scale per row (scales[M]); axis=0 -> one per column (scales[N]). */
+int tessera_gfx950_quantize_i8_f32(const float* x, int M, int N, int axis, void* q, float* scales);
+int tessera_gfx950_quantize_e4m3_f32_dev(const float* x, int64_t n, float scale, void* codes, float* scale_out_dev, void* stream);
+int tessera_gfx950_quantize_i8_f32_dev(const float* x, int M, int N, int axis, void* q, float* scales, void* stream);
+
+/* ---- flash-attention forward ---------------------------------------------- */
+
+/* Call-compatible with tessera_rocm_wmma_flash_attn_{f16,bf16}
+ * (tessera_rocm_flash_attn.cpp:259-278): Q [B,H,Sq,D], K/V [B,H,Sk,D] 16-bit,
+ * O [B,H,Sq,D] f32; causal mask bottom-right aligned (key j visible to query i
+ * iff j <= i + max(Sk-Sq,0)); D % 16 == 0, D <= 256. */
+int tessera_gfx950_flash_attn_f16(const void* Q, const void* K, const void* V, void* O,
+                                  int B, int H, int Sq, int Sk, int D, float scale, int causal);
+int tessera_gfx950_flash_attn_bf16(const void* Q, const void* K, const void* V, void* O,
+                                   int B, int H, int Sq, int Sk, int D, float scale, int causal);
+/* GQA + LSE superset (executor contract python/tessera/runtime.py:7229-7475; GQA
+ * head map and LSE as avx512_flash_attn_f32.cpp:379-422): Q [B,Hq,Sq,D],
+ * K/V [B,Hkv,Sk,D], kv head = hq*Hkv/Hq; O f32 [B,Hq,Sq,D]; LSE f32 [B,Hq,Sq]
+ * (natural log, scaled logits) may be NULL. */
+int tessera_gfx950_flash_attn_gqa_f16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                      int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale, int causal);
+int tessera_gfx950_flash_attn_gqa_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                       int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale, int causal);
+/* out_dtype: 0 = f32 O, 1 = O in the input storage dtype. */
+int tessera_gfx950_flash_attn_gqa_f16_dev(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                          int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                                          int causal, int out_dtype, void* stream);
+int tessera_gfx950_flash_attn_gqa_bf16_dev(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                           int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                                           int causal, int out_dtype, void* stream);
+
+/* ---- MoE -------------------------------------------------------------------- */
+
+/* Router + packing plan in the canonical int32 device ABI
+ * (python/tessera/compiler/moe_transport.py:194-273).  Restates
+ * distributed.moe.route_tokens (python/tessera/distributed/moe.py:119-206) and
+ * the slot sort of nn.functional.moe_layer (python/tessera/nn/functional.py:463-476):
+ * f32 softmax over E experts, top-k descending (ties -> lowest expert id, the
+ * rule of models/moe_routing.py:69-70), weights renormalised when
+ * normalize != 0 and k > 1, first-come capacity drop in token-major order when
+ * capacity > 0, kept slots stable-sorted by expert.
+ * Outputs: token_of_slot/expert_of_slot int32[T*k], combine_weights f32[T*k]
+ * (first *num_slots entries valid), group_sizes int32[E], group_offsets
+ * int32[E+1]. */
+int tessera_gfx950_moe_route_f32(const float* scores, int T, int E, int k, int normalize, int capacity,
+                                 int32_t* token_of_slot, int32_t* expert_of_slot, float* combine_weights,
+                                 int32_t* group_sizes, int32_t* group_offsets, int32_t* num_slots);
+int tessera_gfx950_moe_route_f32_dev(const float* scores, int T, int E, int k, int normalize, int capacity,
+                                     int32_t* token_of_slot, int32_t* expert_of_slot, float* combine_weights,
+                                     int32_t* group_sizes, int32_t* group_offsets, int32_t* num_slots,
+                                     void* stream);
+
+/* tessera.moe_dispatch: x_perm[s,:] = x[token_of_slot[s],:]  (exact gather,
+ * python/tessera/runtime.py:1791-1806).  elem_bytes = 2 (f16/bf16) or 4 (f32). */
+int tessera_gfx950_moe_dispatch(const void* x, const int32_t* token_of_slot, void* x_perm,
+                                int T, int S, int H, int elem_bytes);
+int tessera_gfx950_moe_dispatch_dev(const void* x, const int32_t* token_of_slot, void* x_perm,
+                                    int T, int S, int H, int elem_bytes, void* stream);
+/* tessera.moe_combine: out[t,:] = sum_{s: token_of_slot[s]=t} y_perm[s,:]*w[s],
+ * f32 accumulation in slot order, out f32 [T,N]
+ * (python/tessera/runtime.py:1807-1824; nn/functional.py:487-490). */
+int tessera_gfx950_moe_combine_bf16(const void* y_perm, const int32_t* token_of_slot, const float* weights,
+                                    float* out, int T, int S, int N);
+int tessera_gfx950_moe_combine_f32(const void* y_perm, const int32_t* token_of_slot, const float* weights,
+                                   float* out, int T, int S, int N);
+int tessera_gfx950_moe_combine_bf16_dev(const void* y_perm, const int32_t* token_of_slot, const float* weights,
+                                        float* out, int T, int S, int N, void* stream);
+int tessera_gfx950_moe_combine_f32_dev(const void* y_perm, const int32_t* token_of_slot, const float* weights,
+                                       float* out, int T, int S, int N, void* stream);
+
+/* tessera.grouped_gemm: y[off_e:off_{e+1}] = x[off_e:off_{e+1}] . w[e] in one
+ * launch over device offsets[E+1] (python/tessera/runtime.py:26657-26715;
+ * python/tessera/__init__.py:291-351).  x [S,K], w [E,K,N] bf16; the _bf16 form
+ * stores y in bf16 (storage rule), the _bf16_f32 form keeps f32. */
+int tessera_gfx950_grouped_gemm_bf16(const void* x, const void* w, const int32_t* offsets, void* y,
+                                     int S, int K, int N, int E);
+int tessera_gfx950_grouped_gemm_bf16_f32(const void* x, const void* w, const int32_t* offsets, void* y,
+                                         int S, int K, int N, int E);
+int tessera_gfx950_grouped_gemm_bf16_dev(const void* x, const void* w, const int32_t* offsets, void* y,
+                                         int S, int K, int N, int E, void* stream);
+int tessera_gfx950_grouped_gemm_bf16_f32_dev(const void* x, const void* w, const int32_t* offsets, void* y,
+                                             int S, int K, int N, int E, void* stream);
+/* tessera.grouped_swiglu / ops.moe_swiglu_block
+ * (python/tessera/runtime.py:20353-20368; python/tessera/__init__.py:592-616):
+ * y = gg(bf16(silu(bf16(gg(x,Wg))) * bf16(gg(x,Wu))), Wd), every intermediate
+ * rounded to bf16 like the reference's storage rule.  x [S,K], wg/wu [E,K,F],
+ * wd [E,F,N], y bf16 [S,N].  hidden (bf16 [S,F]) is workspace; NULL makes the
+ * library allocate it (host-pointer form always allocates). */
+int tessera_gfx950_moe_swiglu_block_bf16(const void* x, const void* wg, const void* wu, const void* wd,
+                                         const int32_t* offsets, void* y, int S, int K, int F, int N, int E);
+int tessera_gfx950_moe_swiglu_block_bf16_dev(const void* x, const void* wg, const void* wu, const void* wd,
+                                             const int32_t* offsets, void* y, void* hidden,
+                                             int S, int K, int F, int N, int E, void* stream);
+/* The whole local layer nn.functional.moe_layer
+ * (python/tessera/nn/functional.py:403-490) with the router logits given:
+ * route -> dispatch -> swiglu block -> combine.  out f32 [T,N].  The five
+ * metadata outputs may each be NULL. */
+int tessera_gfx950_moe_layer_bf16(const void* x, const float* router_logits, const void* wg, const void* wu,
+                                  const void* wd, float* out, int T, int H, int F, int N, int E, int k,
+                                  int normalize, int capacity,
+                                  int32_t* token_of_slot, int32_t* expert_of_slot, float* combine_weights,
+                                  int32_t* group_sizes, int32_t* group_offsets);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TESSERA_GFX950_H */

@@ -1,0 +1,139 @@
+// C ABI: dense and batched GEMM, 16-bit storage (f16 / bf16), f32 accumulate.
+#include <chrono>
+#include <cmath>
+#include "../../include/tessera_gfx950.h"
+#include "gemm16_launch.h"
+
+namespace tsr950 {
+namespace {
+
+bool bad_dims(int batch, int M, int N, int K) { return batch <= 0 || M <= 0 || N <= 0 || K <= 0; }
+
+template <class T, int EPI>
+int gemm16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K, hipStream_t s) {
+  if (bad_dims(batch, M, N, K) || !A || !B || !D) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  Gemm16Params p{};
+  p.A = static_cast<const uint16_t*>(A);
+  p.B = static_cast<const uint16_t*>(B);
+  p.D = D;
+  p.M = M; p.N = N; p.K = K;
+  p.lda = K; p.ldb = N; p.ldd = N;
+  p.strideA = (long)M * K; p.strideB = (long)K * N; p.strideD = (long)M * N;
+  p.groups = batch;
+  return launch_gemm16<T, EPI>(p, s);
+}
+
+template <class T, int EPI>
+int gemm16_host(const void* A, const void* B, void* D, int batch, int M, int N, int K) {
+  if (bad_dims(batch, M, N, K) || !A || !B || !D) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t dsz = (EPI == EPI_F32) ? 4 : 2;
+  const size_t a_bytes = (size_t)batch * M * K * 2, b_bytes = (size_t)batch * K * N * 2;
+  const size_t d_bytes = (size_t)batch * M * N * dsz;
+  DeviceScope scope;
+  void* dA = scope.alloc(a_bytes, A);
+  void* dB = scope.alloc(b_bytes, B);
+  void* dD = scope.alloc(d_bytes);
+  if (scope.failed()) return kDeviceFailed;
+  int rc = gemm16_dev<T, EPI>(dA, dB, dD, batch, M, N, K, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  return scope.download(D, dD, d_bytes) ? kOk : kDeviceFailed;
+}
+
+thread_local int g_last_timer_source = -1;
+
+}  // namespace
+}  // namespace tsr950
+
+using namespace tsr950;
+
+extern "C" {
+
+int tessera_gfx950_gemm_f16(const void* A, const void* B, void* D, int M, int N, int K) {
+  return gemm16_host<F16, EPI_F32>(A, B, D, 1, M, N, K);
+}
+int tessera_gfx950_gemm_bf16(const void* A, const void* B, void* D, int M, int N, int K) {
+  return gemm16_host<BF16, EPI_F32>(A, B, D, 1, M, N, K);
+}
+int tessera_gfx950_gemm_f16_f16(const void* A, const void* B, void* D, int M, int N, int K) {
+  return gemm16_host<F16, EPI_STORE16>(A, B, D, 1, M, N, K);
+}
+int tessera_gfx950_gemm_bf16_bf16(const void* A, const void* B, void* D, int M, int N, int K) {
+  return gemm16_host<BF16, EPI_STORE16>(A, B, D, 1, M, N, K);
+}
+int tessera_gfx950_batched_gemm_f16(const void* A, const void* B, void* D, int batch, int M, int N, int K) {
+  return gemm16_host<F16, EPI_F32>(A, B, D, batch, M, N, K);
+}
+int tessera_gfx950_batched_gemm_bf16(const void* A, const void* B, void* D, int batch, int M, int N, int K) {
+  return gemm16_host<BF16, EPI_F32>(A, B, D, batch, M, N, K);
+}
+
+int tessera_gfx950_gemm_f16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream) {
+  return gemm16_dev<F16, EPI_F32>(A, B, D, 1, M, N, K, as_stream(stream));
+}
+int tessera_gfx950_gemm_bf16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream) {
+  return gemm16_dev<BF16, EPI_F32>(A, B, D, 1, M, N, K, as_stream(stream));
+}
+int tessera_gfx950_gemm_f16_f16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream) {
+  return gemm16_dev<F16, EPI_STORE16>(A, B, D, 1, M, N, K, as_stream(stream));
+}
+int tessera_gfx950_gemm_bf16_bf16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream) {
+  return gemm16_dev<BF16, EPI_STORE16>(A, B, D, 1, M, N, K, as_stream(stream));
+}
+int tessera_gfx950_batched_gemm_f16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K,
+                                        void* stream) {
+  return gemm16_dev<F16, EPI_F32>(A, B, D, batch, M, N, K, as_stream(stream));
+}
+int tessera_gfx950_batched_gemm_bf16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K,
+                                         void* stream) {
+  return gemm16_dev<BF16, EPI_F32>(A, B, D, batch, M, N, K, as_stream(stream));
+}
+
+// Kernel-only timing on resident buffers.  The device-event figure is accepted
+// only when it lies within 0.5x..2x of the wall clock around the same launches;
+// otherwise the wall-clock figure is reported and the source says so.
+int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_ms) {
+  g_last_timer_source = -1;
+  if (bad_dims(1, M, N, K) || iters <= 0 || !avg_ms) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  DeviceScope scope;
+  const size_t a_bytes = (size_t)M * K * 2, b_bytes = (size_t)K * N * 2, d_bytes = (size_t)M * N * 2;
+  void* dA = scope.alloc(a_bytes);
+  void* dB = scope.alloc(b_bytes);
+  void* dD = scope.alloc(d_bytes);
+  if (scope.failed()) return kDeviceFailed;
+  // 0x3c00 pattern bytes: finite, non-trivial bf16 values.
+  if (hipMemset(dA, 0x3c, a_bytes) != hipSuccess || hipMemset(dB, 0x3c, b_bytes) != hipSuccess) return kDeviceFailed;
+  for (int w = 0; w < 5; ++w) {
+    int rc = gemm16_dev<BF16, EPI_STORE16>(dA, dB, dD, 1, M, N, K, nullptr);
+    if (rc != kOk) return rc;
+  }
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess) return kDeviceFailed;
+  if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return kDeviceFailed; }
+  int rc = kOk;
+  const auto t0 = std::chrono::steady_clock::now();
+  (void)hipEventRecord(e0, nullptr);
+  for (int it = 0; it < iters && rc == kOk; ++it) rc = gemm16_dev<BF16, EPI_STORE16>(dA, dB, dD, 1, M, N, K, nullptr);
+  (void)hipEventRecord(e1, nullptr);
+  const bool synced = hipEventSynchronize(e1) == hipSuccess;
+  const double wall_ms =
+      std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+  float ev_ms = 0.f;
+  const bool ev_ok = synced && hipEventElapsedTime(&ev_ms, e0, e1) == hipSuccess && std::isfinite(ev_ms) &&
+                     ev_ms > 0.f && ev_ms <= 2.0 * wall_ms && ev_ms >= 0.5 * wall_ms;
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc != kOk) return rc;
+  if (!synced) return kDeviceFailed;
+  g_last_timer_source = ev_ok ? 0 : 1;
+  *avg_ms = (ev_ok ? (double)ev_ms : wall_ms) / iters;
+  return kOk;
+}
+
+int tessera_gfx950_bench_last_timer_source(void) { return g_last_timer_source; }
+
+}  // extern "C"

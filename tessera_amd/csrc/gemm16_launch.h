@@ -1,0 +1,120 @@
+// Host-side tile selection and launch for the 16-bit MFMA GEMM family.
+#pragma once
+#include <mutex>
+#include "gemm16.h"
+#include "host_util.h"
+
+namespace tsr950 {
+
+// Any-shape fallback: one thread per output element, f32 accumulate in k order.
+// Used when rows are not 16-byte aligned (K or N not a multiple of 8), where the
+// vector loads of the MFMA kernel do not apply.
+template <class T, int EPI>
+__global__ void gemm16_generic_kernel(const Gemm16Params p) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  const int m = blockIdx.y * blockDim.y + threadIdx.y;
+  const int z = blockIdx.z;
+  if (m >= p.M || n >= p.N) return;
+  const uint16_t* A = p.A + (long)z * p.strideA + (long)m * p.lda;
+  const uint16_t* B = p.B + (long)z * p.strideB + n;
+  float acc = 0.f;
+  for (int k = 0; k < p.K; ++k) acc += from_storage<T>(A[k]) * from_storage<T>(B[(long)k * p.ldb]);
+  const long o = (long)z * p.strideD + (long)m * p.ldd + n;
+  if constexpr (EPI == EPI_F32) reinterpret_cast<float*>(p.D)[o] = acc;
+  else reinterpret_cast<uint16_t*>(p.D)[o] = to_storage<T>(acc);
+}
+
+// Grouped any-shape fallback: thread per output element, group found by scan.
+template <class T, int EPI>
+__global__ void gemm16_grouped_generic_kernel(const Gemm16Params p) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  const int m = blockIdx.y * blockDim.y + threadIdx.y;
+  if (m >= p.M || n >= p.N) return;
+  int e = 0;
+  while (e + 1 < p.groups && m >= p.offsets[e + 1]) ++e;
+  if (m < p.offsets[e] || m >= p.offsets[e + 1]) return;
+  const uint16_t* A = p.A + (long)m * p.lda;
+  const uint16_t* B = p.B + (long)e * p.strideB + n;
+  float acc = 0.f;
+  for (int k = 0; k < p.K; ++k) acc += from_storage<T>(A[k]) * from_storage<T>(B[(long)k * p.ldb]);
+  if constexpr (EPI == EPI_SWIGLU16) {
+    const uint16_t* B2 = p.B2 + (long)e * p.strideB + n;
+    float up = 0.f;
+    for (int k = 0; k < p.K; ++k) up += from_storage<T>(A[k]) * from_storage<T>(B2[(long)k * p.ldb]);
+    const float gs = from_storage<T>(to_storage<T>(acc));
+    const float us = from_storage<T>(to_storage<T>(up));
+    acc = (gs / (1.0f + __expf(-gs))) * us;
+  }
+  const long o = (long)m * p.ldd + n;
+  if constexpr (EPI == EPI_F32) reinterpret_cast<float*>(p.D)[o] = acc;
+  else reinterpret_cast<uint16_t*>(p.D)[o] = to_storage<T>(acc);
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED>
+int launch_gemm16_tile(Gemm16Params p, hipStream_t s) {
+  using S = Gemm16Smem<BM, BN>;
+  auto kern = gemm16_kernel<T, BM, BN, WM, WN, EPI, GROUPED>;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
+  });
+  if (attr_err != hipSuccess) return kDeviceFailed;
+  constexpr int BN_OUT = (EPI == EPI_SWIGLU16) ? BN / 2 : BN;
+  p.tiles_n = ceil_div(p.N, BN_OUT);
+  dim3 grid;
+  if constexpr (GROUPED) {
+    // every group contributes at most ceil(rows/BM) <= rows/BM + 1 tiles
+    p.tiles_m = p.M / BM + p.groups;
+    grid = dim3(p.tiles_n, p.tiles_m, 1);
+  } else {
+    p.tiles_m = ceil_div(p.M, BM);
+    grid = dim3(p.tiles_m * p.tiles_n, 1, p.groups);
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(WM * WN * 64), S::kBytes, s, p);
+  return launch_status();
+}
+
+// Dense / batched.  p.groups = batch count (>= 1).
+template <class T, int EPI>
+int launch_gemm16(Gemm16Params p, hipStream_t s) {
+  const int dsz = (EPI == EPI_F32) ? 4 : 2;
+  const bool vec = (p.K % 8 == 0) && (p.N % 8 == 0) && (p.lda % 8 == 0) && (p.ldb % 8 == 0) &&
+                   ((p.ldd * dsz) % (dsz * 4) == 0) && (p.strideA % 8 == 0) && (p.strideB % 8 == 0) &&
+                   ((p.strideD * dsz) % 16 == 0) && aligned16(p.A) && aligned16(p.B) && aligned16(p.D);
+  if (!vec) {
+    dim3 block(32, 8), grid(ceil_div(p.N, 32), ceil_div(p.M, 8), p.groups);
+    hipLaunchKernelGGL((gemm16_generic_kernel<T, EPI>), grid, block, 0, s, p);
+    return launch_status();
+  }
+  const long tiles256 = (long)ceil_div(p.M, 256) * ceil_div(p.N, 256) * p.groups;
+  const long tiles128 = (long)ceil_div(p.M, 128) * ceil_div(p.N, 128) * p.groups;
+  if (tiles256 >= 192) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false>(p, s);
+  if (tiles128 >= 192 || (p.M >= 128 && p.N >= 128)) return launch_gemm16_tile<T, 128, 128, 2, 2, EPI, false>(p, s);
+  return launch_gemm16_tile<T, 64, 64, 2, 2, EPI, false>(p, s);
+}
+
+// Grouped.  p.M = total rows S, p.groups = E, p.offsets = device int32[E+1].
+template <class T, int EPI>
+int launch_gemm16_grouped(Gemm16Params p, hipStream_t s) {
+  const int dsz = (EPI == EPI_F32) ? 4 : 2;
+  const bool vec = (p.K % 8 == 0) && (p.N % 8 == 0) && (p.lda % 8 == 0) && (p.ldb % 8 == 0) &&
+                   ((p.ldd * dsz) % (dsz * 4) == 0) && (p.strideB % 8 == 0) && aligned16(p.A) &&
+                   aligned16(p.B) && aligned16(p.D) && (EPI != EPI_SWIGLU16 || aligned16(p.B2));
+  if (!vec) {
+    dim3 block(32, 8), grid(ceil_div(p.N, 32), ceil_div(p.M, 8), 1);
+    hipLaunchKernelGGL((gemm16_grouped_generic_kernel<T, EPI>), grid, block, 0, s, p);
+    return launch_status();
+  }
+  if constexpr (EPI == EPI_SWIGLU16) {
+    return launch_gemm16_tile<T, 256, 256, 4, 1, EPI, true>(p, s);
+  } else {
+    if ((long)p.M >= 64L * p.groups) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true>(p, s);
+    return launch_gemm16_tile<T, 128, 128, 2, 2, EPI, true>(p, s);
+  }
+}
+
+}  // namespace tsr950

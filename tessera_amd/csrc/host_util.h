@@ -1,0 +1,51 @@
+// Host-side helpers shared by the C-ABI translation units: the cached device
+// probe, RAII device buffers for the host-pointer entry points, error mapping.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <vector>
+#include "common.h"
+
+namespace tsr950 {
+
+// 0 when device 0 is a gfx950 part, else kNoDevice.  Cached after the first call.
+int probe_device();
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Owns device allocations made on behalf of a host-pointer entry point and frees
+// them on scope exit, whichever way the call ends.
+class DeviceScope {
+ public:
+  DeviceScope() = default;
+  DeviceScope(const DeviceScope&) = delete;
+  DeviceScope& operator=(const DeviceScope&) = delete;
+  ~DeviceScope() {
+    for (void* p : ptrs_) (void)hipFree(p);
+  }
+  // Allocates `bytes` (at least 16) and, when `src` is given, copies it in.
+  void* alloc(size_t bytes, const void* src = nullptr) {
+    void* d = nullptr;
+    if (hipMalloc(&d, bytes < 16 ? 16 : bytes) != hipSuccess) { failed_ = true; return nullptr; }
+    ptrs_.push_back(d);
+    if (src && bytes && hipMemcpy(d, src, bytes, hipMemcpyHostToDevice) != hipSuccess) failed_ = true;
+    return d;
+  }
+  bool download(void* dst, const void* src, size_t bytes) {
+    if (!bytes) return true;
+    if (hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost) != hipSuccess) { failed_ = true; return false; }
+    return true;
+  }
+  bool failed() const { return failed_; }
+
+ private:
+  std::vector<void*> ptrs_;
+  bool failed_ = false;
+};
+
+inline int finish(hipError_t e) { return e == hipSuccess ? kOk : kDeviceFailed; }
+
+// Launch status of the kernels just enqueued on `s` (does not synchronise).
+inline int launch_status() { return finish(hipGetLastError()); }
+
+}  // namespace tsr950

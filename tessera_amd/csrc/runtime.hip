@@ -1,0 +1,132 @@
+// Device management half of the C ABI: probe, raw buffers, event timers.
+#include <atomic>
+#include <cstring>
+#include <mutex>
+#include "../../include/tessera_gfx950.h"
+#include "host_util.h"
+
+namespace tsr950 {
+
+int probe_device() {
+  static std::once_flag once;
+  static int cached = kNoDevice;
+  std::call_once(once, [] {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) { (void)hipGetLastError(); return; }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, 0) != hipSuccess) { (void)hipGetLastError(); return; }
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) return;
+    if (hipSetDevice(0) != hipSuccess) { (void)hipGetLastError(); return; }
+    cached = kOk;
+  });
+  return cached;
+}
+
+struct Timer {
+  hipEvent_t start, stop;
+};
+
+}  // namespace tsr950
+
+using namespace tsr950;
+
+extern "C" {
+
+int tessera_gfx950_abi_version(void) { return 1; }
+
+int tessera_gfx950_probe(void) { return probe_device(); }
+
+int tessera_gfx950_device_name(char* buf, int buflen) {
+  if (!buf || buflen <= 0) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, 0) != hipSuccess) return kDeviceFailed;
+  char tmp[512];
+  snprintf(tmp, sizeof tmp, "%s (%s)", prop.name, prop.gcnArchName);
+  std::strncpy(buf, tmp, (size_t)buflen - 1);
+  buf[buflen - 1] = 0;
+  return kOk;
+}
+
+int tessera_gfx950_device_cus(int* cus) {
+  if (!cus) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, 0) != hipSuccess) return kDeviceFailed;
+  *cus = prop.multiProcessorCount;
+  return kOk;
+}
+
+int tessera_gfx950_malloc(void** dptr, size_t bytes) {
+  if (!dptr) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  return finish(hipMalloc(dptr, bytes < 16 ? 16 : bytes));
+}
+
+int tessera_gfx950_free(void* dptr) {
+  if (!dptr) return kOk;
+  if (probe_device() != kOk) return kNoDevice;
+  return finish(hipFree(dptr));
+}
+
+int tessera_gfx950_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+  if (bytes && (!dst || !src)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  return bytes ? finish(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice)) : kOk;
+}
+
+int tessera_gfx950_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+  if (bytes && (!dst || !src)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  return bytes ? finish(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost)) : kOk;
+}
+
+int tessera_gfx950_memset(void* dst, int value, size_t bytes) {
+  if (bytes && !dst) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  return bytes ? finish(hipMemset(dst, value, bytes)) : kOk;
+}
+
+int tessera_gfx950_synchronize(void) {
+  if (probe_device() != kOk) return kNoDevice;
+  return finish(hipDeviceSynchronize());
+}
+
+int tessera_gfx950_timer_create(void** timer) {
+  if (!timer) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  Timer* t = new (std::nothrow) Timer;
+  if (!t) return kDeviceFailed;
+  if (hipEventCreate(&t->start) != hipSuccess) { delete t; return kDeviceFailed; }
+  if (hipEventCreate(&t->stop) != hipSuccess) { (void)hipEventDestroy(t->start); delete t; return kDeviceFailed; }
+  *timer = t;
+  return kOk;
+}
+
+int tessera_gfx950_timer_start(void* timer, void* stream) {
+  if (!timer) return kBadShape;
+  return finish(hipEventRecord(static_cast<Timer*>(timer)->start, as_stream(stream)));
+}
+
+int tessera_gfx950_timer_stop(void* timer, void* stream) {
+  if (!timer) return kBadShape;
+  return finish(hipEventRecord(static_cast<Timer*>(timer)->stop, as_stream(stream)));
+}
+
+int tessera_gfx950_timer_elapsed_ms(void* timer, float* ms) {
+  if (!timer || !ms) return kBadShape;
+  Timer* t = static_cast<Timer*>(timer);
+  if (hipEventSynchronize(t->stop) != hipSuccess) return kDeviceFailed;
+  return finish(hipEventElapsedTime(ms, t->start, t->stop));
+}
+
+int tessera_gfx950_timer_destroy(void* timer) {
+  if (!timer) return kOk;
+  Timer* t = static_cast<Timer*>(timer);
+  (void)hipEventDestroy(t->start);
+  (void)hipEventDestroy(t->stop);
+  delete t;
+  return kOk;
+}
+
+}  // extern "C"
