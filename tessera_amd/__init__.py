@@ -1,0 +1,16 @@
+"""tessera_amd — the MI355X (gfx950 / CDNA4) execution lane for Tessera's dense
+ops: GEMM (f16 / bf16 / int8 / fp8), flash-attention forward and the MoE
+grouped-GEMM block, as hand-written HIP kernels behind a C ABI.
+
+Modules
+-------
+``lane``        ctypes binding of ``lib/libtessera_gfx950.so``
+``ops``         the ``tessera.ops`` / ``nn.functional`` surface of the path
+``executors``   the ``runtime.launch`` executor seam (execution-matrix rows)
+``candidates``  the measured-arbiter ``Candidate`` seam
+``tile_table``  Tile-IR op -> gfx950 kernel table
+``build``       in-tree hipcc build of the library
+"""
+from . import bf16, lane  # noqa: F401
+
+__all__ = ["bf16", "lane", "ops", "executors", "candidates", "tile_table", "build"]

@@ -1,0 +1,281 @@
+// C ABI: quantised GEMMs (int8 -> int32, W8A8 with scales, fp8 e4m3 with
+// per-tensor scales) and the quantisers that produce their operands.
+#include <mutex>
+#include "../../include/tessera_gfx950.h"
+#include "gemm8.h"
+#include "host_util.h"
+
+namespace tsr950 {
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <class T, int EPI>
+int gemm8_dev(Gemm8Params p, hipStream_t s) {
+  if (p.M <= 0 || p.N <= 0 || p.K <= 0 || !p.A || !p.B || !p.D) return kBadShape;
+  if (EPI == EPI8_W8A8_F32 && (!p.row_scale || !p.col_scale)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const bool vec = (p.K % 16 == 0) && (p.N % 16 == 0) && aligned16(p.A) && aligned16(p.B) && aligned16(p.D) &&
+                   (!p.acc_out || aligned16(p.acc_out)) && (!p.col_scale || aligned16(p.col_scale));
+  if (!vec) {
+    dim3 block(32, 8), grid(ceil_div(p.N, 32), ceil_div(p.M, 8), 1);
+    hipLaunchKernelGGL((gemm8_generic_kernel<T, EPI>), grid, block, 0, s, p);
+    return launch_status();
+  }
+  auto kern = gemm8_kernel<T, EPI>;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, G8_SMEM);
+  });
+  if (attr_err != hipSuccess) return kDeviceFailed;
+  p.tiles_m = ceil_div(p.M, G8_BM);
+  p.tiles_n = ceil_div(p.N, G8_BN);
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(256), G8_SMEM, s, p);
+  return launch_status();
+}
+
+// ---- quantisers ---------------------------------------------------------------
+
+__device__ __forceinline__ float warp_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Block-wide max of |x| folded into *out with an atomic max on the bit pattern
+// (valid for non-negative floats).
+__global__ void absmax_kernel(const float* x, long n, unsigned* out) {
+  float m = 0.f;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+    m = fmaxf(m, fabsf(x[i]));
+  m = warp_max(m);
+  if ((threadIdx.x & 63) == 0) atomicMax(out, __builtin_bit_cast(unsigned, m));
+}
+
+// f32 (already clipped to +-448) -> e4m3fn byte, round-to-nearest-even with
+// gradual underflow below 2^-6.
+__device__ __forceinline__ uint8_t f32_to_e4m3(float v) {
+  const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+  const uint8_t sign = (uint8_t)((bits >> 24) & 0x80);
+  const uint32_t ab = bits & 0x7fffffffu;
+  if (ab > 0x7f800000u) return (uint8_t)(sign | 0x7f);            // NaN
+  const float a = __builtin_bit_cast(float, ab);
+  uint32_t code;
+  if (a < 0.015625f) {                                            // below the smallest normal 2^-6
+    code = (uint32_t)__builtin_rintf(a * 512.0f);                 // multiples of 2^-9; 8 carries into 0x08
+  } else {
+    const uint32_t r = (ab + 0x7ffffu + ((ab >> 20) & 1u)) >> 20; // (biased exp << 3) | 3-bit mantissa
+    code = r - (120u << 3);
+    if (code > 0x7eu) code = 0x7eu;                               // saturate at 448
+  }
+  return (uint8_t)(sign | code);
+}
+
+// scale_in > 0: use it; else scale = max(amax / 448, 1e-12) from *amax_bits.
+__global__ void quantize_e4m3_kernel(const float* x, long n, float scale_in, const unsigned* amax_bits,
+                                     uint8_t* codes, float* scale_out) {
+  float scale = scale_in;
+  if (!(scale_in > 0.f)) {
+    const float amax = __builtin_bit_cast(float, *amax_bits);
+    scale = fmaxf(__fdiv_rn(amax, 448.0f), 1e-12f);
+  }
+  if (scale_out && blockIdx.x == 0 && threadIdx.x == 0) *scale_out = scale;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    float t = __fdiv_rn(x[i], scale);
+    t = fminf(fmaxf(t, -448.0f), 448.0f);
+    codes[i] = f32_to_e4m3(t);
+  }
+}
+
+// One workgroup per row: absmax, scale = max(absmax, 1e-12) / 127, q = rint(x / scale).
+__global__ void quantize_i8_rows_kernel(const float* x, int M, int N, int8_t* q, float* scales) {
+  __shared__ float red[4];
+  const int m = blockIdx.x;
+  const float* row = x + (long)m * N;
+  float mx = 0.f;
+  for (int n = threadIdx.x; n < N; n += blockDim.x) mx = fmaxf(mx, fabsf(row[n]));
+  mx = warp_max(mx);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float scale = __fdiv_rn(fmaxf(mx, 1e-12f), 127.0f);
+  if (threadIdx.x == 0) scales[m] = scale;
+  for (int n = threadIdx.x; n < N; n += blockDim.x) {
+    float t = __builtin_rintf(__fdiv_rn(row[n], scale));
+    t = fminf(fmaxf(t, -127.f), 127.f);
+    q[(long)m * N + n] = (int8_t)t;
+  }
+}
+
+// Column scales: each thread owns one column and walks the rows (coalesced
+// across the wavefront); two passes over x.
+__global__ void quantize_i8_cols_kernel(const float* x, int M, int N, int8_t* q, float* scales) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= N) return;
+  float mx = 0.f;
+  for (int m = 0; m < M; ++m) mx = fmaxf(mx, fabsf(x[(long)m * N + n]));
+  const float scale = __fdiv_rn(fmaxf(mx, 1e-12f), 127.0f);
+  scales[n] = scale;
+  for (int m = 0; m < M; ++m) {
+    float t = __builtin_rintf(__fdiv_rn(x[(long)m * N + n], scale));
+    t = fminf(fmaxf(t, -127.f), 127.f);
+    q[(long)m * N + n] = (int8_t)t;
+  }
+}
+
+int quantize_e4m3_dev(const float* x, int64_t n, float scale, void* codes, float* scale_out_dev, hipStream_t s) {
+  if (n <= 0 || !x || !codes) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const int blocks = (int)std::min<int64_t>((n + 255) / 256, 4096);
+  unsigned* amax = nullptr;
+  if (!(scale > 0.f)) {
+    if (hipMallocAsync(reinterpret_cast<void**>(&amax), sizeof(unsigned), s) != hipSuccess) return kDeviceFailed;
+    if (hipMemsetAsync(amax, 0, sizeof(unsigned), s) != hipSuccess) return kDeviceFailed;
+    hipLaunchKernelGGL(absmax_kernel, dim3(blocks), dim3(256), 0, s, x, (long)n, amax);
+  }
+  hipLaunchKernelGGL(quantize_e4m3_kernel, dim3(blocks), dim3(256), 0, s, x, (long)n, scale, amax,
+                     static_cast<uint8_t*>(codes), scale_out_dev);
+  int rc = launch_status();
+  if (amax && hipFreeAsync(amax, s) != hipSuccess) rc = kDeviceFailed;
+  return rc;
+}
+
+int quantize_i8_dev(const float* x, int M, int N, int axis, void* q, float* scales, hipStream_t s) {
+  if (M <= 0 || N <= 0 || !x || !q || !scales || (axis != 0 && axis != 1)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  if (axis == 1)
+    hipLaunchKernelGGL(quantize_i8_rows_kernel, dim3(M), dim3(256), 0, s, x, M, N, static_cast<int8_t*>(q), scales);
+  else
+    hipLaunchKernelGGL(quantize_i8_cols_kernel, dim3(ceil_div(N, 64)), dim3(64), 0, s, x, M, N,
+                       static_cast<int8_t*>(q), scales);
+  return launch_status();
+}
+
+Gemm8Params make_params(const void* A, const void* B, void* D, int M, int N, int K) {
+  Gemm8Params p{};
+  p.A = static_cast<const uint8_t*>(A);
+  p.B = static_cast<const uint8_t*>(B);
+  p.D = D;
+  p.M = M; p.N = N; p.K = K;
+  p.scale_a = p.scale_b = 1.f;
+  return p;
+}
+
+template <class T, int EPI>
+int gemm8_host(const void* A, const void* B, const float* rs, const float* cs, float sa, float sb, void* D,
+               void* acc_out, int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0 || !A || !B || !D) return kBadShape;
+  if (EPI == EPI8_W8A8_F32 && (!rs || !cs)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t dsz = (EPI == EPI8_SCALED_BF16) ? 2 : 4;
+  const size_t d_bytes = (size_t)M * N * dsz, acc_bytes = (size_t)M * N * 4;
+  DeviceScope scope;
+  Gemm8Params p = make_params(scope.alloc((size_t)M * K, A), scope.alloc((size_t)K * N, B), scope.alloc(d_bytes),
+                              M, N, K);
+  if (EPI == EPI8_W8A8_F32) {
+    p.row_scale = static_cast<const float*>(scope.alloc((size_t)M * 4, rs));
+    p.col_scale = static_cast<const float*>(scope.alloc((size_t)N * 4, cs));
+    if (acc_out) p.acc_out = static_cast<int32_t*>(scope.alloc(acc_bytes));
+  }
+  p.scale_a = sa; p.scale_b = sb;
+  if (scope.failed()) return kDeviceFailed;
+  int rc = gemm8_dev<T, EPI>(p, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  if (!scope.download(D, p.D, d_bytes)) return kDeviceFailed;
+  if (p.acc_out && !scope.download(acc_out, p.acc_out, acc_bytes)) return kDeviceFailed;
+  return kOk;
+}
+
+}  // namespace
+}  // namespace tsr950
+
+using namespace tsr950;
+
+extern "C" {
+
+int tessera_gfx950_gemm_i8_i32(const void* A, const void* B, void* C, int M, int N, int K) {
+  return gemm8_host<I8, EPI8_I32>(A, B, nullptr, nullptr, 1.f, 1.f, C, nullptr, M, N, K);
+}
+int tessera_gfx950_gemm_w8a8_f32(const void* A, const void* B, const float* row_scale, const float* col_scale,
+                                 void* D, void* acc_out, int M, int N, int K) {
+  return gemm8_host<I8, EPI8_W8A8_F32>(A, B, row_scale, col_scale, 1.f, 1.f, D, acc_out, M, N, K);
+}
+int tessera_gfx950_gemm_e4m3_bf16(const void* A, const void* B, float scale_a, float scale_b, void* D, int M,
+                                  int N, int K) {
+  return gemm8_host<FP8, EPI8_SCALED_BF16>(A, B, nullptr, nullptr, scale_a, scale_b, D, nullptr, M, N, K);
+}
+int tessera_gfx950_gemm_e4m3_f32(const void* A, const void* B, float scale_a, float scale_b, void* D, int M,
+                                 int N, int K) {
+  return gemm8_host<FP8, EPI8_SCALED_F32>(A, B, nullptr, nullptr, scale_a, scale_b, D, nullptr, M, N, K);
+}
+
+int tessera_gfx950_gemm_i8_i32_dev(const void* A, const void* B, void* C, int M, int N, int K, void* stream) {
+  return gemm8_dev<I8, EPI8_I32>(make_params(A, B, C, M, N, K), as_stream(stream));
+}
+int tessera_gfx950_gemm_w8a8_f32_dev(const void* A, const void* B, const float* row_scale,
+                                     const float* col_scale, void* D, void* acc_out, int M, int N, int K,
+                                     void* stream) {
+  Gemm8Params p = make_params(A, B, D, M, N, K);
+  p.row_scale = row_scale;
+  p.col_scale = col_scale;
+  p.acc_out = static_cast<int32_t*>(acc_out);
+  return gemm8_dev<I8, EPI8_W8A8_F32>(p, as_stream(stream));
+}
+int tessera_gfx950_gemm_e4m3_bf16_dev(const void* A, const void* B, float scale_a, float scale_b, void* D,
+                                      int M, int N, int K, void* stream) {
+  Gemm8Params p = make_params(A, B, D, M, N, K);
+  p.scale_a = scale_a; p.scale_b = scale_b;
+  return gemm8_dev<FP8, EPI8_SCALED_BF16>(p, as_stream(stream));
+}
+int tessera_gfx950_gemm_e4m3_f32_dev(const void* A, const void* B, float scale_a, float scale_b, void* D,
+                                     int M, int N, int K, void* stream) {
+  Gemm8Params p = make_params(A, B, D, M, N, K);
+  p.scale_a = scale_a; p.scale_b = scale_b;
+  return gemm8_dev<FP8, EPI8_SCALED_F32>(p, as_stream(stream));
+}
+
+int tessera_gfx950_quantize_e4m3_f32_dev(const float* x, int64_t n, float scale, void* codes,
+                                         float* scale_out_dev, void* stream) {
+  return quantize_e4m3_dev(x, n, scale, codes, scale_out_dev, as_stream(stream));
+}
+int tessera_gfx950_quantize_i8_f32_dev(const float* x, int M, int N, int axis, void* q, float* scales,
+                                       void* stream) {
+  return quantize_i8_dev(x, M, N, axis, q, scales, as_stream(stream));
+}
+
+int tessera_gfx950_quantize_e4m3_f32(const float* x, int64_t n, float scale, void* codes, float* scale_out) {
+  if (n <= 0 || !x || !codes) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  DeviceScope scope;
+  float* dx = static_cast<float*>(scope.alloc((size_t)n * 4, x));
+  void* dc = scope.alloc((size_t)n);
+  float* ds = static_cast<float*>(scope.alloc(4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = quantize_e4m3_dev(dx, n, scale, dc, ds, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  if (!scope.download(codes, dc, (size_t)n)) return kDeviceFailed;
+  if (scale_out && !scope.download(scale_out, ds, 4)) return kDeviceFailed;
+  return kOk;
+}
+
+int tessera_gfx950_quantize_i8_f32(const float* x, int M, int N, int axis, void* q, float* scales) {
+  if (M <= 0 || N <= 0 || !x || !q || !scales || (axis != 0 && axis != 1)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t n = (size_t)M * N, ns = (size_t)(axis == 1 ? M : N);
+  DeviceScope scope;
+  float* dx = static_cast<float*>(scope.alloc(n * 4, x));
+  void* dq = scope.alloc(n);
+  float* ds = static_cast<float*>(scope.alloc(ns * 4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = quantize_i8_dev(dx, M, N, axis, dq, ds, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  if (!scope.download(q, dq, n) || !scope.download(scales, ds, ns * 4)) return kDeviceFailed;
+  return kOk;
+}
+
+}  // extern "C"

@@ -1,0 +1,626 @@
+// C ABI: MoE routing metadata, dispatch / combine, grouped GEMM and the fused
+// SwiGLU expert block.
+//
+// Routing follows distributed.moe.route_tokens + the slot sort of
+// nn.functional.moe_layer, expressed directly in the int32 transport ABI
+// (token_of_slot, expert_of_slot, combine_weights, group_sizes, group_offsets):
+//
+//   topk_kernel    one wavefront per token: f32 max-subtracted softmax over the
+//                  experts, k rounds of (max value, lowest index) selection,
+//                  optional renormalisation of the k weights.
+//   count_kernel   per-chunk histogram of the selected experts.
+//   scan_kernel    per-expert exclusive scan over chunks (= each chunk's first
+//                  rank inside every expert, in token-major order), capacity
+//                  clamp, group sizes and offsets.
+//   place_kernel   every kept slot lands at offsets[e] + (its token-major rank
+//                  inside expert e): a stable sort by expert without sorting.
+// A slot is kept iff its rank inside its expert is below the capacity, which is
+// the reference's first-come rule (earlier tokens win, slot-minor inside a token).
+#include <algorithm>
+#include <mutex>
+#include "../../include/tessera_gfx950.h"
+#include "gemm16_launch.h"
+#include "host_util.h"
+
+namespace tsr950 {
+namespace {
+
+constexpr int kSlotsPerChunk = 512;   // slots handled by one wavefront in count/place
+constexpr int kMaxExperts = 1024;
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// One wavefront per token.  Lane l owns experts l, l+64, ... (EPL of them).
+template <int EPL>
+__global__ __launch_bounds__(256) void topk_kernel(const float* scores, int T, int E, int k, int normalize,
+                                                   int32_t* expert_ids, float* weights) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  const float* row = scores + (long)t * E;
+  float s[EPL], pr[EPL];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + 64 * i;
+    s[i] = e < E ? row[e] : -INFINITY;
+    mx = fmaxf(mx, s[i]);
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + 64 * i;
+    pr[i] = e < E ? expf(s[i] - mx) : 0.f;
+    sum += pr[i];
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + 64 * i;
+    pr[i] = e < E ? __fdiv_rn(pr[i], sum) : -1.f;    // -1 never wins a selection
+  }
+  float wsum = 0.f;
+  float my_w = 0.f;       // lane j keeps the j-th selected weight
+  int my_e = -1;
+  for (int j = 0; j < k; ++j) {
+    // best (value desc, index asc) among this lane's experts, then across lanes
+    float bv = -2.f;
+    int be = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      const int e = lane + 64 * i;
+      if (pr[i] > bv) { bv = pr[i]; be = e; }      // ascending e inside a lane: first max wins
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oe = __shfl_xor(be, o, 64);
+      if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
+    }
+#pragma unroll
+    for (int i = 0; i < EPL; ++i)
+      if (lane + 64 * i == be) pr[i] = -1.f;       // remove the winner
+    if (lane == (j & 63)) { my_w = bv; my_e = be; }
+    wsum += bv;
+    if ((j & 63) == 63 || j == k - 1) {
+      // flush up to 64 selections (k <= 64 in practice; the loop form keeps it general)
+      const int base = j - (j & 63);
+      if (lane <= (j & 63)) {
+        expert_ids[(long)t * k + base + lane] = my_e;
+        weights[(long)t * k + base + lane] = my_w;
+      }
+    }
+  }
+  if (normalize && k > 1) {
+    const float d = wsum > 0.f ? wsum : 1.f;
+    for (int j = lane; j < k; j += 64) weights[(long)t * k + j] = __fdiv_rn(weights[(long)t * k + j], d);
+  }
+}
+
+__global__ __launch_bounds__(64) void count_kernel(const int32_t* expert_ids, int S, int E, int32_t* chunk_counts) {
+  __shared__ int hist[kMaxExperts];
+  for (int e = threadIdx.x; e < E; e += 64) hist[e] = 0;
+  __syncthreads();
+  const int base = blockIdx.x * kSlotsPerChunk;
+  for (int i = threadIdx.x; i < kSlotsPerChunk; i += 64) {
+    const int s = base + i;
+    if (s < S) atomicAdd(&hist[expert_ids[s]], 1);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 64) chunk_counts[(long)blockIdx.x * E + e] = hist[e];
+}
+
+// One workgroup.  chunk_counts[c][e] becomes the rank of chunk c's first slot in
+// expert e; group sizes (capacity clamped) and offsets follow.
+__global__ __launch_bounds__(256) void scan_kernel(int32_t* chunk_counts, int chunks, int E, int capacity,
+                                                   int32_t* group_sizes, int32_t* group_offsets,
+                                                   int32_t* num_slots) {
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    int run = 0;
+    for (int c = 0; c < chunks; ++c) {
+      const int v = chunk_counts[(long)c * E + e];
+      chunk_counts[(long)c * E + e] = run;
+      run += v;
+    }
+    group_sizes[e] = (capacity > 0 && run > capacity) ? capacity : run;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int off = 0;
+    for (int e = 0; e < E; ++e) {
+      group_offsets[e] = off;
+      off += group_sizes[e];
+    }
+    group_offsets[E] = off;
+    if (num_slots) *num_slots = off;
+  }
+}
+
+__global__ __launch_bounds__(64) void place_kernel(const int32_t* expert_ids, const float* weights, int S, int E,
+                                                   int k, int capacity, const int32_t* chunk_base,
+                                                   const int32_t* group_offsets, int32_t* token_of_slot,
+                                                   int32_t* expert_of_slot, float* combine_weights) {
+  __shared__ int cursor[kMaxExperts];
+  const int lane = threadIdx.x;
+  for (int e = lane; e < E; e += 64) cursor[e] = chunk_base[(long)blockIdx.x * E + e];
+  __syncthreads();
+  const int base = blockIdx.x * kSlotsPerChunk;
+  for (int i0 = 0; i0 < kSlotsPerChunk; i0 += 64) {
+    const int s = base + i0 + lane;
+    const bool valid = s < S;
+    const int e = valid ? expert_ids[s] : -1;
+    int rank = 0;
+    // Rank inside the expert in slot order: lanes sharing an expert are found one
+    // expert at a time; lower lanes are earlier slots.
+    unsigned long long todo = __ballot(valid);
+    while (todo) {
+      const int leader = __ffsll((long long)todo) - 1;
+      const int e0 = __shfl(e, leader, 64);
+      const unsigned long long same = __ballot(valid && e == e0);
+      if (valid && e == e0) rank = cursor[e0] + __popcll(same & ((1ull << lane) - 1ull));
+      __syncthreads();
+      if (lane == leader) cursor[e0] += __popcll(same);
+      __syncthreads();
+      todo &= ~same;
+    }
+    if (valid && (capacity <= 0 || rank < capacity)) {
+      const int pos = group_offsets[e] + rank;
+      token_of_slot[pos] = s / k;
+      expert_of_slot[pos] = e;
+      combine_weights[pos] = weights[s];
+    }
+  }
+}
+
+int route_dev(const float* scores, int T, int E, int k, int normalize, int capacity, int32_t* token_of_slot,
+              int32_t* expert_of_slot, float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
+              int32_t* num_slots, hipStream_t s) {
+  if (T <= 0 || E <= 0 || k <= 0 || k > E || E > kMaxExperts || !scores || !token_of_slot || !expert_of_slot ||
+      !combine_weights || !group_sizes || !group_offsets)
+    return kBadShape;
+  if ((long)T * k > 0x7fffffffL) return kBadShape;     // int32 device ABI
+  if (probe_device() != kOk) return kNoDevice;
+  const int S = T * k;
+  const int chunks = ceil_div(S, kSlotsPerChunk);
+  int32_t* ids = nullptr;
+  float* w = nullptr;
+  int32_t* counts = nullptr;
+  if (hipMallocAsync(reinterpret_cast<void**>(&ids), (size_t)S * 4, s) != hipSuccess) return kDeviceFailed;
+  if (hipMallocAsync(reinterpret_cast<void**>(&w), (size_t)S * 4, s) != hipSuccess) return kDeviceFailed;
+  if (hipMallocAsync(reinterpret_cast<void**>(&counts), (size_t)chunks * E * 4, s) != hipSuccess) return kDeviceFailed;
+  const dim3 tgrid(ceil_div(T, 4));
+  const int epl = ceil_div(E, 64);
+  if (epl <= 1) hipLaunchKernelGGL((topk_kernel<1>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, ids, w);
+  else if (epl <= 2) hipLaunchKernelGGL((topk_kernel<2>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, ids, w);
+  else if (epl <= 4) hipLaunchKernelGGL((topk_kernel<4>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, ids, w);
+  else hipLaunchKernelGGL((topk_kernel<16>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, ids, w);
+  hipLaunchKernelGGL(count_kernel, dim3(chunks), dim3(64), 0, s, ids, S, E, counts);
+  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(256), 0, s, counts, chunks, E, capacity, group_sizes, group_offsets,
+                     num_slots);
+  hipLaunchKernelGGL(place_kernel, dim3(chunks), dim3(64), 0, s, ids, w, S, E, k, capacity, counts, group_offsets,
+                     token_of_slot, expert_of_slot, combine_weights);
+  int rc = launch_status();
+  if (hipFreeAsync(ids, s) != hipSuccess || hipFreeAsync(w, s) != hipSuccess || hipFreeAsync(counts, s) != hipSuccess)
+    rc = kDeviceFailed;
+  return rc;
+}
+
+// ---- dispatch: exact row gather, 16 bytes per lane -------------------------------
+__global__ __launch_bounds__(256) void dispatch_kernel(const char* x, const int32_t* token_of_slot, char* x_perm,
+                                                       int T, int S, long row_bytes) {
+  const int s = blockIdx.x;
+  const int t = token_of_slot[s];
+  if (t < 0 || t >= T) return;
+  const char* src = x + (long)t * row_bytes;
+  char* dst = x_perm + (long)s * row_bytes;
+  if ((row_bytes & 15) == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(x_perm)) & 15) == 0) {
+    for (long o = (long)threadIdx.x * 16; o < row_bytes; o += 256 * 16)
+      *reinterpret_cast<uint4*>(dst + o) = *reinterpret_cast<const uint4*>(src + o);
+  } else {
+    for (long o = threadIdx.x; o < row_bytes; o += 256) dst[o] = src[o];
+  }
+}
+
+// ---- combine ------------------------------------------------------------------------
+// The slots of a token are found by sorting slot ids by token (count, scan,
+// fill); each token then adds its slots in ascending slot order — the order of
+// the reference's unbuffered scatter-add — so the f32 result is reproducible.
+__global__ void combine_count_kernel(const int32_t* token_of_slot, int S, int T, int32_t* cnt) {
+  const int s = blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= S) return;
+  const int t = token_of_slot[s];
+  if (t >= 0 && t < T) atomicAdd(&cnt[t], 1);
+}
+// Single workgroup exclusive scan of cnt[T] -> off[T+1]; cnt is zeroed for reuse as cursors.
+__global__ __launch_bounds__(1024) void combine_scan_kernel(int32_t* cnt, int T, int32_t* off) {
+  __shared__ int part[1024];
+  const int per = (T + 1023) / 1024;
+  const int lo = threadIdx.x * per, hi = min(lo + per, T);
+  int sum = 0;
+  for (int i = lo; i < hi; ++i) sum += cnt[i];
+  part[threadIdx.x] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int i = 0; i < 1024; ++i) { const int v = part[i]; part[i] = run; run += v; }
+    off[T] = run;
+  }
+  __syncthreads();
+  int run = part[threadIdx.x];
+  for (int i = lo; i < hi; ++i) { const int v = cnt[i]; off[i] = run; run += v; cnt[i] = 0; }
+}
+__global__ void combine_fill_kernel(const int32_t* token_of_slot, int S, int T, const int32_t* off, int32_t* cursor,
+                                    int32_t* list) {
+  const int s = blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= S) return;
+  const int t = token_of_slot[s];
+  if (t >= 0 && t < T) list[off[t] + atomicAdd(&cursor[t], 1)] = s;
+}
+// acc + (v * w) with the product rounded to f32 before the add — the reference
+// scales the rows first and scatter-adds afterwards, so no fused multiply-add.
+__device__ __forceinline__ float add_rounded_product(float acc, float v, float w) {
+#pragma clang fp contract(off)
+  const float prod = v * w;
+  return acc + prod;
+}
+
+template <class YT>
+__global__ __launch_bounds__(256) void combine_kernel(const YT* y, const float* w, const int32_t* off,
+                                                      const int32_t* list, float* out, int N) {
+  constexpr int kMaxSorted = 256;
+  __shared__ int sorted[kMaxSorted];
+  __shared__ float sw[kMaxSorted];
+  const int t = blockIdx.x;
+  const int lo = off[t], hi = off[t + 1];
+  const int len = hi - lo;
+  const bool small = len <= kMaxSorted;
+  if (small) {
+    // rank of every slot id inside the token's list -> ascending order in LDS
+    for (int j = threadIdx.x; j < len; j += 256) {
+      const int sl = list[lo + j];
+      int rank = 0;
+      for (int i = 0; i < len; ++i) rank += list[lo + i] < sl;
+      sorted[rank] = sl;
+      sw[rank] = w[sl];
+    }
+    __syncthreads();
+  }
+  for (int n = threadIdx.x; n < N; n += 256) {
+    float acc = 0.f;
+    int prev = -1;
+    for (int i = 0; i < len; ++i) {
+      int slot;
+      float wt;
+      if (small) {
+        slot = sorted[i];
+        wt = sw[i];
+      } else {
+        // next slot in ascending order: smallest id greater than the previous one
+        int best = 0x7fffffff;
+        for (int j = lo; j < hi; ++j) {
+          const int sl = list[j];
+          if (sl > prev && sl < best) best = sl;
+        }
+        prev = slot = best;
+        wt = w[best];
+      }
+      float v;
+      if constexpr (sizeof(YT) == 2) v = bf16_bits_to_f32(y[(long)slot * N + n]);
+      else v = y[(long)slot * N + n];
+      acc = add_rounded_product(acc, v, wt);
+    }
+    out[(long)t * N + n] = acc;
+  }
+}
+
+template <class YT>
+int combine_dev(const void* y, const int32_t* token_of_slot, const float* w, float* out, int T, int S, int N,
+                hipStream_t s) {
+  if (T <= 0 || S < 0 || N <= 0 || !out || (S > 0 && (!y || !token_of_slot || !w))) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  int32_t* cnt = nullptr;
+  int32_t* off = nullptr;
+  int32_t* list = nullptr;
+  if (hipMallocAsync(reinterpret_cast<void**>(&cnt), (size_t)T * 4, s) != hipSuccess) return kDeviceFailed;
+  if (hipMallocAsync(reinterpret_cast<void**>(&off), (size_t)(T + 1) * 4, s) != hipSuccess) return kDeviceFailed;
+  if (hipMallocAsync(reinterpret_cast<void**>(&list), (size_t)(S > 0 ? S : 1) * 4, s) != hipSuccess) return kDeviceFailed;
+  if (hipMemsetAsync(cnt, 0, (size_t)T * 4, s) != hipSuccess) return kDeviceFailed;
+  if (S > 0) hipLaunchKernelGGL(combine_count_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, cnt);
+  hipLaunchKernelGGL(combine_scan_kernel, dim3(1), dim3(1024), 0, s, cnt, T, off);
+  if (S > 0) hipLaunchKernelGGL(combine_fill_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, off, cnt, list);
+  hipLaunchKernelGGL((combine_kernel<YT>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, off, list, out, N);
+  int rc = launch_status();
+  if (hipFreeAsync(cnt, s) != hipSuccess || hipFreeAsync(off, s) != hipSuccess || hipFreeAsync(list, s) != hipSuccess)
+    rc = kDeviceFailed;
+  return rc;
+}
+
+int dispatch_dev(const void* x, const int32_t* token_of_slot, void* x_perm, int T, int S, int H, int elem_bytes,
+                 hipStream_t s) {
+  if (T <= 0 || S < 0 || H <= 0 || (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) || !x ||
+      (S > 0 && (!token_of_slot || !x_perm)))
+    return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  if (S == 0) return kOk;
+  hipLaunchKernelGGL(dispatch_kernel, dim3(S), dim3(256), 0, s, static_cast<const char*>(x), token_of_slot,
+                     static_cast<char*>(x_perm), T, S, (long)H * elem_bytes);
+  return launch_status();
+}
+
+bool bad_grouped(int S, int K, int N, int E) { return S < 0 || K <= 0 || N <= 0 || E <= 0; }
+
+template <int EPI>
+int grouped_dev(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K, int N, int E,
+                hipStream_t s) {
+  if (bad_grouped(S, K, N, E) || !w || !offsets || (S > 0 && (!x || !y))) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  if (S == 0) return kOk;
+  Gemm16Params p{};
+  p.A = static_cast<const uint16_t*>(x);
+  p.B = static_cast<const uint16_t*>(w);
+  p.D = y;
+  p.M = S; p.N = N; p.K = K;
+  p.lda = K; p.ldb = N; p.ldd = N;
+  p.strideB = (long)K * N;
+  p.offsets = offsets;
+  p.groups = E;
+  return launch_gemm16_grouped<BF16, EPI>(p, s);
+}
+
+int swiglu_dev(const void* x, const void* wg, const void* wu, const void* wd, const int32_t* offsets, void* y,
+               void* hidden, int S, int K, int F, int N, int E, hipStream_t s) {
+  if (bad_grouped(S, K, N, E) || F <= 0 || !wg || !wu || !wd || !offsets || (S > 0 && (!x || !y))) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  if (S == 0) return kOk;
+  void* h = hidden;
+  if (!h && hipMallocAsync(&h, (size_t)S * F * 2, s) != hipSuccess) return kDeviceFailed;
+  Gemm16Params p{};
+  p.A = static_cast<const uint16_t*>(x);
+  p.B = static_cast<const uint16_t*>(wg);
+  p.B2 = static_cast<const uint16_t*>(wu);
+  p.D = h;
+  p.M = S; p.N = F; p.K = K;
+  p.lda = K; p.ldb = F; p.ldd = F;
+  p.strideB = (long)K * F;
+  p.offsets = offsets;
+  p.groups = E;
+  int rc = launch_gemm16_grouped<BF16, EPI_SWIGLU16>(p, s);
+  if (rc == kOk) rc = grouped_dev<EPI_STORE16>(h, wd, offsets, y, S, F, N, E, s);
+  if (!hidden && hipFreeAsync(h, s) != hipSuccess) rc = kDeviceFailed;
+  return rc;
+}
+
+int combine_host(const void* y_perm, const int32_t* token_of_slot, const float* weights, float* out, int T,
+                        int S, int N, int ysz) {
+  if (T <= 0 || S < 0 || N <= 0 || !out || (S > 0 && (!y_perm || !token_of_slot || !weights))) return kBadShape;
+  for (int s = 0; s < S; ++s)
+    if (token_of_slot[s] < 0 || token_of_slot[s] >= T) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  DeviceScope scope;
+  void* dy = scope.alloc((size_t)S * N * ysz, y_perm);
+  int32_t* dt = static_cast<int32_t*>(scope.alloc((size_t)S * 4, token_of_slot));
+  float* dw = static_cast<float*>(scope.alloc((size_t)S * 4, weights));
+  float* dout = static_cast<float*>(scope.alloc((size_t)T * N * 4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = ysz == 2 ? combine_dev<uint16_t>(dy, dt, dw, dout, T, S, N, nullptr)
+                    : combine_dev<float>(dy, dt, dw, dout, T, S, N, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  return scope.download(out, dout, (size_t)T * N * 4) ? kOk : kDeviceFailed;
+}
+// offsets must be non-decreasing, start at 0 and end at S.
+bool bad_offsets(const int32_t* offsets, int E, int S) {
+  if (offsets[0] != 0 || offsets[E] != S) return true;
+  for (int e = 0; e < E; ++e)
+    if (offsets[e + 1] < offsets[e]) return true;
+  return false;
+}
+
+template <int EPI>
+int grouped_host(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K, int N, int E) {
+  if (bad_grouped(S, K, N, E) || !w || !offsets || (S > 0 && (!x || !y))) return kBadShape;
+  if (bad_offsets(offsets, E, S)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  if (S == 0) return kOk;
+  const size_t dsz = EPI == EPI_F32 ? 4 : 2;
+  DeviceScope scope;
+  void* dx = scope.alloc((size_t)S * K * 2, x);
+  void* dw = scope.alloc((size_t)E * K * N * 2, w);
+  int32_t* dof = static_cast<int32_t*>(scope.alloc((size_t)(E + 1) * 4, offsets));
+  void* dy = scope.alloc((size_t)S * N * dsz);
+  if (scope.failed()) return kDeviceFailed;
+  int rc = grouped_dev<EPI>(dx, dw, dof, dy, S, K, N, E, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  return scope.download(y, dy, (size_t)S * N * dsz) ? kOk : kDeviceFailed;
+}
+}  // namespace
+}  // namespace tsr950
+
+using namespace tsr950;
+
+extern "C" {
+
+int tessera_gfx950_moe_route_f32_dev(const float* scores, int T, int E, int k, int normalize, int capacity,
+                                     int32_t* token_of_slot, int32_t* expert_of_slot, float* combine_weights,
+                                     int32_t* group_sizes, int32_t* group_offsets, int32_t* num_slots,
+                                     void* stream) {
+  return route_dev(scores, T, E, k, normalize, capacity, token_of_slot, expert_of_slot, combine_weights,
+                   group_sizes, group_offsets, num_slots, as_stream(stream));
+}
+
+int tessera_gfx950_moe_route_f32(const float* scores, int T, int E, int k, int normalize, int capacity,
+                                 int32_t* token_of_slot, int32_t* expert_of_slot, float* combine_weights,
+                                 int32_t* group_sizes, int32_t* group_offsets, int32_t* num_slots) {
+  if (T <= 0 || E <= 0 || k <= 0 || k > E || E > kMaxExperts || !scores || !token_of_slot || !expert_of_slot ||
+      !combine_weights || !group_sizes || !group_offsets)
+    return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t S = (size_t)T * k;
+  DeviceScope scope;
+  float* ds = static_cast<float*>(scope.alloc((size_t)T * E * 4, scores));
+  int32_t* dt = static_cast<int32_t*>(scope.alloc(S * 4));
+  int32_t* de = static_cast<int32_t*>(scope.alloc(S * 4));
+  float* dw = static_cast<float*>(scope.alloc(S * 4));
+  int32_t* dg = static_cast<int32_t*>(scope.alloc((size_t)E * 4));
+  int32_t* dof = static_cast<int32_t*>(scope.alloc((size_t)(E + 1) * 4));
+  int32_t* dn = static_cast<int32_t*>(scope.alloc(4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = route_dev(ds, T, E, k, normalize, capacity, dt, de, dw, dg, dof, dn, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  int32_t n = 0;
+  if (!scope.download(&n, dn, 4)) return kDeviceFailed;
+  if (!scope.download(token_of_slot, dt, (size_t)n * 4) || !scope.download(expert_of_slot, de, (size_t)n * 4) ||
+      !scope.download(combine_weights, dw, (size_t)n * 4) || !scope.download(group_sizes, dg, (size_t)E * 4) ||
+      !scope.download(group_offsets, dof, (size_t)(E + 1) * 4))
+    return kDeviceFailed;
+  if (num_slots) *num_slots = n;
+  return kOk;
+}
+
+int tessera_gfx950_moe_dispatch_dev(const void* x, const int32_t* token_of_slot, void* x_perm, int T, int S, int H,
+                                    int elem_bytes, void* stream) {
+  return dispatch_dev(x, token_of_slot, x_perm, T, S, H, elem_bytes, as_stream(stream));
+}
+
+int tessera_gfx950_moe_dispatch(const void* x, const int32_t* token_of_slot, void* x_perm, int T, int S, int H,
+                                int elem_bytes) {
+  if (T <= 0 || S < 0 || H <= 0 || (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) || !x ||
+      (S > 0 && (!token_of_slot || !x_perm)))
+    return kBadShape;
+  for (int s = 0; s < S; ++s)
+    if (token_of_slot[s] < 0 || token_of_slot[s] >= T) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  if (S == 0) return kOk;
+  const size_t row = (size_t)H * elem_bytes;
+  DeviceScope scope;
+  void* dx = scope.alloc((size_t)T * row, x);
+  int32_t* dt = static_cast<int32_t*>(scope.alloc((size_t)S * 4, token_of_slot));
+  void* dp = scope.alloc((size_t)S * row);
+  if (scope.failed()) return kDeviceFailed;
+  int rc = dispatch_dev(dx, dt, dp, T, S, H, elem_bytes, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  return scope.download(x_perm, dp, (size_t)S * row) ? kOk : kDeviceFailed;
+}
+
+int tessera_gfx950_moe_combine_bf16_dev(const void* y_perm, const int32_t* token_of_slot, const float* weights,
+                                        float* out, int T, int S, int N, void* stream) {
+  return combine_dev<uint16_t>(y_perm, token_of_slot, weights, out, T, S, N, as_stream(stream));
+}
+int tessera_gfx950_moe_combine_f32_dev(const void* y_perm, const int32_t* token_of_slot, const float* weights,
+                                       float* out, int T, int S, int N, void* stream) {
+  return combine_dev<float>(y_perm, token_of_slot, weights, out, T, S, N, as_stream(stream));
+}
+
+int tessera_gfx950_moe_combine_bf16(const void* y_perm, const int32_t* token_of_slot, const float* weights,
+                                    float* out, int T, int S, int N) {
+  return combine_host(y_perm, token_of_slot, weights, out, T, S, N, 2);
+}
+int tessera_gfx950_moe_combine_f32(const void* y_perm, const int32_t* token_of_slot, const float* weights,
+                                   float* out, int T, int S, int N) {
+  return combine_host(y_perm, token_of_slot, weights, out, T, S, N, 4);
+}
+
+int tessera_gfx950_grouped_gemm_bf16_dev(const void* x, const void* w, const int32_t* offsets, void* y, int S,
+                                         int K, int N, int E, void* stream) {
+  return grouped_dev<EPI_STORE16>(x, w, offsets, y, S, K, N, E, as_stream(stream));
+}
+int tessera_gfx950_grouped_gemm_bf16_f32_dev(const void* x, const void* w, const int32_t* offsets, void* y, int S,
+                                             int K, int N, int E, void* stream) {
+  return grouped_dev<EPI_F32>(x, w, offsets, y, S, K, N, E, as_stream(stream));
+}
+
+int tessera_gfx950_grouped_gemm_bf16(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K,
+                                     int N, int E) {
+  return grouped_host<EPI_STORE16>(x, w, offsets, y, S, K, N, E);
+}
+int tessera_gfx950_grouped_gemm_bf16_f32(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K,
+                                         int N, int E) {
+  return grouped_host<EPI_F32>(x, w, offsets, y, S, K, N, E);
+}
+
+int tessera_gfx950_moe_swiglu_block_bf16_dev(const void* x, const void* wg, const void* wu, const void* wd,
+                                             const int32_t* offsets, void* y, void* hidden, int S, int K, int F,
+                                             int N, int E, void* stream) {
+  return swiglu_dev(x, wg, wu, wd, offsets, y, hidden, S, K, F, N, E, as_stream(stream));
+}
+
+int tessera_gfx950_moe_swiglu_block_bf16(const void* x, const void* wg, const void* wu, const void* wd,
+                                         const int32_t* offsets, void* y, int S, int K, int F, int N, int E) {
+  if (bad_grouped(S, K, N, E) || F <= 0 || !wg || !wu || !wd || !offsets || (S > 0 && (!x || !y))) return kBadShape;
+  if (bad_offsets(offsets, E, S)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  if (S == 0) return kOk;
+  DeviceScope scope;
+  void* dx = scope.alloc((size_t)S * K * 2, x);
+  void* dg = scope.alloc((size_t)E * K * F * 2, wg);
+  void* du = scope.alloc((size_t)E * K * F * 2, wu);
+  void* dd = scope.alloc((size_t)E * F * N * 2, wd);
+  int32_t* dof = static_cast<int32_t*>(scope.alloc((size_t)(E + 1) * 4, offsets));
+  void* dh = scope.alloc((size_t)S * F * 2);
+  void* dy = scope.alloc((size_t)S * N * 2);
+  if (scope.failed()) return kDeviceFailed;
+  int rc = swiglu_dev(dx, dg, du, dd, dof, dy, dh, S, K, F, N, E, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  return scope.download(y, dy, (size_t)S * N * 2) ? kOk : kDeviceFailed;
+}
+
+int tessera_gfx950_moe_layer_bf16(const void* x, const float* router_logits, const void* wg, const void* wu,
+                                  const void* wd, float* out, int T, int H, int F, int N, int E, int k,
+                                  int normalize, int capacity, int32_t* token_of_slot, int32_t* expert_of_slot,
+                                  float* combine_weights, int32_t* group_sizes, int32_t* group_offsets) {
+  if (T <= 0 || H <= 0 || F <= 0 || N <= 0 || E <= 0 || k <= 0 || k > E || E > kMaxExperts || !x ||
+      !router_logits || !wg || !wu || !wd || !out)
+    return kBadShape;
+  if ((long)T * k > 0x7fffffffL) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t S = (size_t)T * k;
+  DeviceScope scope;
+  void* dx = scope.alloc((size_t)T * H * 2, x);
+  float* dl = static_cast<float*>(scope.alloc((size_t)T * E * 4, router_logits));
+  void* dg = scope.alloc((size_t)E * H * F * 2, wg);
+  void* du = scope.alloc((size_t)E * H * F * 2, wu);
+  void* dd = scope.alloc((size_t)E * F * N * 2, wd);
+  int32_t* dt = static_cast<int32_t*>(scope.alloc(S * 4));
+  int32_t* de = static_cast<int32_t*>(scope.alloc(S * 4));
+  float* dw = static_cast<float*>(scope.alloc(S * 4));
+  int32_t* dgs = static_cast<int32_t*>(scope.alloc((size_t)E * 4));
+  int32_t* dof = static_cast<int32_t*>(scope.alloc((size_t)(E + 1) * 4));
+  int32_t* dn = static_cast<int32_t*>(scope.alloc(4));
+  void* dxp = scope.alloc(S * H * 2);
+  void* dh = scope.alloc(S * F * 2);
+  void* dy = scope.alloc(S * N * 2);
+  float* dout = static_cast<float*>(scope.alloc((size_t)T * N * 4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = route_dev(dl, T, E, k, normalize, capacity, dt, de, dw, dgs, dof, dn, nullptr);
+  if (rc != kOk) return rc;
+  int32_t n = 0;                       // kept slots (capacity may drop some)
+  if (hipDeviceSynchronize() != hipSuccess || !scope.download(&n, dn, 4)) return kDeviceFailed;
+  rc = dispatch_dev(dx, dt, dxp, T, n, H, 2, nullptr);
+  if (rc == kOk) rc = swiglu_dev(dxp, dg, du, dd, dof, dy, dh, n, H, F, N, E, nullptr);
+  if (rc == kOk) rc = combine_dev<uint16_t>(dy, dt, dw, dout, T, n, N, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  if (!scope.download(out, dout, (size_t)T * N * 4)) return kDeviceFailed;
+  if (token_of_slot && !scope.download(token_of_slot, dt, (size_t)n * 4)) return kDeviceFailed;
+  if (expert_of_slot && !scope.download(expert_of_slot, de, (size_t)n * 4)) return kDeviceFailed;
+  if (combine_weights && !scope.download(combine_weights, dw, (size_t)n * 4)) return kDeviceFailed;
+  if (group_sizes && !scope.download(group_sizes, dgs, (size_t)E * 4)) return kDeviceFailed;
+  if (group_offsets && !scope.download(group_offsets, dof, (size_t)(E + 1) * 4)) return kDeviceFailed;
+  return kOk;
+}
+
+}  // extern "C"

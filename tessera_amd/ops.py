@@ -1,0 +1,555 @@
+"""The dense-op surface of ``tessera.ops`` / ``tessera.nn.functional`` on the
+gfx950 lane.
+
+Same names, argument meaning and error behaviour as the reference's numpy
+definitions, but every function computes on the MI355X through the C ABI
+(:mod:`tessera_amd.lane`).  There is no CPU path: without the library or the
+device the calls raise :class:`~tessera_amd.lane.LaneUnavailable`.
+
+Reference definitions mirrored here (paths under ``python/tessera``):
+
+=====================  ==========================================================
+``gemm`` / ``matmul``   ``__init__.py:239-254`` + storage rule ``:5783-5855``
+``batched_gemm``
+``flash_attn``          ``__init__.py:1304-1356``
+``gqa_attention``       ``nn/functional.py:349-356``
+``grouped_gemm``        ``__init__.py:291-351``
+``moe_swiglu_block``    ``__init__.py:592-616``
+``route_tokens``        ``distributed/moe.py:119-206`` (+ transport ABI
+                        ``compiler/moe_transport.py:194-273``)
+``moe_dispatch`` /      ``stdlib/moe.py:117-134``, ``runtime.py:1791-1824``
+``moe_combine``
+``moe_layer``           ``nn/functional.py:403-490``
+``quantize_fp8``        ``__init__.py:3340-3374``
+``quantize_int8_per_channel`` / ``w8a8_matmul``
+                        ``compiler/smoothquant.py:79-84,115-124``
+=====================  ==========================================================
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
+
+from . import bf16 as _bf16
+from . import lane as _lane
+from .bf16 import BF16Array
+
+GROUPED_KINDS = ("contiguous", "dense", "masked", "k_grouped")
+_SUPPORTED_GROUPED_KINDS = ("contiguous", "dense")
+
+
+# ---------------------------------------------------------------------------
+# storage helpers
+# ---------------------------------------------------------------------------
+
+
+def _storage(a, b=None) -> str:
+    """'f16' or 'bf16' — the 16-bit storage dtype of the operand(s)."""
+    def one(x):
+        if _bf16.is_bf16(x):
+            return "bf16"
+        if getattr(x, "dtype", None) == np.float16:
+            return "f16"
+        raise ValueError(
+            f"gfx950 lane handles f16/bf16 storage (f32 accumulate); got {getattr(x, 'dtype', type(x))}")
+    s = one(a)
+    if b is not None and one(b) != s:
+        raise ValueError("operands must share one 16-bit storage dtype")
+    return s
+
+
+def _bits(a) -> np.ndarray:
+    if _bf16.is_bf16(a):
+        return _bf16.as_bits(a)
+    return np.ascontiguousarray(a, np.float16).view(np.uint16)
+
+
+def _wrap(bits: np.ndarray, storage: str):
+    return bits.view(BF16Array) if storage == "bf16" else bits.view(np.float16)
+
+
+def _unbox(x):
+    return x._data if hasattr(x, "_data") else x
+
+
+# ---------------------------------------------------------------------------
+# GEMM
+# ---------------------------------------------------------------------------
+
+
+def gemm(A, B, *, out: str = "storage"):
+    """``A @ B`` with f32 accumulate.  16-bit operands; leading dims of ``A`` (and
+    of ``B`` when it is not rank 2) are batch dims and must match.
+
+    ``out="storage"`` stores the result in the operands' storage dtype (the
+    ``ops.gemm`` rule for reduced-precision operands); ``out="f32"`` returns the
+    f32 accumulators (the executors' contract)."""
+    A, B = _unbox(A), _unbox(B)
+    st = _storage(A, B)
+    a, b = _bits(A), _bits(B)
+    if a.ndim < 2 or b.ndim < 2:
+        raise ValueError("gemm needs operands of rank >= 2")
+    M, K = a.shape[-2:]
+    if b.shape[-2] != K:
+        raise ValueError(f"gemm: K mismatch — A {a.shape} @ B {b.shape}")
+    N = b.shape[-1]
+    lead = a.shape[:-2]
+    batch = int(np.prod(lead)) if lead else 1
+    if b.ndim > 2:
+        if b.shape[:-2] != lead:
+            raise ValueError(f"batched gemm: leading dims differ — A {a.shape} @ B {b.shape}")
+    elif batch > 1:
+        # one weight for every batch: fold the batch into M
+        M = batch * M
+        batch = 1
+        a = a.reshape(M, K)
+    if out not in ("storage", "f32"):
+        raise ValueError("out must be 'storage' or 'f32'")
+    lib = _lane.load()
+    f32 = out == "f32"
+    shape = tuple(A.shape[:-1]) + (N,)
+    if batch == 1:
+        d = np.empty((M, N), np.float32 if f32 else np.uint16)
+        name = f"tessera_gfx950_gemm_{st}" + ("" if f32 else f"_{st}")
+        _lane.check(getattr(lib, name)(a.ctypes.data, b.ctypes.data, d.ctypes.data, M, N, K), "gemm")
+        return d.reshape(shape) if f32 else _wrap(d.reshape(shape), st)
+    # the batched entry point keeps f32 accumulators; the storage rule rounds after
+    d32 = np.empty((batch, M, N), np.float32)
+    _lane.check(getattr(lib, f"tessera_gfx950_batched_gemm_{st}")(
+        a.ctypes.data, b.ctypes.data, d32.ctypes.data, batch, M, N, K), "batched_gemm")
+    if f32:
+        return d32.reshape(shape)
+    if st == "bf16":
+        return _bf16.from_float32(d32).reshape(shape)
+    return d32.astype(np.float16).reshape(shape)
+
+
+matmul = gemm
+batched_gemm = gemm
+
+
+def gemm_i8(A, B) -> np.ndarray:
+    """``int32(A) @ int32(B)`` for int8 operands — exact."""
+    a = np.ascontiguousarray(_unbox(A))
+    b = np.ascontiguousarray(_unbox(B))
+    if a.dtype != np.int8 or b.dtype != np.int8:
+        raise ValueError("gemm_i8 needs int8 operands")
+    if a.ndim != 2 or b.ndim != 2 or a.shape[1] != b.shape[0]:
+        raise ValueError(f"gemm_i8 needs rank-2 operands with matching K; got {a.shape} @ {b.shape}")
+    M, K = a.shape
+    N = b.shape[1]
+    c = np.empty((M, N), np.int32)
+    _lane.check(_lane.load().tessera_gfx950_gemm_i8_i32(a.ctypes.data, b.ctypes.data, c.ctypes.data, M, N, K),
+                "gemm_i8")
+    return c
+
+
+# ---------------------------------------------------------------------------
+# attention
+# ---------------------------------------------------------------------------
+
+
+def _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa):
+    Q, K, V = _unbox(Q), _unbox(K), _unbox(V)
+    st = _storage(Q, K)
+    if _storage(V) != st:
+        raise ValueError("Q, K, V must share one storage dtype")
+    q, k, v = _bits(Q), _bits(K), _bits(V)
+    if q.ndim < 2 or k.ndim < 2 or v.ndim < 2:
+        raise ValueError("flash_attn Q/K/V must be at least rank 2 ([..., S, D])")
+    D = q.shape[-1]
+    if D <= 0 or D % 16 != 0:
+        raise ValueError(f"gfx950 flash_attn lane needs head_dim a positive multiple of 16; got {D}")
+    Sq, Sk = q.shape[-2], k.shape[-2]
+    if v.shape != k.shape or k.shape[-1] != D:
+        raise ValueError(f"flash_attn requires V to match K and Q's head dim; got Q{q.shape} K{k.shape} V{v.shape}")
+    Hq = q.shape[-3] if q.ndim >= 3 else 1
+    Hkv = k.shape[-3] if k.ndim >= 3 else 1
+    Bq = int(np.prod(q.shape[:-3])) if q.ndim > 3 else 1
+    Bk = int(np.prod(k.shape[:-3])) if k.ndim > 3 else 1
+    if Bq != Bk:
+        raise ValueError("flash_attn: batch dims of Q and K differ")
+    if Hq != Hkv:
+        if not allow_gqa:
+            raise ValueError(f"flash_attn needs matching head counts; got {Hq} vs {Hkv} (use gqa_attention)")
+        if Hkv <= 0 or Hq % Hkv != 0:
+            raise ValueError(f"GQA needs query-heads ({Hq}) divisible by kv-heads ({Hkv})")
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    o = np.empty(q.shape, np.float32)
+    lse = np.empty(q.shape[:-1], np.float32) if return_lse else None
+    fn = getattr(_lane.load(), f"tessera_gfx950_flash_attn_gqa_{st}")
+    rc = fn(q.ctypes.data, k.ctypes.data, v.ctypes.data, o.ctypes.data, _lane.ptr(lse),
+            Bq, Hq, Hkv, Sq, Sk, D, float(scale), 1 if causal else 0)
+    _lane.check(rc, "flash_attn")
+    if out == "storage":
+        o = _bf16.from_float32(o) if st == "bf16" else o.astype(np.float16)
+    elif out != "f32":
+        raise ValueError("out must be 'storage' or 'f32'")
+    return (o, lse) if return_lse else o
+
+
+def flash_attn(Q, K=None, V=None, scale=None, causal: bool = False, *, return_lse: bool = False,
+               out: str = "storage"):
+    """``softmax(scale * Q K^T, causal) V``.  Q/K/V ``[..., H, S, D]`` 16-bit; the
+    causal mask is bottom-right aligned (key ``j`` visible to query ``i`` iff
+    ``j <= i + max(Sk - Sq, 0)``).  Head counts must match (as in the reference)."""
+    return _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa=False)
+
+
+def gqa_attention(Q, K, V, scale=None, causal: bool = False, *, return_lse: bool = False,
+                  out: str = "storage"):
+    """Grouped-query attention: kv head of query head ``h`` is ``h // (Hq / Hkv)``
+    — identical to repeating K/V along the head axis."""
+    return _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa=True)
+
+
+# ---------------------------------------------------------------------------
+# MoE
+# ---------------------------------------------------------------------------
+
+
+def _offsets(group_sizes, total: int, what: str) -> np.ndarray:
+    gs = np.asarray(group_sizes).astype(np.int64).reshape(-1)
+    if gs.size <= 0 or np.any(gs < 0) or int(gs.sum()) != total:
+        raise ValueError(f"{what}: group_sizes sum {int(gs.sum()) if gs.size else 0} != T={total}")
+    off = np.concatenate((np.zeros(1, np.int64), np.cumsum(gs)))
+    if int(off[-1]) > np.iinfo(np.int32).max:
+        raise ValueError("grouped expert offsets exceed the int32 device ABI")
+    return np.ascontiguousarray(off, np.int32)
+
+
+def grouped_gemm(x, weights, group_sizes, *, kind: str = "contiguous", alignment=None, quant=None,
+                 out: str = "storage"):
+    """Ragged grouped matmul: row block ``e`` of the result is
+    ``x[block e] @ weights[e]``.  ``x`` ``(T, K)`` sorted by expert, ``weights``
+    ``(E, K, N)``, ``group_sizes`` ``(E,)`` summing to ``T``."""
+    if kind not in GROUPED_KINDS:
+        raise ValueError(f"grouped_gemm: unknown kind {kind!r}; expected one of {GROUPED_KINDS}")
+    if kind not in _SUPPORTED_GROUPED_KINDS:
+        raise NotImplementedError(
+            f"grouped_gemm: kind={kind!r} is not implemented — supported: "
+            f"{', '.join(_SUPPORTED_GROUPED_KINDS)}")
+    if quant is not None:
+        raise NotImplementedError("grouped_gemm: quantised grouped GEMM is not part of the gfx950 lane")
+    x, weights = _unbox(x), _unbox(weights)
+    if _storage(x, weights) != "bf16":
+        raise ValueError("grouped_gemm on the gfx950 lane takes bf16 storage")
+    xa, w = _bits(x), _bits(weights)
+    gs = np.asarray(group_sizes).astype(np.int64).reshape(-1)
+    if alignment is not None:
+        al = int(alignment)
+        if al <= 0 or np.any(gs % al != 0):
+            raise ValueError(f"grouped_gemm: every group size must be a multiple of alignment={alignment}")
+    if xa.ndim != 2:
+        raise ValueError(f"grouped_gemm: x must be (T, K); got {xa.shape}")
+    if w.ndim != 3 or w.shape[0] != gs.shape[0]:
+        raise ValueError(f"grouped_gemm: weights {w.shape} must be (E, K, N) with E == len(group_sizes)={gs.shape[0]}")
+    if w.shape[1] != xa.shape[1]:
+        raise ValueError(f"grouped_gemm: K mismatch — x K={xa.shape[1]}, weights K={w.shape[1]}")
+    T, K = xa.shape
+    E, _, N = w.shape
+    off = _offsets(gs, T, "grouped_gemm")
+    f32 = out == "f32"
+    y = np.zeros((T, N), np.float32 if f32 else np.uint16)
+    name = "tessera_gfx950_grouped_gemm_bf16" + ("_f32" if f32 else "")
+    _lane.check(getattr(_lane.load(), name)(xa.ctypes.data, w.ctypes.data, off.ctypes.data, y.ctypes.data, T, K, N, E),
+                "grouped_gemm")
+    return y if f32 else y.view(BF16Array)
+
+
+def moe_swiglu_block(x, w_gate, w_up, w_down, group_sizes, *, kind: str = "contiguous", alignment=None,
+                     quant=None):
+    """``gg(silu_mul(gg(x, Wg), gg(x, Wu)), Wd)`` over contiguous expert groups,
+    every intermediate rounded to bf16 as the reference's storage rule does."""
+    if kind not in GROUPED_KINDS:
+        raise ValueError(f"moe_swiglu_block: unknown kind {kind!r}")
+    if kind not in _SUPPORTED_GROUPED_KINDS or quant is not None:
+        raise NotImplementedError("moe_swiglu_block: only contiguous/dense, unquantised on the gfx950 lane")
+    x, w_gate, w_up, w_down = map(_unbox, (x, w_gate, w_up, w_down))
+    for a in (x, w_gate, w_up, w_down):
+        if _storage(a) != "bf16":
+            raise ValueError("moe_swiglu_block on the gfx950 lane takes bf16 storage")
+    xa, wg, wu, wd = map(_bits, (x, w_gate, w_up, w_down))
+    if xa.ndim != 2 or wg.ndim != 3 or wu.shape != wg.shape or wd.ndim != 3:
+        raise ValueError("moe_swiglu_block: x (T,K), w_gate/w_up (E,K,F), w_down (E,F,N)")
+    T, K = xa.shape
+    E, Kw, F = wg.shape
+    if Kw != K or wd.shape[0] != E or wd.shape[1] != F:
+        raise ValueError("moe_swiglu_block: weight shapes disagree")
+    N = wd.shape[2]
+    gs = np.asarray(group_sizes).astype(np.int64).reshape(-1)
+    if gs.shape[0] != E:
+        raise ValueError("moe_swiglu_block: len(group_sizes) != E")
+    if alignment is not None and np.any(gs % int(alignment) != 0):
+        raise ValueError(f"moe_swiglu_block: every group size must be a multiple of alignment={alignment}")
+    off = _offsets(gs, T, "moe_swiglu_block")
+    y = np.zeros((T, N), np.uint16)
+    rc = _lane.load().tessera_gfx950_moe_swiglu_block_bf16(
+        xa.ctypes.data, wg.ctypes.data, wu.ctypes.data, wd.ctypes.data, off.ctypes.data, y.ctypes.data, T, K, F, N, E)
+    _lane.check(rc, "moe_swiglu_block")
+    return y.view(BF16Array)
+
+
+@dataclass
+class MoETransport:
+    """The int32 device ABI of the MoE transport descriptor
+    (``compiler/moe_transport.py:194-273``)."""
+    num_tokens: int
+    top_k: int
+    num_experts: int
+    capacity: Optional[int]
+    token_of_slot: np.ndarray      # int32[S]
+    expert_of_slot: np.ndarray     # int32[S], non-decreasing
+    combine_weights: np.ndarray    # f32[S]
+    group_sizes: np.ndarray        # int32[E]
+    group_offsets: np.ndarray      # int32[E+1]
+
+    @property
+    def num_slots(self) -> int:
+        return int(self.token_of_slot.shape[0])
+
+
+def _capacity_arg(capacity: Optional[int], T: int, k: int) -> int:
+    if capacity is None or capacity >= T * k:
+        return 0            # cannot overflow
+    if capacity < 1:
+        raise ValueError("capacity must be >= 1")
+    return int(capacity)
+
+
+def route_tokens(scores, num_experts: int, top_k: int, *, normalize_weights: bool = True,
+                 capacity_factor: float = 1.25, capacity: Optional[int] = None) -> MoETransport:
+    """Top-k routing + packing plan.  ``scores`` ``(T, E)`` f32 gate logits.
+    capacity defaults to ``ceil(capacity_factor * T / E)``; over-capacity slots are
+    dropped first-come in token-major order.  Ties between equal probabilities go
+    to the lowest expert id."""
+    s = np.ascontiguousarray(_unbox(scores), np.float32)
+    if s.ndim != 2:
+        raise ValueError(f"scores must be 2D (num_tokens, num_experts), got shape {s.shape}")
+    T, E = s.shape
+    if E != num_experts:
+        raise ValueError(f"scores has {E} expert columns but num_experts={num_experts}")
+    if top_k < 1 or top_k > num_experts:
+        raise ValueError(f"top_k must be in [1, num_experts={num_experts}], got {top_k}")
+    if capacity is None:
+        if capacity_factor <= 0:
+            raise ValueError(f"capacity_factor must be > 0, got {capacity_factor}")
+        capacity = int(math.ceil(capacity_factor * T / E))
+    cap = _capacity_arg(capacity, T, top_k)
+    S = T * top_k
+    tos = np.empty(S, np.int32)
+    eos = np.empty(S, np.int32)
+    cw = np.empty(S, np.float32)
+    gs = np.empty(E, np.int32)
+    go = np.empty(E + 1, np.int32)
+    n = np.zeros(1, np.int32)
+    rc = _lane.load().tessera_gfx950_moe_route_f32(
+        s.ctypes.data, T, E, top_k, 1 if normalize_weights else 0, cap,
+        tos.ctypes.data, eos.ctypes.data, cw.ctypes.data, gs.ctypes.data, go.ctypes.data, n.ctypes.data)
+    _lane.check(rc, "route_tokens")
+    k = int(n[0])
+    return MoETransport(T, top_k, E, cap or None, tos[:k].copy(), eos[:k].copy(), cw[:k].copy(), gs, go)
+
+
+def moe_dispatch(x, plan: MoETransport):
+    """Gather the token row of every kept, expert-sorted slot → ``(S, H)``."""
+    x = _unbox(x)
+    if _bf16.is_bf16(x):
+        xa, wrap = _bf16.as_bits(x), (lambda b: b.view(BF16Array))
+    else:
+        xa = np.ascontiguousarray(x)
+        if xa.dtype not in (np.float16, np.float32):
+            raise ValueError("moe_dispatch takes f16, bf16 or f32 rows")
+        wrap = lambda b: b
+    if xa.ndim != 2:
+        raise ValueError(f"moe_dispatch x must be 2-D (T,H); got {xa.shape}")
+    T, H = xa.shape
+    if T != plan.num_tokens:
+        raise ValueError("moe_dispatch: x rows != plan.num_tokens")
+    S = plan.num_slots
+    outp = np.empty((S, H), xa.dtype)
+    tos = np.ascontiguousarray(plan.token_of_slot, np.int32)
+    rc = _lane.load().tessera_gfx950_moe_dispatch(xa.ctypes.data, tos.ctypes.data, outp.ctypes.data, T, S, H,
+                                                  xa.dtype.itemsize)
+    _lane.check(rc, "moe_dispatch")
+    return wrap(outp)
+
+
+def moe_combine(y_packed, plan: MoETransport) -> np.ndarray:
+    """Weighted scatter-add of the packed expert rows back to ``(T, N)`` f32;
+    dropped slots contribute zero."""
+    y = _unbox(y_packed)
+    S = plan.num_slots
+    tos = np.ascontiguousarray(plan.token_of_slot, np.int32)
+    w = np.ascontiguousarray(plan.combine_weights, np.float32)
+    lib = _lane.load()
+    if _bf16.is_bf16(y):
+        ya = _bf16.as_bits(y)
+        fn = lib.tessera_gfx950_moe_combine_bf16
+    else:
+        ya = np.ascontiguousarray(y, np.float32)
+        fn = lib.tessera_gfx950_moe_combine_f32
+    if ya.ndim != 2 or ya.shape[0] != S:
+        raise ValueError(f"moe_combine partials must be 2-D (S,H) with S={S}; got {ya.shape}")
+    N = ya.shape[1]
+    outp = np.zeros((plan.num_tokens, N), np.float32)
+    _lane.check(fn(ya.ctypes.data, tos.ctypes.data, w.ctypes.data, outp.ctypes.data, plan.num_tokens, S, N),
+                "moe_combine")
+    return outp
+
+
+def moe_layer(x, W_router, W_gate, W_up, W_down, *, top_k: int = 1, normalize_weights: bool = True,
+              capacity_factor: float = 0.0, kind: str = "contiguous", alignment=None, quant=None,
+              router_logits=None, return_plan: bool = False):
+    """Single-device top-k SwiGLU MoE layer: router → permute → expert FFN →
+    combine.  ``x`` ``(T, K)``, ``W_router`` ``(K, E)``, ``W_gate``/``W_up``
+    ``(E, K, F)``, ``W_down`` ``(E, F, N)`` in bf16; returns ``(T, N)`` f32.
+    ``capacity_factor <= 0`` disables capacity drops.  ``router_logits``
+    ``(T, E)`` f32 may be given instead of ``W_router``."""
+    if kind not in _SUPPORTED_GROUPED_KINDS or quant is not None or alignment is not None:
+        raise NotImplementedError("moe_layer: contiguous, unquantised, unaligned form only on the gfx950 lane")
+    x, W_gate, W_up, W_down = map(_unbox, (x, W_gate, W_up, W_down))
+    for a in (x, W_gate, W_up, W_down):
+        if _storage(a) != "bf16":
+            raise ValueError("moe_layer on the gfx950 lane takes bf16 storage")
+    xa, wg, wu, wd = map(_bits, (x, W_gate, W_up, W_down))
+    T, H = xa.shape
+    E, _, F = wg.shape
+    N = wd.shape[2]
+    if router_logits is None:
+        scores = gemm(x, W_router)                       # storage-rounded, as ops.gemm
+        logits = scores.to_float32() if isinstance(scores, BF16Array) else np.asarray(scores, np.float32)
+    else:
+        logits = np.ascontiguousarray(router_logits, np.float32)
+    if logits.shape != (T, E):
+        raise ValueError(f"router logits must be (T, E)=({T}, {E}); got {logits.shape}")
+    logits = np.ascontiguousarray(logits, np.float32)
+    cap = 0
+    if capacity_factor > 0:
+        cap = _capacity_arg(int(math.ceil(capacity_factor * T / E)), T, top_k)
+    S = T * top_k
+    outp = np.zeros((T, N), np.float32)
+    tos = np.empty(S, np.int32)
+    eos = np.empty(S, np.int32)
+    cw = np.empty(S, np.float32)
+    gs = np.empty(E, np.int32)
+    go = np.empty(E + 1, np.int32)
+    rc = _lane.load().tessera_gfx950_moe_layer_bf16(
+        xa.ctypes.data, logits.ctypes.data, wg.ctypes.data, wu.ctypes.data, wd.ctypes.data, outp.ctypes.data,
+        T, H, F, N, E, top_k, 1 if normalize_weights else 0, cap,
+        tos.ctypes.data, eos.ctypes.data, cw.ctypes.data, gs.ctypes.data, go.ctypes.data)
+    _lane.check(rc, "moe_layer")
+    if not return_plan:
+        return outp
+    n = int(go[E])
+    return outp, MoETransport(T, top_k, E, cap or None, tos[:n].copy(), eos[:n].copy(), cw[:n].copy(), gs, go)
+
+
+# ---------------------------------------------------------------------------
+# quantisation
+# ---------------------------------------------------------------------------
+
+_E4M3_TABLE: Optional[np.ndarray] = None
+
+
+def e4m3_table() -> np.ndarray:
+    """The 256 OCP e4m3fn code values as f32."""
+    global _E4M3_TABLE
+    if _E4M3_TABLE is None:
+        c = np.arange(256)
+        e = (c >> 3) & 0xF
+        m = (c & 7).astype(np.float64)
+        v = np.where(e == 0, m * 2.0 ** -9, (1.0 + m / 8.0) * np.exp2(e.astype(np.float64) - 7.0))
+        v = np.where((e == 15) & ((c & 7) == 7), np.nan, v)
+        _E4M3_TABLE = np.where(c & 0x80, -v, v).astype(np.float32)
+    return _E4M3_TABLE
+
+
+def quantize_fp8_codes(x, *, scale=None):
+    """Per-tensor e4m3 quantisation on the device → ``(codes uint8, scale f32)``."""
+    xa = np.ascontiguousarray(_unbox(x), np.float32)
+    codes = np.empty(xa.shape, np.uint8)
+    s_out = ctypes.c_float(0)
+    rc = _lane.load().tessera_gfx950_quantize_e4m3_f32(
+        xa.ctypes.data, xa.size, float(scale) if scale is not None else 0.0, codes.ctypes.data,
+        ctypes.byref(s_out))
+    _lane.check(rc, "quantize_fp8")
+    return codes, np.float32(s_out.value)
+
+
+def quantize_fp8(x, *, format: str = "e4m3", scale=None):
+    """Per-tensor symmetric fp8 quantisation → ``(x_q_as_fp32, scale)`` where
+    ``x_q_as_fp32`` is the fp8-rounded value cast back to f32 (``grid * scale``)."""
+    if format not in ("e4m3", "e5m2"):
+        raise ValueError(f"format must be 'e4m3' or 'e5m2'; got {format!r}")
+    if format != "e4m3":
+        raise NotImplementedError("the gfx950 lane quantises to e4m3 (the GEMM operand format)")
+    codes, s = quantize_fp8_codes(x, scale=scale)
+    return e4m3_table()[codes] * np.float32(s), np.float32(s)
+
+
+def gemm_fp8(a_codes, b_codes, scale_a, scale_b, *, out: str = "bf16"):
+    """``f32acc(Aq . Bq) * scale_a * scale_b`` over e4m3 codes; bf16 or f32 result."""
+    a = np.ascontiguousarray(a_codes, np.uint8)
+    b = np.ascontiguousarray(b_codes, np.uint8)
+    if a.ndim != 2 or b.ndim != 2 or a.shape[1] != b.shape[0]:
+        raise ValueError(f"gemm_fp8 needs rank-2 operands with matching K; got {a.shape} @ {b.shape}")
+    M, K = a.shape
+    N = b.shape[1]
+    if out == "bf16":
+        d = np.empty((M, N), np.uint16)
+        fn = _lane.load().tessera_gfx950_gemm_e4m3_bf16
+    elif out == "f32":
+        d = np.empty((M, N), np.float32)
+        fn = _lane.load().tessera_gfx950_gemm_e4m3_f32
+    else:
+        raise ValueError("out must be 'bf16' or 'f32'")
+    _lane.check(fn(a.ctypes.data, b.ctypes.data, float(scale_a), float(scale_b), d.ctypes.data, M, N, K), "gemm_fp8")
+    return d.view(BF16Array) if out == "bf16" else d
+
+
+def quantize_int8_per_channel(M, axis: int):
+    """Symmetric int8 quantise along the kept axis → ``(q int8, scale f32)`` with
+    ``scale`` shaped like numpy's ``keepdims`` reduction over ``axis``."""
+    a = np.ascontiguousarray(_unbox(M), np.float32)
+    if a.ndim != 2 or axis not in (0, 1):
+        raise ValueError("quantize_int8_per_channel takes a 2-D array and axis 0 or 1")
+    R, C = a.shape
+    q = np.empty((R, C), np.int8)
+    sc = np.empty(R if axis == 1 else C, np.float32)
+    _lane.check(_lane.load().tessera_gfx950_quantize_i8_f32(a.ctypes.data, R, C, axis, q.ctypes.data, sc.ctypes.data),
+                "quantize_int8_per_channel")
+    return q, (sc.reshape(R, 1) if axis == 1 else sc.reshape(1, C))
+
+
+def w8a8_gemm(x_q, w_q, a_scale, w_scale, *, return_acc: bool = False):
+    """``f32(int32(x_q) @ int32(w_q)) * a_scale[:, None] * w_scale[None, :]``."""
+    a = np.ascontiguousarray(x_q, np.int8)
+    b = np.ascontiguousarray(w_q, np.int8)
+    if a.ndim != 2 or b.ndim != 2 or a.shape[1] != b.shape[0]:
+        raise ValueError(f"w8a8_gemm needs rank-2 operands with matching K; got {a.shape} @ {b.shape}")
+    M, K = a.shape
+    N = b.shape[1]
+    rs = np.ascontiguousarray(np.asarray(a_scale, np.float32).reshape(-1))
+    cs = np.ascontiguousarray(np.asarray(w_scale, np.float32).reshape(-1))
+    if rs.shape[0] != M or cs.shape[0] != N:
+        raise ValueError("w8a8_gemm: a_scale must have M entries and w_scale N entries")
+    d = np.empty((M, N), np.float32)
+    acc = np.empty((M, N), np.int32) if return_acc else None
+    rc = _lane.load().tessera_gfx950_gemm_w8a8_f32(a.ctypes.data, b.ctypes.data, rs.ctypes.data, cs.ctypes.data,
+                                                   d.ctypes.data, _lane.ptr(acc), M, N, K)
+    _lane.check(rc, "w8a8_gemm")
+    return (d, acc) if return_acc else d
+
+
+def w8a8_matmul(X, W):
+    """The W8A8 direct-consume path without smoothing: quantise activations per
+    row and weights per column on the device, integer GEMM, rescale."""
+    x_q, a_scale = quantize_int8_per_channel(X, axis=1)
+    w_q, w_scale = quantize_int8_per_channel(W, axis=0)
+    return w8a8_gemm(x_q, w_q, a_scale, w_scale)

@@ -1,0 +1,126 @@
+"""Flash-attention forward parity on the MI355X (through the C ABI) vs the oracle.
+
+Tolerances (written here as the north star states them): O max relative error
+<= 2e-3 normwise against an fp32-or-better reference of the same 16-bit inputs;
+LSE absolute error <= 2e-3.  The reference's own test budgets are looser
+(f16 2e-2, bf16 6e-2 absolute, tests/unit/test_rocm_flash_attn_runtime_symbol.py:90-132).
+"""
+import numpy as np
+import pytest
+
+import tessera_oracle as orc
+from tessera_amd import bf16 as b16
+from tessera_amd import ops
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+def _qkv(B, Hq, Hkv, Sq, Sk, D, seed, st, scale=1.0):
+    rng = np.random.default_rng(seed)
+    q = (rng.standard_normal((B, Hq, Sq, D)) * scale).astype(np.float32)
+    k = (rng.standard_normal((B, Hkv, Sk, D)) * scale).astype(np.float32)
+    v = (rng.standard_normal((B, Hkv, Sk, D)) * scale).astype(np.float32)
+    if st == "bf16":
+        return tuple(b16.from_float32(x) for x in (q, k, v))
+    return tuple(x.astype(np.float16) for x in (q, k, v))
+
+
+def _f32(x):
+    return x.to_float32() if isinstance(x, b16.BF16Array) else np.asarray(x, np.float32)
+
+
+CASES = [
+    # B, Hq, Hkv, Sq, Sk, D, causal
+    (1, 1, 1, 16, 16, 16, False), (1, 1, 1, 16, 16, 16, True),
+    (1, 2, 2, 64, 64, 128, False), (1, 2, 2, 64, 64, 128, True),
+    (2, 4, 2, 300, 300, 128, True), (1, 8, 2, 257, 511, 128, True),
+    (2, 4, 1, 256, 512, 128, True), (1, 2, 2, 100, 77, 64, False),
+    (1, 2, 1, 200, 333, 64, True), (1, 2, 2, 333, 200, 64, True),
+    (1, 1, 1, 50, 60, 32, True), (1, 3, 3, 40, 40, 48, False),
+    (1, 2, 2, 1, 129, 128, True), (1, 4, 4, 513, 1, 128, False),
+    (1, 2, 2, 700, 700, 256, True),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal", CASES)
+@pytest.mark.parametrize("st", ["bf16", "f16"])
+def test_attention_matches_oracle(lane, B, Hq, Hkv, Sq, Sk, D, causal, st):
+    q, k, v = _qkv(B, Hq, Hkv, Sq, Sk, D, 17, st)
+    ref_o, ref_lse = orc.flash_attn_dense(_f32(q), _f32(k), _f32(v), causal=causal)
+    o, lse = ops.gqa_attention(q, k, v, causal=causal, return_lse=True, out="f32")
+    assert o.shape == (B, Hq, Sq, D) and lse.shape == (B, Hq, Sq)
+    assert not np.isnan(o).any()
+    assert orc.max_rel_err(o, ref_o) <= TOL
+    assert np.max(np.abs(lse - ref_lse)) <= TOL
+
+
+def test_attention_special_cases(lane):
+    """Closed forms: causal row 0 sees only key 0 -> O[0] = V[0], LSE[0] = s00;
+    identical keys -> uniform weights -> prefix mean of V."""
+    B, H, S, D = 1, 2, 192, 128
+    q, k, v = _qkv(B, H, H, S, S, D, 3, "bf16")
+    o, lse = ops.flash_attn(q, k, v, causal=True, return_lse=True, out="f32")
+    qf, kf, vf = _f32(q), _f32(k), _f32(v)
+    assert np.allclose(o[:, :, 0], vf[:, :, 0], rtol=0, atol=1e-6)
+    s00 = (qf[:, :, 0] * kf[:, :, 0]).sum(-1) / np.sqrt(D)
+    assert np.allclose(lse[:, :, 0], s00, atol=1e-4)
+    k_same = b16.from_float32(np.broadcast_to(kf[:, :, :1], kf.shape).copy())
+    o2 = ops.flash_attn(q, k_same, v, causal=True, out="f32")
+    prefix_mean = np.cumsum(vf.astype(np.float64), axis=2) / np.arange(1, S + 1)[None, None, :, None]
+    assert orc.max_rel_err(o2, prefix_mean) <= TOL
+
+
+def test_gqa_equals_repeated_kv(lane):
+    q, k, v = _qkv(2, 8, 2, 160, 160, 128, 5, "bf16")
+    o_gqa = ops.gqa_attention(q, k, v, causal=True, out="f32")
+    k_rep = b16.from_bits(np.repeat(np.asarray(k, np.uint16), 4, axis=1))
+    v_rep = b16.from_bits(np.repeat(np.asarray(v, np.uint16), 4, axis=1))
+    o_mha = ops.flash_attn(q, k_rep, v_rep, causal=True, out="f32")
+    assert np.array_equal(o_gqa, o_mha)
+    with pytest.raises(ValueError):
+        ops.flash_attn(q, k, v)
+
+
+def test_legacy_signature_and_storage_output(lane):
+    """The MHA-only entry point (call-compatible with the shipped ROCm symbol)
+    and the storage-dtype output."""
+    q, k, v = _qkv(1, 2, 2, 96, 96, 64, 9, "f16")
+    ref_o, _ = orc.flash_attn_dense(_f32(q), _f32(k), _f32(v), causal=True)
+    o = np.empty(q.shape, np.float32)
+    rc = lane.load().tessera_gfx950_flash_attn_f16(
+        q.view(np.uint16).ctypes.data, k.view(np.uint16).ctypes.data, v.view(np.uint16).ctypes.data,
+        o.ctypes.data, 1, 2, 96, 96, 64, float(1 / np.sqrt(64)), 1)
+    assert rc == 0
+    assert orc.max_rel_err(o, ref_o) <= TOL
+    o16 = ops.flash_attn(q, k, v, causal=True)
+    assert o16.dtype == np.float16 and np.array_equal(o16, o.astype(np.float16))
+
+
+def test_headline_config_properties(lane):
+    """B=4 Hq=32 Hkv=8 S=4096 D=128 causal: checked head-by-head against the
+    blockwise oracle on a sample of (batch, head) pairs, plus the row-0 identity
+    on every head."""
+    B, Hq, Hkv, S, D = 4, 32, 8, 4096, 128
+    q, k, v = _qkv(B, Hq, Hkv, S, S, D, 21, "bf16")
+    o, lse = ops.gqa_attention(q, k, v, causal=True, return_lse=True, out="f32")
+    assert not np.isnan(o).any()
+    vf = _f32(v)
+    assert np.allclose(o[:, :, 0], np.repeat(vf[:, :, 0], Hq // Hkv, axis=1), atol=1e-6)
+    pairs = [(0, 0), (1, 13), (3, 31)]
+    ref_o, ref_lse = orc.flash_attn_blockwise(_f32(q), _f32(k), _f32(v), causal=True, heads=pairs,
+                                               dtype=np.float64)
+    for (b, h) in pairs:
+        assert orc.max_rel_err(o[b, h], ref_o[b, h]) <= TOL
+        assert np.max(np.abs(lse[b, h] - ref_lse[b, h])) <= TOL
+
+
+def test_attention_rejects_bad_shapes(lane):
+    lib = lane.load()
+    z = np.zeros(1024, np.uint16)
+    o = np.zeros(1024, np.float32)
+    f = lib.tessera_gfx950_flash_attn_bf16
+    assert f(z.ctypes.data, z.ctypes.data, z.ctypes.data, o.ctypes.data, 1, 1, 8, 8, 20, 1.0, 0) == 1   # D % 16
+    assert f(z.ctypes.data, z.ctypes.data, z.ctypes.data, o.ctypes.data, 1, 1, 0, 8, 16, 1.0, 0) == 1
+    g = lib.tessera_gfx950_flash_attn_gqa_bf16
+    assert g(z.ctypes.data, z.ctypes.data, z.ctypes.data, o.ctypes.data, None, 1, 3, 2, 8, 8, 16, 1.0, 0) == 1

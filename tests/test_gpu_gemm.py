@@ -1,0 +1,148 @@
+"""GEMM parity on the MI355X: HIP kernels (through the C ABI) vs the oracle.
+
+Tolerance: north-star bound max relative error <= 2e-3 for f16/bf16 against an
+fp32-or-better reference (normwise: max|x-ref| / max|ref|).  The f32-output
+entry points are far inside it; the bound is binding for the 16-bit-output
+forms, whose final rounding alone is up to 2^-9 = 1.95e-3.
+"""
+import numpy as np
+import pytest
+
+import tessera_oracle as orc
+from tessera_amd import bf16 as b16
+from tessera_amd import ops
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+def _rand(shape, scale, seed):
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal(shape) * scale).astype(np.float32)
+
+
+@pytest.mark.parametrize("M,N,K", [
+    (16, 16, 16), (32, 16, 32), (128, 256, 64), (256, 256, 128), (300, 520, 200),
+    (512, 1024, 1088), (1, 64, 64), (7, 13, 5), (33, 40, 24), (1024, 1024, 1024),
+])
+@pytest.mark.parametrize("st", ["bf16", "f16"])
+def test_gemm_f32_out_matches_oracle(lane, M, N, K, st):
+    A = _rand((M, K), 0.5, 1)
+    B = _rand((K, N), 0.5, 2)
+    ref = orc.gemm_f64(A, B, st)
+    a = b16.from_float32(A) if st == "bf16" else A.astype(np.float16)
+    b = b16.from_float32(B) if st == "bf16" else B.astype(np.float16)
+    got = ops.gemm(a, b, out="f32")
+    assert got.shape == (M, N) and got.dtype == np.float32
+    assert orc.max_rel_err(got, ref) <= 1e-5
+    # reference test budget: f16 atol 1e-2 (K<=256) / 5e-2 (tests/unit/test_rocm_wmma_runtime_symbol.py:74-89)
+    assert np.max(np.abs(got - ref)) <= (1e-2 if K <= 256 else 5e-2)
+
+
+# Unit roundoff of the storage formats: a value stored in bf16 carries up to 2^-8
+# relative error from the store alone (f16: 2^-11), so a bf16-stored result cannot
+# meet 2e-3 against an fp32 reference elementwise; the bound applies to the f32
+# accumulators, and the stored form must be exactly their correct rounding.
+U_STORE = {"bf16": 2.0 ** -8, "f16": 2.0 ** -11}
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 256, 64), (512, 768, 320), (96, 72, 40)])
+@pytest.mark.parametrize("st", ["bf16", "f16"])
+def test_gemm_storage_out(lane, M, N, K, st):
+    A = _rand((M, K), 1.0 / np.sqrt(K), 3)
+    B = _rand((K, N), 1.0, 4)
+    ref = orc.gemm_f64(A, B, st)
+    a = b16.from_float32(A) if st == "bf16" else A.astype(np.float16)
+    b = b16.from_float32(B) if st == "bf16" else B.astype(np.float16)
+    got = ops.gemm(a, b)
+    gf = got.to_float32() if st == "bf16" else got.astype(np.float32)
+    acc = ops.gemm(a, b, out="f32")
+    assert orc.max_rel_err(acc, ref) <= 1e-5
+    # stored result == RNE(store) of the f32 accumulators, bit for bit
+    assert np.array_equal(gf, orc.round_to_storage(acc, st))
+    assert orc.max_rel_err(gf, ref) <= TOL + U_STORE[st]
+
+
+def test_readme_batched_gemm_config(lane):
+    """A[4,128,64] f16 x W[4,64,256] f16 -> f32 accumulate (README step())."""
+    rng = np.random.default_rng(0)
+    A = (rng.standard_normal((4, 128, 64)) / 8).astype(np.float16)
+    W = (rng.standard_normal((4, 64, 256)) / 8).astype(np.float16)
+    ref = np.matmul(A.astype(np.float64), W.astype(np.float64))
+    got = ops.batched_gemm(A, W, out="f32")
+    assert got.shape == (4, 128, 256)
+    assert orc.max_rel_err(got, ref) <= 1e-5
+    stored = ops.batched_gemm(A, W)
+    assert stored.dtype == np.float16
+    assert np.array_equal(stored, got.astype(np.float16))
+    assert orc.max_rel_err(stored.astype(np.float32), ref) <= TOL
+
+
+def test_gemm_closed_forms(lane):
+    """Identity, ones and a K-ramp: answers known without any reference code."""
+    n = 256
+    eye = b16.from_float32(np.eye(n, dtype=np.float32))
+    rng = np.random.default_rng(5)
+    X = np.round(rng.standard_normal((n, n)) * 8).astype(np.float32)      # bf16-exact integers
+    xb = b16.from_float32(X)
+    assert np.array_equal(ops.gemm(eye, xb, out="f32"), X)
+    assert np.array_equal(ops.gemm(xb, eye, out="f32"), X)
+    ones = b16.from_float32(np.ones((64, 512), np.float32))
+    ramp = b16.from_float32(np.tile((np.arange(512) % 4).astype(np.float32)[:, None], (1, 32)))
+    got = ops.gemm(ones, ramp, out="f32")
+    assert np.all(got == 128 * (0 + 1 + 2 + 3))
+    # transposed-operand guard: A @ B != B^T @ A^T layout mistakes show up on a non-symmetric product
+    A = np.arange(32 * 16, dtype=np.float32).reshape(32, 16) % 7
+    B = np.arange(16 * 48, dtype=np.float32).reshape(16, 48) % 5
+    assert np.array_equal(ops.gemm(b16.from_float32(A), b16.from_float32(B), out="f32"), A @ B)
+
+
+def test_decode_shapes(lane):
+    """M in {1, 16, 128} with N = K = 8192 (HBM-bound decode shapes)."""
+    K = N = 8192
+    B = _rand((K, N), 1.0 / np.sqrt(K), 7)
+    bb = b16.from_float32(B)
+    Bq = bb.to_float32().astype(np.float64)
+    for M in (1, 16, 128):
+        A = _rand((M, K), 1.0, 8 + M)
+        ab = b16.from_float32(A)
+        ref = ab.to_float32().astype(np.float64) @ Bq
+        got = ops.gemm(ab, bb, out="f32")
+        assert orc.max_rel_err(got, ref) <= 1e-5
+
+
+def test_full_size_bf16_gemm_properties(lane):
+    """8192^3 is too large for a CPU product inside the test budget; check
+    size-independent properties instead: linearity in A and agreement with
+    exactly computable rows/columns."""
+    n = 8192
+    rng = np.random.default_rng(11)
+    A = (rng.standard_normal((n, n)) / np.sqrt(n)).astype(np.float32)
+    B = (rng.standard_normal((n, n)) / np.sqrt(n)).astype(np.float32)
+    ab, bb = b16.from_float32(A), b16.from_float32(B)
+    got = ops.gemm(ab, bb, out="f32")
+    Aq, Bq = ab.to_float32().astype(np.float64), bb.to_float32().astype(np.float64)
+    rows = rng.choice(n, 24, replace=False)
+    cols = rng.choice(n, 24, replace=False)
+    assert orc.max_rel_err(got[rows], Aq[rows] @ Bq) <= 1e-5
+    assert orc.max_rel_err(got[:, cols], Aq @ Bq[:, cols]) <= 1e-5
+    # checksum of checksums: ones^T (A B) ones == (ones^T A)(B ones)
+    lhs = float(got.astype(np.float64).sum())
+    rhs = float(Aq.sum(axis=0) @ Bq.sum(axis=1))
+    assert abs(lhs - rhs) <= 1e-6 * max(1.0, np.abs(Aq).sum(axis=0) @ np.abs(Bq).sum(axis=1))
+    # stored bf16 result within the north-star bound on the sampled rows
+    stored = ops.gemm(ab, bb)
+    assert np.array_equal(stored.to_float32(), orc.round_to_storage(got, "bf16"))
+
+
+def test_bad_shapes_rejected(lane):
+    a = b16.from_float32(np.zeros((4, 8), np.float32))
+    b = b16.from_float32(np.zeros((9, 8), np.float32))
+    with pytest.raises(ValueError):
+        ops.gemm(a, b)
+    import ctypes
+    lib = lane.load()
+    z = np.zeros(16, np.uint16)
+    d = np.zeros(16, np.float32)
+    assert lib.tessera_gfx950_gemm_bf16(z.ctypes.data, z.ctypes.data, d.ctypes.data, 0, 4, 4) == 1
+    assert lib.tessera_gfx950_gemm_bf16(z.ctypes.data, z.ctypes.data, d.ctypes.data, 4, -1, 4) == 1
