@@ -1,0 +1,260 @@
+#!/usr/bin/env python3
+"""Headline benchmark of the gfx950 dense-op lane on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input: one
+``D = A . B`` with A, B bf16 8192 x 8192 (entries N(0,1)/sqrt(K), seeded), f32
+accumulate, bf16 output — BASELINE.json's configs[1].  Inputs are resident in
+HBM before the timed region; the timed region is K launches through the C ABI's
+device-pointer entry point, bracketed by a device synchronise on both sides.
+
+One JSON line is printed.  ``roofline`` prices the GEMM kernel against the
+MI355X dense bf16 MFMA peak from its average launch duration, measured with HIP
+events on the launch stream over the same timed region.  ``cpu_baseline`` times
+the oracle's numpy restatement of the reference's CPU path on this host's cores.
+``also`` carries the same measurement for the other kernels of the path
+(flash-attention forward, fp8 / int8 GEMM, decode-shaped GEMM, the MoE expert
+block); they are reported, not part of ``value``.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16/f16 MFMA
+PEAK_FP8_TFLOPS = 5000.0
+PEAK_INT8_TOPS = 5000.0
+PEAK_HBM_GBS = 8000.0
+
+
+def _timed(lane, launch, steps, warmup):
+    """(wall ms/step, event ms/step) for `steps` launches after `warmup`."""
+    for _ in range(warmup):
+        launch()
+    lane.synchronize()
+    timer = lane.DeviceTimer()
+    t0 = time.perf_counter()
+    timer.start()
+    for _ in range(steps):
+        launch()
+    timer.stop()
+    lane.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    ev = timer.elapsed_ms() / steps
+    timer.close()
+    return wall, ev
+
+
+def _bf16(x):
+    from tessera_amd import bf16
+    return np.ascontiguousarray(np.asarray(bf16.from_float32(x), np.uint16))
+
+
+def bench_gemm(lane, M, N, K, steps, warmup, seed=0):
+    rng = np.random.default_rng(seed)
+    A = (rng.standard_normal((M, K), dtype=np.float32) / np.sqrt(K)).astype(np.float32)
+    B = (rng.standard_normal((K, N), dtype=np.float32) / np.sqrt(K)).astype(np.float32)
+    a, b = _bf16(A), _bf16(B)
+    da, db = lane.DeviceBuffer.from_host(a), lane.DeviceBuffer.from_host(b)
+    dd = lane.DeviceBuffer(M * N * 2)
+    fn = lane.load().tessera_gfx950_gemm_bf16_bf16_dev
+
+    def launch():
+        lane.check(fn(da.ptr, db.ptr, dd.ptr, M, N, K, None), "gemm_bf16")
+
+    wall, ev = _timed(lane, launch, steps, warmup)
+    out = dd.download((M, N), np.uint16)
+    for buf in (da, db, dd):
+        buf.close()
+    return wall, ev, (A, B, a, b, out)
+
+
+def bench_attention(lane, steps, warmup):
+    B, Hq, Hkv, S, D = 4, 32, 8, 4096, 128
+    rng = np.random.default_rng(1)
+    q = _bf16(rng.standard_normal((B, Hq, S, D), dtype=np.float32))
+    k = _bf16(rng.standard_normal((B, Hkv, S, D), dtype=np.float32))
+    v = _bf16(rng.standard_normal((B, Hkv, S, D), dtype=np.float32))
+    dq, dk, dv = (lane.DeviceBuffer.from_host(x) for x in (q, k, v))
+    do = lane.DeviceBuffer(q.size * 2)
+    dl = lane.DeviceBuffer(B * Hq * S * 4)
+    fn = lane.load().tessera_gfx950_flash_attn_gqa_bf16_dev
+    scale = 1.0 / np.sqrt(D)
+
+    def launch():
+        lane.check(fn(dq.ptr, dk.ptr, dv.ptr, do.ptr, dl.ptr, B, Hq, Hkv, S, S, D, scale, 1, 1, None), "flash_attn")
+
+    wall, ev = _timed(lane, launch, steps, warmup)
+    for buf in (dq, dk, dv, do, dl):
+        buf.close()
+    flop = 4.0 * B * Hq * (S * (S + 1) / 2) * D          # the reference's causal FLOP model
+    return {"workload": "flash_attn_fwd_bf16_causal_B4_Hq32_Hkv8_S4096_D128", "ms": ev,
+            "tflops": flop / ev / 1e9, "frac_mfma_peak": flop / ev / 1e9 / PEAK_BF16_TFLOPS}
+
+
+def bench_quant(lane, steps, warmup):
+    M, N, K = 4096, 8192, 8192
+    rng = np.random.default_rng(2)
+    out = {}
+    a8 = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    b8 = rng.integers(-127, 128, (K, N)).astype(np.int8)
+    da, db = lane.DeviceBuffer.from_host(a8), lane.DeviceBuffer.from_host(b8)
+    dd = lane.DeviceBuffer(M * N * 4)
+    lib = lane.load()
+    _, ev = _timed(lane, lambda: lane.check(lib.tessera_gfx950_gemm_i8_i32_dev(da.ptr, db.ptr, dd.ptr, M, N, K, None),
+                                            "gemm_i8"), steps, warmup)
+    ops = 2.0 * M * N * K
+    out["gemm_int8_4096x8192x8192"] = {"ms": ev, "tops": ops / ev / 1e9, "frac_mfma_peak": ops / ev / 1e9 / PEAK_INT8_TOPS}
+    # e4m3 codes with |value| <= 15 (no NaN codes)
+    af = ((a8.view(np.uint8) & 0x80) | np.minimum(a8.view(np.uint8) & 0x7F, 0x47)).astype(np.uint8)
+    bf = ((b8.view(np.uint8) & 0x80) | np.minimum(b8.view(np.uint8) & 0x7F, 0x47)).astype(np.uint8)
+    da.upload(af)
+    db.upload(bf)
+    _, ev = _timed(lane, lambda: lane.check(
+        lib.tessera_gfx950_gemm_e4m3_bf16_dev(da.ptr, db.ptr, 1.0, 1.0, dd.ptr, M, N, K, None), "gemm_e4m3"), steps, warmup)
+    out["gemm_fp8_e4m3_4096x8192x8192"] = {"ms": ev, "tflops": ops / ev / 1e9,
+                                           "frac_mfma_peak": ops / ev / 1e9 / PEAK_FP8_TFLOPS}
+    for buf in (da, db, dd):
+        buf.close()
+    return out
+
+
+def bench_decode(lane, steps, warmup):
+    N = K = 8192
+    rng = np.random.default_rng(3)
+    b = _bf16(rng.standard_normal((K, N), dtype=np.float32) / np.sqrt(K))
+    db = lane.DeviceBuffer.from_host(b)
+    out = {}
+    fn = lane.load().tessera_gfx950_gemm_bf16_bf16_dev
+    for M in (1, 16, 128):
+        a = _bf16(rng.standard_normal((M, K), dtype=np.float32))
+        da = lane.DeviceBuffer.from_host(a)
+        dd = lane.DeviceBuffer(M * N * 2)
+        _, ev = _timed(lane, lambda: lane.check(fn(da.ptr, db.ptr, dd.ptr, M, N, K, None), "gemm"), steps, warmup)
+        nbytes = K * N * 2 + M * K * 2 + M * N * 2
+        out[f"gemm_bf16_decode_M{M}_8192x8192"] = {"ms": ev, "gbs": nbytes / ev / 1e6,
+                                                   "frac_hbm_peak": nbytes / ev / 1e6 / PEAK_HBM_GBS}
+        da.close()
+        dd.close()
+    db.close()
+    return out
+
+
+def bench_moe(lane, steps, warmup):
+    T, H, F, E, k = 8192, 4096, 1408, 64, 8
+    rng = np.random.default_rng(4)
+    S = T * k
+    logits = rng.standard_normal((T, E), dtype=np.float32)
+    lib = lane.load()
+    dlog = lane.DeviceBuffer.from_host(logits)
+    dtos, deos, dcw = lane.DeviceBuffer(S * 4), lane.DeviceBuffer(S * 4), lane.DeviceBuffer(S * 4)
+    dgs, dgo, dn = lane.DeviceBuffer(E * 4), lane.DeviceBuffer((E + 1) * 4), lane.DeviceBuffer(4)
+    route = lambda: lane.check(lib.tessera_gfx950_moe_route_f32_dev(
+        dlog.ptr, T, E, k, 1, 0, dtos.ptr, deos.ptr, dcw.ptr, dgs.ptr, dgo.ptr, dn.ptr, None), "route")
+    _, ev_route = _timed(lane, route, steps, warmup)
+    x = _bf16(rng.standard_normal((T, H), dtype=np.float32))
+    dx = lane.DeviceBuffer.from_host(x)
+    dxp = lane.DeviceBuffer(S * H * 2)
+    disp = lambda: lane.check(lib.tessera_gfx950_moe_dispatch_dev(dx.ptr, dtos.ptr, dxp.ptr, T, S, H, 2, None), "dispatch")
+    _, ev_disp = _timed(lane, disp, steps, warmup)
+    w = lambda shape: _bf16(0.02 * rng.standard_normal(shape, dtype=np.float32))
+    dwg, dwu = lane.DeviceBuffer.from_host(w((E, H, F))), lane.DeviceBuffer.from_host(w((E, H, F)))
+    dwd = lane.DeviceBuffer.from_host(w((E, F, H)))
+    dh, dy = lane.DeviceBuffer(S * F * 2), lane.DeviceBuffer(S * H * 2)
+    ffn = lambda: lane.check(lib.tessera_gfx950_moe_swiglu_block_bf16_dev(
+        dxp.ptr, dwg.ptr, dwu.ptr, dwd.ptr, dgo.ptr, dy.ptr, dh.ptr, S, H, F, H, E, None), "swiglu")
+    _, ev_ffn = _timed(lane, ffn, steps, warmup)
+    dout = lane.DeviceBuffer(T * H * 4)
+    comb = lambda: lane.check(lib.tessera_gfx950_moe_combine_bf16_dev(dy.ptr, dtos.ptr, dcw.ptr, dout.ptr, T, S, H, None),
+                              "combine")
+    _, ev_comb = _timed(lane, comb, steps, warmup)
+    for buf in (dlog, dtos, deos, dcw, dgs, dgo, dn, dx, dxp, dwg, dwu, dwd, dh, dy, dout):
+        buf.close()
+    flop = 6.0 * S * H * F
+    return {"workload": "moe_T8192_H4096_E64_top8_F1408_bf16", "route_ms": ev_route, "dispatch_ms": ev_disp,
+            "expert_ffn_ms": ev_ffn, "combine_ms": ev_comb, "expert_ffn_tflops": flop / ev_ffn / 1e9,
+            "frac_mfma_peak": flop / ev_ffn / 1e9 / PEAK_BF16_TFLOPS,
+            "dispatch_gbs": 2.0 * S * H * 2 / ev_disp / 1e6}
+
+
+def cpu_baseline(A, B):
+    """The reference's CPU path for this config is ``np.matmul`` on f32-promoted
+    operands; the oracle restates it.  Timed once on the full workload."""
+    sys.path.insert(0, str(ROOT / "oracle"))
+    import tessera_oracle as orc
+    threads = os.cpu_count() or 1
+    try:
+        from threadpoolctl import threadpool_info
+        blas = [p for p in threadpool_info() if p.get("user_api") == "blas"]
+        if blas:
+            threads = int(blas[0]["num_threads"])
+    except Exception:
+        pass
+    orc.gemm_f32(A[:256], B[:, :256])                         # warm the BLAS pool
+    t0 = time.perf_counter()
+    ref = orc.gemm_f32(A, B)
+    dt = time.perf_counter() - t0
+    M, K = A.shape
+    N = B.shape[1]
+    return ref, {"value": 2.0 * M * N * K / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                 "sample": f"full {M}x{N}x{K} product once, numpy f32 matmul of the bf16-rounded operands, {dt:.2f} s"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only-headline", action="store_true", help="skip the `also` measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X; this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        return 2
+    from tessera_amd import lane
+    lane.load()
+    if not lane.available():
+        print("gfx950 lane unavailable: no MI355X or library not built", file=sys.stderr)
+        return 3
+
+    M = N = K = 8192
+    wall, ev, (A, B, a, b, out) = bench_gemm(lane, M, N, K, args.steps, args.warmup)
+    flop = 2.0 * M * N * K
+    result = {
+        "metric": "TFLOP/s and % MFMA peak: bf16 GEMM 8192^3 + causal flash-attn fwd, 1 MI355X",
+        "value": flop / wall / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (seeded N(0,1)/sqrt(K) operands, resident in HBM)",
+        "config": {"workload": "gemm_bf16_8192x8192x8192_f32acc_bf16out", "M": M, "N": N, "K": K,
+                   "device": lane.device_name()},
+        "roofline": {"bound": "mfma", "achieved": flop / ev / 1e9, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flop / ev / 1e9 / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "gemm16_kernel<BF16,256,256,2,2,STORE16>", "avg_launch_ms": ev},
+    }
+    if not args.no_cpu:
+        ref, result["cpu_baseline"] = cpu_baseline(A, B)
+        got = (out.astype(np.uint32) << 16).view(np.float32)
+        err = float(np.max(np.abs(got - ref)) / np.max(np.abs(ref)))
+        result["parity_max_rel_vs_cpu"] = err                 # includes the bf16 store (<= 2^-8)
+    if not args.only_headline:
+        also = {}
+        s, w = max(3, args.steps // 2), max(2, args.warmup // 2)
+        also["flash_attn"] = bench_attention(lane, s, w)
+        also.update(bench_quant(lane, s, w))
+        also.update(bench_decode(lane, s, w))
+        also["moe"] = bench_moe(lane, s, w)
+        result["also"] = also
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,266 @@
+"""Pins for the numpy oracle: library routines, closed forms, brute force and
+the published format tables — chosen so that a dropped term, a wrong sign or a
+transposed operand in the oracle fails one of them.  No GPU."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import tessera_oracle as orc
+
+
+# ---- bf16 rounding ------------------------------------------------------------------
+
+def test_bf16_round_trip_and_ties():
+    codes = np.arange(1 << 16, dtype=np.uint16)
+    vals = orc.bf16_bits_to_f32(codes)
+    finite = np.isfinite(vals)
+    assert np.array_equal(orc.f32_to_bf16_bits(vals[finite]), codes[finite])
+    # ties: 1 + 2^-8 is halfway between 1 (even mantissa) and 1 + 2^-7 -> rounds to 1;
+    # 1 + 3*2^-8 is halfway between 1+2^-7 (odd) and 1+2^-6 (even) -> rounds up.
+    x = np.array([1 + 2.0 ** -8, 1 + 3 * 2.0 ** -8, -(1 + 2.0 ** -8), 1 + 2.0 ** -8 + 2.0 ** -20], np.float32)
+    got = orc.bf16_bits_to_f32(orc.f32_to_bf16_bits(x))
+    assert list(got) == [1.0, 1 + 2.0 ** -6, -1.0, 1 + 2.0 ** -7]
+
+
+def test_bf16_matches_torch():
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal(200000) * np.exp(rng.uniform(-30, 30, 200000))).astype(np.float32)
+    ours = orc.round_to_storage(x, "bf16")
+    theirs = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(ours, theirs)
+    assert np.array_equal(orc.round_to_storage(x, "f16"), x.astype(np.float16).astype(np.float32))
+
+
+# ---- GEMM -----------------------------------------------------------------------------
+
+def test_gemm_closed_forms_and_orientation():
+    A = (np.arange(6 * 4) % 5).astype(np.float32).reshape(6, 4)
+    B = (np.arange(4 * 3) % 7).astype(np.float32).reshape(4, 3)
+    brute = np.array([[sum(A[i, k] * B[k, j] for k in range(4)) for j in range(3)] for i in range(6)])
+    assert np.array_equal(orc.gemm_f32(A, B), brute)
+    assert np.array_equal(orc.gemm_f64(A, B), brute)
+    # operands are rounded to storage BEFORE the product
+    a = np.array([[1 + 2.0 ** -10]], np.float32)
+    assert orc.gemm_f32(a, np.array([[1024.0]], np.float32))[0, 0] == 1024.0
+    assert orc.gemm_f32(a, np.array([[1024.0]], np.float32), "f16")[0, 0] == 1025.0
+    # storage rule re-rounds the result; batched leading dims broadcast like np.matmul
+    x = np.array([[1.0, 2.0 ** -9]], np.float32)
+    y = np.array([[1.0], [1.0]], np.float32)
+    assert orc.gemm_f32(x, y)[0, 0] == 1 + 2.0 ** -9
+    assert orc.gemm_storage(x, y)[0, 0] == 1.0
+    rng = np.random.default_rng(1)
+    Ab = rng.standard_normal((4, 8, 16)).astype(np.float32)
+    Bb = rng.standard_normal((4, 16, 8)).astype(np.float32)
+    got = orc.gemm_f32(Ab, Bb, "f16")
+    for i in range(4):
+        assert np.allclose(got[i], orc.gemm_f32(Ab[i], Bb[i], "f16"))
+
+
+# ---- attention --------------------------------------------------------------------------
+
+def _brute_attention(q, k, v, scale, causal):
+    B, Hq, Sq, D = q.shape
+    Hkv, Sk = k.shape[1], k.shape[2]
+    off = max(Sk - Sq, 0)
+    O = np.zeros((B, Hq, Sq, D))
+    L = np.zeros((B, Hq, Sq))
+    for b in range(B):
+        for h in range(Hq):
+            kh = h // (Hq // Hkv)
+            for i in range(Sq):
+                js = [j for j in range(Sk) if (not causal) or j <= i + off]
+                s = [scale * float(np.dot(q[b, h, i].astype(np.float64), k[b, kh, j])) for j in js]
+                m = max(s)
+                e = [math.exp(x - m) for x in s]
+                z = sum(e)
+                O[b, h, i] = sum(ei / z * v[b, kh, j].astype(np.float64) for ei, j in zip(e, js))
+                L[b, h, i] = m + math.log(z)
+    return O, L
+
+
+@pytest.mark.parametrize("Sq,Sk,causal", [(5, 5, False), (5, 5, True), (3, 7, True), (7, 3, True)])
+def test_attention_against_brute_force(Sq, Sk, causal):
+    rng = np.random.default_rng(2)
+    q = rng.standard_normal((2, 4, Sq, 8)).astype(np.float32)
+    k = rng.standard_normal((2, 2, Sk, 8)).astype(np.float32)
+    v = rng.standard_normal((2, 2, Sk, 8)).astype(np.float32)
+    bo, bl = _brute_attention(q, k, v, 0.3, causal)
+    o, lse = orc.flash_attn_dense(q, k, v, scale=0.3, causal=causal)
+    assert np.allclose(o, bo, atol=1e-12) and np.allclose(lse, bl, atol=1e-12)
+    o2, lse2 = orc.flash_attn_blockwise(q, k, v, scale=0.3, causal=causal, block=2, dtype=np.float64)
+    assert np.allclose(o2, bo, atol=1e-12) and np.allclose(lse2, bl, atol=1e-12)
+
+
+def test_attention_matches_torch_sdpa_and_gqa_repeat():
+    rng = np.random.default_rng(3)
+    q = rng.standard_normal((2, 8, 33, 16)).astype(np.float32)
+    k = rng.standard_normal((2, 2, 33, 16)).astype(np.float32)
+    v = rng.standard_normal((2, 2, 33, 16)).astype(np.float32)
+    o, _ = orc.flash_attn_dense(q, k, v, causal=True)
+    kr, vr = np.repeat(k, 4, axis=1), np.repeat(v, 4, axis=1)        # nn/functional.py:349-356
+    o_rep, _ = orc.flash_attn_dense(q, kr, vr, causal=True)
+    assert np.array_equal(o, o_rep)
+    t = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(q).double(), torch.from_numpy(kr).double(), torch.from_numpy(vr).double(), is_causal=True)
+    assert np.allclose(o, t.numpy(), atol=1e-10)
+    o_nc, _ = orc.flash_attn_dense(q, kr, vr, causal=False, scale=0.5)
+    t2 = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(q).double(), torch.from_numpy(kr).double(), torch.from_numpy(vr).double(), scale=0.5)
+    assert np.allclose(o_nc, t2.numpy(), atol=1e-10)
+
+
+def test_attention_region_reference_is_top_left_causal():
+    rng = np.random.default_rng(4)
+    Q, K, V = (rng.standard_normal((8, 16)).astype(np.float32) * .2 for _ in range(3))
+    ref = orc.attention_region_reference(Q, K, V, scale=0.7, causal=True)
+    o, _ = orc.flash_attn_dense(Q[None, None], K[None, None], V[None, None], scale=0.7, causal=True)
+    assert np.allclose(ref, o[0, 0], atol=1e-6)
+
+
+# ---- MoE --------------------------------------------------------------------------------
+
+def _brute_route(scores, k, normalize, capacity):
+    T, E = scores.shape
+    slots = []
+    fill = [0] * E
+    for t in range(T):
+        s = scores[t].astype(np.float32)
+        e = np.exp(s - s.max())
+        p = e / e.sum()
+        order = sorted(range(E), key=lambda i: (-float(p[i]), i))[:k]
+        w = np.array([p[i] for i in order], np.float32)
+        if normalize and k > 1:
+            w = w / w.sum()
+        for j, ex in enumerate(order):
+            if capacity is not None and fill[ex] >= capacity:
+                continue
+            fill[ex] += 1
+            slots.append((ex, t, float(w[j])))
+    slots.sort(key=lambda x: x[0])                       # stable by expert
+    return slots
+
+
+@pytest.mark.parametrize("T,E,k,cap", [(6, 4, 2, None), (9, 3, 3, None), (12, 4, 2, 3), (5, 5, 1, 1)])
+def test_routing_against_brute_force(T, E, k, cap):
+    rng = np.random.default_rng(T * 7 + E)
+    lg = rng.standard_normal((T, E)).astype(np.float32)
+    r = orc.route_tokens(lg, E, k, capacity=cap if cap is not None else 10 ** 9)
+    d = orc.plan_dispatch(r.assignment, r.weights, E)
+    brute = _brute_route(lg, k, True, cap)
+    assert [s[1] for s in brute] == list(d.token_of_slot)
+    assert [s[0] for s in brute] == list(d.expert_of_slot)
+    assert np.allclose([s[2] for s in brute], d.combine_weights, rtol=1e-6)
+    assert r.overflow == T * k - len(brute)
+    assert np.array_equal(d.group_offsets, np.concatenate(([0], np.cumsum(d.group_sizes))))
+    assert np.array_equal(r.load, np.bincount(orc.topk_desc_lowest_index(orc.router_probs(lg), k).ravel(), minlength=E))
+
+
+def test_the_two_routers_pick_the_same_experts():
+    """softmax is monotonic, so top-k of the probabilities (route_tokens) and
+    top-k of the logits (route_top_k) select the same expert set absent ties;
+    with normalisation both weight vectors are the softmax over the selection."""
+    rng = np.random.default_rng(5)
+    lg = rng.standard_normal((500, 16)).astype(np.float32)
+    assert not orc.has_routing_ties(orc.router_probs(lg), 4)
+    r = orc.route_tokens(lg, 16, 4)
+    ids, w = orc.route_top_k_stable(lg, 4)
+    assert np.array_equal(np.sort(r.assignment, 1), np.sort(ids, 1))
+    assert np.array_equal(r.assignment, ids)
+    assert np.allclose(r.weights, w, rtol=2e-6)
+    assert np.allclose(r.weights.sum(1), 1.0, atol=1e-6)
+
+
+def test_packing_invariants_and_round_trip():
+    rng = np.random.default_rng(6)
+    lg = rng.standard_normal((300, 8)).astype(np.float32)
+    r = orc.route_tokens(lg, 8, 2)
+    d = orc.plan_dispatch(r.assignment, r.weights, 8)
+    assert int(d.group_sizes.sum()) == 600
+    assert np.all(np.diff(d.expert_of_slot) >= 0)
+    for e in range(8):
+        seg = d.token_of_slot[d.group_offsets[e]:d.group_offsets[e + 1]]
+        assert np.all(np.diff(seg) > 0)
+    inv = np.empty_like(d.sort_perm)
+    inv[d.sort_perm] = np.arange(600)
+    assert np.array_equal(d.sort_perm[inv], np.arange(600))          # models/moe_routing.py:47-51
+    # dispatch then combine with unit expert (identity FFN) returns sum_k w * x = x
+    x = rng.standard_normal((300, 5)).astype(np.float32)
+    y = x[d.token_of_slot]
+    back = orc.moe_combine(y, d, 300)
+    assert np.allclose(back, x, atol=1e-6)
+
+
+def test_grouped_gemm_and_swiglu_reductions():
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((10, 6)).astype(np.float32)
+    w = rng.standard_normal((3, 6, 4)).astype(np.float32)
+    sizes = [4, 0, 6]
+    got = orc.grouped_gemm(x, w, sizes, store=False)
+    xq, wq = orc.round_to_storage(x, "bf16"), orc.round_to_storage(w, "bf16")
+    assert np.allclose(got[:4], xq[:4].astype(np.float64) @ wq[0])
+    assert np.allclose(got[4:], xq[4:].astype(np.float64) @ wq[2])
+    with pytest.raises(ValueError):
+        orc.grouped_gemm(x, w, [4, 1, 6])
+    # E = 1 reduces to the dense SwiGLU MLP with the same storage roundings
+    wg, wu = rng.standard_normal((1, 6, 8)).astype(np.float32), rng.standard_normal((1, 6, 8)).astype(np.float32)
+    wd = rng.standard_normal((1, 8, 5)).astype(np.float32)
+    blk = orc.moe_swiglu_block(x, wg, wu, wd, [10])
+    g, u = orc.gemm_storage(x, wg[0]), orc.gemm_storage(x, wu[0])
+    h = orc.round_to_storage(orc.silu_mul(g, u), "bf16")
+    assert np.array_equal(blk, orc.gemm_storage(h, wd[0]))
+    a = np.array([0.0, 1.0, -2.0], np.float32)
+    assert np.allclose(orc.silu_mul(a, np.ones(3, np.float32)), a / (1 + np.exp(-a)))
+
+
+# ---- quantisation -------------------------------------------------------------------------
+
+def test_e4m3_table_matches_torch_and_spec():
+    table = orc.e4m3_decode_table()
+    t = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    assert np.array_equal(np.isnan(table), np.isnan(t))
+    assert np.array_equal(table[~np.isnan(table)], t[~np.isnan(t)])
+    assert table[0x7E] == 448.0 and table[0x01] == 2.0 ** -9 and table[0x08] == 2.0 ** -6 and table[0x38] == 1.0
+
+
+def test_e4m3_rounding_matches_torch_cast():
+    rng = np.random.default_rng(8)
+    x = np.concatenate([rng.standard_normal(100000) * 100, rng.standard_normal(100000) * 0.01,
+                        np.linspace(-448, 448, 50001), [0.0, -0.0, 2.0 ** -10, 3 * 2.0 ** -10, 447.9, 448.0]])
+    x = np.clip(x, -448, 448).astype(np.float32)
+    grid = orc.fpquant_grid(x)
+    tq = torch.from_numpy(x).to(torch.float8_e4m3fn)
+    assert np.array_equal(grid, tq.to(torch.float32).numpy())
+    assert np.array_equal(orc.e4m3_encode(grid) & 0x7F, tq.view(torch.uint8).numpy() & 0x7F)
+    table = orc.e4m3_decode_table()
+    assert np.array_equal(table[orc.e4m3_encode(grid)], grid)
+
+
+def test_quantize_fp8_scale_and_saturation():
+    x = np.array([0.5, -2.0, 896.0, 1e-9], np.float32)
+    codes, grid, scale = orc.quantize_fp8_e4m3(x)
+    assert scale == np.float32(2.0) and grid[2] == 448.0 and grid[1] == -1.0
+    z_codes, z_grid, z_scale = orc.quantize_fp8_e4m3(np.zeros(4, np.float32))
+    assert z_scale == np.float32(1e-12) and not z_grid.any()          # amax floor
+    c, g, s = orc.quantize_fp8_e4m3(np.array([1e6, -1e6], np.float32), scale=1.0)
+    assert list(c) == [0x7E, 0xFE]                                     # tests/unit/test_phase_e_f.py:498-511
+
+
+def test_int8_quantiser_and_w8a8():
+    M = np.array([[1.0, -2.0, 0.5], [0.0, 0.0, 0.0], [127.0, 63.5, -64.5]], np.float32)
+    q, s = orc.quantize_int8_per_channel(M, axis=1)
+    assert np.allclose(s[:, 0], [2 / 127, 1e-12 / 127, 1.0])
+    assert list(q[0]) == [64, -127, 32] and list(q[2]) == [127, 64, -64]   # half-to-even
+    qc, sc = orc.quantize_int8_per_channel(M, axis=0)
+    assert sc.shape == (1, 3) and np.allclose(sc[0], [1.0, 63.5 / 127, 64.5 / 127])
+    rng = np.random.default_rng(9)
+    X = rng.standard_normal((7, 11)).astype(np.float32)
+    W = rng.standard_normal((11, 5)).astype(np.float32)
+    y, acc, xq, a_s, wq, w_s = orc.w8a8_matmul(X, W)
+    brute = np.array([[sum(int(xq[i, k]) * int(wq[k, j]) for k in range(11)) for j in range(5)] for i in range(7)])
+    assert np.array_equal(acc, brute)
+    assert np.array_equal(y, acc.astype(np.float32) * a_s * w_s[None, :])
+    assert orc.max_rel_err(y, X @ W) < 0.05
+    big = np.full((2, 70000), 127, np.int8)
+    assert orc.gemm_i8_i32(big, big.T.copy())[0, 0] == 127 * 127 * 70000
