@@ -63,7 +63,19 @@ struct Gemm16Params {
 
 constexpr int G16_BK = 64;          // K step, elements
 constexpr int G16_APITCH = 128;     // bytes per A row in LDS
-constexpr int G16_BPAD = 16;        // B row pad, elements
+#ifndef TSR_BPAD
+#define TSR_BPAD 32
+#endif
+#ifndef TSR_ASWZ
+#define TSR_ASWZ(row) (((row) >> 1) & 7)
+#endif
+#ifndef TSR_EARLY_GLOAD
+#define TSR_EARLY_GLOAD 0
+#endif
+#ifndef TSR_WRITES_LATE
+#define TSR_WRITES_LATE 0
+#endif
+constexpr int G16_BPAD = TSR_BPAD;  // B row pad, elements
 
 template <int BM, int BN>
 struct Gemm16Smem {
@@ -163,10 +175,14 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
 #pragma unroll
   for (int q = 0; q < A_CHUNKS; ++q) {
     const int row = (tid >> 3) + (NT / 8) * q;
+#ifdef TSR_ABL_SAMETILE
+    int gr = row;
+#else
     int gr = m_begin + row;
+#endif
     gr = gr < m_end ? gr : m_end - 1;            // clamp: rows past the edge are never stored
     a_ptr[q] = Ab + (long)gr * p.lda + a_chunk * 8;
-    a_lds[q] = row * G16_APITCH + ((a_chunk ^ (row & 7)) << 4);
+    a_lds[q] = row * G16_APITCH + ((a_chunk ^ TSR_ASWZ(row)) << 4);
   }
   // B: chunk v = tid + NT*q -> k row v/(BN/8), n chunk v%(BN/8).
   const uint16_t* b_ptr[B_CHUNKS];
@@ -182,46 +198,75 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     if constexpr (SWIGLU) {
       if (col >= BN / 2) { src = B2b; col -= BN / 2; }
     }
+#ifdef TSR_ABL_SAMETILE
+    int gc = col;
+#else
     int gc = n_begin + col;
+#endif
     gc = gc < p.N ? gc : (p.N - 8);              // clamp: columns past the edge are never stored
     b_ptr[q] = src + (long)krow * p.ldb + gc;
     b_lds[q] = S::kAStage + krow * S::kBPitch + nch * 16;
     b_krow[q] = krow;
   }
 
-  uint4 ra[A_CHUNKS], rb[B_CHUNKS];
-  // Global -> register prefetch of the K step starting at k0.  The guarded form
-  // is for a step that may be partial: out-of-range K must contribute exact
-  // zeros on both operands, so the load address is pulled back in range and the
-  // value replaced.  Only the last step can be partial; the hot loop uses the
-  // plain form.
-  auto gload = [&](int k0, auto guarded_c) {
-    if constexpr (!decltype(guarded_c)::value) {
-#pragma unroll
-      for (int q = 0; q < A_CHUNKS; ++q) ra[q] = *reinterpret_cast<const uint4*>(a_ptr[q] + k0);
-#pragma unroll
-      for (int q = 0; q < B_CHUNKS; ++q) rb[q] = *reinterpret_cast<const uint4*>(b_ptr[q] + (long)k0 * p.ldb);
-    } else {
-#pragma unroll
-      for (int q = 0; q < A_CHUNKS; ++q) {
+  // ---- staging registers ------------------------------------------------------
+  // st[q] holds one 16-byte chunk on its way from global memory to LDS:
+  // q < A_CHUNKS is A chunk q, the rest are B chunks.  The chunks of a K step are
+  // split into KS groups; a group is written to LDS and immediately refilled with
+  // the same chunks of the K step two ahead, so every global load has a full K
+  // step of MFMA time to land and loads / LDS writes are spread evenly over it.
+  constexpr int KS = G16_BK / 16;
+  constexpr int NC = A_CHUNKS + B_CHUNKS;
+  static_assert(NC % KS == 0, "chunks must split evenly over the k steps");
+  constexpr int CPG = NC / KS;
+  uint4 st[NC];
+  using std::true_type;
+  using std::false_type;
+  // Load chunk q of the K step starting at k0.  The guarded form is for a step
+  // that may be partial: out-of-range K must contribute exact zeros on both
+  // operands, so the address is pulled back in range and the value replaced.
+  auto gload1 = [&](int q, int k0, auto guarded_c) {
+#ifdef TSR_ABL_NOGLOAD
+    if (k0 > 0) return;
+#endif
+    constexpr bool GUARD = decltype(guarded_c)::value;
+    if (q < A_CHUNKS) {
+      if constexpr (!GUARD) {
+        st[q] = *reinterpret_cast<const uint4*>(a_ptr[q] + k0);
+      } else {
         const bool ok = k0 + a_chunk * 8 < K;
         const uint4 v = *reinterpret_cast<const uint4*>(a_ptr[q] + (ok ? k0 : -(a_chunk * 8)));
-        ra[q].x = ok ? v.x : 0u; ra[q].y = ok ? v.y : 0u; ra[q].z = ok ? v.z : 0u; ra[q].w = ok ? v.w : 0u;
+        st[q].x = ok ? v.x : 0u; st[q].y = ok ? v.y : 0u; st[q].z = ok ? v.z : 0u; st[q].w = ok ? v.w : 0u;
       }
-#pragma unroll
-      for (int q = 0; q < B_CHUNKS; ++q) {
-        const bool ok = k0 + b_krow[q] < K;
-        const uint4 v = *reinterpret_cast<const uint4*>(b_ptr[q] + (ok ? (long)k0 : -(long)b_krow[q]) * p.ldb);
-        rb[q].x = ok ? v.x : 0u; rb[q].y = ok ? v.y : 0u; rb[q].z = ok ? v.z : 0u; rb[q].w = ok ? v.w : 0u;
+    } else {
+      const int qb = q - A_CHUNKS;
+      if constexpr (!GUARD) {
+        st[q] = *reinterpret_cast<const uint4*>(b_ptr[qb] + (long)k0 * p.ldb);
+      } else {
+        const bool ok = k0 + b_krow[qb] < K;
+        const uint4 v = *reinterpret_cast<const uint4*>(b_ptr[qb] + (ok ? (long)k0 : -(long)b_krow[qb]) * p.ldb);
+        st[q].x = ok ? v.x : 0u; st[q].y = ok ? v.y : 0u; st[q].z = ok ? v.z : 0u; st[q].w = ok ? v.w : 0u;
       }
     }
   };
-  auto lstore = [&](int buf) {
+  auto lstore1 = [&](int q, int buf) {
+#ifdef TSR_ABL_NOLSTORE
+    return;
+#endif
     char* base = smem + buf * S::kStage;
+    if (q < A_CHUNKS) lds_write_b128(base, a_lds[q], st[q]);
+    else lds_write_b128(base, b_lds[q - A_CHUNKS], st[q]);
+  };
+  // Group g: write its chunks (K step `write` done by the caller's choice of
+  // buffer) and refill them.  MODE 0 = no refill, 1 = full step, 2 = guarded.
+  auto stream_group = [&](int g, int buf_dst, int k0_load, auto mode_c) {
+    constexpr int MODE = decltype(mode_c)::value;
 #pragma unroll
-    for (int q = 0; q < A_CHUNKS; ++q) lds_write_b128(base, a_lds[q], ra[q]);
-#pragma unroll
-    for (int q = 0; q < B_CHUNKS; ++q) lds_write_b128(base, b_lds[q], rb[q]);
+    for (int q = g * CPG; q < (g + 1) * CPG; ++q) {
+      lstore1(q, buf_dst);
+      if constexpr (MODE == 1) gload1(q, k0_load, false_type{});
+      if constexpr (MODE == 2) gload1(q, k0_load, true_type{});
+    }
   };
 
   // ---- operand read addressing --------------------------------------------
@@ -232,7 +277,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   for (int i = 0; i < MI; ++i) {
     const int row = wm * TM + i * 32 + l32;
     a_rd[i] = row * G16_APITCH;
-    a_sw[i] = row & 7;
+    a_sw[i] = TSR_ASWZ(row);
   }
   // transposing read: lane supplies row (k) = 8*lh + r/4 (+4 for the second
   // half), columns n = 32j + 16*((lane>>4)&1) + 4*(r%4), r = lane & 15.
@@ -252,6 +297,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   // step s+1 are issued before the MFMAs of step s, which hide their latency.
   uint4 af[2][MI], bf[2][NJ];
   auto frag_load = [&](int buf, int ks, int slot) {
+#ifdef TSR_ABL_NOFRAG
+    if (ks > 0 || buf > 0) return;
+#endif
     const char* base = smem + buf * S::kStage;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
@@ -265,80 +313,94 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     }
   };
   auto mma = [&](int slot) {
-#ifdef TSR_WAIT_LGKM0
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-#endif
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < NJ; ++j) acc[i][j] = mfma_32x32x16<T>(bf[slot][j], af[slot][i], acc[i][j]);
   };
-  // Scheduling hint: pair every LDS read with an MFMA so the reads issue in the
-  // shadow of the matrix pipe instead of in a burst in front of it.
-  auto interleave_reads = [&]() {
+  // Scheduling hint for one k step of NM MFMAs that carries RD operand reads and
+  // (when `stream`) CPG LDS writes + CPG global loads.  The writes cannot pass
+  // the reads (the compiler cannot prove the two LDS buffers disjoint), so the
+  // reads ride the first MFMAs and the write/load pairs the last ones; every
+  // memory instruction issues in the shadow of an MFMA instead of in a burst.
+  constexpr int NM = MI * NJ, RD = MI + 2 * NJ;
+  auto hint_step = [&](auto stream_c, auto loads_c) {
+    constexpr bool STREAM = decltype(stream_c)::value;
+    constexpr bool LOADS = decltype(loads_c)::value;
+    if constexpr (NM >= 4) {
+      constexpr int WSLOTS = CPG < NM / 2 ? CPG : NM / 2;
+      constexpr int wslots = STREAM ? WSLOTS : 0;
+      constexpr int rslots = NM - wslots;
+      constexpr int rper = (RD + rslots - 1) / rslots;
+      constexpr int wper = (CPG + WSLOTS - 1) / WSLOTS;
 #pragma unroll
-    for (int x = 0; x < MI + 2 * NJ; ++x) {
-      TSR_SGB(0x008, 1, 0);   // 1 MFMA
-      TSR_SGB(0x100, 1, 0);   // 1 DS read
+      for (int x = 0; x < NM; ++x) {
+        TSR_SGB(0x008, 1, 0);
+        if (x < rslots) {
+          TSR_SGB(0x100, rper, 0);
+        } else {
+          TSR_SGB(0x200, wper, 0);
+          if constexpr (LOADS) TSR_SGB(0x020, wper, 0);
+        }
+      }
     }
   };
 
-  constexpr int KS = G16_BK / 16;
   const int ktiles = (K + G16_BK - 1) / G16_BK;
-  using std::true_type;
-  using std::false_type;
-  using no_prefetch = std::integral_constant<int, 0>;
-  using full_prefetch = std::integral_constant<int, 1>;
-  using tail_prefetch = std::integral_constant<int, 2>;
-  gload(0, true_type{});
-  lstore(0);
+  using mode0 = std::integral_constant<int, 0>;
+  using mode1 = std::integral_constant<int, 1>;
+  using mode2 = std::integral_constant<int, 2>;
+
+  // ---- prologue: K step 0 in buffer 0, group 0 of step 1 in buffer 1, the rest
+  // of step 1 and group 0 of step 2 in registers -------------------------------
+#pragma unroll
+  for (int q = 0; q < NC; ++q) gload1(q, 0, true_type{});
+#pragma unroll
+  for (int q = 0; q < NC; ++q) lstore1(q, 0);
+  if (ktiles > 1) {
+#pragma unroll
+    for (int q = 0; q < NC; ++q) gload1(q, G16_BK, true_type{});
+    if (ktiles > 2) stream_group(0, 1, 2 * G16_BK, mode2{});
+    else stream_group(0, 1, 0, mode0{});
+  }
   __syncthreads();
-  if (ktiles > 1) gload(G16_BK, true_type{});
   frag_load(0, 0, 0);
 
-  // One K step.  MORE: another step follows (its tile is in registers and goes to
-  // the other LDS buffer now).  PREFETCH: the step after that exists and is
-  // fetched from global memory (1 = known full tile, 2 = possibly partial).
-  // Both are compile-time so the body is one straight-line block.
-  auto kstep = [&](int kt, auto more_c, auto prefetch_c) {
-    constexpr bool MORE = decltype(more_c)::value;
-    constexpr int PREFETCH = decltype(prefetch_c)::value;
+  // One K step.  HAS1: step kt+1 exists (its groups 1.. go to the other buffer
+  // during k steps 0..KS-2).  L2 / L3: how steps kt+2 / kt+3 are fetched
+  // (0 absent, 1 full, 2 possibly partial).  All compile-time: the body is one
+  // straight-line block per barrier interval.
+  auto kstep = [&](int kt, auto has1_c, auto l2_c, auto l3_c) {
+    constexpr bool HAS1 = decltype(has1_c)::value;
+    constexpr int L2 = decltype(l2_c)::value;
+    constexpr int L3 = decltype(l3_c)::value;
     const int buf = kt & 1;
 #pragma unroll
     for (int ks = 0; ks < KS - 1; ++ks) {
       frag_load(buf, ks + 1, (ks + 1) & 1);
-      if (MORE && ks == KS - 2) lstore(buf ^ 1);
+      if constexpr (HAS1) stream_group(ks + 1, buf ^ 1, (kt + 2) * G16_BK, l2_c);
       mma(ks & 1);
-      if (MORE && ks == KS - 2) {
-#pragma unroll
-        for (int x = 0; x < MI + 2 * NJ; ++x) {
-          TSR_SGB(0x008, 1, 0);
-          TSR_SGB(0x100, 1, 0);
-          TSR_SGB(0x200, (A_CHUNKS + B_CHUNKS + MI + 2 * NJ - 1) / (MI + 2 * NJ), 0);
-        }
-      } else {
-        interleave_reads();
-      }
+      hint_step(std::integral_constant<bool, HAS1>{}, std::integral_constant<bool, (L2 != 0)>{});
       TSR_SB();
     }
-    // All of this wave's reads of the current buffer are issued; once every wave
-    // passes the barrier the other buffer is complete and this one is free.
+    // Every wave has issued all its reads of this buffer and all its writes of
+    // the other one; past the barrier the other buffer is complete and this one
+    // is free to take group 0 of step kt+2.
+#ifndef TSR_ABL_NOBARRIER
     __syncthreads();
-    if constexpr (MORE) {
-      if constexpr (PREFETCH == 1) gload((kt + 2) * G16_BK, false_type{});
-      if constexpr (PREFETCH == 2) gload((kt + 2) * G16_BK, true_type{});
-      frag_load(buf ^ 1, 0, KS & 1);
-    }
+#endif
+    if constexpr (HAS1) frag_load(buf ^ 1, 0, KS & 1);
+    if constexpr (L2 != 0) stream_group(0, buf, (kt + 3) * G16_BK, l3_c);
     mma((KS - 1) & 1);
-    if constexpr (MORE) interleave_reads();
+    if constexpr (HAS1) hint_step(std::integral_constant<bool, (L2 != 0)>{}, std::integral_constant<bool, (L3 != 0)>{});
     TSR_SB();
   };
   int kt = 0;
-  // Tile kt+2 <= ktiles-2 is always a full tile; only the last one can be partial.
-  for (; kt + 3 < ktiles; ++kt) kstep(kt, true_type{}, full_prefetch{});
-  if (kt + 2 < ktiles) { kstep(kt, true_type{}, tail_prefetch{}); ++kt; }
-  if (kt + 1 < ktiles) { kstep(kt, true_type{}, no_prefetch{}); ++kt; }
-  kstep(kt, false_type{}, no_prefetch{});
+  for (; kt + 4 < ktiles; ++kt) kstep(kt, true_type{}, mode1{}, mode1{});
+  if (kt + 3 < ktiles) { kstep(kt, true_type{}, mode1{}, mode2{}); ++kt; }
+  if (kt + 2 < ktiles) { kstep(kt, true_type{}, mode2{}, mode0{}); ++kt; }
+  if (kt + 1 < ktiles) { kstep(kt, true_type{}, mode0{}, mode0{}); ++kt; }
+  kstep(kt, false_type{}, mode0{}, mode0{});
 
   // ---- epilogue -------------------------------------------------------------
   // acc[i][j][r]: row m = 32i + l32, col n = 32j + 8*(r/4) + 4*lh + (r%4).
