@@ -25,8 +25,8 @@ int launch_flash(const FlashParams& p, hipStream_t s) {
                                    hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   });
   if (attr_err != hipSuccess) return kDeviceFailed;
-  dim3 grid(ceil_div(p.Sq, FA_BQ), p.B * p.Hq, 1);
-  hipLaunchKernelGGL(kern, grid, dim3(256), kSmem, s, p);
+  dim3 grid(ceil_div(p.Sq, FA_BQ) * p.B * p.Hq, 1, 1);
+  hipLaunchKernelGGL(kern, grid, dim3(FA_THREADS), kSmem, s, p);
   return launch_status();
 }
 

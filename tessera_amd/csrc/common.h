@@ -26,11 +26,9 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 struct BF16 {};
 struct F16 {};
 
-// f32 -> bf16 bits, round-to-nearest-even (NaN kept quiet).
+// f32 -> bf16 bits, round-to-nearest-even (the hardware conversion, v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-  return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
   return __builtin_bit_cast(float, (uint32_t)b << 16);
@@ -50,9 +48,18 @@ template <class T> __device__ __forceinline__ float from_storage(uint16_t b);
 template <> __device__ __forceinline__ float from_storage<BF16>(uint16_t b) { return bf16_bits_to_f32(b); }
 template <> __device__ __forceinline__ float from_storage<F16>(uint16_t b) { return f16_bits_to_f32(b); }
 
-// Two f32 -> one dword of two storage values (lo = a, hi = b).
-template <class T> __device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return (uint32_t)to_storage<T>(a) | ((uint32_t)to_storage<T>(b) << 16);
+// Two f32 -> one dword of two storage values (lo = a, hi = b), one packed convert.
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+template <class T> __device__ __forceinline__ uint32_t pack2(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack2<BF16>(float a, float b) {
+  const f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+template <> __device__ __forceinline__ uint32_t pack2<F16>(float a, float b) {
+  const f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
 }
 
 // 32x32x16 MFMA on 16-bit operands held as raw 128-bit registers.

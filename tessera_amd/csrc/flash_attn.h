@@ -1,9 +1,10 @@
 // Flash-attention forward for gfx950: O = softmax(scale * Q K^T, causal) V with
 // GQA and the per-row log-sum-exp, 16-bit storage, f32 softmax and accumulate.
 //
-// One workgroup (4 waves, one per SIMD) owns 256 query rows of one (batch, q
-// head); each wave owns 64 of them as two 32-row MFMA tiles.  K/V are walked in
-// 64-key tiles staged through LDS (double buffered, one barrier per tile).
+// One workgroup of 8 waves (two per SIMD) owns 256 query rows of one (batch, q
+// head); each wave owns 32 of them as one MFMA tile.  K/V are walked in 64-key
+// tiles staged through LDS (double buffered, one barrier per tile).  Two waves
+// per SIMD let one wave's softmax (VALU) run under the other's MFMAs.
 //
 // Both products are issued TRANSPOSED so that everything a lane holds belongs
 // to ONE query row (q = lane % 32):
@@ -21,8 +22,8 @@
 // are lane-local, with one exchange between the two lane halves per row.
 //
 // LDS tiles keep the natural row-major layout; 16-byte chunks are XOR-swizzled so
-// the K operand reads (8 consecutive rows, one chunk column) and the V patch
-// reads (4 consecutive rows, 32 bytes) spread over all banks.
+// the K operand reads (16 consecutive rows, one chunk column, per LDS cycle) and
+// the V patch reads (4 consecutive rows x 64 bytes) spread over all 64 banks.
 #pragma once
 #include "common.h"
 
@@ -40,8 +41,10 @@ struct FlashParams {
   int out_storage;     // 0: f32 O, 1: O in the storage dtype
 };
 
-constexpr int FA_BQ = 256;     // query rows per workgroup
-constexpr int FA_BKV = 64;     // keys per LDS tile
+constexpr int FA_WAVES = 8;
+constexpr int FA_THREADS = FA_WAVES * 64;
+constexpr int FA_BQ = FA_WAVES * 32;   // query rows per workgroup
+constexpr int FA_BKV = 64;             // keys per LDS tile
 constexpr float FA_NEG = -1.0e30f;
 
 // Exchange a value with the lane 32 positions away.
@@ -50,30 +53,51 @@ __device__ __forceinline__ float swap_half(float v) {
 }
 
 template <class T, int D>
-__global__ __launch_bounds__(256, 1) void flash_fwd_kernel(const FlashParams p) {
+__global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashParams p) {
   constexpr int KSTEPS = D / 16;         // MFMA k steps of the score product
   constexpr int DT = D / 32;             // 32-wide d tiles of the output
   constexpr int ROWB = D * 2;            // bytes per K/V row
   constexpr int CHUNKS = D / 8;          // 16-byte chunks per row
   constexpr int TILE = FA_BKV * ROWB;    // bytes per K (or V) tile
-  constexpr int LD_PER_THREAD = FA_BKV * CHUNKS / 256;
-  static_assert(FA_BKV * CHUNKS % 256 == 0, "tile/thread mismatch");
+  constexpr int LD_PER_THREAD = FA_BKV * CHUNKS / FA_THREADS;
+  static_assert(FA_BKV * CHUNKS % FA_THREADS == 0, "tile/thread mismatch");
+  // K swizzle: the 16 rows an LDS cycle serves must hit 16 different 16-byte slots
+  // of the 256-byte bank line.  V swizzle: the 4 rows of a patch, 64 bytes each.
+  auto kswz = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
+  auto vswz = [](int key) { return D == 128 ? ((key & 3) << 2) : (((key >> 1) & 1) << 2); };
 
   extern __shared__ __attribute__((aligned(16))) char smem[];   // [2][K tile | V tile]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  // Heavy (late) query blocks first: with a causal mask their key range is longest.
+  // Work order.  Workgroups are dealt to the 8 XCDs round-robin by their linear id.
+  // Levels of equal cost (one query block index for every (batch, head)) are
+  // issued heaviest first — with a causal mask the last block has the longest key
+  // range — so every XCD receives the same mix, and inside a level the (batch,
+  // head) pairs are permuted so that all query heads sharing one KV head land on
+  // the same XCD and find its K/V in that XCD's L2.
   const int qblocks = (p.Sq + FA_BQ - 1) / FA_BQ;
-  const int qb = qblocks - 1 - (int)blockIdx.x;
-  const int bh = blockIdx.y;
-  const int b = bh / p.Hq, hq = bh % p.Hq;
+  const int BH = p.B * p.Hq;
+  const int id = blockIdx.x;
+  const int qb = qblocks - 1 - id / BH;
+  const int u = id % BH;
+  const int ratio = p.Hq / p.Hkv;
+  int b, hq;
+  if ((p.B * p.Hkv) % 8 == 0) {
+    const int w = u % (8 * ratio);
+    const int g = (u / (8 * ratio)) * 8 + (w & 7);   // kv group = (batch, kv head)
+    b = g / p.Hkv;
+    hq = (g % p.Hkv) * ratio + (w >> 3);
+  } else {
+    b = u / p.Hq;
+    hq = u % p.Hq;
+  }
   const int hkv = (int)(((long)hq * p.Hkv) / p.Hq);
   const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
 
   const int q0 = qb * FA_BQ;             // first query row of the workgroup
-  const int qw = q0 + wave * 64;         // first query row of the wave
+  const int qw = q0 + wave * 32;         // first query row of the wave
   const uint16_t* Qb = p.Q + ((long)(b * p.Hq + hq) * p.Sq) * D;
   const uint16_t* Kb = p.K + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
   const uint16_t* Vb = p.V + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
@@ -87,24 +111,22 @@ __global__ __launch_bounds__(256, 1) void flash_fwd_kernel(const FlashParams p) 
   const int ntiles = (kv_end + FA_BKV - 1) / FA_BKV;
 
   // ---- Q fragments: lane (q = l32, h) holds Q[q][16 ks + 8 h .. +7] -----------
-  uint4 qf[2][KSTEPS];
-#pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
-    int row = qw + qt * 32 + l32;
+  uint4 qf[KSTEPS];
+  {
+    int row = qw + l32;
     row = row < p.Sq ? row : p.Sq - 1;
     const uint16_t* src = Qb + (long)row * D + 8 * lh;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qf[qt][ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
+    for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
   }
 
-  // ---- K/V tile loaders --------------------------------------------------------
-  // chunk v = tid + 256 q -> row v / CHUNKS, chunk v % CHUNKS.
+  // ---- K/V tile loaders: chunk v = tid + THREADS q -> row v / CHUNKS, chunk v % CHUNKS
   uint4 rk[LD_PER_THREAD], rv[LD_PER_THREAD];
   auto gload = [&](int tile) {
     const int kv0 = tile * FA_BKV;
 #pragma unroll
     for (int q = 0; q < LD_PER_THREAD; ++q) {
-      const int v = tid + 256 * q;
+      const int v = tid + FA_THREADS * q;
       int row = kv0 + v / CHUNKS;
       row = row < p.Sk ? row : p.Sk - 1;          // rows past the end are masked below
       const long o = (long)row * D + (v % CHUNKS) * 8;
@@ -117,29 +139,40 @@ __global__ __launch_bounds__(256, 1) void flash_fwd_kernel(const FlashParams p) 
     char* vb = kb + TILE;
 #pragma unroll
     for (int q = 0; q < LD_PER_THREAD; ++q) {
-      const int v = tid + 256 * q;
+      const int v = tid + FA_THREADS * q;
       const int row = v / CHUNKS, ch = v % CHUNKS;
-      lds_write_b128(kb, row * ROWB + ((ch ^ (row & 7)) << 4), rk[q]);
-      lds_write_b128(vb, row * ROWB + ((ch ^ ((row & 3) << 1)) << 4), rv[q]);
+      lds_write_b128(kb, row * ROWB + ((ch ^ kswz(row)) << 4), rk[q]);
+      lds_write_b128(vb, row * ROWB + ((ch ^ vswz(row)) << 4), rv[q]);
     }
   };
 
   // ---- state -----------------------------------------------------------------
-  f32x16 o_acc[DT][2];
+  f32x16 o_acc[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o_acc[dt][qt][r] = 0.f;
-  float m_run[2] = {FA_NEG, FA_NEG};     // running max of the raw (unscaled) scores
-  float l_run[2] = {0.f, 0.f};           // this lane half's share of the running sum
+    for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.f;
+  float m_run = FA_NEG;                  // running max of the raw (unscaled) scores
+  float l_run = 0.f;                     // this lane half's share of the running sum
   const float c = p.scale * 1.44269504088896340736f;   // scale * log2(e)
 
   // Per-wave range: tiles past the wave's own diagonal contribute nothing.
   int wave_kv_end = kv_end;
-  if (p.causal) wave_kv_end = min(kv_end, min(qw + 64, p.Sq) - 1 + off + 1);
+  if (p.causal) wave_kv_end = min(kv_end, min(qw + 32, p.Sq) - 1 + off + 1);
   const bool wave_active = qw < p.Sq;
+  const int qi = qw + l32;               // this lane's query row
+  const int lim = p.causal ? min(qi + off, p.Sk - 1) : p.Sk - 1;   // last visible key
+
+  // per-lane LDS read offsets
+  const int r16 = lane & 15;
+  uint32_t k_rd[2];
+  int k_sw[2];
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt) {
+    const int row = kt * 32 + l32;
+    k_rd[kt] = row * ROWB;
+    k_sw[kt] = kswz(row);
+  }
 
   if (ntiles > 0) {
     gload(0);
@@ -147,154 +180,132 @@ __global__ __launch_bounds__(256, 1) void flash_fwd_kernel(const FlashParams p) 
   }
   __syncthreads();
 
-  for (int t = 0; t < ntiles; ++t) {
+  auto process = [&](int t) {
     const int buf = t & 1;
     const int kv0 = t * FA_BKV;
     const char* kb = smem + buf * 2 * TILE;
     const char* vb = kb + TILE;
-    if (t + 1 < ntiles) gload(t + 1);
-
     if (wave_active && kv0 < wave_kv_end) {
       // ---- S^T = K . Q^T ------------------------------------------------------
-      f32x16 s[2][2];
+      f32x16 s[2];
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[kt][qt][r] = 0.f;
+        for (int r = 0; r < 16; ++r) s[kt][r] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
-        uint4 kf[2];
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt) {
-          const int row = kt * 32 + l32;
-          kf[kt] = lds_read_b128(kb, row * ROWB + ((((ks << 1) | lh) ^ (row & 7)) << 4));
+          const uint4 kf = lds_read_b128(kb, k_rd[kt] + ((((ks << 1) | lh) ^ k_sw[kt]) << 4));
+          s[kt] = mfma_32x32x16<T>(kf, qf[ks], s[kt]);
         }
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int qt = 0; qt < 2; ++qt) s[kt][qt] = mfma_32x32x16<T>(kf[kt], qf[qt][ks], s[kt][qt]);
       }
 
       // ---- mask (only tiles that touch the diagonal or the end of K) ------------
       const bool need_mask = (kv0 + FA_BKV > p.Sk) || (p.causal && (kv0 + FA_BKV - 1 > qw + off));
       if (need_mask) {
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
-          const int qi = qw + qt * 32 + l32;
-          const int lim = p.causal ? min(qi + off, p.Sk - 1) : p.Sk - 1;   // last visible key
-#pragma unroll
-          for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int key = kv0 + kt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-              if (key > lim) s[kt][qt][r] = FA_NEG;
-            }
-        }
-      }
-
-      // ---- online softmax; P stays in the S registers as packed 16-bit ---------
-      uint4 pf[2][2][2];   // [kt][g][qt]: B operand of the (kt, g) 16-key step
-#pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
-        float mx = s[0][qt][0];
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kt][qt][r]);
-        mx = fmaxf(mx, swap_half(mx));
-        const float m_new = fmaxf(m_run[qt], mx);
-        const float corr = fast_exp2((m_run[qt] - m_new) * c);
-        const float mc = m_new * c;
-        m_run[qt] = m_new;
-        float sum = 0.f;
-#pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float e = fast_exp2(fmaf(s[kt][qt][r], c, -mc));
-            s[kt][qt][r] = e;
-            sum += e;
+            const int key = kv0 + kt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+            if (key > lim) s[kt][r] = FA_NEG;
           }
-        l_run[qt] = l_run[qt] * corr + sum;
+      }
+
+      // ---- online softmax; P stays in the S registers -----------------------------
+      float mx = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
+      mx = fmaxf(mx, swap_half(mx));
+      const float m_new = fmaxf(m_run, mx);
+      const float mc = m_new * c;
+      // Rescale the accumulator only when some row of the wave raised its maximum.
+      if (__any(m_new > m_run)) {
+        const float corr = fast_exp2((m_run - m_new) * c);
+        l_run *= corr;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) o_acc[dt][qt][r] *= corr;
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int g = 0; g < 2; ++g) {
-            uint4 v;
-            v.x = pack2<T>(s[kt][qt][8 * g + 0], s[kt][qt][8 * g + 1]);
-            v.y = pack2<T>(s[kt][qt][8 * g + 2], s[kt][qt][8 * g + 3]);
-            v.z = pack2<T>(s[kt][qt][8 * g + 4], s[kt][qt][8 * g + 5]);
-            v.w = pack2<T>(s[kt][qt][8 * g + 6], s[kt][qt][8 * g + 7]);
-            pf[kt][g][qt] = v;
-          }
+          for (int r = 0; r < 16; ++r) o_acc[dt][r] *= corr;
+        m_run = m_new;
       }
+      float sum = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float e = fast_exp2(fmaf(s[kt][r], c, -mc));
+          s[kt][r] = e;
+          sum += e;
+        }
+      l_run += sum;
+      uint4 pf[2][2];   // [kt][g]: B operand of the (kt, g) 16-key step
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          pf[kt][g].x = pack2<T>(s[kt][8 * g + 0], s[kt][8 * g + 1]);
+          pf[kt][g].y = pack2<T>(s[kt][8 * g + 2], s[kt][8 * g + 3]);
+          pf[kt][g].z = pack2<T>(s[kt][8 * g + 4], s[kt][8 * g + 5]);
+          pf[kt][g].w = pack2<T>(s[kt][8 * g + 6], s[kt][8 * g + 7]);
+        }
 
       // ---- O^T += V^T . P^T ------------------------------------------------------
       // 16-key step (kt, g) covers keys 32 kt + 16 g + {4h + 0..3, 8 + 4h + 0..3}.
       // Transposing read: lane r of a 16-lane block supplies row (key) r/4 of a
       // 4-key patch and columns 4 (r % 4) .. +3 of a 16-column slab.
-      const int r16 = lane & 15;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
-          uint4 vf[DT];
+          const int key_lo = kt * 32 + g * 16 + 4 * lh + (r16 >> 2);
+          const int key_hi = key_lo + 8;
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) {
             const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (r16 & 3);   // element column
-            const int key_lo = kt * 32 + g * 16 + 4 * lh + (r16 >> 2);
-            const int key_hi = key_lo + 8;
             const int ch = col >> 3, within = (col & 7) * 2;
-            const uint2 lo = lds_read_tr16_b64(vb + key_lo * ROWB + ((ch ^ ((key_lo & 3) << 1)) << 4) + within);
-            const uint2 hi = lds_read_tr16_b64(vb + key_hi * ROWB + ((ch ^ ((key_hi & 3) << 1)) << 4) + within);
-            vf[dt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            const uint2 lo = lds_read_tr16_b64(vb + key_lo * ROWB + ((ch ^ vswz(key_lo)) << 4) + within);
+            const uint2 hi = lds_read_tr16_b64(vb + key_hi * ROWB + ((ch ^ vswz(key_hi)) << 4) + within);
+            o_acc[dt] = mfma_32x32x16<T>(make_uint4(lo.x, lo.y, hi.x, hi.y), pf[kt][g], o_acc[dt]);
           }
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int qt = 0; qt < 2; ++qt)
-              o_acc[dt][qt] = mfma_32x32x16<T>(vf[dt], pf[kt][g][qt], o_acc[dt][qt]);
         }
     }
-
-    if (t + 1 < ntiles) lstore(buf ^ 1);
+  };
+  // Tile t+1 is fetched into registers while tile t is consumed, then stored to
+  // the other buffer; the last tile has nothing to fetch.
+  for (int t = 0; t + 1 < ntiles; ++t) {
+    gload(t + 1);
+    process(t);
+    lstore((t & 1) ^ 1);
     __syncthreads();
   }
+  if (ntiles > 0) process(ntiles - 1);
 
   // ---- epilogue -------------------------------------------------------------------
   if (!wave_active) return;
+  const float l = l_run + swap_half(l_run);
+  if (qi >= p.Sq) return;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  const long row = (long)(b * p.Hq + hq) * p.Sq + qi;
+  if (p.LSE && lh == 0)
+    p.LSE[row] = l > 0.f ? (m_run * c + __log2f(l)) * 0.69314718055994530942f : -INFINITY;
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
-    const int qi = qw + qt * 32 + l32;
-    const float l = l_run[qt] + swap_half(l_run[qt]);
-    if (qi >= p.Sq) continue;
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    const long row = (long)(b * p.Hq + hq) * p.Sq + qi;
-    if (p.LSE && lh == 0)
-      p.LSE[row] = l > 0.f ? (m_run[qt] * c + __log2f(l)) * 0.69314718055994530942f : -INFINITY;
+  for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        const int d = dt * 32 + 8 * a + 4 * lh;
-        const float v0 = o_acc[dt][qt][4 * a + 0] * inv, v1 = o_acc[dt][qt][4 * a + 1] * inv;
-        const float v2 = o_acc[dt][qt][4 * a + 2] * inv, v3 = o_acc[dt][qt][4 * a + 3] * inv;
-        if (p.out_storage) {
-          uint2 pk;
-          pk.x = pack2<T>(v0, v1);
-          pk.y = pack2<T>(v2, v3);
-          *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.O) + row * D + d) = pk;
-        } else {
-          *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.O) + row * D + d) = make_float4(v0, v1, v2, v3);
-        }
+    for (int a = 0; a < 4; ++a) {
+      const int d = dt * 32 + 8 * a + 4 * lh;
+      const float v0 = o_acc[dt][4 * a + 0] * inv, v1 = o_acc[dt][4 * a + 1] * inv;
+      const float v2 = o_acc[dt][4 * a + 2] * inv, v3 = o_acc[dt][4 * a + 3] * inv;
+      if (p.out_storage) {
+        uint2 pk;
+        pk.x = pack2<T>(v0, v1);
+        pk.y = pack2<T>(v2, v3);
+        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.O) + row * D + d) = pk;
+      } else {
+        *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.O) + row * D + d) = make_float4(v0, v1, v2, v3);
       }
-  }
+    }
 }
 
 // Any head dimension: one thread per query row, streaming online softmax in f32.
