@@ -33,6 +33,10 @@ PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16/f16 MFMA
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_INT8_TOPS = 5000.0
 PEAK_HBM_GBS = 8000.0
+# HBM-side bytes one launch of the headline kernel moves: FETCH_SIZE + WRITE_SIZE per
+# dispatch from two counter runs of this script, each scaled by the same counter's
+# reading for the 1 GiB copy kernel (profiles/bench_all_kernels_hbm_bytes.txt).
+TRAFFIC_BYTES_GEMM_BF16_8192 = 1.7738e9
 
 
 def _timed(lane, launch, steps, warmup):
@@ -75,6 +79,19 @@ def bench_gemm(lane, M, N, K, steps, warmup, seed=0):
     for buf in (da, db, dd):
         buf.close()
     return wall, ev, (A, B, a, b, out)
+
+
+def calibrate_copy(lane, reps=3, nbytes=1 << 30):
+    """Launch the library's plain copy kernel on `nbytes` (reads nbytes, writes
+    nbytes): the known-size kernel the FETCH_SIZE / WRITE_SIZE counters of a
+    profiled run are scaled by."""
+    src, dst = lane.DeviceBuffer(nbytes), lane.DeviceBuffer(nbytes)
+    src.zero()
+    fn = lane.load().tessera_gfx950_memcpy_d2d_dev
+    _, ev = _timed(lane, lambda: lane.check(fn(dst.ptr, src.ptr, nbytes, None), "copy"), reps, 1)
+    src.close()
+    dst.close()
+    return {"bytes_each_way": nbytes, "ms": ev, "gbs": 2.0 * nbytes / ev / 1e6}
 
 
 def bench_attention(lane, steps, warmup):
@@ -215,6 +232,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true", help="skip the `also` measurements")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch a 1 GiB copy kernel (counter calibration for profiled runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X; this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -225,6 +244,7 @@ def main() -> int:
         print("gfx950 lane unavailable: no MI355X or library not built", file=sys.stderr)
         return 3
 
+    copy_cal = calibrate_copy(lane) if args.calibrate_copy else None
     M = N = K = 8192
     wall, ev, (A, B, a, b, out) = bench_gemm(lane, M, N, K, args.steps, args.warmup)
     flop = 2.0 * M * N * K
@@ -236,9 +256,11 @@ def main() -> int:
         "config": {"workload": "gemm_bf16_8192x8192x8192_f32acc_bf16out", "M": M, "N": N, "K": K,
                    "device": lane.device_name()},
         "roofline": {"bound": "mfma", "achieved": flop / ev / 1e9, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flop / ev / 1e9 / PEAK_BF16_TFLOPS, "traffic": None,
+                     "frac": flop / ev / 1e9 / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BYTES_GEMM_BF16_8192,
                      "kernel": "gemm16_kernel<BF16,256,256,2,2,STORE16>", "avg_launch_ms": ev},
     }
+    if copy_cal:
+        result["copy_calibration"] = copy_cal
     if not args.no_cpu:
         ref, result["cpu_baseline"] = cpu_baseline(A, B)
         got = (out.astype(np.uint32) << 16).view(np.float32)

@@ -62,6 +62,11 @@ int tessera_gfx950_free(void* dptr);
 int tessera_gfx950_memcpy_h2d(void* dst, const void* src, size_t bytes);
 int tessera_gfx950_memcpy_d2h(void* dst, const void* src, size_t bytes);
 int tessera_gfx950_memset(void* dst, int value, size_t bytes);
+/* Device-to-device copy kernel on a stream (bytes and both pointers multiples of
+ * 16).  Lets a caller chain resident buffers without a host round trip, the role
+ * of the device-operand lease in python/tessera/runtime.py:1549-1614; also the
+ * known-size kernel HBM byte counters are calibrated against. */
+int tessera_gfx950_memcpy_d2d_dev(void* dst, const void* src, size_t bytes, void* stream);
 int tessera_gfx950_synchronize(void);
 
 /* Device-event timer on a stream (NULL = default stream): the timing clock the

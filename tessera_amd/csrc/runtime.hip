@@ -26,6 +26,12 @@ struct Timer {
   hipEvent_t start, stop;
 };
 
+// Grid-stride 16-byte copy: one coalesced global_load_dwordx4 / store per lane.
+__global__ void __launch_bounds__(256) copy16_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
 }  // namespace tsr950
 
 using namespace tsr950;
@@ -85,6 +91,19 @@ int tessera_gfx950_memset(void* dst, int value, size_t bytes) {
   if (bytes && !dst) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
   return bytes ? finish(hipMemset(dst, value, bytes)) : kOk;
+}
+
+int tessera_gfx950_memcpy_d2d_dev(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes && (!dst || !src)) return kBadShape;
+  if (bytes % 16 != 0 || ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  if (!bytes) return kOk;
+  const size_t n = bytes / 16;
+  const size_t want = (n + 255) / 256;
+  const unsigned grid = (unsigned)(want < 256 * 32 ? want : 256 * 32);
+  hipLaunchKernelGGL(copy16_kernel, dim3(grid), dim3(256), 0, as_stream(stream),
+                     static_cast<uint4*>(dst), static_cast<const uint4*>(src), n);
+  return launch_status();
 }
 
 int tessera_gfx950_synchronize(void) {

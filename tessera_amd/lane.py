@@ -68,6 +68,7 @@ _SIGNATURES = {
     "tessera_gfx950_memcpy_h2d": [_c_vp, _c_vp, _c_sz],
     "tessera_gfx950_memcpy_d2h": [_c_vp, _c_vp, _c_sz],
     "tessera_gfx950_memset": [_c_vp, _c_int, _c_sz],
+    "tessera_gfx950_memcpy_d2d_dev": [_c_vp, _c_vp, _c_sz, _c_vp],
     "tessera_gfx950_synchronize": [],
     "tessera_gfx950_timer_create": [_P(_c_vp)],
     "tessera_gfx950_timer_start": [_c_vp, _c_vp],
