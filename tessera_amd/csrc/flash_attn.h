@@ -3,8 +3,13 @@
 //
 // One workgroup of 8 waves (two per SIMD) owns 256 query rows of one (batch, q
 // head); each wave owns 32 of them as one MFMA tile.  K/V are walked in 64-key
-// tiles staged through LDS (double buffered, one barrier per tile).  Two waves
-// per SIMD let one wave's softmax (VALU) run under the other's MFMAs.
+// tiles that stream from global memory straight into LDS (two stages each, one
+// barrier per tile).  The loop is software-pipelined: the score MFMAs of tile
+// t+1 are issued under the softmax arithmetic of tile t, and the exponentials of
+// each 8-key group just ahead of the P.V MFMAs that consume it; the second wave
+// on each SIMD fills what is left.  (FA_QT = 2, four waves of 64 rows sharing
+// each K/V fragment between two query tiles, halves the LDS reads but leaves one
+// wave per SIMD and measured 40 % slower.)
 //
 // Both products are issued TRANSPOSED so that everything a lane holds belongs
 // to ONE query row (q = lane % 32):
@@ -25,6 +30,7 @@
 // the K operand reads (16 consecutive rows, one chunk column, per LDS cycle) and
 // the V patch reads (4 consecutive rows x 64 bytes) spread over all 64 banks.
 #pragma once
+#include <type_traits>
 #include "common.h"
 
 namespace tsr950 {
@@ -41,10 +47,12 @@ struct FlashParams {
   int out_storage;     // 0: f32 O, 1: O in the storage dtype
 };
 
-constexpr int FA_WAVES = 8;
+constexpr int FA_BQ = 256;             // query rows per workgroup
+constexpr int FA_QT = 1;               // 32-row query tiles per wave
+constexpr int FA_WAVES = FA_BQ / (32 * FA_QT);
 constexpr int FA_THREADS = FA_WAVES * 64;
-constexpr int FA_BQ = FA_WAVES * 32;   // query rows per workgroup
 constexpr int FA_BKV = 64;             // keys per LDS tile
+constexpr int FA_KT = FA_BKV / 32;     // 32-key MFMA tiles per LDS tile
 constexpr float FA_NEG = -1.0e30f;
 
 // Exchange a value with the lane 32 positions away.
@@ -52,9 +60,45 @@ __device__ __forceinline__ float swap_half(float v) {
   return __shfl_xor(v, 32, 64);
 }
 
+// max(a, b, c) in one instruction; the operands are finite MFMA results, so the
+// NaN canonicalisation fmaxf() would add per operand is not needed.
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+  float d;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+  return d;
+}
+
+// 16 bytes per lane from global memory straight into LDS: lane i's data lands at
+// lds_base + 16 i (lds_base wave-uniform); the global address is a uniform base
+// plus a per-lane byte offset.  Issued as inline assembly so that the compiler
+// does not serialise later LDS reads of OTHER stages behind it; the kernel waits
+// for these loads itself (fa_wait_loads) before the barrier that publishes the
+// stage.
+__device__ __forceinline__ void load16_to_lds(const void* base, uint32_t byte_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(lds_base), "v"(byte_off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void fa_wait_loads() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// acc *= corr for an accumulator element that lives in the accumulation register
+// file: the output accumulators are touched by vector arithmetic only here (a rare
+// path), so keeping them out of the ordinary register file leaves that file to the
+// score tiles and operand fragments.
+__device__ __forceinline__ float scale_acc(float acc, float corr) {
+  float tmp;
+  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
+               : "+a"(acc), "=&v"(tmp) : "v"(corr));
+  return acc;
+}
+
 template <class T, int D>
-__global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashParams p) {
+__global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel(const FlashParams p) {
+  constexpr int QT = FA_QT;
   constexpr int KSTEPS = D / 16;         // MFMA k steps of the score product
+  constexpr int KA = (KSTEPS + 3) / 4;   // score k steps issued under the row-max phase
+  constexpr int KB = (KSTEPS + KA) / 2;  // ... and up to here under the first exponentials
   constexpr int DT = D / 32;             // 32-wide d tiles of the output
   constexpr int ROWB = D * 2;            // bytes per K/V row
   constexpr int CHUNKS = D / 8;          // 16-byte chunks per row
@@ -66,9 +110,12 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
   auto kswz = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
   auto vswz = [](int key) { return D == 128 ? ((key & 3) << 2) : (((key >> 1) & 1) << 2); };
 
-  extern __shared__ __attribute__((aligned(16))) char smem[];   // [2][K tile | V tile]
+  // LDS: K stages at 0 and TILE, V stages at 2 TILE and 3 TILE.
+  extern __shared__ __attribute__((aligned(16))) char smem[];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(TSR_LDS char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, lh = lane >> 5;
 
   // Work order.  Workgroups are dealt to the 8 XCDs round-robin by their linear id.
@@ -96,8 +143,8 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
   const int hkv = (int)(((long)hq * p.Hkv) / p.Hq);
   const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
 
-  const int q0 = qb * FA_BQ;             // first query row of the workgroup
-  const int qw = q0 + wave * 32;         // first query row of the wave
+  const int q0 = qb * FA_BQ;                  // first query row of the workgroup
+  const int qw = q0 + wave * (32 * QT);       // first query row of the wave
   const uint16_t* Qb = p.Q + ((long)(b * p.Hq + hq) * p.Sq) * D;
   const uint16_t* Kb = p.K + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
   const uint16_t* Vb = p.V + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
@@ -109,203 +156,303 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
     kv_end = min(p.Sk, last_q + off + 1);
   }
   const int ntiles = (kv_end + FA_BKV - 1) / FA_BKV;
+  // Tiles this wave computes on: those below its own diagonal.
+  int nt_w = 0;
+  if (qw < p.Sq) {
+    int wave_kv_end = kv_end;
+    if (p.causal) wave_kv_end = min(kv_end, min(qw + 32 * QT, p.Sq) - 1 + off + 1);
+    nt_w = (wave_kv_end + FA_BKV - 1) / FA_BKV;
+  }
 
   // ---- Q fragments: lane (q = l32, h) holds Q[q][16 ks + 8 h .. +7] -----------
-  uint4 qf[KSTEPS];
-  {
-    int row = qw + l32;
+  uint4 qf[QT][KSTEPS];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    int row = qw + 32 * qt + l32;
     row = row < p.Sq ? row : p.Sq - 1;
     const uint16_t* src = Qb + (long)row * D + 8 * lh;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
+    for (int ks = 0; ks < KSTEPS; ++ks) qf[qt][ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
   }
 
-  // ---- K/V tile loaders: chunk v = tid + THREADS q -> row v / CHUNKS, chunk v % CHUNKS
-  uint4 rk[LD_PER_THREAD], rv[LD_PER_THREAD];
-  auto gload = [&](int tile) {
-    const int kv0 = tile * FA_BKV;
+  // ---- K/V tile loaders: straight from global memory into LDS ----------------------
+  // One wave instruction fills 64 consecutive 16-byte LDS slots; slot P is (row
+  // P / CHUNKS, physical chunk P % CHUNKS) and holds the row's logical chunk
+  // (physical ^ swizzle(row)), so the swizzle is applied on the global address.
+  int ld_row[LD_PER_THREAD];
+  uint32_t ld_koff[LD_PER_THREAD], ld_voff[LD_PER_THREAD];   // byte offsets inside a full tile
+#pragma unroll
+  for (int q = 0; q < LD_PER_THREAD; ++q) {
+    const int P = (wave * LD_PER_THREAD + q) * 64 + lane;
+    const int row = P / CHUNKS, chp = P % CHUNKS;
+    ld_row[q] = row;
+    ld_koff[q] = row * ROWB + ((chp ^ kswz(row)) << 4);
+    ld_voff[q] = row * ROWB + ((chp ^ vswz(row)) << 4);
+  }
+  // Full tiles use the precomputed per-lane offsets on a uniform tile base; the
+  // ragged last tile clamps its rows (rows past the end are masked in the scores
+  // and meet P = 0 in the second product).
+  auto load_tile = [&](const uint16_t* base, const uint32_t (&offs)[LD_PER_THREAD], int tile, int lds_stage) {
+    const uint16_t* tb = base + (long)tile * FA_BKV * D;
+    const bool full = (tile + 1) * FA_BKV <= p.Sk;
 #pragma unroll
     for (int q = 0; q < LD_PER_THREAD; ++q) {
-      const int v = tid + FA_THREADS * q;
-      int row = kv0 + v / CHUNKS;
-      row = row < p.Sk ? row : p.Sk - 1;          // rows past the end are masked below
-      const long o = (long)row * D + (v % CHUNKS) * 8;
-      rk[q] = *reinterpret_cast<const uint4*>(Kb + o);
-      rv[q] = *reinterpret_cast<const uint4*>(Vb + o);
+      uint32_t o = offs[q];
+      if (!full) {
+        const int last = p.Sk - 1 - tile * FA_BKV;        // last valid row of this tile
+        if (ld_row[q] > last) o -= (uint32_t)(ld_row[q] - last) * ROWB;
+      }
+      load16_to_lds(tb, o, lds0 + lds_stage * TILE + (wave * LD_PER_THREAD + q) * 1024);
     }
   };
-  auto lstore = [&](int buf) {
-    char* kb = smem + buf * 2 * TILE;
-    char* vb = kb + TILE;
-#pragma unroll
-    for (int q = 0; q < LD_PER_THREAD; ++q) {
-      const int v = tid + FA_THREADS * q;
-      const int row = v / CHUNKS, ch = v % CHUNKS;
-      lds_write_b128(kb, row * ROWB + ((ch ^ kswz(row)) << 4), rk[q]);
-      lds_write_b128(vb, row * ROWB + ((ch ^ vswz(row)) << 4), rv[q]);
-    }
-  };
+  auto load_k = [&](int tile, int stage) { load_tile(Kb, ld_koff, tile, stage); };
+  auto load_v = [&](int tile, int stage) { load_tile(Vb, ld_voff, tile, 2 + stage); };
 
   // ---- state -----------------------------------------------------------------
-  f32x16 o_acc[DT];
+  f32x16 o_acc[QT][DT];
+  float m_run[QT], l_run[QT];            // running max of the raw scores; this lane half's sum
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int qt = 0; qt < QT; ++qt) {
+    m_run[qt] = FA_NEG;
+    l_run[qt] = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.f;
-  float m_run = FA_NEG;                  // running max of the raw (unscaled) scores
-  float l_run = 0.f;                     // this lane half's share of the running sum
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o_acc[qt][dt][r] = 0.f;
+  }
   const float c = p.scale * 1.44269504088896340736f;   // scale * log2(e)
+  int lim[QT];                           // last visible key of this lane's query rows
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const int qi = qw + 32 * qt + l32;
+    lim[qt] = p.causal ? min(qi + off, p.Sk - 1) : p.Sk - 1;
+  }
 
-  // Per-wave range: tiles past the wave's own diagonal contribute nothing.
-  int wave_kv_end = kv_end;
-  if (p.causal) wave_kv_end = min(kv_end, min(qw + 32, p.Sq) - 1 + off + 1);
-  const bool wave_active = qw < p.Sq;
-  const int qi = qw + l32;               // this lane's query row
-  const int lim = p.causal ? min(qi + off, p.Sk - 1) : p.Sk - 1;   // last visible key
-
-  // per-lane LDS read offsets
+  // ---- per-lane LDS read addresses (stage and tile-row offsets are immediates) ----
+  // K operand: row l32 (+32 kt), logical chunk 2 ks + lh.
+  uint32_t k_rd[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) k_rd[ks] = l32 * ROWB + ((((ks << 1) | lh) ^ kswz(l32)) << 4);
+  // V operand: transposing read; lane r of a 16-lane block supplies key r/4 of a
+  // 4-key patch and columns 4 (r % 4) .. +3 of a 16-column slab.
   const int r16 = lane & 15;
-  uint32_t k_rd[2];
-  int k_sw[2];
+  uint32_t v_rd[DT];
 #pragma unroll
-  for (int kt = 0; kt < 2; ++kt) {
-    const int row = kt * 32 + l32;
-    k_rd[kt] = row * ROWB;
-    k_sw[kt] = kswz(row);
+  for (int dt = 0; dt < DT; ++dt) {
+    const int key = 4 * lh + (r16 >> 2);
+    const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (r16 & 3);
+    v_rd[dt] = 2 * TILE + key * ROWB + (((col >> 3) ^ vswz(key)) << 4) + (col & 7) * 2;
   }
 
-  if (ntiles > 0) {
-    gload(0);
-    lstore(0);
-  }
-  __syncthreads();
-
-  auto process = [&](int t) {
-    const int buf = t & 1;
-    const int kv0 = t * FA_BKV;
-    const char* kb = smem + buf * 2 * TILE;
-    const char* vb = kb + TILE;
-    if (wave_active && kv0 < wave_kv_end) {
-      // ---- S^T = K . Q^T ------------------------------------------------------
-      f32x16 s[2];
+  // S^T(tile in K stage `stage`) = K . Q^T, k steps [ks0, ks1); one K fragment
+  // feeds the wave's QT query tiles.
+  auto score_steps = [&](f32x16 (&sn)[QT][FA_KT], int stage, int ks0, int ks1) {
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
+    for (int ks = ks0; ks < ks1; ++ks)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[kt][r] = 0.f;
+      for (int kt = 0; kt < FA_KT; ++kt) {
+        const uint4 kf = lds_read_b128(smem, k_rd[ks] + stage * TILE + kt * 32 * ROWB);
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
+        for (int qt = 0; qt < QT; ++qt) {
+          if (ks == 0) {
+            f32x16 z;
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-          const uint4 kf = lds_read_b128(kb, k_rd[kt] + ((((ks << 1) | lh) ^ k_sw[kt]) << 4));
-          s[kt] = mfma_32x32x16<T>(kf, qf[ks], s[kt]);
+            for (int r = 0; r < 16; ++r) z[r] = 0.f;
+            sn[qt][kt] = mfma_32x32x16<T>(kf, qf[qt][ks], z);
+          } else {
+            sn[qt][kt] = mfma_32x32x16<T>(kf, qf[qt][ks], sn[qt][kt]);
+          }
         }
       }
-
-      // ---- mask (only tiles that touch the diagonal or the end of K) ------------
-      const bool need_mask = (kv0 + FA_BKV > p.Sk) || (p.causal && (kv0 + FA_BKV - 1 > qw + off));
-      if (need_mask) {
+  };
+  // exp2 of one 8-key group of a score tile (in place), its sum, packed to P.
+  auto exp_group = [&](f32x16& sv, int g, float mc, float& sum) -> uint4 {
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
+    for (int r = 8 * g; r < 8 * g + 8; ++r) {
+      const float e = fast_exp2(fmaf(sv[r], c, -mc));
+      sv[r] = e;
+      sum += e;
+    }
+    uint4 pf;
+    pf.x = pack2<T>(sv[8 * g + 0], sv[8 * g + 1]);
+    pf.y = pack2<T>(sv[8 * g + 2], sv[8 * g + 3]);
+    pf.z = pack2<T>(sv[8 * g + 4], sv[8 * g + 5]);
+    pf.w = pack2<T>(sv[8 * g + 6], sv[8 * g + 7]);
+    return pf;
+  };
+
+  // One pipeline step for tile t.  The score MFMAs of tile t+1 are issued first and
+  // run under the softmax arithmetic of tile t (whose scores `sc` were produced one
+  // step earlier); the exponentials are produced in 8-key groups, each group just
+  // ahead of the P.V MFMAs that consume it.  K(t+2) and V(t+1) stream into the
+  // stages the previous step released.
+  auto step = [&](auto has_next_c, auto par_c, f32x16 (&sc)[QT][FA_KT], f32x16 (&sn)[QT][FA_KT], int t) {
+    constexpr bool HAS_NEXT = decltype(has_next_c)::value;
+    constexpr int PAR = decltype(par_c)::value;        // t & 1
+    if (t + 2 < ntiles) load_k(t + 2, PAR);
+    if (t + 1 < ntiles) load_v(t + 1, PAR ^ 1);
+    const int kv0 = t * FA_BKV;
+    // mask (only tiles that touch the diagonal or the end of K)
+    const bool need_mask = (kv0 + FA_BKV > p.Sk) || (p.causal && (kv0 + FA_BKV - 1 > qw + off));
+    if (need_mask) {
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+        for (int kt = 0; kt < FA_KT; ++kt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int key = kv0 + kt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-            if (key > lim) s[kt][r] = FA_NEG;
+            if (key > lim[qt]) sc[qt][kt][r] = FA_NEG;
           }
-      }
-
-      // ---- online softmax; P stays in the S registers -----------------------------
-      float mx = fmaxf(s[0][0], s[1][0]);
+    }
+    if constexpr (HAS_NEXT) score_steps(sn, PAR ^ 1, 0, KA);
+    // row max
+    float m_new[QT], mc[QT];
+    bool grow = false;
 #pragma unroll
-      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
+    for (int qt = 0; qt < QT; ++qt) {
+      float mx = max3_raw(sc[qt][0][0], sc[qt][0][1], sc[qt][0][2]);
+#pragma unroll
+      for (int kt = 0; kt < FA_KT; ++kt)
+#pragma unroll
+        for (int r = (kt == 0 ? 3 : 0); r < 16; r += 2)
+          mx = (r + 1 < 16) ? max3_raw(mx, sc[qt][kt][r], sc[qt][kt][r + 1]) : fmaxf(mx, sc[qt][kt][r]);
       mx = fmaxf(mx, swap_half(mx));
-      const float m_new = fmaxf(m_run, mx);
-      const float mc = m_new * c;
-      // Rescale the accumulator only when some row of the wave raised its maximum.
-      if (__any(m_new > m_run)) {
-        const float corr = fast_exp2((m_run - m_new) * c);
-        l_run *= corr;
+      m_new[qt] = fmaxf(m_run[qt], mx);
+      grow = grow || (m_new[qt] > m_run[qt]);
+    }
+    // Rescale the accumulators only when some row of the wave raised its maximum.
+    if (__any(grow)) {
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) {
+        const float corr = fast_exp2((m_run[qt] - m_new[qt]) * c);
+        l_run[qt] *= corr;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) o_acc[dt][r] *= corr;
-        m_run = m_new;
-      }
-      float sum = 0.f;
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float e = fast_exp2(fmaf(s[kt][r], c, -mc));
-          s[kt][r] = e;
-          sum += e;
-        }
-      l_run += sum;
-      uint4 pf[2][2];   // [kt][g]: B operand of the (kt, g) 16-key step
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
-          pf[kt][g].x = pack2<T>(s[kt][8 * g + 0], s[kt][8 * g + 1]);
-          pf[kt][g].y = pack2<T>(s[kt][8 * g + 2], s[kt][8 * g + 3]);
-          pf[kt][g].z = pack2<T>(s[kt][8 * g + 4], s[kt][8 * g + 5]);
-          pf[kt][g].w = pack2<T>(s[kt][8 * g + 6], s[kt][8 * g + 7]);
-        }
-
-      // ---- O^T += V^T . P^T ------------------------------------------------------
-      // 16-key step (kt, g) covers keys 32 kt + 16 g + {4h + 0..3, 8 + 4h + 0..3}.
-      // Transposing read: lane r of a 16-lane block supplies row (key) r/4 of a
-      // 4-key patch and columns 4 (r % 4) .. +3 of a 16-column slab.
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
-          const int key_lo = kt * 32 + g * 16 + 4 * lh + (r16 >> 2);
-          const int key_hi = key_lo + 8;
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) {
-            const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (r16 & 3);   // element column
-            const int ch = col >> 3, within = (col & 7) * 2;
-            const uint2 lo = lds_read_tr16_b64(vb + key_lo * ROWB + ((ch ^ vswz(key_lo)) << 4) + within);
-            const uint2 hi = lds_read_tr16_b64(vb + key_hi * ROWB + ((ch ^ vswz(key_hi)) << 4) + within);
-            o_acc[dt] = mfma_32x32x16<T>(make_uint4(lo.x, lo.y, hi.x, hi.y), pf[kt][g], o_acc[dt]);
+          for (int r = 0; r < 16; ++r) {
+            if constexpr (QT > 1) o_acc[qt][dt][r] = scale_acc(o_acc[qt][dt][r], corr);
+            else o_acc[qt][dt][r] *= corr;
           }
-        }
+        m_run[qt] = m_new[qt];
+      }
+      if constexpr (QT > 1) asm volatile("s_nop 4");   // accumulator writes settle before the next MFMA
     }
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) mc[qt] = m_new[qt] * c;
+
+    // Units of 8 keys x one query tile, in consumption order: i -> (kt, g, qt).
+    constexpr int NU = 2 * FA_KT * QT;
+    constexpr int AHEAD = 3 < NU ? 3 : NU;             // units exponentiated ahead of their P.V step
+    uint4 pf[NU];
+    float sum[QT][2];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) sum[qt][0] = sum[qt][1] = 0.f;
+    auto unit = [&](int i) {
+      const int qt = i % QT, g = (i / QT) & 1, kt = i / (2 * QT);
+      pf[i] = exp_group(sc[qt][kt], g, mc[qt], sum[qt][g]);
+    };
+    if constexpr (HAS_NEXT) score_steps(sn, PAR ^ 1, KA, KB);
+    unit(0);
+    if (AHEAD > 1) unit(1);
+    if constexpr (HAS_NEXT) score_steps(sn, PAR ^ 1, KB, KSTEPS);
+    if (AHEAD > 2) unit(2);
+    // O^T += V^T . P^T; the 16-key step (kt, g) covers keys
+    // 32 kt + 16 g + {4h + 0..3, 8 + 4h + 0..3} and feeds all QT query tiles.
+#pragma unroll
+    for (int sgi = 0; sgi < 2 * FA_KT; ++sgi) {
+      const int kt = sgi >> 1, g = sgi & 1;
+      uint4 vf[DT];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const uint32_t a = v_rd[dt] + PAR * TILE + (kt * 32 + g * 16) * ROWB;
+        const uint2 lo = lds_read_tr16_b64(smem + a);
+        const uint2 hi = lds_read_tr16_b64(smem + a + 8 * ROWB);
+        vf[dt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) {
+        const int i = sgi * QT + qt;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] = mfma_32x32x16<T>(vf[dt], pf[i], o_acc[qt][dt]);
+        if (i + AHEAD < NU) unit(i + AHEAD);
+      }
+    }
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) l_run[qt] += sum[qt][0] + sum[qt][1];
+    fa_wait_loads();
+    __syncthreads();
   };
-  // Tile t+1 is fetched into registers while tile t is consumed, then stored to
-  // the other buffer; the last tile has nothing to fetch.
-  for (int t = 0; t + 1 < ntiles; ++t) {
-    gload(t + 1);
-    process(t);
-    lstore((t & 1) ^ 1);
+  using std::true_type;
+  using std::false_type;
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+
+  // ---- prologue: K(0), V(0), K(1) resident; scores of tile 0 ----------------------
+  if (ntiles > 0) {
+    load_k(0, 0);
+    load_v(0, 0);
+  }
+  if (ntiles > 1) load_k(1, 1);
+  fa_wait_loads();
+  __syncthreads();
+  f32x16 sA[QT][FA_KT], sB[QT][FA_KT];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+    for (int kt = 0; kt < FA_KT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { sA[qt][kt][r] = 0.f; sB[qt][kt][r] = 0.f; }
+  if (nt_w > 0) score_steps(sA, 0, 0, KSTEPS);
+
+  int t = 0;
+  for (; t + 2 < nt_w; t += 2) {
+    step(true_type{}, P0{}, sA, sB, t);
+    step(true_type{}, P1{}, sB, sA, t + 1);
+  }
+  if (t + 2 == nt_w) {
+    step(true_type{}, P0{}, sA, sB, t);
+    step(false_type{}, P1{}, sB, sA, t + 1);
+    t += 2;
+  } else if (t + 1 == nt_w) {
+    step(false_type{}, P0{}, sA, sB, t);
+    t += 1;
+  }
+  // Waves past their diagonal keep feeding the loads the others depend on.
+  for (; t < ntiles; ++t) {
+    if (t + 2 < ntiles) load_k(t + 2, t & 1);
+    if (t + 1 < ntiles) load_v(t + 1, (t & 1) ^ 1);
+    fa_wait_loads();
     __syncthreads();
   }
-  if (ntiles > 0) process(ntiles - 1);
 
   // ---- epilogue -------------------------------------------------------------------
-  if (!wave_active) return;
-  const float l = l_run + swap_half(l_run);
-  if (qi >= p.Sq) return;
-  const float inv = l > 0.f ? 1.0f / l : 0.f;
-  const long row = (long)(b * p.Hq + hq) * p.Sq + qi;
-  if (p.LSE && lh == 0)
-    p.LSE[row] = l > 0.f ? (m_run * c + __log2f(l)) * 0.69314718055994530942f : -INFINITY;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int qt = 0; qt < QT; ++qt) {
+    const int qi = qw + 32 * qt + l32;
+    const float l = l_run[qt] + swap_half(l_run[qt]);
+    if (qi >= p.Sq) continue;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    const long row = (long)(b * p.Hq + hq) * p.Sq + qi;
+    if (p.LSE && lh == 0)
+      p.LSE[row] = l > 0.f ? (m_run[qt] * c + __log2f(l)) * 0.69314718055994530942f : -INFINITY;
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      const int d = dt * 32 + 8 * a + 4 * lh;
-      const float v0 = o_acc[dt][4 * a + 0] * inv, v1 = o_acc[dt][4 * a + 1] * inv;
-      const float v2 = o_acc[dt][4 * a + 2] * inv, v3 = o_acc[dt][4 * a + 3] * inv;
-      if (p.out_storage) {
-        uint2 pk;
-        pk.x = pack2<T>(v0, v1);
-        pk.y = pack2<T>(v2, v3);
-        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.O) + row * D + d) = pk;
-      } else {
-        *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.O) + row * D + d) = make_float4(v0, v1, v2, v3);
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const int d = dt * 32 + 8 * a + 4 * lh;
+        const float v0 = o_acc[qt][dt][4 * a + 0] * inv, v1 = o_acc[qt][dt][4 * a + 1] * inv;
+        const float v2 = o_acc[qt][dt][4 * a + 2] * inv, v3 = o_acc[qt][dt][4 * a + 3] * inv;
+        if (p.out_storage) {
+          uint2 pk;
+          pk.x = pack2<T>(v0, v1);
+          pk.y = pack2<T>(v2, v3);
+          *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.O) + row * D + d) = pk;
+        } else {
+          *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.O) + row * D + d) = make_float4(v0, v1, v2, v3);
+        }
       }
-    }
+  }
 }
 
 // Any head dimension: one thread per query row, streaming online softmax in f32.

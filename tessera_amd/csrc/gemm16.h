@@ -137,19 +137,30 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   char* Db = (char*)p.D;
   constexpr int DSZ = (EPI == EPI_F32) ? 4 : 2;
   if constexpr (GROUPED) {
-    // blockIdx.x = n tile, blockIdx.y = running m-tile index over all groups.
-    tn = blockIdx.x;
-    int want = blockIdx.y, e = 0, acc_tiles = 0, g_lo = 0, g_hi = 0;
-    bool found = false;
+    // 1-D grid over the real tiles of all groups, ordered group-major, then n tile,
+    // then m tile.  Workgroup ids are dealt to the 8 XCDs round-robin, so XCD j takes
+    // the j-th contiguous eighth of that order: the tiles running together on one XCD
+    // then belong to one or two experts and share its weight slabs and row tiles in
+    // that XCD's L2.  The grid is sized from an upper bound; surplus blocks exit.
+    int total_m = 0;
+    for (int g = 0; g < p.groups; ++g) total_m += (p.offsets[g + 1] - p.offsets[g] + BM - 1) / BM;
+    const int total = total_m * p.tiles_n;
+    const int per = (total + 7) / 8;
+    const int slot = blockIdx.x >> 3;
+    const int lin = (blockIdx.x & 7) * per + slot;
+    if (slot >= per || lin >= total) return;
+    int e = 0, acc = 0, g_lo = 0, g_hi = 0, mt = 0;
     for (e = 0; e < p.groups; ++e) {
       g_lo = p.offsets[e];
       g_hi = p.offsets[e + 1];
-      const int t = (g_hi - g_lo + BM - 1) / BM;
-      if (want < acc_tiles + t) { found = true; break; }
-      acc_tiles += t;
+      mt = (g_hi - g_lo + BM - 1) / BM;
+      if (lin < acc + mt * p.tiles_n) break;
+      acc += mt * p.tiles_n;
     }
-    if (!found) return;
-    tm = want - acc_tiles;
+    if (e >= p.groups) return;
+    const int r = lin - acc;
+    tn = r / mt;
+    tm = r - tn * mt;
     m_begin = g_lo + tm * BM;
     m_end = g_hi;
     Bb += (long)e * p.strideB;

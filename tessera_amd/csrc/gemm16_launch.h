@@ -68,8 +68,9 @@ int launch_gemm16_tile(Gemm16Params p, hipStream_t s) {
   dim3 grid;
   if constexpr (GROUPED) {
     // every group contributes at most ceil(rows/BM) <= rows/BM + 1 tiles
+    // (+8: the kernel deals ceil(real tiles / 8) slots to each of the 8 XCDs)
     p.tiles_m = p.M / BM + p.groups;
-    grid = dim3(p.tiles_n, p.tiles_m, 1);
+    grid = dim3(p.tiles_n * p.tiles_m + 8, 1, 1);
   } else {
     p.tiles_m = ceil_div(p.M, BM);
     grid = dim3(p.tiles_m * p.tiles_n, 1, p.groups);
