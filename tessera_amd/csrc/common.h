@@ -93,6 +93,18 @@ __device__ __forceinline__ uint2 lds_read_tr8_b64(const char* p) {
   return __builtin_bit_cast(uint2, v);
 }
 
+// 16-byte buffer load: wave-uniform base (scalar registers) + 32-bit per-lane byte
+// offset.  The range is 2 GiB from the base; any offset at or past it (use
+// kOutOfRange) reads as zero without touching memory.
+constexpr uint32_t kBufferRange = 0x7fffffffu;
+constexpr uint32_t kOutOfRange = 0x80000000u;
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 buffer_load_b128(const void* base, uint32_t byte_off) {
+  __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, kBufferRange, 0x00020000);
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }

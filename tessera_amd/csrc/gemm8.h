@@ -6,12 +6,12 @@
 // Same structure as the 16-bit kernel: 256x256 output tile, 2x2 waves of 128x128,
 // K walked in steps of 128 bytes, LDS double buffered with one barrier per step,
 // operand fragments double buffered in registers.
-//   A tile  [256][128 B], 16-byte chunks XOR-swizzled by (row & 7), ds_read_b128.
-//   B tile  [128][256 + 16 B] natural layout; the operand (16 or 32 consecutive k
+//   A tile  [256][128 B], 16-byte chunks XOR-swizzled by ((row >> 1) & 7), ds_read_b128.
+//   B tile  [128][256 + 32 B] natural layout; the operand (16 or 32 consecutive k
 //           bytes of one column per lane) is read with the transposing
 //           ds_read_b64_tr_b8: a 16-lane block reads an 8(k) x 16(n) patch and
-//           every lane receives 8 consecutive k of one column.  The 16-byte row
-//           pad spreads the 8 rows of a patch over all banks.
+//           every lane receives 8 consecutive k of one column.  The 32-byte row
+//           pad interleaves the two patches a half-wave reads over all 64 banks.
 // Both operands enumerate k in the same order, which is all the MFMA needs: for
 // the 64-deep fp8 instruction a lane's 32 bytes are bytes [16h,16h+16) of two
 // consecutive 32-byte k groups rather than one contiguous run.
@@ -46,7 +46,7 @@ struct Gemm8Params {
 constexpr int G8_BK = 128;       // K step in bytes (= elements)
 constexpr int G8_BM = 256, G8_BN = 256;
 constexpr int G8_APITCH = 128;
-constexpr int G8_BPITCH = G8_BN + 16;
+constexpr int G8_BPITCH = G8_BN + 32;
 constexpr int G8_ASTAGE = G8_BM * G8_APITCH;
 constexpr int G8_BSTAGE = G8_BK * G8_BPITCH;
 constexpr int G8_STAGE = G8_ASTAGE + G8_BSTAGE;
@@ -88,59 +88,75 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
   const int m_begin = tm * G8_BM, n_begin = tn * G8_BN;
   const int K = p.K;
 
-  const uint8_t* a_ptr[A_CHUNKS];
-  uint32_t a_lds[A_CHUNKS];
+  // Global addressing: a wave-uniform tile base (advanced along K on the scalar unit)
+  // plus a fixed 32-bit per-lane offset, so a chunk costs one address register.
+  const uint8_t* a_base = p.A + (long)m_begin * K;
+  const uint8_t* b_base = p.B + n_begin;
+  uint32_t a_off[A_CHUNKS], a_lds[A_CHUNKS];
   const int a_chunk = tid & 7;
 #pragma unroll
   for (int q = 0; q < A_CHUNKS; ++q) {
     const int row = (tid >> 3) + 32 * q;
-    int gr = m_begin + row;
-    gr = gr < p.M ? gr : p.M - 1;
-    a_ptr[q] = p.A + (long)gr * K + a_chunk * 16;
-    a_lds[q] = row * G8_APITCH + ((a_chunk ^ (row & 7)) << 4);
+    int gr = row;
+    gr = m_begin + gr < p.M ? gr : p.M - 1 - m_begin;          // clamp: rows past the edge are never stored
+    a_off[q] = (uint32_t)gr * (uint32_t)K + a_chunk * 16;
+    a_lds[q] = row * G8_APITCH + ((a_chunk ^ ((row >> 1) & 7)) << 4);
   }
-  const uint8_t* b_ptr[B_CHUNKS];
-  uint32_t b_lds[B_CHUNKS];
+  uint32_t b_off[B_CHUNKS], b_lds[B_CHUNKS];
   int b_krow[B_CHUNKS];
 #pragma unroll
   for (int q = 0; q < B_CHUNKS; ++q) {
     const int v = tid + NT * q;
     const int krow = v / (G8_BN / 16), nch = v % (G8_BN / 16);
-    int gc = n_begin + nch * 16;
-    gc = gc < p.N ? gc : p.N - 16;
-    b_ptr[q] = p.B + (long)krow * p.N + gc;
+    int gc = nch * 16;
+    gc = n_begin + gc < p.N ? gc : p.N - 16 - n_begin;         // clamp: columns past the edge are never stored
+    b_off[q] = (uint32_t)krow * (uint32_t)p.N + gc;
     b_lds[q] = G8_ASTAGE + krow * G8_BPITCH + nch * 16;
     b_krow[q] = krow;
   }
 
-  uint4 ra[A_CHUNKS], rb[B_CHUNKS];
-  auto gload = [&](int k0, auto guarded_c) {
-    if constexpr (!decltype(guarded_c)::value) {
-#pragma unroll
-      for (int q = 0; q < A_CHUNKS; ++q) ra[q] = *reinterpret_cast<const uint4*>(a_ptr[q] + k0);
-#pragma unroll
-      for (int q = 0; q < B_CHUNKS; ++q) rb[q] = *reinterpret_cast<const uint4*>(b_ptr[q] + (long)k0 * p.N);
+  // Global -> register -> LDS staging.  Chunk q < A_CHUNKS is A chunk q, the rest are
+  // B chunks.  The chunks of a K step are split into KS groups; a group is written
+  // to LDS and immediately refilled with the same chunks of the K step two ahead,
+  // so every global load has a full K step of MFMA time to land and loads / LDS
+  // writes are spread evenly over it.
+  constexpr int NC = A_CHUNKS + B_CHUNKS;
+  constexpr int CPG = NC / KS;
+  static_assert(NC % KS == 0, "chunks must split evenly over the k steps");
+  uint4 st[NC];
+  using std::true_type;
+  using std::false_type;
+  // The guarded form is for a step that may be partial: out-of-range K must
+  // contribute exact zeros, which a buffer load returns by itself for an offset
+  // past the end of its range.
+  auto gload1 = [&](int q, int k0, auto guarded_c) {
+    constexpr bool GUARD = decltype(guarded_c)::value;
+    if (q < A_CHUNKS) {
+      uint32_t off = a_off[q];
+      if constexpr (GUARD) off = (k0 + a_chunk * 16 < K) ? off : kOutOfRange;
+      st[q] = buffer_load_b128(a_base + k0, off);
     } else {
-#pragma unroll
-      for (int q = 0; q < A_CHUNKS; ++q) {
-        const bool ok = k0 + a_chunk * 16 < K;
-        const uint4 v = *reinterpret_cast<const uint4*>(a_ptr[q] + (ok ? k0 : -(a_chunk * 16)));
-        ra[q].x = ok ? v.x : 0u; ra[q].y = ok ? v.y : 0u; ra[q].z = ok ? v.z : 0u; ra[q].w = ok ? v.w : 0u;
-      }
-#pragma unroll
-      for (int q = 0; q < B_CHUNKS; ++q) {
-        const bool ok = k0 + b_krow[q] < K;
-        const uint4 v = *reinterpret_cast<const uint4*>(b_ptr[q] + (ok ? (long)k0 : -(long)b_krow[q]) * p.N);
-        rb[q].x = ok ? v.x : 0u; rb[q].y = ok ? v.y : 0u; rb[q].z = ok ? v.z : 0u; rb[q].w = ok ? v.w : 0u;
-      }
+      const int qb = q - A_CHUNKS;
+      uint32_t off = b_off[qb];
+      if constexpr (GUARD) off = (k0 + b_krow[qb] < K) ? off : kOutOfRange;
+      st[q] = buffer_load_b128(b_base + (long)k0 * p.N, off);
     }
   };
-  auto lstore = [&](int buf) {
+  auto lstore1 = [&](int q, int buf) {
     char* base = smem + buf * G8_STAGE;
+    if (q < A_CHUNKS) lds_write_b128(base, a_lds[q], st[q]);
+    else lds_write_b128(base, b_lds[q - A_CHUNKS], st[q]);
+  };
+  // Group g: write its chunks and refill them.  MODE 0 = no refill, 1 = full step,
+  // 2 = possibly partial step.
+  auto stream_group = [&](int g, int buf_dst, int k0_load, auto mode_c) {
+    constexpr int MODE = decltype(mode_c)::value;
 #pragma unroll
-    for (int q = 0; q < A_CHUNKS; ++q) lds_write_b128(base, a_lds[q], ra[q]);
-#pragma unroll
-    for (int q = 0; q < B_CHUNKS; ++q) lds_write_b128(base, b_lds[q], rb[q]);
+    for (int q = g * CPG; q < (g + 1) * CPG; ++q) {
+      lstore1(q, buf_dst);
+      if constexpr (MODE == 1) gload1(q, k0_load, false_type{});
+      if constexpr (MODE == 2) gload1(q, k0_load, true_type{});
+    }
   };
 
   uint32_t a_rd[MI];
@@ -149,7 +165,7 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
   for (int i = 0; i < MI; ++i) {
     const int row = wm * 128 + i * 32 + l32;
     a_rd[i] = row * G8_APITCH;
-    a_sw[i] = row & 7;
+    a_sw[i] = (row >> 1) & 7;
   }
   // Transposing byte read: lane r of a 16-lane block supplies row k0 + r/2 and
   // columns n0 + 8 (r % 2) .. +7; lane i receives column n0 + i, k0 .. k0+7.
@@ -206,41 +222,81 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
       }
   };
 
+  // Scheduling hint for one k step of NM MFMAs carrying RD operand reads and (when
+  // streaming) CPG LDS writes + CPG global loads: the reads ride the first MFMAs,
+  // the write/load pairs the last ones, so every memory instruction issues in the
+  // shadow of an MFMA instead of in a burst.
+  constexpr int NM = MI * NJ, RD = FR * (MI + 2 * NJ);
+  auto hint_step = [&](auto stream_c, auto loads_c) {
+    constexpr bool STREAM = decltype(stream_c)::value;
+    constexpr bool LOADS = decltype(loads_c)::value;
+    constexpr int WSLOTS = CPG < NM / 2 ? CPG : NM / 2;
+    constexpr int wslots = STREAM ? WSLOTS : 0;
+    constexpr int rslots = NM - wslots;
+    constexpr int rper = (RD + rslots - 1) / rslots;
+    constexpr int wper = (CPG + WSLOTS - 1) / WSLOTS;
+#pragma unroll
+    for (int x = 0; x < NM; ++x) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (x < rslots) {
+        __builtin_amdgcn_sched_group_barrier(0x100, rper, 0);
+      } else {
+        __builtin_amdgcn_sched_group_barrier(0x200, wper, 0);
+        if constexpr (LOADS) __builtin_amdgcn_sched_group_barrier(0x020, wper, 0);
+      }
+    }
+  };
+
   const int ktiles = (K + G8_BK - 1) / G8_BK;
-  using std::true_type;
-  using std::false_type;
-  using no_prefetch = std::integral_constant<int, 0>;
-  using full_prefetch = std::integral_constant<int, 1>;
-  using tail_prefetch = std::integral_constant<int, 2>;
-  gload(0, true_type{});
-  lstore(0);
+  using mode0 = std::integral_constant<int, 0>;
+  using mode1 = std::integral_constant<int, 1>;
+  using mode2 = std::integral_constant<int, 2>;
+
+  // ---- prologue: K step 0 in buffer 0, group 0 of step 1 in buffer 1, the rest of
+  // step 1 and group 0 of step 2 in registers ---------------------------------------
+#pragma unroll
+  for (int q = 0; q < NC; ++q) gload1(q, 0, true_type{});
+#pragma unroll
+  for (int q = 0; q < NC; ++q) lstore1(q, 0);
+  if (ktiles > 1) {
+#pragma unroll
+    for (int q = 0; q < NC; ++q) gload1(q, G8_BK, true_type{});
+    if (ktiles > 2) stream_group(0, 1, 2 * G8_BK, mode2{});
+    else stream_group(0, 1, 0, mode0{});
+  }
   __syncthreads();
-  if (ktiles > 1) gload(G8_BK, true_type{});
   frag_load(0, 0, 0);
 
-  auto kstep = [&](int kt, auto more_c, auto prefetch_c) {
-    constexpr bool MORE = decltype(more_c)::value;
-    constexpr int PREFETCH = decltype(prefetch_c)::value;
+  // One K step.  HAS1: step kt+1 exists (its groups 1.. go to the other buffer during
+  // k steps 0..KS-2).  L2 / L3: how steps kt+2 / kt+3 are fetched (0 absent, 1 full,
+  // 2 possibly partial).  All compile-time: one straight-line block per barrier
+  // interval, with a single load form inside the hot loop.
+  auto kstep = [&](int kt, auto has1_c, auto l2_c, auto l3_c) {
+    constexpr bool HAS1 = decltype(has1_c)::value;
+    constexpr int L2 = decltype(l2_c)::value;
+    constexpr int L3 = decltype(l3_c)::value;
     const int buf = kt & 1;
 #pragma unroll
     for (int ks = 0; ks < KS - 1; ++ks) {
       frag_load(buf, ks + 1, (ks + 1) & 1);
-      if (MORE && ks == KS - 2) lstore(buf ^ 1);
+      if constexpr (HAS1) stream_group(ks + 1, buf ^ 1, (kt + 2) * G8_BK, l2_c);
       mma(ks & 1);
+      hint_step(std::integral_constant<bool, HAS1>{}, std::integral_constant<bool, (L2 != 0)>{});
+      __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
-    if constexpr (MORE) {
-      if constexpr (PREFETCH == 1) gload((kt + 2) * G8_BK, false_type{});
-      if constexpr (PREFETCH == 2) gload((kt + 2) * G8_BK, true_type{});
-      frag_load(buf ^ 1, 0, KS & 1);
-    }
+    if constexpr (HAS1) frag_load(buf ^ 1, 0, KS & 1);
+    if constexpr (L2 != 0) stream_group(0, buf, (kt + 3) * G8_BK, l3_c);
     mma((KS - 1) & 1);
+    if constexpr (HAS1) hint_step(std::integral_constant<bool, (L2 != 0)>{}, std::integral_constant<bool, (L3 != 0)>{});
+    __builtin_amdgcn_sched_barrier(0);
   };
   int kt = 0;
-  for (; kt + 3 < ktiles; ++kt) kstep(kt, true_type{}, full_prefetch{});
-  if (kt + 2 < ktiles) { kstep(kt, true_type{}, tail_prefetch{}); ++kt; }
-  if (kt + 1 < ktiles) { kstep(kt, true_type{}, no_prefetch{}); ++kt; }
-  kstep(kt, false_type{}, no_prefetch{});
+  for (; kt + 4 < ktiles; ++kt) kstep(kt, true_type{}, mode1{}, mode1{});
+  if (kt + 3 < ktiles) { kstep(kt, true_type{}, mode1{}, mode2{}); ++kt; }
+  if (kt + 2 < ktiles) { kstep(kt, true_type{}, mode2{}, mode0{}); ++kt; }
+  if (kt + 1 < ktiles) { kstep(kt, true_type{}, mode0{}, mode0{}); ++kt; }
+  kstep(kt, false_type{}, mode0{}, mode0{});
 
   // acc[i][j][r]: row m = 32 i + l32, col n = 32 j + 8 (r / 4) + 4 h + (r % 4).
 #pragma unroll
