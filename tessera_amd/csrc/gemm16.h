@@ -69,12 +69,6 @@ constexpr int G16_APITCH = 128;     // bytes per A row in LDS
 #ifndef TSR_ASWZ
 #define TSR_ASWZ(row) (((row) >> 1) & 7)
 #endif
-#ifndef TSR_EARLY_GLOAD
-#define TSR_EARLY_GLOAD 0
-#endif
-#ifndef TSR_WRITES_LATE
-#define TSR_WRITES_LATE 0
-#endif
 constexpr int G16_BPAD = TSR_BPAD;  // B row pad, elements
 
 template <int BM, int BN>
@@ -178,45 +172,43 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   const int n_begin = tn * BN_OUT;
   const int K = p.K;
 
-  // ---- global load addressing (fixed per thread, advanced by BK each step) --
+  // ---- global load addressing ----------------------------------------------------
+  // Buffer loads: a wave-uniform tile base (advanced along K on the scalar unit) plus
+  // a fixed 32-bit per-lane byte offset, one address register per chunk.
   // A: chunk v = tid + NT*q  -> row v/8, 16-byte chunk v%8.
-  const uint16_t* a_ptr[A_CHUNKS];
-  uint32_t a_lds[A_CHUNKS];
+  const uint16_t* a_base = Ab + (long)m_begin * p.lda;
+  uint32_t a_off[A_CHUNKS], a_lds[A_CHUNKS];
   const int a_chunk = tid & 7;
 #pragma unroll
   for (int q = 0; q < A_CHUNKS; ++q) {
     const int row = (tid >> 3) + (NT / 8) * q;
-#ifdef TSR_ABL_SAMETILE
     int gr = row;
-#else
-    int gr = m_begin + row;
-#endif
-    gr = gr < m_end ? gr : m_end - 1;            // clamp: rows past the edge are never stored
-    a_ptr[q] = Ab + (long)gr * p.lda + a_chunk * 8;
+    gr = m_begin + gr < m_end ? gr : m_end - 1 - m_begin;   // clamp: rows past the edge are never stored
+    a_off[q] = ((uint32_t)gr * (uint32_t)p.lda + a_chunk * 8) * 2;
     a_lds[q] = row * G16_APITCH + ((a_chunk ^ TSR_ASWZ(row)) << 4);
   }
-  // B: chunk v = tid + NT*q -> k row v/(BN/8), n chunk v%(BN/8).
-  const uint16_t* b_ptr[B_CHUNKS];
-  uint32_t b_lds[B_CHUNKS];
+  // B: the tile's columns come from one matrix, or (SwiGLU) half from the gate and
+  // half from the up matrix; the first B_CHUNKS / HALVES chunks of a thread belong to
+  // the first source.  Within a source: chunk v = tid + NT*q' -> k row v/CPR, n chunk v%CPR.
+  constexpr int HALVES = SWIGLU ? 2 : 1;
+  constexpr int CPR = BN / HALVES / 8;           // 16-byte chunks per row and source
+  constexpr int B_PER = B_CHUNKS / HALVES;
+  static_assert(B_CHUNKS % HALVES == 0, "B chunks must split over the sources");
+  const uint16_t* b_base[HALVES];
+  b_base[0] = Bb + n_begin;
+  if constexpr (SWIGLU) b_base[1] = B2b + n_begin;
+  uint32_t b_off[B_CHUNKS], b_lds[B_CHUNKS];
   int b_krow[B_CHUNKS];
 #pragma unroll
   for (int q = 0; q < B_CHUNKS; ++q) {
-    const int v = tid + NT * q;
-    const int krow = v / (BN / 8);
-    const int nch = v % (BN / 8);
-    const uint16_t* src = Bb;
+    const int half = q / B_PER;
+    const int v = tid + NT * (q % B_PER);
+    const int krow = v / CPR;
+    const int nch = v % CPR;
     int col = nch * 8;
-    if constexpr (SWIGLU) {
-      if (col >= BN / 2) { src = B2b; col -= BN / 2; }
-    }
-#ifdef TSR_ABL_SAMETILE
-    int gc = col;
-#else
-    int gc = n_begin + col;
-#endif
-    gc = gc < p.N ? gc : (p.N - 8);              // clamp: columns past the edge are never stored
-    b_ptr[q] = src + (long)krow * p.ldb + gc;
-    b_lds[q] = S::kAStage + krow * S::kBPitch + nch * 16;
+    col = n_begin + col < p.N ? col : p.N - 8 - n_begin;    // clamp: columns past the edge are never stored
+    b_off[q] = ((uint32_t)krow * (uint32_t)p.ldb + col) * 2;
+    b_lds[q] = S::kAStage + krow * S::kBPitch + (half * CPR + nch) * 16;
     b_krow[q] = krow;
   }
 
@@ -235,35 +227,21 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   using std::false_type;
   // Load chunk q of the K step starting at k0.  The guarded form is for a step
   // that may be partial: out-of-range K must contribute exact zeros on both
-  // operands, so the address is pulled back in range and the value replaced.
+  // operands, which a buffer load returns by itself for an offset past its range.
   auto gload1 = [&](int q, int k0, auto guarded_c) {
-#ifdef TSR_ABL_NOGLOAD
-    if (k0 > 0) return;
-#endif
     constexpr bool GUARD = decltype(guarded_c)::value;
     if (q < A_CHUNKS) {
-      if constexpr (!GUARD) {
-        st[q] = *reinterpret_cast<const uint4*>(a_ptr[q] + k0);
-      } else {
-        const bool ok = k0 + a_chunk * 8 < K;
-        const uint4 v = *reinterpret_cast<const uint4*>(a_ptr[q] + (ok ? k0 : -(a_chunk * 8)));
-        st[q].x = ok ? v.x : 0u; st[q].y = ok ? v.y : 0u; st[q].z = ok ? v.z : 0u; st[q].w = ok ? v.w : 0u;
-      }
+      uint32_t off = a_off[q];
+      if constexpr (GUARD) off = (k0 + a_chunk * 8 < K) ? off : kOutOfRange;
+      st[q] = buffer_load_b128(a_base + k0, off);
     } else {
       const int qb = q - A_CHUNKS;
-      if constexpr (!GUARD) {
-        st[q] = *reinterpret_cast<const uint4*>(b_ptr[qb] + (long)k0 * p.ldb);
-      } else {
-        const bool ok = k0 + b_krow[qb] < K;
-        const uint4 v = *reinterpret_cast<const uint4*>(b_ptr[qb] + (ok ? (long)k0 : -(long)b_krow[qb]) * p.ldb);
-        st[q].x = ok ? v.x : 0u; st[q].y = ok ? v.y : 0u; st[q].z = ok ? v.z : 0u; st[q].w = ok ? v.w : 0u;
-      }
+      uint32_t off = b_off[qb];
+      if constexpr (GUARD) off = (k0 + b_krow[qb] < K) ? off : kOutOfRange;
+      st[q] = buffer_load_b128(b_base[qb / B_PER] + (long)k0 * p.ldb, off);
     }
   };
   auto lstore1 = [&](int q, int buf) {
-#ifdef TSR_ABL_NOLSTORE
-    return;
-#endif
     char* base = smem + buf * S::kStage;
     if (q < A_CHUNKS) lds_write_b128(base, a_lds[q], st[q]);
     else lds_write_b128(base, b_lds[q - A_CHUNKS], st[q]);
@@ -308,9 +286,6 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   // step s+1 are issued before the MFMAs of step s, which hide their latency.
   uint4 af[2][MI], bf[2][NJ];
   auto frag_load = [&](int buf, int ks, int slot) {
-#ifdef TSR_ABL_NOFRAG
-    if (ks > 0 || buf > 0) return;
-#endif
     const char* base = smem + buf * S::kStage;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
@@ -397,9 +372,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     // Every wave has issued all its reads of this buffer and all its writes of
     // the other one; past the barrier the other buffer is complete and this one
     // is free to take group 0 of step kt+2.
-#ifndef TSR_ABL_NOBARRIER
     __syncthreads();
-#endif
     if constexpr (HAS1) frag_load(buf ^ 1, 0, KS & 1);
     if constexpr (L2 != 0) stream_group(0, buf, (kt + 3) * G16_BK, l3_c);
     mma((KS - 1) & 1);

@@ -83,7 +83,9 @@ int launch_gemm16_tile(Gemm16Params p, hipStream_t s) {
 template <class T, int EPI>
 int launch_gemm16(Gemm16Params p, hipStream_t s) {
   const int dsz = (EPI == EPI_F32) ? 4 : 2;
+  // (32-bit per-lane byte offsets inside a tile bound the leading dimensions)
   const bool vec = (p.K % 8 == 0) && (p.N % 8 == 0) && (p.lda % 8 == 0) && (p.ldb % 8 == 0) &&
+                   (p.lda < (1L << 21)) && (p.ldb < (1L << 21)) &&
                    ((p.ldd * dsz) % (dsz * 4) == 0) && (p.strideA % 8 == 0) && (p.strideB % 8 == 0) &&
                    ((p.strideD * dsz) % 16 == 0) && aligned16(p.A) && aligned16(p.B) && aligned16(p.D);
   if (!vec) {
@@ -102,7 +104,9 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
 template <class T, int EPI>
 int launch_gemm16_grouped(Gemm16Params p, hipStream_t s) {
   const int dsz = (EPI == EPI_F32) ? 4 : 2;
+  // (32-bit per-lane byte offsets inside a tile bound the leading dimensions)
   const bool vec = (p.K % 8 == 0) && (p.N % 8 == 0) && (p.lda % 8 == 0) && (p.ldb % 8 == 0) &&
+                   (p.lda < (1L << 21)) && (p.ldb < (1L << 21)) &&
                    ((p.ldd * dsz) % (dsz * 4) == 0) && (p.strideB % 8 == 0) && aligned16(p.A) &&
                    aligned16(p.B) && aligned16(p.D) && (EPI != EPI_SWIGLU16 || aligned16(p.B2));
   if (!vec) {

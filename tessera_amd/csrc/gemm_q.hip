@@ -15,7 +15,8 @@ int gemm8_dev(Gemm8Params p, hipStream_t s) {
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || !p.A || !p.B || !p.D) return kBadShape;
   if (EPI == EPI8_W8A8_F32 && (!p.row_scale || !p.col_scale)) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
-  const bool vec = (p.K % 16 == 0) && (p.N % 16 == 0) && aligned16(p.A) && aligned16(p.B) && aligned16(p.D) &&
+  // (32-bit per-lane byte offsets inside a tile bound K and N)
+  const bool vec = (p.K % 16 == 0) && (p.N % 16 == 0) && (p.K < (1 << 22)) && (p.N < (1 << 22)) && aligned16(p.A) && aligned16(p.B) && aligned16(p.D) &&
                    (!p.acc_out || aligned16(p.acc_out)) && (!p.col_scale || aligned16(p.col_scale));
   if (!vec) {
     dim3 block(32, 8), grid(ceil_div(p.N, 32), ceil_div(p.M, 8), 1);
