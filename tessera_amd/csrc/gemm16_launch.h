@@ -1,5 +1,6 @@
 // Host-side tile selection and launch for the 16-bit MFMA GEMM family.
 #pragma once
+#include <algorithm>
 #include <mutex>
 #include "gemm16.h"
 #include "host_util.h"
@@ -79,6 +80,31 @@ int launch_gemm16_tile(Gemm16Params p, hipStream_t s) {
   return launch_status();
 }
 
+// D[m][n] = sum over splits (in split order) of the f32 partials, stored as f32 or in
+// the storage dtype; four columns per thread (N % 8 == 0 on this path).
+template <class T, int EPI>
+__global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restrict__ D, int M, int N, long ldd,
+                                     int splits) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const int nq = N / 4;
+  if (i >= (long)M * nq) return;
+  const int m = (int)(i / nq), n = (int)(i % nq) * 4;
+  const size_t mn = (size_t)M * N;
+  float4 acc = *reinterpret_cast<const float4*>(ws + (size_t)m * N + n);
+  for (int z = 1; z < splits; ++z) {
+    const float4 v = *reinterpret_cast<const float4*>(ws + z * mn + (size_t)m * N + n);
+    acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+  }
+  if constexpr (EPI == EPI_F32) {
+    *reinterpret_cast<float4*>(reinterpret_cast<float*>(D) + (long)m * ldd + n) = acc;
+  } else {
+    uint2 pk;
+    pk.x = pack2<T>(acc.x, acc.y);
+    pk.y = pack2<T>(acc.z, acc.w);
+    *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(D) + (long)m * ldd + n) = pk;
+  }
+}
+
 // Dense / batched.  p.groups = batch count (>= 1).
 template <class T, int EPI>
 int launch_gemm16(Gemm16Params p, hipStream_t s) {
@@ -96,7 +122,43 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
   const long tiles256 = (long)ceil_div(p.M, 256) * ceil_div(p.N, 256) * p.groups;
   const long tiles128 = (long)ceil_div(p.M, 128) * ceil_div(p.N, 128) * p.groups;
   if (tiles256 >= 192) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false>(p, s);
-  if (tiles128 >= 192 || (p.M >= 128 && p.N >= 128)) return launch_gemm16_tile<T, 128, 128, 2, 2, EPI, false>(p, s);
+  const bool t128 = tiles128 >= 192 || (p.M > 64 && p.N >= 128);
+  // Few output tiles and a long K (decode-shaped products: the weight matrix streams
+  // from HBM once): split K over enough workgroups to cover the chip.  Every split
+  // is one "batch" of the same kernel writing f32 partials, summed in split order
+  // by a second kernel, so the result does not depend on scheduling.
+  if (p.groups == 1) {
+    const long tiles = t128 ? tiles128 : (long)ceil_div(p.M, 64) * ceil_div(p.N, 64);
+    int splits = (int)std::min<long>((768 + tiles - 1) / tiles, p.K / 512);
+    while (splits > 1 && p.K % (splits * G16_BK) != 0) --splits;
+    if (splits > 1) {
+      float* ws = nullptr;
+      const size_t mn = (size_t)p.M * p.N;
+      if (hipMallocAsync(reinterpret_cast<void**>(&ws), mn * splits * sizeof(float), s) != hipSuccess) {
+        (void)hipGetLastError();
+        return kDeviceFailed;
+      }
+      Gemm16Params q = p;
+      q.K = p.K / splits;
+      q.groups = splits;
+      q.strideA = q.K;                       // split z reads A[:, z Ks ..) and B[z Ks .., :)
+      q.strideB = (long)q.K * p.ldb;
+      q.D = ws;
+      q.ldd = p.N;
+      q.strideD = (long)mn;
+      int rc = t128 ? launch_gemm16_tile<T, 128, 128, 2, 2, EPI_F32, false>(q, s)
+                    : launch_gemm16_tile<T, 64, 64, 2, 2, EPI_F32, false>(q, s);
+      if (rc == kOk) {
+        const long quads = (long)p.M * (p.N / 4);
+        hipLaunchKernelGGL((splitk_reduce_kernel<T, EPI>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s,
+                           ws, p.D, p.M, p.N, p.ldd, splits);
+        rc = launch_status();
+      }
+      if (hipFreeAsync(ws, s) != hipSuccess) { (void)hipGetLastError(); rc = rc == kOk ? kDeviceFailed : rc; }
+      return rc;
+    }
+  }
+  if (t128) return launch_gemm16_tile<T, 128, 128, 2, 2, EPI, false>(p, s);
   return launch_gemm16_tile<T, 64, 64, 2, 2, EPI, false>(p, s);
 }
 

@@ -109,6 +109,10 @@ def test_decode_shapes(lane):
         ref = ab.to_float32().astype(np.float64) @ Bq
         got = ops.gemm(ab, bb, out="f32")
         assert orc.max_rel_err(got, ref) <= 1e-5
+        # split-K partials are summed in a fixed order: the stored result is the
+        # RNE of the same accumulators, and a second run is bit-identical
+        assert np.array_equal(ops.gemm(ab, bb).to_float32(), orc.round_to_storage(got, "bf16"))
+        assert np.array_equal(ops.gemm(ab, bb, out="f32"), got)
 
 
 def test_full_size_bf16_gemm_properties(lane):
