@@ -126,6 +126,34 @@ int tessera_gfx950_gemm_e4m3_bf16_dev(const void* A, const void* B, float scale_
 int tessera_gfx950_gemm_e4m3_f32_dev(const void* A, const void* B, float scale_a, float scale_b,
                                      void* D, int M, int N, int K, void* stream);
 
+/* Fused matmul epilogue  D f32 = act(A . B + bias[n]):  the bias operand and
+ * `activation` kwarg of the compiled-GEMM executor's tessera.fused_epilogue op
+ * (python/tessera/runtime.py:6603-6650) and the (has_bias, activation) epilogue of
+ * the matrix-core candidate (python/tessera/compiler/emit/rocm_hip.py:679-699).
+ * bias is f32[N] or NULL; activation: 0 none, 1 relu, 2 gelu (tanh form, argument
+ * clamped to +-30), 3 silu, 4 sigmoid, 5 tanh — the reference's epilogue
+ * vocabulary (python/tessera/compiler/fusion_core.py:121-138).  Any other code is
+ * a bad-shape error. */
+int tessera_gfx950_gemm_bias_act_f16(const void* A, const void* B, const float* bias, int activation,
+                                     void* D, int M, int N, int K);
+int tessera_gfx950_gemm_bias_act_bf16(const void* A, const void* B, const float* bias, int activation,
+                                      void* D, int M, int N, int K);
+int tessera_gfx950_gemm_bias_act_f16_dev(const void* A, const void* B, const float* bias, int activation,
+                                         void* D, int M, int N, int K, void* stream);
+int tessera_gfx950_gemm_bias_act_bf16_dev(const void* A, const void* B, const float* bias, int activation,
+                                          void* D, int M, int N, int K, void* stream);
+/* Gated projection  D f32 [M,H] = act(A . Wg) * (A . Wu),  A [M,K], Wg/Wu [K,H]:
+ * GatedMatmulRegion (python/tessera/compiler/fusion_core.py:747-782); f32
+ * accumulators go through the activation and the product unrounded. */
+int tessera_gfx950_gated_gemm_f16(const void* A, const void* Wg, const void* Wu, int activation, void* D,
+                                  int M, int H, int K);
+int tessera_gfx950_gated_gemm_bf16(const void* A, const void* Wg, const void* Wu, int activation, void* D,
+                                   int M, int H, int K);
+int tessera_gfx950_gated_gemm_f16_dev(const void* A, const void* Wg, const void* Wu, int activation, void* D,
+                                      int M, int H, int K, void* stream);
+int tessera_gfx950_gated_gemm_bf16_dev(const void* A, const void* Wg, const void* Wu, int activation, void* D,
+                                       int M, int H, int K, void* stream);
+
 /* Kernel-only benchmark with resident, library-owned buffers: warm-up, `iters`
  * launches between HIP events, cross-checked against wall clock
  * (tessera_rocm_gemm.cpp:551-667).  *avg_ms = mean per-launch ms. */

@@ -25,6 +25,8 @@ flash_attn (+GQA, +LSE)    dense textbook softmax in f64; row 0 -> V[0];
                            ``tessera_x86_flash_attn_ext_lse_f32``
 route_tokens / moe_layer   brute force on tiny inputs; partition invariants;
                            agreement of the two routers' expert sets
+fused epilogue / gated     torch.nn.functional relu / gelu(tanh) / silu / sigmoid /
+                           tanh library cross-check; relu and zero-bias closed forms
 grouped_gemm / swiglu      per-group matmul; E=1 reduces to dense SwiGLU
 quantize_int8 / W8A8       exact integer arithmetic; compiled reference twin
                            ``tessera_x86_reference_gemm_u8s8_s32`` on the
@@ -117,6 +119,51 @@ def gemm_storage(A: np.ndarray, B: np.ndarray, dtype: str = "bf16") -> np.ndarra
     lie on the storage grid).  ``__init__.py:5771-5781,5824-5855``.
     """
     return round_to_storage(gemm_f32(A, B, dtype), dtype)
+
+
+# ---------------------------------------------------------------------------
+# fused matmul epilogue and gated projection
+# ---------------------------------------------------------------------------
+
+
+def _gelu_tanh(x: np.ndarray) -> np.ndarray:
+    """``compiler/fusion_core.py:104-106``: tanh-form GELU, argument clamped to +-30."""
+    t = np.clip(0.7978845608028654 * (x + 0.044715 * x ** 3), -30.0, 30.0)
+    return 0.5 * x * (1.0 + np.tanh(t))
+
+
+#: the pointwise epilogue vocabulary (``compiler/fusion_core.py:121-138``)
+EPILOGUE_REFS = {
+    "relu": lambda x: np.maximum(x, 0.0),
+    "gelu": _gelu_tanh,
+    "silu": lambda x: x / (1.0 + np.exp(-x)),
+    "sigmoid": lambda x: 1.0 / (1.0 + np.exp(-x)),
+    "tanh": np.tanh,
+}
+
+
+def fused_epilogue(A, B, bias=None, epilogue=()) -> np.ndarray:
+    """Matmul then the ordered pointwise chain — ``FusedRegion.reference``
+    (``compiler/fusion_core.py:318-345``) for regions without prologue, residual or
+    reduction.  Computed in f64 on the given operands (round them to storage
+    first), returned as f32."""
+    out = np.asarray(A, np.float64) @ np.asarray(B, np.float64)
+    for op in epilogue:
+        if op == "bias":
+            if bias is None:
+                raise ValueError("region needs a bias")
+            out = out + np.asarray(bias, np.float64)
+        else:
+            out = EPILOGUE_REFS[op](out)
+    return out.astype(np.float32)
+
+
+def gated_matmul(A, Wg, Wu, gate_act: str = "silu") -> np.ndarray:
+    """``act(A @ Wg) * (A @ Wu)`` — ``GatedMatmulRegion.reference``
+    (``compiler/fusion_core.py:776-782``), f64 inside, f32 out."""
+    a = np.asarray(A, np.float64)
+    gate = EPILOGUE_REFS[gate_act](a @ np.asarray(Wg, np.float64))
+    return (gate * (a @ np.asarray(Wu, np.float64))).astype(np.float32)
 
 
 # ---------------------------------------------------------------------------

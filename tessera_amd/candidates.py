@@ -53,6 +53,8 @@ TARGET = "rocm_gfx950"
 GEMM_TAG = "gfx950_mfma_gemm"
 ATTN_TAG = "gfx950_mfma_flash_attn"
 GROUPED_TAG = "gfx950_mfma_grouped_gemm"
+FUSED_TAG = "gfx950_mfma_fused_gemm"
+GATED_TAG = "gfx950_mfma_gated_gemm"
 
 
 class ArbiterError(RuntimeError):
@@ -122,6 +124,76 @@ class AttentionRegion:
         s = s - s.max(-1, keepdims=True)
         e = np.exp(s)
         return ((e / e.sum(-1, keepdims=True)) @ V).astype(np.float32)
+
+
+def _gelu(x):
+    t = np.clip(0.7978845608028654 * (x + 0.044715 * x ** 3), -30.0, 30.0)
+    return 0.5 * x * (1.0 + np.tanh(t))
+
+
+#: numpy side of the pointwise epilogue vocabulary (``fusion_core.py:121-138``)
+EPILOGUE_REFS: dict = {
+    "bias": None,
+    "relu": lambda x: np.maximum(x, 0.0),
+    "gelu": _gelu,
+    "silu": lambda x: x / (1.0 + np.exp(-x)),
+    "sigmoid": lambda x: 1.0 / (1.0 + np.exp(-x)),
+    "tanh": np.tanh,
+}
+
+
+@dataclass(frozen=True)
+class FusedRegion:
+    """``fusion_core.FusedRegion`` (``:226-345``): a matmul root plus an ordered
+    pointwise epilogue chain.  The fields the gfx950 candidate cannot honour
+    (reduction, residual, prologue) are carried so it can decline them."""
+    epilogue: tuple = ()
+    reduction: Optional[str] = None
+    residual: bool = False
+    prologue: tuple = ()
+    storage_dtype: str = "f16"
+
+    def __post_init__(self) -> None:
+        for op in self.epilogue:
+            if op not in EPILOGUE_REFS:
+                raise ValueError(f"E_FUSED_EPILOGUE_BAD_OP: unknown epilogue op {op!r}")
+        if sum(1 for op in self.epilogue if op == "bias") > 1:
+            raise ValueError("E_FUSED_EPILOGUE_BAD_ORDER: at most one bias op per region")
+
+    @property
+    def has_bias(self) -> bool:
+        return "bias" in self.epilogue
+
+    def reference(self, A, B, bias=None, residual=None) -> np.ndarray:
+        out = np.asarray(A, np.float32) @ np.asarray(B, np.float32)
+        for op in self.epilogue:
+            if op == "bias":
+                if bias is None:
+                    raise ValueError("E_FUSED_EPILOGUE_MISSING_OPERAND: region needs a bias for 'bias'")
+                out = out + np.asarray(bias, np.float32)
+            else:
+                out = EPILOGUE_REFS[op](out)
+        if self.residual:
+            if residual is None:
+                raise ValueError("E_FUSED_EPILOGUE_MISSING_OPERAND: region needs a residual")
+            out = out + np.asarray(residual, np.float32)
+        return out.astype(np.float32)
+
+
+@dataclass(frozen=True)
+class GatedMatmulRegion:
+    """``fusion_core.GatedMatmulRegion`` (``:747-782``): ``act(A Wg) * (A Wu)``."""
+    gate_act: str = "silu"
+    storage_dtype: str = "f16"
+
+    def __post_init__(self) -> None:
+        if self.gate_act not in EPILOGUE_REFS or self.gate_act == "bias":
+            raise ValueError(f"gate activation must be a unary pointwise op, got {self.gate_act!r}")
+
+    def reference(self, A, Wg, Wu) -> np.ndarray:
+        a = np.asarray(A, np.float32)
+        gate = EPILOGUE_REFS[self.gate_act](a @ np.asarray(Wg, np.float32))
+        return (gate * (a @ np.asarray(Wu, np.float32))).astype(np.float32)
 
 
 @dataclass(frozen=True)
@@ -228,6 +300,20 @@ def verify_candidate(candidate: Candidate, region: Any, *, atol: float = 1e-3, s
         Q, K, V = ((rng.standard_normal((8, 16)) * .2).astype(np.float32) for _ in range(3))
         out, tag = candidate.run(region, Q, K, V)
         ref = region.reference(Q, K, V)
+    elif candidate.op == OP_FUSED_REGION:
+        # fusion_core.py:1046-1062
+        A = (rng.standard_normal((8, 12)) * .2).astype(np.float32)
+        B = (rng.standard_normal((12, 16)) * .2).astype(np.float32)
+        bias = (rng.standard_normal((16,)) * .2).astype(np.float32) if region.has_bias else None
+        out, tag = candidate.run(region, A, B, bias)
+        ref = region.reference(A, B, bias)
+    elif candidate.op == OP_GATED_MATMUL:
+        # fusion_core.py:809-822
+        A = (rng.standard_normal((8, 12)) * .2).astype(np.float32)
+        Wg = (rng.standard_normal((12, 16)) * .2).astype(np.float32)
+        Wu = (rng.standard_normal((12, 16)) * .2).astype(np.float32)
+        out, tag = candidate.run(region, A, Wg, Wu)
+        ref = region.reference(A, Wg, Wu)
     else:
         return False
     if tag in REFERENCE_EXECUTIONS:
@@ -431,12 +517,91 @@ class Gfx950GroupedGemmCandidate(Candidate):
         return out, GROUPED_TAG
 
 
+#: Activations the MFMA epilogue fuses after the optional bias.
+_MFMA_ACTS = ("relu", "gelu", "silu", "sigmoid", "tanh")
+
+
+def mfma_epilogue(region: Any):
+    """``(has_bias, activation)`` when ``region`` fits the kernel's epilogue — bias
+    first, then at most one activation, no reduction / residual / prologue — else
+    ``None``.  The rule of ``_wmma_epilogue`` (``emit/rocm_hip.py:679-699``)."""
+    if not isinstance(region, FusedRegion):
+        return None
+    if region.reduction is not None or region.residual or region.prologue:
+        return None
+    epi = list(region.epilogue)
+    has_bias = False
+    if epi and epi[0] == "bias":
+        has_bias = True
+        epi = epi[1:]
+    if not epi:
+        return has_bias, "none"
+    if len(epi) == 1 and epi[0] in _MFMA_ACTS:
+        return has_bias, epi[0]
+    return None
+
+
+class Gfx950FusedGemmCandidate(Candidate):
+    """Tier-3 matmul with the bias / activation epilogue fused on the MFMA GEMM."""
+    name = "gfx950_mfma_fused_gemm"
+    tier = Tier.HAND_TUNED
+    target = TARGET
+    op = OP_FUSED_REGION
+    accuracy_atol = 5e-3
+    mma_target = "rocm"
+    mma_arch = "gfx950"
+
+    def mma_dtype(self, region: Any) -> Optional[str]:
+        return "bf16" if getattr(region, "storage_dtype", "f16") == "bf16" else "fp16"
+
+    def available(self) -> bool:
+        return _lane.available()
+
+    def applies_to(self, region: Any) -> bool:
+        return mfma_epilogue(region) is not None and getattr(region, "storage_dtype", "f16") in ("f16", "bf16")
+
+    def run(self, region: Any, A: Any, B: Any, bias: Any = None, *a: Any, **k: Any) -> tuple:
+        epi = mfma_epilogue(region)
+        if epi is None:
+            raise ValueError("region's epilogue is not representable on the gfx950 fused GEMM")
+        has_bias, activation = epi
+        if has_bias and bias is None:
+            raise ValueError("E_FUSED_EPILOGUE_MISSING_OPERAND: region needs a bias")
+        dt = region.storage_dtype
+        out = _ops.fused_gemm(_to_storage(A, dt), _to_storage(B, dt), bias if has_bias else None, activation)
+        return out, FUSED_TAG
+
+
+class Gfx950GatedGemmCandidate(Candidate):
+    """Tier-3 gated projection ``act(A Wg) * (A Wu)`` in one MFMA kernel."""
+    name = "gfx950_mfma_gated_gemm"
+    tier = Tier.HAND_TUNED
+    target = TARGET
+    op = OP_GATED_MATMUL
+    accuracy_atol = 5e-3
+    mma_target = "rocm"
+    mma_arch = "gfx950"
+
+    def available(self) -> bool:
+        return _lane.available()
+
+    def applies_to(self, region: Any) -> bool:
+        return isinstance(region, GatedMatmulRegion) and region.storage_dtype in ("f16", "bf16")
+
+    def run(self, region: Any, A: Any, Wg: Any, Wu: Any, *a: Any, **k: Any) -> tuple:
+        dt = region.storage_dtype
+        out = _ops.gated_gemm(_to_storage(A, dt), _to_storage(Wg, dt), _to_storage(Wu, dt), region.gate_act)
+        return out, GATED_TAG
+
+
 def register_all() -> None:
     """Plug the lane's candidates in (idempotent), as each backend module does at
     import (``compiler/emit/rocm_hip.py:809-818``)."""
     register_candidate(Gfx950MfmaGemmCandidate())
     register_candidate(Gfx950FlashAttnCandidate())
     register_candidate(Gfx950GroupedGemmCandidate())
+    register_candidate(Gfx950FusedGemmCandidate())
+    register_candidate(Gfx950GatedGemmCandidate())
 
 
 register_all()

@@ -42,6 +42,79 @@ int gemm16_host(const void* A, const void* B, void* D, int batch, int M, int N, 
   return scope.download(D, dD, d_bytes) ? kOk : kDeviceFailed;
 }
 
+bool bad_activation(int act) { return act < ACT_NONE || act > ACT_TANH; }
+
+// D f32 = act(A B + bias): the fused matmul epilogue.
+template <class T>
+int fused_dev(const void* A, const void* B, const float* bias, int act, void* D, int M, int N, int K,
+              hipStream_t s) {
+  if (bad_dims(1, M, N, K) || !A || !B || !D || bad_activation(act)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  Gemm16Params p{};
+  p.A = static_cast<const uint16_t*>(A);
+  p.B = static_cast<const uint16_t*>(B);
+  p.D = D;
+  p.bias = bias;
+  p.act = act;
+  p.M = M; p.N = N; p.K = K;
+  p.lda = K; p.ldb = N; p.ldd = N;
+  p.strideA = (long)M * K; p.strideB = (long)K * N; p.strideD = (long)M * N;
+  p.groups = 1;
+  return launch_gemm16<T, EPI_F32>(p, s);
+}
+
+template <class T>
+int fused_host(const void* A, const void* B, const float* bias, int act, void* D, int M, int N, int K) {
+  if (bad_dims(1, M, N, K) || !A || !B || !D || bad_activation(act)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t d_bytes = (size_t)M * N * 4;
+  DeviceScope scope;
+  void* dA = scope.alloc((size_t)M * K * 2, A);
+  void* dB = scope.alloc((size_t)K * N * 2, B);
+  void* dBias = bias ? scope.alloc((size_t)N * 4, bias) : nullptr;
+  void* dD = scope.alloc(d_bytes);
+  if (scope.failed()) return kDeviceFailed;
+  int rc = fused_dev<T>(dA, dB, static_cast<const float*>(dBias), act, dD, M, N, K, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  return scope.download(D, dD, d_bytes) ? kOk : kDeviceFailed;
+}
+
+// D f32 [M,H] = act(A Wg) * (A Wu): the gated projection.
+template <class T>
+int gated_dev(const void* A, const void* Wg, const void* Wu, int act, void* D, int M, int H, int K,
+              hipStream_t s) {
+  if (bad_dims(1, M, H, K) || !A || !Wg || !Wu || !D || bad_activation(act)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  Gemm16Params p{};
+  p.A = static_cast<const uint16_t*>(A);
+  p.B = static_cast<const uint16_t*>(Wg);
+  p.B2 = static_cast<const uint16_t*>(Wu);
+  p.D = D;
+  p.act = act;
+  p.M = M; p.N = H; p.K = K;
+  p.lda = K; p.ldb = H; p.ldd = H;
+  p.groups = 1;
+  return launch_gemm16_gated<T>(p, s);
+}
+
+template <class T>
+int gated_host(const void* A, const void* Wg, const void* Wu, int act, void* D, int M, int H, int K) {
+  if (bad_dims(1, M, H, K) || !A || !Wg || !Wu || !D || bad_activation(act)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t d_bytes = (size_t)M * H * 4;
+  DeviceScope scope;
+  void* dA = scope.alloc((size_t)M * K * 2, A);
+  void* dG = scope.alloc((size_t)K * H * 2, Wg);
+  void* dU = scope.alloc((size_t)K * H * 2, Wu);
+  void* dD = scope.alloc(d_bytes);
+  if (scope.failed()) return kDeviceFailed;
+  int rc = gated_dev<T>(dA, dG, dU, act, dD, M, H, K, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  return scope.download(D, dD, d_bytes) ? kOk : kDeviceFailed;
+}
+
 thread_local int g_last_timer_source = -1;
 
 }  // namespace
@@ -89,6 +162,39 @@ int tessera_gfx950_batched_gemm_f16_dev(const void* A, const void* B, void* D, i
 int tessera_gfx950_batched_gemm_bf16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K,
                                          void* stream) {
   return gemm16_dev<BF16, EPI_F32>(A, B, D, batch, M, N, K, as_stream(stream));
+}
+
+int tessera_gfx950_gemm_bias_act_f16(const void* A, const void* B, const float* bias, int activation, void* D,
+                                     int M, int N, int K) {
+  return fused_host<F16>(A, B, bias, activation, D, M, N, K);
+}
+int tessera_gfx950_gemm_bias_act_bf16(const void* A, const void* B, const float* bias, int activation, void* D,
+                                      int M, int N, int K) {
+  return fused_host<BF16>(A, B, bias, activation, D, M, N, K);
+}
+int tessera_gfx950_gemm_bias_act_f16_dev(const void* A, const void* B, const float* bias, int activation, void* D,
+                                         int M, int N, int K, void* stream) {
+  return fused_dev<F16>(A, B, bias, activation, D, M, N, K, as_stream(stream));
+}
+int tessera_gfx950_gemm_bias_act_bf16_dev(const void* A, const void* B, const float* bias, int activation, void* D,
+                                          int M, int N, int K, void* stream) {
+  return fused_dev<BF16>(A, B, bias, activation, D, M, N, K, as_stream(stream));
+}
+int tessera_gfx950_gated_gemm_f16(const void* A, const void* Wg, const void* Wu, int activation, void* D, int M,
+                                  int H, int K) {
+  return gated_host<F16>(A, Wg, Wu, activation, D, M, H, K);
+}
+int tessera_gfx950_gated_gemm_bf16(const void* A, const void* Wg, const void* Wu, int activation, void* D, int M,
+                                   int H, int K) {
+  return gated_host<BF16>(A, Wg, Wu, activation, D, M, H, K);
+}
+int tessera_gfx950_gated_gemm_f16_dev(const void* A, const void* Wg, const void* Wu, int activation, void* D,
+                                      int M, int H, int K, void* stream) {
+  return gated_dev<F16>(A, Wg, Wu, activation, D, M, H, K, as_stream(stream));
+}
+int tessera_gfx950_gated_gemm_bf16_dev(const void* A, const void* Wg, const void* Wu, int activation, void* D,
+                                       int M, int H, int K, void* stream) {
+  return gated_dev<BF16>(A, Wg, Wu, activation, D, M, H, K, as_stream(stream));
 }
 
 // Kernel-only timing on resident buffers.  The device-event figure is accepted

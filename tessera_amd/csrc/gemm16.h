@@ -35,7 +35,27 @@ enum GemmEpilogue : int {
   EPI_F32 = 0,        // D f32
   EPI_STORE16 = 1,    // D in the storage dtype (RNE)
   EPI_SWIGLU16 = 2,   // D = storage(silu(storage(gate)) * storage(up)); B2 holds "up"
+  EPI_GATED_F32 = 3,  // D f32 = act(gate) * up, no intermediate rounding; B2 holds "up"
 };
+
+// Pointwise activations of the fused epilogue (the reference's matmul-epilogue
+// vocabulary, python/tessera/compiler/fusion_core.py:121-138).
+enum Activation : int { ACT_NONE = 0, ACT_RELU = 1, ACT_GELU = 2, ACT_SILU = 3, ACT_SIGMOID = 4, ACT_TANH = 5 };
+
+// All of them but relu are a logistic function of a linear or cubic argument:
+//   silu v sig(v); sigmoid sig(v); tanh 2 sig(2v) - 1;
+//   gelu (tanh form, argument clamped to +-30) 0.5 v (1 + tanh t) = v sig(2t).
+__device__ __forceinline__ float activate(float v, int act) {
+  if (act == ACT_NONE) return v;
+  if (act == ACT_RELU) return fmaxf(v, 0.f);
+  float x = v;
+  if (act == ACT_GELU) x = 2.f * fminf(fmaxf(0.7978845608028654f * (v + 0.044715f * v * v * v), -30.f), 30.f);
+  if (act == ACT_TANH) x = 2.f * v;
+  const float sg = 1.0f / (1.0f + __expf(-x));
+  if (act == ACT_SIGMOID) return sg;
+  if (act == ACT_TANH) return 2.f * sg - 1.f;
+  return v * sg;
+}
 
 struct Gemm16Params {
   const uint16_t* A;
@@ -45,6 +65,8 @@ struct Gemm16Params {
   int M, N, K;
   long lda, ldb, ldd;     // in elements
   long strideA, strideB, strideD;   // batch / expert strides in elements
+  const float* bias;      // fused epilogue: f32[N] added to every row, or null
+  int act;                // fused epilogue / gate activation (enum Activation)
   const int* offsets;     // grouped: device int32[E+1] row offsets into A and D; else null
   int groups;             // E (grouped) or batch count
   int tiles_m, tiles_n;   // tile grid (grouped: tiles_m is an upper bound)
@@ -107,7 +129,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN;     // wave tile
   constexpr int MI = TM / 32, NJ = TN / 32;     // 32x32 MFMA tiles per wave
-  constexpr bool SWIGLU = (EPI == EPI_SWIGLU16);
+  constexpr bool SWIGLU = (EPI == EPI_SWIGLU16 || EPI == EPI_GATED_F32);   // two-source B tile
   // SwiGLU: the BN columns of the LDS B tile are [gate n0..n0+BN/2) | up n0..n0+BN/2);
   // a wave's first NJ/2 column tiles are gate and the rest the matching up columns.
   static_assert(!SWIGLU || (WN == 1 && NJ % 2 == 0), "SwiGLU form needs WN == 1");
@@ -129,7 +151,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   const uint16_t* Bb = p.B;
   const uint16_t* B2b = p.B2;
   char* Db = (char*)p.D;
-  constexpr int DSZ = (EPI == EPI_F32) ? 4 : 2;
+  constexpr int DSZ = (EPI == EPI_F32 || EPI == EPI_GATED_F32) ? 4 : 2;
   if constexpr (GROUPED) {
     // 1-D grid over the real tiles of all groups, ordered group-major, then n tile,
     // then m tile.  Workgroup ids are dealt to the 8 XCDs round-robin, so XCD j takes
@@ -389,6 +411,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   // ---- epilogue -------------------------------------------------------------
   // acc[i][j][r]: row m = 32i + l32, col n = 32j + 8*(r/4) + 4*lh + (r%4).
   constexpr int NJ_OUT = SWIGLU ? NJ / 2 : NJ;
+  const bool fused = p.bias != nullptr || p.act != ACT_NONE;
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
     const int m = m_begin + wm * TM + i * 32 + l32;
@@ -402,10 +425,25 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
         if (n >= p.N) continue;                  // N % 8 == 0 on this path: all-or-nothing per run of 4
         float v0 = acc[i][j][q * 4 + 0], v1 = acc[i][j][q * 4 + 1];
         float v2 = acc[i][j][q * 4 + 2], v3 = acc[i][j][q * 4 + 3];
-        if constexpr (EPI == EPI_F32) {
+        if constexpr (EPI == EPI_F32 || EPI == EPI_STORE16) {
+          if (fused) {
+            if (p.bias) {
+              const float4 bv = *reinterpret_cast<const float4*>(p.bias + n);
+              v0 += bv.x; v1 += bv.y; v2 += bv.z; v3 += bv.w;
+            }
+            v0 = activate(v0, p.act); v1 = activate(v1, p.act);
+            v2 = activate(v2, p.act); v3 = activate(v3, p.act);
+          }
+        }
+        if constexpr (EPI == EPI_GATED_F32) {
+          const f32x16& u = acc[i][j + NJ / 2];
+          v0 = activate(v0, p.act) * u[q * 4 + 0]; v1 = activate(v1, p.act) * u[q * 4 + 1];
+          v2 = activate(v2, p.act) * u[q * 4 + 2]; v3 = activate(v3, p.act) * u[q * 4 + 3];
+        }
+        if constexpr (EPI == EPI_F32 || EPI == EPI_GATED_F32) {
           *reinterpret_cast<float4*>(drow + (long)n * 4) = make_float4(v0, v1, v2, v3);
         } else {
-          if constexpr (SWIGLU) {
+          if constexpr (EPI == EPI_SWIGLU16) {
             const f32x16& u = acc[i][j + NJ / 2];
             float g[4] = {v0, v1, v2, v3};
             float o[4];

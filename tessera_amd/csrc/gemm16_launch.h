@@ -20,8 +20,17 @@ __global__ void gemm16_generic_kernel(const Gemm16Params p) {
   const uint16_t* B = p.B + (long)z * p.strideB + n;
   float acc = 0.f;
   for (int k = 0; k < p.K; ++k) acc += from_storage<T>(A[k]) * from_storage<T>(B[(long)k * p.ldb]);
+  if constexpr (EPI == EPI_GATED_F32) {
+    const uint16_t* B2 = p.B2 + (long)z * p.strideB + n;
+    float up = 0.f;
+    for (int k = 0; k < p.K; ++k) up += from_storage<T>(A[k]) * from_storage<T>(B2[(long)k * p.ldb]);
+    acc = activate(acc, p.act) * up;
+  } else {
+    if (p.bias) acc += p.bias[n];
+    acc = activate(acc, p.act);
+  }
   const long o = (long)z * p.strideD + (long)m * p.ldd + n;
-  if constexpr (EPI == EPI_F32) reinterpret_cast<float*>(p.D)[o] = acc;
+  if constexpr (EPI == EPI_F32 || EPI == EPI_GATED_F32) reinterpret_cast<float*>(p.D)[o] = acc;
   else reinterpret_cast<uint16_t*>(p.D)[o] = to_storage<T>(acc);
 }
 
@@ -64,7 +73,7 @@ int launch_gemm16_tile(Gemm16Params p, hipStream_t s) {
                                    hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
   });
   if (attr_err != hipSuccess) return kDeviceFailed;
-  constexpr int BN_OUT = (EPI == EPI_SWIGLU16) ? BN / 2 : BN;
+  constexpr int BN_OUT = (EPI == EPI_SWIGLU16 || EPI == EPI_GATED_F32) ? BN / 2 : BN;
   p.tiles_n = ceil_div(p.N, BN_OUT);
   dim3 grid;
   if constexpr (GROUPED) {
@@ -84,7 +93,7 @@ int launch_gemm16_tile(Gemm16Params p, hipStream_t s) {
 // the storage dtype; four columns per thread (N % 8 == 0 on this path).
 template <class T, int EPI>
 __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restrict__ D, int M, int N, long ldd,
-                                     int splits) {
+                                     int splits, const float* __restrict__ bias, int act) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const int nq = N / 4;
   if (i >= (long)M * nq) return;
@@ -95,6 +104,12 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restr
     const float4 v = *reinterpret_cast<const float4*>(ws + z * mn + (size_t)m * N + n);
     acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
   }
+  if (bias) {
+    const float4 bv = *reinterpret_cast<const float4*>(bias + n);
+    acc.x += bv.x; acc.y += bv.y; acc.z += bv.z; acc.w += bv.w;
+  }
+  acc.x = activate(acc.x, act); acc.y = activate(acc.y, act);
+  acc.z = activate(acc.z, act); acc.w = activate(acc.w, act);
   if constexpr (EPI == EPI_F32) {
     *reinterpret_cast<float4*>(reinterpret_cast<float*>(D) + (long)m * ldd + n) = acc;
   } else {
@@ -113,7 +128,8 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
   const bool vec = (p.K % 8 == 0) && (p.N % 8 == 0) && (p.lda % 8 == 0) && (p.ldb % 8 == 0) &&
                    (p.lda < (1L << 21)) && (p.ldb < (1L << 21)) &&
                    ((p.ldd * dsz) % (dsz * 4) == 0) && (p.strideA % 8 == 0) && (p.strideB % 8 == 0) &&
-                   ((p.strideD * dsz) % 16 == 0) && aligned16(p.A) && aligned16(p.B) && aligned16(p.D);
+                   ((p.strideD * dsz) % 16 == 0) && aligned16(p.A) && aligned16(p.B) && aligned16(p.D) &&
+                   (!p.bias || aligned16(p.bias));
   if (!vec) {
     dim3 block(32, 8), grid(ceil_div(p.N, 32), ceil_div(p.M, 8), p.groups);
     hipLaunchKernelGGL((gemm16_generic_kernel<T, EPI>), grid, block, 0, s, p);
@@ -144,6 +160,8 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
       q.strideA = q.K;                       // split z reads A[:, z Ks ..) and B[z Ks .., :)
       q.strideB = (long)q.K * p.ldb;
       q.D = ws;
+      q.bias = nullptr;                      // the epilogue runs once, on the summed partials
+      q.act = ACT_NONE;
       q.ldd = p.N;
       q.strideD = (long)mn;
       int rc = t128 ? launch_gemm16_tile<T, 128, 128, 2, 2, EPI_F32, false>(q, s)
@@ -151,7 +169,7 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
       if (rc == kOk) {
         const long quads = (long)p.M * (p.N / 4);
         hipLaunchKernelGGL((splitk_reduce_kernel<T, EPI>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s,
-                           ws, p.D, p.M, p.N, p.ldd, splits);
+                           ws, p.D, p.M, p.N, p.ldd, splits, p.bias, p.act);
         rc = launch_status();
       }
       if (hipFreeAsync(ws, s) != hipSuccess) { (void)hipGetLastError(); rc = rc == kOk ? kDeviceFailed : rc; }
@@ -160,6 +178,20 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
   }
   if (t128) return launch_gemm16_tile<T, 128, 128, 2, 2, EPI, false>(p, s);
   return launch_gemm16_tile<T, 64, 64, 2, 2, EPI, false>(p, s);
+}
+
+// Dense gated product D f32 = act(A Wg) * (A Wu); p.B = Wg, p.B2 = Wu, p.N = H.
+template <class T>
+int launch_gemm16_gated(Gemm16Params p, hipStream_t s) {
+  const bool vec = (p.K % 8 == 0) && (p.N % 8 == 0) && (p.lda % 8 == 0) && (p.ldb % 8 == 0) &&
+                   (p.lda < (1L << 21)) && (p.ldb < (1L << 21)) && (p.ldd % 4 == 0) && aligned16(p.A) &&
+                   aligned16(p.B) && aligned16(p.B2) && aligned16(p.D);
+  if (!vec || (long)p.M * p.N < 128L * 128L) {
+    dim3 block(32, 8), grid(ceil_div(p.N, 32), ceil_div(p.M, 8), 1);
+    hipLaunchKernelGGL((gemm16_generic_kernel<T, EPI_GATED_F32>), grid, block, 0, s, p);
+    return launch_status();
+  }
+  return launch_gemm16_tile<T, 256, 256, 4, 1, EPI_GATED_F32, false>(p, s);
 }
 
 // Grouped.  p.M = total rows S, p.groups = E, p.offsets = device int32[E+1].

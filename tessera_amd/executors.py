@@ -71,8 +71,9 @@ class ExecutionRow:
 
 #: docstring registry, as ``KNOWN_EXECUTORS`` (``execution_matrix.py:103``).
 KNOWN_EXECUTORS: dict[str, str] = {
-    "gfx950_gemm": "single tessera.matmul/gemm op, rank-2, f16/bf16 -> f32 or int8 -> int32, "
-                   "hand-written CDNA4 MFMA GEMM (tessera_gfx950_gemm_* C ABI)",
+    "gfx950_gemm": "single tessera.matmul/gemm/fused_epilogue op, rank-2, f16/bf16 -> f32 (optional bias[N] "
+                   "+ relu/gelu/silu fused) or int8 -> int32, hand-written CDNA4 MFMA GEMM "
+                   "(tessera_gfx950_gemm_* C ABI)",
     "gfx950_flash_attn": "flash_attn / multi_head / gqa / mqa attention forward, f16/bf16 -> f32, "
                          "causal + GQA, MFMA FA-2 (tessera_gfx950_flash_attn_gqa_* C ABI)",
     "gfx950_moe_transport": "tessera.moe_dispatch / moe_combine / grouped_gemm / grouped_swiglu on "
@@ -148,23 +149,37 @@ def _single_op(artifact: RuntimeArtifact, allowed: tuple, who: str) -> dict:
 # ---- executors -------------------------------------------------------------------------
 
 def execute_gfx950_gemm(artifact: RuntimeArtifact, args: Any):
-    """One ``tessera.matmul`` / ``tessera.gemm`` op: rank-2 operands with matching
-    K; f16/bf16 storage -> f32 result, int8 -> int32 result."""
+    """One ``tessera.matmul`` / ``tessera.gemm`` / ``tessera.fused_epilogue`` op:
+    rank-2 operands with matching K; f16/bf16 storage -> f32 result, int8 -> int32
+    result.  An optional third operand is the per-output-column bias ``[N]`` and
+    ``kwargs["activation"]`` (none / relu / gelu / silu) selects the fused
+    activation — float only (``runtime.py:6603-6660``)."""
     md = artifact.metadata or {}
-    op = _single_op(artifact, ("tessera.matmul", "tessera.gemm"), "gfx950_gemm")
+    op = _single_op(artifact, ("tessera.matmul", "tessera.gemm", "tessera.fused_epilogue"), "gfx950_gemm")
     values = _bind_launch_args(args, list(md.get("arg_names") or []))
     names = [str(n) for n in op.get("operands", [])]
-    if len(names) != 2:
-        raise ValueError("matmul requires exactly two operands")
+    kwargs = op.get("kwargs") or {}
+    activation = str(kwargs.get("activation") or "none")
+    if activation not in ("none", "relu", "gelu", "silu"):
+        raise ValueError(f"gfx950 epilogue activation must be one of none/relu/gelu/silu; got {activation!r}")
+    if len(names) not in (2, 3):
+        raise ValueError(f"matmul takes two operands (a, b) plus an optional third bias operand; got {len(names)}")
+    has_bias = len(names) == 3
     a, b = _as_array(values[names[0]]), _as_array(values[names[1]])
     if a.ndim != 2 or b.ndim != 2 or a.shape[1] != b.shape[0]:
         raise ValueError(f"gfx950 matmul needs rank-2 operands with matching K; got {a.shape} @ {b.shape}")
-    kwargs = op.get("kwargs") or {}
-    if kwargs.get("epilogue") or kwargs.get("bias") is not None:
-        raise ValueError("gfx950 matmul executor runs the bare product; fused bias/activation is not on this lane")
     if a.dtype == np.int8 and b.dtype == np.int8:
+        if has_bias or activation != "none":
+            raise ValueError("gfx950 fused epilogue (bias/activation) is float-only; got integer dtype int8")
         return _ops.gemm_i8(a, b)
-    return _ops.gemm(a, b, out="f32")
+    if not has_bias and activation == "none":
+        return _ops.gemm(a, b, out="f32")
+    bias = None
+    if has_bias:
+        bias = np.ascontiguousarray(np.asarray(_as_array(values[names[2]])), dtype=np.float32)
+        if bias.shape != (b.shape[1],):
+            raise ValueError(f"bias must have shape ({b.shape[1]},) (one per output column); got {bias.shape}")
+    return _ops.fused_gemm(a, b, bias, activation)
 
 
 _FA_OPS = ("tessera.flash_attn", "tessera.multi_head_attention", "tessera.gqa_attention", "tessera.mqa_attention")

@@ -91,6 +91,14 @@ _SIGNATURES = {
     "tessera_gfx950_gemm_bf16_bf16_dev": _GEMM + [_c_vp],
     "tessera_gfx950_batched_gemm_f16_dev": [_c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_batched_gemm_bf16_dev": [_c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_vp],
+    "tessera_gfx950_gemm_bias_act_f16": [_c_vp, _c_vp, _c_vp, _c_int, _c_vp, _c_int, _c_int, _c_int],
+    "tessera_gfx950_gemm_bias_act_bf16": [_c_vp, _c_vp, _c_vp, _c_int, _c_vp, _c_int, _c_int, _c_int],
+    "tessera_gfx950_gemm_bias_act_f16_dev": [_c_vp, _c_vp, _c_vp, _c_int, _c_vp, _c_int, _c_int, _c_int, _c_vp],
+    "tessera_gfx950_gemm_bias_act_bf16_dev": [_c_vp, _c_vp, _c_vp, _c_int, _c_vp, _c_int, _c_int, _c_int, _c_vp],
+    "tessera_gfx950_gated_gemm_f16": [_c_vp, _c_vp, _c_vp, _c_int, _c_vp, _c_int, _c_int, _c_int],
+    "tessera_gfx950_gated_gemm_bf16": [_c_vp, _c_vp, _c_vp, _c_int, _c_vp, _c_int, _c_int, _c_int],
+    "tessera_gfx950_gated_gemm_f16_dev": [_c_vp, _c_vp, _c_vp, _c_int, _c_vp, _c_int, _c_int, _c_int, _c_vp],
+    "tessera_gfx950_gated_gemm_bf16_dev": [_c_vp, _c_vp, _c_vp, _c_int, _c_vp, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_gemm_i8_i32_dev": _GEMM + [_c_vp],
     "tessera_gfx950_gemm_w8a8_f32_dev": [_c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_gemm_e4m3_bf16_dev": [_c_vp, _c_vp, _c_f, _c_f, _c_vp, _c_int, _c_int, _c_int, _c_vp],

@@ -131,6 +131,61 @@ def gemm(A, B, *, out: str = "storage"):
 matmul = gemm
 batched_gemm = gemm
 
+#: activation codes of the fused-epilogue entry points
+ACTIVATIONS = {"none": 0, "relu": 1, "gelu": 2, "silu": 3, "sigmoid": 4, "tanh": 5}
+
+
+def _activation_code(name) -> int:
+    key = str(name or "none")
+    if key not in ACTIVATIONS:
+        raise ValueError(f"activation must be one of {sorted(ACTIVATIONS)}; got {name!r}")
+    return ACTIVATIONS[key]
+
+
+def fused_gemm(A, B, bias=None, activation: str = "none") -> np.ndarray:
+    """``act(A @ B + bias)`` in one kernel → f32.  Rank-2 16-bit operands, ``bias``
+    f32 ``[N]`` or None, ``activation`` from the reference's epilogue vocabulary
+    (none / relu / gelu / silu / sigmoid / tanh)."""
+    A, B = _unbox(A), _unbox(B)
+    st = _storage(A, B)
+    a, b = _bits(A), _bits(B)
+    if a.ndim != 2 or b.ndim != 2 or a.shape[1] != b.shape[0]:
+        raise ValueError(f"fused_gemm needs rank-2 operands with matching K; got {a.shape} @ {b.shape}")
+    M, K = a.shape
+    N = b.shape[1]
+    act = _activation_code(activation)
+    bias_arr = None
+    if bias is not None:
+        bias_arr = np.ascontiguousarray(bias, np.float32)
+        if bias_arr.shape != (N,):
+            raise ValueError(f"bias must have shape ({N},) (one per output column); got {bias_arr.shape}")
+    d = np.empty((M, N), np.float32)
+    fn = getattr(_lane.load(), f"tessera_gfx950_gemm_bias_act_{st}")
+    _lane.check(fn(a.ctypes.data, b.ctypes.data, bias_arr.ctypes.data if bias_arr is not None else None, act,
+                   d.ctypes.data, M, N, K), "fused_gemm")
+    return d
+
+
+def gated_gemm(A, Wg, Wu, gate_act: str = "silu") -> np.ndarray:
+    """``act(A @ Wg) * (A @ Wu)`` in one kernel → f32 ``[M, H]`` (the gated MLP
+    projection; ``silu`` gives the SwiGLU gate)."""
+    A, Wg, Wu = _unbox(A), _unbox(Wg), _unbox(Wu)
+    st = _storage(A, Wg)
+    if _storage(A, Wu) != st:
+        raise ValueError("operands must share one 16-bit storage dtype")
+    a, g, u = _bits(A), _bits(Wg), _bits(Wu)
+    if a.ndim != 2 or g.ndim != 2 or g.shape != u.shape or a.shape[1] != g.shape[0]:
+        raise ValueError(f"gated_gemm needs A (M,K) and Wg, Wu (K,H); got {a.shape}, {g.shape}, {u.shape}")
+    act = _activation_code(gate_act)
+    if act == 0:
+        raise ValueError("gate activation must be a unary pointwise op")
+    M, K = a.shape
+    H = g.shape[1]
+    d = np.empty((M, H), np.float32)
+    fn = getattr(_lane.load(), f"tessera_gfx950_gated_gemm_{st}")
+    _lane.check(fn(a.ctypes.data, g.ctypes.data, u.ctypes.data, act, d.ctypes.data, M, H, K), "gated_gemm")
+    return d
+
 
 def gemm_i8(A, B) -> np.ndarray:
     """``int32(A) @ int32(B)`` for int8 operands — exact."""

@@ -78,6 +78,11 @@ KERNEL_TABLE: tuple = (
                 "v_mfma_i32_32x32x32_i8", ("int8",),
                 ("tessera_gfx950_gemm_i8_i32", "tessera_gfx950_gemm_w8a8_f32"),
                 "gfx950_gemm", "256x256x128, 2x2 waves of 128x128", 135168),
+    KernelEntry("tessera.fused_epilogue", ("tile.matmul", "tile.mma"), "tessera_rocm.mfma_gemm", "m32n32k16",
+                "v_mfma_f32_32x32x16_{f16,bf16}", ("f16", "bf16"),
+                ("tessera_gfx950_gemm_bias_act_f16", "tessera_gfx950_gemm_bias_act_bf16",
+                 "tessera_gfx950_gated_gemm_f16", "tessera_gfx950_gated_gemm_bf16"),
+                "gfx950_gemm", "256x256x64, bias + activation (or gate * up) in the epilogue", 135168),
     KernelEntry("tessera.fp8_gemm", ("tile.matmul", "tile.mma"), "tessera_rocm.mfma_gemm", "m32n32k64",
                 "v_mfma_f32_32x32x64_f8f6f4", ("fp8_e4m3",),
                 ("tessera_gfx950_gemm_e4m3_bf16", "tessera_gfx950_gemm_e4m3_f32"),
