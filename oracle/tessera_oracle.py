@@ -60,12 +60,18 @@ def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
     ``(u + 0x7FFF + ((u >> 16) & 1)) >> 16``.  NaNs are kept quiet.
     """
     a = np.ascontiguousarray(x, np.float32)
-    u = a.view(np.uint32).astype(np.uint64)
-    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
-    nan = np.isnan(a)
-    if nan.any():
-        r = np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), r)
-    return r
+    flat = a.reshape(-1)
+    out = np.empty(flat.shape, np.uint16)
+    step = 1 << 22                       # chunks keep the 64-bit temporaries small
+    for i in range(0, flat.size, step):
+        c = flat[i:i + step]
+        u = c.view(np.uint32).astype(np.uint64)
+        r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+        nan = np.isnan(c)
+        if nan.any():
+            r = np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), r)
+        out[i:i + step] = r
+    return out.reshape(a.shape)
 
 
 def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:

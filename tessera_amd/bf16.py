@@ -22,11 +22,20 @@ def from_float32(x) -> BF16Array:
     """f32 -> bf16 bits, round-to-nearest-even (the rounding the reference's
     ``_round_to_storage`` fallback applies, ``compiler/fusion_core.py:358-361``)."""
     a = np.ascontiguousarray(x, np.float32)
-    u = a.view(np.uint32).astype(np.uint64)
-    bits = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
-    nan = np.isnan(a)
-    if nan.any():
-        bits = np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), bits)
+    flat = a.reshape(-1)
+    bits = np.empty(flat.shape, np.uint16)
+    step = 1 << 22                                   # chunked: 32-bit temporaries stay cache-sized
+    for i in range(0, flat.size, step):
+        u = flat[i:i + step].view(np.uint32)
+        r = (u >> 16) & np.uint32(1)
+        r += np.uint32(0x7FFF)
+        r += u                                       # wraps only for NaN patterns, fixed below
+        r >>= 16
+        nan = np.isnan(flat[i:i + step])
+        if nan.any():
+            r = np.where(nan, (u >> 16) | np.uint32(0x40), r)
+        bits[i:i + step] = r
+    bits = bits.reshape(a.shape)
     return bits.view(BF16Array)
 
 

@@ -192,3 +192,47 @@ def test_moe_layer_with_router_gemm(lane):
     out, plan = ops.moe_layer(xb, rb, *(b16.from_float32(a) for a in (wg, wu, wd)), top_k=k, return_plan=True)
     _check_plan(plan, desc)
     assert orc.max_rel_err(out, ref) <= TOL + 2.0 ** -8
+
+
+def test_moe_headline_config(lane):
+    """The full MoE configuration (8192 tokens, hidden 4096, 64 experts, top-8,
+    F = 1408): routing / permutation indices bit-exact, and the layer output of a
+    sample of tokens against the oracle's expert FFN on exactly those rows.  The
+    expert weights are one seeded N(0, 0.02) block per matrix, re-used for every
+    expert with a different row rotation and sign pattern (drawing 1.1e9 normals
+    would dominate the test)."""
+    T, H, F, E, k = 8192, 4096, 1408, 64, 8
+    rng = np.random.default_rng(2024)
+    x = b16.from_float32(rng.standard_normal((T, H), dtype=np.float32))
+    lg = _logits(T, E, 500, k)
+
+    def expert_weights(rows, cols, seed):
+        r = np.random.default_rng(seed)
+        base = np.asarray(b16.from_float32(0.02 * r.standard_normal((rows, cols), dtype=np.float32)), np.uint16)
+        flip = (r.integers(0, 2, (rows, cols), dtype=np.uint16) << 15).astype(np.uint16)
+        w = np.empty((E, rows, cols), np.uint16)
+        for e in range(E):
+            w[e] = np.roll(base, 17 * e + 3, axis=0) ^ np.roll(flip, 5 * e + 1, axis=1)
+        return b16.from_bits(w)
+
+    wg, wu, wd = expert_weights(H, F, 1), expert_weights(H, F, 2), expert_weights(F, H, 3)
+    out, plan = ops.moe_layer(x, None, wg, wu, wd, top_k=k, router_logits=lg, return_plan=True)
+    r = orc.route_tokens(lg, E, k)
+    desc = orc.plan_dispatch(r.assignment, r.weights, E)
+    _check_plan(plan, desc)
+    assert out.shape == (T, H) and not np.isnan(np.asarray(out, np.float32)).any()
+
+    tokens = np.sort(rng.choice(T, 20, replace=False))
+    slots = np.flatnonzero(np.isin(desc.token_of_slot, tokens))           # slot order: expert-major
+    tok_of = desc.token_of_slot[slots].astype(np.int64)
+    exp_of = desc.expert_of_slot[slots].astype(np.int64)
+    xs = x.to_float32()[tok_of]
+    y = np.zeros((slots.size, H), np.float32)
+    for e in np.unique(exp_of):
+        rows = np.flatnonzero(exp_of == e)
+        y[rows] = orc.moe_swiglu_block(xs[rows], wg[e:e + 1].to_float32(), wu[e:e + 1].to_float32(),
+                                       wd[e:e + 1].to_float32(), [rows.size])
+    ref = np.zeros((T, H), np.float64)
+    np.add.at(ref, tok_of, y.astype(np.float64) * desc.combine_weights[slots][:, None].astype(np.float64))
+    got = np.asarray(out, np.float32)[tokens]
+    assert orc.max_rel_err(got, ref[tokens]) <= TOL + 2.0 ** -8
