@@ -36,7 +36,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes one launch of the headline kernel moves: FETCH_SIZE + WRITE_SIZE per
 # dispatch from two counter runs of this script, each scaled by the same counter's
 # reading for the 1 GiB copy kernel (profiles/bench_all_kernels_hbm_bytes.txt).
-TRAFFIC_BYTES_GEMM_BF16_8192 = 1.7738e9
+TRAFFIC_BYTES_GEMM_BF16_8192 = 1.7497e9
 
 
 def _timed(lane, launch, steps, warmup):
