@@ -117,6 +117,34 @@ def bench_attention(lane, steps, warmup):
             "tflops": flop / ev / 1e9, "frac_mfma_peak": flop / ev / 1e9 / PEAK_BF16_TFLOPS}
 
 
+def bench_attention_bwd(lane, steps, warmup):
+    """Backward of the same attention configuration with the forward's O and LSE
+    saved (dQ, dK, dV kernels + the Delta pass), and with the forward recomputed."""
+    B, Hq, Hkv, S, D = 4, 32, 8, 4096, 128
+    rng = np.random.default_rng(5)
+    q, do = (_bf16(rng.standard_normal((B, Hq, S, D), dtype=np.float32)) for _ in range(2))
+    k, v = (_bf16(rng.standard_normal((B, Hkv, S, D), dtype=np.float32)) for _ in range(2))
+    dq, dk, dv, ddo = (lane.DeviceBuffer.from_host(x) for x in (q, k, v, do))
+    o32, lse = lane.DeviceBuffer(q.size * 4), lane.DeviceBuffer(B * Hq * S * 4)
+    gq, gk, gv = lane.DeviceBuffer(q.size * 4), lane.DeviceBuffer(k.size * 4), lane.DeviceBuffer(k.size * 4)
+    lib = lane.load()
+    scale = 1.0 / np.sqrt(D)
+    lane.check(lib.tessera_gfx950_flash_attn_gqa_bf16_dev(dq.ptr, dk.ptr, dv.ptr, o32.ptr, lse.ptr, B, Hq, Hkv, S, S,
+                                                          D, scale, 1, 0, None), "flash_attn")
+    fn = lib.tessera_gfx950_flash_attn_bwd_bf16_dev
+    saved = lambda: lane.check(fn(ddo.ptr, dq.ptr, dk.ptr, dv.ptr, o32.ptr, lse.ptr, gq.ptr, gk.ptr, gv.ptr,
+                                  B, Hq, Hkv, S, S, D, scale, 1, None), "flash_attn_bwd")
+    recomp = lambda: lane.check(fn(ddo.ptr, dq.ptr, dk.ptr, dv.ptr, None, None, gq.ptr, gk.ptr, gv.ptr,
+                                   B, Hq, Hkv, S, S, D, scale, 1, None), "flash_attn_bwd")
+    _, ev = _timed(lane, saved, steps, warmup)
+    _, ev_re = _timed(lane, recomp, steps, warmup)
+    for buf in (dq, dk, dv, ddo, o32, lse, gq, gk, gv):
+        buf.close()
+    flop = 2.5 * 4.0 * B * Hq * (S * (S + 1) / 2) * D        # five S x S x D products against the forward's two
+    return {"workload": "flash_attn_bwd_bf16_causal_B4_Hq32_Hkv8_S4096_D128", "ms": ev, "ms_with_forward_recompute": ev_re,
+            "tflops": flop / ev / 1e9, "frac_mfma_peak": flop / ev / 1e9 / PEAK_BF16_TFLOPS}
+
+
 def bench_quant(lane, steps, warmup):
     M, N, K = 4096, 8192, 8192
     rng = np.random.default_rng(2)
@@ -270,6 +298,7 @@ def main() -> int:
         also = {}
         s, w = max(3, args.steps // 2), max(2, args.warmup // 2)
         also["flash_attn"] = bench_attention(lane, s, w)
+        also["flash_attn_bwd"] = bench_attention_bwd(lane, s, w)
         also.update(bench_quant(lane, s, w))
         also.update(bench_decode(lane, s, w))
         also["moe"] = bench_moe(lane, s, w)

@@ -201,6 +201,32 @@ int tessera_gfx950_flash_attn_gqa_bf16_dev(const void* Q, const void* K, const v
                                            int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
                                            int causal, int out_dtype, void* stream);
 
+/* ---- flash-attention backward -------------------------------------------- */
+
+/* (dQ, dK, dV) of O = softmax(scale Q K^T, causal) V given dO: the contract of the
+ * reference's backward lane (python/tessera/runtime.py:7598-7665: operands
+ * (dO, Q, K, V), Q/dO [B,Hq,Sq,D], K/V [B,Hkv,Sk,D], Hq % Hkv == 0, head_dim a
+ * multiple of 16, f16/bf16 storage, f32 accumulate) and the arithmetic of
+ * vjp_flash_attn (python/tessera/autodiff/vjp.py:1311-1377).  dQ, dK, dV are f32,
+ * shaped like Q, K, V; dK / dV of a KV head sum over the query heads of its group.
+ * The host-pointer forms recompute the forward (nothing saved), as the reference
+ * does.  The _dev forms also accept the forward's saved O (f32) and LSE; pass both
+ * NULL to recompute. */
+int tessera_gfx950_flash_attn_bwd_f16(const void* dO, const void* Q, const void* K, const void* V,
+                                      void* dQ, void* dK, void* dV, int B, int Hq, int Hkv,
+                                      int Sq, int Sk, int D, float scale, int causal);
+int tessera_gfx950_flash_attn_bwd_bf16(const void* dO, const void* Q, const void* K, const void* V,
+                                       void* dQ, void* dK, void* dV, int B, int Hq, int Hkv,
+                                       int Sq, int Sk, int D, float scale, int causal);
+int tessera_gfx950_flash_attn_bwd_f16_dev(const void* dO, const void* Q, const void* K, const void* V,
+                                          const void* O, const void* LSE, void* dQ, void* dK, void* dV,
+                                          int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                                          int causal, void* stream);
+int tessera_gfx950_flash_attn_bwd_bf16_dev(const void* dO, const void* Q, const void* K, const void* V,
+                                           const void* O, const void* LSE, void* dQ, void* dK, void* dV,
+                                           int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                                           int causal, void* stream);
+
 /* ---- MoE -------------------------------------------------------------------- */
 
 /* Router + packing plan in the canonical int32 device ABI

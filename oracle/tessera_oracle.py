@@ -19,6 +19,8 @@ bf16 rounding              all 2^16 bf16 codes round-trip; RNE ties table;
 gemm / batched_gemm        f64 matmul of storage-rounded operands; identity /
                            ones / K-ramp closed forms; compiled reference twin
                            ``tessera_x86_reference_gemm_bf16``
+flash_attn_backward        torch autograd of scaled_dot_product_attention (library);
+                           central finite differences of the forward oracle
 flash_attn (+GQA, +LSE)    dense textbook softmax in f64; row 0 -> V[0];
                            identical keys -> prefix mean; torch SDPA library
                            cross-check; compiled reference
@@ -224,6 +226,44 @@ def flash_attn_dense(Q, K, V, scale=None, causal=False, dtype=np.float64):
                 LSE[b, h] = np.where(l[:, 0] > 0, msafe[:, 0] + np.log(l[:, 0]), -np.inf)
             O[b, h] = p @ V[b, kh]
     return O, LSE
+
+
+def flash_attn_backward(dO, Q, K, V, scale=None, causal=False):
+    """Adjoint of ``softmax(scale*Q K^T, causal) V`` — ``vjp_flash_attn``
+    (``autodiff/vjp.py:1311-1377``) restated with GQA: ``dK`` / ``dV`` of a kv head
+    are the sums over the query heads that share it
+    (``runtime.py:7640-7649``).  f64 inside; returns ``(dQ, dK, dV)`` shaped like
+    ``(Q, K, V)``.  Recomputes S and P; ``dS = (dP - rowsum(dP * P)) * P``."""
+    Q = np.asarray(Q, np.float64)
+    K = np.asarray(K, np.float64)
+    V = np.asarray(V, np.float64)
+    dO = np.asarray(dO, np.float64)
+    B, Hq, Sq, D = Q.shape
+    _, Hkv, Sk, _ = K.shape
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    dQ, dK, dV = np.zeros_like(Q), np.zeros_like(K), np.zeros_like(V)
+    off = _causal_limit(Sq, Sk)
+    for b in range(B):
+        for h in range(Hq):
+            kh = h * Hkv // Hq
+            s = (Q[b, h] @ K[b, kh].T) * scale
+            if causal:
+                i = np.arange(Sq)[:, None]
+                j = np.arange(Sk)[None, :]
+                mask = j > i + off
+                s = np.where(mask, -np.inf, s)
+            m = s.max(axis=-1, keepdims=True)
+            m = np.where(np.isfinite(m), m, 0.0)
+            e = np.exp(s - m)
+            l = e.sum(axis=-1, keepdims=True)
+            p = np.where(l > 0, e / np.where(l > 0, l, 1.0), 0.0)
+            dV[b, kh] += p.T @ dO[b, h]
+            dp = dO[b, h] @ V[b, kh].T
+            ds = (dp - (dp * p).sum(axis=-1, keepdims=True)) * p
+            dQ[b, h] = (ds @ K[b, kh]) * scale
+            dK[b, kh] += (ds.T @ Q[b, h]) * scale
+    return dQ, dK, dV
 
 
 def flash_attn_blockwise(Q, K, V, scale=None, causal=False, block=512,

@@ -2,6 +2,7 @@
 #include <mutex>
 #include "../../include/tessera_gfx950.h"
 #include "flash_attn.h"
+#include "flash_bwd.h"
 #include "host_util.h"
 
 namespace tsr950 {
@@ -76,6 +77,113 @@ int flash_host(const void* Q, const void* K, const void* V, void* O, void* LSE, 
   return kOk;
 }
 
+template <class T, int D>
+int launch_bwd(const FlashBwdParams& p, hipStream_t s) {
+  constexpr int kDqSmem = 4 * FB_BKV * D * 2;
+  constexpr int kDkvSmem = 2 * (2 * FB_BQT * D * 2 + 2 * FB_BQT * 4);
+  auto dq_kern = flash_bwd_dq_kernel<T, D>;
+  auto dkv_kern = flash_bwd_dkdv_kernel<T, D>;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(dq_kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, kDqSmem);
+    if (attr_err == hipSuccess)
+      attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(dkv_kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kDkvSmem);
+  });
+  if (attr_err != hipSuccess) return kDeviceFailed;
+  hipLaunchKernelGGL(dq_kern, dim3(ceil_div(p.Sq, FB_BQ) * p.B * p.Hq), dim3(FB_DQ_THREADS), kDqSmem, s, p);
+  if (int rc = launch_status(); rc != kOk) return rc;
+  hipLaunchKernelGGL(dkv_kern, dim3(ceil_div(p.Sk, FB_BK) * p.B * p.Hkv), dim3(FB_DKV_THREADS), kDkvSmem, s, p);
+  return launch_status();
+}
+
+// (dQ, dK, dV) from (dO, Q, K, V).  O and LSE may be passed in (saved by the forward
+// call); when either is null the forward kernel is run first to recompute both.
+template <class T>
+int flash_bwd_dev(const void* dO, const void* Q, const void* K, const void* V, const float* O, const float* LSE,
+                  float* dQ, float* dK, float* dV, int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                  int causal, hipStream_t s) {
+  if (bad_attn(B, Hq, Hkv, Sq, Sk, D) || !dO || !Q || !K || !V || !dQ || !dK || !dV) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t rows = (size_t)B * Hq * Sq;
+  const bool recompute = !O || !LSE;
+  float* ws = nullptr;                       // [O (rows * D) | LSE (rows)]? | Delta (rows)
+  const size_t ws_floats = rows + (recompute ? rows * D + rows : 0);
+  if (hipMallocAsync(reinterpret_cast<void**>(&ws), ws_floats * sizeof(float), s) != hipSuccess) {
+    (void)hipGetLastError();
+    return kDeviceFailed;
+  }
+  int rc = kOk;
+  float* delta = ws;
+  if (recompute) {
+    float* o_ws = ws + rows;
+    float* lse_ws = o_ws + rows * D;
+    rc = flash_dev<T>(Q, K, V, o_ws, lse_ws, B, Hq, Hkv, Sq, Sk, D, scale, causal, 0, s);
+    O = o_ws;
+    LSE = lse_ws;
+  }
+  if (rc == kOk) {
+    FlashBwdParams p{};
+    p.Q = static_cast<const uint16_t*>(Q);
+    p.K = static_cast<const uint16_t*>(K);
+    p.V = static_cast<const uint16_t*>(V);
+    p.dO = static_cast<const uint16_t*>(dO);
+    p.O = O; p.LSE = LSE; p.Delta = delta;
+    p.dQ = dQ; p.dK = dK; p.dV = dV;
+    p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Sq = Sq; p.Sk = Sk;
+    p.scale = scale;
+    p.causal = causal ? 1 : 0;
+    hipLaunchKernelGGL((flash_bwd_delta_kernel<T>), dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, s,
+                       p.dO, p.O, delta, (long)rows, D);
+    rc = launch_status();
+    const bool al = ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
+                      reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(dO) |
+                      reinterpret_cast<uintptr_t>(dQ) | reinterpret_cast<uintptr_t>(dK) |
+                      reinterpret_cast<uintptr_t>(dV)) & 15) == 0;
+    if (rc == kOk) {
+      if (al && D == 128) rc = launch_bwd<T, 128>(p, s);
+      else if (al && D == 64) rc = launch_bwd<T, 64>(p, s);
+      else {
+        const long kvrows = (long)B * Hkv * Sk;
+        hipLaunchKernelGGL((flash_bwd_generic_dq_kernel<T>), dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, p, D);
+        hipLaunchKernelGGL((flash_bwd_generic_dkdv_kernel<T>), dim3((unsigned)((kvrows + 63) / 64)), dim3(64), 0, s,
+                           p, D);
+        rc = launch_status();
+      }
+    }
+  }
+  if (hipFreeAsync(ws, s) != hipSuccess) { (void)hipGetLastError(); rc = rc == kOk ? kDeviceFailed : rc; }
+  return rc;
+}
+
+template <class T>
+int flash_bwd_host(const void* dO, const void* Q, const void* K, const void* V, void* dQ, void* dK, void* dV, int B,
+                   int Hq, int Hkv, int Sq, int Sk, int D, float scale, int causal) {
+  if (bad_attn(B, Hq, Hkv, Sq, Sk, D) || !dO || !Q || !K || !V || !dQ || !dK || !dV) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t q_elems = (size_t)B * Hq * Sq * D, kv_elems = (size_t)B * Hkv * Sk * D;
+  DeviceScope scope;
+  void* ddO = scope.alloc(q_elems * 2, dO);
+  void* dQin = scope.alloc(q_elems * 2, Q);
+  void* dKin = scope.alloc(kv_elems * 2, K);
+  void* dVin = scope.alloc(kv_elems * 2, V);
+  void* gQ = scope.alloc(q_elems * 4);
+  void* gK = scope.alloc(kv_elems * 4);
+  void* gV = scope.alloc(kv_elems * 4);
+  if (scope.failed()) return kDeviceFailed;
+  int rc = flash_bwd_dev<T>(ddO, dQin, dKin, dVin, nullptr, nullptr, static_cast<float*>(gQ),
+                            static_cast<float*>(gK), static_cast<float*>(gV), B, Hq, Hkv, Sq, Sk, D, scale, causal,
+                            nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  if (!scope.download(dQ, gQ, q_elems * 4) || !scope.download(dK, gK, kv_elems * 4) ||
+      !scope.download(dV, gV, kv_elems * 4))
+    return kDeviceFailed;
+  return kOk;
+}
+
 }  // namespace
 }  // namespace tsr950
 
@@ -108,6 +216,33 @@ int tessera_gfx950_flash_attn_gqa_bf16_dev(const void* Q, const void* K, const v
                                            int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
                                            int causal, int out_dtype, void* stream) {
   return flash_dev<BF16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, out_dtype, as_stream(stream));
+}
+
+int tessera_gfx950_flash_attn_bwd_f16(const void* dO, const void* Q, const void* K, const void* V, void* dQ,
+                                      void* dK, void* dV, int B, int Hq, int Hkv, int Sq, int Sk, int D,
+                                      float scale, int causal) {
+  return flash_bwd_host<F16>(dO, Q, K, V, dQ, dK, dV, B, Hq, Hkv, Sq, Sk, D, scale, causal);
+}
+int tessera_gfx950_flash_attn_bwd_bf16(const void* dO, const void* Q, const void* K, const void* V, void* dQ,
+                                       void* dK, void* dV, int B, int Hq, int Hkv, int Sq, int Sk, int D,
+                                       float scale, int causal) {
+  return flash_bwd_host<BF16>(dO, Q, K, V, dQ, dK, dV, B, Hq, Hkv, Sq, Sk, D, scale, causal);
+}
+int tessera_gfx950_flash_attn_bwd_f16_dev(const void* dO, const void* Q, const void* K, const void* V,
+                                          const void* O, const void* LSE, void* dQ, void* dK, void* dV, int B,
+                                          int Hq, int Hkv, int Sq, int Sk, int D, float scale, int causal,
+                                          void* stream) {
+  return flash_bwd_dev<F16>(dO, Q, K, V, static_cast<const float*>(O), static_cast<const float*>(LSE),
+                            static_cast<float*>(dQ), static_cast<float*>(dK), static_cast<float*>(dV), B, Hq, Hkv,
+                            Sq, Sk, D, scale, causal, as_stream(stream));
+}
+int tessera_gfx950_flash_attn_bwd_bf16_dev(const void* dO, const void* Q, const void* K, const void* V,
+                                           const void* O, const void* LSE, void* dQ, void* dK, void* dV, int B,
+                                           int Hq, int Hkv, int Sq, int Sk, int D, float scale, int causal,
+                                           void* stream) {
+  return flash_bwd_dev<BF16>(dO, Q, K, V, static_cast<const float*>(O), static_cast<const float*>(LSE),
+                             static_cast<float*>(dQ), static_cast<float*>(dK), static_cast<float*>(dV), B, Hq, Hkv,
+                             Sq, Sk, D, scale, causal, as_stream(stream));
 }
 
 }  // extern "C"

@@ -1,0 +1,494 @@
+// Flash-attention backward for gfx950: (dQ, dK, dV) of O = softmax(scale Q K^T, causal) V
+// from dO, Q, K, V and the forward's O and log-sum-exp; GQA, 16-bit storage, f32
+// accumulate, f32 gradients.
+//
+// Three kernels, no atomics, results independent of scheduling:
+//   flash_bwd_delta_kernel   Delta[q] = sum_d dO[q][d] O[q][d]
+//   flash_bwd_dq_kernel      one workgroup per 256 query rows, walks the key tiles
+//   flash_bwd_dkdv_kernel    one workgroup per 128 keys of one KV head, walks the
+//                            query tiles of every query head that shares the KV head
+// Both walkers recompute P = exp(scale S - LSE) and dS = P (dP - Delta) tile by tile.
+// As in the forward kernel the products are oriented so that the index a lane owns
+// (its query row in the dQ kernel, its key in the dK/dV kernel) is the one the
+// second product does NOT contract over, so P and dS go from accumulator registers
+// straight into the next MFMA as its B operand:
+//   dQ kernel    S^T = K Q^T, dP^T = V dO^T        (lane: one query, 16 keys / tile)
+//                dQ^T += K^T dS^T                   (K^T by transposing LDS read)
+//   dK/dV kernel S = Q K^T, dP = dO V^T             (lane: one key, 16 queries / tile)
+//                dV^T += dO^T P,  dK^T += Q^T dS    (dO^T, Q^T by transposing LDS read)
+// Every LDS tile keeps the natural [row][D] layout and is read both by rows
+// (ds_read_b128) and transposed (ds_read_b64_tr_b16); one chunk swizzle serves both.
+#pragma once
+#include "flash_attn.h"
+
+namespace tsr950 {
+
+struct FlashBwdParams {
+  const uint16_t* Q;    // [B, Hq, Sq, D]
+  const uint16_t* K;    // [B, Hkv, Sk, D]
+  const uint16_t* V;    // [B, Hkv, Sk, D]
+  const uint16_t* dO;   // [B, Hq, Sq, D]
+  const float* O;       // [B, Hq, Sq, D]  forward output
+  const float* LSE;     // [B, Hq, Sq]     forward log-sum-exp (natural log, of scaled scores)
+  float* Delta;         // [B, Hq, Sq]     workspace
+  float* dQ;            // [B, Hq, Sq, D]
+  float* dK;            // [B, Hkv, Sk, D]
+  float* dV;            // [B, Hkv, Sk, D]
+  int B, Hq, Hkv, Sq, Sk;
+  float scale;
+  int causal;
+};
+
+constexpr float kLog2e = 1.44269504088896340736f;
+
+// Chunk swizzle of a [row][D] tile of 16-byte chunks that is conflict-free both for
+// row reads (16 consecutive rows, one chunk column) and for transposing reads
+// (4 consecutive rows x two adjacent chunks): a bit permutation of the row index
+// that is a bijection over the rows sharing a 256-byte bank line and moves the
+// row's low bits away from bit 0 of the chunk index.
+template <int D>
+__device__ __forceinline__ int bwd_swz(int row) {
+  if constexpr (D == 128) return ((row & 3) << 2) | ((row >> 2) & 3);
+  const int t = (row >> 1) & 7;
+  return ((t & 1) << 2) | (t >> 1);
+}
+
+// Delta[row] = sum_d dO[row][d] * O[row][d]; 16 lanes per row, 8 columns per lane per pass.
+template <class T>
+__global__ void flash_bwd_delta_kernel(const uint16_t* __restrict__ dO, const float* __restrict__ O,
+                                       float* __restrict__ Delta, long rows, int D) {
+  const long row = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+  const int part = threadIdx.x & 15;
+  float acc = 0.f;
+  if (row < rows) {
+    for (int d = part * 8; d < D; d += 128) {
+      const uint4 g = *reinterpret_cast<const uint4*>(dO + row * D + d);
+      const float4 o0 = *reinterpret_cast<const float4*>(O + row * D + d);
+      const float4 o1 = *reinterpret_cast<const float4*>(O + row * D + d + 4);
+      const uint32_t w[4] = {g.x, g.y, g.z, g.w};
+      const float ov[8] = {o0.x, o0.y, o0.z, o0.w, o1.x, o1.y, o1.z, o1.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc += from_storage<T>((uint16_t)(w[e] & 0xffff)) * ov[2 * e];
+        acc += from_storage<T>((uint16_t)(w[e] >> 16)) * ov[2 * e + 1];
+      }
+    }
+  }
+#pragma unroll
+  for (int s = 8; s >= 1; s >>= 1) acc += __shfl_xor(acc, s, 64);
+  if (row < rows && part == 0) Delta[row] = acc;
+}
+
+// ---------------------------------------------------------------------------------
+// dQ: 8 waves x 32 query rows; K/V tiles of 64 keys stream global -> LDS.
+// ---------------------------------------------------------------------------------
+constexpr int FB_BQ = 256, FB_BKV = 64, FB_DQ_THREADS = 512;
+
+template <class T, int D>
+__global__ __launch_bounds__(FB_DQ_THREADS, 1) void flash_bwd_dq_kernel(const FlashBwdParams p) {
+  constexpr int KSTEPS = D / 16, DT = D / 32, ROWB = D * 2, CHUNKS = D / 8;
+  constexpr int TILE = FB_BKV * ROWB;
+  constexpr int LD_PER_THREAD = FB_BKV * CHUNKS / FB_DQ_THREADS;
+  static_assert(FB_BKV * CHUNKS % FB_DQ_THREADS == 0, "tile/thread mismatch");
+  extern __shared__ __attribute__((aligned(16))) char smem[];   // K stages 0,1 | V stages 2,3
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(TSR_LDS char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, lh = lane >> 5, r16 = lane & 15;
+
+  const int qblocks = (p.Sq + FB_BQ - 1) / FB_BQ;
+  const int qb = qblocks - 1 - blockIdx.x / (p.B * p.Hq);      // heavy causal blocks first
+  const int bh = blockIdx.x % (p.B * p.Hq);
+  const int b = bh / p.Hq, hq = bh % p.Hq;
+  const int hkv = (int)(((long)hq * p.Hkv) / p.Hq);
+  const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
+  const int q0 = qb * FB_BQ, qw = q0 + wave * 32;
+  const long qrow0 = (long)(b * p.Hq + hq) * p.Sq;
+  const uint16_t* Kb = p.K + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
+  const uint16_t* Vb = p.V + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
+
+  int kv_end = p.Sk;
+  if (p.causal) kv_end = min(p.Sk, min(q0 + FB_BQ, p.Sq) - 1 + off + 1);
+  const int ntiles = (kv_end + FB_BKV - 1) / FB_BKV;
+  int nt_w = 0;
+  if (qw < p.Sq) {
+    int e = kv_end;
+    if (p.causal) e = min(kv_end, min(qw + 32, p.Sq) - 1 + off + 1);
+    nt_w = (e + FB_BKV - 1) / FB_BKV;
+  }
+
+  // resident operands of this lane's query row
+  const int qi = qw + l32;
+  const int qrow = qi < p.Sq ? qi : p.Sq - 1;
+  uint4 qf[KSTEPS], dof[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) {
+    qf[ks] = *reinterpret_cast<const uint4*>(p.Q + (qrow0 + qrow) * D + 16 * ks + 8 * lh);
+    dof[ks] = *reinterpret_cast<const uint4*>(p.dO + (qrow0 + qrow) * D + 16 * ks + 8 * lh);
+  }
+  const float c = p.scale * kLog2e;
+  const float lse2 = p.LSE[qrow0 + qrow] * kLog2e;
+  const float delta = p.Delta[qrow0 + qrow];
+  const int lim = qi >= p.Sq ? -1 : (p.causal ? min(qi + off, p.Sk - 1) : p.Sk - 1);
+
+  // tile loaders (global -> LDS, swizzle applied on the global address)
+  int ld_row[LD_PER_THREAD];
+  uint32_t ld_off[LD_PER_THREAD];
+#pragma unroll
+  for (int q = 0; q < LD_PER_THREAD; ++q) {
+    const int P = (wave * LD_PER_THREAD + q) * 64 + lane;
+    const int row = P / CHUNKS, chp = P % CHUNKS;
+    ld_row[q] = row;
+    ld_off[q] = row * ROWB + ((chp ^ bwd_swz<D>(row)) << 4);
+  }
+  auto load_tile = [&](const uint16_t* base, int tile, int lds_stage) {
+    const uint16_t* tb = base + (long)tile * FB_BKV * D;
+    const bool full = (tile + 1) * FB_BKV <= p.Sk;
+#pragma unroll
+    for (int q = 0; q < LD_PER_THREAD; ++q) {
+      uint32_t o = ld_off[q];
+      if (!full) {
+        const int last = p.Sk - 1 - tile * FB_BKV;
+        if (ld_row[q] > last) o -= (uint32_t)(ld_row[q] - last) * ROWB;
+      }
+      load16_to_lds(tb, o, lds0 + lds_stage * TILE + (wave * LD_PER_THREAD + q) * 1024);
+    }
+  };
+
+  // read addresses: rows (b128) and transposed (tr16) forms of a tile
+  uint32_t row_rd[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) row_rd[ks] = l32 * ROWB + ((((ks << 1) | lh) ^ bwd_swz<D>(l32)) << 4);
+  uint32_t tr_lo[DT], tr_hi[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const int key = 4 * lh + (r16 >> 2);
+    const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (r16 & 3);
+    tr_lo[dt] = key * ROWB + (((col >> 3) ^ bwd_swz<D>(key)) << 4) + (col & 7) * 2;
+    tr_hi[dt] = (key + 8) * ROWB + (((col >> 3) ^ bwd_swz<D>(key + 8)) << 4) + (col & 7) * 2;
+  }
+
+  f32x16 dq[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dq[dt][r] = 0.f;
+
+  if (ntiles > 0) {
+    load_tile(Kb, 0, 0);
+    load_tile(Vb, 0, 2);
+  }
+  fa_wait_loads();
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    const int st = t & 1;
+    if (t + 1 < ntiles) {
+      load_tile(Kb, t + 1, st ^ 1);
+      load_tile(Vb, t + 1, 2 + (st ^ 1));
+    }
+    if (t < nt_w) {
+      const int kv0 = t * FB_BKV;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const uint4 kf = lds_read_b128(smem, row_rd[ks] + st * TILE + kt * 32 * ROWB);
+          const uint4 vf = lds_read_b128(smem, row_rd[ks] + (2 + st) * TILE + kt * 32 * ROWB);
+          s = mfma_32x32x16<T>(kf, qf[ks], s);
+          dp = mfma_32x32x16<T>(vf, dof[ks], dp);
+        }
+        // lane: query qi, keys kv0 + 32 kt + 8 (r/4) + 4 lh + r % 4
+        uint4 dsf[2];
+        uint32_t w[8];
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          float ds2[2];
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const int rr = r + e;
+            const int key = kv0 + kt * 32 + 8 * (rr >> 2) + 4 * lh + (rr & 3);
+            const float pr = key <= lim ? fast_exp2(fmaf(s[rr], c, -lse2)) : 0.f;
+            ds2[e] = pr * (dp[rr] - delta);
+          }
+          w[r >> 1] = pack2<T>(ds2[0], ds2[1]);
+        }
+        dsf[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        dsf[1] = make_uint4(w[4], w[5], w[6], w[7]);
+        // dQ^T += K^T dS^T over the 16-key steps (kt, g)
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            const uint32_t o = st * TILE + (kt * 32 + g * 16) * ROWB;
+            const uint2 lo = lds_read_tr16_b64(smem + tr_lo[dt] + o);
+            const uint2 hi = lds_read_tr16_b64(smem + tr_hi[dt] + o);
+            dq[dt] = mfma_32x32x16<T>(make_uint4(lo.x, lo.y, hi.x, hi.y), dsf[g], dq[dt]);
+          }
+      }
+    }
+    fa_wait_loads();
+    __syncthreads();
+  }
+  if (qi >= p.Sq) return;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int d = dt * 32 + 8 * a + 4 * lh;
+      *reinterpret_cast<float4*>(p.dQ + (qrow0 + qi) * D + d) =
+          make_float4(dq[dt][4 * a] * p.scale, dq[dt][4 * a + 1] * p.scale, dq[dt][4 * a + 2] * p.scale,
+                      dq[dt][4 * a + 3] * p.scale);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// dK, dV: 4 waves x 32 keys; Q / dO tiles of 64 query rows (plus their LSE and Delta)
+// are staged through LDS for every query head of the KV head's group.
+// ---------------------------------------------------------------------------------
+constexpr int FB_BK = 128, FB_BQT = 64, FB_DKV_THREADS = 256;
+
+template <class T, int D>
+__global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const FlashBwdParams p) {
+  constexpr int KSTEPS = D / 16, DT = D / 32, ROWB = D * 2, CHUNKS = D / 8;
+  constexpr int TILE = FB_BQT * ROWB;                      // bytes of a Q (or dO) tile
+  constexpr int STAGE = 2 * TILE + 2 * FB_BQT * 4;         // Q | dO | lse2[64] | delta[64]
+  constexpr int LD_PER_THREAD = FB_BQT * CHUNKS / FB_DKV_THREADS;
+  static_assert(FB_BQT * CHUNKS % FB_DKV_THREADS == 0, "tile/thread mismatch");
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, lh = lane >> 5, r16 = lane & 15;
+
+  const int kblocks = (p.Sk + FB_BK - 1) / FB_BK;
+  const int kb = blockIdx.x % kblocks;
+  const int bh = blockIdx.x / kblocks;
+  const int b = bh / p.Hkv, hkv = bh % p.Hkv;
+  const int ratio = p.Hq / p.Hkv;
+  const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
+  const int k0 = kb * FB_BK;
+  const int key = k0 + wave * 32 + l32;                    // this lane's key
+  const int krow = key < p.Sk ? key : p.Sk - 1;
+  const long kvrow0 = (long)(b * p.Hkv + hkv) * p.Sk;
+
+  uint4 kf[KSTEPS], vf[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) {
+    kf[ks] = *reinterpret_cast<const uint4*>(p.K + (kvrow0 + krow) * D + 16 * ks + 8 * lh);
+    vf[ks] = *reinterpret_cast<const uint4*>(p.V + (kvrow0 + krow) * D + 16 * ks + 8 * lh);
+  }
+  const float c = p.scale * kLog2e;
+
+  // first query row that can see this workgroup's keys
+  int q_first = 0;
+  if (p.causal) q_first = max(0, k0 - off);
+  const int t_first = q_first / FB_BQT;
+  const int qtiles = (p.Sq + FB_BQT - 1) / FB_BQT;
+  const int steps_per_head = max(qtiles - t_first, 0);
+  const int nsteps = steps_per_head * ratio;
+
+  // loaders: chunk v = tid + THREADS q -> row v / CHUNKS, chunk v % CHUNKS
+  uint4 rq[LD_PER_THREAD], rdo[LD_PER_THREAD];
+  float rl = 0.f, rd = 0.f;
+  auto gload = [&](int step) {
+    const int hq = hkv * ratio + step / steps_per_head;
+    const int qt0 = (t_first + step % steps_per_head) * FB_BQT;
+    const long qrow0 = (long)(b * p.Hq + hq) * p.Sq;
+#pragma unroll
+    for (int q = 0; q < LD_PER_THREAD; ++q) {
+      const int v = tid + FB_DKV_THREADS * q;
+      int row = qt0 + v / CHUNKS;
+      row = row < p.Sq ? row : p.Sq - 1;
+      const long o = (qrow0 + row) * D + (v % CHUNKS) * 8;
+      rq[q] = *reinterpret_cast<const uint4*>(p.Q + o);
+      rdo[q] = *reinterpret_cast<const uint4*>(p.dO + o);
+    }
+    if (tid < FB_BQT) {
+      int row = qt0 + tid;
+      row = row < p.Sq ? row : p.Sq - 1;
+      rl = p.LSE[qrow0 + row] * kLog2e;
+      rd = p.Delta[qrow0 + row];
+    }
+  };
+  auto lstore = [&](int stage) {
+    char* base = smem + stage * STAGE;
+#pragma unroll
+    for (int q = 0; q < LD_PER_THREAD; ++q) {
+      const int v = tid + FB_DKV_THREADS * q;
+      const int row = v / CHUNKS, ch = v % CHUNKS;
+      const uint32_t o = row * ROWB + ((ch ^ bwd_swz<D>(row)) << 4);
+      lds_write_b128(base, o, rq[q]);
+      lds_write_b128(base, TILE + o, rdo[q]);
+    }
+    if (tid < FB_BQT) {
+      reinterpret_cast<float*>(base + 2 * TILE)[tid] = rl;
+      reinterpret_cast<float*>(base + 2 * TILE + FB_BQT * 4)[tid] = rd;
+    }
+  };
+
+  uint32_t row_rd[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) row_rd[ks] = l32 * ROWB + ((((ks << 1) | lh) ^ bwd_swz<D>(l32)) << 4);
+  uint32_t tr_lo[DT], tr_hi[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const int qq = 4 * lh + (r16 >> 2);
+    const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (r16 & 3);
+    tr_lo[dt] = qq * ROWB + (((col >> 3) ^ bwd_swz<D>(qq)) << 4) + (col & 7) * 2;
+    tr_hi[dt] = (qq + 8) * ROWB + (((col >> 3) ^ bwd_swz<D>(qq + 8)) << 4) + (col & 7) * 2;
+  }
+
+  f32x16 dk[DT], dv[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.f; dv[dt][r] = 0.f; }
+
+  if (nsteps > 0) {
+    gload(0);
+    lstore(0);
+  }
+  __syncthreads();
+  for (int step = 0; step < nsteps; ++step) {
+    const int st = step & 1;
+    if (step + 1 < nsteps) gload(step + 1);
+    const char* base = smem + st * STAGE;
+    const int qt0 = (t_first + step % steps_per_head) * FB_BQT;
+    // this wave's keys see the tile at all?  (uniform per wave)
+    const int wave_k0 = k0 + wave * 32;
+    const bool live = wave_k0 < p.Sk && (!p.causal || wave_k0 <= min(qt0 + FB_BQT, p.Sq) - 1 + off);
+    if (live) {
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const uint4 qfr = lds_read_b128(base, row_rd[ks] + qt * 32 * ROWB);
+          const uint4 dofr = lds_read_b128(base, TILE + row_rd[ks] + qt * 32 * ROWB);
+          s = mfma_32x32x16<T>(qfr, kf[ks], s);
+          dp = mfma_32x32x16<T>(dofr, vf[ks], dp);
+        }
+        // lane: key, queries qt0 + 32 qt + 8 (r/4) + 4 lh + r % 4
+        uint32_t pw[8], dw[8];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          const int qoff = 32 * qt + 8 * a + 4 * lh;
+          const float4 l4 = *reinterpret_cast<const float4*>(base + 2 * TILE + qoff * 4);
+          const float4 d4 = *reinterpret_cast<const float4*>(base + 2 * TILE + FB_BQT * 4 + qoff * 4);
+          const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
+          float pr[4], ds[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int q = qt0 + qoff + e;
+            const bool ok = q < p.Sq && key < p.Sk && (!p.causal || key <= q + off);
+            pr[e] = ok ? fast_exp2(fmaf(s[4 * a + e], c, -lv[e])) : 0.f;
+            ds[e] = pr[e] * (dp[4 * a + e] - dl[e]);
+          }
+          pw[2 * a] = pack2<T>(pr[0], pr[1]);
+          pw[2 * a + 1] = pack2<T>(pr[2], pr[3]);
+          dw[2 * a] = pack2<T>(ds[0], ds[1]);
+          dw[2 * a + 1] = pack2<T>(ds[2], ds[3]);
+        }
+        const uint4 pf[2] = {make_uint4(pw[0], pw[1], pw[2], pw[3]), make_uint4(pw[4], pw[5], pw[6], pw[7])};
+        const uint4 dsf[2] = {make_uint4(dw[0], dw[1], dw[2], dw[3]), make_uint4(dw[4], dw[5], dw[6], dw[7])};
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            const uint32_t o = (qt * 32 + g * 16) * ROWB;
+            const uint2 qlo = lds_read_tr16_b64(base + tr_lo[dt] + o);
+            const uint2 qhi = lds_read_tr16_b64(base + tr_hi[dt] + o);
+            const uint2 olo = lds_read_tr16_b64(base + TILE + tr_lo[dt] + o);
+            const uint2 ohi = lds_read_tr16_b64(base + TILE + tr_hi[dt] + o);
+            dv[dt] = mfma_32x32x16<T>(make_uint4(olo.x, olo.y, ohi.x, ohi.y), pf[g], dv[dt]);
+            dk[dt] = mfma_32x32x16<T>(make_uint4(qlo.x, qlo.y, qhi.x, qhi.y), dsf[g], dk[dt]);
+          }
+      }
+    }
+    if (step + 1 < nsteps) lstore(st ^ 1);
+    __syncthreads();
+  }
+  if (key >= p.Sk) return;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int d = dt * 32 + 8 * a + 4 * lh;
+      const long o = (kvrow0 + key) * D + d;
+      *reinterpret_cast<float4*>(p.dK + o) = make_float4(dk[dt][4 * a] * p.scale, dk[dt][4 * a + 1] * p.scale,
+                                                         dk[dt][4 * a + 2] * p.scale, dk[dt][4 * a + 3] * p.scale);
+      *reinterpret_cast<float4*>(p.dV + o) =
+          make_float4(dv[dt][4 * a], dv[dt][4 * a + 1], dv[dt][4 * a + 2], dv[dt][4 * a + 3]);
+    }
+}
+
+// Any head dimension: thread per query row (dQ) and thread per key row (dK, dV),
+// f32, recomputing P from the saved LSE.  Serves head dims other than 64 / 128.
+template <class T>
+__global__ void flash_bwd_generic_dq_kernel(const FlashBwdParams p, int D) {
+  const long row = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= (long)p.B * p.Hq * p.Sq) return;
+  const int qi = (int)(row % p.Sq), hq = (int)((row / p.Sq) % p.Hq), b = (int)(row / ((long)p.Sq * p.Hq));
+  const int hkv = (int)(((long)hq * p.Hkv) / p.Hq);
+  const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
+  const uint16_t* q = p.Q + row * D;
+  const uint16_t* g = p.dO + row * D;
+  const uint16_t* Kb = p.K + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
+  const uint16_t* Vb = p.V + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
+  float acc[256];
+  for (int d = 0; d < D; ++d) acc[d] = 0.f;
+  const int jmax = p.causal ? min(qi + off, p.Sk - 1) : p.Sk - 1;
+  const float lse = p.LSE[row], delta = p.Delta[row];
+  for (int j = 0; j <= jmax; ++j) {
+    float s = 0.f, dp = 0.f;
+    for (int d = 0; d < D; ++d) {
+      s += from_storage<T>(q[d]) * from_storage<T>(Kb[(long)j * D + d]);
+      dp += from_storage<T>(g[d]) * from_storage<T>(Vb[(long)j * D + d]);
+    }
+    const float ds = __expf(s * p.scale - lse) * (dp - delta);
+    for (int d = 0; d < D; ++d) acc[d] += ds * from_storage<T>(Kb[(long)j * D + d]);
+  }
+  for (int d = 0; d < D; ++d) p.dQ[row * D + d] = acc[d] * p.scale;
+}
+
+template <class T>
+__global__ void flash_bwd_generic_dkdv_kernel(const FlashBwdParams p, int D) {
+  const long row = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= (long)p.B * p.Hkv * p.Sk) return;
+  const int j = (int)(row % p.Sk), hkv = (int)((row / p.Sk) % p.Hkv), b = (int)(row / ((long)p.Sk * p.Hkv));
+  const int ratio = p.Hq / p.Hkv;
+  const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
+  const uint16_t* k = p.K + row * D;
+  const uint16_t* v = p.V + row * D;
+  float ak[256], av[256];
+  for (int d = 0; d < D; ++d) { ak[d] = 0.f; av[d] = 0.f; }
+  for (int r = 0; r < ratio; ++r) {
+    const int hq = hkv * ratio + r;
+    const long qrow0 = (long)(b * p.Hq + hq) * p.Sq;
+    const int i0 = p.causal ? max(0, j - off) : 0;
+    for (int i = i0; i < p.Sq; ++i) {
+      const uint16_t* q = p.Q + (qrow0 + i) * D;
+      const uint16_t* g = p.dO + (qrow0 + i) * D;
+      float s = 0.f, dp = 0.f;
+      for (int d = 0; d < D; ++d) {
+        s += from_storage<T>(q[d]) * from_storage<T>(k[d]);
+        dp += from_storage<T>(g[d]) * from_storage<T>(v[d]);
+      }
+      const float pr = __expf(s * p.scale - p.LSE[qrow0 + i]);
+      const float ds = pr * (dp - p.Delta[qrow0 + i]);
+      for (int d = 0; d < D; ++d) {
+        av[d] += pr * from_storage<T>(g[d]);
+        ak[d] += ds * from_storage<T>(q[d]);
+      }
+    }
+  }
+  for (int d = 0; d < D; ++d) {
+    p.dK[row * D + d] = ak[d] * p.scale;
+    p.dV[row * D + d] = av[d];
+  }
+}
+
+}  // namespace tsr950

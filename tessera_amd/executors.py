@@ -76,6 +76,8 @@ KNOWN_EXECUTORS: dict[str, str] = {
                    "(tessera_gfx950_gemm_* C ABI)",
     "gfx950_flash_attn": "flash_attn / multi_head / gqa / mqa attention forward, f16/bf16 -> f32, "
                          "causal + GQA, MFMA FA-2 (tessera_gfx950_flash_attn_gqa_* C ABI)",
+    "gfx950_flash_attn_bwd": "flash_attn_bwd / flash_attn_vjp: (dO, Q, K, V) -> (dQ, dK, dV) f32, causal + GQA, "
+                             "forward recomputed on device (tessera_gfx950_flash_attn_bwd_* C ABI)",
     "gfx950_moe_transport": "tessera.moe_dispatch / moe_combine / grouped_gemm / grouped_swiglu on "
                             "device gather, slot-ordered scatter-add and grouped MFMA GEMM",
     "gfx950_quant_gemm": "tessera.fp8_gemm (e4m3 codes + per-tensor scales) and tessera.w8a8_gemm "
@@ -93,6 +95,11 @@ EXECUTION_ROWS: dict[tuple[str, str], ExecutionRow] = {
         compiler_path="gfx950_flash_attn", executor_id="gfx950_flash_attn",
         reason="attention forward runs the hand-written gfx950 MFMA FA-2 kernel "
                "(causal, GQA, LSE)", **_ROW),
+    (TARGET, "gfx950_flash_attn_bwd"): ExecutionRow(
+        compiler_path="gfx950_flash_attn_bwd", executor_id="gfx950_flash_attn_bwd",
+        reason="attention backward runs the gfx950 MFMA dQ and dK/dV kernels; O and the "
+               "log-sum-exp are recomputed by the forward kernel (nothing saved)",
+        direction="backward", op_family="flash_attn", **_ROW),
     (TARGET, "gfx950_moe_transport"): ExecutionRow(
         compiler_path="gfx950_moe_transport", executor_id="gfx950_moe_transport",
         reason="MoE dispatch / combine / grouped GEMM / grouped SwiGLU on the gfx950 lane", **_ROW),
@@ -204,6 +211,27 @@ def execute_gfx950_flash_attn(artifact: RuntimeArtifact, args: Any):
     return _ops.gqa_attention(q, k, v, scale=kwargs.get("scale"), causal=bool(kwargs.get("causal", False)), out="f32")
 
 
+_FA_BWD_OPS = ("tessera.flash_attn_bwd", "tessera.flash_attn_vjp")
+
+
+def execute_gfx950_flash_attn_bwd(artifact: RuntimeArtifact, args: Any):
+    """Attention backward: operands ``(dO, Q, K, V)`` -> the tuple ``(dQ, dK, dV)``
+    in f32 shaped like ``(Q, K, V)`` (``runtime.py:7598-7665``).  ``kwargs``:
+    ``causal``, ``scale``; an additive bias, sliding window or logit soft-cap is
+    not on this lane and is rejected."""
+    md = artifact.metadata or {}
+    op = _single_op(artifact, _FA_BWD_OPS, "gfx950_flash_attn_bwd")
+    names = [str(n) for n in op.get("operands", [])]
+    if len(names) != 4:
+        raise ValueError("gfx950 flash_attn backward requires exactly the (dO, Q, K, V) operands")
+    values = _bind_launch_args(args, list(md.get("arg_names") or []))
+    do, q, k, v = (_as_array(values[n]) for n in names)
+    kwargs = op.get("kwargs") or {}
+    if kwargs.get("window") or kwargs.get("logit_softcap") or kwargs.get("attn_bias") is not None:
+        raise ValueError("gfx950 flash_attn backward handles scale + causal only (no bias / window / soft-cap)")
+    return _ops.flash_attn_backward(do, q, k, v, scale=kwargs.get("scale"), causal=bool(kwargs.get("causal", False)))
+
+
 def _plan_to_transport(plan: Any) -> _ops.MoETransport:
     """Accept the lane's own :class:`MoETransport` or a stdlib ``DispatchPlan``-like
     object (``expert_ids``, ``weights``, ``sort_perm``, ``group_sizes``,
@@ -292,6 +320,7 @@ def executor_table() -> dict[str, Callable[[RuntimeArtifact, Any], Any]]:
     return {
         "gfx950_gemm": execute_gfx950_gemm,
         "gfx950_flash_attn": execute_gfx950_flash_attn,
+        "gfx950_flash_attn_bwd": execute_gfx950_flash_attn_bwd,
         "gfx950_moe_transport": execute_gfx950_moe_transport,
         "gfx950_quant_gemm": execute_gfx950_quant_gemm,
     }

@@ -248,6 +248,44 @@ def _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa):
     return (o, lse) if return_lse else o
 
 
+def flash_attn_backward(dO, Q, K, V, scale=None, causal: bool = False):
+    """``(dQ, dK, dV)`` of ``softmax(scale * Q K^T, causal) V`` for the cotangent
+    ``dO`` — f32 arrays shaped like ``Q``, ``K``, ``V``.  ``Q``/``dO``
+    ``[..., Hq, Sq, D]``, ``K``/``V`` ``[..., Hkv, Sk, D]`` in one 16-bit storage
+    dtype; with ``Hkv < Hq`` the gradients of a KV head sum over its query heads.
+    The forward is recomputed on the device (nothing saved)."""
+    dO, Q, K, V = _unbox(dO), _unbox(Q), _unbox(K), _unbox(V)
+    st = _storage(Q, K)
+    if _storage(V) != st or _storage(dO) != st:
+        raise ValueError("dO, Q, K, V must share one storage dtype")
+    g, q, k, v = _bits(dO), _bits(Q), _bits(K), _bits(V)
+    for name, arr in (("dO", g), ("Q", q), ("K", k), ("V", v)):
+        if arr.ndim < 2:
+            raise ValueError(f"flash_attn backward {name} must be rank >= 2 ([..., S, D]); got {arr.shape}")
+    D = q.shape[-1]
+    if D <= 0 or D % 16 != 0:
+        raise ValueError(f"gfx950 flash_attn backward needs head_dim a positive multiple of 16; got {D}")
+    Hq = q.shape[-3] if q.ndim >= 3 else 1
+    Hkv = k.shape[-3] if k.ndim >= 3 else 1
+    if Hkv <= 0 or Hq % Hkv != 0:
+        raise ValueError(f"flash_attn backward GQA needs query-heads ({Hq}) divisible by kv-heads ({Hkv})")
+    if v.shape != k.shape or g.shape != q.shape or k.shape[-1] != D or q.shape[:-3] != k.shape[:-3]:
+        raise ValueError("flash_attn backward requires V==K, dO==Q, matching batch dims and a shared head_dim; "
+                         f"got Q{q.shape} K{k.shape} V{v.shape} dO{g.shape}")
+    Bq = int(np.prod(q.shape[:-3])) if q.ndim > 3 else 1
+    Sq, Sk = q.shape[-2], k.shape[-2]
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    dq = np.empty(q.shape, np.float32)
+    dk = np.empty(k.shape, np.float32)
+    dv = np.empty(k.shape, np.float32)
+    fn = getattr(_lane.load(), f"tessera_gfx950_flash_attn_bwd_{st}")
+    rc = fn(g.ctypes.data, q.ctypes.data, k.ctypes.data, v.ctypes.data, dq.ctypes.data, dk.ctypes.data,
+            dv.ctypes.data, Bq, Hq, Hkv, Sq, Sk, D, float(scale), 1 if causal else 0)
+    _lane.check(rc, "flash_attn_backward")
+    return dq, dk, dv
+
+
 def flash_attn(Q, K=None, V=None, scale=None, causal: bool = False, *, return_lse: bool = False,
                out: str = "storage"):
     """``softmax(scale * Q K^T, causal) V``.  Q/K/V ``[..., H, S, D]`` 16-bit; the

@@ -92,6 +92,10 @@ KERNEL_TABLE: tuple = (
                 ("tessera_gfx950_flash_attn_f16", "tessera_gfx950_flash_attn_bf16",
                  "tessera_gfx950_flash_attn_gqa_f16", "tessera_gfx950_flash_attn_gqa_bf16"),
                 "gfx950_flash_attn", "256 q rows x 64 keys, 8 waves of 32 rows", 65536),
+    KernelEntry("tessera.flash_attn_bwd", ("tessera_attn.backward",), "tessera_rocm.mfma_flash_attn_bwd", "m32n32k16",
+                "v_mfma_f32_32x32x16_{f16,bf16}", ("f16", "bf16"),
+                ("tessera_gfx950_flash_attn_bwd_f16", "tessera_gfx950_flash_attn_bwd_bf16"),
+                "gfx950_flash_attn_bwd", "dQ: 256 q rows x 64 keys; dK/dV: 128 keys x 64 q rows", 66560),
     KernelEntry("tessera.grouped_gemm", ("tile.matmul", "tile.mma"), "tessera_rocm.grouped_gemm", "m32n32k16",
                 "v_mfma_f32_32x32x16_bf16", ("bf16",),
                 ("tessera_gfx950_grouped_gemm_bf16", "tessera_gfx950_grouped_gemm_bf16_f32",

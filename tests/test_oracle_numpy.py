@@ -264,3 +264,42 @@ def test_int8_quantiser_and_w8a8():
     assert orc.max_rel_err(y, X @ W) < 0.05
     big = np.full((2, 70000), 127, np.int8)
     assert orc.gemm_i8_i32(big, big.T.copy())[0, 0] == 127 * 127 * 70000
+
+
+def test_flash_attn_backward_matches_torch_autograd_and_finite_differences():
+    import torch
+    rng = np.random.default_rng(5)
+    for (B, Hq, Hkv, Sq, Sk, D, causal) in [(1, 2, 2, 5, 5, 4, False), (2, 4, 2, 6, 9, 8, True), (1, 3, 1, 7, 7, 4, True)]:
+        q = rng.standard_normal((B, Hq, Sq, D))
+        k = rng.standard_normal((B, Hkv, Sk, D))
+        v = rng.standard_normal((B, Hkv, Sk, D))
+        do = rng.standard_normal((B, Hq, Sq, D))
+        dq, dk, dv = orc.flash_attn_backward(do, q, k, v, causal=causal)
+        # library: autograd through torch's attention with K/V repeated along heads
+        tq, tk, tv = (torch.tensor(a, requires_grad=True) for a in (q, k, v))
+        rep = Hq // Hkv
+        kk, vv = tk.repeat_interleave(rep, dim=1), tv.repeat_interleave(rep, dim=1)
+        mask = None
+        if causal:
+            i = torch.arange(Sq)[:, None]
+            j = torch.arange(Sk)[None, :]
+            mask = j <= i + max(Sk - Sq, 0)
+        out = torch.nn.functional.scaled_dot_product_attention(tq, kk, vv, attn_mask=mask)
+        out.backward(torch.tensor(do))
+        assert np.allclose(dq, tq.grad.numpy(), atol=1e-10)
+        assert np.allclose(dk, tk.grad.numpy(), atol=1e-10)
+        assert np.allclose(dv, tv.grad.numpy(), atol=1e-10)
+        # finite differences of the forward oracle on a few coordinates
+        def loss(qq, kk_, vv_):
+            o, _ = orc.flash_attn_dense(qq, kk_, vv_, causal=causal)
+            return float((o * do).sum())
+        eps = 1e-6
+        for arr, grad in ((q, dq), (k, dk), (v, dv)):
+            idx = tuple(rng.integers(0, n) for n in arr.shape)
+            hi, lo = arr.copy(), arr.copy()
+            hi[idx] += eps
+            lo[idx] -= eps
+            args_hi = [hi if a is arr else a for a in (q, k, v)]
+            args_lo = [lo if a is arr else a for a in (q, k, v)]
+            fd = (loss(*args_hi) - loss(*args_lo)) / (2 * eps)
+            assert abs(fd - grad[idx]) <= 1e-6 * max(1.0, abs(fd))
