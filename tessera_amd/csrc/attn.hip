@@ -109,8 +109,8 @@ int flash_bwd_dev(const void* dO, const void* Q, const void* K, const void* V, c
   if (probe_device() != kOk) return kNoDevice;
   const size_t rows = (size_t)B * Hq * Sq;
   const bool recompute = !O || !LSE;
-  float* ws = nullptr;                       // [O (rows * D) | LSE (rows)]? | Delta (rows)
-  const size_t ws_floats = rows + (recompute ? rows * D + rows : 0);
+  float* ws = nullptr;                       // Delta (rows) | LSE2 (rows) | [O (rows * D) | LSE (rows)]?
+  const size_t ws_floats = 2 * rows + (recompute ? rows * D + rows : 0);
   if (hipMallocAsync(reinterpret_cast<void**>(&ws), ws_floats * sizeof(float), s) != hipSuccess) {
     (void)hipGetLastError();
     return kDeviceFailed;
@@ -118,7 +118,7 @@ int flash_bwd_dev(const void* dO, const void* Q, const void* K, const void* V, c
   int rc = kOk;
   float* delta = ws;
   if (recompute) {
-    float* o_ws = ws + rows;
+    float* o_ws = ws + 2 * rows;
     float* lse_ws = o_ws + rows * D;
     rc = flash_dev<T>(Q, K, V, o_ws, lse_ws, B, Hq, Hkv, Sq, Sk, D, scale, causal, 0, s);
     O = o_ws;
@@ -130,13 +130,13 @@ int flash_bwd_dev(const void* dO, const void* Q, const void* K, const void* V, c
     p.K = static_cast<const uint16_t*>(K);
     p.V = static_cast<const uint16_t*>(V);
     p.dO = static_cast<const uint16_t*>(dO);
-    p.O = O; p.LSE = LSE; p.Delta = delta;
+    p.O = O; p.LSE = LSE; p.Delta = delta; p.LSE2 = ws + rows;
     p.dQ = dQ; p.dK = dK; p.dV = dV;
     p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Sq = Sq; p.Sk = Sk;
     p.scale = scale;
     p.causal = causal ? 1 : 0;
     hipLaunchKernelGGL((flash_bwd_delta_kernel<T>), dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, s,
-                       p.dO, p.O, delta, (long)rows, D);
+                       p.dO, p.O, p.LSE, delta, p.LSE2, (long)rows, D);
     rc = launch_status();
     const bool al = ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
                       reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(dO) |

@@ -31,6 +31,7 @@ struct FlashBwdParams {
   const float* O;       // [B, Hq, Sq, D]  forward output
   const float* LSE;     // [B, Hq, Sq]     forward log-sum-exp (natural log, of scaled scores)
   float* Delta;         // [B, Hq, Sq]     workspace
+  float* LSE2;          // [B, Hq, Sq]     workspace: LSE * log2(e)
   float* dQ;            // [B, Hq, Sq, D]
   float* dK;            // [B, Hkv, Sk, D]
   float* dV;            // [B, Hkv, Sk, D]
@@ -40,6 +41,12 @@ struct FlashBwdParams {
 };
 
 constexpr float kLog2e = 1.44269504088896340736f;
+
+// 4 bytes per lane from global memory straight into LDS: lane i lands at lds_base + 4 i.
+__device__ __forceinline__ void load4_to_lds(const void* base, uint32_t byte_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :: "s"(lds_base), "v"(byte_off), "s"(base) : "memory");
+}
 
 // Chunk swizzle of a [row][D] tile of 16-byte chunks that is conflict-free both for
 // row reads (16 consecutive rows, one chunk column) and for transposing reads
@@ -53,10 +60,12 @@ __device__ __forceinline__ int bwd_swz(int row) {
   return ((t & 1) << 2) | (t >> 1);
 }
 
-// Delta[row] = sum_d dO[row][d] * O[row][d]; 16 lanes per row, 8 columns per lane per pass.
+// Delta[row] = sum_d dO[row][d] * O[row][d] and LSE2[row] = LSE[row] * log2(e);
+// 16 lanes per row, 8 columns per lane per pass.
 template <class T>
 __global__ void flash_bwd_delta_kernel(const uint16_t* __restrict__ dO, const float* __restrict__ O,
-                                       float* __restrict__ Delta, long rows, int D) {
+                                       const float* __restrict__ LSE, float* __restrict__ Delta,
+                                       float* __restrict__ LSE2, long rows, int D) {
   const long row = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
   const int part = threadIdx.x & 15;
   float acc = 0.f;
@@ -76,7 +85,10 @@ __global__ void flash_bwd_delta_kernel(const uint16_t* __restrict__ dO, const fl
   }
 #pragma unroll
   for (int s = 8; s >= 1; s >>= 1) acc += __shfl_xor(acc, s, 64);
-  if (row < rows && part == 0) Delta[row] = acc;
+  if (row < rows && part == 0) {
+    Delta[row] = acc;
+    LSE2[row] = LSE[row] * kLog2e;
+  }
 }
 
 // ---------------------------------------------------------------------------------
@@ -127,7 +139,7 @@ __global__ __launch_bounds__(FB_DQ_THREADS, 1) void flash_bwd_dq_kernel(const Fl
     dof[ks] = *reinterpret_cast<const uint4*>(p.dO + (qrow0 + qrow) * D + 16 * ks + 8 * lh);
   }
   const float c = p.scale * kLog2e;
-  const float lse2 = p.LSE[qrow0 + qrow] * kLog2e;
+  const float lse2 = p.LSE2[qrow0 + qrow];
   const float delta = p.Delta[qrow0 + qrow];
   const int lim = qi >= p.Sq ? -1 : (p.causal ? min(qi + off, p.Sk - 1) : p.Sk - 1);
 
@@ -210,7 +222,9 @@ __global__ __launch_bounds__(FB_DQ_THREADS, 1) void flash_bwd_dq_kernel(const Fl
           for (int e = 0; e < 2; ++e) {
             const int rr = r + e;
             const int key = kv0 + kt * 32 + 8 * (rr >> 2) + 4 * lh + (rr & 3);
-            const float pr = key <= lim ? fast_exp2(fmaf(s[rr], c, -lse2)) : 0.f;
+            // masked keys get exponent -inf (P = 0) by a select on the argument, so the
+            // exponential itself is unconditional straight-line code
+            const float pr = fast_exp2(key <= lim ? fmaf(s[rr], c, -lse2) : -INFINITY);
             ds2[e] = pr * (dp[rr] - delta);
           }
           w[r >> 1] = pack2<T>(ds2[0], ds2[1]);
@@ -255,15 +269,18 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
   constexpr int KSTEPS = D / 16, DT = D / 32, ROWB = D * 2, CHUNKS = D / 8;
   constexpr int TILE = FB_BQT * ROWB;                      // bytes of a Q (or dO) tile
   constexpr int STAGE = 2 * TILE + 2 * FB_BQT * 4;         // Q | dO | lse2[64] | delta[64]
-  constexpr int LD_PER_THREAD = FB_BQT * CHUNKS / FB_DKV_THREADS;
+  constexpr int LD_PER_WAVE = FB_BQT * CHUNKS / 64 / (FB_DKV_THREADS / 64);
   static_assert(FB_BQT * CHUNKS % FB_DKV_THREADS == 0, "tile/thread mismatch");
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(TSR_LDS char*)smem;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, lh = lane >> 5, r16 = lane & 15;
 
+  // heavy key blocks (seen by the most query rows under a causal mask) first
   const int kblocks = (p.Sk + FB_BK - 1) / FB_BK;
-  const int kb = blockIdx.x % kblocks;
-  const int bh = blockIdx.x / kblocks;
+  const int kb = blockIdx.x / (p.B * p.Hkv);
+  const int bh = blockIdx.x % (p.B * p.Hkv);
   const int b = bh / p.Hkv, hkv = bh % p.Hkv;
   const int ratio = p.Hq / p.Hkv;
   const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
@@ -271,6 +288,7 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
   const int key = k0 + wave * 32 + l32;                    // this lane's key
   const int krow = key < p.Sk ? key : p.Sk - 1;
   const long kvrow0 = (long)(b * p.Hkv + hkv) * p.Sk;
+  (void)kblocks;
 
   uint4 kf[KSTEPS], vf[KSTEPS];
 #pragma unroll
@@ -288,42 +306,35 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
   const int steps_per_head = max(qtiles - t_first, 0);
   const int nsteps = steps_per_head * ratio;
 
-  // loaders: chunk v = tid + THREADS q -> row v / CHUNKS, chunk v % CHUNKS
-  uint4 rq[LD_PER_THREAD], rdo[LD_PER_THREAD];
-  float rl = 0.f, rd = 0.f;
-  auto gload = [&](int step) {
+  // loaders: global -> LDS, one wave instruction = 64 consecutive 16-byte slots
+  int ld_row[LD_PER_WAVE];
+  uint32_t ld_off[LD_PER_WAVE];
+#pragma unroll
+  for (int q = 0; q < LD_PER_WAVE; ++q) {
+    const int P = (wave * LD_PER_WAVE + q) * 64 + lane;
+    const int row = P / CHUNKS, chp = P % CHUNKS;
+    ld_row[q] = row;
+    ld_off[q] = row * ROWB + ((chp ^ bwd_swz<D>(row)) << 4);
+  }
+  auto load_step = [&](int step, int stage) {
     const int hq = hkv * ratio + step / steps_per_head;
     const int qt0 = (t_first + step % steps_per_head) * FB_BQT;
     const long qrow0 = (long)(b * p.Hq + hq) * p.Sq;
+    const uint16_t* qb = p.Q + (qrow0 + qt0) * D;
+    const uint16_t* gb = p.dO + (qrow0 + qt0) * D;
+    const int last = p.Sq - 1 - qt0;                       // last valid row of this tile
+    const uint32_t sbase = lds0 + stage * STAGE;
 #pragma unroll
-    for (int q = 0; q < LD_PER_THREAD; ++q) {
-      const int v = tid + FB_DKV_THREADS * q;
-      int row = qt0 + v / CHUNKS;
-      row = row < p.Sq ? row : p.Sq - 1;
-      const long o = (qrow0 + row) * D + (v % CHUNKS) * 8;
-      rq[q] = *reinterpret_cast<const uint4*>(p.Q + o);
-      rdo[q] = *reinterpret_cast<const uint4*>(p.dO + o);
+    for (int q = 0; q < LD_PER_WAVE; ++q) {
+      uint32_t o = ld_off[q];
+      if (ld_row[q] > last) o -= (uint32_t)(ld_row[q] - last) * ROWB;   // rows past the end: masked later
+      load16_to_lds(qb, o, sbase + (wave * LD_PER_WAVE + q) * 1024);
+      load16_to_lds(gb, o, sbase + TILE + (wave * LD_PER_WAVE + q) * 1024);
     }
-    if (tid < FB_BQT) {
-      int row = qt0 + tid;
-      row = row < p.Sq ? row : p.Sq - 1;
-      rl = p.LSE[qrow0 + row] * kLog2e;
-      rd = p.Delta[qrow0 + row];
-    }
-  };
-  auto lstore = [&](int stage) {
-    char* base = smem + stage * STAGE;
-#pragma unroll
-    for (int q = 0; q < LD_PER_THREAD; ++q) {
-      const int v = tid + FB_DKV_THREADS * q;
-      const int row = v / CHUNKS, ch = v % CHUNKS;
-      const uint32_t o = row * ROWB + ((ch ^ bwd_swz<D>(row)) << 4);
-      lds_write_b128(base, o, rq[q]);
-      lds_write_b128(base, TILE + o, rdo[q]);
-    }
-    if (tid < FB_BQT) {
-      reinterpret_cast<float*>(base + 2 * TILE)[tid] = rl;
-      reinterpret_cast<float*>(base + 2 * TILE + FB_BQT * 4)[tid] = rd;
+    if (wave < 2) {
+      const float* src = (wave == 0 ? p.LSE2 : p.Delta) + qrow0 + qt0;
+      const int r = lane <= last ? lane : last;
+      load4_to_lds(src, (uint32_t)r * 4, sbase + 2 * TILE + wave * FB_BQT * 4);
     }
   };
 
@@ -345,33 +356,55 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.f; dv[dt][r] = 0.f; }
 
-  if (nsteps > 0) {
-    gload(0);
-    lstore(0);
-  }
+  if (nsteps > 0) load_step(0, 0);
+  fa_wait_loads();
   __syncthreads();
+  const int wave_k0 = k0 + wave * 32;
   for (int step = 0; step < nsteps; ++step) {
     const int st = step & 1;
-    if (step + 1 < nsteps) gload(step + 1);
+    if (step + 1 < nsteps) load_step(step + 1, st ^ 1);
     const char* base = smem + st * STAGE;
     const int qt0 = (t_first + step % steps_per_head) * FB_BQT;
-    // this wave's keys see the tile at all?  (uniform per wave)
-    const int wave_k0 = k0 + wave * 32;
+    // do this wave's keys see the tile at all?  (uniform per wave)
     const bool live = wave_k0 < p.Sk && (!p.causal || wave_k0 <= min(qt0 + FB_BQT, p.Sq) - 1 + off);
     if (live) {
+      // S = Q K^T and dP = dO V^T for both 32-row halves: four independent MFMA chains
+      // (operand fragments are read one k step ahead of the MFMAs that use them)
+      f32x16 s[2], dp[2];
+      uint4 qfr[2][2], dofr[2][2];                         // [buffer][qt]
 #pragma unroll
       for (int qt = 0; qt < 2; ++qt) {
-        f32x16 s, dp;
+        qfr[0][qt] = lds_read_b128(base, row_rd[0] + qt * 32 * ROWB);
+        dofr[0][qt] = lds_read_b128(base, TILE + row_rd[0] + qt * 32 * ROWB);
+      }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int cur = ks & 1;
+        if (ks + 1 < KSTEPS) {
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          const uint4 qfr = lds_read_b128(base, row_rd[ks] + qt * 32 * ROWB);
-          const uint4 dofr = lds_read_b128(base, TILE + row_rd[ks] + qt * 32 * ROWB);
-          s = mfma_32x32x16<T>(qfr, kf[ks], s);
-          dp = mfma_32x32x16<T>(dofr, vf[ks], dp);
+          for (int qt = 0; qt < 2; ++qt) {
+            qfr[cur ^ 1][qt] = lds_read_b128(base, row_rd[ks + 1] + qt * 32 * ROWB);
+            dofr[cur ^ 1][qt] = lds_read_b128(base, TILE + row_rd[ks + 1] + qt * 32 * ROWB);
+          }
         }
-        // lane: key, queries qt0 + 32 qt + 8 (r/4) + 4 lh + r % 4
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+          if (ks == 0) {
+            f32x16 z;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) z[r] = 0.f;
+            s[qt] = mfma_32x32x16<T>(qfr[cur][qt], kf[ks], z);
+            dp[qt] = mfma_32x32x16<T>(dofr[cur][qt], vf[ks], z);
+          } else {
+            s[qt] = mfma_32x32x16<T>(qfr[cur][qt], kf[ks], s[qt]);
+            dp[qt] = mfma_32x32x16<T>(dofr[cur][qt], vf[ks], dp[qt]);
+          }
+        }
+      }
+      // lane: key, queries qt0 + 32 qt + 8 (r/4) + 4 lh + r % 4
+      uint4 pf[2][2], dsf[2][2];
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
         uint32_t pw[8], dw[8];
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
@@ -383,32 +416,45 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int q = qt0 + qoff + e;
-            const bool ok = q < p.Sq && key < p.Sk && (!p.causal || key <= q + off);
-            pr[e] = ok ? fast_exp2(fmaf(s[4 * a + e], c, -lv[e])) : 0.f;
-            ds[e] = pr[e] * (dp[4 * a + e] - dl[e]);
+            const bool ok = (q < p.Sq) & (key < p.Sk) & (!p.causal | (key <= q + off));
+            // masked pairs get exponent -inf (P = 0) by a select on the argument
+            pr[e] = fast_exp2(ok ? fmaf(s[qt][4 * a + e], c, -lv[e]) : -INFINITY);
+            ds[e] = pr[e] * (dp[qt][4 * a + e] - dl[e]);
           }
           pw[2 * a] = pack2<T>(pr[0], pr[1]);
           pw[2 * a + 1] = pack2<T>(pr[2], pr[3]);
           dw[2 * a] = pack2<T>(ds[0], ds[1]);
           dw[2 * a + 1] = pack2<T>(ds[2], ds[3]);
         }
-        const uint4 pf[2] = {make_uint4(pw[0], pw[1], pw[2], pw[3]), make_uint4(pw[4], pw[5], pw[6], pw[7])};
-        const uint4 dsf[2] = {make_uint4(dw[0], dw[1], dw[2], dw[3]), make_uint4(dw[4], dw[5], dw[6], dw[7])};
+        pf[qt][0] = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+        pf[qt][1] = make_uint4(pw[4], pw[5], pw[6], pw[7]);
+        dsf[qt][0] = make_uint4(dw[0], dw[1], dw[2], dw[3]);
+        dsf[qt][1] = make_uint4(dw[4], dw[5], dw[6], dw[7]);
+      }
+      // second products, their transposed operands read one step ahead
+      constexpr int NSTEP = 4 * DT;                        // (qt, g, dt) steps
+      auto tr_frags = [&](int i, uint4& qT, uint4& oT) {
+        const int dt = i % DT, g = (i / DT) & 1, qt = i / (2 * DT);
+        const uint32_t o = (qt * 32 + g * 16) * ROWB;
+        const uint2 qlo = lds_read_tr16_b64(base + tr_lo[dt] + o);
+        const uint2 qhi = lds_read_tr16_b64(base + tr_hi[dt] + o);
+        const uint2 olo = lds_read_tr16_b64(base + TILE + tr_lo[dt] + o);
+        const uint2 ohi = lds_read_tr16_b64(base + TILE + tr_hi[dt] + o);
+        qT = make_uint4(qlo.x, qlo.y, qhi.x, qhi.y);
+        oT = make_uint4(olo.x, olo.y, ohi.x, ohi.y);
+      };
+      uint4 qT[2], oT[2];
+      tr_frags(0, qT[0], oT[0]);
 #pragma unroll
-        for (int g = 0; g < 2; ++g)
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) {
-            const uint32_t o = (qt * 32 + g * 16) * ROWB;
-            const uint2 qlo = lds_read_tr16_b64(base + tr_lo[dt] + o);
-            const uint2 qhi = lds_read_tr16_b64(base + tr_hi[dt] + o);
-            const uint2 olo = lds_read_tr16_b64(base + TILE + tr_lo[dt] + o);
-            const uint2 ohi = lds_read_tr16_b64(base + TILE + tr_hi[dt] + o);
-            dv[dt] = mfma_32x32x16<T>(make_uint4(olo.x, olo.y, ohi.x, ohi.y), pf[g], dv[dt]);
-            dk[dt] = mfma_32x32x16<T>(make_uint4(qlo.x, qlo.y, qhi.x, qhi.y), dsf[g], dk[dt]);
-          }
+      for (int i = 0; i < NSTEP; ++i) {
+        const int cur = i & 1;
+        if (i + 1 < NSTEP) tr_frags(i + 1, qT[cur ^ 1], oT[cur ^ 1]);
+        const int dt = i % DT, g = (i / DT) & 1, qt = i / (2 * DT);
+        dv[dt] = mfma_32x32x16<T>(oT[cur], pf[qt][g], dv[dt]);
+        dk[dt] = mfma_32x32x16<T>(qT[cur], dsf[qt][g], dk[dt]);
       }
     }
-    if (step + 1 < nsteps) lstore(st ^ 1);
+    fa_wait_loads();
     __syncthreads();
   }
   if (key >= p.Sk) return;
