@@ -111,3 +111,30 @@ def test_bench_abi(lane):
     assert 0 < ms.value < 100
     assert lib.tessera_gfx950_bench_last_timer_source() in (0, 1)
     assert "gfx950" in lane.device_name() and lane.device_cus() > 0
+
+
+def test_measured_arbitration_on_device(lane):
+    """Measure-at-first-miss on the real candidates: the verdict is keyed by the
+    rocm:gfx950 device tag and reused from the cache on the second call."""
+    from tessera_amd import autotune as at
+    from tessera_amd import candidates as cand
+    cand.register_all()
+    rng = np.random.default_rng(0)
+    A = (rng.standard_normal((256, 128)) * .1).astype(np.float32)
+    B = (rng.standard_normal((128, 192)) * .1).astype(np.float32)
+    region = cand.MatmulRegion(dtype="bfloat16")
+    cache = at.MeasureCache()
+    w = at.measured_arbitrate(region, cand.OP_MATMUL, cand.TARGET, A, B, dtype="bfloat16", cache=cache, reps=5,
+                              warmup=1, timing=at.TIMING_DEVICE)
+    assert w is not None and w.name == "gfx950_mfma_gemm"
+    (key, rec), = cache.items()
+    assert key[0] == "rocm:gfx950" and key[3] == (256, 256, 128) and rec.latency_ms > 0
+    hits = cache.hits
+    out, tag = at.run_measured_arbitrated(region, cand.OP_MATMUL, cand.TARGET, A, B, dtype="bfloat16", cache=cache,
+                                          timing=at.TIMING_DEVICE)
+    assert cache.hits == hits + 1 and tag == cand.GEMM_TAG
+    assert np.allclose(out, region.reference(A, B), atol=5e-3)
+    # the packaged corpus recommends the same winner for the headline GEMM bucket
+    big = np.zeros((8192, 8192), np.float32)
+    assert at.corpus_winner(region, cand.OP_MATMUL, cand.TARGET, big, big, dtype="bfloat16",
+                            timing=at.TIMING_DEVICE) == "gfx950_mfma_gemm"
