@@ -212,25 +212,34 @@ __global__ __launch_bounds__(FB_DQ_THREADS, 1) void flash_bwd_dq_kernel(const Fl
           s = mfma_32x32x16<T>(kf, qf[ks], s);
           dp = mfma_32x32x16<T>(vf, dof[ks], dp);
         }
-        // lane: query qi, keys kv0 + 32 kt + 8 (r/4) + 4 lh + r % 4
+        // lane: query qi, keys kv0 + 32 kt + 8 (r/4) + 4 lh + r % 4.  Only tiles that
+        // touch the causal diagonal or the end of Q / K pay for the per-key mask.
         uint4 dsf[2];
-        uint32_t w[8];
+        auto ds_part = [&](auto masked_c) {
+          constexpr bool MASKED = decltype(masked_c)::value;
+          uint32_t w[8];
 #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          float ds2[2];
+          for (int r = 0; r < 16; r += 2) {
+            float ds2[2];
 #pragma unroll
-          for (int e = 0; e < 2; ++e) {
-            const int rr = r + e;
-            const int key = kv0 + kt * 32 + 8 * (rr >> 2) + 4 * lh + (rr & 3);
-            // masked keys get exponent -inf (P = 0) by a select on the argument, so the
-            // exponential itself is unconditional straight-line code
-            const float pr = fast_exp2(key <= lim ? fmaf(s[rr], c, -lse2) : -INFINITY);
-            ds2[e] = pr * (dp[rr] - delta);
+            for (int e = 0; e < 2; ++e) {
+              const int rr = r + e;
+              float x = fmaf(s[rr], c, -lse2);
+              if constexpr (MASKED) {
+                const int key = kv0 + kt * 32 + 8 * (rr >> 2) + 4 * lh + (rr & 3);
+                x = key <= lim ? x : -INFINITY;          // exponent -inf: P = 0, no branch
+              }
+              ds2[e] = fast_exp2(x) * (dp[rr] - delta);
+            }
+            w[r >> 1] = pack2<T>(ds2[0], ds2[1]);
           }
-          w[r >> 1] = pack2<T>(ds2[0], ds2[1]);
-        }
-        dsf[0] = make_uint4(w[0], w[1], w[2], w[3]);
-        dsf[1] = make_uint4(w[4], w[5], w[6], w[7]);
+          dsf[0] = make_uint4(w[0], w[1], w[2], w[3]);
+          dsf[1] = make_uint4(w[4], w[5], w[6], w[7]);
+        };
+        const bool need_mask = (kv0 + kt * 32 + 32 > p.Sk) || (qw + 32 > p.Sq) ||
+                               (p.causal && kv0 + kt * 32 + 31 > qw + off);
+        if (need_mask) ds_part(std::true_type{});
+        else ds_part(std::false_type{});
         // dQ^T += K^T dS^T over the 16-key steps (kt, g)
 #pragma unroll
         for (int g = 0; g < 2; ++g)
@@ -401,36 +410,47 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
           }
         }
       }
-      // lane: key, queries qt0 + 32 qt + 8 (r/4) + 4 lh + r % 4
+      // lane: key, queries qt0 + 32 qt + 8 (r/4) + 4 lh + r % 4.  Only tiles that touch
+      // the causal diagonal or the end of Q / K pay for the per-pair mask.
       uint4 pf[2][2], dsf[2][2];
+      auto softmax_part = [&](auto masked_c) {
+        constexpr bool MASKED = decltype(masked_c)::value;
 #pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
-        uint32_t pw[8], dw[8];
+        for (int qt = 0; qt < 2; ++qt) {
+          uint32_t pw[8], dw[8];
 #pragma unroll
-        for (int a = 0; a < 4; ++a) {
-          const int qoff = 32 * qt + 8 * a + 4 * lh;
-          const float4 l4 = *reinterpret_cast<const float4*>(base + 2 * TILE + qoff * 4);
-          const float4 d4 = *reinterpret_cast<const float4*>(base + 2 * TILE + FB_BQT * 4 + qoff * 4);
-          const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
-          float pr[4], ds[4];
+          for (int a = 0; a < 4; ++a) {
+            const int qoff = 32 * qt + 8 * a + 4 * lh;
+            const float4 l4 = *reinterpret_cast<const float4*>(base + 2 * TILE + qoff * 4);
+            const float4 d4 = *reinterpret_cast<const float4*>(base + 2 * TILE + FB_BQT * 4 + qoff * 4);
+            const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
+            float pr[4], ds[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int q = qt0 + qoff + e;
-            const bool ok = (q < p.Sq) & (key < p.Sk) & (!p.causal | (key <= q + off));
-            // masked pairs get exponent -inf (P = 0) by a select on the argument
-            pr[e] = fast_exp2(ok ? fmaf(s[qt][4 * a + e], c, -lv[e]) : -INFINITY);
-            ds[e] = pr[e] * (dp[qt][4 * a + e] - dl[e]);
+            for (int e = 0; e < 4; ++e) {
+              float x = fmaf(s[qt][4 * a + e], c, -lv[e]);
+              if constexpr (MASKED) {
+                const int q = qt0 + qoff + e;
+                const bool ok = (q < p.Sq) & (key < p.Sk) & (!p.causal | (key <= q + off));
+                x = ok ? x : -INFINITY;                  // exponent -inf: P = 0, no branch
+              }
+              pr[e] = fast_exp2(x);
+              ds[e] = pr[e] * (dp[qt][4 * a + e] - dl[e]);
+            }
+            pw[2 * a] = pack2<T>(pr[0], pr[1]);
+            pw[2 * a + 1] = pack2<T>(pr[2], pr[3]);
+            dw[2 * a] = pack2<T>(ds[0], ds[1]);
+            dw[2 * a + 1] = pack2<T>(ds[2], ds[3]);
           }
-          pw[2 * a] = pack2<T>(pr[0], pr[1]);
-          pw[2 * a + 1] = pack2<T>(pr[2], pr[3]);
-          dw[2 * a] = pack2<T>(ds[0], ds[1]);
-          dw[2 * a + 1] = pack2<T>(ds[2], ds[3]);
+          pf[qt][0] = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+          pf[qt][1] = make_uint4(pw[4], pw[5], pw[6], pw[7]);
+          dsf[qt][0] = make_uint4(dw[0], dw[1], dw[2], dw[3]);
+          dsf[qt][1] = make_uint4(dw[4], dw[5], dw[6], dw[7]);
         }
-        pf[qt][0] = make_uint4(pw[0], pw[1], pw[2], pw[3]);
-        pf[qt][1] = make_uint4(pw[4], pw[5], pw[6], pw[7]);
-        dsf[qt][0] = make_uint4(dw[0], dw[1], dw[2], dw[3]);
-        dsf[qt][1] = make_uint4(dw[4], dw[5], dw[6], dw[7]);
-      }
+      };
+      const bool need_mask = (qt0 + FB_BQT > p.Sq) || (wave_k0 + 32 > p.Sk) ||
+                             (p.causal && wave_k0 + 31 > qt0 + off);
+      if (need_mask) softmax_part(std::true_type{});
+      else softmax_part(std::false_type{});
       // second products, their transposed operands read one step ahead
       constexpr int NSTEP = 4 * DT;                        // (qt, g, dt) steps
       auto tr_frags = [&](int i, uint4& qT, uint4& oT) {

@@ -72,26 +72,13 @@ struct Gemm16Params {
   int tiles_m, tiles_n;   // tile grid (grouped: tiles_m is an upper bound)
 };
 
-#ifndef TSR_NO_SGB
-#define TSR_SGB(mask, n, id) __builtin_amdgcn_sched_group_barrier(mask, n, id)
-#else
-#define TSR_SGB(mask, n, id)
-#endif
-#ifndef TSR_NO_SB
-#define TSR_SB() __builtin_amdgcn_sched_barrier(0)
-#else
-#define TSR_SB()
-#endif
 
 constexpr int G16_BK = 64;          // K step, elements
 constexpr int G16_APITCH = 128;     // bytes per A row in LDS
-#ifndef TSR_BPAD
-#define TSR_BPAD 32
-#endif
-#ifndef TSR_ASWZ
-#define TSR_ASWZ(row) (((row) >> 1) & 7)
-#endif
-constexpr int G16_BPAD = TSR_BPAD;  // B row pad, elements
+constexpr int G16_BPAD = 32;        // B row pad, elements
+// A-tile chunk swizzle: 16 consecutive rows of one chunk column hit 16 different
+// 16-byte slots of the 256-byte bank line.
+__device__ __forceinline__ int g16_aswz(int row) { return (row >> 1) & 7; }
 
 template <int BM, int BN>
 struct Gemm16Smem {
@@ -207,7 +194,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     int gr = row;
     gr = m_begin + gr < m_end ? gr : m_end - 1 - m_begin;   // clamp: rows past the edge are never stored
     a_off[q] = ((uint32_t)gr * (uint32_t)p.lda + a_chunk * 8) * 2;
-    a_lds[q] = row * G16_APITCH + ((a_chunk ^ TSR_ASWZ(row)) << 4);
+    a_lds[q] = row * G16_APITCH + ((a_chunk ^ g16_aswz(row)) << 4);
   }
   // B: the tile's columns come from one matrix, or (SwiGLU) half from the gate and
   // half from the up matrix; the first B_CHUNKS / HALVES chunks of a thread belong to
@@ -288,7 +275,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   for (int i = 0; i < MI; ++i) {
     const int row = wm * TM + i * 32 + l32;
     a_rd[i] = row * G16_APITCH;
-    a_sw[i] = TSR_ASWZ(row);
+    a_sw[i] = g16_aswz(row);
   }
   // transposing read: lane supplies row (k) = 8*lh + r/4 (+4 for the second
   // half), columns n = 32j + 16*((lane>>4)&1) + 4*(r%4), r = lane & 15.
@@ -343,12 +330,12 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
       constexpr int wper = (CPG + WSLOTS - 1) / WSLOTS;
 #pragma unroll
       for (int x = 0; x < NM; ++x) {
-        TSR_SGB(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         if (x < rslots) {
-          TSR_SGB(0x100, rper, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, rper, 0);
         } else {
-          TSR_SGB(0x200, wper, 0);
-          if constexpr (LOADS) TSR_SGB(0x020, wper, 0);
+          __builtin_amdgcn_sched_group_barrier(0x200, wper, 0);
+          if constexpr (LOADS) __builtin_amdgcn_sched_group_barrier(0x020, wper, 0);
         }
       }
     }
@@ -389,7 +376,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
       if constexpr (HAS1) stream_group(ks + 1, buf ^ 1, (kt + 2) * G16_BK, l2_c);
       mma(ks & 1);
       hint_step(std::integral_constant<bool, HAS1>{}, std::integral_constant<bool, (L2 != 0)>{});
-      TSR_SB();
+      __builtin_amdgcn_sched_barrier(0);
     }
     // Every wave has issued all its reads of this buffer and all its writes of
     // the other one; past the barrier the other buffer is complete and this one
@@ -399,7 +386,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     if constexpr (L2 != 0) stream_group(0, buf, (kt + 3) * G16_BK, l3_c);
     mma((KS - 1) & 1);
     if constexpr (HAS1) hint_step(std::integral_constant<bool, (L2 != 0)>{}, std::integral_constant<bool, (L3 != 0)>{});
-    TSR_SB();
+    __builtin_amdgcn_sched_barrier(0);
   };
   int kt = 0;
   for (; kt + 4 < ktiles; ++kt) kstep(kt, true_type{}, mode1{}, mode1{});
