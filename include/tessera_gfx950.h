@@ -201,6 +201,28 @@ int tessera_gfx950_flash_attn_gqa_bf16_dev(const void* Q, const void* K, const v
                                            int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
                                            int causal, int out_dtype, void* stream);
 
+/* Sliding window and logit soft cap, the kwargs `window` / `logit_softcap` of the
+ * reference's attention executor (python/tessera/runtime.py:7318-7335) with the
+ * bounds and score transform of its CPU kernel (avx512_flash_attn_f32.cpp:115-196):
+ * window > 0 keeps, per query row i, the `window` keys ending at the causal diagonal
+ * i + max(Sk - Sq, 0) (causal != 0) or window/2 keys either side of it (causal == 0);
+ * softcap > 0 passes each scaled score through cap * tanh(s / cap) before the
+ * softmax.  0 disables either.  A row with no visible key gives O = 0, LSE = -inf. */
+int tessera_gfx950_flash_attn_ext_f16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                      int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                                      int causal, int window, float softcap);
+int tessera_gfx950_flash_attn_ext_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                       int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                                       int causal, int window, float softcap);
+int tessera_gfx950_flash_attn_ext_f16_dev(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                          int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                                          int causal, int window, float softcap, int out_dtype,
+                                          void* stream);
+int tessera_gfx950_flash_attn_ext_bf16_dev(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                           int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                                           int causal, int window, float softcap, int out_dtype,
+                                           void* stream);
+
 /* ---- flash-attention backward -------------------------------------------- */
 
 /* (dQ, dK, dV) of O = softmax(scale Q K^T, causal) V given dO: the contract of the

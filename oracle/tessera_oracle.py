@@ -188,8 +188,26 @@ def _causal_limit(sq: int, sk: int) -> int:
     return max(sk - sq, 0)
 
 
-def flash_attn_dense(Q, K, V, scale=None, causal=False, dtype=np.float64):
-    """Dense ``softmax(scale*Q K^T, causal) V`` with GQA and LSE.
+def key_bounds(i: int, sq: int, sk: int, causal: bool, window: int = 0):
+    """First and last visible key of query row ``i`` — ``attention_bounds``
+    (``avx512_flash_attn_f32.cpp:180-196``): the causal diagonal is bottom-right
+    aligned; a window keeps ``window`` keys ending at the diagonal (causal) or
+    ``window // 2`` keys either side of it."""
+    off = _causal_limit(sq, sk)
+    lo, hi = 0, (i + off if causal else sk - 1)
+    if window > 0:
+        if causal:
+            lo, hi = i + off - window + 1, i + off
+        else:
+            lo, hi = i + off - window // 2, i + off + window // 2
+    return max(lo, 0), min(hi, sk - 1)
+
+
+def flash_attn_dense(Q, K, V, scale=None, causal=False, dtype=np.float64, window: int = 0,
+                     softcap: float = 0.0):
+    """Dense ``softmax(scale*Q K^T, causal) V`` with GQA and LSE; optional sliding
+    ``window`` (see :func:`key_bounds`) and logit soft cap (scaled scores pass
+    through ``cap * tanh(s / cap)``, ``avx512_flash_attn_f32.cpp:115,161``).
 
     Q ``[B,Hq,Sq,D]``; K, V ``[B,Hkv,Sk,D]``.  kv head of q head ``h`` is
     ``h * Hkv // Hq`` (``avx512_flash_attn_f32.cpp:386``), which equals
@@ -213,10 +231,12 @@ def flash_attn_dense(Q, K, V, scale=None, causal=False, dtype=np.float64):
         for h in range(Hq):
             kh = h * Hkv // Hq
             s = (Q[b, h] @ K[b, kh].T) * dtype(scale)
-            if causal:
-                i = np.arange(Sq)[:, None]
+            if softcap > 0:
+                s = dtype(softcap) * np.tanh(s / dtype(softcap))
+            if causal or window > 0:
+                bounds = np.array([key_bounds(i, Sq, Sk, causal, window) for i in range(Sq)])
                 j = np.arange(Sk)[None, :]
-                s = np.where(j > i + off, -np.inf, s)
+                s = np.where((j < bounds[:, :1]) | (j > bounds[:, 1:]), -np.inf, s)
             m = s.max(axis=-1, keepdims=True)
             msafe = np.where(np.isfinite(m), m, 0.0)
             e = np.exp(s - msafe)

@@ -15,10 +15,10 @@ bool bad_attn(int B, int Hq, int Hkv, int Sq, int Sk, int D) {
   return false;
 }
 
-template <class T, int D>
+template <class T, int D, bool SOFTCAP>
 int launch_flash(const FlashParams& p, hipStream_t s) {
   constexpr int kSmem = 2 * 2 * FA_BKV * D * 2;
-  auto kern = flash_fwd_kernel<T, D>;
+  auto kern = flash_fwd_kernel<T, D, SOFTCAP>;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [&] {
@@ -33,8 +33,10 @@ int launch_flash(const FlashParams& p, hipStream_t s) {
 
 template <class T>
 int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, int B, int Hq, int Hkv,
-              int Sq, int Sk, int D, float scale, int causal, int out_storage, hipStream_t s) {
+              int Sq, int Sk, int D, float scale, int causal, int out_storage, hipStream_t s, int window = 0,
+              float softcap = 0.f) {
   if (bad_attn(B, Hq, Hkv, Sq, Sk, D) || !Q || !K || !V || !O) return kBadShape;
+  if (window < 0 || !(softcap >= 0.f)) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
   FlashParams p{};
   p.Q = static_cast<const uint16_t*>(Q);
@@ -46,10 +48,12 @@ int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, i
   p.scale = scale;
   p.causal = causal ? 1 : 0;
   p.out_storage = out_storage ? 1 : 0;
+  p.window = window;
+  p.softcap = softcap;
   const bool al = ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
                     reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(O)) & 15) == 0;
-  if (al && D == 128) return launch_flash<T, 128>(p, s);
-  if (al && D == 64) return launch_flash<T, 64>(p, s);
+  if (al && D == 128) return p.softcap > 0.f ? launch_flash<T, 128, true>(p, s) : launch_flash<T, 128, false>(p, s);
+  if (al && D == 64) return p.softcap > 0.f ? launch_flash<T, 64, true>(p, s) : launch_flash<T, 64, false>(p, s);
   const long rows = (long)B * Hq * Sq;
   hipLaunchKernelGGL((flash_fwd_generic_kernel<T>), dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, p, D);
   return launch_status();
@@ -57,8 +61,9 @@ int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, i
 
 template <class T>
 int flash_host(const void* Q, const void* K, const void* V, void* O, void* LSE, int B, int Hq, int Hkv,
-               int Sq, int Sk, int D, float scale, int causal) {
+               int Sq, int Sk, int D, float scale, int causal, int window = 0, float softcap = 0.f) {
   if (bad_attn(B, Hq, Hkv, Sq, Sk, D) || !Q || !K || !V || !O) return kBadShape;
+  if (window < 0 || !(softcap >= 0.f)) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
   const size_t q_bytes = (size_t)B * Hq * Sq * D * 2, kv_bytes = (size_t)B * Hkv * Sk * D * 2;
   const size_t o_bytes = (size_t)B * Hq * Sq * D * 4, l_bytes = (size_t)B * Hq * Sq * 4;
@@ -69,7 +74,7 @@ int flash_host(const void* Q, const void* K, const void* V, void* O, void* LSE, 
   void* dO = scope.alloc(o_bytes);
   void* dL = LSE ? scope.alloc(l_bytes) : nullptr;
   if (scope.failed()) return kDeviceFailed;
-  int rc = flash_dev<T>(dQ, dK, dV, dO, dL, B, Hq, Hkv, Sq, Sk, D, scale, causal, 0, nullptr);
+  int rc = flash_dev<T>(dQ, dK, dV, dO, dL, B, Hq, Hkv, Sq, Sk, D, scale, causal, 0, nullptr, window, softcap);
   if (rc != kOk) return rc;
   if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
   if (!scope.download(O, dO, o_bytes)) return kDeviceFailed;
@@ -216,6 +221,29 @@ int tessera_gfx950_flash_attn_gqa_bf16_dev(const void* Q, const void* K, const v
                                            int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
                                            int causal, int out_dtype, void* stream) {
   return flash_dev<BF16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, out_dtype, as_stream(stream));
+}
+
+int tessera_gfx950_flash_attn_ext_f16(const void* Q, const void* K, const void* V, void* O, void* LSE, int B,
+                                      int Hq, int Hkv, int Sq, int Sk, int D, float scale, int causal, int window,
+                                      float softcap) {
+  return flash_host<F16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, window, softcap);
+}
+int tessera_gfx950_flash_attn_ext_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE, int B,
+                                       int Hq, int Hkv, int Sq, int Sk, int D, float scale, int causal, int window,
+                                       float softcap) {
+  return flash_host<BF16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, window, softcap);
+}
+int tessera_gfx950_flash_attn_ext_f16_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, int B,
+                                          int Hq, int Hkv, int Sq, int Sk, int D, float scale, int causal,
+                                          int window, float softcap, int out_dtype, void* stream) {
+  return flash_dev<F16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, out_dtype, as_stream(stream), window,
+                        softcap);
+}
+int tessera_gfx950_flash_attn_ext_bf16_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, int B,
+                                           int Hq, int Hkv, int Sq, int Sk, int D, float scale, int causal,
+                                           int window, float softcap, int out_dtype, void* stream) {
+  return flash_dev<BF16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, out_dtype, as_stream(stream), window,
+                         softcap);
 }
 
 int tessera_gfx950_flash_attn_bwd_f16(const void* dO, const void* Q, const void* K, const void* V, void* dQ,

@@ -45,7 +45,25 @@ struct FlashParams {
   float scale;
   int causal;
   int out_storage;     // 0: f32 O, 1: O in the storage dtype
+  int window;          // > 0: band of keys per query (see key_bounds); 0: none
+  float softcap;       // > 0: scaled scores pass through cap * tanh(s / cap); 0: none
 };
+
+// Visible keys [lo, hi] of query row i — the reference's attention_bounds
+// (avx512_flash_attn_f32.cpp:180-196): causal masks keys past the bottom-right
+// aligned diagonal; a window keeps the `window` keys ending at the diagonal (causal)
+// or window/2 keys either side of it.
+__host__ __device__ inline void key_bounds(int i, int Sq, int Sk, int causal, int window, int& lo, int& hi) {
+  const int off = Sk > Sq ? Sk - Sq : 0;
+  lo = 0;
+  hi = causal ? i + off : Sk - 1;
+  if (window > 0) {
+    if (causal) { lo = i + off - window + 1; hi = i + off; }
+    else { lo = i + off - window / 2; hi = i + off + window / 2; }
+  }
+  lo = lo > 0 ? lo : 0;
+  hi = hi < Sk - 1 ? hi : Sk - 1;
+}
 
 constexpr int FA_BQ = 256;             // query rows per workgroup
 constexpr int FA_QT = 1;               // 32-row query tiles per wave
@@ -93,8 +111,8 @@ __device__ __forceinline__ float scale_acc(float acc, float corr) {
   return acc;
 }
 
-template <class T, int D>
-__global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel(const FlashParams p) {
+template <class T, int D, bool SOFTCAP>
+__global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashParams p) {
   constexpr int QT = FA_QT;
   constexpr int KSTEPS = D / 16;         // MFMA k steps of the score product
   constexpr int KA = (KSTEPS + 3) / 4;   // score k steps issued under the row-max phase
@@ -149,19 +167,23 @@ __global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel
   const uint16_t* Kb = p.K + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
   const uint16_t* Vb = p.V + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
 
-  // Keys this workgroup needs: all of them, or up to the diagonal of its last row.
-  int kv_end = p.Sk;
-  if (p.causal) {
-    const int last_q = min(q0 + FA_BQ, p.Sq) - 1;
-    kv_end = min(p.Sk, last_q + off + 1);
-  }
-  const int ntiles = (kv_end + FA_BKV - 1) / FA_BKV;
-  // Tiles this wave computes on: those below its own diagonal.
-  int nt_w = 0;
+  // Key tiles this workgroup needs: from the first visible key of its first row to
+  // the last visible key of its last row (bounds are monotone in the row index).
+  // `t` below counts tiles from tile_base.
+  int lo_first, hi_first, lo_last, hi_last;
+  key_bounds(q0, p.Sq, p.Sk, p.causal, p.window, lo_first, hi_first);
+  key_bounds(min(q0 + FA_BQ, p.Sq) - 1, p.Sq, p.Sk, p.causal, p.window, lo_last, hi_last);
+  const int tile_base = lo_first / FA_BKV;
+  const int ntiles = max((hi_last + FA_BKV) / FA_BKV - tile_base, 0);
+  // Tiles this wave computes on: from (an even number of tiles before) its first
+  // row's first key to its last row's last key.
+  int nt_w = 0, t_w0 = 0;
+  int wlo_first = 0, whi_first = 0, wlo_last = 0, whi_last = 0;   // bounds of the wave's first / last row
   if (qw < p.Sq) {
-    int wave_kv_end = kv_end;
-    if (p.causal) wave_kv_end = min(kv_end, min(qw + 32 * QT, p.Sq) - 1 + off + 1);
-    nt_w = (wave_kv_end + FA_BKV - 1) / FA_BKV;
+    key_bounds(qw, p.Sq, p.Sk, p.causal, p.window, wlo_first, whi_first);
+    key_bounds(min(qw + 32 * QT, p.Sq) - 1, p.Sq, p.Sk, p.causal, p.window, wlo_last, whi_last);
+    nt_w = min(max((whi_last + FA_BKV) / FA_BKV - tile_base, 0), ntiles);
+    t_w0 = min(max(wlo_first / FA_BKV - tile_base, 0) & ~1, nt_w);
   }
 
   // ---- Q fragments: lane (q = l32, h) holds Q[q][16 ks + 8 h .. +7] -----------
@@ -221,12 +243,20 @@ __global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel
       for (int r = 0; r < 16; ++r) o_acc[qt][dt][r] = 0.f;
   }
   const float c = p.scale * 1.44269504088896340736f;   // scale * log2(e)
-  int lim[QT];                           // last visible key of this lane's query rows
+  int klo[QT], khi[QT];                  // visible keys of this lane's query rows
 #pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    const int qi = qw + 32 * qt + l32;
-    lim[qt] = p.causal ? min(qi + off, p.Sk - 1) : p.Sk - 1;
-  }
+  for (int qt = 0; qt < QT; ++qt) key_bounds(qw + 32 * qt + l32, p.Sq, p.Sk, p.causal, p.window, klo[qt], khi[qt]);
+  // Exponent argument of a raw score, in base 2: scale * log2(e) * s, or with a
+  // soft cap  cap * log2(e) * tanh(scale * s / cap)  (tanh y = 1 - 2 / (e^{2y} + 1)).
+  const float cap2 = p.softcap * 1.44269504088896340736f;
+  const float incap = SOFTCAP ? 2.0f * 1.44269504088896340736f * p.scale / p.softcap : 0.f;
+  // With a soft cap the score tiles are transformed in place (before masking) and
+  // already are exponent arguments; without one the raw scores are kept and the
+  // factor cs = scale * log2(e) is folded into the exponential's FMA.
+  const float cs = SOFTCAP ? 1.0f : c;
+  auto capped = [&](float sraw) -> float {
+    return cap2 * (1.0f - 2.0f * __builtin_amdgcn_rcpf(fast_exp2(sraw * incap) + 1.0f));
+  };
 
   // ---- per-lane LDS read addresses (stage and tile-row offsets are immediates) ----
   // K operand: row l32 (+32 kt), logical chunk 2 ks + lh.
@@ -269,7 +299,7 @@ __global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel
   auto exp_group = [&](f32x16& sv, int g, float mc, float& sum) -> uint4 {
 #pragma unroll
     for (int r = 8 * g; r < 8 * g + 8; ++r) {
-      const float e = fast_exp2(fmaf(sv[r], c, -mc));
+      const float e = fast_exp2(fmaf(sv[r], cs, -mc));
       sv[r] = e;
       sum += e;
     }
@@ -289,11 +319,19 @@ __global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel
   auto step = [&](auto has_next_c, auto par_c, f32x16 (&sc)[QT][FA_KT], f32x16 (&sn)[QT][FA_KT], int t) {
     constexpr bool HAS_NEXT = decltype(has_next_c)::value;
     constexpr int PAR = decltype(par_c)::value;        // t & 1
-    if (t + 2 < ntiles) load_k(t + 2, PAR);
-    if (t + 1 < ntiles) load_v(t + 1, PAR ^ 1);
-    const int kv0 = t * FA_BKV;
-    // mask (only tiles that touch the diagonal or the end of K)
-    const bool need_mask = (kv0 + FA_BKV > p.Sk) || (p.causal && (kv0 + FA_BKV - 1 > qw + off));
+    if (t + 2 < ntiles) load_k(tile_base + t + 2, PAR);
+    if (t + 1 < ntiles) load_v(tile_base + t + 1, PAR ^ 1);
+    const int kv0 = (tile_base + t) * FA_BKV;
+    if constexpr (SOFTCAP) {
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+        for (int kt = 0; kt < FA_KT; ++kt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sc[qt][kt][r] = capped(sc[qt][kt][r]);
+    }
+    // mask (only tiles that cross a bound of one of the wave's rows)
+    const bool need_mask = (kv0 + FA_BKV - 1 > whi_first) || (kv0 < wlo_last);
     if (need_mask) {
 #pragma unroll
       for (int qt = 0; qt < QT; ++qt)
@@ -302,7 +340,7 @@ __global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int key = kv0 + kt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-            if (key > lim[qt]) sc[qt][kt][r] = FA_NEG;
+            if (key > khi[qt] || key < klo[qt]) sc[qt][kt][r] = FA_NEG;
           }
     }
     if constexpr (HAS_NEXT) score_steps(sn, PAR ^ 1, 0, KA);
@@ -325,7 +363,7 @@ __global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel
     if (__any(grow)) {
 #pragma unroll
       for (int qt = 0; qt < QT; ++qt) {
-        const float corr = fast_exp2((m_run[qt] - m_new[qt]) * c);
+        const float corr = fast_exp2((m_run[qt] - m_new[qt]) * cs);
         l_run[qt] *= corr;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -339,7 +377,9 @@ __global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel
       if constexpr (QT > 1) asm volatile("s_nop 4");   // accumulator writes settle before the next MFMA
     }
 #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) mc[qt] = m_new[qt] * c;
+    // (a row that has met no visible key yet keeps the sentinel maximum: give it the
+    // reference 0 so its masked entries underflow to P = 0 instead of cancelling)
+    for (int qt = 0; qt < QT; ++qt) mc[qt] = m_new[qt] > 0.5f * FA_NEG ? m_new[qt] * cs : 0.f;
 
     // Units of 8 keys x one query tile, in consumption order: i -> (kt, g, qt).
     constexpr int NU = 2 * FA_KT * QT;
@@ -390,10 +430,10 @@ __global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel
 
   // ---- prologue: K(0), V(0), K(1) resident; scores of tile 0 ----------------------
   if (ntiles > 0) {
-    load_k(0, 0);
-    load_v(0, 0);
+    load_k(tile_base, 0);
+    load_v(tile_base, 0);
   }
-  if (ntiles > 1) load_k(1, 1);
+  if (ntiles > 1) load_k(tile_base + 1, 1);
   fa_wait_loads();
   __syncthreads();
   f32x16 sA[QT][FA_KT], sB[QT][FA_KT];
@@ -403,9 +443,26 @@ __global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel
     for (int kt = 0; kt < FA_KT; ++kt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) { sA[qt][kt][r] = 0.f; sB[qt][kt][r] = 0.f; }
-  if (nt_w > 0) score_steps(sA, 0, 0, KSTEPS);
-
+  // Tiles before the wave's first key (a sliding window): keep the loads going.
+  auto idle_step = [&](int t) {
+    if (t + 2 < ntiles) load_k(tile_base + t + 2, t & 1);
+    if (t + 1 < ntiles) load_v(tile_base + t + 1, (t & 1) ^ 1);
+    fa_wait_loads();
+    __syncthreads();
+  };
+  // A wave that starts late computes the scores of its first tile (t_w0, even, so its
+  // K tile sits in stage 0) inside the idle step before it: from step t_w0 on the
+  // other waves already refill that stage.
   int t = 0;
+  if (t_w0 == 0 && nt_w > 0) score_steps(sA, 0, 0, KSTEPS);
+  for (; t < t_w0; ++t) {
+    if (t + 2 < ntiles) load_k(tile_base + t + 2, t & 1);
+    if (t + 1 < ntiles) load_v(tile_base + t + 1, (t & 1) ^ 1);
+    if (t + 1 == t_w0 && nt_w > t_w0) score_steps(sA, 0, 0, KSTEPS);
+    fa_wait_loads();
+    __syncthreads();
+  }
+
   for (; t + 2 < nt_w; t += 2) {
     step(true_type{}, P0{}, sA, sB, t);
     step(true_type{}, P1{}, sB, sA, t + 1);
@@ -419,23 +476,19 @@ __global__ __launch_bounds__(FA_THREADS, 512 / FA_THREADS) void flash_fwd_kernel
     t += 1;
   }
   // Waves past their diagonal keep feeding the loads the others depend on.
-  for (; t < ntiles; ++t) {
-    if (t + 2 < ntiles) load_k(t + 2, t & 1);
-    if (t + 1 < ntiles) load_v(t + 1, (t & 1) ^ 1);
-    fa_wait_loads();
-    __syncthreads();
-  }
+  for (; t < ntiles; ++t) idle_step(t);
 
   // ---- epilogue -------------------------------------------------------------------
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     const int qi = qw + 32 * qt + l32;
-    const float l = l_run[qt] + swap_half(l_run[qt]);
+    float l = l_run[qt] + swap_half(l_run[qt]);
     if (qi >= p.Sq) continue;
+    if (khi[qt] < klo[qt]) l = 0.f;                      // no visible key: O = 0, LSE = -inf
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     const long row = (long)(b * p.Hq + hq) * p.Sq + qi;
     if (p.LSE && lh == 0)
-      p.LSE[row] = l > 0.f ? (m_run[qt] * c + __log2f(l)) * 0.69314718055994530942f : -INFINITY;
+      p.LSE[row] = l > 0.f ? (m_run[qt] * cs + __log2f(l)) * 0.69314718055994530942f : -INFINITY;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -473,11 +526,14 @@ __global__ void flash_fwd_generic_kernel(const FlashParams p, int D) {
   float acc[256];
   for (int d = 0; d < D; ++d) acc[d] = 0.f;
   float m = -INFINITY, l = 0.f;
-  const int jmax = p.causal ? min(qi + off, p.Sk - 1) : p.Sk - 1;
-  for (int j = 0; j <= jmax; ++j) {
+  int jmin, jmax;
+  key_bounds(qi, p.Sq, p.Sk, p.causal, p.window, jmin, jmax);
+  (void)off;
+  for (int j = jmin; j <= jmax; ++j) {
     float s = 0.f;
     for (int d = 0; d < D; ++d) s += from_storage<T>(q[d]) * from_storage<T>(Kb[(long)j * D + d]);
     s *= p.scale;
+    if (p.softcap > 0.f) s = p.softcap * tanhf(s / p.softcap);
     const float mn = fmaxf(m, s);
     const float cr = __expf(m - mn);       // exp(-inf) = 0 on the first key
     const float e = __expf(s - mn);

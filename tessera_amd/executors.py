@@ -189,12 +189,15 @@ def execute_gfx950_gemm(artifact: RuntimeArtifact, args: Any):
     return _ops.fused_gemm(a, b, bias, activation)
 
 
-_FA_OPS = ("tessera.flash_attn", "tessera.multi_head_attention", "tessera.gqa_attention", "tessera.mqa_attention")
+_FA_OPS = ("tessera.flash_attn", "tessera.multi_head_attention", "tessera.gqa_attention", "tessera.mqa_attention",
+           "tessera.attn_sliding_window")
 
 
 def execute_gfx950_flash_attn(artifact: RuntimeArtifact, args: Any):
     """Attention forward: Q ``[..., Hq, Sq, D]``, K/V ``[..., Hkv, Sk, D]`` in
-    f16/bf16 -> f32 O shaped like Q.  ``kwargs``: ``causal``, ``scale``."""
+    f16/bf16 -> f32 O shaped like Q.  ``kwargs``: ``causal``, ``scale``, ``window``
+    (a positive width; required by ``tessera.attn_sliding_window``) and
+    ``logit_softcap`` (``runtime.py:7312-7340``)."""
     md = artifact.metadata or {}
     op = _single_op(artifact, _FA_OPS, "gfx950_flash_attn")
     names = [str(n) for n in op.get("operands", [])]
@@ -205,10 +208,21 @@ def execute_gfx950_flash_attn(artifact: RuntimeArtifact, args: Any):
     values = _bind_launch_args(args, list(md.get("arg_names") or []))
     q, k, v = (_as_array(values[n]) for n in names[:3])
     kwargs = op.get("kwargs") or {}
-    for unsupported in ("window", "logit_softcap", "dropout_p"):
-        if kwargs.get(unsupported):
-            raise ValueError(f"gfx950 flash_attn lane does not implement `{unsupported}`")
-    return _ops.gqa_attention(q, k, v, scale=kwargs.get("scale"), causal=bool(kwargs.get("causal", False)), out="f32")
+    if kwargs.get("dropout_p"):
+        raise ValueError("gfx950 flash_attn lane does not implement `dropout_p`")
+    window = int(kwargs.get("window") or 0)
+    if window < 0:
+        raise ValueError(f"gfx950 flash_attn window must be a non-negative width; got {window}")
+    if str(op.get("op_name")) == "tessera.attn_sliding_window" and window <= 0:
+        raise ValueError(f"tessera.attn_sliding_window requires a positive `window` width kwarg; got {window}")
+    softcap = kwargs.get("logit_softcap")
+    softcap = float(softcap) if softcap else 0.0
+    if softcap < 0:
+        raise ValueError(f"gfx950 flash_attn logit_softcap must be non-negative; got {softcap}")
+    # the windowed kernel of the reference is implicitly causal (runtime.py:7318-7321)
+    causal = bool(kwargs.get("causal", False)) or window > 0
+    return _ops.gqa_attention(q, k, v, scale=kwargs.get("scale"), causal=causal, out="f32", window=window,
+                              logit_softcap=softcap)
 
 
 _FA_BWD_OPS = ("tessera.flash_attn_bwd", "tessera.flash_attn_vjp")

@@ -208,7 +208,7 @@ def gemm_i8(A, B) -> np.ndarray:
 # ---------------------------------------------------------------------------
 
 
-def _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa):
+def _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa, window=0, logit_softcap=0.0):
     Q, K, V = _unbox(Q), _unbox(K), _unbox(V)
     st = _storage(Q, K)
     if _storage(V) != st:
@@ -235,11 +235,22 @@ def _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa):
             raise ValueError(f"GQA needs query-heads ({Hq}) divisible by kv-heads ({Hkv})")
     if scale is None:
         scale = 1.0 / math.sqrt(D)
+    window = int(window or 0)
+    softcap = float(logit_softcap or 0.0)
+    if window < 0:
+        raise ValueError(f"flash_attn window must be a non-negative width; got {window}")
+    if softcap < 0:
+        raise ValueError(f"flash_attn logit_softcap must be non-negative; got {softcap}")
     o = np.empty(q.shape, np.float32)
     lse = np.empty(q.shape[:-1], np.float32) if return_lse else None
-    fn = getattr(_lane.load(), f"tessera_gfx950_flash_attn_gqa_{st}")
-    rc = fn(q.ctypes.data, k.ctypes.data, v.ctypes.data, o.ctypes.data, _lane.ptr(lse),
-            Bq, Hq, Hkv, Sq, Sk, D, float(scale), 1 if causal else 0)
+    if window or softcap:
+        fn = getattr(_lane.load(), f"tessera_gfx950_flash_attn_ext_{st}")
+        rc = fn(q.ctypes.data, k.ctypes.data, v.ctypes.data, o.ctypes.data, _lane.ptr(lse),
+                Bq, Hq, Hkv, Sq, Sk, D, float(scale), 1 if causal else 0, window, softcap)
+    else:
+        fn = getattr(_lane.load(), f"tessera_gfx950_flash_attn_gqa_{st}")
+        rc = fn(q.ctypes.data, k.ctypes.data, v.ctypes.data, o.ctypes.data, _lane.ptr(lse),
+                Bq, Hq, Hkv, Sq, Sk, D, float(scale), 1 if causal else 0)
     _lane.check(rc, "flash_attn")
     if out == "storage":
         o = _bf16.from_float32(o) if st == "bf16" else o.astype(np.float16)
@@ -287,18 +298,18 @@ def flash_attn_backward(dO, Q, K, V, scale=None, causal: bool = False):
 
 
 def flash_attn(Q, K=None, V=None, scale=None, causal: bool = False, *, return_lse: bool = False,
-               out: str = "storage"):
+               out: str = "storage", window: int = 0, logit_softcap: float = 0.0):
     """``softmax(scale * Q K^T, causal) V``.  Q/K/V ``[..., H, S, D]`` 16-bit; the
     causal mask is bottom-right aligned (key ``j`` visible to query ``i`` iff
     ``j <= i + max(Sk - Sq, 0)``).  Head counts must match (as in the reference)."""
-    return _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa=False)
+    return _attention(Q, K, V, scale, causal, return_lse, out, False, window, logit_softcap)
 
 
 def gqa_attention(Q, K, V, scale=None, causal: bool = False, *, return_lse: bool = False,
-                  out: str = "storage"):
+                  out: str = "storage", window: int = 0, logit_softcap: float = 0.0):
     """Grouped-query attention: kv head of query head ``h`` is ``h // (Hq / Hkv)``
     — identical to repeating K/V along the head axis."""
-    return _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa=True)
+    return _attention(Q, K, V, scale, causal, return_lse, out, True, window, logit_softcap)
 
 
 # ---------------------------------------------------------------------------

@@ -37,19 +37,24 @@ def main() -> int:
     out["gemm_i8_c"] = co.ref_gemm_u8s8(au, bs)
     # flash attention with LSE and GQA: tessera_x86_flash_attn_ext_lse_f32
     # (avx512_flash_attn_f32.cpp:379-422); causal with Sk > Sq (bottom-right aligned)
-    for tag, (B, Hq, Hkv, Sq, Sk, D, causal) in {
-        "fa_causal_gqa": (2, 4, 2, 48, 48, 32, True),
-        "fa_causal_offset": (1, 2, 1, 20, 52, 16, True),
-        "fa_full": (1, 3, 3, 33, 40, 64, False),
+    for tag, (B, Hq, Hkv, Sq, Sk, D, causal, window, cap) in {
+        "fa_causal_gqa": (2, 4, 2, 48, 48, 32, True, 0, 0.0),
+        "fa_causal_offset": (1, 2, 1, 20, 52, 16, True, 0, 0.0),
+        "fa_full": (1, 3, 3, 33, 40, 64, False, 0, 0.0),
+        "fa_window_causal": (1, 2, 1, 70, 90, 32, True, 24, 0.0),      # sliding window, Sk > Sq
+        "fa_window_centered": (1, 2, 2, 50, 50, 16, False, 14, 0.0),    # non-causal band
+        "fa_softcap": (1, 2, 2, 40, 40, 64, True, 0, 4.0),               # logit soft cap
     }.items():
         q = rng.standard_normal((B, Hq, Sq, D), dtype=np.float32)
         k = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32)
         v = rng.standard_normal((B, Hkv, Sk, D), dtype=np.float32)
         q, k, v = (orc.bf16_bits_to_f32(orc.f32_to_bf16_bits(t)).reshape(t.shape) for t in (q, k, v))
-        o, lse = co.ref_flash_attn_lse(q, k, v, 1.0 / np.sqrt(D), causal)
+        o, lse = co.ref_flash_attn_lse(q, k, v, 1.0 / np.sqrt(D), causal, window, cap)
         out[f"{tag}_q"], out[f"{tag}_k"], out[f"{tag}_v"] = q, k, v
         out[f"{tag}_o"], out[f"{tag}_lse"] = o, lse
         out[f"{tag}_causal"] = np.array(int(causal))
+        out[f"{tag}_window"] = np.array(int(window))
+        out[f"{tag}_softcap"] = np.array(float(cap))
     # fp8 grid: scalar_fpquant(v, 448, 3, -6) (avx512_fpquant_f32.cpp:28-41)
     x = np.concatenate([
         rng.standard_normal(512).astype(np.float32) * 4,

@@ -21,10 +21,12 @@ def test_gemm_int8_golden():
     assert np.array_equal(orc.gemm_i8_i32(a, GOLD["gemm_i8_b"]), GOLD["gemm_i8_c"])
 
 
-@pytest.mark.parametrize("tag", ["fa_causal_gqa", "fa_causal_offset", "fa_full"])
+@pytest.mark.parametrize("tag", ["fa_causal_gqa", "fa_causal_offset", "fa_full", "fa_window_causal",
+                                 "fa_window_centered", "fa_softcap"])
 def test_flash_attn_golden(tag):
     q, k, v = GOLD[f"{tag}_q"], GOLD[f"{tag}_k"], GOLD[f"{tag}_v"]
-    o, lse = orc.flash_attn_dense(q, k, v, causal=bool(GOLD[f"{tag}_causal"]))
+    o, lse = orc.flash_attn_dense(q, k, v, causal=bool(GOLD[f"{tag}_causal"]), window=int(GOLD[f"{tag}_window"]),
+                                  softcap=float(GOLD[f"{tag}_softcap"]))
     assert orc.max_rel_err(o, GOLD[f"{tag}_o"]) <= 1e-5
     assert np.max(np.abs(lse - GOLD[f"{tag}_lse"])) <= 1e-5
 

@@ -124,3 +124,51 @@ def test_attention_rejects_bad_shapes(lane):
     assert f(z.ctypes.data, z.ctypes.data, z.ctypes.data, o.ctypes.data, 1, 1, 0, 8, 16, 1.0, 0) == 1
     g = lib.tessera_gfx950_flash_attn_gqa_bf16
     assert g(z.ctypes.data, z.ctypes.data, z.ctypes.data, o.ctypes.data, None, 1, 3, 2, 8, 8, 16, 1.0, 0) == 1
+
+
+WINDOW_CASES = [
+    # B, Hq, Hkv, Sq, Sk, D, causal, window, softcap
+    (1, 2, 2, 300, 300, 128, True, 64, 0.0), (1, 4, 2, 700, 700, 128, True, 200, 0.0),
+    (1, 2, 1, 257, 511, 128, True, 33, 0.0), (1, 2, 2, 513, 513, 64, True, 128, 0.0),
+    (1, 2, 2, 300, 300, 128, False, 90, 0.0), (1, 2, 2, 400, 250, 64, False, 40, 0.0),
+    (1, 2, 2, 300, 300, 128, True, 0, 5.0), (1, 4, 1, 257, 300, 64, True, 0, 2.5),
+    (1, 2, 2, 520, 520, 128, True, 100, 8.0), (1, 2, 2, 100, 100, 48, True, 20, 3.0),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,window,cap", WINDOW_CASES)
+def test_sliding_window_and_softcap(lane, B, Hq, Hkv, Sq, Sk, D, causal, window, cap):
+    q, k, v = _qkv(B, Hq, Hkv, Sq, Sk, D, 29, "bf16")
+    ref_o, ref_lse = orc.flash_attn_dense(_f32(q), _f32(k), _f32(v), causal=causal, window=window, softcap=cap)
+    o, lse = ops.gqa_attention(q, k, v, causal=causal, return_lse=True, out="f32", window=window, logit_softcap=cap)
+    assert not np.isnan(o).any()
+    assert orc.max_rel_err(o, ref_o) <= TOL
+    finite = np.isfinite(ref_lse)
+    assert np.array_equal(np.isfinite(lse), finite)
+    assert np.max(np.abs(lse[finite] - ref_lse[finite])) <= TOL
+
+
+def test_window_closed_forms(lane):
+    """window = 1 (causal): every query sees exactly its diagonal key -> O = V row,
+    LSE = that score.  A window wider than the sequence equals plain causal."""
+    q, k, v = _qkv(1, 2, 2, 200, 200, 128, 5, "bf16")
+    o, lse = ops.flash_attn(q, k, v, causal=True, window=1, return_lse=True, out="f32")
+    assert np.allclose(o, _f32(v), atol=1e-6)
+    s = np.einsum("bhqd,bhqd->bhq", _f32(q).astype(np.float64), _f32(k).astype(np.float64)) / np.sqrt(128)
+    assert np.max(np.abs(lse - s)) <= 2e-3
+    wide = ops.flash_attn(q, k, v, causal=True, window=4096, out="f32")
+    assert np.array_equal(wide, ops.flash_attn(q, k, v, causal=True, out="f32"))
+
+
+def test_sliding_window_executor_op(lane):
+    from tessera_amd import executors as ex
+    q, k, v = (np.asarray(_f32(x), np.float16) for x in _qkv(1, 2, 2, 128, 128, 64, 7, "f16"))
+    art = ex.make_artifact("tessera.attn_sliding_window", ["q", "k", "v"], ["q", "k", "v"], "gfx950_flash_attn",
+                           kwargs={"window": 32})
+    res = ex.launch(art, (q, k, v))
+    assert res["ok"], res
+    ref, _ = orc.flash_attn_dense(q.astype(np.float32), k.astype(np.float32), v.astype(np.float32), causal=True,
+                                  window=32)
+    assert orc.max_rel_err(res["output"], ref) <= TOL
+    bad = ex.make_artifact("tessera.attn_sliding_window", ["q", "k", "v"], ["q", "k", "v"], "gfx950_flash_attn")
+    assert not ex.launch(bad, (q, k, v))["ok"]

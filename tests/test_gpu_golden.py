@@ -24,10 +24,12 @@ def test_gemm_int8_golden(lane):
     assert np.array_equal(c, GOLD["gemm_i8_c"])
 
 
-@pytest.mark.parametrize("tag", ["fa_causal_gqa", "fa_causal_offset", "fa_full"])
+@pytest.mark.parametrize("tag", ["fa_causal_gqa", "fa_causal_offset", "fa_full", "fa_window_causal",
+                                 "fa_window_centered", "fa_softcap"])
 def test_flash_attn_golden(lane, tag):
     q, k, v = (b16.from_float32(GOLD[f"{tag}_{n}"]) for n in "qkv")   # already bf16-representable
-    o, lse = ops.gqa_attention(q, k, v, causal=bool(GOLD[f"{tag}_causal"]), return_lse=True, out="f32")
+    o, lse = ops.gqa_attention(q, k, v, causal=bool(GOLD[f"{tag}_causal"]), return_lse=True, out="f32",
+                               window=int(GOLD[f"{tag}_window"]), logit_softcap=float(GOLD[f"{tag}_softcap"]))
     assert orc.max_rel_err(o, GOLD[f"{tag}_o"]) <= 2e-3
     assert np.max(np.abs(lse - GOLD[f"{tag}_lse"])) <= 2e-3
 

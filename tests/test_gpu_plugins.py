@@ -44,8 +44,10 @@ def test_launch_flash_attn_executor(lane):
     ref, _ = orc.flash_attn_dense(q.to_float32(), k.to_float32(), v.to_float32(), causal=True)
     assert orc.max_rel_err(res["output"], ref) <= 2e-3
     bad = ex.make_artifact("tessera.flash_attn", ["q", "k", "v"], ["q", "k", "v"], "gfx950_flash_attn",
-                           kwargs={"window": 16})
+                           kwargs={"window": -16})
     assert ex.launch(bad, (q, k, v))["runtime_status"] == "invalid_artifact"
+    bias = ex.make_artifact("tessera.flash_attn", ["q", "k", "v", "b"], ["q", "k", "v", "b"], "gfx950_flash_attn")
+    assert ex.launch(bias, (q, k, v, np.zeros((130, 130), np.float32)))["runtime_status"] == "invalid_artifact"
 
 
 def test_launch_moe_transport_executor(lane):

@@ -64,3 +64,22 @@ def test_c_router_matches_numpy(T, E, k, cap):
     assert np.array_equal(tos, d.token_of_slot) and np.array_equal(eos, d.expert_of_slot)
     assert np.array_equal(gs, d.group_sizes) and np.array_equal(go, d.group_offsets)
     assert np.allclose(cw, d.combine_weights, rtol=2e-6)
+
+
+def test_window_and_softcap_match_the_reference_kernel():
+    """Sliding window (both forms) and logit soft cap of the numpy oracle against the
+    reference's compiled CPU kernel."""
+    if co.ref() is None:
+        pytest.skip("compiled reference twins unavailable on this host")
+    rng = np.random.default_rng(12)
+    for (B, Hq, Hkv, Sq, Sk, D, causal, window, cap) in [
+            (1, 2, 1, 40, 40, 16, True, 8, 0.0), (1, 2, 2, 24, 50, 16, True, 13, 0.0),
+            (1, 1, 1, 33, 33, 8, False, 10, 0.0), (2, 4, 2, 20, 20, 16, True, 0, 3.0),
+            (1, 2, 2, 31, 47, 16, True, 9, 5.0)]:
+        q = rng.standard_normal((B, Hq, Sq, D)).astype(np.float32)
+        k = rng.standard_normal((B, Hkv, Sk, D)).astype(np.float32)
+        v = rng.standard_normal((B, Hkv, Sk, D)).astype(np.float32)
+        o, lse = orc.flash_attn_dense(q, k, v, causal=causal, window=window, softcap=cap)
+        ro, rl = co.ref_flash_attn_lse(q, k, v, 1.0 / np.sqrt(D), causal, window, cap)
+        assert orc.max_rel_err(o, ro) <= 1e-5
+        assert np.max(np.abs(lse - rl)) <= 1e-5
