@@ -154,6 +154,14 @@ int tessera_gfx950_gated_gemm_f16_dev(const void* A, const void* Wg, const void*
 int tessera_gfx950_gated_gemm_bf16_dev(const void* A, const void* Wg, const void* Wu, int activation, void* D,
                                        int M, int H, int K, void* stream);
 
+/* The schedule the GEMM launcher picks for an aligned problem (workgroup tile and
+ * K split), as a host-only query: the gfx950 counterpart of
+ * select_rocm_gemm_schedule (python/tessera/compiler/rocm_schedule.py:94-154), which
+ * the reference's executor consults before building a kernel
+ * (python/tessera/runtime.py:6676-6679).  elem_bytes 2 = f16/bf16, 1 = int8/fp8. */
+int tessera_gfx950_gemm_schedule(int M, int N, int K, int batch, int elem_bytes,
+                                 int* tile_m, int* tile_n, int* tile_k, int* split_k);
+
 /* Kernel-only benchmark with resident, library-owned buffers: warm-up, `iters`
  * launches between HIP events, cross-checked against wall clock
  * (tessera_rocm_gemm.cpp:551-667).  *avg_ms = mean per-launch ms. */

@@ -197,6 +197,26 @@ int tessera_gfx950_gated_gemm_bf16_dev(const void* A, const void* Wg, const void
   return gated_dev<BF16>(A, Wg, Wu, activation, D, M, H, K, as_stream(stream));
 }
 
+// Host-only: the tile / split-K schedule the launcher picks (no device needed).
+int tessera_gfx950_gemm_schedule(int M, int N, int K, int batch, int elem_bytes, int* tile_m, int* tile_n,
+                                 int* tile_k, int* split_k) {
+  if (bad_dims(batch, M, N, K) || !tile_m || !tile_n || !tile_k || !split_k) return kBadShape;
+  if (elem_bytes == 2) {
+    const Gemm16Schedule sch = select_gemm16_schedule(M, N, K, batch);
+    *tile_m = *tile_n = sch.tile;
+    *tile_k = G16_BK;
+    *split_k = sch.split_k;
+    return kOk;
+  }
+  if (elem_bytes == 1) {                     // int8 / fp8: one 256 x 256 x 128 tile shape
+    *tile_m = *tile_n = 256;
+    *tile_k = 128;
+    *split_k = 1;
+    return kOk;
+  }
+  return kBadShape;
+}
+
 // Kernel-only timing on resident buffers.  The device-event figure is accepted
 // only when it lies within 0.5x..2x of the wall clock around the same launches;
 // otherwise the wall-clock figure is reported and the source says so.

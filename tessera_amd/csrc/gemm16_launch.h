@@ -120,6 +120,29 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restr
   }
 }
 
+// Tile and split-K choice of the dense 16-bit GEMM for an aligned problem — the one
+// place the decision lives (the launcher below and the schedule query of the C ABI
+// both call it).  256x256 when that alone fills the chip; else 128x128 or 64x64
+// tiles, and for a single product with few tiles and a long K (decode-shaped: the
+// weight matrix streams from HBM once) K is split over about 768 workgroups.
+struct Gemm16Schedule {
+  int tile;      // square workgroup tile edge: 256, 128 or 64
+  int split_k;   // number of K splits (1 = none)
+};
+inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
+  const long tiles256 = (long)ceil_div(M, 256) * ceil_div(N, 256) * batch;
+  const long tiles128 = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch;
+  if (tiles256 >= 192) return {256, 1};
+  const bool t128 = tiles128 >= 192 || (M > 64 && N >= 128);
+  int splits = 1;
+  if (batch == 1) {
+    const long tiles = t128 ? tiles128 : (long)ceil_div(M, 64) * ceil_div(N, 64);
+    splits = (int)std::max<long>(1, std::min<long>((768 + tiles - 1) / tiles, K / 512));
+    while (splits > 1 && K % (splits * G16_BK) != 0) --splits;
+  }
+  return {t128 ? 128 : 64, splits};
+}
+
 // Dense / batched.  p.groups = batch count (>= 1).
 template <class T, int EPI>
 int launch_gemm16(Gemm16Params p, hipStream_t s) {
@@ -135,18 +158,13 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
     hipLaunchKernelGGL((gemm16_generic_kernel<T, EPI>), grid, block, 0, s, p);
     return launch_status();
   }
-  const long tiles256 = (long)ceil_div(p.M, 256) * ceil_div(p.N, 256) * p.groups;
-  const long tiles128 = (long)ceil_div(p.M, 128) * ceil_div(p.N, 128) * p.groups;
-  if (tiles256 >= 192) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false>(p, s);
-  const bool t128 = tiles128 >= 192 || (p.M > 64 && p.N >= 128);
-  // Few output tiles and a long K (decode-shaped products: the weight matrix streams
-  // from HBM once): split K over enough workgroups to cover the chip.  Every split
-  // is one "batch" of the same kernel writing f32 partials, summed in split order
-  // by a second kernel, so the result does not depend on scheduling.
-  if (p.groups == 1) {
-    const long tiles = t128 ? tiles128 : (long)ceil_div(p.M, 64) * ceil_div(p.N, 64);
-    int splits = (int)std::min<long>((768 + tiles - 1) / tiles, p.K / 512);
-    while (splits > 1 && p.K % (splits * G16_BK) != 0) --splits;
+  const Gemm16Schedule sch = select_gemm16_schedule(p.M, p.N, p.K, p.groups);
+  if (sch.tile == 256) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false>(p, s);
+  const bool t128 = sch.tile == 128;
+  // Every K split is one "batch" of the same kernel writing f32 partials, summed in
+  // split order by a second kernel, so the result does not depend on scheduling.
+  {
+    const int splits = sch.split_k;
     if (splits > 1) {
       float* ws = nullptr;
       const size_t mn = (size_t)p.M * p.N;

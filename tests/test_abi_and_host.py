@@ -230,3 +230,26 @@ def test_tile_table():
     for e in tile_table.KERNEL_TABLE:
         assert e.runtime_lane in lanes
         assert set(e.symbols) <= declared
+
+
+def test_gemm_schedule_query_needs_no_device():
+    """The schedule descriptor reads the launcher's own tile / split-K decision."""
+    from tessera_amd.schedule import select_gfx950_gemm_schedule as sel
+    big = sel(8192, 8192, 8192, dtype="bf16")
+    assert big.workgroup_tile == (256, 256, 64) and big.macro_tile == (8, 8) and big.split_k == 1
+    assert big.instruction_tile == (32, 32, 16) and big.target_ir_attrs()["schedule_arch"] == "gfx950"
+    dec = sel(16, 8192, 8192, dtype="bf16")
+    assert dec.workgroup_tile[:2] == (64, 64) and dec.split_k > 1 and 8192 % (dec.split_k * 64) == 0
+    assert sel(128, 8192, 8192).workgroup_tile[:2] == (128, 128)
+    assert sel(128, 256, 64, batch=4).split_k == 1                      # batched products never split K
+    q = sel(4096, 8192, 8192, dtype="int8")
+    assert q.workgroup_tile == (256, 256, 128) and q.instruction_tile == (32, 32, 32)
+    assert sel(4096, 8192, 8192, dtype="fp8_e4m3").instruction_tile == (32, 32, 64)
+    assert big.cache_key() != dec.cache_key()
+    import pytest
+    with pytest.raises(ValueError):
+        sel(0, 8, 8)
+    with pytest.raises(ValueError):
+        sel(8, 8, 8, arch="gfx1151")
+    with pytest.raises(ValueError):
+        sel(8, 8, 8, dtype="f64")
