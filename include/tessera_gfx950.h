@@ -231,6 +231,25 @@ int tessera_gfx950_flash_attn_ext_bf16_dev(const void* Q, const void* K, const v
                                            int causal, int window, float softcap, int out_dtype,
                                            void* stream);
 
+/* Additive attention bias: O = softmax(scale Q K^T + bias, ...) V with bias an f32
+ * tensor [B, Hq, Sq, Sk] (the caller broadcasts, as the reference's executor does for
+ * its fourth operand, python/tessera/runtime.py:7270-7274); NULL means none.  With a
+ * soft cap the bias is added after the cap (avx512_flash_attn_f32.cpp:199-206). */
+int tessera_gfx950_flash_attn_bias_f16(const void* Q, const void* K, const void* V, const float* bias,
+                                       void* O, void* LSE, int B, int Hq, int Hkv, int Sq, int Sk,
+                                       int D, float scale, int causal, int window, float softcap);
+int tessera_gfx950_flash_attn_bias_bf16(const void* Q, const void* K, const void* V, const float* bias,
+                                        void* O, void* LSE, int B, int Hq, int Hkv, int Sq, int Sk,
+                                        int D, float scale, int causal, int window, float softcap);
+int tessera_gfx950_flash_attn_bias_f16_dev(const void* Q, const void* K, const void* V, const float* bias,
+                                           void* O, void* LSE, int B, int Hq, int Hkv, int Sq, int Sk,
+                                           int D, float scale, int causal, int window, float softcap,
+                                           int out_dtype, void* stream);
+int tessera_gfx950_flash_attn_bias_bf16_dev(const void* Q, const void* K, const void* V, const float* bias,
+                                            void* O, void* LSE, int B, int Hq, int Hkv, int Sq, int Sk,
+                                            int D, float scale, int causal, int window, float softcap,
+                                            int out_dtype, void* stream);
+
 /* ---- flash-attention backward -------------------------------------------- */
 
 /* (dQ, dK, dV) of O = softmax(scale Q K^T, causal) V given dO: the contract of the

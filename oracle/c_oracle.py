@@ -151,7 +151,7 @@ def ref_gemm_u8s8(a_u8, b_s8) -> np.ndarray:
     return c
 
 
-def ref_flash_attn_lse(q, k, v, scale: float, causal: bool, window: int = 0, softcap: float = 0.0):
+def ref_flash_attn_lse(q, k, v, scale: float, causal: bool, window: int = 0, softcap: float = 0.0, bias=None):
     q = np.ascontiguousarray(q, np.float32)
     k = np.ascontiguousarray(k, np.float32)
     v = np.ascontiguousarray(v, np.float32)
@@ -160,7 +160,9 @@ def ref_flash_attn_lse(q, k, v, scale: float, causal: bool, window: int = 0, sof
     o = np.empty_like(q)
     lse = np.empty((B, Hq, Sq), np.float32)
     i64 = _c_i64
-    ref().tessera_x86_flash_attn_ext_lse_f32(_p(q), _p(k), _p(v), None, i64(B), i64(Hq), i64(Hkv), i64(Sq), i64(Sk),
+    if bias is not None:
+        bias = np.ascontiguousarray(np.broadcast_to(bias, (B, Hq, Sq, Sk)), np.float32)
+    ref().tessera_x86_flash_attn_ext_lse_f32(_p(q), _p(k), _p(v), _p(bias) if bias is not None else None, i64(B), i64(Hq), i64(Hkv), i64(Sq), i64(Sk),
                                              i64(D), i64(D), _c_f(scale), 1 if causal else 0, i64(window), _c_f(softcap),
                                              _p(o), _p(lse))
     return o, lse

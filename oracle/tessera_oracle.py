@@ -204,10 +204,12 @@ def key_bounds(i: int, sq: int, sk: int, causal: bool, window: int = 0):
 
 
 def flash_attn_dense(Q, K, V, scale=None, causal=False, dtype=np.float64, window: int = 0,
-                     softcap: float = 0.0):
+                     softcap: float = 0.0, bias=None):
     """Dense ``softmax(scale*Q K^T, causal) V`` with GQA and LSE; optional sliding
-    ``window`` (see :func:`key_bounds`) and logit soft cap (scaled scores pass
-    through ``cap * tanh(s / cap)``, ``avx512_flash_attn_f32.cpp:115,161``).
+    ``window`` (see :func:`key_bounds`), logit soft cap (scaled scores pass
+    through ``cap * tanh(s / cap)``, ``avx512_flash_attn_f32.cpp:115,161``) and
+    additive ``bias`` ``[B,Hq,Sq,Sk]`` added after the cap
+    (``avx512_flash_attn_f32.cpp:198-208``).
 
     Q ``[B,Hq,Sq,D]``; K, V ``[B,Hkv,Sk,D]``.  kv head of q head ``h`` is
     ``h * Hkv // Hq`` (``avx512_flash_attn_f32.cpp:386``), which equals
@@ -233,6 +235,8 @@ def flash_attn_dense(Q, K, V, scale=None, causal=False, dtype=np.float64, window
             s = (Q[b, h] @ K[b, kh].T) * dtype(scale)
             if softcap > 0:
                 s = dtype(softcap) * np.tanh(s / dtype(softcap))
+            if bias is not None:
+                s = s + np.asarray(bias[b, h], dtype)
             if causal or window > 0:
                 bounds = np.array([key_bounds(i, Sq, Sk, causal, window) for i in range(Sq)])
                 j = np.arange(Sk)[None, :]

@@ -15,10 +15,10 @@ bool bad_attn(int B, int Hq, int Hkv, int Sq, int Sk, int D) {
   return false;
 }
 
-template <class T, int D, bool SOFTCAP>
+template <class T, int D, bool EXT>
 int launch_flash(const FlashParams& p, hipStream_t s) {
   constexpr int kSmem = 2 * 2 * FA_BKV * D * 2;
-  auto kern = flash_fwd_kernel<T, D, SOFTCAP>;
+  auto kern = flash_fwd_kernel<T, D, EXT>;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [&] {
@@ -34,7 +34,7 @@ int launch_flash(const FlashParams& p, hipStream_t s) {
 template <class T>
 int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, int B, int Hq, int Hkv,
               int Sq, int Sk, int D, float scale, int causal, int out_storage, hipStream_t s, int window = 0,
-              float softcap = 0.f) {
+              float softcap = 0.f, const float* bias = nullptr) {
   if (bad_attn(B, Hq, Hkv, Sq, Sk, D) || !Q || !K || !V || !O) return kBadShape;
   if (window < 0 || !(softcap >= 0.f)) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
@@ -50,10 +50,12 @@ int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, i
   p.out_storage = out_storage ? 1 : 0;
   p.window = window;
   p.softcap = softcap;
+  p.bias = bias;
   const bool al = ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
                     reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(O)) & 15) == 0;
-  if (al && D == 128) return p.softcap > 0.f ? launch_flash<T, 128, true>(p, s) : launch_flash<T, 128, false>(p, s);
-  if (al && D == 64) return p.softcap > 0.f ? launch_flash<T, 64, true>(p, s) : launch_flash<T, 64, false>(p, s);
+  const bool ext = p.softcap > 0.f || p.bias != nullptr;
+  if (al && D == 128) return ext ? launch_flash<T, 128, true>(p, s) : launch_flash<T, 128, false>(p, s);
+  if (al && D == 64) return ext ? launch_flash<T, 64, true>(p, s) : launch_flash<T, 64, false>(p, s);
   const long rows = (long)B * Hq * Sq;
   hipLaunchKernelGGL((flash_fwd_generic_kernel<T>), dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, p, D);
   return launch_status();
@@ -61,7 +63,8 @@ int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, i
 
 template <class T>
 int flash_host(const void* Q, const void* K, const void* V, void* O, void* LSE, int B, int Hq, int Hkv,
-               int Sq, int Sk, int D, float scale, int causal, int window = 0, float softcap = 0.f) {
+               int Sq, int Sk, int D, float scale, int causal, int window = 0, float softcap = 0.f,
+               const float* bias = nullptr) {
   if (bad_attn(B, Hq, Hkv, Sq, Sk, D) || !Q || !K || !V || !O) return kBadShape;
   if (window < 0 || !(softcap >= 0.f)) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
@@ -73,8 +76,10 @@ int flash_host(const void* Q, const void* K, const void* V, void* O, void* LSE, 
   void* dV = scope.alloc(kv_bytes, V);
   void* dO = scope.alloc(o_bytes);
   void* dL = LSE ? scope.alloc(l_bytes) : nullptr;
+  void* dBias = bias ? scope.alloc((size_t)B * Hq * Sq * Sk * 4, bias) : nullptr;
   if (scope.failed()) return kDeviceFailed;
-  int rc = flash_dev<T>(dQ, dK, dV, dO, dL, B, Hq, Hkv, Sq, Sk, D, scale, causal, 0, nullptr, window, softcap);
+  int rc = flash_dev<T>(dQ, dK, dV, dO, dL, B, Hq, Hkv, Sq, Sk, D, scale, causal, 0, nullptr, window, softcap,
+                        static_cast<const float*>(dBias));
   if (rc != kOk) return rc;
   if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
   if (!scope.download(O, dO, o_bytes)) return kDeviceFailed;
@@ -244,6 +249,31 @@ int tessera_gfx950_flash_attn_ext_bf16_dev(const void* Q, const void* K, const v
                                            int window, float softcap, int out_dtype, void* stream) {
   return flash_dev<BF16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, out_dtype, as_stream(stream), window,
                          softcap);
+}
+
+int tessera_gfx950_flash_attn_bias_f16(const void* Q, const void* K, const void* V, const float* bias, void* O,
+                                       void* LSE, int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                                       int causal, int window, float softcap) {
+  return flash_host<F16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, window, softcap, bias);
+}
+int tessera_gfx950_flash_attn_bias_bf16(const void* Q, const void* K, const void* V, const float* bias, void* O,
+                                        void* LSE, int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                                        int causal, int window, float softcap) {
+  return flash_host<BF16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, window, softcap, bias);
+}
+int tessera_gfx950_flash_attn_bias_f16_dev(const void* Q, const void* K, const void* V, const float* bias,
+                                           void* O, void* LSE, int B, int Hq, int Hkv, int Sq, int Sk, int D,
+                                           float scale, int causal, int window, float softcap, int out_dtype,
+                                           void* stream) {
+  return flash_dev<F16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, out_dtype, as_stream(stream), window,
+                        softcap, bias);
+}
+int tessera_gfx950_flash_attn_bias_bf16_dev(const void* Q, const void* K, const void* V, const float* bias,
+                                            void* O, void* LSE, int B, int Hq, int Hkv, int Sq, int Sk, int D,
+                                            float scale, int causal, int window, float softcap, int out_dtype,
+                                            void* stream) {
+  return flash_dev<BF16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, out_dtype, as_stream(stream), window,
+                         softcap, bias);
 }
 
 int tessera_gfx950_flash_attn_bwd_f16(const void* dO, const void* Q, const void* K, const void* V, void* dQ,

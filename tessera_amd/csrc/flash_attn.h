@@ -47,6 +47,7 @@ struct FlashParams {
   int out_storage;     // 0: f32 O, 1: O in the storage dtype
   int window;          // > 0: band of keys per query (see key_bounds); 0: none
   float softcap;       // > 0: scaled scores pass through cap * tanh(s / cap); 0: none
+  const float* bias;   // additive bias [B, Hq, Sq, Sk] f32 added to the (capped) scaled scores, or null
 };
 
 // Visible keys [lo, hi] of query row i — the reference's attention_bounds
@@ -111,7 +112,7 @@ __device__ __forceinline__ float scale_acc(float acc, float corr) {
   return acc;
 }
 
-template <class T, int D, bool SOFTCAP>
+template <class T, int D, bool EXT>
 __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashParams p) {
   constexpr int QT = FA_QT;
   constexpr int KSTEPS = D / 16;         // MFMA k steps of the score product
@@ -249,11 +250,17 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
   // Exponent argument of a raw score, in base 2: scale * log2(e) * s, or with a
   // soft cap  cap * log2(e) * tanh(scale * s / cap)  (tanh y = 1 - 2 / (e^{2y} + 1)).
   const float cap2 = p.softcap * 1.44269504088896340736f;
-  const float incap = SOFTCAP ? 2.0f * 1.44269504088896340736f * p.scale / p.softcap : 0.f;
-  // With a soft cap the score tiles are transformed in place (before masking) and
-  // already are exponent arguments; without one the raw scores are kept and the
-  // factor cs = scale * log2(e) is folded into the exponential's FMA.
-  const float cs = SOFTCAP ? 1.0f : c;
+  const float incap = (EXT && p.softcap > 0.f) ? 2.0f * 1.44269504088896340736f * p.scale / p.softcap : 0.f;
+  // The extended variant (soft cap and / or additive bias) turns the score tiles into
+  // exponent arguments in place, before masking; the plain variant keeps the raw
+  // scores and folds cs = scale * log2(e) into the exponential's FMA.
+  const float cs = EXT ? 1.0f : c;
+  const float* bias_row[QT];             // this lane's row of the additive bias, or null
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const int qi = min(qw + 32 * qt + l32, p.Sq - 1);
+    bias_row[qt] = (EXT && p.bias) ? p.bias + ((long)(b * p.Hq + hq) * p.Sq + qi) * p.Sk : nullptr;
+  }
   auto capped = [&](float sraw) -> float {
     return cap2 * (1.0f - 2.0f * __builtin_amdgcn_rcpf(fast_exp2(sraw * incap) + 1.0f));
   };
@@ -322,13 +329,21 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
     if (t + 2 < ntiles) load_k(tile_base + t + 2, PAR);
     if (t + 1 < ntiles) load_v(tile_base + t + 1, PAR ^ 1);
     const int kv0 = (tile_base + t) * FA_BKV;
-    if constexpr (SOFTCAP) {
+    if constexpr (EXT) {
+      const bool cap = p.softcap > 0.f;
 #pragma unroll
       for (int qt = 0; qt < QT; ++qt)
 #pragma unroll
         for (int kt = 0; kt < FA_KT; ++kt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) sc[qt][kt][r] = capped(sc[qt][kt][r]);
+          for (int r = 0; r < 16; ++r) {
+            float x = cap ? capped(sc[qt][kt][r]) : sc[qt][kt][r] * c;
+            if (bias_row[qt]) {
+              const int key = kv0 + kt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+              x += bias_row[qt][key < p.Sk ? key : p.Sk - 1] * 1.44269504088896340736f;
+            }
+            sc[qt][kt][r] = x;
+          }
     }
     // mask (only tiles that cross a bound of one of the wave's rows)
     const bool need_mask = (kv0 + FA_BKV - 1 > whi_first) || (kv0 < wlo_last);
@@ -455,6 +470,9 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
   // other waves already refill that stage.
   int t = 0;
   if (t_w0 == 0 && nt_w > 0) score_steps(sA, 0, 0, KSTEPS);
+  // Step 0 refills K stage 0: every wave must have read tile 0's keys first (a wave
+  // that starts late issues those loads without any arithmetic ahead of them).
+  __syncthreads();
   for (; t < t_w0; ++t) {
     if (t + 2 < ntiles) load_k(tile_base + t + 2, t & 1);
     if (t + 1 < ntiles) load_v(tile_base + t + 1, (t & 1) ^ 1);
@@ -534,6 +552,7 @@ __global__ void flash_fwd_generic_kernel(const FlashParams p, int D) {
     for (int d = 0; d < D; ++d) s += from_storage<T>(q[d]) * from_storage<T>(Kb[(long)j * D + d]);
     s *= p.scale;
     if (p.softcap > 0.f) s = p.softcap * tanhf(s / p.softcap);
+    if (p.bias) s += p.bias[row * p.Sk + j];
     const float mn = fmaxf(m, s);
     const float cr = __expf(m - mn);       // exp(-inf) = 0 on the first key
     const float e = __expf(s - mn);

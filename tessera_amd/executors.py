@@ -195,18 +195,20 @@ _FA_OPS = ("tessera.flash_attn", "tessera.multi_head_attention", "tessera.gqa_at
 
 def execute_gfx950_flash_attn(artifact: RuntimeArtifact, args: Any):
     """Attention forward: Q ``[..., Hq, Sq, D]``, K/V ``[..., Hkv, Sk, D]`` in
-    f16/bf16 -> f32 O shaped like Q.  ``kwargs``: ``causal``, ``scale``, ``window``
-    (a positive width; required by ``tessera.attn_sliding_window``) and
-    ``logit_softcap`` (``runtime.py:7312-7340``)."""
+    f16/bf16 -> f32 O shaped like Q; an optional fourth operand is the additive
+    attention bias, broadcastable to ``[..., Hq, Sq, Sk]`` (``runtime.py:7270-7274``).
+    ``kwargs``: ``causal``, ``scale``, ``window`` (a positive width; required by
+    ``tessera.attn_sliding_window``) and ``logit_softcap`` (``runtime.py:7312-7340``)."""
     md = artifact.metadata or {}
     op = _single_op(artifact, _FA_OPS, "gfx950_flash_attn")
     names = [str(n) for n in op.get("operands", [])]
     if len(names) < 3:
         raise ValueError("flash_attn requires Q, K, V operands")
-    if len(names) > 3:
-        raise ValueError("gfx950 flash_attn lane has no additive-bias operand")
+    if len(names) > 4:
+        raise ValueError(f"flash_attn takes Q, K, V plus an optional attn_bias operand; got {len(names)}")
     values = _bind_launch_args(args, list(md.get("arg_names") or []))
     q, k, v = (_as_array(values[n]) for n in names[:3])
+    bias = np.asarray(_as_array(values[names[3]])) if len(names) == 4 else None
     kwargs = op.get("kwargs") or {}
     if kwargs.get("dropout_p"):
         raise ValueError("gfx950 flash_attn lane does not implement `dropout_p`")
@@ -222,7 +224,7 @@ def execute_gfx950_flash_attn(artifact: RuntimeArtifact, args: Any):
     # the windowed kernel of the reference is implicitly causal (runtime.py:7318-7321)
     causal = bool(kwargs.get("causal", False)) or window > 0
     return _ops.gqa_attention(q, k, v, scale=kwargs.get("scale"), causal=causal, out="f32", window=window,
-                              logit_softcap=softcap)
+                              logit_softcap=softcap, attn_bias=bias)
 
 
 _FA_BWD_OPS = ("tessera.flash_attn_bwd", "tessera.flash_attn_vjp")

@@ -120,6 +120,10 @@ _SIGNATURES = {
     "tessera_gfx950_flash_attn_ext_bf16": [_c_vp] * 5 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f],
     "tessera_gfx950_flash_attn_ext_f16_dev": [_c_vp] * 5 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f, _c_int, _c_vp],
     "tessera_gfx950_flash_attn_ext_bf16_dev": [_c_vp] * 5 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f, _c_int, _c_vp],
+    "tessera_gfx950_flash_attn_bias_f16": [_c_vp] * 6 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f],
+    "tessera_gfx950_flash_attn_bias_bf16": [_c_vp] * 6 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f],
+    "tessera_gfx950_flash_attn_bias_f16_dev": [_c_vp] * 6 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f, _c_int, _c_vp],
+    "tessera_gfx950_flash_attn_bias_bf16_dev": [_c_vp] * 6 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f, _c_int, _c_vp],
     "tessera_gfx950_flash_attn_bwd_f16": [_c_vp] * 7 + [_c_int] * 6 + [_c_f, _c_int],
     "tessera_gfx950_flash_attn_bwd_bf16": [_c_vp] * 7 + [_c_int] * 6 + [_c_f, _c_int],
     "tessera_gfx950_flash_attn_bwd_f16_dev": [_c_vp] * 9 + [_c_int] * 6 + [_c_f, _c_int, _c_vp],

@@ -208,7 +208,7 @@ def gemm_i8(A, B) -> np.ndarray:
 # ---------------------------------------------------------------------------
 
 
-def _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa, window=0, logit_softcap=0.0):
+def _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa, window=0, logit_softcap=0.0, attn_bias=None):
     Q, K, V = _unbox(Q), _unbox(K), _unbox(V)
     st = _storage(Q, K)
     if _storage(V) != st:
@@ -241,9 +241,22 @@ def _attention(Q, K, V, scale, causal, return_lse, out, allow_gqa, window=0, log
         raise ValueError(f"flash_attn window must be a non-negative width; got {window}")
     if softcap < 0:
         raise ValueError(f"flash_attn logit_softcap must be non-negative; got {softcap}")
+    bias = None
+    if attn_bias is not None:
+        # host-broadcast to [..., Hq, Sq, Sk], as the reference's executor does (runtime.py:7341-7355)
+        try:
+            bias = np.broadcast_to(np.asarray(_unbox(attn_bias), dtype=np.float32), tuple(q.shape[:-2]) + (Sq, Sk))
+        except ValueError:
+            raise ValueError(f"flash_attn attn_bias {np.asarray(attn_bias).shape} is not broadcastable to "
+                             f"{tuple(q.shape[:-2]) + (Sq, Sk)}") from None
+        bias = np.ascontiguousarray(bias, dtype=np.float32)
     o = np.empty(q.shape, np.float32)
     lse = np.empty(q.shape[:-1], np.float32) if return_lse else None
-    if window or softcap:
+    if bias is not None:
+        fn = getattr(_lane.load(), f"tessera_gfx950_flash_attn_bias_{st}")
+        rc = fn(q.ctypes.data, k.ctypes.data, v.ctypes.data, bias.ctypes.data, o.ctypes.data, _lane.ptr(lse),
+                Bq, Hq, Hkv, Sq, Sk, D, float(scale), 1 if causal else 0, window, softcap)
+    elif window or softcap:
         fn = getattr(_lane.load(), f"tessera_gfx950_flash_attn_ext_{st}")
         rc = fn(q.ctypes.data, k.ctypes.data, v.ctypes.data, o.ctypes.data, _lane.ptr(lse),
                 Bq, Hq, Hkv, Sq, Sk, D, float(scale), 1 if causal else 0, window, softcap)
@@ -298,18 +311,20 @@ def flash_attn_backward(dO, Q, K, V, scale=None, causal: bool = False):
 
 
 def flash_attn(Q, K=None, V=None, scale=None, causal: bool = False, *, return_lse: bool = False,
-               out: str = "storage", window: int = 0, logit_softcap: float = 0.0):
+               out: str = "storage", window: int = 0, logit_softcap: float = 0.0, attn_bias=None):
     """``softmax(scale * Q K^T, causal) V``.  Q/K/V ``[..., H, S, D]`` 16-bit; the
     causal mask is bottom-right aligned (key ``j`` visible to query ``i`` iff
-    ``j <= i + max(Sk - Sq, 0)``).  Head counts must match (as in the reference)."""
-    return _attention(Q, K, V, scale, causal, return_lse, out, False, window, logit_softcap)
+    ``j <= i + max(Sk - Sq, 0)``).  Head counts must match (as in the reference).
+    ``attn_bias`` (f32, broadcastable to ``[..., H, Sq, Sk]``) is added to the scaled
+    (and, with ``logit_softcap``, capped) scores before the softmax."""
+    return _attention(Q, K, V, scale, causal, return_lse, out, False, window, logit_softcap, attn_bias)
 
 
 def gqa_attention(Q, K, V, scale=None, causal: bool = False, *, return_lse: bool = False,
-                  out: str = "storage", window: int = 0, logit_softcap: float = 0.0):
+                  out: str = "storage", window: int = 0, logit_softcap: float = 0.0, attn_bias=None):
     """Grouped-query attention: kv head of query head ``h`` is ``h // (Hq / Hkv)``
     — identical to repeating K/V along the head axis."""
-    return _attention(Q, K, V, scale, causal, return_lse, out, True, window, logit_softcap)
+    return _attention(Q, K, V, scale, causal, return_lse, out, True, window, logit_softcap, attn_bias)
 
 
 # ---------------------------------------------------------------------------

@@ -172,3 +172,57 @@ def test_sliding_window_executor_op(lane):
     assert orc.max_rel_err(res["output"], ref) <= TOL
     bad = ex.make_artifact("tessera.attn_sliding_window", ["q", "k", "v"], ["q", "k", "v"], "gfx950_flash_attn")
     assert not ex.launch(bad, (q, k, v))["ok"]
+
+
+BIAS_CASES = [
+    # B, Hq, Hkv, Sq, Sk, D, causal, window, softcap, storage
+    (1, 2, 2, 300, 300, 128, False, 0, 0.0, "bf16"), (2, 4, 2, 257, 511, 128, True, 0, 0.0, "f16"),
+    (1, 4, 1, 513, 513, 64, True, 0, 0.0, "bf16"), (1, 2, 2, 520, 520, 128, True, 100, 0.0, "bf16"),
+    (1, 2, 2, 300, 300, 128, True, 0, 5.0, "bf16"), (1, 2, 1, 100, 130, 48, True, 0, 0.0, "f16"),
+    (1, 2, 2, 64, 1000, 128, False, 0, 3.0, "f16"),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,window,cap,st", BIAS_CASES)
+def test_additive_bias(lane, B, Hq, Hkv, Sq, Sk, D, causal, window, cap, st):
+    q, k, v = _qkv(B, Hq, Hkv, Sq, Sk, D, 31, st)
+    bias = (np.random.default_rng(32).standard_normal((B, Hq, Sq, Sk)) * 2).astype(np.float32)
+    ref_o, ref_lse = orc.flash_attn_dense(_f32(q), _f32(k), _f32(v), causal=causal, window=window, softcap=cap,
+                                          bias=bias)
+    o, lse = ops.gqa_attention(q, k, v, causal=causal, return_lse=True, out="f32", window=window,
+                               logit_softcap=cap, attn_bias=bias)
+    assert not np.isnan(o).any()
+    assert orc.max_rel_err(o, ref_o) <= TOL
+    assert np.max(np.abs(lse - ref_lse)) <= TOL
+
+
+def test_bias_broadcast_and_closed_forms(lane):
+    """A bias constant along the keys leaves O unchanged and shifts LSE by it; a
+    (Sq, Sk) bias broadcasts over batch and heads; a -inf bias acts as a mask
+    (the causal mask written as a bias equals the causal kernel)."""
+    q, k, v = _qkv(2, 4, 2, 200, 200, 128, 9, "bf16")
+    plain_o, plain_lse = ops.gqa_attention(q, k, v, return_lse=True, out="f32")
+    row = np.linspace(-3, 3, 200, dtype=np.float32)[:, None] * np.ones((1, 200), np.float32)
+    o, lse = ops.gqa_attention(q, k, v, return_lse=True, out="f32", attn_bias=row)
+    assert orc.max_rel_err(o, plain_o) <= 1e-5
+    assert np.max(np.abs(lse - (plain_lse + row[:, 0]))) <= 1e-4
+    tri = np.where(np.tril(np.ones((200, 200), bool)), 0.0, -np.inf).astype(np.float32)
+    masked = ops.gqa_attention(q, k, v, out="f32", attn_bias=tri)
+    assert orc.max_rel_err(masked, ops.gqa_attention(q, k, v, causal=True, out="f32")) <= 1e-5
+    with pytest.raises(ValueError):
+        ops.gqa_attention(q, k, v, attn_bias=np.zeros((3, 200), np.float32))
+
+
+def test_bias_executor_operand(lane):
+    from tessera_amd import executors as ex
+    q, k, v = (np.asarray(_f32(x), np.float16) for x in _qkv(1, 2, 2, 130, 130, 64, 11, "f16"))
+    bias = np.random.default_rng(3).standard_normal((130, 130)).astype(np.float32)
+    art = ex.make_artifact("tessera.flash_attn", ["q", "k", "v", "b"], ["q", "k", "v", "b"], "gfx950_flash_attn",
+                           kwargs={"causal": True})
+    res = ex.launch(art, (q, k, v, bias))
+    assert res["ok"], res
+    ref, _ = orc.flash_attn_dense(q.astype(np.float32), k.astype(np.float32), v.astype(np.float32), causal=True,
+                                  bias=np.broadcast_to(bias, (1, 2, 130, 130)))
+    assert orc.max_rel_err(res["output"], ref) <= TOL
+    bad = ex.launch(art, (q, k, v, np.zeros((7, 130), np.float32)))
+    assert bad["runtime_status"] == "invalid_artifact"

@@ -46,8 +46,9 @@ def test_launch_flash_attn_executor(lane):
     bad = ex.make_artifact("tessera.flash_attn", ["q", "k", "v"], ["q", "k", "v"], "gfx950_flash_attn",
                            kwargs={"window": -16})
     assert ex.launch(bad, (q, k, v))["runtime_status"] == "invalid_artifact"
-    bias = ex.make_artifact("tessera.flash_attn", ["q", "k", "v", "b"], ["q", "k", "v", "b"], "gfx950_flash_attn")
-    assert ex.launch(bias, (q, k, v, np.zeros((130, 130), np.float32)))["runtime_status"] == "invalid_artifact"
+    drop = ex.make_artifact("tessera.flash_attn", ["q", "k", "v"], ["q", "k", "v"], "gfx950_flash_attn",
+                            kwargs={"dropout_p": 0.1})
+    assert ex.launch(drop, (q, k, v))["runtime_status"] == "invalid_artifact"
 
 
 def test_launch_moe_transport_executor(lane):

@@ -83,3 +83,25 @@ def test_window_and_softcap_match_the_reference_kernel():
         ro, rl = co.ref_flash_attn_lse(q, k, v, 1.0 / np.sqrt(D), causal, window, cap)
         assert orc.max_rel_err(o, ro) <= 1e-5
         assert np.max(np.abs(lse - rl)) <= 1e-5
+
+
+def test_additive_bias_matches_the_reference_kernel():
+    """Additive attention bias of the numpy oracle (alone, with the causal mask, a
+    window and a soft cap, where it is added after the cap) against the reference's
+    compiled CPU kernel."""
+    if co.ref() is None:
+        pytest.skip("compiled reference twins unavailable on this host")
+    rng = np.random.default_rng(13)
+    for (B, Hq, Hkv, Sq, Sk, D, causal, window, cap) in [
+            (1, 2, 1, 40, 40, 16, False, 0, 0.0), (2, 4, 2, 24, 50, 16, True, 0, 0.0),
+            (1, 2, 2, 33, 33, 8, True, 10, 0.0), (1, 2, 2, 31, 47, 16, True, 0, 4.0)]:
+        q = rng.standard_normal((B, Hq, Sq, D)).astype(np.float32)
+        k = rng.standard_normal((B, Hkv, Sk, D)).astype(np.float32)
+        v = rng.standard_normal((B, Hkv, Sk, D)).astype(np.float32)
+        bias = (rng.standard_normal((B, Hq, Sq, Sk)) * 2).astype(np.float32)
+        o, lse = orc.flash_attn_dense(q, k, v, causal=causal, window=window, softcap=cap, bias=bias)
+        ro, rl = co.ref_flash_attn_lse(q, k, v, 1.0 / np.sqrt(D), causal, window, cap, bias=bias)
+        assert orc.max_rel_err(o, ro) <= 1e-5
+        assert np.max(np.abs(lse - rl)) <= 1e-5
+        # a dropped bias would be seen: the biased result differs from the plain one
+        assert orc.max_rel_err(o, orc.flash_attn_dense(q, k, v, causal=causal, window=window, softcap=cap)[0]) > 1e-2
