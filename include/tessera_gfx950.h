@@ -166,6 +166,11 @@ int tessera_gfx950_gemm_schedule(int M, int N, int K, int batch, int elem_bytes,
  * launches between HIP events, cross-checked against wall clock
  * (tessera_rocm_gemm.cpp:551-667).  *avg_ms = mean per-launch ms. */
 int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_ms);
+/* The same loop cycling over `weights` (1..64) distinct B matrices: a weight matrix
+ * that would fit the memory-side cache is then streamed from HBM on every launch,
+ * as the layers of a decode step are.  No counterpart in the reference. */
+int tessera_gfx950_gemm_bf16_bench_rotating(int M, int N, int K, int iters, int weights,
+                                            double* avg_ms);
 /* 0 = device events, 1 = host wall clock, -1 = no measurement yet
  * (tessera_rocm_bench_last_timer_source, tessera_rocm_gemm.cpp:567-580). */
 int tessera_gfx950_bench_last_timer_source(void);

@@ -203,8 +203,9 @@ int tessera_gfx950_gemm_schedule(int M, int N, int K, int batch, int elem_bytes,
   if (bad_dims(batch, M, N, K) || !tile_m || !tile_n || !tile_k || !split_k) return kBadShape;
   if (elem_bytes == 2) {
     const Gemm16Schedule sch = select_gemm16_schedule(M, N, K, batch);
-    *tile_m = *tile_n = sch.tile;
-    *tile_k = G16_BK;
+    *tile_m = sch.skinny ? 32 : sch.tile;
+    *tile_n = sch.tile;
+    *tile_k = sch.skinny ? 32 : G16_BK;
     *split_k = sch.split_k;
     return kOk;
   }
@@ -220,20 +221,25 @@ int tessera_gfx950_gemm_schedule(int M, int N, int K, int batch, int elem_bytes,
 // Kernel-only timing on resident buffers.  The device-event figure is accepted
 // only when it lies within 0.5x..2x of the wall clock around the same launches;
 // otherwise the wall-clock figure is reported and the source says so.
-int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_ms) {
+// `weights` > 1 cycles the launches over that many distinct B matrices, so that a
+// weight matrix smaller than the 256 MB memory-side cache is still read from HBM.
+static int bench_gemm_bf16(int M, int N, int K, int iters, int weights, double* avg_ms) {
   g_last_timer_source = -1;
-  if (bad_dims(1, M, N, K) || iters <= 0 || !avg_ms) return kBadShape;
+  if (bad_dims(1, M, N, K) || iters <= 0 || weights <= 0 || weights > 64 || !avg_ms) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
   DeviceScope scope;
   const size_t a_bytes = (size_t)M * K * 2, b_bytes = (size_t)K * N * 2, d_bytes = (size_t)M * N * 2;
   void* dA = scope.alloc(a_bytes);
-  void* dB = scope.alloc(b_bytes);
+  void* dBs[64];
+  for (int i = 0; i < weights; ++i) dBs[i] = scope.alloc(b_bytes);
   void* dD = scope.alloc(d_bytes);
   if (scope.failed()) return kDeviceFailed;
   // 0x3c00 pattern bytes: finite, non-trivial bf16 values.
-  if (hipMemset(dA, 0x3c, a_bytes) != hipSuccess || hipMemset(dB, 0x3c, b_bytes) != hipSuccess) return kDeviceFailed;
+  if (hipMemset(dA, 0x3c, a_bytes) != hipSuccess) return kDeviceFailed;
+  for (int i = 0; i < weights; ++i)
+    if (hipMemset(dBs[i], 0x3c, b_bytes) != hipSuccess) return kDeviceFailed;
   for (int w = 0; w < 5; ++w) {
-    int rc = gemm16_dev<BF16, EPI_STORE16>(dA, dB, dD, 1, M, N, K, nullptr);
+    int rc = gemm16_dev<BF16, EPI_STORE16>(dA, dBs[w % weights], dD, 1, M, N, K, nullptr);
     if (rc != kOk) return rc;
   }
   if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
@@ -243,7 +249,8 @@ int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_m
   int rc = kOk;
   const auto t0 = std::chrono::steady_clock::now();
   (void)hipEventRecord(e0, nullptr);
-  for (int it = 0; it < iters && rc == kOk; ++it) rc = gemm16_dev<BF16, EPI_STORE16>(dA, dB, dD, 1, M, N, K, nullptr);
+  for (int it = 0; it < iters && rc == kOk; ++it)
+    rc = gemm16_dev<BF16, EPI_STORE16>(dA, dBs[it % weights], dD, 1, M, N, K, nullptr);
   (void)hipEventRecord(e1, nullptr);
   const bool synced = hipEventSynchronize(e1) == hipSuccess;
   const double wall_ms =
@@ -258,6 +265,13 @@ int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_m
   g_last_timer_source = ev_ok ? 0 : 1;
   *avg_ms = (ev_ok ? (double)ev_ms : wall_ms) / iters;
   return kOk;
+}
+
+int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_ms) {
+  return bench_gemm_bf16(M, N, K, iters, 1, avg_ms);
+}
+int tessera_gfx950_gemm_bf16_bench_rotating(int M, int N, int K, int iters, int weights, double* avg_ms) {
+  return bench_gemm_bf16(M, N, K, iters, weights, avg_ms);
 }
 
 int tessera_gfx950_bench_last_timer_source(void) { return g_last_timer_source; }

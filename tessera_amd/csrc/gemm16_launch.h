@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <mutex>
 #include "gemm16.h"
+#include "gemm16_skinny.h"
 #include "host_util.h"
 
 namespace tsr950 {
@@ -99,10 +100,17 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restr
   if (i >= (long)M * nq) return;
   const int m = (int)(i / nq), n = (int)(i % nq) * 4;
   const size_t mn = (size_t)M * N;
-  float4 acc = *reinterpret_cast<const float4*>(ws + (size_t)m * N + n);
-  for (int z = 1; z < splits; ++z) {
-    const float4 v = *reinterpret_cast<const float4*>(ws + z * mn + (size_t)m * N + n);
-    acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+  // (the partials of four splits are fetched together: they were written by other
+  // XCDs, so every one of these loads pays a trip to memory)
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int z0 = 0; z0 < splits; z0 += 4) {
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      v[u] = z0 + u < splits ? *reinterpret_cast<const float4*>(ws + (z0 + u) * mn + (size_t)m * N + n)
+                             : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) { acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w; }
   }
   if (bias) {
     const float4 bv = *reinterpret_cast<const float4*>(bias + n);
@@ -128,11 +136,23 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restr
 struct Gemm16Schedule {
   int tile;      // square workgroup tile edge: 256, 128 or 64
   int split_k;   // number of K splits (1 = none)
+  bool skinny;   // M <= 8: the streaming kernel (32 x 64 workgroup tile, K slices of 32)
 };
+#ifndef TSR_SKINNY_MAX_M
+#define TSR_SKINNY_MAX_M 8
+#endif
+constexpr int kSkinnyMaxM = TSR_SKINNY_MAX_M;
 inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
+  if (batch == 1 && M <= kSkinnyMaxM && K % 32 == 0 && K >= 512) {
+    // one workgroup per 64-column strip and K split; about one workgroup per CU, and
+    // at least two 32-row slices for each of a workgroup's 8 waves
+    const int strips = ceil_div(N, 64);
+    int splits = std::max(1, std::min((256 + strips / 2) / strips, K / 512));
+    return {64, splits, true};
+  }
   const long tiles256 = (long)ceil_div(M, 256) * ceil_div(N, 256) * batch;
   const long tiles128 = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch;
-  if (tiles256 >= 192) return {256, 1};
+  if (tiles256 >= 192) return {256, 1, false};
   const bool t128 = tiles128 >= 192 || (M > 64 && N >= 128);
   int splits = 1;
   if (batch == 1) {
@@ -140,7 +160,23 @@ inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
     splits = (int)std::max<long>(1, std::min<long>((768 + tiles - 1) / tiles, K / 512));
     while (splits > 1 && K % (splits * G16_BK) != 0) --splits;
   }
-  return {t128 ? 128 : 64, splits};
+  return {t128 ? 128 : 64, splits, false};
+}
+
+template <class T, int EPI>
+int launch_gemm16_skinny(const Gemm16Params& p, int kps, int splits, hipStream_t s) {
+  constexpr int MI = 1, NW = 8, NJ = 2, KS = 2;
+  auto kern = gemm16_skinny_kernel<T, MI, NW, NJ, KS, EPI>;
+  constexpr int lds = skinny_lds_bytes<MI, NW, NJ, KS>();
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  });
+  if (attr_err != hipSuccess) return kDeviceFailed;
+  hipLaunchKernelGGL(kern, dim3(ceil_div(p.N, 32 * NJ), splits), dim3(NW * 64), lds, s, p, kps);
+  return launch_status();
 }
 
 // Dense / batched.  p.groups = batch count (>= 1).
@@ -161,17 +197,15 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
   const Gemm16Schedule sch = select_gemm16_schedule(p.M, p.N, p.K, p.groups);
   if (sch.tile == 256) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false>(p, s);
   const bool t128 = sch.tile == 128;
+  if (sch.skinny && sch.split_k == 1) return launch_gemm16_skinny<T, EPI>(p, p.K, 1, s);
   // Every K split is one "batch" of the same kernel writing f32 partials, summed in
   // split order by a second kernel, so the result does not depend on scheduling.
   {
     const int splits = sch.split_k;
     if (splits > 1) {
-      float* ws = nullptr;
       const size_t mn = (size_t)p.M * p.N;
-      if (hipMallocAsync(reinterpret_cast<void**>(&ws), mn * splits * sizeof(float), s) != hipSuccess) {
-        (void)hipGetLastError();
-        return kDeviceFailed;
-      }
+      float* ws = static_cast<float*>(stream_workspace(s, mn * splits * sizeof(float)));
+      if (!ws) return kDeviceFailed;
       Gemm16Params q = p;
       q.K = p.K / splits;
       q.groups = splits;
@@ -182,15 +216,21 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
       q.act = ACT_NONE;
       q.ldd = p.N;
       q.strideD = (long)mn;
-      int rc = t128 ? launch_gemm16_tile<T, 128, 128, 2, 2, EPI_F32, false>(q, s)
-                    : launch_gemm16_tile<T, 64, 64, 2, 2, EPI_F32, false>(q, s);
+      int rc;
+      if (sch.skinny) {
+        // the skinny kernel takes the whole problem and splits K by blockIdx.y itself
+        q.K = p.K;
+        rc = launch_gemm16_skinny<T, EPI_F32>(q, ceil_div(ceil_div(p.K, splits), 32) * 32, splits, s);
+      } else {
+        rc = t128 ? launch_gemm16_tile<T, 128, 128, 2, 2, EPI_F32, false>(q, s)
+                  : launch_gemm16_tile<T, 64, 64, 2, 2, EPI_F32, false>(q, s);
+      }
       if (rc == kOk) {
         const long quads = (long)p.M * (p.N / 4);
         hipLaunchKernelGGL((splitk_reduce_kernel<T, EPI>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s,
                            ws, p.D, p.M, p.N, p.ldd, splits, p.bias, p.act);
         rc = launch_status();
       }
-      if (hipFreeAsync(ws, s) != hipSuccess) { (void)hipGetLastError(); rc = rc == kOk ? kDeviceFailed : rc; }
       return rc;
     }
   }

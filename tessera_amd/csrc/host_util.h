@@ -43,6 +43,12 @@ class DeviceScope {
   bool failed_ = false;
 };
 
+// Device scratch for kernels that need it between two launches of one call (split-K
+// partials): one buffer per (device, stream), grown on demand and kept until the
+// process ends.  Calls on one stream run in order, so they can share the buffer;
+// calls on different streams get different buffers.  Returns null on failure.
+void* stream_workspace(hipStream_t s, size_t bytes);
+
 inline int finish(hipError_t e) { return e == hipSuccess ? kOk : kDeviceFailed; }
 
 // Launch status of the kernels just enqueued on `s` (does not synchronise).

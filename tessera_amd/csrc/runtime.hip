@@ -1,7 +1,9 @@
 // Device management half of the C ABI: probe, raw buffers, event timers.
 #include <atomic>
 #include <cstring>
+#include <map>
 #include <mutex>
+#include <utility>
 #include "../../include/tessera_gfx950.h"
 #include "host_util.h"
 
@@ -20,6 +22,27 @@ int probe_device() {
     cached = kOk;
   });
   return cached;
+}
+
+void* stream_workspace(hipStream_t s, size_t bytes) {
+  struct Slot { void* ptr; size_t bytes; };
+  static std::mutex mu;
+  static std::map<std::pair<int, hipStream_t>, Slot> slots;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  std::lock_guard<std::mutex> lock(mu);
+  Slot& slot = slots[{dev, s}];
+  if (slot.bytes >= bytes && slot.ptr) return slot.ptr;
+  if (slot.ptr) {
+    // work already queued on the stream may still use the old buffer
+    if (hipStreamSynchronize(s) != hipSuccess || hipFree(slot.ptr) != hipSuccess) (void)hipGetLastError();
+    slot = Slot{nullptr, 0};
+  }
+  const size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+  void* p = nullptr;
+  if (hipMalloc(&p, want) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  slot = Slot{p, want};
+  return p;
 }
 
 struct Timer {

@@ -25,7 +25,7 @@ _DTYPES = {
 }
 _INSTRUCTION_TILE = {"f16": (32, 32, 16), "bf16": (32, 32, 16), "int8": (32, 32, 32), "fp8_e4m3": (32, 32, 64)}
 # accumulators + operand fragments + staging of one wave, from the assembler's report
-_VGPRS = {256: 456, 128: 170, 64: 96}
+_VGPRS = {256: 456, 128: 170, 64: 96, 32: 137}
 
 
 @dataclass(frozen=True)
@@ -90,8 +90,9 @@ def select_gfx950_gemm_schedule(m: int, n: int, k: int, *, dtype: str = "bf16", 
         arch="gfx950", dtype=name, instruction_tile=inst,
         macro_tile=(tm.value // inst[0], tn.value // inst[1]),
         workgroup_tile=(tm.value, tn.value, tk.value),
-        waves_per_cu=4, pipeline_stages=2,
-        lds_layout="A xor-swizzled 16B chunks; B natural [k][n] + transposing ds_read",
+        waves_per_cu=8 if tm.value == 32 else 4, pipeline_stages=2,
+        lds_layout=("A from global in operand order; B wave-private [k][n] slices + transposing ds_read"
+                    if tm.value == 32 else "A xor-swizzled 16B chunks; B natural [k][n] + transposing ds_read"),
         ownership="wave", vgpr_estimate=_VGPRS[tm.value], split_k=sk.value,
         source="tessera_gfx950_gemm_schedule (the launcher's own decision)")
 

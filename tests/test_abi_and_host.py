@@ -238,8 +238,11 @@ def test_gemm_schedule_query_needs_no_device():
     big = sel(8192, 8192, 8192, dtype="bf16")
     assert big.workgroup_tile == (256, 256, 64) and big.macro_tile == (8, 8) and big.split_k == 1
     assert big.instruction_tile == (32, 32, 16) and big.target_ir_attrs()["schedule_arch"] == "gfx950"
-    dec = sel(16, 8192, 8192, dtype="bf16")
-    assert dec.workgroup_tile[:2] == (64, 64) and dec.split_k > 1 and 8192 % (dec.split_k * 64) == 0
+    dec = sel(4, 8192, 8192, dtype="bf16")                              # a few rows: the streaming kernel
+    assert dec.workgroup_tile == (32, 64, 32) and dec.split_k == 2 and dec.waves_per_cu == 8
+    assert sel(4, 32768, 8192).split_k == 1                             # enough column strips to fill the chip
+    mid = sel(64, 8192, 8192, dtype="bf16")
+    assert mid.workgroup_tile[:2] == (64, 64) and mid.split_k > 1 and 8192 % (mid.split_k * 64) == 0
     assert sel(128, 8192, 8192).workgroup_tile[:2] == (128, 128)
     assert sel(128, 256, 64, batch=4).split_k == 1                      # batched products never split K
     q = sel(4096, 8192, 8192, dtype="int8")

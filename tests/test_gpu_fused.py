@@ -24,8 +24,10 @@ def _f32(x):
     return x.to_float32() if isinstance(x, b16.BF16Array) else np.asarray(x, np.float32)
 
 
-# tile kernel (aligned), split-K decode shape, ragged generic path
-SHAPES = [(512, 768, 256), (300, 520, 136), (16, 1024, 4096), (8, 16, 12), (37, 29, 50)]
+# tile kernel (aligned), split-K decode shape, single-split decode shape (epilogue in
+# the streaming kernel itself), ragged generic path
+SHAPES = [(512, 768, 256), (300, 520, 136), (16, 1024, 4096), (6, 16384, 512), (8, 1024, 2048), (8, 16, 12),
+          (37, 29, 50)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)

@@ -115,6 +115,30 @@ def test_decode_shapes(lane):
         assert np.array_equal(ops.gemm(ab, bb, out="f32"), got)
 
 
+# The streaming kernel for M <= 8 (K % 32 == 0, K >= 512): column-strip tails, a
+# K range that does not divide evenly over the splits, one split and many.
+SKINNY = [(1, 64, 512), (7, 72, 1056), (8, 1000, 2048), (4, 8192, 512), (5, 16384, 544),
+          (3, 4096, 8192), (8, 24, 4096), (2, 2048, 7200)]
+
+
+@pytest.mark.parametrize("M,N,K", SKINNY)
+@pytest.mark.parametrize("st", ["bf16", "f16"])
+def test_skinny_gemm(lane, M, N, K, st):
+    from tessera_amd.schedule import select_gfx950_gemm_schedule as sel
+    assert sel(M, N, K).workgroup_tile == (32, 64, 32)                  # this shape takes the streaming kernel
+    A = _rand((M, K), 1.0, 21)
+    B = _rand((K, N), 1.0 / np.sqrt(K), 22)
+    ref = orc.gemm_f64(A, B, st)
+    a = b16.from_float32(A) if st == "bf16" else A.astype(np.float16)
+    b = b16.from_float32(B) if st == "bf16" else B.astype(np.float16)
+    got = ops.gemm(a, b, out="f32")
+    assert orc.max_rel_err(got, ref) <= 1e-5
+    stored = ops.gemm(a, b)
+    sf = stored.to_float32() if st == "bf16" else stored.astype(np.float32)
+    assert np.array_equal(sf, orc.round_to_storage(got, st))
+    assert np.array_equal(ops.gemm(a, b, out="f32"), got)               # fixed summation order
+
+
 def test_full_size_bf16_gemm_properties(lane):
     """8192^3 is too large for a CPU product inside the test budget; check
     size-independent properties instead: linearity in A and agreement with
