@@ -138,10 +138,8 @@ struct Gemm16Schedule {
   int split_k;   // number of K splits (1 = none)
   bool skinny;   // M <= 8: the streaming kernel (32 x 64 workgroup tile, K slices of 32)
 };
-#ifndef TSR_SKINNY_MAX_M
-#define TSR_SKINNY_MAX_M 8
-#endif
-constexpr int kSkinnyMaxM = TSR_SKINNY_MAX_M;
+constexpr int kSkinnyMaxM = 8;
+constexpr long kSplitTargetWgs = 768;
 inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
   if (batch == 1 && M <= kSkinnyMaxM && K % 32 == 0 && K >= 512) {
     // one workgroup per 64-column strip and K split; about one workgroup per CU, and
@@ -157,7 +155,10 @@ inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
   int splits = 1;
   if (batch == 1) {
     const long tiles = t128 ? tiles128 : (long)ceil_div(M, 64) * ceil_div(N, 64);
-    splits = (int)std::max<long>(1, std::min<long>((768 + tiles - 1) / tiles, K / 512));
+    splits = (int)std::max<long>(1, std::min<long>((kSplitTargetWgs + tiles - 1) / tiles, K / 512));
+    // the f32 partials are written and read once per split (8 M N splits bytes against
+    // 2 K N bytes of B): beyond two splits keep that under about 0.4 of the weight traffic
+    splits = (int)std::min<long>(splits, std::max<long>(2, K / (10L * M)));
     while (splits > 1 && K % (splits * G16_BK) != 0) --splits;
   }
   return {t128 ? 128 : 64, splits, false};
