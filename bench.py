@@ -39,8 +39,22 @@ PEAK_HBM_GBS = 8000.0
 TRAFFIC_BYTES_GEMM_BF16_8192 = 1.7497e9
 
 
+RAMP_SECONDS = 0.1
+
+
 def _timed(lane, launch, steps, warmup):
-    """(wall ms/step, event ms/step) for `steps` launches after `warmup`."""
+    """(wall ms/step, event ms/step) for `steps` launches after `warmup`.
+
+    After the host-side data preparation the GPU has idled and its clocks ramp back
+    up over the first tens of milliseconds of load (measured: the first 25 launches
+    of the headline GEMM run 3-70 % slower than the steady state).  The untimed
+    warm-up therefore first keeps the kernel running for RAMP_SECONDS, then does the
+    `warmup` steps; the timed region is exactly `steps` launches."""
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < RAMP_SECONDS:
+        for _ in range(4):
+            launch()
+        lane.synchronize()
     for _ in range(warmup):
         launch()
     lane.synchronize()

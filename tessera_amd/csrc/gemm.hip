@@ -238,9 +238,13 @@ static int bench_gemm_bf16(int M, int N, int K, int iters, int weights, double* 
   if (hipMemset(dA, 0x3c, a_bytes) != hipSuccess) return kDeviceFailed;
   for (int i = 0; i < weights; ++i)
     if (hipMemset(dBs[i], 0x3c, b_bytes) != hipSuccess) return kDeviceFailed;
-  for (int w = 0; w < 5; ++w) {
+  // Warm-up: at least five launches, and at least 60 ms of them, so that the clocks
+  // (which ramp up over tens of milliseconds after idle) are steady when timing starts.
+  const auto warm0 = std::chrono::steady_clock::now();
+  for (int w = 0; w < 5 || std::chrono::steady_clock::now() - warm0 < std::chrono::milliseconds(60); ++w) {
     int rc = gemm16_dev<BF16, EPI_STORE16>(dA, dBs[w % weights], dD, 1, M, N, K, nullptr);
     if (rc != kOk) return rc;
+    if ((w & 15) == 15 && hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
   }
   if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
   hipEvent_t e0, e1;
