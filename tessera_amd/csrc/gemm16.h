@@ -36,6 +36,7 @@ enum GemmEpilogue : int {
   EPI_STORE16 = 1,    // D in the storage dtype (RNE)
   EPI_SWIGLU16 = 2,   // D = storage(silu(storage(gate)) * storage(up)); B2 holds "up"
   EPI_GATED_F32 = 3,  // D f32 = act(gate) * up, no intermediate rounding; B2 holds "up"
+  EPI_F32_FUSED = 4,  // D f32 = act(acc + bias[n]); tile kernels only (p.bias / p.act)
 };
 
 // Pointwise activations of the fused epilogue (the reference's matmul-epilogue
@@ -45,6 +46,18 @@ enum Activation : int { ACT_NONE = 0, ACT_RELU = 1, ACT_GELU = 2, ACT_SILU = 3, 
 // All of them but relu are a logistic function of a linear or cubic argument:
 //   silu v sig(v); sigmoid sig(v); tanh 2 sig(2v) - 1;
 //   gelu (tanh form, argument clamped to +-30) 0.5 v (1 + tanh t) = v sig(2t).
+template <int ACT>
+__device__ __forceinline__ float activate_as(float v) {
+  if constexpr (ACT == ACT_NONE) return v;
+  if constexpr (ACT == ACT_RELU) return fmaxf(v, 0.f);
+  float x = v;
+  if constexpr (ACT == ACT_GELU) x = 2.f * fminf(fmaxf(0.7978845608028654f * (v + 0.044715f * v * v * v), -30.f), 30.f);
+  if constexpr (ACT == ACT_TANH) x = 2.f * v;
+  const float sg = 1.0f / (1.0f + __expf(-x));
+  if constexpr (ACT == ACT_SIGMOID) return sg;
+  if constexpr (ACT == ACT_TANH) return 2.f * sg - 1.f;
+  return v * sg;
+}
 __device__ __forceinline__ float activate(float v, int act) {
   if (act == ACT_NONE) return v;
   if (act == ACT_RELU) return fmaxf(v, 0.f);
@@ -138,7 +151,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   const uint16_t* Bb = p.B;
   const uint16_t* B2b = p.B2;
   char* Db = (char*)p.D;
-  constexpr int DSZ = (EPI == EPI_F32 || EPI == EPI_GATED_F32) ? 4 : 2;
+  constexpr int DSZ = (EPI == EPI_F32 || EPI == EPI_GATED_F32 || EPI == EPI_F32_FUSED) ? 4 : 2;
   if constexpr (GROUPED) {
     // 1-D grid over the real tiles of all groups, ordered group-major, then n tile,
     // then m tile.  Workgroup ids are dealt to the 8 XCDs round-robin, so XCD j takes
@@ -396,60 +409,118 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   kstep(kt, false_type{}, mode0{}, mode0{});
 
   // ---- epilogue -------------------------------------------------------------
-  // acc[i][j][r]: row m = 32i + l32, col n = 32j + 8*(r/4) + 4*lh + (r%4).
+  // acc[i][j][r]: row m = 32i + l32, col n = 32j + 8*(r/4) + 4*lh + (r%4): a lane owns
+  // runs of four columns of 32 different rows.  Stored like that, every store
+  // instruction would touch 32 cache lines with 16 bytes each, and the output write
+  // would cost a tenth of a long-K product and half of a short-K one.  The wave
+  // therefore stages its tile through its share of the (now free) LDS and writes
+  // whole row segments: 16 bytes per lane, consecutive lanes along a row.
   constexpr int NJ_OUT = SWIGLU ? NJ / 2 : NJ;
-  const bool fused = p.bias != nullptr || p.act != ACT_NONE;
+  constexpr int ROWB = NJ_OUT * 32 * DSZ;              // bytes of one row of the wave's output tile
+  constexpr int PITCH = ROWB + 16;
+  constexpr int WAVE_LDS = S::kBytes / (WM * WN);
+  constexpr int IB_FIT = WAVE_LDS / (32 * PITCH);      // 32-row blocks that fit the wave's share
+  constexpr int IB = IB_FIT >= MI ? MI : (IB_FIT >= 2 ? 2 : 1);
+  static_assert(IB_FIT >= 1 && MI % IB == 0, "epilogue staging does not fit");
+  constexpr int LPR = ROWB / 16;                       // lanes per row
+  constexpr int RPI = 64 / LPR;                        // rows per store instruction
+  static_assert(LPR <= 64 && (IB * 32) % RPI == 0, "epilogue row mapping");
+  // every wave has consumed its last fragments once its MFMAs are issued: past this
+  // barrier nobody reads the operand tiles any more
+  __syncthreads();
+  char* stg = smem + wave * WAVE_LDS;
+  const int nw0 = n_begin + (SWIGLU ? 0 : wn * TN);    // first output column of the wave
+  const int st_row = lane / LPR, st_chunk = lane % LPR;
+  const int st_n = nw0 + st_chunk * (16 / DSZ);
+  // The activation and the presence of a bias are compile-time here: one compact,
+  // straight-line instance runs per launch.  (With the choice made per element at run
+  // time the epilogue was 23,000 instructions that the plain path hopped through,
+  // missing the instruction cache at every hop: 12 us per 256 x 256 tile.)
+  auto emit = [&](auto act_c, auto bias_c) __attribute__((always_inline)) {
+    constexpr int ACT = decltype(act_c)::value;
+    constexpr bool HAS_BIAS = decltype(bias_c)::value;
 #pragma unroll
-  for (int i = 0; i < MI; ++i) {
-    const int m = m_begin + wm * TM + i * 32 + l32;
-    if (m >= m_end) continue;
-    char* drow = Db + (long)m * p.ldd * DSZ;
+    for (int i0 = 0; i0 < MI; i0 += IB) {
 #pragma unroll
-    for (int j = 0; j < NJ_OUT; ++j) {
+      for (int ii = 0; ii < IB; ++ii) {
+        const int i = i0 + ii;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n_begin + (SWIGLU ? 0 : wn * TN) + j * 32 + q * 8 + lh * 4;
-        if (n >= p.N) continue;                  // N % 8 == 0 on this path: all-or-nothing per run of 4
-        float v0 = acc[i][j][q * 4 + 0], v1 = acc[i][j][q * 4 + 1];
-        float v2 = acc[i][j][q * 4 + 2], v3 = acc[i][j][q * 4 + 3];
-        if constexpr (EPI == EPI_F32 || EPI == EPI_STORE16) {
-          if (fused) {
-            if (p.bias) {
-              const float4 bv = *reinterpret_cast<const float4*>(p.bias + n);
-              v0 += bv.x; v1 += bv.y; v2 += bv.z; v3 += bv.w;
+        for (int j = 0; j < NJ_OUT; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int n = nw0 + j * 32 + q * 8 + lh * 4;
+            float v0 = acc[i][j][q * 4 + 0], v1 = acc[i][j][q * 4 + 1];
+            float v2 = acc[i][j][q * 4 + 2], v3 = acc[i][j][q * 4 + 3];
+            if constexpr (EPI == EPI_F32_FUSED) {
+              if constexpr (HAS_BIAS) {
+                // (a column past N is never stored; its bias read stays in range)
+                const float4 bv = *reinterpret_cast<const float4*>(p.bias + (n < p.N ? n : 0));
+                v0 += bv.x; v1 += bv.y; v2 += bv.z; v3 += bv.w;
+              }
+              v0 = activate_as<ACT>(v0); v1 = activate_as<ACT>(v1);
+              v2 = activate_as<ACT>(v2); v3 = activate_as<ACT>(v3);
             }
-            v0 = activate(v0, p.act); v1 = activate(v1, p.act);
-            v2 = activate(v2, p.act); v3 = activate(v3, p.act);
-          }
-        }
-        if constexpr (EPI == EPI_GATED_F32) {
-          const f32x16& u = acc[i][j + NJ / 2];
-          v0 = activate(v0, p.act) * u[q * 4 + 0]; v1 = activate(v1, p.act) * u[q * 4 + 1];
-          v2 = activate(v2, p.act) * u[q * 4 + 2]; v3 = activate(v3, p.act) * u[q * 4 + 3];
-        }
-        if constexpr (EPI == EPI_F32 || EPI == EPI_GATED_F32) {
-          *reinterpret_cast<float4*>(drow + (long)n * 4) = make_float4(v0, v1, v2, v3);
-        } else {
-          if constexpr (EPI == EPI_SWIGLU16) {
-            const f32x16& u = acc[i][j + NJ / 2];
-            float g[4] = {v0, v1, v2, v3};
-            float o[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              // every intermediate lives on the storage grid, as in the reference
-              const float gs = from_storage<T>(to_storage<T>(g[e]));
-              const float us = from_storage<T>(to_storage<T>(u[q * 4 + e]));
-              o[e] = (gs / (1.0f + __expf(-gs))) * us;
+            if constexpr (EPI == EPI_GATED_F32) {
+              const f32x16& u = acc[i][j + NJ / 2];
+              v0 = activate_as<ACT>(v0) * u[q * 4 + 0]; v1 = activate_as<ACT>(v1) * u[q * 4 + 1];
+              v2 = activate_as<ACT>(v2) * u[q * 4 + 2]; v3 = activate_as<ACT>(v3) * u[q * 4 + 3];
             }
-            v0 = o[0]; v1 = o[1]; v2 = o[2]; v3 = o[3];
+            char* dst = stg + (ii * 32 + l32) * PITCH + (j * 32 + q * 8 + lh * 4) * DSZ;
+            if constexpr (DSZ == 4) {
+              *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
+            } else {
+              if constexpr (EPI == EPI_SWIGLU16) {
+                const f32x16& u = acc[i][j + NJ / 2];
+                float g[4] = {v0, v1, v2, v3};
+                float o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  // every intermediate lives on the storage grid, as in the reference
+                  const float gs = from_storage<T>(to_storage<T>(g[e]));
+                  const float us = from_storage<T>(to_storage<T>(u[q * 4 + e]));
+                  o[e] = (gs / (1.0f + __expf(-gs))) * us;
+                }
+                v0 = o[0]; v1 = o[1]; v2 = o[2]; v3 = o[3];
+              }
+              uint2 pk;
+              pk.x = pack2<T>(v0, v1);
+              pk.y = pack2<T>(v2, v3);
+              *reinterpret_cast<uint2*>(dst) = pk;
+            }
           }
-          uint2 pk;
-          pk.x = pack2<T>(v0, v1);
-          pk.y = pack2<T>(v2, v3);
-          *reinterpret_cast<uint2*>(drow + (long)n * 2) = pk;
         }
       }
+      __builtin_amdgcn_wave_barrier();                 // the wave's LDS operations run in order
+#pragma unroll
+      for (int it = 0; it < IB * 32 / RPI; ++it) {
+        const int row = it * RPI + st_row;
+        const uint4 v = lds_read_b128(stg, row * PITCH + st_chunk * 16);
+        const int m = m_begin + wm * TM + i0 * 32 + row;
+        // N % 8 == 0 on this path: a 16-byte chunk is inside or outside as a whole
+        if (m < m_end && st_n < p.N)
+          *reinterpret_cast<uint4*>(Db + ((long)m * p.ldd + st_n) * DSZ) = v;
+      }
+      __builtin_amdgcn_wave_barrier();
     }
+  };
+  using A0 = std::integral_constant<int, ACT_NONE>;
+  auto by_activation = [&](auto bias_c) __attribute__((always_inline)) {
+    switch (p.act) {
+      case ACT_RELU: emit(std::integral_constant<int, ACT_RELU>{}, bias_c); break;
+      case ACT_GELU: emit(std::integral_constant<int, ACT_GELU>{}, bias_c); break;
+      case ACT_SILU: emit(std::integral_constant<int, ACT_SILU>{}, bias_c); break;
+      case ACT_SIGMOID: emit(std::integral_constant<int, ACT_SIGMOID>{}, bias_c); break;
+      case ACT_TANH: emit(std::integral_constant<int, ACT_TANH>{}, bias_c); break;
+      default: emit(A0{}, bias_c); break;
+    }
+  };
+  if constexpr (EPI == EPI_GATED_F32) {
+    by_activation(false_type{});
+  } else if constexpr (EPI == EPI_F32_FUSED) {
+    if (p.bias) by_activation(true_type{});
+    else by_activation(false_type{});
+  } else {
+    emit(A0{}, false_type{});
   }
 }
 

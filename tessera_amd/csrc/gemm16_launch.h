@@ -187,7 +187,7 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
   // (32-bit per-lane byte offsets inside a tile bound the leading dimensions)
   const bool vec = (p.K % 8 == 0) && (p.N % 8 == 0) && (p.lda % 8 == 0) && (p.ldb % 8 == 0) &&
                    (p.lda < (1L << 21)) && (p.ldb < (1L << 21)) &&
-                   ((p.ldd * dsz) % (dsz * 4) == 0) && (p.strideA % 8 == 0) && (p.strideB % 8 == 0) &&
+                   ((p.ldd * dsz) % 16 == 0) && (p.strideA % 8 == 0) && (p.strideB % 8 == 0) &&
                    ((p.strideD * dsz) % 16 == 0) && aligned16(p.A) && aligned16(p.B) && aligned16(p.D) &&
                    (!p.bias || aligned16(p.bias));
   if (!vec) {
@@ -196,7 +196,17 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
     return launch_status();
   }
   const Gemm16Schedule sch = select_gemm16_schedule(p.M, p.N, p.K, p.groups);
-  if (sch.tile == 256) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false>(p, s);
+  // bias / activation: the tile kernels have a separate instantiation for it (f32 out)
+  const bool fused = p.bias != nullptr || p.act != ACT_NONE;
+  if constexpr (EPI != EPI_F32) {
+    if (fused) return kBadShape;
+  }
+  if (sch.tile == 256) {
+    if constexpr (EPI == EPI_F32) {
+      if (fused) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI_F32_FUSED, false>(p, s);
+    }
+    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false>(p, s);
+  }
   const bool t128 = sch.tile == 128;
   if (sch.skinny && sch.split_k == 1) return launch_gemm16_skinny<T, EPI>(p, p.K, 1, s);
   // Every K split is one "batch" of the same kernel writing f32 partials, summed in
@@ -235,6 +245,12 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
       return rc;
     }
   }
+  if constexpr (EPI == EPI_F32) {
+    if (fused) {
+      if (t128) return launch_gemm16_tile<T, 128, 128, 2, 2, EPI_F32_FUSED, false>(p, s);
+      return launch_gemm16_tile<T, 64, 64, 2, 2, EPI_F32_FUSED, false>(p, s);
+    }
+  }
   if (t128) return launch_gemm16_tile<T, 128, 128, 2, 2, EPI, false>(p, s);
   return launch_gemm16_tile<T, 64, 64, 2, 2, EPI, false>(p, s);
 }
@@ -260,7 +276,7 @@ int launch_gemm16_grouped(Gemm16Params p, hipStream_t s) {
   // (32-bit per-lane byte offsets inside a tile bound the leading dimensions)
   const bool vec = (p.K % 8 == 0) && (p.N % 8 == 0) && (p.lda % 8 == 0) && (p.ldb % 8 == 0) &&
                    (p.lda < (1L << 21)) && (p.ldb < (1L << 21)) &&
-                   ((p.ldd * dsz) % (dsz * 4) == 0) && (p.strideB % 8 == 0) && aligned16(p.A) &&
+                   ((p.ldd * dsz) % 16 == 0) && (p.strideB % 8 == 0) && aligned16(p.A) &&
                    aligned16(p.B) && aligned16(p.D) && (EPI != EPI_SWIGLU16 || aligned16(p.B2));
   if (!vec) {
     dim3 block(32, 8), grid(ceil_div(p.N, 32), ceil_div(p.M, 8), 1);
