@@ -158,22 +158,55 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     // the j-th contiguous eighth of that order: the tiles running together on one XCD
     // then belong to one or two experts and share its weight slabs and row tiles in
     // that XCD's L2.  The grid is sized from an upper bound; surplus blocks exit.
-    int total_m = 0;
-    for (int g = 0; g < p.groups; ++g) total_m += (p.offsets[g + 1] - p.offsets[g] + BM - 1) / BM;
-    const int total = total_m * p.tiles_n;
+    // The decode reads all E + 1 offsets.  Walking them with dependent scalar loads
+    // costs microseconds per workgroup, so each wave reads 64 groups per step with one
+    // coalesced load, scans their tile counts across its lanes and finds the group of
+    // its tile with a ballot.
+    auto tiles_of = [&](int g, int& lo, int& hi) -> int {
+      lo = g < p.groups ? p.offsets[g] : 0;
+      hi = g < p.groups ? p.offsets[g + 1] : 0;
+      return ((hi - lo + BM - 1) / BM) * p.tiles_n;
+    };
+    auto wave_scan = [&](int v) -> int {             // inclusive prefix sum over the 64 lanes
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int u = __shfl_up(v, d, 64);
+        if (lane >= d) v += u;
+      }
+      return v;
+    };
+    int total = 0;
+    for (int g0 = 0; g0 < p.groups; g0 += 64) {
+      int lo, hi;
+      total += __shfl(wave_scan(tiles_of(g0 + lane, lo, hi)), 63, 64);
+    }
+    total = __builtin_amdgcn_readfirstlane(total);
     const int per = (total + 7) / 8;
     const int slot = blockIdx.x >> 3;
     const int lin = (blockIdx.x & 7) * per + slot;
     if (slot >= per || lin >= total) return;
-    int e = 0, acc = 0, g_lo = 0, g_hi = 0, mt = 0;
-    for (e = 0; e < p.groups; ++e) {
-      g_lo = p.offsets[e];
-      g_hi = p.offsets[e + 1];
-      mt = (g_hi - g_lo + BM - 1) / BM;
-      if (lin < acc + mt * p.tiles_n) break;
-      acc += mt * p.tiles_n;
+    int e = -1, acc = 0, g_lo = 0, g_hi = 0, mt = 0;
+    for (int g0 = 0, base = 0; g0 < p.groups && e < 0; g0 += 64) {
+      int lo, hi;
+      const int cnt = tiles_of(g0 + lane, lo, hi);
+      const int incl = base + wave_scan(cnt);
+      const unsigned long long hit = __ballot(lin >= incl - cnt && lin < incl);
+      if (hit) {
+        const int src = __ffsll((long long)hit) - 1;
+        e = g0 + src;
+        acc = __shfl(incl - cnt, src, 64);
+        g_lo = __shfl(lo, src, 64);
+        g_hi = __shfl(hi, src, 64);
+        mt = (g_hi - g_lo + BM - 1) / BM;
+      }
+      base = __shfl(incl, 63, 64);
     }
-    if (e >= p.groups) return;
+    if (e < 0) return;
+    e = __builtin_amdgcn_readfirstlane(e);
+    acc = __builtin_amdgcn_readfirstlane(acc);
+    g_lo = __builtin_amdgcn_readfirstlane(g_lo);
+    g_hi = __builtin_amdgcn_readfirstlane(g_hi);
+    mt = __builtin_amdgcn_readfirstlane(mt);
     const int r = lin - acc;
     tn = r / mt;
     tm = r - tn * mt;
