@@ -250,13 +250,14 @@ __global__ __launch_bounds__(1024) void combine_scan_kernel(int32_t* cnt, int T,
   for (int i = lo; i < hi; ++i) sum += cnt[i];
   part[threadIdx.x] = sum;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int i = 0; i < 1024; ++i) { const int v = part[i]; part[i] = run; run += v; }
-    off[T] = run;
+  for (int d = 1; d < 1024; d <<= 1) {               // inclusive scan of the 1024 partial sums
+    const int v = (int)threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+    __syncthreads();
+    part[threadIdx.x] += v;
+    __syncthreads();
   }
-  __syncthreads();
-  int run = part[threadIdx.x];
+  if (threadIdx.x == 1023) off[T] = part[1023];
+  int run = part[threadIdx.x] - sum;
   for (int i = lo; i < hi; ++i) { const int v = cnt[i]; off[i] = run; run += v; cnt[i] = 0; }
 }
 __global__ void combine_fill_kernel(const int32_t* token_of_slot, int S, int T, const int32_t* off, int32_t* cursor,
@@ -274,10 +275,15 @@ __device__ __forceinline__ float add_rounded_product(float acc, float v, float w
   return acc + prod;
 }
 
-template <class YT>
+// One workgroup per token.  VEC: every thread owns runs of 16 bytes of y (8 storage
+// or 4 f32 columns), so a slot row is read with 16-byte loads; needs N a multiple of
+// the run and 16-byte aligned rows.  The sum over a token's slots runs in ascending
+// slot order for every column either way.
+template <class YT, bool VEC>
 __global__ __launch_bounds__(256) void combine_kernel(const YT* y, const float* w, const int32_t* off,
                                                       const int32_t* list, float* out, int N) {
   constexpr int kMaxSorted = 256;
+  constexpr int RUN = VEC ? 16 / (int)sizeof(YT) : 1;
   __shared__ int sorted[kMaxSorted];
   __shared__ float sw[kMaxSorted];
   const int t = blockIdx.x;
@@ -295,31 +301,67 @@ __global__ __launch_bounds__(256) void combine_kernel(const YT* y, const float* 
     }
     __syncthreads();
   }
-  for (int n = threadIdx.x; n < N; n += 256) {
-    float acc = 0.f;
-    int prev = -1;
-    for (int i = 0; i < len; ++i) {
-      int slot;
-      float wt;
-      if (small) {
-        slot = sorted[i];
-        wt = sw[i];
-      } else {
-        // next slot in ascending order: smallest id greater than the previous one
-        int best = 0x7fffffff;
-        for (int j = lo; j < hi; ++j) {
-          const int sl = list[j];
-          if (sl > prev && sl < best) best = sl;
-        }
-        prev = slot = best;
-        wt = w[best];
+  for (int n = threadIdx.x * RUN; n < N; n += 256 * RUN) {
+    float acc[RUN];
+#pragma unroll
+    for (int e = 0; e < RUN; ++e) acc[e] = 0.f;
+    auto add_row = [&](const uint4& raw, float wt) {
+      const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int e = 0; e < RUN; ++e) {
+        float v;
+        if constexpr (sizeof(YT) == 2) v = __uint_as_float((e & 1) ? (u[e >> 1] & 0xffff0000u) : (u[e >> 1] << 16));
+        else v = __uint_as_float(u[e]);
+        acc[e] = add_rounded_product(acc[e], v, wt);
       }
-      float v;
-      if constexpr (sizeof(YT) == 2) v = bf16_bits_to_f32(y[(long)slot * N + n]);
-      else v = y[(long)slot * N + n];
-      acc = add_rounded_product(acc, v, wt);
+    };
+    if (VEC && small) {
+      // four rows are requested before the first is added (the order of the adds stays)
+      int i = 0;
+      for (; i + 4 <= len; i += 4) {
+        uint4 raw[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) raw[u] = *reinterpret_cast<const uint4*>(y + (long)sorted[i + u] * N + n);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) add_row(raw[u], sw[i + u]);
+      }
+      for (; i < len; ++i) add_row(*reinterpret_cast<const uint4*>(y + (long)sorted[i] * N + n), sw[i]);
+    } else {
+      int prev = -1;
+      for (int i = 0; i < len; ++i) {
+        int slot;
+        float wt;
+        if (small) {
+          slot = sorted[i];
+          wt = sw[i];
+        } else {
+          // next slot in ascending order: smallest id greater than the previous one
+          int best = 0x7fffffff;
+          for (int j = lo; j < hi; ++j) {
+            const int sl = list[j];
+            if (sl > prev && sl < best) best = sl;
+          }
+          prev = slot = best;
+          wt = w[best];
+        }
+        const YT* src = y + (long)slot * N + n;
+        if constexpr (VEC) {
+          add_row(*reinterpret_cast<const uint4*>(src), wt);
+        } else {
+          float v;
+          if constexpr (sizeof(YT) == 2) v = bf16_bits_to_f32(src[0]);
+          else v = src[0];
+          acc[0] = add_rounded_product(acc[0], v, wt);
+        }
+      }
     }
-    out[(long)t * N + n] = acc;
+    if constexpr (VEC) {
+#pragma unroll
+      for (int e = 0; e < RUN; e += 4)
+        *reinterpret_cast<float4*>(out + (long)t * N + n + e) = make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
+    } else {
+      out[(long)t * N + n] = acc[0];
+    }
   }
 }
 
@@ -338,7 +380,11 @@ int combine_dev(const void* y, const int32_t* token_of_slot, const float* w, flo
   if (S > 0) hipLaunchKernelGGL(combine_count_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, cnt);
   hipLaunchKernelGGL(combine_scan_kernel, dim3(1), dim3(1024), 0, s, cnt, T, off);
   if (S > 0) hipLaunchKernelGGL(combine_fill_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, off, cnt, list);
-  hipLaunchKernelGGL((combine_kernel<YT>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, off, list, out, N);
+  const bool vec = N % (16 / (int)sizeof(YT)) == 0 && aligned16(y) && aligned16(out);
+  if (vec)
+    hipLaunchKernelGGL((combine_kernel<YT, true>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, off, list, out, N);
+  else
+    hipLaunchKernelGGL((combine_kernel<YT, false>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, off, list, out, N);
   int rc = launch_status();
   if (hipFreeAsync(cnt, s) != hipSuccess || hipFreeAsync(off, s) != hipSuccess || hipFreeAsync(list, s) != hipSuccess)
     rc = kDeviceFailed;
