@@ -127,10 +127,15 @@ __global__ __launch_bounds__(256) void scan_kernel(int32_t* chunk_counts, int ch
                                                    int32_t* num_slots) {
   for (int e = threadIdx.x; e < E; e += blockDim.x) {
     int run = 0;
-    for (int c = 0; c < chunks; ++c) {
-      const int v = chunk_counts[(long)c * E + e];
-      chunk_counts[(long)c * E + e] = run;
-      run += v;
+    for (int c0 = 0; c0 < chunks; c0 += 16) {          // 16 independent loads per round trip
+      int v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = c0 + u < chunks ? chunk_counts[(long)(c0 + u) * E + e] : 0;
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        if (c0 + u < chunks) chunk_counts[(long)(c0 + u) * E + e] = run;
+        run += v[u];
+      }
     }
     group_sizes[e] = (capacity > 0 && run > capacity) ? capacity : run;
   }
@@ -167,10 +172,14 @@ __global__ __launch_bounds__(64) void place_kernel(const int32_t* expert_ids, co
       const int leader = __ffsll((long long)todo) - 1;
       const int e0 = __shfl(e, leader, 64);
       const unsigned long long same = __ballot(valid && e == e0);
+      // (the workgroup is one wave: its LDS operations execute in program order, so
+      // the leader's update is seen by the next round's reads without a barrier)
       if (valid && e == e0) rank = cursor[e0] + __popcll(same & ((1ull << lane) - 1ull));
-      __syncthreads();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
       if (lane == leader) cursor[e0] += __popcll(same);
-      __syncthreads();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
       todo &= ~same;
     }
     if (valid && (capacity <= 0 || rank < capacity)) {
