@@ -129,19 +129,20 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
   // The guarded form is for a step that may be partial: out-of-range K must
   // contribute exact zeros, which a buffer load returns by itself for an offset
   // past the end of its range.
-  auto gload1 = [&](int q, int k0, auto guarded_c) {
+  auto gfetch = [&](int q, int k0, auto guarded_c) -> uint4 {
     constexpr bool GUARD = decltype(guarded_c)::value;
     if (q < A_CHUNKS) {
       uint32_t off = a_off[q];
       if constexpr (GUARD) off = (k0 + a_chunk * 16 < K) ? off : kOutOfRange;
-      st[q] = buffer_load_b128(a_base + k0, off);
+      return buffer_load_b128(a_base + k0, off);
     } else {
       const int qb = q - A_CHUNKS;
       uint32_t off = b_off[qb];
       if constexpr (GUARD) off = (k0 + b_krow[qb] < K) ? off : kOutOfRange;
-      st[q] = buffer_load_b128(b_base + (long)k0 * p.N, off);
+      return buffer_load_b128(b_base + (long)k0 * p.N, off);
     }
   };
+  auto gload1 = [&](int q, int k0, auto guarded_c) { st[q] = gfetch(q, k0, guarded_c); };
   auto lstore1 = [&](int q, int buf) {
     char* base = smem + buf * G8_STAGE;
     if (q < A_CHUNKS) lds_write_b128(base, a_lds[q], st[q]);
@@ -254,13 +255,24 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
 
   // ---- prologue: K step 0 in buffer 0, group 0 of step 1 in buffer 1, the rest of
   // step 1 and group 0 of step 2 in registers ---------------------------------------
+  // (the first half of step 1 is requested before step 0 has landed, into registers the
+  // operand fragments use later: group 0 of step 1 is then not a second full memory
+  // latency behind step 0)
+  constexpr int PRE = NC / 2;
 #pragma unroll
   for (int q = 0; q < NC; ++q) gload1(q, 0, true_type{});
+  uint4 pre[PRE];
+  if (ktiles > 1) {
+#pragma unroll
+    for (int q = 0; q < PRE; ++q) pre[q] = gfetch(q, G8_BK, true_type{});
+  }
 #pragma unroll
   for (int q = 0; q < NC; ++q) lstore1(q, 0);
   if (ktiles > 1) {
 #pragma unroll
-    for (int q = 0; q < NC; ++q) gload1(q, G8_BK, true_type{});
+    for (int q = PRE; q < NC; ++q) gload1(q, G8_BK, true_type{});
+#pragma unroll
+    for (int q = 0; q < PRE; ++q) st[q] = pre[q];
     if (ktiles > 2) stream_group(0, 1, 2 * G8_BK, mode2{});
     else stream_group(0, 1, 0, mode0{});
   }
