@@ -244,6 +244,10 @@ def bench_moe(lane, steps, warmup):
     ffn = lambda: lane.check(lib.tessera_gfx950_moe_swiglu_block_bf16_dev(
         dxp.ptr, dwg.ptr, dwu.ptr, dwd.ptr, dgo.ptr, dy.ptr, dh.ptr, S, H, F, H, E, None), "swiglu")
     _, ev_ffn = _timed(lane, ffn, steps, warmup)
+    # the same block reading x through the dispatch map (no dispatch pass, no x_perm)
+    ffn_g = lambda: lane.check(lib.tessera_gfx950_moe_swiglu_block_gather_bf16_dev(
+        dx.ptr, dtos.ptr, dwg.ptr, dwu.ptr, dwd.ptr, dgo.ptr, dy.ptr, dh.ptr, T, S, H, F, H, E, None), "swiglu_gather")
+    _, ev_ffn_g = _timed(lane, ffn_g, steps, warmup)
     dout = lane.DeviceBuffer(T * H * 4)
     comb = lambda: lane.check(lib.tessera_gfx950_moe_combine_bf16_dev(dy.ptr, dtos.ptr, dcw.ptr, dout.ptr, T, S, H, None),
                               "combine")
@@ -252,7 +256,8 @@ def bench_moe(lane, steps, warmup):
         buf.close()
     flop = 6.0 * S * H * F
     return {"workload": "moe_T8192_H4096_E64_top8_F1408_bf16", "route_ms": ev_route, "dispatch_ms": ev_disp,
-            "expert_ffn_ms": ev_ffn, "combine_ms": ev_comb, "expert_ffn_tflops": flop / ev_ffn / 1e9,
+            "expert_ffn_ms": ev_ffn, "dispatch_fused_expert_ffn_ms": ev_ffn_g, "combine_ms": ev_comb,
+            "layer_ms": ev_route + ev_ffn_g + ev_comb, "expert_ffn_tflops": flop / ev_ffn / 1e9,
             "frac_mfma_peak": flop / ev_ffn / 1e9 / PEAK_BF16_TFLOPS,
             "dispatch_gbs": 2.0 * S * H * 2 / ev_disp / 1e6}
 

@@ -343,9 +343,19 @@ int tessera_gfx950_moe_swiglu_block_bf16(const void* x, const void* wg, const vo
 int tessera_gfx950_moe_swiglu_block_bf16_dev(const void* x, const void* wg, const void* wu, const void* wd,
                                              const int32_t* offsets, void* y, void* hidden,
                                              int S, int K, int F, int N, int E, void* stream);
+/* The same block reading its input through the dispatch map: row m of the block's
+ * input is x[token_of_slot[m]], x the unpermuted bf16 [T,K] activation, so
+ * moe_dispatch (python/tessera/stdlib/moe.py:117-125) needs no pass and no x_perm
+ * buffer of its own.  token_of_slot: device int32[S] with values in [0, T);
+ * T * K * 2 must stay under 4 GiB. */
+int tessera_gfx950_moe_swiglu_block_gather_bf16_dev(const void* x, const int32_t* token_of_slot,
+                                                    const void* wg, const void* wu, const void* wd,
+                                                    const int32_t* offsets, void* y, void* hidden,
+                                                    int T, int S, int K, int F, int N, int E, void* stream);
 /* The whole local layer nn.functional.moe_layer
  * (python/tessera/nn/functional.py:403-490) with the router logits given:
- * route -> dispatch -> swiglu block -> combine.  out f32 [T,N].  The five
+ * route -> swiglu block (reading x through the dispatch map) -> combine.  out f32
+ * [T,N].  The five
  * metadata outputs may each be NULL. */
 int tessera_gfx950_moe_layer_bf16(const void* x, const float* router_logits, const void* wg, const void* wu,
                                   const void* wd, float* out, int T, int H, int F, int N, int E, int k,

@@ -81,6 +81,8 @@ struct Gemm16Params {
   const float* bias;      // fused epilogue: f32[N] added to every row, or null
   int act;                // fused epilogue / gate activation (enum Activation)
   const int* offsets;     // grouped: device int32[E+1] row offsets into A and D; else null
+  const int* gather;      // grouped: row m of A is row gather[m] of p.A (the dispatch fused
+                          // into the A load); null: row m
   int groups;             // E (grouped) or batch count
   int tiles_m, tiles_n;   // tile grid (grouped: tiles_m is an upper bound)
 };
@@ -231,7 +233,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   // Buffer loads: a wave-uniform tile base (advanced along K on the scalar unit) plus
   // a fixed 32-bit per-lane byte offset, one address register per chunk.
   // A: chunk v = tid + NT*q  -> row v/8, 16-byte chunk v%8.
-  const uint16_t* a_base = Ab + (long)m_begin * p.lda;
+  const bool gathered = GROUPED && p.gather != nullptr;
+  const uint16_t* a_base = gathered ? Ab : Ab + (long)m_begin * p.lda;
   uint32_t a_off[A_CHUNKS], a_lds[A_CHUNKS];
   const int a_chunk = tid & 7;
 #pragma unroll
@@ -239,6 +242,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     const int row = (tid >> 3) + (NT / 8) * q;
     int gr = row;
     gr = m_begin + gr < m_end ? gr : m_end - 1 - m_begin;   // clamp: rows past the edge are never stored
+    if constexpr (GROUPED) {
+      if (gathered) gr = p.gather[m_begin + gr];            // source row (the launcher bounds rows * lda)
+    }
     a_off[q] = ((uint32_t)gr * (uint32_t)p.lda + a_chunk * 8) * 2;
     a_lds[q] = row * G16_APITCH + ((a_chunk ^ g16_aswz(row)) << 4);
   }

@@ -44,7 +44,7 @@ __global__ void gemm16_grouped_generic_kernel(const Gemm16Params p) {
   int e = 0;
   while (e + 1 < p.groups && m >= p.offsets[e + 1]) ++e;
   if (m < p.offsets[e] || m >= p.offsets[e + 1]) return;
-  const uint16_t* A = p.A + (long)m * p.lda;
+  const uint16_t* A = p.A + (long)(p.gather ? p.gather[m] : m) * p.lda;
   const uint16_t* B = p.B + (long)e * p.strideB + n;
   float acc = 0.f;
   for (int k = 0; k < p.K; ++k) acc += from_storage<T>(A[k]) * from_storage<T>(B[(long)k * p.ldb]);

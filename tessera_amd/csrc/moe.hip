@@ -432,9 +432,15 @@ int grouped_dev(const void* x, const void* w, const int32_t* offsets, void* y, i
   return launch_gemm16_grouped<BF16, EPI>(p, s);
 }
 
+// `gather` (device int32[S], or null): row m of the block's input is x[gather[m]], i.e.
+// x is the unpermuted (T, K) activation and the dispatch is part of the first GEMM's
+// operand load.  x_rows = number of rows of x (T with a gather, else S).
 int swiglu_dev(const void* x, const void* wg, const void* wu, const void* wd, const int32_t* offsets, void* y,
-               void* hidden, int S, int K, int F, int N, int E, hipStream_t s) {
+               void* hidden, int S, int K, int F, int N, int E, hipStream_t s, const int32_t* gather = nullptr,
+               int x_rows = 0) {
   if (bad_grouped(S, K, N, E) || F <= 0 || !wg || !wu || !wd || !offsets || (S > 0 && (!x || !y))) return kBadShape;
+  // (the kernels address a gathered row with a 32-bit byte offset from x)
+  if (gather && (x_rows <= 0 || (long)x_rows * K * 2 >= (1L << 32))) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
   if (S == 0) return kOk;
   void* h = hidden;
@@ -448,6 +454,7 @@ int swiglu_dev(const void* x, const void* wg, const void* wu, const void* wd, co
   p.lda = K; p.ldb = F; p.ldd = F;
   p.strideB = (long)K * F;
   p.offsets = offsets;
+  p.gather = gather;
   p.groups = E;
   int rc = launch_gemm16_grouped<BF16, EPI_SWIGLU16>(p, s);
   if (rc == kOk) rc = grouped_dev<EPI_STORE16>(h, wd, offsets, y, S, F, N, E, s);
@@ -633,6 +640,14 @@ int tessera_gfx950_moe_swiglu_block_bf16(const void* x, const void* wg, const vo
   return scope.download(y, dy, (size_t)S * N * 2) ? kOk : kDeviceFailed;
 }
 
+int tessera_gfx950_moe_swiglu_block_gather_bf16_dev(const void* x, const int32_t* token_of_slot, const void* wg,
+                                                    const void* wu, const void* wd, const int32_t* offsets, void* y,
+                                                    void* hidden, int T, int S, int K, int F, int N, int E,
+                                                    void* stream) {
+  if (!token_of_slot) return kBadShape;
+  return swiglu_dev(x, wg, wu, wd, offsets, y, hidden, S, K, F, N, E, as_stream(stream), token_of_slot, T);
+}
+
 int tessera_gfx950_moe_layer_bf16(const void* x, const float* router_logits, const void* wg, const void* wu,
                                   const void* wd, float* out, int T, int H, int F, int N, int E, int k,
                                   int normalize, int capacity, int32_t* token_of_slot, int32_t* expert_of_slot,
@@ -655,7 +670,6 @@ int tessera_gfx950_moe_layer_bf16(const void* x, const float* router_logits, con
   int32_t* dgs = static_cast<int32_t*>(scope.alloc((size_t)E * 4));
   int32_t* dof = static_cast<int32_t*>(scope.alloc((size_t)(E + 1) * 4));
   int32_t* dn = static_cast<int32_t*>(scope.alloc(4));
-  void* dxp = scope.alloc(S * H * 2);
   void* dh = scope.alloc(S * F * 2);
   void* dy = scope.alloc(S * N * 2);
   float* dout = static_cast<float*>(scope.alloc((size_t)T * N * 4));
@@ -664,8 +678,8 @@ int tessera_gfx950_moe_layer_bf16(const void* x, const float* router_logits, con
   if (rc != kOk) return rc;
   int32_t n = 0;                       // kept slots (capacity may drop some)
   if (hipDeviceSynchronize() != hipSuccess || !scope.download(&n, dn, 4)) return kDeviceFailed;
-  rc = dispatch_dev(dx, dt, dxp, T, n, H, 2, nullptr);
-  if (rc == kOk) rc = swiglu_dev(dxp, dg, du, dd, dof, dy, dh, n, H, F, N, E, nullptr);
+  // the dispatch x[token_of_slot] is the first GEMM's operand load
+  rc = swiglu_dev(dx, dg, du, dd, dof, dy, dh, n, H, F, N, E, nullptr, dt, T);
   if (rc == kOk) rc = combine_dev<uint16_t>(dy, dt, dw, dout, T, n, N, nullptr);
   if (rc != kOk) return rc;
   if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;

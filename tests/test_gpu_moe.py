@@ -140,6 +140,32 @@ def test_moe_swiglu_block(lane, sizes, K, F, N):
     assert np.mean(got != ref) < 0.05
 
 
+@pytest.mark.parametrize("T,K,F,N,E,k", [(300, 256, 384, 128, 8, 2), (1024, 128, 1408, 256, 16, 4),
+                                          (77, 64, 128, 64, 4, 1)])
+def test_swiglu_block_reading_through_the_dispatch_map(lane, T, K, F, N, E, k):
+    """The block with the dispatch fused into its first operand load equals
+    dispatch followed by the block, bit for bit (the gather is exact)."""
+    rng = np.random.default_rng(T)
+    plan = ops.route_tokens(_logits(T, E, 3, k), E, k, capacity_factor=1e9)
+    S = plan.num_slots
+    xb = b16.from_float32(rng.standard_normal((T, K)).astype(np.float32))
+    wg, wu = (b16.from_float32((rng.standard_normal((E, K, F)) * 0.1).astype(np.float32)) for _ in range(2))
+    wd = b16.from_float32((rng.standard_normal((E, F, N)) * 0.1).astype(np.float32))
+    want = ops.moe_swiglu_block(ops.moe_dispatch(xb, plan), wg, wu, wd, plan.group_sizes)
+    bufs = [lane.DeviceBuffer.from_host(np.asarray(a, np.uint16)) for a in (xb, wg, wu, wd)]
+    dtos = lane.DeviceBuffer.from_host(np.ascontiguousarray(plan.token_of_slot, np.int32))
+    doff = lane.DeviceBuffer.from_host(np.ascontiguousarray(plan.group_offsets, np.int32))
+    dy = lane.DeviceBuffer(S * N * 2)
+    rc = lane.load().tessera_gfx950_moe_swiglu_block_gather_bf16_dev(
+        bufs[0].ptr, dtos.ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, doff.ptr, dy.ptr, None, T, S, K, F, N, E, None)
+    lane.check(rc, "swiglu_gather")
+    lane.synchronize()
+    got = dy.download((S, N), np.uint16)
+    assert np.array_equal(got, np.asarray(want, np.uint16))
+    for b in bufs + [dtos, doff, dy]:
+        b.close()
+
+
 def test_single_expert_reduces_to_dense_swiglu(lane):
     """E = 1 is the dense SwiGLU MLP (tests/unit/test_moe_layer.py:74-79)."""
     x, wg, wu, wd = _swiglu_inputs([200], 128, 256, 128, 9)
