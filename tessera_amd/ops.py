@@ -353,13 +353,13 @@ def grouped_gemm(x, weights, group_sizes, *, kind: str = "contiguous", alignment
         raise NotImplementedError(
             f"grouped_gemm: kind={kind!r} is not implemented — supported: "
             f"{', '.join(_SUPPORTED_GROUPED_KINDS)}")
-    if quant is not None:
-        raise NotImplementedError("grouped_gemm: quantised grouped GEMM is not part of the gfx950 lane")
     x, weights = _unbox(x), _unbox(weights)
     if _storage(x, weights) != "bf16":
         raise ValueError("grouped_gemm on the gfx950 lane takes bf16 storage")
     xa, w = _bits(x), _bits(weights)
     gs = np.asarray(group_sizes).astype(np.int64).reshape(-1)
+    if quant is not None:
+        return _grouped_gemm_fp8(x, weights, xa, w, gs, quant, alignment, out)
     if alignment is not None:
         al = int(alignment)
         if al <= 0 or np.any(gs % al != 0):
@@ -378,6 +378,46 @@ def grouped_gemm(x, weights, group_sizes, *, kind: str = "contiguous", alignment
     name = "tessera_gfx950_grouped_gemm_bf16" + ("_f32" if f32 else "")
     _lane.check(getattr(_lane.load(), name)(xa.ctypes.data, w.ctypes.data, off.ctypes.data, y.ctypes.data, T, K, N, E),
                 "grouped_gemm")
+    return y if f32 else y.view(BF16Array)
+
+
+#: quant schemes of the reference's grouped GEMM that map onto the lane's e4m3 operand format
+_FP8_GROUPED_QUANT = ("fp8_e4m3", "fp8")
+
+
+def _grouped_gemm_fp8(x, weights, xa, w, gs, quant, alignment, out):
+    """``quant="fp8_e4m3"``: x is quantised per tensor and every expert's weight per
+    tensor (the reference's scale layout, ``compiler/grouped_layout.py:353-392``),
+    and each group is one e4m3 GEMM with f32 accumulation, scaled by both scales.
+    The reference dequantises on the host and multiplies in f32; the products of two
+    e4m3 values are exact in f32, so the two differ only in summation order."""
+    q = str(quant).lower()
+    if q not in _FP8_GROUPED_QUANT:
+        raise NotImplementedError(
+            f"grouped_gemm: quant={quant!r} is not implemented on the gfx950 lane — supported: "
+            f"{', '.join(_FP8_GROUPED_QUANT)}")
+    if alignment is not None:
+        al = int(alignment)
+        if al <= 0 or np.any(gs % al != 0):
+            raise ValueError(f"grouped_gemm: every group size must be a multiple of alignment={alignment}")
+    if xa.ndim != 2 or w.ndim != 3 or w.shape[0] != gs.shape[0] or w.shape[1] != xa.shape[1]:
+        raise ValueError(f"grouped_gemm: x {xa.shape} / weights {w.shape} / group_sizes {gs.shape} disagree")
+    T, K = xa.shape
+    E, _, N = w.shape
+    _offsets(gs, T, "grouped_gemm")
+    xf = x.to_float32() if isinstance(x, BF16Array) else _bf16.from_bits(xa).to_float32()
+    wf = weights.to_float32() if isinstance(weights, BF16Array) else _bf16.from_bits(w).to_float32()
+    x_codes, sx = quantize_fp8_codes(xf)
+    f32 = out == "f32"
+    y = np.zeros((T, N), np.float32 if f32 else np.uint16)
+    row = 0
+    for e in range(E):
+        n = int(gs[e])
+        if n:
+            w_codes, sw = quantize_fp8_codes(wf[e])
+            y[row:row + n] = np.asarray(gemm_fp8(x_codes[row:row + n], w_codes, sx, sw, out="f32" if f32 else "bf16"),
+                                        y.dtype)
+        row += n
     return y if f32 else y.view(BF16Array)
 
 

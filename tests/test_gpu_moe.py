@@ -166,6 +166,33 @@ def test_swiglu_block_reading_through_the_dispatch_map(lane, T, K, F, N, E, k):
         b.close()
 
 
+def test_grouped_gemm_fp8_quant(lane):
+    """quant="fp8_e4m3": per-tensor e4m3 for x and for every expert's weight, then the
+    grouped product (compiler/grouped_layout.py:353-392).  Checked against the oracle's
+    quantise-dequantise followed by the f64 grouped product."""
+    sizes, K, N = [40, 0, 130, 7], 128, 96
+    rng = np.random.default_rng(17)
+    x = b16.from_float32(rng.standard_normal((sum(sizes), K)).astype(np.float32))
+    w = b16.from_float32((rng.standard_normal((len(sizes), K, N)) * 0.2).astype(np.float32))
+    got = ops.grouped_gemm(x, w, sizes, quant="fp8_e4m3", out="f32")
+    def qdq(a):
+        _, grid, scale = orc.quantize_fp8_e4m3(a)
+        return grid.astype(np.float64) * np.float64(scale)
+    xq = qdq(x.to_float32())
+    ref = np.zeros((sum(sizes), N))
+    row = 0
+    for e, n in enumerate(sizes):
+        ref[row:row + n] = xq[row:row + n] @ qdq(w.to_float32()[e])
+        row += n
+    assert orc.max_rel_err(got, ref) <= 1e-4              # f32 accumulation of exact products
+    # and within the fp8 budget of the unquantised product
+    assert orc.max_rel_err(got, orc.grouped_gemm(x.to_float32(), w.to_float32(), sizes, store=False)) <= 3e-2 * 4
+    stored = ops.grouped_gemm(x, w, sizes, quant="fp8")
+    assert np.array_equal(np.asarray(stored, np.uint16), np.asarray(b16.from_float32(got), np.uint16))
+    with pytest.raises(NotImplementedError):
+        ops.grouped_gemm(x, w, sizes, quant="nvfp4")
+
+
 def test_single_expert_reduces_to_dense_swiglu(lane):
     """E = 1 is the dense SwiGLU MLP (tests/unit/test_moe_layer.py:74-79)."""
     x, wg, wu, wd = _swiglu_inputs([200], 128, 256, 128, 9)
