@@ -26,7 +26,9 @@ int launch_flash(const FlashParams& p, hipStream_t s) {
                                    hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   });
   if (attr_err != hipSuccess) return kDeviceFailed;
-  dim3 grid(ceil_div(p.Sq, FA_BQ) * p.B * p.Hq, 1, 1);
+  const int qblocks = ceil_div(p.Sq, FA_BQ);
+  const bool xcd_grouped = (p.B * p.Hkv) % 8 == 0;
+  const dim3 grid = xcd_grouped ? dim3(8 * p.ratio, p.B * p.Hkv / 8, qblocks) : dim3(p.B * p.Hq, 1, qblocks);
   hipLaunchKernelGGL(kern, grid, dim3(FA_THREADS), kSmem, s, p);
   return launch_status();
 }
@@ -45,6 +47,7 @@ int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, i
   p.O = O;
   p.LSE = static_cast<float*>(LSE);
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Sq = Sq; p.Sk = Sk;
+  p.ratio = Hq / Hkv;
   p.scale = scale;
   p.causal = causal ? 1 : 0;
   p.out_storage = out_storage ? 1 : 0;

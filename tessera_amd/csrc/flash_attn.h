@@ -47,6 +47,7 @@ struct FlashParams {
   int out_storage;     // 0: f32 O, 1: O in the storage dtype
   int window;          // > 0: band of keys per query (see key_bounds); 0: none
   float softcap;       // > 0: scaled scores pass through cap * tanh(s / cap); 0: none
+  int ratio;           // Hq / Hkv
   const float* bias;   // additive bias [B, Hq, Sq, Sk] f32 added to the (capped) scaled scores, or null
 };
 
@@ -143,30 +144,27 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
   // range — so every XCD receives the same mix, and inside a level the (batch,
   // head) pairs are permuted so that all query heads sharing one KV head land on
   // the same XCD and find its K/V in that XCD's L2.
-  const int qblocks = (p.Sq + FA_BQ - 1) / FA_BQ;
-  const int BH = p.B * p.Hq;
-  const int id = blockIdx.x;
-  const int qb = qblocks - 1 - id / BH;
-  const int u = id % BH;
-  const int ratio = p.Hq / p.Hkv;
-  int b, hq;
-  if ((p.B * p.Hkv) % 8 == 0) {
-    const int w = u % (8 * ratio);
-    const int g = (u / (8 * ratio)) * 8 + (w & 7);   // kv group = (batch, kv head)
-    b = g / p.Hkv;
-    hq = (g % p.Hkv) * ratio + (w >> 3);
+  // The grid is (8 * ratio, B * Hkv / 8, query blocks) when B * Hkv is a multiple of 8,
+  // else (B * Hq, 1, query blocks): x runs fastest in the dispatch order, so the
+  // linear order is the one described above and no index needs a division.
+  // qlin / kvlin: linear (batch, head) index of the query head / of its KV head.
+  const int qb = (int)gridDim.z - 1 - (int)blockIdx.z;
+  int qlin, kvlin;
+  if (gridDim.y > 1 || (int)gridDim.x == 8 * p.ratio) {
+    const int w = blockIdx.x;
+    kvlin = blockIdx.y * 8 + (w & 7);
+    qlin = kvlin * p.ratio + (w >> 3);
   } else {
-    b = u / p.Hq;
-    hq = u % p.Hq;
+    qlin = blockIdx.x;
+    kvlin = qlin / p.ratio;
   }
-  const int hkv = (int)(((long)hq * p.Hkv) / p.Hq);
   const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
 
   const int q0 = qb * FA_BQ;                  // first query row of the workgroup
   const int qw = q0 + wave * (32 * QT);       // first query row of the wave
-  const uint16_t* Qb = p.Q + ((long)(b * p.Hq + hq) * p.Sq) * D;
-  const uint16_t* Kb = p.K + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
-  const uint16_t* Vb = p.V + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
+  const uint16_t* Qb = p.Q + ((long)qlin * p.Sq) * D;
+  const uint16_t* Kb = p.K + ((long)kvlin * p.Sk) * D;
+  const uint16_t* Vb = p.V + ((long)kvlin * p.Sk) * D;
 
   // Key tiles this workgroup needs: from the first visible key of its first row to
   // the last visible key of its last row (bounds are monotone in the row index).
@@ -259,7 +257,7 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     const int qi = min(qw + 32 * qt + l32, p.Sq - 1);
-    bias_row[qt] = (EXT && p.bias) ? p.bias + ((long)(b * p.Hq + hq) * p.Sq + qi) * p.Sk : nullptr;
+    bias_row[qt] = (EXT && p.bias) ? p.bias + ((long)qlin * p.Sq + qi) * p.Sk : nullptr;
   }
   auto capped = [&](float sraw) -> float {
     return cap2 * (1.0f - 2.0f * __builtin_amdgcn_rcpf(fast_exp2(sraw * incap) + 1.0f));
@@ -504,7 +502,7 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
     if (qi >= p.Sq) continue;
     if (khi[qt] < klo[qt]) l = 0.f;                      // no visible key: O = 0, LSE = -inf
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    const long row = (long)(b * p.Hq + hq) * p.Sq + qi;
+    const long row = (long)qlin * p.Sq + qi;
     if (p.LSE && lh == 0)
       p.LSE[row] = l > 0.f ? (m_run[qt] * cs + __log2f(l)) * 0.69314718055994530942f : -INFINITY;
 #pragma unroll
