@@ -325,27 +325,40 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
     ld_row[q] = row;
     ld_off[q] = row * ROWB + ((chp ^ bwd_swz<D>(row)) << 4);
   }
-  auto load_step = [&](int step, int stage) {
-    const int hq = hkv * ratio + step / steps_per_head;
-    const int qt0 = (t_first + step % steps_per_head) * FB_BQT;
-    const long qrow0 = (long)(b * p.Hq + hq) * p.Sq;
+  // Tile of step s: query head hkv * ratio + s / steps_per_head, query tile t_first +
+  // s % steps_per_head.  The loop keeps both as counters (no division per step).
+  // The loads of a step are issued in two halves (`part`): a burst of 17 per wave
+  // sits in the issue queue for over a thousand cycles.
+  auto load_part = [&](int head, int tile, int stage, int part) {
+    const int qt0 = tile * FB_BQT;
+    const long qrow0 = (long)(b * p.Hq + hkv * ratio + head) * p.Sq;
     const uint16_t* qb = p.Q + (qrow0 + qt0) * D;
     const uint16_t* gb = p.dO + (qrow0 + qt0) * D;
     const int last = p.Sq - 1 - qt0;                       // last valid row of this tile
     const uint32_t sbase = lds0 + stage * STAGE;
+    constexpr int HALF = LD_PER_WAVE / 2;
+    if (last >= FB_BQT - 1) {                              // full tile (uniform): no row clamp
 #pragma unroll
-    for (int q = 0; q < LD_PER_WAVE; ++q) {
-      uint32_t o = ld_off[q];
-      if (ld_row[q] > last) o -= (uint32_t)(ld_row[q] - last) * ROWB;   // rows past the end: masked later
-      load16_to_lds(qb, o, sbase + (wave * LD_PER_WAVE + q) * 1024);
-      load16_to_lds(gb, o, sbase + TILE + (wave * LD_PER_WAVE + q) * 1024);
+      for (int q = part * HALF; q < (part + 1) * HALF; ++q) {
+        load16_to_lds(qb, ld_off[q], sbase + (wave * LD_PER_WAVE + q) * 1024);
+        load16_to_lds(gb, ld_off[q], sbase + TILE + (wave * LD_PER_WAVE + q) * 1024);
+      }
+    } else {
+#pragma unroll
+      for (int q = part * HALF; q < (part + 1) * HALF; ++q) {
+        uint32_t o = ld_off[q];
+        if (ld_row[q] > last) o -= (uint32_t)(ld_row[q] - last) * ROWB;   // rows past the end: masked later
+        load16_to_lds(qb, o, sbase + (wave * LD_PER_WAVE + q) * 1024);
+        load16_to_lds(gb, o, sbase + TILE + (wave * LD_PER_WAVE + q) * 1024);
+      }
     }
-    if (wave < 2) {
+    if (part == 1 && wave < 2) {
       const float* src = (wave == 0 ? p.LSE2 : p.Delta) + qrow0 + qt0;
       const int r = lane <= last ? lane : last;
       load4_to_lds(src, (uint32_t)r * 4, sbase + 2 * TILE + wave * FB_BQT * 4);
     }
   };
+  static_assert(LD_PER_WAVE % 2 == 0, "loads are issued in two halves");
 
   uint32_t row_rd[KSTEPS];
 #pragma unroll
@@ -365,15 +378,22 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.f; dv[dt][r] = 0.f; }
 
-  if (nsteps > 0) load_step(0, 0);
+  if (nsteps > 0) {
+    load_part(0, t_first, 0, 0);
+    load_part(0, t_first, 0, 1);
+  }
   fa_wait_loads();
   __syncthreads();
   const int wave_k0 = k0 + wave * 32;
+  int cur_head = 0, cur_tile = t_first;                    // (head, tile) of this step
   for (int step = 0; step < nsteps; ++step) {
     const int st = step & 1;
-    if (step + 1 < nsteps) load_step(step + 1, st ^ 1);
+    int nxt_head = cur_head, nxt_tile = cur_tile + 1;      // ... and of the next
+    if (nxt_tile == qtiles) { nxt_tile = t_first; ++nxt_head; }
+    const bool has_next = step + 1 < nsteps;
+    if (has_next) load_part(nxt_head, nxt_tile, st ^ 1, 0);
     const char* base = smem + st * STAGE;
-    const int qt0 = (t_first + step % steps_per_head) * FB_BQT;
+    const int qt0 = cur_tile * FB_BQT;
     // do this wave's keys see the tile at all?  (uniform per wave)
     const bool live = wave_k0 < p.Sk && (!p.causal || wave_k0 <= min(qt0 + FB_BQT, p.Sq) - 1 + off);
     if (live) {
@@ -410,6 +430,7 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
           }
         }
       }
+      if (has_next) load_part(nxt_head, nxt_tile, st ^ 1, 1);
       // lane: key, queries qt0 + 32 qt + 8 (r/4) + 4 lh + r % 4.  Only tiles that touch
       // the causal diagonal or the end of Q / K pay for the per-pair mask.
       uint4 pf[2][2], dsf[2][2];
@@ -473,7 +494,11 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
         dv[dt] = mfma_32x32x16<T>(oT[cur], pf[qt][g], dv[dt]);
         dk[dt] = mfma_32x32x16<T>(qT[cur], dsf[qt][g], dk[dt]);
       }
+    } else if (has_next) {
+      load_part(nxt_head, nxt_tile, st ^ 1, 1);
     }
+    cur_head = nxt_head;
+    cur_tile = nxt_tile;
     fa_wait_loads();
     __syncthreads();
   }
