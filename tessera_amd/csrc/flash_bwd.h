@@ -397,103 +397,117 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
     // do this wave's keys see the tile at all?  (uniform per wave)
     const bool live = wave_k0 < p.Sk && (!p.causal || wave_k0 <= min(qt0 + FB_BQT, p.Sq) - 1 + off);
     if (live) {
-      // S = Q K^T and dP = dO V^T for both 32-row halves: four independent MFMA chains
-      // (operand fragments are read one k step ahead of the MFMAs that use them)
+      // The step runs as a pipeline over the two 32-row halves of the query tile, so
+      // that the softmax arithmetic (VALU) of one half rides in the shadow of the other
+      // half's MFMAs — one wave per SIMD has nobody else to overlap with:
+      //   first products (S = Q K^T, dP = dO V^T) of half 0
+      //   first products of half 1          | softmax of half 0
+      //   second products (dV, dK) of half 0 | softmax of half 1
+      //   second products of half 1
+      // Operand fragments are read one MFMA pair ahead of their use.
       f32x16 s[2], dp[2];
-      uint4 qfr[2][2], dofr[2][2];                         // [buffer][qt]
+      uint32_t pw[2][8], dw[2][8];                         // packed P and dS per half
+      // one eighth of a half's softmax: elements 4 a + 2 h2 + {0, 1} of the lane's 16
+      auto softmax_piece = [&](int qt, int piece, auto masked_c) __attribute__((always_inline)) {
+        constexpr bool MASKED = decltype(masked_c)::value;
+        const int a = piece >> 1, h2 = piece & 1;
+        const int qoff = 32 * qt + 8 * a + 4 * lh + 2 * h2;
+        const float2 l2 = *reinterpret_cast<const float2*>(base + 2 * TILE + qoff * 4);
+        const float2 d2 = *reinterpret_cast<const float2*>(base + 2 * TILE + FB_BQT * 4 + qoff * 4);
+        const float lv[2] = {l2.x, l2.y}, dl[2] = {d2.x, d2.y};
+        float pr[2], ds[2];
 #pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
-        qfr[0][qt] = lds_read_b128(base, row_rd[0] + qt * 32 * ROWB);
-        dofr[0][qt] = lds_read_b128(base, TILE + row_rd[0] + qt * 32 * ROWB);
-      }
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        const int cur = ks & 1;
-        if (ks + 1 < KSTEPS) {
-#pragma unroll
-          for (int qt = 0; qt < 2; ++qt) {
-            qfr[cur ^ 1][qt] = lds_read_b128(base, row_rd[ks + 1] + qt * 32 * ROWB);
-            dofr[cur ^ 1][qt] = lds_read_b128(base, TILE + row_rd[ks + 1] + qt * 32 * ROWB);
+        for (int e = 0; e < 2; ++e) {
+          const int r = 4 * a + 2 * h2 + e;
+          float x = fmaf(s[qt][r], c, -lv[e]);
+          if constexpr (MASKED) {
+            const int q = qt0 + qoff + e;
+            const bool ok = (q < p.Sq) & (key < p.Sk) & (!p.causal | (key <= q + off));
+            x = ok ? x : -INFINITY;                        // exponent -inf: P = 0, no branch
           }
+          pr[e] = fast_exp2(x);
+          ds[e] = pr[e] * (dp[qt][r] - dl[e]);
         }
+        pw[qt][2 * a + h2] = pack2<T>(pr[0], pr[1]);
+        dw[qt][2 * a + h2] = pack2<T>(ds[0], ds[1]);
+      };
+      // S and dP of one half: 8 k steps of two MFMAs; `between(ks)` follows each pair
+      auto first_products = [&](int qt, auto&& between) __attribute__((always_inline)) {
+        uint4 qfr[2], dofr[2];
+        qfr[0] = lds_read_b128(base, row_rd[0] + qt * 32 * ROWB);
+        dofr[0] = lds_read_b128(base, TILE + row_rd[0] + qt * 32 * ROWB);
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const int cur = ks & 1;
+          if (ks + 1 < KSTEPS) {
+            qfr[cur ^ 1] = lds_read_b128(base, row_rd[ks + 1] + qt * 32 * ROWB);
+            dofr[cur ^ 1] = lds_read_b128(base, TILE + row_rd[ks + 1] + qt * 32 * ROWB);
+          }
           if (ks == 0) {
             f32x16 z;
 #pragma unroll
             for (int r = 0; r < 16; ++r) z[r] = 0.f;
-            s[qt] = mfma_32x32x16<T>(qfr[cur][qt], kf[ks], z);
-            dp[qt] = mfma_32x32x16<T>(dofr[cur][qt], vf[ks], z);
+            s[qt] = mfma_32x32x16<T>(qfr[cur], kf[ks], z);
+            dp[qt] = mfma_32x32x16<T>(dofr[cur], vf[ks], z);
           } else {
-            s[qt] = mfma_32x32x16<T>(qfr[cur][qt], kf[ks], s[qt]);
-            dp[qt] = mfma_32x32x16<T>(dofr[cur][qt], vf[ks], dp[qt]);
+            s[qt] = mfma_32x32x16<T>(qfr[cur], kf[ks], s[qt]);
+            dp[qt] = mfma_32x32x16<T>(dofr[cur], vf[ks], dp[qt]);
           }
+          between(ks);
         }
-      }
-      if (has_next) load_part(nxt_head, nxt_tile, st ^ 1, 1);
+      };
+      // dV += dO^T P and dK += Q^T dS of one half: (g, dt) steps of two MFMAs
+      auto second_products = [&](int qt, auto&& between) __attribute__((always_inline)) {
+        const uint4 pf[2] = {make_uint4(pw[qt][0], pw[qt][1], pw[qt][2], pw[qt][3]),
+                             make_uint4(pw[qt][4], pw[qt][5], pw[qt][6], pw[qt][7])};
+        const uint4 dsf[2] = {make_uint4(dw[qt][0], dw[qt][1], dw[qt][2], dw[qt][3]),
+                              make_uint4(dw[qt][4], dw[qt][5], dw[qt][6], dw[qt][7])};
+        auto tr_frags = [&](int i, uint4& qT, uint4& oT) {
+          const int dt = i % DT, g = i / DT;
+          const uint32_t o = (qt * 32 + g * 16) * ROWB;
+          const uint2 qlo = lds_read_tr16_b64(base + tr_lo[dt] + o);
+          const uint2 qhi = lds_read_tr16_b64(base + tr_hi[dt] + o);
+          const uint2 olo = lds_read_tr16_b64(base + TILE + tr_lo[dt] + o);
+          const uint2 ohi = lds_read_tr16_b64(base + TILE + tr_hi[dt] + o);
+          qT = make_uint4(qlo.x, qlo.y, qhi.x, qhi.y);
+          oT = make_uint4(olo.x, olo.y, ohi.x, ohi.y);
+        };
+        constexpr int NSTEP = 2 * DT;
+        uint4 qT[2], oT[2];
+        tr_frags(0, qT[0], oT[0]);
+#pragma unroll
+        for (int i = 0; i < NSTEP; ++i) {
+          const int cur = i & 1;
+          if (i + 1 < NSTEP) tr_frags(i + 1, qT[cur ^ 1], oT[cur ^ 1]);
+          const int dt = i % DT, g = i / DT;
+          dv[dt] = mfma_32x32x16<T>(oT[cur], pf[g], dv[dt]);
+          dk[dt] = mfma_32x32x16<T>(qT[cur], dsf[g], dk[dt]);
+          between(i);
+        }
+      };
+      static_assert(KSTEPS == 8 || KSTEPS == 4, "softmax pieces are spread over the k steps");
+      auto none = [](int) {};
       // lane: key, queries qt0 + 32 qt + 8 (r/4) + 4 lh + r % 4.  Only tiles that touch
       // the causal diagonal or the end of Q / K pay for the per-pair mask.
-      uint4 pf[2][2], dsf[2][2];
-      auto softmax_part = [&](auto masked_c) {
-        constexpr bool MASKED = decltype(masked_c)::value;
-#pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
-          uint32_t pw[8], dw[8];
-#pragma unroll
-          for (int a = 0; a < 4; ++a) {
-            const int qoff = 32 * qt + 8 * a + 4 * lh;
-            const float4 l4 = *reinterpret_cast<const float4*>(base + 2 * TILE + qoff * 4);
-            const float4 d4 = *reinterpret_cast<const float4*>(base + 2 * TILE + FB_BQT * 4 + qoff * 4);
-            const float lv[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
-            float pr[4], ds[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              float x = fmaf(s[qt][4 * a + e], c, -lv[e]);
-              if constexpr (MASKED) {
-                const int q = qt0 + qoff + e;
-                const bool ok = (q < p.Sq) & (key < p.Sk) & (!p.causal | (key <= q + off));
-                x = ok ? x : -INFINITY;                  // exponent -inf: P = 0, no branch
-              }
-              pr[e] = fast_exp2(x);
-              ds[e] = pr[e] * (dp[qt][4 * a + e] - dl[e]);
-            }
-            pw[2 * a] = pack2<T>(pr[0], pr[1]);
-            pw[2 * a + 1] = pack2<T>(pr[2], pr[3]);
-            dw[2 * a] = pack2<T>(ds[0], ds[1]);
-            dw[2 * a + 1] = pack2<T>(ds[2], ds[3]);
-          }
-          pf[qt][0] = make_uint4(pw[0], pw[1], pw[2], pw[3]);
-          pf[qt][1] = make_uint4(pw[4], pw[5], pw[6], pw[7]);
-          dsf[qt][0] = make_uint4(dw[0], dw[1], dw[2], dw[3]);
-          dsf[qt][1] = make_uint4(dw[4], dw[5], dw[6], dw[7]);
-        }
-      };
       const bool need_mask = (qt0 + FB_BQT > p.Sq) || (wave_k0 + 32 > p.Sk) ||
                              (p.causal && wave_k0 + 31 > qt0 + off);
-      if (need_mask) softmax_part(std::true_type{});
-      else softmax_part(std::false_type{});
-      // second products, their transposed operands read one step ahead
-      constexpr int NSTEP = 4 * DT;                        // (qt, g, dt) steps
-      auto tr_frags = [&](int i, uint4& qT, uint4& oT) {
-        const int dt = i % DT, g = (i / DT) & 1, qt = i / (2 * DT);
-        const uint32_t o = (qt * 32 + g * 16) * ROWB;
-        const uint2 qlo = lds_read_tr16_b64(base + tr_lo[dt] + o);
-        const uint2 qhi = lds_read_tr16_b64(base + tr_hi[dt] + o);
-        const uint2 olo = lds_read_tr16_b64(base + TILE + tr_lo[dt] + o);
-        const uint2 ohi = lds_read_tr16_b64(base + TILE + tr_hi[dt] + o);
-        qT = make_uint4(qlo.x, qlo.y, qhi.x, qhi.y);
-        oT = make_uint4(olo.x, olo.y, ohi.x, ohi.y);
-      };
-      uint4 qT[2], oT[2];
-      tr_frags(0, qT[0], oT[0]);
+      auto run = [&](auto masked_c) __attribute__((always_inline)) {
+        // 8 softmax pieces per half over KSTEPS (first products) or 2 DT (second) slots
+        constexpr int PER1 = 8 / KSTEPS, PER2 = 8 / (2 * DT);
+        first_products(0, none);
+        if (has_next) load_part(nxt_head, nxt_tile, st ^ 1, 1);
+        first_products(1, [&](int ks) {
 #pragma unroll
-      for (int i = 0; i < NSTEP; ++i) {
-        const int cur = i & 1;
-        if (i + 1 < NSTEP) tr_frags(i + 1, qT[cur ^ 1], oT[cur ^ 1]);
-        const int dt = i % DT, g = (i / DT) & 1, qt = i / (2 * DT);
-        dv[dt] = mfma_32x32x16<T>(oT[cur], pf[qt][g], dv[dt]);
-        dk[dt] = mfma_32x32x16<T>(qT[cur], dsf[qt][g], dk[dt]);
-      }
+          for (int u = 0; u < PER1; ++u) softmax_piece(0, ks * PER1 + u, masked_c);
+        });
+        second_products(0, [&](int i) {
+#pragma unroll
+          for (int u = 0; u < PER2; ++u) softmax_piece(1, i * PER2 + u, masked_c);
+        });
+        second_products(1, none);
+      };
+      if (need_mask) run(std::true_type{});
+      else run(std::false_type{});
     } else if (has_next) {
       load_part(nxt_head, nxt_tile, st ^ 1, 1);
     }
