@@ -1,4 +1,5 @@
 // C ABI: flash-attention forward (causal, GQA, LSE), 16-bit storage.
+#include <cmath>
 #include <mutex>
 #include "../../include/tessera_gfx950.h"
 #include "flash_attn.h"
@@ -123,6 +124,9 @@ int flash_bwd_dev(const void* dO, const void* Q, const void* K, const void* V, c
   const size_t rows = (size_t)B * Hq * Sq;
   const bool recompute = !O || !LSE;
   float* ws = nullptr;                       // Delta (rows) | LSE2 (rows) | [O (rows * D) | LSE (rows)]?
+  // The MFMA kernels fold -LSE / scale into their accumulators: they need a scale it
+  // can be divided by; anything else takes the generic kernels.
+  const bool scale_ok = std::isfinite(scale) && std::fabs(scale) >= 1e-20f;
   const size_t ws_floats = 2 * rows + (recompute ? rows * D + rows : 0);
   if (hipMallocAsync(reinterpret_cast<void**>(&ws), ws_floats * sizeof(float), s) != hipSuccess) {
     (void)hipGetLastError();
@@ -148,16 +152,18 @@ int flash_bwd_dev(const void* dO, const void* Q, const void* K, const void* V, c
     p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Sq = Sq; p.Sk = Sk;
     p.scale = scale;
     p.causal = causal ? 1 : 0;
-    hipLaunchKernelGGL((flash_bwd_delta_kernel<T>), dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, s,
-                       p.dO, p.O, p.LSE, delta, p.LSE2, (long)rows, D);
-    rc = launch_status();
     const bool al = ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
                       reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(dO) |
                       reinterpret_cast<uintptr_t>(dQ) | reinterpret_cast<uintptr_t>(dK) |
                       reinterpret_cast<uintptr_t>(dV)) & 15) == 0;
+    const bool mfma = al && scale_ok && (D == 128 || D == 64);
+    hipLaunchKernelGGL((flash_bwd_delta_kernel<T>), dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, s,
+                       p.dO, p.O, p.LSE, delta, p.LSE2, (long)rows, D, mfma ? -1.f : 1.f,
+                       mfma ? -1.f / scale : 1.f);
+    rc = launch_status();
     if (rc == kOk) {
-      if (al && D == 128) rc = launch_bwd<T, 128>(p, s);
-      else if (al && D == 64) rc = launch_bwd<T, 64>(p, s);
+      if (mfma && D == 128) rc = launch_bwd<T, 128>(p, s);
+      else if (mfma) rc = launch_bwd<T, 64>(p, s);
       else {
         const long kvrows = (long)B * Hkv * Sk;
         hipLaunchKernelGGL((flash_bwd_generic_dq_kernel<T>), dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, p, D);

@@ -30,8 +30,8 @@ struct FlashBwdParams {
   const uint16_t* dO;   // [B, Hq, Sq, D]
   const float* O;       // [B, Hq, Sq, D]  forward output
   const float* LSE;     // [B, Hq, Sq]     forward log-sum-exp (natural log, of scaled scores)
-  float* Delta;         // [B, Hq, Sq]     workspace
-  float* LSE2;          // [B, Hq, Sq]     workspace: LSE * log2(e)
+  float* Delta;         // [B, Hq, Sq]     workspace: Delta, or -Delta for the MFMA kernels
+  float* LSE2;          // [B, Hq, Sq]     workspace of the MFMA kernels: -LSE / scale
   float* dQ;            // [B, Hq, Sq, D]
   float* dK;            // [B, Hkv, Sk, D]
   float* dV;            // [B, Hkv, Sk, D]
@@ -60,12 +60,16 @@ __device__ __forceinline__ int bwd_swz(int row) {
   return ((t & 1) << 2) | (t >> 1);
 }
 
-// Delta[row] = sum_d dO[row][d] * O[row][d] and LSE2[row] = LSE[row] * log2(e);
-// 16 lanes per row, 8 columns per lane per pass.
+// Delta[row] = delta_mul * sum_d dO[row][d] * O[row][d] and LSE2[row] = lse_mul * LSE[row];
+// 16 lanes per row, 8 columns per lane per pass.  The MFMA kernels take both negated,
+// the log-sum-exp also divided by the softmax scale (multipliers -1 and -1 / scale):
+// they start the S and dP accumulators from these values, so that the products come
+// out as S - LSE / scale and dP - Delta with no further arithmetic per element.
 template <class T>
 __global__ void flash_bwd_delta_kernel(const uint16_t* __restrict__ dO, const float* __restrict__ O,
                                        const float* __restrict__ LSE, float* __restrict__ Delta,
-                                       float* __restrict__ LSE2, long rows, int D) {
+                                       float* __restrict__ LSE2, long rows, int D, float delta_mul,
+                                       float lse_mul) {
   const long row = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
   const int part = threadIdx.x & 15;
   float acc = 0.f;
@@ -86,8 +90,8 @@ __global__ void flash_bwd_delta_kernel(const uint16_t* __restrict__ dO, const fl
 #pragma unroll
   for (int s = 8; s >= 1; s >>= 1) acc += __shfl_xor(acc, s, 64);
   if (row < rows && part == 0) {
-    Delta[row] = acc;
-    LSE2[row] = LSE[row] * kLog2e;
+    Delta[row] = acc * delta_mul;
+    LSE2[row] = LSE[row] * lse_mul;
   }
 }
 
@@ -139,8 +143,8 @@ __global__ __launch_bounds__(FB_DQ_THREADS, 1) void flash_bwd_dq_kernel(const Fl
     dof[ks] = *reinterpret_cast<const uint4*>(p.dO + (qrow0 + qrow) * D + 16 * ks + 8 * lh);
   }
   const float c = p.scale * kLog2e;
-  const float lse2 = p.LSE2[qrow0 + qrow];
-  const float delta = p.Delta[qrow0 + qrow];
+  const float neg_lse = p.LSE2[qrow0 + qrow];             // -LSE / scale
+  const float neg_delta = p.Delta[qrow0 + qrow];          // -Delta
   const int lim = qi >= p.Sq ? -1 : (p.causal ? min(qi + off, p.Sk - 1) : p.Sk - 1);
 
   // tile loaders (global -> LDS, swizzle applied on the global address)
@@ -204,7 +208,7 @@ __global__ __launch_bounds__(FB_DQ_THREADS, 1) void flash_bwd_dq_kernel(const Fl
       for (int kt = 0; kt < 2; ++kt) {
         f32x16 s, dp;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+        for (int r = 0; r < 16; ++r) { s[r] = neg_lse; dp[r] = neg_delta; }   // S - LSE / scale, dP - Delta
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
           const uint4 kf = lds_read_b128(smem, row_rd[ks] + st * TILE + kt * 32 * ROWB);
@@ -224,12 +228,12 @@ __global__ __launch_bounds__(FB_DQ_THREADS, 1) void flash_bwd_dq_kernel(const Fl
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
               const int rr = r + e;
-              float x = fmaf(s[rr], c, -lse2);
+              float x = s[rr] * c;
               if constexpr (MASKED) {
                 const int key = kv0 + kt * 32 + 8 * (rr >> 2) + 4 * lh + (rr & 3);
                 x = key <= lim ? x : -INFINITY;          // exponent -inf: P = 0, no branch
               }
-              ds2[e] = fast_exp2(x) * (dp[rr] - delta);
+              ds2[e] = fast_exp2(x) * dp[rr];
             }
             w[r >> 1] = pack2<T>(ds2[0], ds2[1]);
           }
@@ -277,7 +281,7 @@ template <class T, int D>
 __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const FlashBwdParams p) {
   constexpr int KSTEPS = D / 16, DT = D / 32, ROWB = D * 2, CHUNKS = D / 8;
   constexpr int TILE = FB_BQT * ROWB;                      // bytes of a Q (or dO) tile
-  constexpr int STAGE = 2 * TILE + 2 * FB_BQT * 4;         // Q | dO | lse2[64] | delta[64]
+  constexpr int STAGE = 2 * TILE + 2 * FB_BQT * 4;         // Q | dO | -LSE/scale [64] | -Delta [64]
   constexpr int LD_PER_WAVE = FB_BQT * CHUNKS / 64 / (FB_DKV_THREADS / 64);
   static_assert(FB_BQT * CHUNKS % FB_DKV_THREADS == 0, "tile/thread mismatch");
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -412,27 +416,35 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
         constexpr bool MASKED = decltype(masked_c)::value;
         const int a = piece >> 1, h2 = piece & 1;
         const int qoff = 32 * qt + 8 * a + 4 * lh + 2 * h2;
-        const float2 l2 = *reinterpret_cast<const float2*>(base + 2 * TILE + qoff * 4);
-        const float2 d2 = *reinterpret_cast<const float2*>(base + 2 * TILE + FB_BQT * 4 + qoff * 4);
-        const float lv[2] = {l2.x, l2.y}, dl[2] = {d2.x, d2.y};
         float pr[2], ds[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
           const int r = 4 * a + 2 * h2 + e;
-          float x = fmaf(s[qt][r], c, -lv[e]);
+          float x = s[qt][r] * c;
           if constexpr (MASKED) {
             const int q = qt0 + qoff + e;
             const bool ok = (q < p.Sq) & (key < p.Sk) & (!p.causal | (key <= q + off));
             x = ok ? x : -INFINITY;                        // exponent -inf: P = 0, no branch
           }
           pr[e] = fast_exp2(x);
-          ds[e] = pr[e] * (dp[qt][r] - dl[e]);
+          ds[e] = pr[e] * dp[qt][r];
         }
         pw[qt][2 * a + h2] = pack2<T>(pr[0], pr[1]);
         dw[qt][2 * a + h2] = pack2<T>(ds[0], ds[1]);
       };
-      // S and dP of one half: 8 k steps of two MFMAs; `between(ks)` follows each pair
+      // S - LSE / scale and dP - Delta of one half: the accumulators start from the
+      // staged -LSE / scale and -Delta of their rows (lane's rows 8 a + 4 lh + 0..3),
+      // then 8 k steps of two MFMAs; `between(ks)` follows each pair
       auto first_products = [&](int qt, auto&& between) __attribute__((always_inline)) {
+        f32x16 s0, dp0;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          const int qoff = 32 * qt + 8 * a + 4 * lh;
+          const float4 l4 = *reinterpret_cast<const float4*>(base + 2 * TILE + qoff * 4);
+          const float4 d4 = *reinterpret_cast<const float4*>(base + 2 * TILE + FB_BQT * 4 + qoff * 4);
+          s0[4 * a] = l4.x; s0[4 * a + 1] = l4.y; s0[4 * a + 2] = l4.z; s0[4 * a + 3] = l4.w;
+          dp0[4 * a] = d4.x; dp0[4 * a + 1] = d4.y; dp0[4 * a + 2] = d4.z; dp0[4 * a + 3] = d4.w;
+        }
         uint4 qfr[2], dofr[2];
         qfr[0] = lds_read_b128(base, row_rd[0] + qt * 32 * ROWB);
         dofr[0] = lds_read_b128(base, TILE + row_rd[0] + qt * 32 * ROWB);
@@ -444,11 +456,8 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
             dofr[cur ^ 1] = lds_read_b128(base, TILE + row_rd[ks + 1] + qt * 32 * ROWB);
           }
           if (ks == 0) {
-            f32x16 z;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) z[r] = 0.f;
-            s[qt] = mfma_32x32x16<T>(qfr[cur], kf[ks], z);
-            dp[qt] = mfma_32x32x16<T>(dofr[cur], vf[ks], z);
+            s[qt] = mfma_32x32x16<T>(qfr[cur], kf[ks], s0);
+            dp[qt] = mfma_32x32x16<T>(dofr[cur], vf[ks], dp0);
           } else {
             s[qt] = mfma_32x32x16<T>(qfr[cur], kf[ks], s[qt]);
             dp[qt] = mfma_32x32x16<T>(dofr[cur], vf[ks], dp[qt]);
