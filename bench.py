@@ -262,6 +262,88 @@ def bench_moe(lane, steps, warmup):
             "dispatch_gbs": 2.0 * S * H * 2 / ev_disp / 1e6}
 
 
+def clock_and_power_trace(lane, seconds=4.0):
+    """Shader clock (mean over the XCDs) and socket power, sampled with amd-smi while
+    each kernel runs back to back on a second thread, on random and on constant
+    operands.  Shows which figures are set by the board's power limit rather than by
+    the kernel's schedule: the MFMA peak is quoted at 2400 MHz, and a launch that runs
+    at 1700 MHz cannot pass 71 % of it whatever its instruction stream."""
+    import ctypes
+    import subprocess
+    import threading
+
+    def sample():
+        r = subprocess.run(["/opt/rocm/bin/amd-smi", "metric", "-p", "-c", "--json"], capture_output=True, text=True)
+        try:
+            j = json.loads(r.stdout)
+            g = j[0] if isinstance(j, list) else j["gpu_data"][0]
+            clk = [v["clk"]["value"] for k, v in g["clock"].items() if k.startswith("gfx_")]
+            return float(np.mean(clk)), float(g["power"]["socket_power"]["value"])
+        except (ValueError, KeyError, IndexError, TypeError):
+            return None
+
+    def measure(fn):
+        stop, count = [False], [0]
+
+        def loop():
+            while not stop[0]:
+                for _ in range(20):
+                    fn()
+                lane.synchronize()
+                count[0] += 20
+        th = threading.Thread(target=loop)
+        th.start()
+        time.sleep(1.0)                                       # clocks settle
+        n0, t0, seen = count[0], time.perf_counter(), []
+        while time.perf_counter() - t0 < seconds:
+            got = sample()
+            if got:
+                seen.append(got)
+        n1, t1 = count[0], time.perf_counter()
+        stop[0] = True
+        th.join()
+        if not seen:
+            return {"error": "amd-smi gave no reading"}
+        return {"ms": (t1 - t0) / max(n1 - n0, 1) * 1e3, "gfx_clock_mhz": float(np.mean([c for c, _ in seen])),
+                "socket_power_w": float(np.mean([w for _, w in seen])), "samples": len(seen)}
+
+    lib = lane.load()
+    rng = np.random.default_rng(1)
+
+    def operand(shape, constant):
+        if constant:
+            return lane.DeviceBuffer.from_host(np.full(shape, 0x3C3C, np.uint16))
+        return lane.DeviceBuffer.from_host(_bf16(rng.standard_normal(shape, dtype=np.float32)))
+
+    out = {"idle": dict(zip(("gfx_clock_mhz", "socket_power_w"), sample() or (None, None)))}
+    M = N = K = 8192
+    B, Hq, Hkv, S, D = 4, 32, 8, 4096, 128
+    scale = ctypes.c_float(1.0 / np.sqrt(D))
+    for constant in (False, True):
+        tag = "constant" if constant else "random"
+        a, b, c = operand((M, K), constant), operand((K, N), constant), lane.DeviceBuffer(M * N * 2)
+        r = measure(lambda: lib.tessera_gfx950_gemm_bf16_bf16_dev(a.ptr, b.ptr, c.ptr, M, N, K, None))
+        r["tflops"] = 2.0 * M * N * K / r["ms"] / 1e9 if "ms" in r else None
+        out[f"gemm_bf16_8192_{tag}"] = r
+        del a, b, c
+        q, do = operand((B, Hq, S, D), constant), operand((B, Hq, S, D), constant)
+        k, v = operand((B, Hkv, S, D), constant), operand((B, Hkv, S, D), constant)
+        o32, lse = lane.DeviceBuffer(B * Hq * S * D * 4), lane.DeviceBuffer(B * Hq * S * 4)
+        r = measure(lambda: lib.tessera_gfx950_flash_attn_gqa_bf16_dev(q.ptr, k.ptr, v.ptr, o32.ptr, lse.ptr, B, Hq,
+                                                                      Hkv, S, S, D, scale, 1, 0, None))
+        fwd_flop = 4.0 * B * Hq * (S * (S + 1) / 2) * D
+        r["tflops"] = fwd_flop / r["ms"] / 1e9 if "ms" in r else None
+        out[f"flash_attn_fwd_{tag}"] = r
+        gq, gk, gv = (lane.DeviceBuffer(n * 4) for n in (B * Hq * S * D, B * Hkv * S * D, B * Hkv * S * D))
+        r = measure(lambda: lib.tessera_gfx950_flash_attn_bwd_bf16_dev(do.ptr, q.ptr, k.ptr, v.ptr, o32.ptr, lse.ptr,
+                                                                      gq.ptr, gk.ptr, gv.ptr, B, Hq, Hkv, S, S, D,
+                                                                      scale, 1, None))
+        r["tflops"] = 2.5 * fwd_flop / r["ms"] / 1e9 if "ms" in r else None
+        out[f"flash_attn_bwd_{tag}"] = r
+        del q, do, k, v, o32, lse, gq, gk, gv
+    return out
+
+
 def cpu_baseline(A, B):
     """The reference's CPU path for this config is ``np.matmul`` on f32-promoted
     operands; the oracle restates it.  Timed once on the full workload."""
@@ -294,6 +376,8 @@ def main() -> int:
     ap.add_argument("--only-headline", action="store_true", help="skip the `also` measurements")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a 1 GiB copy kernel (counter calibration for profiled runs)")
+    ap.add_argument("--clocks", action="store_true",
+                    help="instead of the bench line: shader clock and socket power under each kernel")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X; this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -304,6 +388,9 @@ def main() -> int:
         print("gfx950 lane unavailable: no MI355X or library not built", file=sys.stderr)
         return 3
 
+    if args.clocks:
+        print(json.dumps(clock_and_power_trace(lane), indent=1))
+        return 0
     copy_cal = calibrate_copy(lane) if args.calibrate_copy else None
     M = N = K = 8192
     wall, ev, (A, B, a, b, out) = bench_gemm(lane, M, N, K, args.steps, args.warmup)

@@ -57,7 +57,9 @@ int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, i
   p.bias = bias;
   const bool al = ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
                     reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(O)) & 15) == 0;
-  const bool ext = p.softcap > 0.f || p.bias != nullptr;
+  // The plain variant takes row maxima of the raw scores, which needs scale > 0; the
+  // extended one scales first and serves every other scale.
+  const bool ext = p.softcap > 0.f || p.bias != nullptr || !(scale > 0.f);
   if (al && D == 128) return ext ? launch_flash<T, 128, true>(p, s) : launch_flash<T, 128, false>(p, s);
   if (al && D == 64) return ext ? launch_flash<T, 64, true>(p, s) : launch_flash<T, 64, false>(p, s);
   const long rows = (long)B * Hq * Sq;
@@ -94,7 +96,7 @@ int flash_host(const void* Q, const void* K, const void* V, void* O, void* LSE, 
 template <class T, int D>
 int launch_bwd(const FlashBwdParams& p, hipStream_t s) {
   constexpr int kDqSmem = 4 * FB_BKV * D * 2;
-  constexpr int kDkvSmem = 2 * (2 * FB_BQT * D * 2 + 2 * FB_BQT * 4);
+  constexpr int kDkvSmem = flash_bwd_dkdv_lds_bytes<D>();
   auto dq_kern = flash_bwd_dq_kernel<T, D>;
   auto dkv_kern = flash_bwd_dkdv_kernel<T, D>;
   static std::once_flag once;

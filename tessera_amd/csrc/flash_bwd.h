@@ -6,7 +6,8 @@
 //   flash_bwd_delta_kernel   Delta[q] = sum_d dO[q][d] O[q][d]
 //   flash_bwd_dq_kernel      one workgroup per 256 query rows, walks the key tiles
 //   flash_bwd_dkdv_kernel    one workgroup per 128 keys of one KV head, walks the
-//                            query tiles of every query head that shares the KV head
+//                            query tiles of every query head that shares the KV head;
+//                            producer waves (S, dP, softmax) feed consumer waves (dK, dV)
 // Both walkers recompute P = exp(scale S - LSE) and dS = P (dP - Delta) tile by tile.
 // As in the forward kernel the products are oriented so that the index a lane owns
 // (its query row in the dQ kernel, its key in the dK/dV kernel) is the one the
@@ -271,47 +272,58 @@ __global__ __launch_bounds__(FB_DQ_THREADS, 1) void flash_bwd_dq_kernel(const Fl
     }
 }
 
+constexpr int FB_BK = 128, FB_BQT = 64;                   // keys per workgroup, query rows per tile
+
 // ---------------------------------------------------------------------------------
-// dK, dV: 4 waves x 32 keys; Q / dO tiles of 64 query rows (plus their LSE and Delta)
-// are staged through LDS for every query head of the KV head's group.
+// dK, dV: one workgroup per 128 keys of a KV head, eight waves.  The four key groups of 32 keys each have a producer wave and a
+// consumer wave on the same SIMD (waves g and g + 4).  The producer holds the K and V
+// fragments of its keys, computes S and dP of a query tile and the softmax arithmetic,
+// and hands P and dS (16-bit, in MFMA operand order) to the consumer through LDS; the
+// consumer holds the dK and dV accumulators and does the second products of the tile
+// the producer finished one iteration earlier.  Each wave stays under 256 registers
+// (no accumulation-file traffic) and the two instruction streams of a SIMD fill each
+// other's gaps: the producer's exponentials run under the consumer's MFMAs.
+//
+// Iteration i: loads of tile i + 1 are issued into stage (i + 1) % 3; the consumer reads
+// P / dS of tile i - 1 into registers; barrier; the producer works on tile i (stage
+// i % 3) and writes P / dS at its end, the consumer on tile i - 1 (stage (i - 1) % 3);
+// barrier.  The exchange buffer is single: it is read before the first barrier and
+// written after it.
 // ---------------------------------------------------------------------------------
-constexpr int FB_BK = 128, FB_BQT = 64, FB_DKV_THREADS = 256;
+constexpr int FB_DKV_THREADS = 512;
+
+template <int D>
+constexpr int flash_bwd_dkdv_lds_bytes() {
+  return 3 * (2 * FB_BQT * D * 2 + 2 * FB_BQT * 4) + 4 * 8 * 1024;
+}
 
 template <class T, int D>
-__global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const FlashBwdParams p) {
+__global__ __launch_bounds__(FB_DKV_THREADS) void flash_bwd_dkdv_kernel(const FlashBwdParams p) {
   constexpr int KSTEPS = D / 16, DT = D / 32, ROWB = D * 2, CHUNKS = D / 8;
   constexpr int TILE = FB_BQT * ROWB;                      // bytes of a Q (or dO) tile
   constexpr int STAGE = 2 * TILE + 2 * FB_BQT * 4;         // Q | dO | -LSE/scale [64] | -Delta [64]
-  constexpr int LD_PER_WAVE = FB_BQT * CHUNKS / 64 / (FB_DKV_THREADS / 64);
+  constexpr int XCH = 3 * STAGE;                           // exchange: [group][half][P | dS][quad][lane] x 16 B
+  constexpr int LD_PER_WAVE = FB_BQT * CHUNKS / 64 / 8;
   static_assert(FB_BQT * CHUNKS % FB_DKV_THREADS == 0, "tile/thread mismatch");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)(TSR_LDS char*)smem;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool producer = wave < 4;
+  const int grp = wave & 3;
   const int l32 = lane & 31, lh = lane >> 5, r16 = lane & 15;
 
-  // heavy key blocks (seen by the most query rows under a causal mask) first
-  const int kblocks = (p.Sk + FB_BK - 1) / FB_BK;
-  const int kb = blockIdx.x / (p.B * p.Hkv);
+  const int kb = blockIdx.x / (p.B * p.Hkv);               // heavy key blocks first
   const int bh = blockIdx.x % (p.B * p.Hkv);
   const int b = bh / p.Hkv, hkv = bh % p.Hkv;
   const int ratio = p.Hq / p.Hkv;
   const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
   const int k0 = kb * FB_BK;
-  const int key = k0 + wave * 32 + l32;                    // this lane's key
-  const int krow = key < p.Sk ? key : p.Sk - 1;
+  const int wave_k0 = k0 + grp * 32;
+  const int key = wave_k0 + l32;                           // this lane's key
   const long kvrow0 = (long)(b * p.Hkv + hkv) * p.Sk;
-  (void)kblocks;
-
-  uint4 kf[KSTEPS], vf[KSTEPS];
-#pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks) {
-    kf[ks] = *reinterpret_cast<const uint4*>(p.K + (kvrow0 + krow) * D + 16 * ks + 8 * lh);
-    vf[ks] = *reinterpret_cast<const uint4*>(p.V + (kvrow0 + krow) * D + 16 * ks + 8 * lh);
-  }
   const float c = p.scale * kLog2e;
 
-  // first query row that can see this workgroup's keys
   int q_first = 0;
   if (p.causal) q_first = max(0, k0 - off);
   const int t_first = q_first / FB_BQT;
@@ -329,44 +341,129 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
     ld_row[q] = row;
     ld_off[q] = row * ROWB + ((chp ^ bwd_swz<D>(row)) << 4);
   }
-  // Tile of step s: query head hkv * ratio + s / steps_per_head, query tile t_first +
-  // s % steps_per_head.  The loop keeps both as counters (no division per step).
-  // The loads of a step are issued in two halves (`part`): a burst of 17 per wave
-  // sits in the issue queue for over a thousand cycles.
-  auto load_part = [&](int head, int tile, int stage, int part) {
+  auto load_tile = [&](int head, int tile, int stage) {
     const int qt0 = tile * FB_BQT;
     const long qrow0 = (long)(b * p.Hq + hkv * ratio + head) * p.Sq;
     const uint16_t* qb = p.Q + (qrow0 + qt0) * D;
     const uint16_t* gb = p.dO + (qrow0 + qt0) * D;
     const int last = p.Sq - 1 - qt0;                       // last valid row of this tile
     const uint32_t sbase = lds0 + stage * STAGE;
-    constexpr int HALF = LD_PER_WAVE / 2;
-    if (last >= FB_BQT - 1) {                              // full tile (uniform): no row clamp
 #pragma unroll
-      for (int q = part * HALF; q < (part + 1) * HALF; ++q) {
-        load16_to_lds(qb, ld_off[q], sbase + (wave * LD_PER_WAVE + q) * 1024);
-        load16_to_lds(gb, ld_off[q], sbase + TILE + (wave * LD_PER_WAVE + q) * 1024);
-      }
-    } else {
-#pragma unroll
-      for (int q = part * HALF; q < (part + 1) * HALF; ++q) {
-        uint32_t o = ld_off[q];
-        if (ld_row[q] > last) o -= (uint32_t)(ld_row[q] - last) * ROWB;   // rows past the end: masked later
-        load16_to_lds(qb, o, sbase + (wave * LD_PER_WAVE + q) * 1024);
-        load16_to_lds(gb, o, sbase + TILE + (wave * LD_PER_WAVE + q) * 1024);
-      }
+    for (int q = 0; q < LD_PER_WAVE; ++q) {
+      uint32_t o = ld_off[q];
+      if (ld_row[q] > last) o -= (uint32_t)(ld_row[q] - last) * ROWB;     // rows past the end: masked later
+      load16_to_lds(qb, o, sbase + (wave * LD_PER_WAVE + q) * 1024);
+      load16_to_lds(gb, o, sbase + TILE + (wave * LD_PER_WAVE + q) * 1024);
     }
-    if (part == 1 && wave < 2) {
-      const float* src = (wave == 0 ? p.LSE2 : p.Delta) + qrow0 + qt0;
+    if (wave >= 6) {
+      const float* src = (wave == 6 ? p.LSE2 : p.Delta) + qrow0 + qt0;
       const int r = lane <= last ? lane : last;
-      load4_to_lds(src, (uint32_t)r * 4, sbase + 2 * TILE + wave * FB_BQT * 4);
+      load4_to_lds(src, (uint32_t)r * 4, sbase + 2 * TILE + (wave - 6) * FB_BQT * 4);
     }
   };
-  static_assert(LD_PER_WAVE % 2 == 0, "loads are issued in two halves");
+  // does this group's keys see the tile at all?  (uniform per wave, same answer in
+  // the producer and the consumer of a group)
+  auto tile_live = [&](int tile) {
+    const int qt0 = tile * FB_BQT;
+    return wave_k0 < p.Sk && (!p.causal || wave_k0 <= min(qt0 + FB_BQT, p.Sq) - 1 + off);
+  };
+  auto next_of = [&](int& head, int& tile) {
+    if (++tile == qtiles) { tile = t_first; ++head; }
+  };
+  char* xch = smem + XCH + grp * 8192;
 
-  uint32_t row_rd[KSTEPS];
+  if (nsteps > 0) load_tile(0, t_first, 0);
+  fa_wait_loads();
+  __syncthreads();
+
+  if (producer) {
+    const int krow = key < p.Sk ? key : p.Sk - 1;
+    uint4 kf[KSTEPS], vf[KSTEPS];
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks) row_rd[ks] = l32 * ROWB + ((((ks << 1) | lh) ^ bwd_swz<D>(l32)) << 4);
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      kf[ks] = *reinterpret_cast<const uint4*>(p.K + (kvrow0 + krow) * D + 16 * ks + 8 * lh);
+      vf[ks] = *reinterpret_cast<const uint4*>(p.V + (kvrow0 + krow) * D + 16 * ks + 8 * lh);
+    }
+    uint32_t row_rd[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) row_rd[ks] = l32 * ROWB + ((((ks << 1) | lh) ^ bwd_swz<D>(l32)) << 4);
+
+    int cur_head = 0, cur_tile = t_first, st = 0;          // tile of this iteration and its stage
+    for (int i = 0; i <= nsteps; ++i) {
+      int nxt_head = cur_head, nxt_tile = cur_tile;
+      next_of(nxt_head, nxt_tile);
+      const int nst = st == 2 ? 0 : st + 1;
+      if (i + 1 < nsteps) load_tile(nxt_head, nxt_tile, nst);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();                        // the consumer has taken P / dS of tile i - 1
+      asm volatile("" ::: "memory");
+      if (i < nsteps && tile_live(cur_tile)) {
+        const char* base = smem + st * STAGE;
+        const int qt0 = cur_tile * FB_BQT;
+        const bool need_mask = (qt0 + FB_BQT > p.Sq) || (wave_k0 + 32 > p.Sk) ||
+                               (p.causal && wave_k0 + 31 > qt0 + off);
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+          // accumulators start from -LSE / scale and -Delta of the lane's rows 8 a + 4 lh + 0..3
+          f32x16 sv, dp;
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            const int qoff = 32 * qt + 8 * a + 4 * lh;
+            const float4 l4 = *reinterpret_cast<const float4*>(base + 2 * TILE + qoff * 4);
+            const float4 d4 = *reinterpret_cast<const float4*>(base + 2 * TILE + FB_BQT * 4 + qoff * 4);
+            sv[4 * a] = l4.x; sv[4 * a + 1] = l4.y; sv[4 * a + 2] = l4.z; sv[4 * a + 3] = l4.w;
+            dp[4 * a] = d4.x; dp[4 * a + 1] = d4.y; dp[4 * a + 2] = d4.z; dp[4 * a + 3] = d4.w;
+          }
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            const uint4 qfr = lds_read_b128(base, row_rd[ks] + qt * 32 * ROWB);
+            const uint4 dofr = lds_read_b128(base, TILE + row_rd[ks] + qt * 32 * ROWB);
+            sv = mfma_32x32x16<T>(qfr, kf[ks], sv);
+            dp = mfma_32x32x16<T>(dofr, vf[ks], dp);
+          }
+          // lane: key, queries qt0 + 32 qt + 8 (r/4) + 4 lh + r % 4
+          uint32_t pw[8], dw[8];
+          auto softmax = [&](auto masked_c) __attribute__((always_inline)) {
+            constexpr bool MASKED = decltype(masked_c)::value;
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+              float pr[2], ds[2];
+#pragma unroll
+              for (int e = 0; e < 2; ++e) {
+                float x = sv[r + e] * c;
+                if constexpr (MASKED) {
+                  const int q = qt0 + 32 * qt + 8 * ((r + e) >> 2) + 4 * lh + ((r + e) & 3);
+                  const bool ok = (q < p.Sq) & (key < p.Sk) & (!p.causal | (key <= q + off));
+                  x = ok ? x : -INFINITY;                  // exponent -inf: P = 0, no branch
+                }
+                pr[e] = fast_exp2(x);
+                ds[e] = pr[e] * dp[r + e];
+              }
+              pw[r >> 1] = pack2<T>(pr[0], pr[1]);
+              dw[r >> 1] = pack2<T>(ds[0], ds[1]);
+            }
+          };
+          if (need_mask) softmax(std::true_type{});
+          else softmax(std::false_type{});
+#pragma unroll
+          for (int g = 0; g < 2; ++g) {
+            lds_write_b128(xch, ((qt * 2 + 0) * 2 + g) * 1024 + lane * 16,
+                           make_uint4(pw[4 * g], pw[4 * g + 1], pw[4 * g + 2], pw[4 * g + 3]));
+            lds_write_b128(xch, ((qt * 2 + 1) * 2 + g) * 1024 + lane * 16,
+                           make_uint4(dw[4 * g], dw[4 * g + 1], dw[4 * g + 2], dw[4 * g + 3]));
+          }
+        }
+      }
+      cur_head = nxt_head;
+      cur_tile = nxt_tile;
+      st = nst;
+      fa_wait_loads();
+      __syncthreads();
+    }
+    return;
+  }
+
+  // ---- consumer ----
   uint32_t tr_lo[DT], tr_hi[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
@@ -375,153 +472,55 @@ __global__ __launch_bounds__(FB_DKV_THREADS, 1) void flash_bwd_dkdv_kernel(const
     tr_lo[dt] = qq * ROWB + (((col >> 3) ^ bwd_swz<D>(qq)) << 4) + (col & 7) * 2;
     tr_hi[dt] = (qq + 8) * ROWB + (((col >> 3) ^ bwd_swz<D>(qq + 8)) << 4) + (col & 7) * 2;
   }
-
   f32x16 dk[DT], dv[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.f; dv[dt][r] = 0.f; }
 
-  if (nsteps > 0) {
-    load_part(0, t_first, 0, 0);
-    load_part(0, t_first, 0, 1);
-  }
-  fa_wait_loads();
-  __syncthreads();
-  const int wave_k0 = k0 + wave * 32;
-  int cur_head = 0, cur_tile = t_first;                    // (head, tile) of this step
-  for (int step = 0; step < nsteps; ++step) {
-    const int st = step & 1;
-    int nxt_head = cur_head, nxt_tile = cur_tile + 1;      // ... and of the next
-    if (nxt_tile == qtiles) { nxt_tile = t_first; ++nxt_head; }
-    const bool has_next = step + 1 < nsteps;
-    if (has_next) load_part(nxt_head, nxt_tile, st ^ 1, 0);
-    const char* base = smem + st * STAGE;
-    const int qt0 = cur_tile * FB_BQT;
-    // do this wave's keys see the tile at all?  (uniform per wave)
-    const bool live = wave_k0 < p.Sk && (!p.causal || wave_k0 <= min(qt0 + FB_BQT, p.Sq) - 1 + off);
+  int ld_head = 0, ld_tile = t_first, lst = 0;             // tile i (whose successor is loaded) and its stage
+  int cur_tile = t_first, st = 0;                          // tile i - 1 and its stage (from i = 1 on)
+  for (int i = 0; i <= nsteps; ++i) {
+    int nxt_head = ld_head, nxt_tile = ld_tile;
+    next_of(nxt_head, nxt_tile);
+    const int nst = lst == 2 ? 0 : lst + 1;
+    if (i + 1 < nsteps) load_tile(nxt_head, nxt_tile, nst);
+    const bool live = i >= 1 && tile_live(cur_tile);
+    uint4 pf[2][2], dsf[2][2];
     if (live) {
-      // The step runs as a pipeline over the two 32-row halves of the query tile, so
-      // that the softmax arithmetic (VALU) of one half rides in the shadow of the other
-      // half's MFMAs — one wave per SIMD has nobody else to overlap with:
-      //   first products (S = Q K^T, dP = dO V^T) of half 0
-      //   first products of half 1          | softmax of half 0
-      //   second products (dV, dK) of half 0 | softmax of half 1
-      //   second products of half 1
-      // Operand fragments are read one MFMA pair ahead of their use.
-      f32x16 s[2], dp[2];
-      uint32_t pw[2][8], dw[2][8];                         // packed P and dS per half
-      // one eighth of a half's softmax: elements 4 a + 2 h2 + {0, 1} of the lane's 16
-      auto softmax_piece = [&](int qt, int piece, auto masked_c) __attribute__((always_inline)) {
-        constexpr bool MASKED = decltype(masked_c)::value;
-        const int a = piece >> 1, h2 = piece & 1;
-        const int qoff = 32 * qt + 8 * a + 4 * lh + 2 * h2;
-        float pr[2], ds[2];
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          const int r = 4 * a + 2 * h2 + e;
-          float x = s[qt][r] * c;
-          if constexpr (MASKED) {
-            const int q = qt0 + qoff + e;
-            const bool ok = (q < p.Sq) & (key < p.Sk) & (!p.causal | (key <= q + off));
-            x = ok ? x : -INFINITY;                        // exponent -inf: P = 0, no branch
-          }
-          pr[e] = fast_exp2(x);
-          ds[e] = pr[e] * dp[qt][r];
+      for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          pf[qt][g] = lds_read_b128(xch, ((qt * 2 + 0) * 2 + g) * 1024 + lane * 16);
+          dsf[qt][g] = lds_read_b128(xch, ((qt * 2 + 1) * 2 + g) * 1024 + lane * 16);
         }
-        pw[qt][2 * a + h2] = pack2<T>(pr[0], pr[1]);
-        dw[qt][2 * a + h2] = pack2<T>(ds[0], ds[1]);
-      };
-      // S - LSE / scale and dP - Delta of one half: the accumulators start from the
-      // staged -LSE / scale and -Delta of their rows (lane's rows 8 a + 4 lh + 0..3),
-      // then 8 k steps of two MFMAs; `between(ks)` follows each pair
-      auto first_products = [&](int qt, auto&& between) __attribute__((always_inline)) {
-        f32x16 s0, dp0;
-#pragma unroll
-        for (int a = 0; a < 4; ++a) {
-          const int qoff = 32 * qt + 8 * a + 4 * lh;
-          const float4 l4 = *reinterpret_cast<const float4*>(base + 2 * TILE + qoff * 4);
-          const float4 d4 = *reinterpret_cast<const float4*>(base + 2 * TILE + FB_BQT * 4 + qoff * 4);
-          s0[4 * a] = l4.x; s0[4 * a + 1] = l4.y; s0[4 * a + 2] = l4.z; s0[4 * a + 3] = l4.w;
-          dp0[4 * a] = d4.x; dp0[4 * a + 1] = d4.y; dp0[4 * a + 2] = d4.z; dp0[4 * a + 3] = d4.w;
-        }
-        uint4 qfr[2], dofr[2];
-        qfr[0] = lds_read_b128(base, row_rd[0] + qt * 32 * ROWB);
-        dofr[0] = lds_read_b128(base, TILE + row_rd[0] + qt * 32 * ROWB);
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-          const int cur = ks & 1;
-          if (ks + 1 < KSTEPS) {
-            qfr[cur ^ 1] = lds_read_b128(base, row_rd[ks + 1] + qt * 32 * ROWB);
-            dofr[cur ^ 1] = lds_read_b128(base, TILE + row_rd[ks + 1] + qt * 32 * ROWB);
-          }
-          if (ks == 0) {
-            s[qt] = mfma_32x32x16<T>(qfr[cur], kf[ks], s0);
-            dp[qt] = mfma_32x32x16<T>(dofr[cur], vf[ks], dp0);
-          } else {
-            s[qt] = mfma_32x32x16<T>(qfr[cur], kf[ks], s[qt]);
-            dp[qt] = mfma_32x32x16<T>(dofr[cur], vf[ks], dp[qt]);
-          }
-          between(ks);
-        }
-      };
-      // dV += dO^T P and dK += Q^T dS of one half: (g, dt) steps of two MFMAs
-      auto second_products = [&](int qt, auto&& between) __attribute__((always_inline)) {
-        const uint4 pf[2] = {make_uint4(pw[qt][0], pw[qt][1], pw[qt][2], pw[qt][3]),
-                             make_uint4(pw[qt][4], pw[qt][5], pw[qt][6], pw[qt][7])};
-        const uint4 dsf[2] = {make_uint4(dw[qt][0], dw[qt][1], dw[qt][2], dw[qt][3]),
-                              make_uint4(dw[qt][4], dw[qt][5], dw[qt][6], dw[qt][7])};
-        auto tr_frags = [&](int i, uint4& qT, uint4& oT) {
-          const int dt = i % DT, g = i / DT;
-          const uint32_t o = (qt * 32 + g * 16) * ROWB;
-          const uint2 qlo = lds_read_tr16_b64(base + tr_lo[dt] + o);
-          const uint2 qhi = lds_read_tr16_b64(base + tr_hi[dt] + o);
-          const uint2 olo = lds_read_tr16_b64(base + TILE + tr_lo[dt] + o);
-          const uint2 ohi = lds_read_tr16_b64(base + TILE + tr_hi[dt] + o);
-          qT = make_uint4(qlo.x, qlo.y, qhi.x, qhi.y);
-          oT = make_uint4(olo.x, olo.y, ohi.x, ohi.y);
-        };
-        constexpr int NSTEP = 2 * DT;
-        uint4 qT[2], oT[2];
-        tr_frags(0, qT[0], oT[0]);
-#pragma unroll
-        for (int i = 0; i < NSTEP; ++i) {
-          const int cur = i & 1;
-          if (i + 1 < NSTEP) tr_frags(i + 1, qT[cur ^ 1], oT[cur ^ 1]);
-          const int dt = i % DT, g = i / DT;
-          dv[dt] = mfma_32x32x16<T>(oT[cur], pf[g], dv[dt]);
-          dk[dt] = mfma_32x32x16<T>(qT[cur], dsf[g], dk[dt]);
-          between(i);
-        }
-      };
-      static_assert(KSTEPS == 8 || KSTEPS == 4, "softmax pieces are spread over the k steps");
-      auto none = [](int) {};
-      // lane: key, queries qt0 + 32 qt + 8 (r/4) + 4 lh + r % 4.  Only tiles that touch
-      // the causal diagonal or the end of Q / K pay for the per-pair mask.
-      const bool need_mask = (qt0 + FB_BQT > p.Sq) || (wave_k0 + 32 > p.Sk) ||
-                             (p.causal && wave_k0 + 31 > qt0 + off);
-      auto run = [&](auto masked_c) __attribute__((always_inline)) {
-        // 8 softmax pieces per half over KSTEPS (first products) or 2 DT (second) slots
-        constexpr int PER1 = 8 / KSTEPS, PER2 = 8 / (2 * DT);
-        first_products(0, none);
-        if (has_next) load_part(nxt_head, nxt_tile, st ^ 1, 1);
-        first_products(1, [&](int ks) {
-#pragma unroll
-          for (int u = 0; u < PER1; ++u) softmax_piece(0, ks * PER1 + u, masked_c);
-        });
-        second_products(0, [&](int i) {
-#pragma unroll
-          for (int u = 0; u < PER2; ++u) softmax_piece(1, i * PER2 + u, masked_c);
-        });
-        second_products(1, none);
-      };
-      if (need_mask) run(std::true_type{});
-      else run(std::false_type{});
-    } else if (has_next) {
-      load_part(nxt_head, nxt_tile, st ^ 1, 1);
     }
-    cur_head = nxt_head;
-    cur_tile = nxt_tile;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();                          // P / dS taken: the producer may overwrite them
+    asm volatile("" ::: "memory");
+    if (live) {
+      const char* base = smem + st * STAGE;
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            const uint32_t o = (qt * 32 + g * 16) * ROWB;
+            const uint2 qlo = lds_read_tr16_b64(base + tr_lo[dt] + o);
+            const uint2 qhi = lds_read_tr16_b64(base + tr_hi[dt] + o);
+            const uint2 olo = lds_read_tr16_b64(base + TILE + tr_lo[dt] + o);
+            const uint2 ohi = lds_read_tr16_b64(base + TILE + tr_hi[dt] + o);
+            dv[dt] = mfma_32x32x16<T>(make_uint4(olo.x, olo.y, ohi.x, ohi.y), pf[qt][g], dv[dt]);
+            dk[dt] = mfma_32x32x16<T>(make_uint4(qlo.x, qlo.y, qhi.x, qhi.y), dsf[qt][g], dk[dt]);
+          }
+    }
+    cur_tile = ld_tile;
+    st = lst;
+    ld_head = nxt_head;
+    ld_tile = nxt_tile;
+    lst = nst;
     fa_wait_loads();
     __syncthreads();
   }

@@ -55,6 +55,17 @@ def test_attention_matches_oracle(lane, B, Hq, Hkv, Sq, Sk, D, causal, st):
     assert np.max(np.abs(lse - ref_lse)) <= TOL
 
 
+@pytest.mark.parametrize("scale", [0.3, 1e-3, 0.0, -0.07])
+def test_attention_scales(lane, scale):
+    """Any finite scale: a negative one turns the row maximum of the raw scores into
+    the minimum of the scaled ones, a zero one gives uniform weights."""
+    q, k, v = _qkv(1, 4, 2, 130, 200, 128, 19, "f16")
+    ref_o, ref_lse = orc.flash_attn_dense(_f32(q), _f32(k), _f32(v), scale=scale, causal=True)
+    o, lse = ops.gqa_attention(q, k, v, scale=scale, causal=True, return_lse=True, out="f32")
+    assert orc.max_rel_err(o, ref_o) <= TOL
+    assert np.max(np.abs(lse - ref_lse)) <= TOL
+
+
 def test_attention_special_cases(lane):
     """Closed forms: causal row 0 sees only key 0 -> O[0] = V[0], LSE[0] = s00;
     identical keys -> uniform weights -> prefix mean of V."""

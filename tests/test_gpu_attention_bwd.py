@@ -56,6 +56,22 @@ def test_attention_backward_matches_oracle(lane, B, Hq, Hkv, Sq, Sk, D, causal, 
         assert orc.max_rel_err(got, ref) <= TOL[st], name
 
 
+@pytest.mark.parametrize("scale", [0.25, -0.05, 1e-3, 0.0])
+def test_attention_backward_scales(lane, scale):
+    """The kernels fold -LSE / scale into their accumulators; a negative or tiny
+    scale goes the same way, a zero one (uniform P over the visible keys) is served
+    by the kernels that do not divide by it."""
+    do, q, k, v = _inputs(1, 4, 2, 130, 200, 128, 41, "f16")
+    ref = orc.flash_attn_backward(_f32(do), _f32(q), _f32(k), _f32(v), scale=scale, causal=True)
+    got = ops.flash_attn_backward(do, q, k, v, scale=scale, causal=True)
+    for g, r, name in zip(got, ref, ("dQ", "dK", "dV")):
+        assert not np.isnan(g).any(), name
+        if np.abs(r).max() == 0:
+            assert np.abs(g).max() <= 1e-6, name
+        else:
+            assert orc.max_rel_err(g, r) <= TOL["f16"], name
+
+
 def test_attention_backward_closed_forms(lane):
     """One key: P = 1 for every query, so dV = sum of dO rows, dQ = dK = 0.
     dO = 0 gives all-zero gradients."""
