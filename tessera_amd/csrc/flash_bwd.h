@@ -115,7 +115,15 @@ __global__ __launch_bounds__(FB_DQ_THREADS, 1) void flash_bwd_dq_kernel(const Fl
 
   const int qblocks = (p.Sq + FB_BQ - 1) / FB_BQ;
   const int qb = qblocks - 1 - blockIdx.x / (p.B * p.Hq);      // heavy causal blocks first
-  const int bh = blockIdx.x % (p.B * p.Hq);
+  int bh = blockIdx.x % (p.B * p.Hq);
+  if ((p.B * p.Hkv) % 8 == 0) {
+    // Workgroups go to the XCDs round robin.  Runs of 8 ratio workgroups take 8 KV heads,
+    // one per XCD, with all the query heads of a group on their KV head's XCD: the
+    // workgroups that walk the same K / V tiles share one L2.
+    const int ratio = p.Hq / p.Hkv;
+    const int w = bh % (8 * ratio);
+    bh = ((bh / (8 * ratio)) * 8 + (w & 7)) * ratio + (w >> 3);
+  }
   const int b = bh / p.Hq, hq = bh % p.Hq;
   const int hkv = (int)(((long)hq * p.Hkv) / p.Hq);
   const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
@@ -367,12 +375,17 @@ __global__ __launch_bounds__(FB_DKV_THREADS) void flash_bwd_dkdv_kernel(const Fl
     const int qt0 = tile * FB_BQT;
     return wave_k0 < p.Sk && (!p.causal || wave_k0 <= min(qt0 + FB_BQT, p.Sq) - 1 + off);
   };
+  // Walk order: query tiles from the last one down, the group's query heads innermost.
+  // Every key block of a KV head starts at the same tile and moves at the same pace, so
+  // the workgroups that share Q / dO tiles (same XCD: blockIdx % 8 is the head's) read
+  // them at the same time and the XCD's L2 serves all but one of those reads.
   auto next_of = [&](int& head, int& tile) {
-    if (++tile == qtiles) { tile = t_first; ++head; }
+    if (++head == ratio) { head = 0; --tile; }
   };
+  const int t_last = qtiles - 1;
   char* xch = smem + XCH + grp * 8192;
 
-  if (nsteps > 0) load_tile(0, t_first, 0);
+  if (nsteps > 0) load_tile(0, t_last, 0);
   fa_wait_loads();
   __syncthreads();
 
@@ -388,7 +401,7 @@ __global__ __launch_bounds__(FB_DKV_THREADS) void flash_bwd_dkdv_kernel(const Fl
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) row_rd[ks] = l32 * ROWB + ((((ks << 1) | lh) ^ bwd_swz<D>(l32)) << 4);
 
-    int cur_head = 0, cur_tile = t_first, st = 0;          // tile of this iteration and its stage
+    int cur_head = 0, cur_tile = t_last, st = 0;           // tile of this iteration and its stage
     for (int i = 0; i <= nsteps; ++i) {
       int nxt_head = cur_head, nxt_tile = cur_tile;
       next_of(nxt_head, nxt_tile);
@@ -478,8 +491,8 @@ __global__ __launch_bounds__(FB_DKV_THREADS) void flash_bwd_dkdv_kernel(const Fl
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dk[dt][r] = 0.f; dv[dt][r] = 0.f; }
 
-  int ld_head = 0, ld_tile = t_first, lst = 0;             // tile i (whose successor is loaded) and its stage
-  int cur_tile = t_first, st = 0;                          // tile i - 1 and its stage (from i = 1 on)
+  int ld_head = 0, ld_tile = t_last, lst = 0;              // tile i (whose successor is loaded) and its stage
+  int cur_tile = t_last, st = 0;                           // tile i - 1 and its stage (from i = 1 on)
   for (int i = 0; i <= nsteps; ++i) {
     int nxt_head = ld_head, nxt_tile = ld_tile;
     next_of(nxt_head, nxt_tile);
