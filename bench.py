@@ -33,6 +33,7 @@ PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16/f16 MFMA
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_INT8_TOPS = 5000.0
 PEAK_HBM_GBS = 8000.0
+PEAK_CLOCK_MHZ = 2400.0         # shader clock the MFMA peaks are quoted at
 # HBM-side bytes one launch of the headline kernel moves: FETCH_SIZE + WRITE_SIZE per
 # dispatch from two counter runs of this script, each scaled by the same counter's
 # reading for the 1 GiB copy kernel (profiles/bench_all_kernels_hbm_bytes.txt).
@@ -262,6 +263,51 @@ def bench_moe(lane, steps, warmup):
             "dispatch_gbs": 2.0 * S * H * 2 / ev_disp / 1e6}
 
 
+def _smi_sample():
+    """(mean shader clock over the XCDs in MHz, socket power in W) from amd-smi, or None."""
+    import subprocess
+    try:
+        r = subprocess.run(["/opt/rocm/bin/amd-smi", "metric", "-p", "-c", "--json"], capture_output=True, text=True,
+                           timeout=20)
+        j = json.loads(r.stdout)
+        g = j[0] if isinstance(j, list) else j["gpu_data"][0]
+        clk = [v["clk"]["value"] for k, v in g["clock"].items() if k.startswith("gfx_")]
+        return float(np.mean(clk)), float(g["power"]["socket_power"]["value"])
+    except (OSError, ValueError, KeyError, IndexError, TypeError, subprocess.SubprocessError):
+        return None
+
+
+def _sustained(lane, fn, seconds):
+    """Launch `fn` back to back on a second thread for 1 s + `seconds` and sample clock and
+    power over the last `seconds`: ms per launch, mean clock, mean power."""
+    import threading
+    stop, count = [False], [0]
+
+    def loop():
+        while not stop[0]:
+            for _ in range(20):
+                fn()
+            lane.synchronize()
+            count[0] += 20
+    th = threading.Thread(target=loop)
+    th.start()
+    time.sleep(1.0)                                           # clocks settle
+    n0, t0, seen = count[0], time.perf_counter(), []
+    while time.perf_counter() - t0 < seconds:
+        got = _smi_sample()
+        if got:
+            seen.append(got)
+        else:
+            time.sleep(0.1)
+    n1, t1 = count[0], time.perf_counter()
+    stop[0] = True
+    th.join()
+    if not seen:
+        return {"error": "amd-smi gave no reading"}
+    return {"ms": (t1 - t0) / max(n1 - n0, 1) * 1e3, "gfx_clock_mhz": float(np.mean([c for c, _ in seen])),
+            "socket_power_w": float(np.mean([w for _, w in seen])), "samples": len(seen)}
+
+
 def clock_and_power_trace(lane, seconds=4.0):
     """Shader clock (mean over the XCDs) and socket power, sampled with amd-smi while
     each kernel runs back to back on a second thread, on random and on constant
@@ -269,43 +315,9 @@ def clock_and_power_trace(lane, seconds=4.0):
     the kernel's schedule: the MFMA peak is quoted at 2400 MHz, and a launch that runs
     at 1700 MHz cannot pass 71 % of it whatever its instruction stream."""
     import ctypes
-    import subprocess
-    import threading
-
-    def sample():
-        r = subprocess.run(["/opt/rocm/bin/amd-smi", "metric", "-p", "-c", "--json"], capture_output=True, text=True)
-        try:
-            j = json.loads(r.stdout)
-            g = j[0] if isinstance(j, list) else j["gpu_data"][0]
-            clk = [v["clk"]["value"] for k, v in g["clock"].items() if k.startswith("gfx_")]
-            return float(np.mean(clk)), float(g["power"]["socket_power"]["value"])
-        except (ValueError, KeyError, IndexError, TypeError):
-            return None
 
     def measure(fn):
-        stop, count = [False], [0]
-
-        def loop():
-            while not stop[0]:
-                for _ in range(20):
-                    fn()
-                lane.synchronize()
-                count[0] += 20
-        th = threading.Thread(target=loop)
-        th.start()
-        time.sleep(1.0)                                       # clocks settle
-        n0, t0, seen = count[0], time.perf_counter(), []
-        while time.perf_counter() - t0 < seconds:
-            got = sample()
-            if got:
-                seen.append(got)
-        n1, t1 = count[0], time.perf_counter()
-        stop[0] = True
-        th.join()
-        if not seen:
-            return {"error": "amd-smi gave no reading"}
-        return {"ms": (t1 - t0) / max(n1 - n0, 1) * 1e3, "gfx_clock_mhz": float(np.mean([c for c, _ in seen])),
-                "socket_power_w": float(np.mean([w for _, w in seen])), "samples": len(seen)}
+        return _sustained(lane, fn, seconds)
 
     lib = lane.load()
     rng = np.random.default_rng(1)
@@ -315,7 +327,7 @@ def clock_and_power_trace(lane, seconds=4.0):
             return lane.DeviceBuffer.from_host(np.full(shape, 0x3C3C, np.uint16))
         return lane.DeviceBuffer.from_host(_bf16(rng.standard_normal(shape, dtype=np.float32)))
 
-    out = {"idle": dict(zip(("gfx_clock_mhz", "socket_power_w"), sample() or (None, None)))}
+    out = {"idle": dict(zip(("gfx_clock_mhz", "socket_power_w"), _smi_sample() or (None, None)))}
     M = N = K = 8192
     B, Hq, Hkv, S, D = 4, 32, 8, 4096, 128
     scale = ctypes.c_float(1.0 / np.sqrt(D))
@@ -376,6 +388,7 @@ def main() -> int:
     ap.add_argument("--only-headline", action="store_true", help="skip the `also` measurements")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a 1 GiB copy kernel (counter calibration for profiled runs)")
+    ap.add_argument("--no-clock", action="store_true", help="skip the 3 s clock / power reading of the headline kernel")
     ap.add_argument("--clocks", action="store_true",
                     help="instead of the bench line: shader clock and socket power under each kernel")
     args = ap.parse_args()
@@ -408,6 +421,21 @@ def main() -> int:
     }
     if copy_cal:
         result["copy_calibration"] = copy_cal
+    if not args.no_clock:
+        # the same launches kept up for 3 s: what clock the board grants this kernel on this
+        # data (the peak is quoted at PEAK_CLOCK_MHZ), and the busy fraction at that clock
+        lib = lane.load()
+        da, db, dd = lane.DeviceBuffer.from_host(a), lane.DeviceBuffer.from_host(b), lane.DeviceBuffer(M * N * 2)
+        held = _sustained(lane, lambda: lib.tessera_gfx950_gemm_bf16_bf16_dev(da.ptr, db.ptr, dd.ptr, M, N, K, None),
+                          2.0)
+        for buf in (da, db, dd):
+            buf.close()
+        if "ms" in held:
+            tf = flop / held["ms"] / 1e9
+            held.update({"tflops_sustained": tf, "peak_clock_mhz": PEAK_CLOCK_MHZ,
+                         "frac_of_peak_at_measured_clock":
+                             tf / (PEAK_BF16_TFLOPS * held["gfx_clock_mhz"] / PEAK_CLOCK_MHZ)})
+        result["clock_under_load"] = held
     if not args.no_cpu:
         ref, result["cpu_baseline"] = cpu_baseline(A, B)
         got = (out.astype(np.uint32) << 16).view(np.float32)
