@@ -158,7 +158,6 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
     qlin = blockIdx.x;
     kvlin = qlin / p.ratio;
   }
-  const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
 
   const int q0 = qb * FA_BQ;                  // first query row of the workgroup
   const int qw = q0 + wave * (32 * QT);       // first query row of the wave
@@ -535,7 +534,6 @@ __global__ void flash_fwd_generic_kernel(const FlashParams p, int D) {
   const int hq = (int)((row / p.Sq) % p.Hq);
   const int b = (int)(row / ((long)p.Sq * p.Hq));
   const int hkv = (int)(((long)hq * p.Hkv) / p.Hq);
-  const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
   const uint16_t* q = p.Q + row * D;
   const uint16_t* Kb = p.K + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
   const uint16_t* Vb = p.V + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
@@ -544,7 +542,6 @@ __global__ void flash_fwd_generic_kernel(const FlashParams p, int D) {
   float m = -INFINITY, l = 0.f;
   int jmin, jmax;
   key_bounds(qi, p.Sq, p.Sk, p.causal, p.window, jmin, jmax);
-  (void)off;
   for (int j = jmin; j <= jmax; ++j) {
     float s = 0.f;
     for (int d = 0; d < D; ++d) s += from_storage<T>(q[d]) * from_storage<T>(Kb[(long)j * D + d]);

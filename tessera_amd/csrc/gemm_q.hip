@@ -94,6 +94,7 @@ __global__ void quantize_e4m3_kernel(const float* x, long n, float scale_in, con
 __global__ void quantize_i8_rows_kernel(const float* x, int M, int N, int8_t* q, float* scales) {
   __shared__ float red[4];
   const int m = blockIdx.x;
+  if (m >= M) return;
   const float* row = x + (long)m * N;
   float mx = 0.f;
   for (int n = threadIdx.x; n < N; n += blockDim.x) mx = fmaxf(mx, fabsf(row[n]));

@@ -228,6 +228,7 @@ int route_dev(const float* scores, int T, int E, int k, int normalize, int capac
 __global__ __launch_bounds__(256) void dispatch_kernel(const char* x, const int32_t* token_of_slot, char* x_perm,
                                                        int T, int S, long row_bytes) {
   const int s = blockIdx.x;
+  if (s >= S) return;
   const int t = token_of_slot[s];
   if (t < 0 || t >= T) return;
   const char* src = x + (long)t * row_bytes;
