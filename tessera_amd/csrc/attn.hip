@@ -29,7 +29,7 @@ int launch_flash(const FlashParams& p, hipStream_t s) {
   if (attr_err != hipSuccess) return kDeviceFailed;
   const int qblocks = ceil_div(p.Sq, FA_BQ);
   const bool xcd_grouped = (p.B * p.Hkv) % 8 == 0;
-  const dim3 grid = xcd_grouped ? dim3(8 * p.ratio, p.B * p.Hkv / 8, qblocks) : dim3(p.B * p.Hq, 1, qblocks);
+  const dim3 grid = xcd_grouped ? dim3(8 * p.ratio, qblocks, p.B * p.Hkv / 8) : dim3(p.B * p.Hq, qblocks, 1);
   hipLaunchKernelGGL(kern, grid, dim3(FA_THREADS), kSmem, s, p);
   return launch_status();
 }

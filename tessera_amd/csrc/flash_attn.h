@@ -139,20 +139,21 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
   const int l32 = lane & 31, lh = lane >> 5;
 
   // Work order.  Workgroups are dealt to the 8 XCDs round-robin by their linear id.
-  // Levels of equal cost (one query block index for every (batch, head)) are
-  // issued heaviest first — with a causal mask the last block has the longest key
-  // range — so every XCD receives the same mix, and inside a level the (batch,
-  // head) pairs are permuted so that all query heads sharing one KV head land on
-  // the same XCD and find its K/V in that XCD's L2.
-  // The grid is (8 * ratio, B * Hkv / 8, query blocks) when B * Hkv is a multiple of 8,
-  // else (B * Hq, 1, query blocks): x runs fastest in the dispatch order, so the
-  // linear order is the one described above and no index needs a division.
+  // The grid is (8 * ratio, query blocks, B * Hkv / 8) when B * Hkv is a multiple of 8:
+  // x runs fastest in the dispatch order, so a run of 8 * ratio workgroups puts the
+  // query heads that share a KV head on one XCD, where they find its K / V in that
+  // XCD's L2; then come the query blocks of those heads, heaviest first (with a causal
+  // mask the last block has the longest key range); then the next 8 KV heads.  An XCD
+  // therefore works on one or two KV heads at a time (2 MB of K and V each at
+  // S = 4096, against 4 MB of L2) instead of on all of its heads at once.  Otherwise
+  // the grid is (B * Hq, query blocks, 1), heaviest blocks first.  No index needs a
+  // division either way.
   // qlin / kvlin: linear (batch, head) index of the query head / of its KV head.
-  const int qb = (int)gridDim.z - 1 - (int)blockIdx.z;
+  const int qb = (int)gridDim.y - 1 - (int)blockIdx.y;
   int qlin, kvlin;
-  if (gridDim.y > 1 || (int)gridDim.x == 8 * p.ratio) {
+  if (gridDim.z > 1 || (int)gridDim.x == 8 * p.ratio) {
     const int w = blockIdx.x;
-    kvlin = blockIdx.y * 8 + (w & 7);
+    kvlin = blockIdx.z * 8 + (w & 7);
     qlin = kvlin * p.ratio + (w >> 3);
   } else {
     qlin = blockIdx.x;
