@@ -114,15 +114,18 @@ __global__ __launch_bounds__(FB_DQ_THREADS, 1) void flash_bwd_dq_kernel(const Fl
   const int l32 = lane & 31, lh = lane >> 5, r16 = lane & 15;
 
   const int qblocks = (p.Sq + FB_BQ - 1) / FB_BQ;
-  const int qb = qblocks - 1 - blockIdx.x / (p.B * p.Hq);      // heavy causal blocks first
+  int qb = qblocks - 1 - blockIdx.x / (p.B * p.Hq);            // heavy causal blocks first
   int bh = blockIdx.x % (p.B * p.Hq);
   if ((p.B * p.Hkv) % 8 == 0) {
     // Workgroups go to the XCDs round robin.  Runs of 8 ratio workgroups take 8 KV heads,
-    // one per XCD, with all the query heads of a group on their KV head's XCD: the
-    // workgroups that walk the same K / V tiles share one L2.
+    // one per XCD, with all the query heads of a group on their KV head's XCD; then
+    // come the query blocks of those heads, heaviest first, then the next 8 KV heads.
+    // The workgroups that walk the same K / V tiles share one L2, and an XCD works on
+    // one or two KV heads at a time.
     const int ratio = p.Hq / p.Hkv;
-    const int w = bh % (8 * ratio);
-    bh = ((bh / (8 * ratio)) * 8 + (w & 7)) * ratio + (w >> 3);
+    const int w = blockIdx.x % (8 * ratio), r = blockIdx.x / (8 * ratio);
+    qb = qblocks - 1 - r % qblocks;
+    bh = ((r / qblocks) * 8 + (w & 7)) * ratio + (w >> 3);
   }
   const int b = bh / p.Hq, hq = bh % p.Hq;
   const int hkv = (int)(((long)hq * p.Hkv) / p.Hq);
@@ -321,8 +324,19 @@ __global__ __launch_bounds__(FB_DKV_THREADS) void flash_bwd_dkdv_kernel(const Fl
   const int grp = wave & 3;
   const int l32 = lane & 31, lh = lane >> 5, r16 = lane & 15;
 
-  const int kb = blockIdx.x / (p.B * p.Hkv);               // heavy key blocks first
-  const int bh = blockIdx.x % (p.B * p.Hkv);
+  // Heavy key blocks (low indices under a causal mask) first.  When B Hkv is a multiple
+  // of 8, an XCD (blockIdx % 8) takes one KV head after the other, all key blocks of a
+  // head together: they start at the same query tile and walk at the same pace, so the
+  // XCD's L2 serves all but one of their Q / dO reads; and a compute unit that ends a
+  // light block of one head takes a heavy block of the next, which evens the load out.
+  int kb = blockIdx.x / (p.B * p.Hkv);
+  int bh = blockIdx.x % (p.B * p.Hkv);
+  if ((p.B * p.Hkv) % 8 == 0) {
+    const int kblocks = (p.Sk + FB_BK - 1) / FB_BK;
+    const int r = blockIdx.x >> 3;
+    kb = r % kblocks;
+    bh = (r / kblocks) * 8 + (blockIdx.x & 7);
+  }
   const int b = bh / p.Hkv, hkv = bh % p.Hkv;
   const int ratio = p.Hq / p.Hkv;
   const int off = p.Sk > p.Sq ? p.Sk - p.Sq : 0;
