@@ -40,6 +40,8 @@ CASES = [
     (1, 1, 1, 50, 60, 32, True), (1, 3, 3, 40, 40, 48, False),
     (1, 2, 2, 1, 129, 128, True), (1, 4, 4, 513, 1, 128, False),
     (1, 2, 2, 700, 700, 256, True),
+    # B * Hkv a multiple of 8: the XCD-aware workgroup order
+    (2, 8, 4, 300, 520, 128, True), (1, 16, 8, 260, 260, 64, True), (2, 24, 8, 70, 330, 128, False),
 ]
 
 

@@ -41,6 +41,8 @@ CASES = [
     (1, 2, 2, 100, 77, 64, False), (1, 2, 1, 200, 333, 64, True), (1, 2, 2, 333, 200, 64, True),
     (1, 4, 4, 513, 129, 128, False), (1, 2, 2, 1, 129, 128, True),
     (1, 3, 3, 40, 40, 48, False), (1, 2, 1, 50, 60, 32, True),      # generic head dims
+    # B * Hkv a multiple of 8: the XCD-aware workgroup order
+    (2, 8, 4, 200, 264, 128, True), (1, 16, 8, 130, 130, 64, True), (2, 24, 8, 70, 330, 128, False),
 ]
 
 
