@@ -310,49 +310,92 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
   if (kt + 1 < ktiles) { kstep(kt, true_type{}, mode0{}, mode0{}); ++kt; }
   kstep(kt, false_type{}, mode0{}, mode0{});
 
-  // acc[i][j][r]: row m = 32 i + l32, col n = 32 j + 8 (r / 4) + 4 h + (r % 4).
+  // ---- epilogue ----
+  // acc[i][j][r]: row m = 32 i + l32, col n = 32 j + 8 (r / 4) + 4 h + (r % 4): a lane owns
+  // runs of four columns of 32 different rows, and a store issued from that layout
+  // touches 32 cache lines with 16 (or 8) bytes each.  The wave stages its tile through
+  // its share of the (now free) LDS instead and writes whole row segments, 16 bytes per
+  // lane with consecutive lanes along a row.
+  constexpr int DSZ = EPI == EPI8_SCALED_BF16 ? 2 : 4;
+  constexpr int ROWB = NJ * 32 * DSZ;                  // bytes of one row of the wave's 128-column tile
+  constexpr int PITCH = ROWB + 16;
+  constexpr int WAVE_LDS = G8_SMEM / 4;
+  constexpr int IB = WAVE_LDS / (32 * PITCH) >= MI ? MI : 2;   // 32-row blocks staged per pass
+  static_assert(IB * 32 * PITCH <= WAVE_LDS && MI % IB == 0, "epilogue staging does not fit");
+  constexpr int LPR = ROWB / 16, RPI = 64 / LPR;       // lanes per row, rows per store instruction
+  __syncthreads();                                     // nobody reads the operand tiles any more
+  char* stg = smem + wave * WAVE_LDS;
+  const int st_row = lane / LPR, st_chunk = lane % LPR;
+  const int st_n = n_begin + wn * 128 + st_chunk * (16 / DSZ);
+  // one staged pass: `raw` stores the int32 accumulators themselves (the plain int8
+  // result, or the optional accumulator copy of the W8A8 form) into `out`
+  auto pass = [&](char* out, auto raw_c) __attribute__((always_inline)) {
+    constexpr bool RAW = decltype(raw_c)::value;
+    constexpr int PDSZ = RAW ? 4 : DSZ;
+    static_assert(!RAW || DSZ == 4, "raw accumulators are 4 bytes");
 #pragma unroll
-  for (int i = 0; i < MI; ++i) {
-    const int m = m_begin + wm * 128 + i * 32 + l32;
-    if (m >= p.M) continue;
-    float rs = 1.f;
-    if constexpr (EPI == EPI8_W8A8_F32) rs = p.row_scale[m];
+    for (int i0 = 0; i0 < MI; i0 += IB) {
 #pragma unroll
-    for (int j = 0; j < NJ; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n_begin + wn * 128 + j * 32 + q * 8 + lh * 4;
-        if (n >= p.N) continue;
-        const long o = (long)m * p.N + n;
-        if constexpr (EPI == EPI8_I32) {
-          *reinterpret_cast<int4*>(reinterpret_cast<int32_t*>(p.D) + o) =
-              make_int4(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
-        } else if constexpr (EPI == EPI8_W8A8_F32) {
-          const float4 cs = *reinterpret_cast<const float4*>(p.col_scale + n);
-          float4 out;
-          out.x = ((float)acc[i][j][q * 4 + 0] * rs) * cs.x;
-          out.y = ((float)acc[i][j][q * 4 + 1] * rs) * cs.y;
-          out.z = ((float)acc[i][j][q * 4 + 2] * rs) * cs.z;
-          out.w = ((float)acc[i][j][q * 4 + 3] * rs) * cs.w;
-          *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.D) + o) = out;
-          if (p.acc_out)
-            *reinterpret_cast<int4*>(p.acc_out + o) =
-                make_int4(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
-        } else {
-          const float v0 = ((float)acc[i][j][q * 4 + 0] * p.scale_a) * p.scale_b;
-          const float v1 = ((float)acc[i][j][q * 4 + 1] * p.scale_a) * p.scale_b;
-          const float v2 = ((float)acc[i][j][q * 4 + 2] * p.scale_a) * p.scale_b;
-          const float v3 = ((float)acc[i][j][q * 4 + 3] * p.scale_a) * p.scale_b;
-          if constexpr (EPI == EPI8_SCALED_F32) {
-            *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.D) + o) = make_float4(v0, v1, v2, v3);
-          } else {
-            uint2 pk;
-            pk.x = pack2<BF16>(v0, v1);
-            pk.y = pack2<BF16>(v2, v3);
-            *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.D) + o) = pk;
-          }
+      for (int ii = 0; ii < IB; ++ii) {
+        const int i = i0 + ii;
+        float rs = 1.f;
+        if constexpr (EPI == EPI8_W8A8_F32 && !RAW) {
+          const int m = m_begin + wm * 128 + i * 32 + l32;
+          rs = p.row_scale[m < p.M ? m : p.M - 1];
         }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            char* dst = stg + (ii * 32 + l32) * PITCH + (j * 32 + q * 8 + lh * 4) * PDSZ;
+            if constexpr (RAW) {
+              *reinterpret_cast<int4*>(dst) =
+                  make_int4(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+            } else if constexpr (EPI == EPI8_W8A8_F32) {
+              const int n = n_begin + wn * 128 + j * 32 + q * 8 + lh * 4;
+              // (a column past N is never stored; its scale read stays in range)
+              const float4 cs = *reinterpret_cast<const float4*>(p.col_scale + (n < p.N ? n : 0));
+              float4 o;
+              o.x = ((float)acc[i][j][q * 4 + 0] * rs) * cs.x;
+              o.y = ((float)acc[i][j][q * 4 + 1] * rs) * cs.y;
+              o.z = ((float)acc[i][j][q * 4 + 2] * rs) * cs.z;
+              o.w = ((float)acc[i][j][q * 4 + 3] * rs) * cs.w;
+              *reinterpret_cast<float4*>(dst) = o;
+            } else {
+              const float v0 = ((float)acc[i][j][q * 4 + 0] * p.scale_a) * p.scale_b;
+              const float v1 = ((float)acc[i][j][q * 4 + 1] * p.scale_a) * p.scale_b;
+              const float v2 = ((float)acc[i][j][q * 4 + 2] * p.scale_a) * p.scale_b;
+              const float v3 = ((float)acc[i][j][q * 4 + 3] * p.scale_a) * p.scale_b;
+              if constexpr (EPI == EPI8_SCALED_F32) {
+                *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
+              } else {
+                uint2 pk;
+                pk.x = pack2<BF16>(v0, v1);
+                pk.y = pack2<BF16>(v2, v3);
+                *reinterpret_cast<uint2*>(dst) = pk;
+              }
+            }
+          }
       }
+      __builtin_amdgcn_wave_barrier();                 // the wave's LDS operations run in order
+#pragma unroll
+      for (int it = 0; it < IB * 32 / RPI; ++it) {
+        const int row = it * RPI + st_row;
+        const uint4 v = lds_read_b128(stg, row * PITCH + st_chunk * 16);
+        const int m = m_begin + wm * 128 + i0 * 32 + row;
+        // N % 16 == 0 on this path: a 16-byte chunk is inside or outside as a whole
+        if (m < p.M && st_n < p.N) *reinterpret_cast<uint4*>(out + ((long)m * p.N + st_n) * PDSZ) = v;
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  };
+  if constexpr (EPI == EPI8_I32) {
+    pass(reinterpret_cast<char*>(p.D), true_type{});
+  } else {
+    pass(reinterpret_cast<char*>(p.D), false_type{});
+    if constexpr (EPI == EPI8_W8A8_F32) {
+      if (p.acc_out) pass(reinterpret_cast<char*>(p.acc_out), true_type{});
+    }
   }
 }
 
