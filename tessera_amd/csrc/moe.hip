@@ -164,24 +164,24 @@ __global__ __launch_bounds__(64) void place_kernel(const int32_t* expert_ids, co
     const int s = base + i0 + lane;
     const bool valid = s < S;
     const int e = valid ? expert_ids[s] : -1;
-    int rank = 0;
-    // Rank inside the expert in slot order: lanes sharing an expert are found one
-    // expert at a time; lower lanes are earlier slots.
-    unsigned long long todo = __ballot(valid);
-    while (todo) {
-      const int leader = __ffsll((long long)todo) - 1;
-      const int e0 = __shfl(e, leader, 64);
-      const unsigned long long same = __ballot(valid && e == e0);
-      // (the workgroup is one wave: its LDS operations execute in program order, so
-      // the leader's update is seen by the next round's reads without a barrier)
-      if (valid && e == e0) rank = cursor[e0] + __popcll(same & ((1ull << lane) - 1ull));
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      if (lane == leader) cursor[e0] += __popcll(same);
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      todo &= ~same;
+    // Rank inside the expert in slot order.  `same` = the lanes that hold this lane's
+    // expert, built from one ballot per bit of the expert index (all lanes at once, no
+    // loop over the experts present); lower lanes are earlier slots.
+    unsigned long long same = __ballot(valid);
+    for (int bit = 0; (1 << bit) < E; ++bit) {
+      const unsigned long long set = __ballot(valid && ((e >> bit) & 1));
+      same &= ((e >> bit) & 1) ? set : ~set;
     }
+    int rank = 0;
+    if (valid) rank = cursor[e] + __popcll(same & ((1ull << lane) - 1ull));
+    // (the workgroup is one wave: its LDS operations execute in program order, so the
+    // update below comes after every lane's read above and before the next round's)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    // the last lane of every expert present advances that expert's cursor
+    if (valid && (same >> lane) == 1ull) cursor[e] += __popcll(same);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
     if (valid && (capacity <= 0 || rank < capacity)) {
       const int pos = group_offsets[e] + rank;
       token_of_slot[pos] = s / k;
