@@ -161,7 +161,11 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
   }
 
   const int q0 = qb * FA_BQ;                  // first query row of the workgroup
-  const int qw = q0 + wave * (32 * QT);       // first query row of the wave
+  // Waves w and w + 4 share a SIMD.  Under a causal mask a wave's key range grows with
+  // its row block, so the upper four waves take the row blocks in reverse: every SIMD
+  // gets one of the blocks 0-3 and its mirror image 7-4, the same work on all four.
+  const int rblk = wave < FA_WAVES / 2 ? wave : FA_WAVES + FA_WAVES / 2 - 1 - wave;
+  const int qw = q0 + rblk * (32 * QT);       // first query row of the wave
   const uint16_t* Qb = p.Q + ((long)qlin * p.Sq) * D;
   const uint16_t* Kb = p.K + ((long)kvlin * p.Sk) * D;
   const uint16_t* Vb = p.V + ((long)kvlin * p.Sk) * D;
