@@ -173,6 +173,23 @@ def bench_quant(lane, steps, warmup):
                                             "gemm_i8"), steps, warmup)
     ops = 2.0 * M * N * K
     out["gemm_int8_4096x8192x8192"] = {"ms": ev, "tops": ops / ev / 1e9, "frac_mfma_peak": ops / ev / 1e9 / PEAK_INT8_TOPS}
+    # W8A8 with scales: f32(acc) * row_scale[m] * col_scale[n], f32 out, no accumulator copy
+    rs = lane.DeviceBuffer.from_host(rng.uniform(0.5, 1.5, M).astype(np.float32) / 127.0)
+    cs = lane.DeviceBuffer.from_host(rng.uniform(0.5, 1.5, N).astype(np.float32) / 127.0)
+    _, ev = _timed(lane, lambda: lane.check(lib.tessera_gfx950_gemm_w8a8_f32_dev(da.ptr, db.ptr, rs.ptr, cs.ptr, dd.ptr,
+                                                                                 None, M, N, K, None), "gemm_w8a8"),
+                   steps, warmup)
+    out["gemm_w8a8_scaled_4096x8192x8192"] = {"ms": ev, "tops": ops / ev / 1e9,
+                                              "frac_mfma_peak": ops / ev / 1e9 / PEAK_INT8_TOPS}
+    # per-row int8 quantiser of the f32 activation (reads 4 M K bytes, writes M K + 4 M)
+    xf = lane.DeviceBuffer.from_host(rng.standard_normal((M, K), dtype=np.float32))
+    xq, xs = lane.DeviceBuffer(M * K), lane.DeviceBuffer(M * 4)
+    _, ev = _timed(lane, lambda: lane.check(lib.tessera_gfx950_quantize_i8_f32_dev(xf.ptr, M, K, 1, xq.ptr, xs.ptr, None),
+                                            "quantize_i8"), steps, warmup)
+    qbytes = 5.0 * M * K + 4.0 * M
+    out["quantize_int8_rows_4096x8192"] = {"ms": ev, "gbs": qbytes / ev / 1e6, "frac_hbm_peak": qbytes / ev / 1e6 / PEAK_HBM_GBS}
+    for buf in (rs, cs, xf, xq, xs):
+        buf.close()
     # e4m3 codes with |value| <= 15 (no NaN codes)
     af = ((a8.view(np.uint8) & 0x80) | np.minimum(a8.view(np.uint8) & 0x7F, 0x47)).astype(np.uint8)
     bf = ((b8.view(np.uint8) & 0x80) | np.minimum(b8.view(np.uint8) & 0x7F, 0x47)).astype(np.uint8)

@@ -111,6 +111,54 @@ __global__ void quantize_i8_rows_kernel(const float* x, int M, int N, int8_t* q,
   }
 }
 
+// The same for rows of up to 256 * 16 * GV elements (a multiple of 16, 16-byte aligned):
+// a thread keeps its runs of 16 elements in registers between the absmax pass and the
+// quantising pass, so x is read from memory once, with 16-byte loads, and every run of
+// 16 codes leaves as one 16-byte store.
+template <int GV>
+__global__ __launch_bounds__(256) void quantize_i8_rows_vec_kernel(const float* x, int M, int N, int8_t* q,
+                                                                   float* scales) {
+  __shared__ float red[4];
+  const int m = blockIdx.x;
+  if (m >= M) return;
+  const float4* row = reinterpret_cast<const float4*>(x + (long)m * N);
+  const int groups = N / 16;
+  float4 v[GV][4];
+  float mx = 0.f;
+#pragma unroll
+  for (int u = 0; u < GV; ++u) {
+    const int g = threadIdx.x + 256 * u;
+    if (g < groups) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        v[u][c] = row[g * 4 + c];
+        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v[u][c].x), fabsf(v[u][c].y)), fmaxf(fabsf(v[u][c].z), fabsf(v[u][c].w))));
+      }
+    }
+  }
+  mx = warp_max(mx);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float scale = __fdiv_rn(fmaxf(mx, 1e-12f), 127.0f);
+  if (threadIdx.x == 0) scales[m] = scale;
+  auto code = [&](float f) -> uint32_t {
+    float t = __builtin_rintf(__fdiv_rn(f, scale));
+    t = fminf(fmaxf(t, -127.f), 127.f);
+    return (uint32_t)(uint8_t)(int8_t)t;
+  };
+  auto pack = [&](const float4& f) -> uint32_t {
+    return code(f.x) | (code(f.y) << 8) | (code(f.z) << 16) | (code(f.w) << 24);
+  };
+#pragma unroll
+  for (int u = 0; u < GV; ++u) {
+    const int g = threadIdx.x + 256 * u;
+    if (g < groups)
+      *reinterpret_cast<uint4*>(q + (long)m * N + g * 16) =
+          make_uint4(pack(v[u][0]), pack(v[u][1]), pack(v[u][2]), pack(v[u][3]));
+  }
+}
+
 // Column scales: each thread owns one column and walks the rows (coalesced
 // across the wavefront); two passes over x.
 __global__ void quantize_i8_cols_kernel(const float* x, int M, int N, int8_t* q, float* scales) {
@@ -147,9 +195,19 @@ int quantize_e4m3_dev(const float* x, int64_t n, float scale, void* codes, float
 int quantize_i8_dev(const float* x, int M, int N, int axis, void* q, float* scales, hipStream_t s) {
   if (M <= 0 || N <= 0 || !x || !q || !scales || (axis != 0 && axis != 1)) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
-  if (axis == 1)
-    hipLaunchKernelGGL(quantize_i8_rows_kernel, dim3(M), dim3(256), 0, s, x, M, N, static_cast<int8_t*>(q), scales);
-  else
+  if (axis == 1) {
+    int8_t* codes = static_cast<int8_t*>(q);
+    const int groups = N / 16;
+    const bool vec = N % 16 == 0 && groups <= 4 * 256 && aligned16(x) && aligned16(q);
+    if (vec && groups <= 256)
+      hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<1>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales);
+    else if (vec && groups <= 512)
+      hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<2>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales);
+    else if (vec)
+      hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<4>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales);
+    else
+      hipLaunchKernelGGL(quantize_i8_rows_kernel, dim3(M), dim3(256), 0, s, x, M, N, codes, scales);
+  } else
     hipLaunchKernelGGL(quantize_i8_cols_kernel, dim3(ceil_div(N, 64)), dim3(64), 0, s, x, M, N,
                        static_cast<int8_t*>(q), scales);
   return launch_status();

@@ -31,7 +31,9 @@ def test_int8_extremes(lane):
     assert np.all(ops.gemm_i8(a, b) == 128 * 128 * 4096)
 
 
-@pytest.mark.parametrize("M,N,K", [(64, 128, 256), (200, 304, 144), (33, 20, 17)])
+@pytest.mark.parametrize("M,N,K", [(64, 128, 256), (200, 304, 144), (33, 20, 17),
+                                   # row lengths on each side of the register-resident row quantiser's limits
+                                   (9, 16, 4096), (7, 16, 8192), (6, 16, 16384), (3, 16, 16400), (4, 16, 4104)])
 def test_quantize_int8_matches_oracle(lane, M, N, K):
     rng = np.random.default_rng(3)
     X = rng.standard_normal((M, K)).astype(np.float32)
