@@ -188,6 +188,13 @@ def bench_quant(lane, steps, warmup):
                                             "quantize_i8"), steps, warmup)
     qbytes = 5.0 * M * K + 4.0 * M
     out["quantize_int8_rows_4096x8192"] = {"ms": ev, "gbs": qbytes / ev / 1e6, "frac_hbm_peak": qbytes / ev / 1e6 / PEAK_HBM_GBS}
+    # per-tensor e4m3 quantiser with a dynamic scale: absmax pass + quantising pass
+    # (reads 8 M K bytes, writes M K)
+    _, ev = _timed(lane, lambda: lane.check(lib.tessera_gfx950_quantize_e4m3_f32_dev(xf.ptr, M * K, 0.0, xq.ptr, xs.ptr,
+                                                                                     None), "quantize_e4m3"),
+                   steps, warmup)
+    ebytes = 9.0 * M * K
+    out["quantize_e4m3_tensor_4096x8192"] = {"ms": ev, "gbs": ebytes / ev / 1e6, "frac_hbm_peak": ebytes / ev / 1e6 / PEAK_HBM_GBS}
     for buf in (rs, cs, xf, xq, xs):
         buf.close()
     # e4m3 codes with |value| <= 15 (no NaN codes)

@@ -45,14 +45,28 @@ __device__ __forceinline__ float warp_max(float v) {
   return v;
 }
 
-// Block-wide max of |x| folded into *out with an atomic max on the bit pattern
+// Workgroup-wide max of |x| folded into *out with one atomic max on the bit pattern
 // (valid for non-negative floats).
+// (x 16-byte aligned: the body runs on float4, the last n % 4 elements one by one)
 __global__ void absmax_kernel(const float* x, long n, unsigned* out) {
   float m = 0.f;
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
-    m = fmaxf(m, fabsf(x[i]));
+  const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x, nthreads = (long)gridDim.x * blockDim.x;
+  const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+  const long n4 = vec ? n / 4 : 0;
+  for (long i = tid; i < n4; i += nthreads) {
+    const float4 v = reinterpret_cast<const float4*>(x)[i];
+    m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+  }
+  for (long i = n4 * 4 + tid; i < n; i += nthreads) m = fmaxf(m, fabsf(x[i]));
+  // one atomic per workgroup: thousands of them on one address serialise
+  __shared__ float red[16];
   m = warp_max(m);
-  if ((threadIdx.x & 63) == 0) atomicMax(out, __builtin_bit_cast(unsigned, m));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < (int)(blockDim.x + 63) / 64; ++w) m = fmaxf(m, red[w]);
+    atomicMax(out, __builtin_bit_cast(unsigned, m));
+  }
 }
 
 // f32 (already clipped to +-448) -> e4m3fn byte, round-to-nearest-even with
@@ -83,11 +97,30 @@ __global__ void quantize_e4m3_kernel(const float* x, long n, float scale_in, con
     scale = fmaxf(__fdiv_rn(amax, 448.0f), 1e-12f);
   }
   if (scale_out && blockIdx.x == 0 && threadIdx.x == 0) *scale_out = scale;
-  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
-    float t = __fdiv_rn(x[i], scale);
+  auto code = [&](float f) -> uint32_t {
+    float t = __fdiv_rn(f, scale);
     t = fminf(fmaxf(t, -448.0f), 448.0f);
-    codes[i] = f32_to_e4m3(t);
+    return f32_to_e4m3(t);
+  };
+  const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x, nthreads = (long)gridDim.x * blockDim.x;
+  // runs of 16 elements: four 16-byte loads, one 16-byte store (both pointers 16-byte aligned)
+  const bool vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(codes)) & 15) == 0;
+  const long n16 = vec ? n / 16 : 0;
+  for (long g = tid; g < n16; g += nthreads) {
+    uint32_t w[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const float4 v = reinterpret_cast<const float4*>(x)[g * 4 + c];
+      // the hardware conversion (OCP e4m3, round to nearest even, gradual underflow) on
+      // values already clipped to +-448 gives the codes of f32_to_e4m3
+      auto clip = [&](float f) { return fminf(fmaxf(__fdiv_rn(f, scale), -448.0f), 448.0f); };
+      int pk = __builtin_amdgcn_cvt_pk_fp8_f32(clip(v.x), clip(v.y), 0, false);
+      pk = __builtin_amdgcn_cvt_pk_fp8_f32(clip(v.z), clip(v.w), pk, true);
+      w[c] = (uint32_t)pk;
+    }
+    reinterpret_cast<uint4*>(codes)[g] = make_uint4(w[0], w[1], w[2], w[3]);
   }
+  for (long i = n16 * 16 + tid; i < n; i += nthreads) codes[i] = (uint8_t)code(x[i]);
 }
 
 // One workgroup per row: absmax, scale = max(absmax, 1e-12) / 127, q = rint(x / scale).
@@ -181,15 +214,16 @@ int quantize_e4m3_dev(const float* x, int64_t n, float scale, void* codes, float
   const int blocks = (int)std::min<int64_t>((n + 255) / 256, 4096);
   unsigned* amax = nullptr;
   if (!(scale > 0.f)) {
-    if (hipMallocAsync(reinterpret_cast<void**>(&amax), sizeof(unsigned), s) != hipSuccess) return kDeviceFailed;
+    // the running maximum lives in the stream's own workspace (work on one stream runs in
+    // order, so nothing else on it uses the workspace meanwhile): no allocation per call
+    amax = static_cast<unsigned*>(stream_workspace(s, 256));
+    if (!amax) return kDeviceFailed;
     if (hipMemsetAsync(amax, 0, sizeof(unsigned), s) != hipSuccess) return kDeviceFailed;
     hipLaunchKernelGGL(absmax_kernel, dim3(blocks), dim3(256), 0, s, x, (long)n, amax);
   }
   hipLaunchKernelGGL(quantize_e4m3_kernel, dim3(blocks), dim3(256), 0, s, x, (long)n, scale, amax,
                      static_cast<uint8_t*>(codes), scale_out_dev);
-  int rc = launch_status();
-  if (amax && hipFreeAsync(amax, s) != hipSuccess) rc = kDeviceFailed;
-  return rc;
+  return launch_status();
 }
 
 int quantize_i8_dev(const float* x, int M, int N, int axis, void* q, float* scales, hipStream_t s) {

@@ -93,6 +93,17 @@ def test_e4m3_quantiser_matches_oracle(lane):
     assert np.array_equal(table[c2], table[finite])
     c3, _ = ops.quantize_fp8_codes(np.array([1e9, -1e9, 449.0, 0.0], np.float32), scale=1.0)
     assert list(c3) == [0x7E, 0xFE, 0x7E, 0x00]
+    # rounding boundaries: the midpoint of every pair of neighbouring grid values and the
+    # f32 on either side of it (ties to even), both signs, through the 16-wide path and
+    # the element-wise tail alike
+    grid = np.sort(np.unique(np.abs(table[finite]))).astype(np.float32)
+    mid = ((grid[:-1].astype(np.float64) + grid[1:].astype(np.float64)) / 2).astype(np.float32)
+    probe = np.concatenate([mid, np.nextafter(mid, np.float32(np.inf)), np.nextafter(mid, np.float32(-np.inf))])
+    probe = np.concatenate([probe, -probe]).astype(np.float32)
+    assert probe.size % 16 != 0
+    c4, _ = ops.quantize_fp8_codes(probe, scale=1.0)
+    o4, _, _ = orc.quantize_fp8_e4m3(probe, scale=1.0)
+    assert np.array_equal(c4, o4)
 
 
 @pytest.mark.parametrize("M,N,K", [(64, 64, 64), (256, 512, 1024), (130, 272, 208), (9, 21, 13)])
