@@ -208,6 +208,50 @@ __global__ void quantize_i8_cols_kernel(const float* x, int M, int N, int8_t* q,
   }
 }
 
+// Column scales for a wide matrix, in two fully parallel passes: a thread owns four
+// adjacent columns (16-byte loads, coalesced across the wavefront) and a chunk of
+// kColRows rows.  Pass 1 folds the chunk's absmax into amax_bits[n] with an atomic max on
+// the bit pattern (non-negative floats order like unsigned integers); pass 2 derives the
+// scale and writes the codes, four per 4-byte store.  N % 4 == 0, 16-byte aligned x.
+constexpr int kColRows = 64;
+__global__ __launch_bounds__(256) void absmax_cols_kernel(const float* x, int M, int N, unsigned* amax_bits) {
+  const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (n >= N) return;
+  const int m0 = blockIdx.y * kColRows, m1 = min(m0 + kColRows, M);
+  float4 mx = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int m = m0; m < m1; ++m) {
+    const float4 v = *reinterpret_cast<const float4*>(x + (long)m * N + n);
+    mx.x = fmaxf(mx.x, fabsf(v.x)); mx.y = fmaxf(mx.y, fabsf(v.y));
+    mx.z = fmaxf(mx.z, fabsf(v.z)); mx.w = fmaxf(mx.w, fabsf(v.w));
+  }
+  atomicMax(amax_bits + n + 0, __builtin_bit_cast(unsigned, mx.x));
+  atomicMax(amax_bits + n + 1, __builtin_bit_cast(unsigned, mx.y));
+  atomicMax(amax_bits + n + 2, __builtin_bit_cast(unsigned, mx.z));
+  atomicMax(amax_bits + n + 3, __builtin_bit_cast(unsigned, mx.w));
+}
+__global__ __launch_bounds__(256) void quantize_i8_cols_vec_kernel(const float* x, int M, int N,
+                                                                   const unsigned* amax_bits, int8_t* q,
+                                                                   float* scales) {
+  const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (n >= N) return;
+  const int m0 = blockIdx.y * kColRows, m1 = min(m0 + kColRows, M);
+  float sc[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    sc[e] = __fdiv_rn(fmaxf(__builtin_bit_cast(float, amax_bits[n + e]), 1e-12f), 127.0f);
+  if (blockIdx.y == 0) *reinterpret_cast<float4*>(scales + n) = make_float4(sc[0], sc[1], sc[2], sc[3]);
+  auto code = [&](float f, float scale) -> uint32_t {
+    float t = __builtin_rintf(__fdiv_rn(f, scale));
+    t = fminf(fmaxf(t, -127.f), 127.f);
+    return (uint32_t)(uint8_t)(int8_t)t;
+  };
+  for (int m = m0; m < m1; ++m) {
+    const float4 v = *reinterpret_cast<const float4*>(x + (long)m * N + n);
+    *reinterpret_cast<uint32_t*>(q + (long)m * N + n) =
+        code(v.x, sc[0]) | (code(v.y, sc[1]) << 8) | (code(v.z, sc[2]) << 16) | (code(v.w, sc[3]) << 24);
+  }
+}
+
 int quantize_e4m3_dev(const float* x, int64_t n, float scale, void* codes, float* scale_out_dev, hipStream_t s) {
   if (n <= 0 || !x || !codes) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
@@ -241,9 +285,20 @@ int quantize_i8_dev(const float* x, int M, int N, int axis, void* q, float* scal
       hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<4>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales);
     else
       hipLaunchKernelGGL(quantize_i8_rows_kernel, dim3(M), dim3(256), 0, s, x, M, N, codes, scales);
-  } else
+  } else if (N % 4 == 0 && aligned16(x) && aligned16(scales) && (reinterpret_cast<uintptr_t>(q) & 3) == 0 &&
+             ceil_div(M, kColRows) <= 65535) {
+    // the per-column running maxima live in the stream's own workspace
+    unsigned* amax = static_cast<unsigned*>(stream_workspace(s, (size_t)N * sizeof(unsigned)));
+    if (!amax) return kDeviceFailed;
+    if (hipMemsetAsync(amax, 0, (size_t)N * sizeof(unsigned), s) != hipSuccess) return kDeviceFailed;
+    const dim3 grid(ceil_div(N, 1024), ceil_div(M, kColRows));
+    hipLaunchKernelGGL(absmax_cols_kernel, grid, dim3(256), 0, s, x, M, N, amax);
+    hipLaunchKernelGGL(quantize_i8_cols_vec_kernel, grid, dim3(256), 0, s, x, M, N, amax, static_cast<int8_t*>(q),
+                       scales);
+  } else {
     hipLaunchKernelGGL(quantize_i8_cols_kernel, dim3(ceil_div(N, 64)), dim3(64), 0, s, x, M, N,
                        static_cast<int8_t*>(q), scales);
+  }
   return launch_status();
 }
 

@@ -33,7 +33,9 @@ def test_int8_extremes(lane):
 
 @pytest.mark.parametrize("M,N,K", [(64, 128, 256), (200, 304, 144), (33, 20, 17),
                                    # row lengths on each side of the register-resident row quantiser's limits
-                                   (9, 16, 4096), (7, 16, 8192), (6, 16, 16384), (3, 16, 16400), (4, 16, 4104)])
+                                   (9, 16, 4096), (7, 16, 8192), (6, 16, 16384), (3, 16, 16400), (4, 16, 4104),
+                                   # column counts that do / do not take the four-column weight quantiser
+                                   (10, 18, 200), (12, 1028, 130)])
 def test_quantize_int8_matches_oracle(lane, M, N, K):
     rng = np.random.default_rng(3)
     X = rng.standard_normal((M, K)).astype(np.float32)
