@@ -126,105 +126,31 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
   tn = r / rows;
 }
 
+// One BM x BN output tile: rows [m_begin, min(m_begin + BM, m_end)), column tile tn, of
+// the product whose operand and output bases are Ab / Bb / B2b / Db.  All threads of the
+// workgroup call it with the same arguments.
 template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED>
-__global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Params p) {
+__device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, const int m_begin, const int m_end,
+                                            const int tn, const uint16_t* Ab, const uint16_t* Bb,
+                                            const uint16_t* B2b, char* Db) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN;     // wave tile
   constexpr int MI = TM / 32, NJ = TN / 32;     // 32x32 MFMA tiles per wave
   constexpr bool SWIGLU = (EPI == EPI_SWIGLU16 || EPI == EPI_GATED_F32);   // two-source B tile
   // SwiGLU: the BN columns of the LDS B tile are [gate n0..n0+BN/2) | up n0..n0+BN/2);
-  // a wave's first NJ/2 column tiles are gate and the rest the matching up columns.
-  static_assert(!SWIGLU || (WN == 1 && NJ % 2 == 0), "SwiGLU form needs WN == 1");
+  // a wave's first NJ/2 column tiles are gate columns and the rest the matching up
+  // columns (wave column wn owns output columns wn*TN/2 .. of the tile).
+  static_assert(!SWIGLU || NJ % 2 == 0, "SwiGLU form needs an even number of column tiles per wave");
   using S = Gemm16Smem<BM, BN>;
   constexpr int A_CHUNKS = BM * 8 / NT;         // 16-byte chunks per thread per stage
   constexpr int B_CHUNKS = G16_BK * (BN / 8) / NT;
   static_assert(BM * 8 % NT == 0 && G16_BK * (BN / 8) % NT == 0, "tile/thread mismatch");
-
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int DSZ = (EPI == EPI_F32 || EPI == EPI_GATED_F32 || EPI == EPI_F32_FUSED) ? 4 : 2;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
-
-  // ---- which tile ---------------------------------------------------------
-  int tm, tn, m_begin, m_end;
-  const uint16_t* Ab = p.A;
-  const uint16_t* Bb = p.B;
-  const uint16_t* B2b = p.B2;
-  char* Db = (char*)p.D;
-  constexpr int DSZ = (EPI == EPI_F32 || EPI == EPI_GATED_F32 || EPI == EPI_F32_FUSED) ? 4 : 2;
-  if constexpr (GROUPED) {
-    // 1-D grid over the real tiles of all groups, ordered group-major, then n tile,
-    // then m tile.  Workgroup ids are dealt to the 8 XCDs round-robin, so XCD j takes
-    // the j-th contiguous eighth of that order: the tiles running together on one XCD
-    // then belong to one or two experts and share its weight slabs and row tiles in
-    // that XCD's L2.  The grid is sized from an upper bound; surplus blocks exit.
-    // The decode reads all E + 1 offsets.  Walking them with dependent scalar loads
-    // costs microseconds per workgroup, so each wave reads 64 groups per step with one
-    // coalesced load, scans their tile counts across its lanes and finds the group of
-    // its tile with a ballot.
-    auto tiles_of = [&](int g, int& lo, int& hi) -> int {
-      lo = g < p.groups ? p.offsets[g] : 0;
-      hi = g < p.groups ? p.offsets[g + 1] : 0;
-      return ((hi - lo + BM - 1) / BM) * p.tiles_n;
-    };
-    auto wave_scan = [&](int v) -> int {             // inclusive prefix sum over the 64 lanes
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        const int u = __shfl_up(v, d, 64);
-        if (lane >= d) v += u;
-      }
-      return v;
-    };
-    int total = 0;
-    for (int g0 = 0; g0 < p.groups; g0 += 64) {
-      int lo, hi;
-      total += __shfl(wave_scan(tiles_of(g0 + lane, lo, hi)), 63, 64);
-    }
-    total = __builtin_amdgcn_readfirstlane(total);
-    const int per = (total + 7) / 8;
-    const int slot = blockIdx.x >> 3;
-    const int lin = (blockIdx.x & 7) * per + slot;
-    if (slot >= per || lin >= total) return;
-    int e = -1, acc = 0, g_lo = 0, g_hi = 0, mt = 0;
-    for (int g0 = 0, base = 0; g0 < p.groups && e < 0; g0 += 64) {
-      int lo, hi;
-      const int cnt = tiles_of(g0 + lane, lo, hi);
-      const int incl = base + wave_scan(cnt);
-      const unsigned long long hit = __ballot(lin >= incl - cnt && lin < incl);
-      if (hit) {
-        const int src = __ffsll((long long)hit) - 1;
-        e = g0 + src;
-        acc = __shfl(incl - cnt, src, 64);
-        g_lo = __shfl(lo, src, 64);
-        g_hi = __shfl(hi, src, 64);
-        mt = (g_hi - g_lo + BM - 1) / BM;
-      }
-      base = __shfl(incl, 63, 64);
-    }
-    if (e < 0) return;
-    e = __builtin_amdgcn_readfirstlane(e);
-    acc = __builtin_amdgcn_readfirstlane(acc);
-    g_lo = __builtin_amdgcn_readfirstlane(g_lo);
-    g_hi = __builtin_amdgcn_readfirstlane(g_hi);
-    mt = __builtin_amdgcn_readfirstlane(mt);
-    const int r = lin - acc;
-    tn = r / mt;
-    tm = r - tn * mt;
-    m_begin = g_lo + tm * BM;
-    m_end = g_hi;
-    Bb += (long)e * p.strideB;
-    if constexpr (SWIGLU) B2b += (long)e * p.strideB;
-  } else {
-    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
-    const int z = blockIdx.z;
-    Ab += (long)z * p.strideA;
-    Bb += (long)z * p.strideB;
-    Db += (long)z * p.strideD * DSZ;
-    m_begin = tm * BM;
-    m_end = p.M;
-  }
   constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;   // output columns per tile
   const int n_begin = tn * BN_OUT;
   const int K = p.K;
@@ -281,8 +207,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   // step of MFMA time to land and loads / LDS writes are spread evenly over it.
   constexpr int KS = G16_BK / 16;
   constexpr int NC = A_CHUNKS + B_CHUNKS;
-  static_assert(NC % KS == 0, "chunks must split evenly over the k steps");
-  constexpr int CPG = NC / KS;
+  constexpr int CPG = (NC + KS - 1) / KS;       // (the last group is short when KS does not divide NC)
   uint4 st[NC];
   using std::true_type;
   using std::false_type;
@@ -314,9 +239,11 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     constexpr int MODE = decltype(mode_c)::value;
 #pragma unroll
     for (int q = g * CPG; q < (g + 1) * CPG; ++q) {
-      lstore1(q, buf_dst);
-      if constexpr (MODE == 1) gload1(q, k0_load, false_type{});
-      if constexpr (MODE == 2) gload1(q, k0_load, true_type{});
+      if (q < NC) {
+        lstore1(q, buf_dst);
+        if constexpr (MODE == 1) gload1(q, k0_load, false_type{});
+        if constexpr (MODE == 2) gload1(q, k0_load, true_type{});
+      }
     }
   };
 
@@ -334,7 +261,12 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   // half), columns n = 32j + 16*((lane>>4)&1) + 4*(r%4), r = lane & 15.
   const int r16 = lane & 15;
   const uint32_t b_rd0 = S::kAStage + (8 * lh + (r16 >> 2)) * S::kBPitch +
-                         (wn * TN + 16 * ((lane >> 4) & 1) + 4 * (r16 & 3)) * 2;
+                         (wn * (SWIGLU ? TN / 2 : TN) + 16 * ((lane >> 4) & 1) + 4 * (r16 & 3)) * 2;
+  // byte offset of the wave's j-th column tile inside its B rows (SwiGLU: the up
+  // columns start BN/2 columns after the gate columns)
+  auto b_col = [](int j) constexpr -> int {
+    return (SWIGLU && j >= NJ / 2) ? (BN / 2 + (j - NJ / 2) * 32) * 2 : j * 64;
+  };
 
   f32x16 acc[MI][NJ];
 #pragma unroll
@@ -354,7 +286,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
       af[slot][i] = lds_read_b128(base, a_rd[i] + ((((ks << 1) | lh) ^ a_sw[i]) << 4));
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      const char* pb = base + b_rd0 + ks * 16 * S::kBPitch + j * 64;
+      const char* pb = base + b_rd0 + ks * 16 * S::kBPitch + b_col(j);
       const uint2 lo = lds_read_tr16_b64(pb);
       const uint2 hi = lds_read_tr16_b64(pb + 4 * S::kBPitch);
       bf[slot][j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
@@ -480,7 +412,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   // barrier nobody reads the operand tiles any more
   __syncthreads();
   char* stg = smem + wave * WAVE_LDS;
-  const int nw0 = n_begin + (SWIGLU ? 0 : wn * TN);    // first output column of the wave
+  const int nw0 = n_begin + wn * (SWIGLU ? TN / 2 : TN);   // first output column of the wave
   const int st_row = lane / LPR, st_chunk = lane % LPR;
   const int st_n = nw0 + st_chunk * (16 / DSZ);
   // The activation and the presence of a bias are compile-time here: one compact,
@@ -573,6 +505,103 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   } else {
     emit(A0{}, false_type{});
   }
+}
+
+template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED>
+__global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Params p) {
+  constexpr bool SWIGLU = (EPI == EPI_SWIGLU16 || EPI == EPI_GATED_F32);
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int lane = threadIdx.x & 63;
+
+  // ---- which tile ---------------------------------------------------------
+  int tm, tn, m_begin, m_end;
+  const uint16_t* Ab = p.A;
+  const uint16_t* Bb = p.B;
+  const uint16_t* B2b = p.B2;
+  char* Db = (char*)p.D;
+  constexpr int DSZ = (EPI == EPI_F32 || EPI == EPI_GATED_F32 || EPI == EPI_F32_FUSED) ? 4 : 2;
+  if constexpr (GROUPED) {
+    // 1-D grid over the real tiles of all groups, ordered group-major, then n tile,
+    // then m tile.  Workgroup ids are dealt to the 8 XCDs round-robin, so XCD j takes
+    // the j-th contiguous eighth of that order: the tiles running together on one XCD
+    // then belong to one or two experts and share its weight slabs and row tiles in
+    // that XCD's L2.  The grid is sized from an upper bound; surplus blocks exit.
+    // The decode reads all E + 1 offsets.  Walking them with dependent scalar loads
+    // costs microseconds per workgroup, so each wave reads 64 groups per step with one
+    // coalesced load, scans their tile counts across its lanes and finds the group of
+    // its tile with a ballot.
+    auto tiles_of = [&](int g, int& lo, int& hi) -> int {
+      lo = g < p.groups ? p.offsets[g] : 0;
+      hi = g < p.groups ? p.offsets[g + 1] : 0;
+      return ((hi - lo + BM - 1) / BM) * p.tiles_n;
+    };
+    auto wave_scan = [&](int v) -> int {             // inclusive prefix sum over the 64 lanes
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int u = __shfl_up(v, d, 64);
+        if (lane >= d) v += u;
+      }
+      return v;
+    };
+    int total = 0;
+    for (int g0 = 0; g0 < p.groups; g0 += 64) {
+      int lo, hi;
+      total += __shfl(wave_scan(tiles_of(g0 + lane, lo, hi)), 63, 64);
+    }
+    total = __builtin_amdgcn_readfirstlane(total);
+    const int per = (total + 7) / 8;
+    const int slot = blockIdx.x >> 3;
+    const int lin = (blockIdx.x & 7) * per + slot;
+    if (slot >= per || lin >= total) return;
+    int e = -1, acc = 0, g_lo = 0, g_hi = 0, mt = 0;
+    for (int g0 = 0, base = 0; g0 < p.groups && e < 0; g0 += 64) {
+      int lo, hi;
+      const int cnt = tiles_of(g0 + lane, lo, hi);
+      const int incl = base + wave_scan(cnt);
+      const unsigned long long hit = __ballot(lin >= incl - cnt && lin < incl);
+      if (hit) {
+        const int src = __ffsll((long long)hit) - 1;
+        e = g0 + src;
+        acc = __shfl(incl - cnt, src, 64);
+        g_lo = __shfl(lo, src, 64);
+        g_hi = __shfl(hi, src, 64);
+        mt = (g_hi - g_lo + BM - 1) / BM;
+      }
+      base = __shfl(incl, 63, 64);
+    }
+    if (e < 0) return;
+    e = __builtin_amdgcn_readfirstlane(e);
+    acc = __builtin_amdgcn_readfirstlane(acc);
+    g_lo = __builtin_amdgcn_readfirstlane(g_lo);
+    g_hi = __builtin_amdgcn_readfirstlane(g_hi);
+    mt = __builtin_amdgcn_readfirstlane(mt);
+    const int r = lin - acc;
+    tn = r / mt;
+    tm = r - tn * mt;
+    m_begin = g_lo + tm * BM;
+    m_end = g_hi;
+    Bb += (long)e * p.strideB;
+    if constexpr (SWIGLU) B2b += (long)e * p.strideB;
+  } else {
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int z = blockIdx.z;
+    Ab += (long)z * p.strideA;
+    Bb += (long)z * p.strideB;
+    Db += (long)z * p.strideD * DSZ;
+    m_begin = tm * BM;
+    m_end = p.M;
+  }
+  if constexpr (GROUPED && BM == 256 && WM * WN == 4) {
+    // A group's last row tile is often nearly empty (rows per expert are a little over a
+    // multiple of BM about half of the time).  With at most 64 rows left the four waves
+    // share the columns of a 64-row tile instead: a quarter of the matrix work of the
+    // full tile, whose other 192 rows would be computed and thrown away.
+    if (m_end - m_begin <= 64) {
+      gemm16_tile<T, 64, BN, 1, 4, EPI, GROUPED>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db);
+      return;
+    }
+  }
+  gemm16_tile<T, BM, BN, WM, WN, EPI, GROUPED>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db);
 }
 
 }  // namespace tsr950

@@ -284,7 +284,7 @@ int launch_gemm16_grouped(Gemm16Params p, hipStream_t s) {
     return launch_status();
   }
   if constexpr (EPI == EPI_SWIGLU16) {
-    return launch_gemm16_tile<T, 256, 256, 4, 1, EPI, true>(p, s);
+    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true>(p, s);
   } else {
     if ((long)p.M >= 64L * p.groups) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true>(p, s);
     return launch_gemm16_tile<T, 128, 128, 2, 2, EPI, true>(p, s);

@@ -97,6 +97,8 @@ def test_dispatch_and_combine(lane):
     ([0, 0, 7], 64, 72),
     ([100, 200, 300, 400], 1408, 512),
     ([3, 5], 24, 40),
+    # last row tiles of 64 / 65 rows: either side of the short last-tile form
+    ([64, 65, 320, 321, 0, 256], 200, 328),
 ])
 def test_grouped_gemm(lane, sizes, K, N):
     E, T = len(sizes), int(sum(sizes))
@@ -129,6 +131,7 @@ def _swiglu_inputs(sizes, K, F, N, seed):
     ([512], 128, 128, 256),
     ([9, 200], 64, 1408, 320),
     ([3, 5, 0], 24, 40, 56),
+    ([64, 65, 320, 321, 0, 256], 200, 328, 136),
 ])
 def test_moe_swiglu_block(lane, sizes, K, F, N):
     x, wg, wu, wd = _swiglu_inputs(sizes, K, F, N, 5)
