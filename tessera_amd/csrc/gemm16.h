@@ -543,8 +543,12 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
       }
       return v;
     };
-    int total = 0;
-    for (int g0 = 0; g0 < p.groups; g0 += 64) {
+    // (the first 64 groups are fetched and scanned once, for the total and for the lookup)
+    int lo0, hi0;
+    const int cnt0 = tiles_of(lane, lo0, hi0);
+    const int incl0 = wave_scan(cnt0);
+    int total = __shfl(incl0, 63, 64);
+    for (int g0 = 64; g0 < p.groups; g0 += 64) {
       int lo, hi;
       total += __shfl(wave_scan(tiles_of(g0 + lane, lo, hi)), 63, 64);
     }
@@ -555,9 +559,11 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     if (slot >= per || lin >= total) return;
     int e = -1, acc = 0, g_lo = 0, g_hi = 0, mt = 0;
     for (int g0 = 0, base = 0; g0 < p.groups && e < 0; g0 += 64) {
-      int lo, hi;
-      const int cnt = tiles_of(g0 + lane, lo, hi);
-      const int incl = base + wave_scan(cnt);
+      int lo = lo0, hi = hi0, cnt = cnt0, incl = incl0;
+      if (g0 > 0) {
+        cnt = tiles_of(g0 + lane, lo, hi);
+        incl = base + wave_scan(cnt);
+      }
       const unsigned long long hit = __ballot(lin >= incl - cnt && lin < incl);
       if (hit) {
         const int src = __ffsll((long long)hit) - 1;

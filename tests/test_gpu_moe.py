@@ -116,6 +116,21 @@ def test_grouped_gemm(lane, sizes, K, N):
         ops.grouped_gemm(b16.from_float32(x), b16.from_float32(w), sizes, kind="masked")
 
 
+def test_grouped_gemm_more_than_64_experts(lane):
+    """The tile kernel looks its expert up 64 groups at a time: 150 experts of 0..300
+    rows cross that boundary twice, with empty groups and short last tiles among them."""
+    rng = np.random.default_rng(150)
+    sizes = [int(v) for v in rng.integers(0, 301, size=150)]
+    sizes[3] = sizes[64] = sizes[129] = 0
+    E, T, K, N = len(sizes), int(sum(sizes)), 192, 264
+    assert T >= 64 * E                      # the 256-row tile form is the one chosen
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    w = (rng.standard_normal((E, K, N)) / np.sqrt(K)).astype(np.float32)
+    ref = orc.grouped_gemm(x, w, sizes, store=False)
+    got = ops.grouped_gemm(b16.from_float32(x), b16.from_float32(w), sizes, out="f32")
+    assert orc.max_rel_err(got, ref) <= 1e-5
+
+
 def _swiglu_inputs(sizes, K, F, N, seed):
     E, T = len(sizes), int(sum(sizes))
     rng = np.random.default_rng(seed)
