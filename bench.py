@@ -226,6 +226,32 @@ def bench_gemm_constant_operands(lane, steps):
             "note": "constant operands: not the metric, shows the power limit on random data"}
 
 
+def bench_batched_small(lane, steps, warmup):
+    """The reference README's step(): A[4,128,64] f16 x W[4,64,256] f16 -> f32, one
+    strided-batched launch.  Launch-latency bound: microseconds per launch and the
+    rate of its 720,896 algorithmic bytes."""
+    Bt, M, K, N = 4, 128, 64, 256
+    rng = np.random.default_rng(0)
+    a = (rng.standard_normal((Bt, M, K)) / 8).astype(np.float16)
+    w = (rng.standard_normal((Bt, K, N)) / 8).astype(np.float16)
+    da, dw = lane.DeviceBuffer.from_host(a), lane.DeviceBuffer.from_host(w)
+    dd = lane.DeviceBuffer(Bt * M * N * 4)
+    fn = lane.load().tessera_gfx950_batched_gemm_f16_dev
+
+    def launch():
+        lane.check(fn(da.ptr, dw.ptr, dd.ptr, Bt, M, N, K, None), "batched_gemm_f16")
+
+    wall, ev = _timed(lane, launch, max(steps, 200), warmup)
+    got = dd.download((Bt, M, N), np.float32)
+    ref = np.matmul(a.astype(np.float32), w.astype(np.float32))
+    for buf in (da, dw, dd):
+        buf.close()
+    nbytes = a.nbytes + w.nbytes + got.nbytes
+    return {"workload": "batched_gemm_f16_4x128x64x256_f32out", "us": ev * 1e3, "us_wall": wall * 1e3,
+            "gbs": nbytes / ev / 1e6, "gflops": 2.0 * Bt * M * N * K / ev / 1e6,
+            "max_rel_vs_f32": float(np.max(np.abs(got - ref)) / np.max(np.abs(ref)))}
+
+
 def bench_decode(lane, steps, warmup):
     """Decode-shaped products (M rows against an 8192 x 8192 weight).  The launches
     cycle over four weight matrices inside the library's own timing loop: one matrix
@@ -472,6 +498,7 @@ def main() -> int:
         also["flash_attn_bwd"] = bench_attention_bwd(lane, s, w)
         also.update(bench_quant(lane, s, w))
         also["gemm_bf16_8192_constant_operands"] = bench_gemm_constant_operands(lane, s)
+        also["batched_gemm_readme_step"] = bench_batched_small(lane, s, w)
         also.update(bench_decode(lane, s, w))
         also["moe"] = bench_moe(lane, s, w)
         result["also"] = also
