@@ -9,6 +9,10 @@
 // registers) — one wave per SIMD, the full 512-register budget — which needs
 // 512 B of LDS operand reads per MFMA, half of the 128 B/clk the LDS sustains.
 //
+// The tile body is a device function (gemm16_tile); the grouped kernel also holds a
+// 64 x BN instantiation of it with the four waves side by side along the columns, used
+// for a group's last row tile when at most 64 rows are left.
+//
 // LDS staging (double buffered, one barrier per K step).
 //   A tile  [BM][64] 16-bit, 128-byte rows, 16-byte chunks XOR-swizzled by
 //           (row & 7): the 8 lanes that read one chunk column of 8 consecutive
