@@ -125,6 +125,7 @@ __global__ __launch_bounds__(64) void count_kernel(const int32_t* expert_ids, in
 __global__ __launch_bounds__(256) void scan_kernel(int32_t* chunk_counts, int chunks, int E, int capacity,
                                                    int32_t* group_sizes, int32_t* group_offsets,
                                                    int32_t* num_slots) {
+  __shared__ int sz[kMaxExperts];
   for (int e = threadIdx.x; e < E; e += blockDim.x) {
     int run = 0;
     for (int c0 = 0; c0 < chunks; c0 += 16) {          // 16 independent loads per round trip
@@ -137,17 +138,34 @@ __global__ __launch_bounds__(256) void scan_kernel(int32_t* chunk_counts, int ch
         run += v[u];
       }
     }
-    group_sizes[e] = (capacity > 0 && run > capacity) ? capacity : run;
+    sz[e] = (capacity > 0 && run > capacity) ? capacity : run;
+    group_sizes[e] = sz[e];
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int off = 0;
-    for (int e = 0; e < E; ++e) {
-      group_offsets[e] = off;
-      off += group_sizes[e];
+  // offsets: the first wave scans the sizes from LDS, a run of consecutive experts per
+  // lane (one thread summing them from global memory, a store between every two loads,
+  // took E dependent memory round trips)
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    const int per = (E + 63) / 64;
+    const int lo = min(lane * per, E), hi = min(lo + per, E);
+    int sum = 0;
+    for (int e = lo; e < hi; ++e) sum += sz[e];
+    int incl = sum;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int u = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += u;
     }
-    group_offsets[E] = off;
-    if (num_slots) *num_slots = off;
+    int run = incl - sum;
+    for (int e = lo; e < hi; ++e) {
+      group_offsets[e] = run;
+      run += sz[e];
+    }
+    if (lane == 63) {
+      group_offsets[E] = incl;
+      if (num_slots) *num_slots = incl;
+    }
   }
 }
 
@@ -253,22 +271,46 @@ __global__ void combine_count_kernel(const int32_t* token_of_slot, int S, int T,
 }
 // Single workgroup exclusive scan of cnt[T] -> off[T+1]; cnt is zeroed for reuse as cursors.
 __global__ __launch_bounds__(1024) void combine_scan_kernel(int32_t* cnt, int T, int32_t* off) {
-  __shared__ int part[1024];
+  __shared__ int wave_total[16];
   const int per = (T + 1023) / 1024;
-  const int lo = threadIdx.x * per, hi = min(lo + per, T);
+  const int lo = min((int)threadIdx.x * per, T), hi = min(lo + per, T);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int sum = 0;
   for (int i = lo; i < hi; ++i) sum += cnt[i];
-  part[threadIdx.x] = sum;
-  __syncthreads();
-  for (int d = 1; d < 1024; d <<= 1) {               // inclusive scan of the 1024 partial sums
-    const int v = (int)threadIdx.x >= d ? part[threadIdx.x - d] : 0;
-    __syncthreads();
-    part[threadIdx.x] += v;
-    __syncthreads();
+  // inclusive scan of the 1024 partial sums: inside each wave by shuffles, then over the
+  // 16 wave totals (two barriers in all)
+  int incl = sum;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int u = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += u;
   }
-  if (threadIdx.x == 1023) off[T] = part[1023];
-  int run = part[threadIdx.x] - sum;
-  for (int i = lo; i < hi; ++i) { const int v = cnt[i]; off[i] = run; run += v; cnt[i] = 0; }
+  if (lane == 63) wave_total[wave] = incl;
+  __syncthreads();
+  int before = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) {
+    const int v = wave_total[w];
+    before += w < wave ? v : 0;
+    total += v;
+  }
+  if (threadIdx.x == 0) off[T] = total;
+  int run = before + incl - sum;
+  // (the counts of a batch are fetched before the first store: a store between every two
+  // loads would make each of them a separate round trip)
+  for (int i0 = lo; i0 < hi; i0 += 8) {
+    int v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = i0 + u < hi ? cnt[i0 + u] : 0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (i0 + u < hi) {
+        off[i0 + u] = run;
+        cnt[i0 + u] = 0;
+      }
+      run += v[u];
+    }
+  }
 }
 __global__ void combine_fill_kernel(const int32_t* token_of_slot, int S, int T, const int32_t* off, int32_t* cursor,
                                     int32_t* list) {
