@@ -219,12 +219,15 @@ int route_dev(const float* scores, int T, int E, int k, int normalize, int capac
   if (probe_device() != kOk) return kNoDevice;
   const int S = T * k;
   const int chunks = ceil_div(S, kSlotsPerChunk);
-  int32_t* ids = nullptr;
-  float* w = nullptr;
-  int32_t* counts = nullptr;
-  if (hipMallocAsync(reinterpret_cast<void**>(&ids), (size_t)S * 4, s) != hipSuccess) return kDeviceFailed;
-  if (hipMallocAsync(reinterpret_cast<void**>(&w), (size_t)S * 4, s) != hipSuccess) return kDeviceFailed;
-  if (hipMallocAsync(reinterpret_cast<void**>(&counts), (size_t)chunks * E * 4, s) != hipSuccess) return kDeviceFailed;
+  // The three temporaries are carved from the stream's own workspace (work on one stream
+  // runs in order and the placement kernel below is their last reader): no allocation,
+  // and three stream-ordered allocate / free pairs less on the host side of a call.
+  const size_t slot_bytes = ((size_t)S * 4 + 255) & ~(size_t)255;
+  char* ws = static_cast<char*>(stream_workspace(s, 2 * slot_bytes + (size_t)chunks * E * 4));
+  if (!ws) return kDeviceFailed;
+  int32_t* ids = reinterpret_cast<int32_t*>(ws);
+  float* w = reinterpret_cast<float*>(ws + slot_bytes);
+  int32_t* counts = reinterpret_cast<int32_t*>(ws + 2 * slot_bytes);
   const dim3 tgrid(ceil_div(T, 4));
   const int epl = ceil_div(E, 64);
   if (epl <= 1) hipLaunchKernelGGL((topk_kernel<1>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, ids, w);
@@ -236,10 +239,7 @@ int route_dev(const float* scores, int T, int E, int k, int normalize, int capac
                      num_slots);
   hipLaunchKernelGGL(place_kernel, dim3(chunks), dim3(64), 0, s, ids, w, S, E, k, capacity, counts, group_offsets,
                      token_of_slot, expert_of_slot, combine_weights);
-  int rc = launch_status();
-  if (hipFreeAsync(ids, s) != hipSuccess || hipFreeAsync(w, s) != hipSuccess || hipFreeAsync(counts, s) != hipSuccess)
-    rc = kDeviceFailed;
-  return rc;
+  return launch_status();
 }
 
 // ---- dispatch: exact row gather, 16 bytes per lane -------------------------------
