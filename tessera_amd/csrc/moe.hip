@@ -422,12 +422,14 @@ int combine_dev(const void* y, const int32_t* token_of_slot, const float* w, flo
                 hipStream_t s) {
   if (T <= 0 || S < 0 || N <= 0 || !out || (S > 0 && (!y || !token_of_slot || !w))) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
-  int32_t* cnt = nullptr;
-  int32_t* off = nullptr;
-  int32_t* list = nullptr;
-  if (hipMallocAsync(reinterpret_cast<void**>(&cnt), (size_t)T * 4, s) != hipSuccess) return kDeviceFailed;
-  if (hipMallocAsync(reinterpret_cast<void**>(&off), (size_t)(T + 1) * 4, s) != hipSuccess) return kDeviceFailed;
-  if (hipMallocAsync(reinterpret_cast<void**>(&list), (size_t)(S > 0 ? S : 1) * 4, s) != hipSuccess) return kDeviceFailed;
+  // the per-token slot lists live in the stream's own workspace (the combine kernel below
+  // is their last reader; work on one stream runs in order)
+  const size_t tok_bytes = ((size_t)(T + 1) * 4 + 255) & ~(size_t)255;
+  char* ws = static_cast<char*>(stream_workspace(s, 2 * tok_bytes + (size_t)(S > 0 ? S : 1) * 4));
+  if (!ws) return kDeviceFailed;
+  int32_t* cnt = reinterpret_cast<int32_t*>(ws);
+  int32_t* off = reinterpret_cast<int32_t*>(ws + tok_bytes);
+  int32_t* list = reinterpret_cast<int32_t*>(ws + 2 * tok_bytes);
   if (hipMemsetAsync(cnt, 0, (size_t)T * 4, s) != hipSuccess) return kDeviceFailed;
   if (S > 0) hipLaunchKernelGGL(combine_count_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, cnt);
   hipLaunchKernelGGL(combine_scan_kernel, dim3(1), dim3(1024), 0, s, cnt, T, off);
@@ -437,10 +439,7 @@ int combine_dev(const void* y, const int32_t* token_of_slot, const float* w, flo
     hipLaunchKernelGGL((combine_kernel<YT, true>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, off, list, out, N);
   else
     hipLaunchKernelGGL((combine_kernel<YT, false>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, off, list, out, N);
-  int rc = launch_status();
-  if (hipFreeAsync(cnt, s) != hipSuccess || hipFreeAsync(off, s) != hipSuccess || hipFreeAsync(list, s) != hipSuccess)
-    rc = kDeviceFailed;
-  return rc;
+  return launch_status();
 }
 
 int dispatch_dev(const void* x, const int32_t* token_of_slot, void* x_perm, int T, int S, int H, int elem_bytes,
