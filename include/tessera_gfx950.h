@@ -26,6 +26,15 @@
  *                               stream); the call enqueues and returns without
  *                               synchronising.  This is the resident-buffer form
  *                               used for chained ops and for timing.
+ *
+ * Temporaries of the _dev entry points (split-K partials, routing and combine lists,
+ * quantiser maxima) come from one workspace per (device, stream) that the library
+ * grows on demand: a call that needs more than any earlier call on its stream makes
+ * one hipMalloc (no free, no synchronisation; the outgrown buffer is kept for the
+ * work still queued on it), every other call allocates nothing.  All calls on one
+ * stream share that workspace from its first byte, so the host threads that enqueue
+ * on one stream must be serialised by the caller; under stream capture run the call
+ * once beforehand so the workspace already has its size.
  */
 #ifndef TESSERA_GFX950_H
 #define TESSERA_GFX950_H

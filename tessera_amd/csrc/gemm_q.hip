@@ -270,7 +270,7 @@ int quantize_e4m3_dev(const float* x, int64_t n, float scale, void* codes, float
     // order, so nothing else on it uses the workspace meanwhile): no allocation per call
     amax = static_cast<unsigned*>(stream_workspace(s, 256));
     if (!amax) return kDeviceFailed;
-    if (hipMemsetAsync(amax, 0, sizeof(unsigned), s) != hipSuccess) return kDeviceFailed;
+    zero_words(amax, 1, s);
     // (each workgroup ends in one atomic on the same word and those serialise at about
     // 8 ns each: two workgroups per CU, not sixteen)
     hipLaunchKernelGGL(absmax_kernel, dim3(std::min(blocks, 512)), dim3(256), 0, s, x, (long)n, amax);
@@ -300,7 +300,7 @@ int quantize_i8_dev(const float* x, int M, int N, int axis, void* q, float* scal
     // the per-column running maxima live in the stream's own workspace
     unsigned* amax = static_cast<unsigned*>(stream_workspace(s, (size_t)N * sizeof(unsigned)));
     if (!amax) return kDeviceFailed;
-    if (hipMemsetAsync(amax, 0, (size_t)N * sizeof(unsigned), s) != hipSuccess) return kDeviceFailed;
+    zero_words(amax, (size_t)N, s);
     const dim3 grid(ceil_div(N, 1024), ceil_div(M, kColRows));
     hipLaunchKernelGGL(absmax_cols_kernel, grid, dim3(256), 0, s, x, M, N, amax);
     hipLaunchKernelGGL(quantize_i8_cols_vec_kernel, grid, dim3(256), 0, s, x, M, N, amax, static_cast<int8_t*>(q),

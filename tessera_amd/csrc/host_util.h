@@ -44,10 +44,30 @@ class DeviceScope {
 };
 
 // Device scratch for kernels that need it between two launches of one call (split-K
-// partials): one buffer per (device, stream), grown on demand and kept until the
-// process ends.  Calls on one stream run in order, so they can share the buffer;
-// calls on different streams get different buffers.  Returns null on failure.
+// partials, routing and combine lists, quantiser maxima): one buffer per (device,
+// stream), grown on demand and kept until the process ends.  Calls on one stream run in
+// order, so they share the buffer from offset 0; calls on different streams get
+// different buffers.  Growing allocates (hipMalloc) but never frees or synchronises: the
+// outgrown buffer is set aside for the work still queued on it.  The host threads that
+// enqueue on one stream must be serialised by the caller (two of them would hand the
+// same bytes to kernels the stream may then interleave); under stream capture the
+// buffer must already have its final size (run the call once outside the capture).
+// Returns null on failure.
 void* stream_workspace(hipStream_t s, size_t bytes);
+
+// Clears `words` 32-bit words on the stream with a fill kernel.  (A memset node recorded
+// into a captured graph has given wrong results on replays after the first, so nothing a
+// caller may capture uses hipMemsetAsync.)
+static __global__ void __launch_bounds__(256) zero_words_kernel(uint32_t* p, size_t words) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < words; i += stride) p[i] = 0u;
+}
+inline void zero_words(void* p, size_t words, hipStream_t s) {
+  if (!words) return;
+  const size_t want = (words + 255) / 256;
+  hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)(want < 1024 ? want : 1024)), dim3(256), 0, s,
+                     static_cast<uint32_t*>(p), words);
+}
 
 inline int finish(hipError_t e) { return e == hipSuccess ? kOk : kDeviceFailed; }
 

@@ -64,10 +64,15 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* scores, int T, i
     sum += pr[i];
   }
   sum = wave_sum(sum);
+  // A NaN or +inf logit, or a row of -inf, makes the sum (the same value in every lane)
+  // and with it every probability of the row NaN, in numpy as here.  NaN compares false
+  // with everything, so such a row is selected on equal keys instead: it takes experts
+  // 0..k-1 (ties go to the lowest id) with NaN weights, and every id stays inside [0, E).
+  const bool nan_row = !(sum == sum);
 #pragma unroll
   for (int i = 0; i < EPL; ++i) {
     const int e = lane + 64 * i;
-    pr[i] = e < E ? __fdiv_rn(pr[i], sum) : -1.f;    // -1 never wins a selection
+    pr[i] = e < E ? (nan_row ? 0.f : __fdiv_rn(pr[i], sum)) : -1.f;    // -1 never wins a selection
   }
   float wsum = 0.f;
   float my_w = 0.f;       // lane j keeps the j-th selected weight
@@ -90,7 +95,7 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* scores, int T, i
 #pragma unroll
     for (int i = 0; i < EPL; ++i)
       if (lane + 64 * i == be) pr[i] = -1.f;       // remove the winner
-    if (lane == (j & 63)) { my_w = bv; my_e = be; }
+    if (lane == (j & 63)) { my_w = nan_row ? __builtin_nanf("") : bv; my_e = be; }
     wsum += bv;
     if ((j & 63) == 63 || j == k - 1) {
       // flush up to 64 selections (k <= 64 in practice; the loop form keeps it general)
@@ -114,7 +119,10 @@ __global__ __launch_bounds__(64) void count_kernel(const int32_t* expert_ids, in
   const int base = blockIdx.x * kSlotsPerChunk;
   for (int i = threadIdx.x; i < kSlotsPerChunk; i += 64) {
     const int s = base + i;
-    if (s < S) atomicAdd(&hist[expert_ids[s]], 1);
+    if (s < S) {
+      const int e = expert_ids[s];
+      if ((unsigned)e < (unsigned)E) atomicAdd(&hist[e], 1);
+    }
   }
   __syncthreads();
   for (int e = threadIdx.x; e < E; e += 64) chunk_counts[(long)blockIdx.x * E + e] = hist[e];
@@ -180,8 +188,9 @@ __global__ __launch_bounds__(64) void place_kernel(const int32_t* expert_ids, co
   const int base = blockIdx.x * kSlotsPerChunk;
   for (int i0 = 0; i0 < kSlotsPerChunk; i0 += 64) {
     const int s = base + i0 + lane;
-    const bool valid = s < S;
-    const int e = valid ? expert_ids[s] : -1;
+    int e = s < S ? expert_ids[s] : -1;
+    const bool valid = (unsigned)e < (unsigned)E;     // an id outside [0, E) is dropped, never an index
+    if (!valid) e = -1;
     // Rank inside the expert in slot order.  `same` = the lanes that hold this lane's
     // expert, built from one ballot per bit of the expert index (all lanes at once, no
     // loop over the experts present); lower lanes are earlier slots.
@@ -209,22 +218,30 @@ __global__ __launch_bounds__(64) void place_kernel(const int32_t* expert_ids, co
   }
 }
 
-int route_dev(const float* scores, int T, int E, int k, int normalize, int capacity, int32_t* token_of_slot,
-              int32_t* expert_of_slot, float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
-              int32_t* num_slots, hipStream_t s) {
+// Bytes of temporaries one routing call needs: the token-major expert ids and weights
+// (S = T * k each) and the per-chunk histograms.
+size_t route_workspace_bytes(int S, int E) {
+  const size_t slot_bytes = ((size_t)S * 4 + 255) & ~(size_t)255;
+  return 2 * slot_bytes + (size_t)ceil_div(S, kSlotsPerChunk) * E * 4;
+}
+
+bool bad_route(const float* scores, int T, int E, int k, const int32_t* token_of_slot, const int32_t* expert_of_slot,
+               const float* combine_weights, const int32_t* group_sizes, const int32_t* group_offsets) {
   if (T <= 0 || E <= 0 || k <= 0 || k > E || E > kMaxExperts || !scores || !token_of_slot || !expert_of_slot ||
       !combine_weights || !group_sizes || !group_offsets)
-    return kBadShape;
-  if ((long)T * k > 0x7fffffffL) return kBadShape;     // int32 device ABI
-  if (probe_device() != kOk) return kNoDevice;
+    return true;
+  return (long)T * k > 0x7fffffffL;      // int32 device ABI
+}
+
+// The four routing kernels on stream `s`, their temporaries in `ws` (device memory of at
+// least route_workspace_bytes(T * k, E) bytes; every byte a kernel reads is written by an
+// earlier kernel of the same call, so `ws` needs no clearing).
+int route_launch(const float* scores, int T, int E, int k, int normalize, int capacity, int32_t* token_of_slot,
+                 int32_t* expert_of_slot, float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
+                 int32_t* num_slots, char* ws, hipStream_t s) {
   const int S = T * k;
   const int chunks = ceil_div(S, kSlotsPerChunk);
-  // The three temporaries are carved from the stream's own workspace (work on one stream
-  // runs in order and the placement kernel below is their last reader): no allocation,
-  // and three stream-ordered allocate / free pairs less on the host side of a call.
   const size_t slot_bytes = ((size_t)S * 4 + 255) & ~(size_t)255;
-  char* ws = static_cast<char*>(stream_workspace(s, 2 * slot_bytes + (size_t)chunks * E * 4));
-  if (!ws) return kDeviceFailed;
   int32_t* ids = reinterpret_cast<int32_t*>(ws);
   float* w = reinterpret_cast<float*>(ws + slot_bytes);
   int32_t* counts = reinterpret_cast<int32_t*>(ws + 2 * slot_bytes);
@@ -240,6 +257,21 @@ int route_dev(const float* scores, int T, int E, int k, int normalize, int capac
   hipLaunchKernelGGL(place_kernel, dim3(chunks), dim3(64), 0, s, ids, w, S, E, k, capacity, counts, group_offsets,
                      token_of_slot, expert_of_slot, combine_weights);
   return launch_status();
+}
+
+int route_dev(const float* scores, int T, int E, int k, int normalize, int capacity, int32_t* token_of_slot,
+              int32_t* expert_of_slot, float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
+              int32_t* num_slots, hipStream_t s) {
+  if (bad_route(scores, T, E, k, token_of_slot, expert_of_slot, combine_weights, group_sizes, group_offsets))
+    return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  // The temporaries are carved from the stream's own workspace (work on one stream runs in
+  // order and the placement kernel is their last reader): no allocation once it has grown,
+  // and three stream-ordered allocate / free pairs less on the host side of a call.
+  char* ws = static_cast<char*>(stream_workspace(s, route_workspace_bytes(T * k, E)));
+  if (!ws) return kDeviceFailed;
+  return route_launch(scores, T, E, k, normalize, capacity, token_of_slot, expert_of_slot, combine_weights,
+                      group_sizes, group_offsets, num_slots, ws, s);
 }
 
 // ---- dispatch: exact row gather, 16 bytes per lane -------------------------------
@@ -430,7 +462,7 @@ int combine_dev(const void* y, const int32_t* token_of_slot, const float* w, flo
   int32_t* cnt = reinterpret_cast<int32_t*>(ws);
   int32_t* off = reinterpret_cast<int32_t*>(ws + tok_bytes);
   int32_t* list = reinterpret_cast<int32_t*>(ws + 2 * tok_bytes);
-  if (hipMemsetAsync(cnt, 0, (size_t)T * 4, s) != hipSuccess) return kDeviceFailed;
+  zero_words(cnt, (size_t)T, s);
   if (S > 0) hipLaunchKernelGGL(combine_count_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, cnt);
   hipLaunchKernelGGL(combine_scan_kernel, dim3(1), dim3(1024), 0, s, cnt, T, off);
   if (S > 0) hipLaunchKernelGGL(combine_fill_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, off, cnt, list);
@@ -455,6 +487,12 @@ int dispatch_dev(const void* x, const int32_t* token_of_slot, void* x_perm, int 
 }
 
 bool bad_grouped(int S, int K, int N, int E) { return S < 0 || K <= 0 || N <= 0 || E <= 0; }
+
+// A gathered row of the (rows, K) 16-bit activation is fetched by a buffer load whose
+// offset is counted from the start of x, and the buffer resource spans kBufferRange
+// bytes: an offset at or past the range reads as zero without an error, so the whole
+// activation has to lie inside it.
+bool gather_out_of_buffer_range(int rows, int K) { return (long)rows * K * 2 > (long)kBufferRange - 16; }
 
 template <int EPI>
 int grouped_dev(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K, int N, int E,
@@ -481,8 +519,8 @@ int swiglu_dev(const void* x, const void* wg, const void* wu, const void* wd, co
                void* hidden, int S, int K, int F, int N, int E, hipStream_t s, const int32_t* gather = nullptr,
                int x_rows = 0) {
   if (bad_grouped(S, K, N, E) || F <= 0 || !wg || !wu || !wd || !offsets || (S > 0 && (!x || !y))) return kBadShape;
-  // (the kernels address a gathered row with a 32-bit byte offset from x)
-  if (gather && (x_rows <= 0 || (long)x_rows * K * 2 >= (1L << 32))) return kBadShape;
+  // (the kernels address a gathered row with a buffer load off x)
+  if (gather && (x_rows <= 0 || gather_out_of_buffer_range(x_rows, K))) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
   if (S == 0) return kOk;
   void* h = hidden;

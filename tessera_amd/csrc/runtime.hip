@@ -4,6 +4,7 @@
 #include <map>
 #include <mutex>
 #include <utility>
+#include <vector>
 #include "../../include/tessera_gfx950.h"
 #include "host_util.h"
 
@@ -28,19 +29,20 @@ void* stream_workspace(hipStream_t s, size_t bytes) {
   struct Slot { void* ptr; size_t bytes; };
   static std::mutex mu;
   static std::map<std::pair<int, hipStream_t>, Slot> slots;
+  static std::vector<void*> retired;      // outgrown buffers: kept until the process ends
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
   std::lock_guard<std::mutex> lock(mu);
   Slot& slot = slots[{dev, s}];
   if (slot.bytes >= bytes && slot.ptr) return slot.ptr;
-  if (slot.ptr) {
-    // work already queued on the stream may still use the old buffer
-    if (hipStreamSynchronize(s) != hipSuccess || hipFree(slot.ptr) != hipSuccess) (void)hipGetLastError();
-    slot = Slot{nullptr, 0};
-  }
-  const size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+  // Work already queued on the stream may still use the old buffer, so it is neither
+  // freed nor waited for: it is set aside, and the new one is at least twice its size,
+  // which bounds everything set aside by the size of the buffer in use.
+  size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+  if (want < 2 * slot.bytes) want = 2 * slot.bytes;
   void* p = nullptr;
   if (hipMalloc(&p, want) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  if (slot.ptr) retired.push_back(slot.ptr);
   slot = Slot{p, want};
   return p;
 }

@@ -577,8 +577,14 @@ def moe_layer(x, W_router, W_gate, W_up, W_down, *, top_k: int = 1, normalize_we
         if _storage(a) != "bf16":
             raise ValueError("moe_layer on the gfx950 lane takes bf16 storage")
     xa, wg, wu, wd = map(_bits, (x, W_gate, W_up, W_down))
+    if xa.ndim != 2 or wg.ndim != 3 or wu.shape != wg.shape or wd.ndim != 3:
+        raise ValueError("moe_layer: x (T,K), W_gate/W_up (E,K,F), W_down (E,F,N)")
     T, H = xa.shape
-    E, _, F = wg.shape
+    E, Kw, F = wg.shape
+    if Kw != H or wd.shape[0] != E or wd.shape[1] != F:
+        raise ValueError(f"moe_layer: weight shapes disagree: x {xa.shape}, W_gate/W_up {wg.shape}, W_down {wd.shape}")
+    if top_k < 1 or top_k > E:
+        raise ValueError(f"top_k must be in [1, num_experts={E}], got {top_k}")
     N = wd.shape[2]
     if router_logits is None:
         scores = gemm(x, W_router)                       # storage-rounded, as ops.gemm

@@ -110,6 +110,38 @@ def test_python_side_argument_errors():
         ops.route_tokens(np.zeros((4, 4), np.float32), 4, 5)
     with pytest.raises(ValueError):
         ops.quantize_fp8(np.zeros(4), format="e3m4")
+    # moe_layer: mismatched expert weights are refused before any pointer is handed over
+    xm = b16.from_float32(np.zeros((4, 8)))
+    lg = np.zeros((4, 2), np.float32)
+    wg = b16.from_float32(np.zeros((2, 8, 16)))
+    wd = b16.from_float32(np.zeros((2, 16, 8)))
+    with pytest.raises(ValueError):
+        ops.moe_layer(xm, None, wg, b16.from_float32(np.zeros((2, 8, 12))), wd, top_k=1, router_logits=lg)
+    with pytest.raises(ValueError):
+        ops.moe_layer(xm, None, b16.from_float32(np.zeros((2, 6, 16))), b16.from_float32(np.zeros((2, 6, 16))), wd,
+                      top_k=1, router_logits=lg)
+    with pytest.raises(ValueError):
+        ops.moe_layer(xm, None, wg, wg, b16.from_float32(np.zeros((3, 16, 8))), top_k=1, router_logits=lg)
+    with pytest.raises(ValueError):
+        ops.moe_layer(xm, None, wg, wg, b16.from_float32(np.zeros((2, 12, 8))), top_k=1, router_logits=lg)
+    with pytest.raises(ValueError):
+        ops.moe_layer(xm, None, wg, wg, wd, top_k=3, router_logits=lg)
+
+
+def test_gather_block_rejects_activations_past_the_buffer_range():
+    """The gather form of the expert block reaches a token row through a buffer load
+    whose range is 2 GiB from the start of x; rows past it would read as zeros, so
+    the launcher refuses such an activation (rc 1) before it touches the device."""
+    lib = lane.load()
+    fake = 0x1000                                   # never dereferenced: the checks come first
+    K = 4096
+    rows_over = (0x7fffffff - 16) // (K * 2) + 1    # first row count whose last byte leaves the range
+    args = lambda T: (fake, fake, fake, fake, fake, fake, fake, fake, T, 64, K, 64, K, 2, None)
+    assert lib.tessera_gfx950_moe_swiglu_block_gather_bf16_dev(*args(rows_over)) == 1
+    assert lib.tessera_gfx950_moe_swiglu_block_gather_bf16_dev(*args(300_000)) == 1      # 2.4 GB: was accepted
+    if not lane.available():
+        # just inside the range the shape is accepted and the call goes on to the device probe
+        assert lib.tessera_gfx950_moe_swiglu_block_gather_bf16_dev(*args(rows_over - 1)) == 2
 
 
 def test_bf16_host_array():

@@ -67,6 +67,30 @@ def test_routing_ties_go_to_lowest_expert(lane):
     assert np.allclose(plan.combine_weights, 1.0 / 3.0)
 
 
+def test_routing_non_finite_rows_stay_in_range(lane):
+    """Rows whose softmax is NaN (a NaN or +inf logit, a row of -inf) take experts
+    0..k-1 with NaN weights, as the oracle's stable sort gives them; every index of the
+    plan stays inside its range and finite rows route as they would alone."""
+    T, E, k = 300, 64, 8
+    lg = _logits(T, E, 31, k)
+    lg[5, 17] = np.nan
+    lg[77, 0] = np.inf
+    lg[123, :] = -np.inf
+    lg[299, 63] = np.nan
+    with np.errstate(invalid="ignore"):
+        r = orc.route_tokens(lg, E, k)
+        desc = orc.plan_dispatch(r.assignment, r.weights, E)
+    plan = ops.route_tokens(lg, E, k, capacity_factor=1e9)
+    assert plan.num_slots == T * k
+    assert np.array_equal(plan.token_of_slot, desc.token_of_slot)
+    assert np.array_equal(plan.expert_of_slot, desc.expert_of_slot)
+    assert np.array_equal(plan.group_offsets, desc.group_offsets)
+    assert np.array_equal(np.isnan(plan.combine_weights), np.isnan(desc.combine_weights))
+    ok = ~np.isnan(desc.combine_weights)
+    np.testing.assert_allclose(plan.combine_weights[ok], desc.combine_weights[ok], rtol=2e-6, atol=1e-9)
+    assert int(np.isnan(plan.combine_weights).sum()) == 4 * k
+
+
 def test_dispatch_and_combine(lane):
     T, H, E, k = 300, 96, 8, 2
     lg = _logits(T, E, 1, k)

@@ -303,3 +303,27 @@ def test_flash_attn_backward_matches_torch_autograd_and_finite_differences():
             args_lo = [lo if a is arr else a for a in (q, k, v)]
             fd = (loss(*args_hi) - loss(*args_lo)) / (2 * eps)
             assert abs(fd - grad[idx]) <= 1e-6 * max(1.0, abs(fd))
+
+
+def test_route_tokens_non_finite_rows_keep_indices_in_range():
+    """A NaN or +inf logit, or a row of -inf, turns the whole row's probabilities into
+    NaN (distributed/moe.py:163-165: the max-subtracted softmax).  numpy's argsort still
+    returns valid indices for such a row; the oracle's stable sort orders the NaNs by
+    index, so the row takes experts 0..k-1 with NaN weights and finite rows are untouched."""
+    rng = np.random.default_rng(11)
+    s = rng.standard_normal((6, 8)).astype(np.float32)
+    s[1, 3] = np.nan
+    s[2, 5] = np.inf
+    s[4, :] = -np.inf
+    with np.errstate(invalid="ignore"):
+        r = orc.route_tokens(s, 8, 3)
+    assert r.assignment.min() >= 0 and r.assignment.max() < 8
+    for t in (1, 2, 4):
+        assert list(r.assignment[t]) == [0, 1, 2]
+        assert np.isnan(r.weights[t]).all()
+    clean = orc.route_tokens(s[[0, 3, 5]], 8, 3)
+    assert np.array_equal(r.assignment[[0, 3, 5]], clean.assignment)
+    assert np.array_equal(r.weights[[0, 3, 5]], clean.weights)
+    with np.errstate(invalid="ignore"):
+        d = orc.plan_dispatch(r.assignment, r.weights, 8)
+    assert d.group_offsets[-1] == 18 and np.array_equal(np.sort(d.token_of_slot), np.repeat(np.arange(6), 3))
