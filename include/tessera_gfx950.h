@@ -311,6 +311,22 @@ int tessera_gfx950_moe_route_f32_dev(const float* scores, int T, int E, int k, i
                                      int32_t* group_sizes, int32_t* group_offsets, int32_t* num_slots,
                                      void* stream);
 
+/* The same routing for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Identical arguments, kernels and results as
+ * tessera_gfx950_moe_route_f32_dev, but the temporaries (token-major expert ids and
+ * weights, per-chunk histograms) live in a fixed 4 MiB device array inside the
+ * library image instead of the per-stream workspace: the call makes no hipMalloc,
+ * hipFree or other allocating call.  Limit: 2 * roundup(T*k*4, 256) +
+ * ceil(T*k / 512) * E * 4 <= 4 MiB (T*k up to about 490,000 slots at E = 64), else
+ * rc 1.  Every call on one GPU shares that array, so two such calls that overlap on
+ * one GPU (different streams, or different host threads) race; calls on one stream
+ * are safe back to back.  All pointers are device memory. */
+int tessera_gfx950_moe_route_f32_noalloc_dev(const float* scores, int T, int E, int k, int normalize, int capacity,
+                                             int32_t* token_of_slot, int32_t* expert_of_slot,
+                                             float* combine_weights, int32_t* group_sizes,
+                                             int32_t* group_offsets, int32_t* num_slots, void* stream);
+
 /* tessera.moe_dispatch: x_perm[s,:] = x[token_of_slot[s],:]  (exact gather,
  * python/tessera/runtime.py:1791-1806).  elem_bytes = 2 (f16/bf16) or 4 (f32). */
 int tessera_gfx950_moe_dispatch(const void* x, const int32_t* token_of_slot, void* x_perm,

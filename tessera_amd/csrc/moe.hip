@@ -22,6 +22,12 @@
 #include "gemm16_launch.h"
 #include "host_util.h"
 
+// Routing temporaries of the entry point that allocates nothing: device memory that is
+// part of the library image, one copy per GPU, held until the process ends.  Host code
+// reaches it only through the address hipGetSymbolAddress returns for the current device.
+constexpr size_t kRouteScratchBytes = size_t(4) << 20;
+static __device__ __align__(256) unsigned char scratch[kRouteScratchBytes];
+
 namespace tsr950 {
 namespace {
 
@@ -272,6 +278,27 @@ int route_dev(const float* scores, int T, int E, int k, int normalize, int capac
   if (!ws) return kDeviceFailed;
   return route_launch(scores, T, E, k, normalize, capacity, token_of_slot, expert_of_slot, combine_weights,
                       group_sizes, group_offsets, num_slots, ws, s);
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+int route_scratch(char** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static char* ptrs[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return kDeviceFailed; }
+  if (dev < 0 || dev >= kMaxDevices) return kDeviceFailed;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return kDeviceFailed;
+    }
+    ptrs[dev] = static_cast<char*>(p);
+  }
+  *out = ptrs[dev];
+  return kOk;
 }
 
 // ---- dispatch: exact row gather, 16 bytes per lane -------------------------------
@@ -599,6 +626,20 @@ int tessera_gfx950_moe_route_f32_dev(const float* scores, int T, int E, int k, i
                                      void* stream) {
   return route_dev(scores, T, E, k, normalize, capacity, token_of_slot, expert_of_slot, combine_weights,
                    group_sizes, group_offsets, num_slots, as_stream(stream));
+}
+
+int tessera_gfx950_moe_route_f32_noalloc_dev(const float* scores, int T, int E, int k, int normalize, int capacity,
+                                             int32_t* token_of_slot, int32_t* expert_of_slot,
+                                             float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
+                                             int32_t* num_slots, void* stream) {
+  if (bad_route(scores, T, E, k, token_of_slot, expert_of_slot, combine_weights, group_sizes, group_offsets))
+    return kBadShape;
+  if (route_workspace_bytes(T * k, E) > kRouteScratchBytes) return kBadShape;    // beyond the fixed scratch
+  if (probe_device() != kOk) return kNoDevice;
+  char* ws = nullptr;
+  if (const int rc = route_scratch(&ws); rc != kOk) return rc;
+  return route_launch(scores, T, E, k, normalize, capacity, token_of_slot, expert_of_slot, combine_weights,
+                      group_sizes, group_offsets, num_slots, ws, as_stream(stream));
 }
 
 int tessera_gfx950_moe_route_f32(const float* scores, int T, int E, int k, int normalize, int capacity,

@@ -131,6 +131,7 @@ _SIGNATURES = {
     "tessera_gfx950_flash_attn_bwd_bf16_dev": [_c_vp] * 9 + [_c_int] * 6 + [_c_f, _c_int, _c_vp],
     "tessera_gfx950_moe_route_f32": [_c_vp] + [_c_int] * 5 + [_c_vp] * 6,
     "tessera_gfx950_moe_route_f32_dev": [_c_vp] + [_c_int] * 5 + [_c_vp] * 6 + [_c_vp],
+    "tessera_gfx950_moe_route_f32_noalloc_dev": [_c_vp] + [_c_int] * 5 + [_c_vp] * 6 + [_c_vp],
     "tessera_gfx950_moe_dispatch": [_c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int],
     "tessera_gfx950_moe_dispatch_dev": [_c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_moe_combine_bf16": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int],
