@@ -7,10 +7,12 @@ Modules
 ``lane``        ctypes binding of ``lib/libtessera_gfx950.so``
 ``ops``         the ``tessera.ops`` / ``nn.functional`` surface of the path
 ``executors``   the ``runtime.launch`` executor seam (execution-matrix rows)
-``candidates``  the measured-arbiter ``Candidate`` seam
+``candidates``  gfx950 candidates for the host's measured arbiter (host API injected)
+``install``     one call that registers candidates, matrix rows and executors with a host
+``autotune``    the lane's autotune corpus (reference schema) and tuning through the host
 ``tile_table``  Tile-IR op -> gfx950 kernel table
 ``build``       in-tree hipcc build of the library
 """
 from . import bf16, lane  # noqa: F401
 
-__all__ = ["bf16", "lane", "ops", "executors", "candidates", "tile_table", "build"]
+__all__ = ["bf16", "lane", "ops", "executors", "candidates", "install", "autotune", "tile_table", "build"]

@@ -1,354 +1,323 @@
-"""Measured arbitration and the persisted autotune corpus for the gfx950 lane.
+"""Measured verdicts for the gfx950 candidates, kept as data.
 
-Mirrors ``python/tessera/compiler/emit/autotune.py``: a :class:`MeasureCache` of
-:class:`MeasureRecord` keyed by ``(device, target, op, shape-bucket, dtype,
-timing)`` (``:40-75,139-206``), measure-at-first-miss arbitration over the F4-gated
-candidates (``:392-447``), and the committed JSON corpus that warm-starts other
-processes (``:215-278``) in the reference's schema (``CORPUS_VERSION = 3``), so the
-records written here can be merged into Tessera's own
-``benchmarks/baselines/autotune_corpus.json``.  Device tags follow the reference's
-``<family>:<arch>`` form (``rocm:gfx950``), so a record only warm-starts a matching
-device.
+The host's autotuner (``python/tessera/compiler/emit/autotune.py``) persists, per
+workload, which candidate was fastest; other processes warm-start from that file.
+This module owns only the lane's side of it:
 
-``python -m tessera_amd.autotune [--out PATH]`` measures the lane's candidates on
-the shapes of the headline configurations and writes the corpus.
+* the *wire format* of such a file — the reference's corpus schema, version 3: a
+  list of flat records with the key fields ``device, target, op, bucket, dtype,
+  timing`` and the verdict fields ``winner, latency_ms, candidates, evidence``
+  (``emit/autotune.py:40-75,170-202``) — so that ``autotune_corpus.json`` beside this
+  file can be merged into Tessera's ``benchmarks/baselines/autotune_corpus.json``;
+* :class:`Corpus`, a small table of those records with file I/O;
+* :func:`tune`, which asks the *host's* arbiter (``api.arbitrate`` with its
+  ``measure=`` hook) to pick the fastest verified candidate on a miss and records
+  the verdict, and :func:`recommended`, which reads one back.
+
+The arbiter, the verification gate and the candidate registry stay the host's; they
+come in as the ``api`` argument (the object :mod:`tessera_amd.candidates` registers
+into).
 """
 from __future__ import annotations
 
 import json
 import os
-import statistics
-import sys
 import time
 from dataclasses import dataclass, field
 from pathlib import Path
-from typing import Any, Mapping, Optional
-
-import numpy as np
+from typing import Any, Iterator, Mapping, Optional
 
 from . import candidates as _cand
 from . import lane as _lane
 
-CORPUS_VERSION = 3
-TIMING_END_TO_END = "end_to_end"
-TIMING_DEVICE = "device"
-_TIMING_MODES = (TIMING_END_TO_END, TIMING_DEVICE)
+SCHEMA_VERSION = 3
+#: what a latency in a record means: wall clock around ``run`` or device events
+TIMINGS = ("end_to_end", "device")
+DEVICE_TAG = "rocm:gfx950"
+PACKAGED = Path(__file__).resolve().parent / "autotune_corpus.json"
+
+
+class NoCandidate(RuntimeError):
+    """No registered candidate applies, is available and passes the host's gate.
+    (The lane has no CPU path to degrade to.)"""
+
+
+def pow2_bucket(dims) -> Optional[tuple]:
+    """Every dim rounded up to a power of two — the reference's shape bucketing
+    (``emit/kernel_emitter.py:72-80``), so records land in the buckets the host uses."""
+    if dims is None:
+        return None
+    return tuple(1 << max(int(d) - 1, 0).bit_length() for d in dims)
 
 
 @dataclass(frozen=True)
-class MeasureRecord:
-    """The measured verdict for one key: the fastest candidate, its median latency
-    (ms), every timed candidate's latency and free-form evidence."""
+class Workload:
+    """The key of one record."""
+    device: str
+    target: str
+    op: str
+    bucket: Optional[tuple]
+    dtype: str
+    timing: str = "end_to_end"
+
+    def __post_init__(self) -> None:
+        if self.timing not in TIMINGS:
+            raise ValueError(f"timing must be one of {TIMINGS}, got {self.timing!r}")
+
+    @classmethod
+    def of(cls, device: str, target: str, op: str, dims, dtype: str, timing: str = "end_to_end") -> "Workload":
+        return cls(device, target, op, pow2_bucket(dims), dtype, timing)
+
+
+@dataclass
+class Verdict:
+    """The value of one record: the fastest candidate, its latency (ms), every timed
+    candidate's latency, and free-form evidence."""
     winner: str
     latency_ms: float
     candidates: dict = field(default_factory=dict)
     evidence: dict = field(default_factory=dict)
-    candidate_descriptors: dict = field(default_factory=dict)
-
-    def as_json(self) -> dict:
-        out = {"winner": self.winner, "latency_ms": self.latency_ms, "candidates": dict(self.candidates)}
-        if self.candidate_descriptors:
-            out["candidate_descriptors"] = dict(self.candidate_descriptors)
-        if self.evidence:
-            out["evidence"] = dict(self.evidence)
-        return out
-
-    @classmethod
-    def from_json(cls, d: Mapping[str, Any]) -> "MeasureRecord":
-        return cls(winner=str(d["winner"]), latency_ms=float(d["latency_ms"]),
-                   candidates={str(k): float(v) for k, v in dict(d.get("candidates", {})).items()},
-                   candidate_descriptors={str(k): dict(v) for k, v in dict(d.get("candidate_descriptors", {})).items()
-                                          if isinstance(v, dict)},
-                   evidence=dict(d.get("evidence", {})))
 
 
-def _dim_bucket(n: int) -> int:
-    """Next power of two (``emit/kernel_emitter.py:72-80``)."""
-    b = 1
-    while b < n:
-        b *= 2
-    return b
+def _record_to_wire(w: Workload, v: Verdict) -> dict:
+    rec = {"device": w.device, "target": w.target, "op": w.op,
+           "bucket": None if w.bucket is None else list(w.bucket), "dtype": w.dtype, "timing": w.timing,
+           "winner": v.winner, "latency_ms": float(v.latency_ms),
+           "candidates": {str(n): float(t) for n, t in v.candidates.items()}}
+    if v.evidence:
+        rec["evidence"] = dict(v.evidence)
+    return rec
 
 
-def bucket_key(dims) -> Optional[tuple]:
-    """Shape-bucket key: every dim coarsened to its power-of-two bucket."""
-    return None if dims is None else tuple(_dim_bucket(int(d)) for d in dims)
+def _record_from_wire(rec: Mapping[str, Any]) -> tuple:
+    bucket = rec.get("bucket")
+    w = Workload(str(rec["device"]), str(rec["target"]), str(rec["op"]),
+                 None if bucket is None else tuple(int(b) for b in bucket), str(rec["dtype"]),
+                 str(rec.get("timing", "end_to_end")))          # records older than version 3 carry no timing
+    v = Verdict(str(rec["winner"]), float(rec["latency_ms"]),
+                {str(n): float(t) for n, t in dict(rec.get("candidates") or {}).items()},
+                dict(rec.get("evidence") or {}))
+    return w, v
 
 
-def _normalize_key(key: tuple) -> tuple:
-    if len(key) == 5:
-        return (*key, TIMING_END_TO_END)
-    if len(key) != 6 or key[5] not in _TIMING_MODES:
-        raise ValueError(f"invalid autotune cache key {key!r}")
-    return key
-
-
-def _key_to_json(key: tuple) -> dict:
-    dev, target, op, bucket, dtype, timing = _normalize_key(key)
-    return {"device": dev, "target": target, "op": op, "bucket": list(bucket) if bucket is not None else None,
-            "dtype": dtype, "timing": timing}
-
-
-def _key_from_json(d: Mapping[str, Any]) -> tuple:
-    b = d.get("bucket")
-    return (d["device"], d["target"], d["op"], tuple(b) if b is not None else None, d["dtype"],
-            d.get("timing", TIMING_END_TO_END))
-
-
-class MeasureCache:
-    """Content-keyed cache of measured verdicts — measure-at-first-miss."""
+class Corpus:
+    """A table ``Workload -> Verdict``."""
 
     def __init__(self) -> None:
-        self._store: dict = {}
-        self.hits = 0
-        self.misses = 0
+        self._table: dict = {}
+        self.lookups = 0
+        self.found = 0
 
-    def get(self, key: tuple) -> Optional[MeasureRecord]:
-        rec = self._store.get(_normalize_key(key))
-        if rec is not None:
-            self.hits += 1
-        else:
-            self.misses += 1
-        return rec
+    def __len__(self) -> int:
+        return len(self._table)
 
-    def put(self, key: tuple, rec: MeasureRecord) -> None:
-        self._store[_normalize_key(key)] = rec
+    def __iter__(self) -> Iterator[tuple]:
+        return iter(self._table.items())
 
-    def clear(self) -> None:
-        self._store.clear()
-        self.hits = self.misses = 0
+    def lookup(self, w: Workload) -> Optional[Verdict]:
+        self.lookups += 1
+        v = self._table.get(w)
+        self.found += v is not None
+        return v
 
-    @property
-    def size(self) -> int:
-        return len(self._store)
+    def record(self, w: Workload, v: Verdict) -> None:
+        self._table[w] = v
 
-    def items(self):
-        return self._store.items()
+    def winners(self, device: str, target: str, op: str, bucket: Optional[tuple], timing: str,
+                dtype: Optional[str] = None) -> set:
+        """Names recorded as winner for this workload over every dtype (or one)."""
+        return {v.winner for w, v in self._table.items()
+                if (w.device, w.target, w.op, w.bucket, w.timing) == (device, target, op, bucket, timing)
+                and dtype in (None, w.dtype)}
 
-    def to_dict(self) -> dict:
-        return {"version": CORPUS_VERSION,
-                "records": [{**_key_to_json(k), **rec.as_json()} for k, rec in self._store.items()]}
+    def to_payload(self) -> dict:
+        return {"version": SCHEMA_VERSION, "records": [_record_to_wire(w, v) for w, v in self._table.items()]}
 
-    def load_dict(self, payload: Mapping[str, Any], *, overwrite: bool = False) -> int:
-        """Merge a :meth:`to_dict` payload (warm start).  A key already present is
-        kept (measured-on-this-box wins) unless ``overwrite``; a payload of another
-        schema version loads nothing."""
-        if int(payload.get("version", -1)) not in (1, 2, CORPUS_VERSION):
+    def absorb(self, payload: Mapping[str, Any], *, replace: bool = False) -> int:
+        """Take in the records of a payload; returns how many were taken.  A record
+        whose key is already present stays (what this process measured outranks a file)
+        unless ``replace``.  A payload of an unknown schema version contributes nothing."""
+        if payload.get("version") not in (1, 2, SCHEMA_VERSION):
             return 0
-        loaded = 0
-        for r in payload.get("records", ()):
-            key = _key_from_json(r)
-            if not overwrite and key in self._store:
-                continue
-            self._store[key] = MeasureRecord.from_json(r)
-            loaded += 1
-        return loaded
+        taken = 0
+        for rec in payload.get("records") or ():
+            w, v = _record_from_wire(rec)
+            if replace or w not in self._table:
+                self._table[w] = v
+                taken += 1
+        return taken
 
+    def save(self, path) -> Path:
+        p = Path(path)
+        p.parent.mkdir(parents=True, exist_ok=True)
+        p.write_text(json.dumps(self.to_payload(), indent=2, sort_keys=True) + "\n")
+        return p
 
-_DEFAULT_CACHE = MeasureCache()
-_CORPUS_PATH = Path(__file__).resolve().parent / "autotune_corpus.json"
-_warm_started = False
-
-
-def default_cache() -> MeasureCache:
-    return _DEFAULT_CACHE
+    def absorb_file(self, path, *, replace: bool = False) -> int:
+        """:meth:`absorb` from a JSON file; a missing or malformed file contributes
+        nothing and does not raise."""
+        try:
+            payload = json.loads(Path(path).read_text())
+            return self.absorb(payload, replace=replace)
+        except (OSError, ValueError, KeyError, TypeError):
+            return 0
 
 
 def corpus_path() -> Path:
-    """``$TESSERA_AUTOTUNE_CORPUS`` overrides the packaged corpus (the reference's
-    own override variable, ``emit/autotune.py:226-230``)."""
-    env = os.environ.get("TESSERA_AUTOTUNE_CORPUS")
-    return Path(env) if env else _CORPUS_PATH
+    """The corpus file: ``$TESSERA_AUTOTUNE_CORPUS`` (the reference's override variable,
+    ``emit/autotune.py:226-230``) or the one packaged beside this module."""
+    return Path(os.environ.get("TESSERA_AUTOTUNE_CORPUS") or PACKAGED)
 
 
-def save_corpus(path=None, cache: Optional[MeasureCache] = None) -> Path:
-    cache = cache if cache is not None else _DEFAULT_CACHE
-    p = Path(path) if path is not None else corpus_path()
-    p.parent.mkdir(parents=True, exist_ok=True)
-    p.write_text(json.dumps(cache.to_dict(), indent=2, sort_keys=True) + "\n")
-    return p
+_shared: Optional[Corpus] = None
 
 
-def load_corpus(path=None, cache: Optional[MeasureCache] = None, *, overwrite: bool = False) -> int:
-    """Merge the corpus file into ``cache``; a missing, unreadable or stale file
-    loads nothing and never raises."""
-    cache = cache if cache is not None else _DEFAULT_CACHE
-    p = Path(path) if path is not None else corpus_path()
-    try:
-        payload = json.loads(p.read_text())
-    except (OSError, ValueError):
-        return 0
-    return cache.load_dict(payload, overwrite=overwrite)
+def shared_corpus() -> Corpus:
+    """The process-wide corpus, warm-started once from :func:`corpus_path` unless
+    ``$TESSERA_AUTOTUNE_NO_WARMSTART`` is set."""
+    global _shared
+    if _shared is None:
+        _shared = Corpus()
+        if not os.environ.get("TESSERA_AUTOTUNE_NO_WARMSTART"):
+            _shared.absorb_file(corpus_path())
+    return _shared
 
 
-def _maybe_warm_start(cache: MeasureCache) -> None:
-    global _warm_started
-    if _warm_started or cache is not _DEFAULT_CACHE:
-        return
-    _warm_started = True
-    if os.environ.get("TESSERA_AUTOTUNE_NO_WARMSTART"):
-        return
-    load_corpus(cache=cache)
+def device_tag(target: str = _cand.TARGET) -> str:
+    """``rocm:gfx950`` (the reference's ``<family>:<arch>`` form) when the lane runs
+    here, else the bare target id, so nothing is keyed as a device it was not measured on."""
+    return DEVICE_TAG if target == _cand.TARGET and _lane.available() else target
 
 
-def measure_latency(run_fn, *, reps: int = 20, warmup: int = 3) -> float:
-    """Median wall-clock latency (ms) of ``run_fn`` — end to end, what a caller pays
-    (``emit/autotune.py:281-304``)."""
+def problem_dims(op: str, inputs: tuple) -> Optional[tuple]:
+    """``(Sq, Sk, D, Dv)`` for the 2-D operands ``(Q, K, V)`` of the ``attention`` op
+    kind, ``(M, N, K)`` for the 2-D operands ``(A[M,K], B[K,N], ...)`` of any other;
+    ``None`` when the operands are not 2-D arrays."""
+    shapes = [tuple(getattr(x, "shape", ())) for x in inputs[:3]]
+    if op == "attention":
+        if len(shapes) == 3 and all(len(s) == 2 for s in shapes):
+            return shapes[0][0], shapes[1][0], shapes[0][1], shapes[2][1]
+        return None
+    if len(shapes) >= 2 and len(shapes[0]) == 2 and len(shapes[1]) == 2:
+        return shapes[0][0], shapes[1][1], shapes[0][1]
+    return None
+
+
+def _wall_ms(fn, reps: int, warmup: int) -> float:
     for _ in range(warmup):
-        run_fn()
-    samples = []
-    for _ in range(reps):
+        fn()
+    laps = []
+    for _ in range(max(reps, 1)):
         t0 = time.perf_counter()
-        run_fn()
-        samples.append((time.perf_counter() - t0) * 1e3)
-    return statistics.median(samples)
+        fn()
+        laps.append((time.perf_counter() - t0) * 1e3)
+    laps.sort()
+    return laps[len(laps) // 2]
 
 
-def device_id(target: str = _cand.TARGET) -> str:
-    """``rocm:gfx950`` on the device; the bare target id when the lane is absent, so
-    nothing measured on one device is keyed as another."""
-    if target == _cand.TARGET and _lane.available():
-        return "rocm:gfx950"
-    return target
-
-
-def _infer_dims(op: str, inputs: tuple) -> Optional[tuple]:
-    try:
-        if op in (_cand.OP_MATMUL, _cand.OP_FUSED_REGION, _cand.OP_GATED_MATMUL) and len(inputs) >= 2:
-            a, b = inputs[0], inputs[1]
-            if len(a.shape) == 2 and len(b.shape) == 2:
-                return (int(a.shape[0]), int(b.shape[1]), int(a.shape[1]))
-        if op == _cand.OP_ATTENTION and len(inputs) >= 3:
-            q, k, v = inputs[:3]
-            if len(q.shape) == len(k.shape) == len(v.shape) == 2:
-                return (int(q.shape[0]), int(k.shape[0]), int(q.shape[1]), int(v.shape[1]))
-    except (AttributeError, IndexError, TypeError, ValueError):
-        pass
+def _named(api: Any, target: str, op: str, name: str, region: Any):
+    for c in api.candidates_for(target, op):
+        if c.name == name and c.applies_to(region) and c.available():
+            return c
     return None
 
 
-def measured_arbitrate(region: Any, op: str, target: str, *inputs: Any, dims=None, dtype: str = "f32",
-                       cache: Optional[MeasureCache] = None, reps: int = 20, warmup: int = 3,
-                       device: Optional[str] = None, timing: str = TIMING_END_TO_END):
-    """The winning candidate by measured latency, or ``None`` when none applies and
-    verifies.  A cache hit returns the recorded winner without re-timing; a miss
-    F4-gates the candidates, times the survivors on ``inputs`` and records the
-    fastest."""
-    if timing not in _TIMING_MODES:
-        raise ValueError(f"unknown autotune timing mode {timing!r}")
-    cache = cache if cache is not None else _DEFAULT_CACHE
-    _maybe_warm_start(cache)
-    dims = dims if dims is not None else _infer_dims(op, inputs)
-    key = (device or device_id(target), target, op, bucket_key(dims), dtype, timing)
-    rec = cache.get(key)
-    if rec is not None:
-        for c in _cand.candidates_for(target, op):
-            if c.name == rec.winner and c.applies_to(region) and c.available():
-                return c
-    latencies: dict = {}
+def tune(api: Any, region: Any, op: str, target: str, *inputs: Any, corpus: Optional[Corpus] = None, dims=None,
+         dtype: str = "f32", device: Optional[str] = None, timing: str = "end_to_end", reps: int = 20,
+         warmup: int = 3):
+    """The candidate to run for this workload, or ``None`` when none is viable.
 
-    def _measure(c) -> float:
-        if timing == TIMING_DEVICE:
-            m = c.measure_device_latency(region, *inputs, reps=reps, warmup=warmup)
-            if m is None:
+    A recorded verdict whose winner is still registered, applicable and available is
+    returned without timing anything.  Otherwise the host's arbiter verifies the
+    candidates and calls back for a latency per survivor (device events through the
+    candidate's ``measure_device_latency`` for ``timing="device"`` — a candidate
+    without one is out of that race — else wall clock around ``run``); the fastest
+    is recorded."""
+    corpus = shared_corpus() if corpus is None else corpus
+    key = Workload.of(device or device_tag(target), target, op, dims if dims is not None else problem_dims(op, inputs),
+                      dtype, timing)
+    known = corpus.lookup(key)
+    if known is not None:
+        c = _named(api, target, op, known.winner, region)
+        if c is not None:
+            return c
+    timed: dict = {}
+
+    def latency(c) -> float:
+        if timing == "device":
+            ms = c.measure_device_latency(region, *inputs, reps=reps, warmup=warmup)
+            if ms is None:
                 return float("inf")
-            t = float(m)
         else:
-            t = measure_latency(lambda: c.run(region, *inputs), reps=reps, warmup=warmup)
-        latencies[c.name] = t
-        return t
+            ms = _wall_ms(lambda: c.run(region, *inputs), reps, warmup)
+        timed[c.name] = float(ms)
+        return float(ms)
 
-    winner = _cand.arbitrate(region, op, target, verify=True, measure=_measure)
-    if winner is not None and winner.name in latencies:
-        cache.put(key, MeasureRecord(winner=winner.name, latency_ms=latencies[winner.name],
-                                     candidates=dict(latencies),
-                                     evidence={"dims": list(dims) if dims is not None else None,
-                                               "reps": reps, "library": Path(_lane.library_path()).name}))
-        return winner
-    return None
+    best = api.arbitrate(region, op, target, verify=True, measure=latency)
+    if best is None or best.name not in timed:
+        return None
+    corpus.record(key, Verdict(best.name, timed[best.name], dict(timed),
+                               {"dims": None if key.bucket is None else list(dims or problem_dims(op, inputs)),
+                                "reps": reps, "library": _lane.library_path().name}))
+    return best
 
 
-def corpus_winner(region: Any, op: str, target: str, *inputs: Any, dims=None, dtype: Optional[str] = None,
-                  cache: Optional[MeasureCache] = None, device: Optional[str] = None,
-                  timing: str = TIMING_END_TO_END) -> Optional[str]:
-    """The persisted winner for this workload when it is unambiguous and still
-    applicable — a selection hint; execution still passes the F4 gate."""
-    cache = cache if cache is not None else _DEFAULT_CACHE
-    _maybe_warm_start(cache)
-    dims = dims if dims is not None else _infer_dims(op, inputs)
+def recommended(api: Any, region: Any, op: str, target: str, *inputs: Any, corpus: Optional[Corpus] = None,
+                dims=None, dtype: Optional[str] = None, device: Optional[str] = None,
+                timing: str = "end_to_end") -> Optional[str]:
+    """The recorded winner for this workload when the records agree on one name and
+    that candidate is still viable here; a hint only — running it still goes through
+    the host's gate."""
+    corpus = shared_corpus() if corpus is None else corpus
+    dims = dims if dims is not None else problem_dims(op, inputs)
     if dims is None:
         return None
-    dev = device or device_id(target)
-    bucket = bucket_key(dims)
-    winners = {rec.winner for (kd, kt, ko, kb, kdt, ktm), rec in cache.items()
-               if kd == dev and kt == target and ko == op and kb == bucket and ktm == timing
-               and (dtype is None or kdt == dtype)}
-    if len(winners) != 1:
+    names = corpus.winners(device or device_tag(target), target, op, pow2_bucket(dims), timing, dtype)
+    if len(names) != 1:
         return None
-    name = next(iter(winners))
-    for c in _cand.candidates_for(target, op):
-        if c.name == name and c.applies_to(region) and c.available():
-            return name
-    return None
+    (name,) = names
+    return name if _named(api, target, op, name, region) is not None else None
 
 
-def run_measured_arbitrated(region: Any, op: str, target: str, *inputs: Any, **kw: Any) -> tuple:
-    """:func:`measured_arbitrate` then run the winner → ``(output, tag)``.  With no
-    viable candidate this raises :class:`~tessera_amd.candidates.ArbiterError`: the
-    lane has no CPU degrade path."""
-    winner = measured_arbitrate(region, op, target, *inputs, **kw)
-    if winner is None:
-        raise _cand.ArbiterError(f"no viable gfx950 candidate for ({target}, {op})")
-    return winner.run(region, *inputs)
+def run_tuned(api: Any, region: Any, op: str, target: str, *inputs: Any, **kw: Any) -> tuple:
+    """:func:`tune`, then run the winner -> ``(output, tag)``; :class:`NoCandidate`
+    when nothing is viable."""
+    best = tune(api, region, op, target, *inputs, **kw)
+    if best is None:
+        raise NoCandidate(f"no viable gfx950 candidate for ({target}, {op})")
+    return best.run(region, *inputs)
 
 
-# ---- corpus generation on the device ----------------------------------------------------
-
-def measure_headline_corpus(cache: Optional[MeasureCache] = None, *, reps: int = 10) -> MeasureCache:
-    """Measure the lane's candidates on the shapes of the headline configurations and
-    record the verdicts (device timing where a candidate offers it)."""
-    cache = cache if cache is not None else MeasureCache()
-    _cand.register_all()
+def measure_headline_corpus(api: Any, regions: Any, corpus: Optional[Corpus] = None, *, reps: int = 10) -> Corpus:
+    """Tune the lane's candidates on the shapes of the headline configurations.
+    ``regions`` supplies the host's region classes (``MatmulRegion``, ``FusedRegion``,
+    ``GatedMatmulRegion``, ``AttentionRegion`` of ``compiler/fusion_core.py``)."""
+    import numpy as np
+    corpus = Corpus() if corpus is None else corpus
+    _cand.register(api)
     rng = np.random.default_rng(0)
-    T = _cand.TARGET
+    tgt = _cand.TARGET
 
     def randn(*shape, s=1.0):
-        return (rng.standard_normal(shape, dtype=np.float32) * np.float32(s))
+        return rng.standard_normal(shape, dtype=np.float32) * np.float32(s)
 
-    for (M, N, K) in ((8192, 8192, 8192), (4096, 8192, 8192), (128, 8192, 8192), (16, 8192, 8192), (1, 8192, 8192),
-                      (512, 256, 64)):
+    for M, N, K in ((8192, 8192, 8192), (4096, 8192, 8192), (128, 8192, 8192), (16, 8192, 8192), (1, 8192, 8192),
+                    (512, 256, 64)):
         A, B = randn(M, K, s=K ** -0.5), randn(K, N, s=K ** -0.5)
         for dt in ("bfloat16", "float16"):
-            measured_arbitrate(_cand.MatmulRegion(dtype=dt), _cand.OP_MATMUL, T, A, B, dtype=dt, cache=cache,
-                               reps=reps, warmup=2, timing=TIMING_DEVICE)
-    for (M, N, K) in ((4096, 4096, 4096), (8192, 1408, 4096)):
+            tune(api, regions.MatmulRegion(dtype=dt), api.OP_MATMUL, tgt, A, B, dtype=dt, corpus=corpus, reps=reps,
+                 warmup=2, timing="device")
+    for M, N, K in ((4096, 4096, 4096), (8192, 1408, 4096)):
         A, B, bias = randn(M, K, s=K ** -0.5), randn(K, N), randn(N)
-        for epi in (("bias", "gelu"), ("bias", "silu"), ("relu",)):
-            measured_arbitrate(_cand.FusedRegion(epilogue=epi, storage_dtype="bf16"), _cand.OP_FUSED_REGION, T, A, B,
-                               bias, dtype="bf16:" + "+".join(epi), cache=cache, reps=max(3, reps // 3), warmup=1)
-        measured_arbitrate(_cand.GatedMatmulRegion("silu", "bf16"), _cand.OP_GATED_MATMUL, T, A, B, randn(K, N),
-                           dtype="bf16", cache=cache, reps=max(3, reps // 3), warmup=1)
-    for (S, D) in ((4096, 128), (1024, 64)):
+        for chain in (("bias", "gelu"), ("bias", "silu"), ("relu",)):
+            tune(api, regions.FusedRegion(epilogue=chain, storage_dtype="bf16"), api.OP_FUSED_REGION, tgt, A, B, bias,
+                 dtype="bf16:" + "+".join(chain), corpus=corpus, reps=max(3, reps // 3), warmup=1)
+        tune(api, regions.GatedMatmulRegion(gate_act="silu", storage_dtype="bf16"), api.OP_GATED_MATMUL, tgt, A, B,
+             randn(K, N), dtype="bf16", corpus=corpus, reps=max(3, reps // 3), warmup=1)
+    for S, D in ((4096, 128), (1024, 64)):
         Q, Kk, V = randn(S, D), randn(S, D), randn(S, D)
         for causal in (False, True):
-            measured_arbitrate(_cand.AttentionRegion(scale=D ** -0.5, causal=causal, storage_dtype="bf16"),
-                               _cand.OP_ATTENTION, T, Q, Kk, V, dtype="bf16:causal" if causal else "bf16",
-                               cache=cache, reps=reps, warmup=2)
-    return cache
-
-
-def _main(argv: list) -> int:
-    out = None
-    if "--out" in argv:
-        out = argv[argv.index("--out") + 1]
-    if not _lane.available():
-        print("gfx950 lane unavailable: the corpus is measured on the MI355X", file=sys.stderr)
-        return 3
-    cache = measure_headline_corpus()
-    p = save_corpus(out, cache)
-    print(f"wrote {cache.size} records to {p}")
-    return 0
-
-
-if __name__ == "__main__":
-    sys.exit(_main(sys.argv[1:]))
+            tune(api, regions.AttentionRegion(scale=D ** -0.5, causal=causal, storage_dtype="bf16"), api.OP_ATTENTION,
+                 tgt, Q, Kk, V, dims=(S, S, D, D), dtype="bf16:causal" if causal else "bf16", corpus=corpus,
+                 reps=reps, warmup=2)
+    return corpus

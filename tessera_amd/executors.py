@@ -84,29 +84,28 @@ KNOWN_EXECUTORS: dict[str, str] = {
                          "(int8 + per-row / per-column scales)",
 }
 
-_ROW = dict(target=TARGET, execution_kind="native_gpu", executable=True, runtime_status="success",
-            execution_mode="hip_runtime")
+_COMMON = dict(target=TARGET, execution_kind="native_gpu", executable=True, runtime_status="success",
+               execution_mode="hip_runtime")
+#: The lane's execution-matrix rows as plain field dicts (the fields of the reference's
+#: ``ExecutionRow``, ``compiler/execution_matrix.py:38-77``), so they can be built with
+#: whichever row class the host hands to :func:`tessera_amd.install.install`.
+ROW_FIELDS: tuple = (
+    dict(_COMMON, compiler_path="gfx950_gemm", executor_id="gfx950_gemm",
+         reason="matmul runs the hand-written gfx950 MFMA GEMM through the "
+                "tessera_gfx950_gemm_{f16,bf16,i8_i32} C ABI symbols"),
+    dict(_COMMON, compiler_path="gfx950_flash_attn", executor_id="gfx950_flash_attn",
+         reason="attention forward runs the hand-written gfx950 MFMA FA-2 kernel (causal, GQA, LSE)"),
+    dict(_COMMON, compiler_path="gfx950_flash_attn_bwd", executor_id="gfx950_flash_attn_bwd",
+         reason="attention backward runs the gfx950 MFMA dQ and dK/dV kernels; O and the "
+                "log-sum-exp are recomputed by the forward kernel (nothing saved)",
+         direction="backward", op_family="flash_attn"),
+    dict(_COMMON, compiler_path="gfx950_moe_transport", executor_id="gfx950_moe_transport",
+         reason="MoE dispatch / combine / grouped GEMM / grouped SwiGLU on the gfx950 lane"),
+    dict(_COMMON, compiler_path="gfx950_quant_gemm", executor_id="gfx950_quant_gemm",
+         reason="fp8-e4m3 and int8 W8A8 GEMM on the gfx950 MFMA lane"),
+)
 EXECUTION_ROWS: dict[tuple[str, str], ExecutionRow] = {
-    (TARGET, "gfx950_gemm"): ExecutionRow(
-        compiler_path="gfx950_gemm", executor_id="gfx950_gemm",
-        reason="matmul runs the hand-written gfx950 MFMA GEMM through the "
-               "tessera_gfx950_gemm_{f16,bf16,i8_i32} C ABI symbols", **_ROW),
-    (TARGET, "gfx950_flash_attn"): ExecutionRow(
-        compiler_path="gfx950_flash_attn", executor_id="gfx950_flash_attn",
-        reason="attention forward runs the hand-written gfx950 MFMA FA-2 kernel "
-               "(causal, GQA, LSE)", **_ROW),
-    (TARGET, "gfx950_flash_attn_bwd"): ExecutionRow(
-        compiler_path="gfx950_flash_attn_bwd", executor_id="gfx950_flash_attn_bwd",
-        reason="attention backward runs the gfx950 MFMA dQ and dK/dV kernels; O and the "
-               "log-sum-exp are recomputed by the forward kernel (nothing saved)",
-        direction="backward", op_family="flash_attn", **_ROW),
-    (TARGET, "gfx950_moe_transport"): ExecutionRow(
-        compiler_path="gfx950_moe_transport", executor_id="gfx950_moe_transport",
-        reason="MoE dispatch / combine / grouped GEMM / grouped SwiGLU on the gfx950 lane", **_ROW),
-    (TARGET, "gfx950_quant_gemm"): ExecutionRow(
-        compiler_path="gfx950_quant_gemm", executor_id="gfx950_quant_gemm",
-        reason="fp8-e4m3 and int8 W8A8 GEMM on the gfx950 MFMA lane", **_ROW),
-}
+    (f["target"], f["compiler_path"]): ExecutionRow(**f) for f in ROW_FIELDS}
 
 
 def lookup(target: str, compiler_path: str) -> Optional[ExecutionRow]:

@@ -8,9 +8,11 @@ from pathlib import Path
 import numpy as np
 import pytest
 
+import standin_host as host
 from tessera_amd import bf16 as b16
 from tessera_amd import candidates as cand
 from tessera_amd import executors as ex
+from tessera_amd import install as inst
 from tessera_amd import lane, ops, tile_table
 
 ROOT = Path(__file__).resolve().parents[1]
@@ -73,10 +75,12 @@ def test_no_device_is_reported_not_faked():
         ops.gemm(b16.from_float32(np.zeros((16, 16))), b16.from_float32(np.zeros((16, 16))))
     with pytest.raises(lane.LaneUnavailable):
         ops.route_tokens(np.zeros((4, 4), np.float32), 4, 2)
-    assert not cand.Gfx950MfmaGemmCandidate().available()
-    assert cand.arbitrate(cand.MatmulRegion(), cand.OP_MATMUL, cand.TARGET) is None
-    with pytest.raises(cand.ArbiterError):
-        cand.run_arbitrated(cand.MatmulRegion(), cand.OP_MATMUL, cand.TARGET, np.zeros((32, 32)), np.zeros((32, 16)))
+    api = host.CandidateHost()
+    made = cand.register(api)
+    assert made and not any(c.available() for c in made)
+    assert api.arbitrate(host.MatmulRegion(), api.OP_MATMUL, cand.TARGET) is None
+    with pytest.raises(host.ArbiterError):
+        api.run(host.MatmulRegion(), api.OP_MATMUL, cand.TARGET, np.zeros((32, 32)), np.zeros((32, 16)))
 
 
 def test_python_side_argument_errors():
@@ -198,53 +202,78 @@ def test_plan_lowering_validates_like_the_reference():
         ex._plan_to_transport(Plan)
 
 
-def test_candidate_registry_semantics():
-    names = [c.name for c in cand.candidates_for(cand.TARGET, cand.OP_MATMUL)]
-    assert names == ["gfx950_mfma_gemm"]
-    cand.register_all()                                           # idempotent
-    assert [c.name for c in cand.candidates_for(cand.TARGET, cand.OP_MATMUL)] == names
-    assert cand.candidates_for(cand.TARGET, cand.OP_GROUPED_GEMM)[0].tier == cand.Tier.HAND_TUNED
+def test_candidates_derive_from_the_injected_host_api():
+    """The plugin owns no registry and no base class: its candidates subclass the
+    Candidate of whichever host API it is given and go through that host's
+    register functions (the reference's backends do the same at import,
+    compiler/emit/rocm_hip.py:809-818)."""
+    api = host.CandidateHost()
+    made = cand.register(api)
+    assert [c.name for c in made] == ["gfx950_mfma_gemm", "gfx950_flash_attn", "gfx950_grouped_gemm",
+                                      "gfx950_mfma_fused_gemm", "gfx950_mfma_gated_gemm"]
+    assert all(isinstance(c, api.Candidate) and c.tier == api.Tier.HAND_TUNED and c.target == cand.TARGET
+               for c in made)
+    by_op = {c.op: c for c in made}
+    assert set(by_op) == {api.OP_MATMUL, api.OP_ATTENTION, cand.OP_GROUPED_GEMM, api.OP_FUSED_REGION,
+                          api.OP_GATED_MATMUL}
+    assert [c.name for c in api.candidates_for(cand.TARGET, api.OP_MATMUL)] == ["gfx950_mfma_gemm"]
+    cand.register(api)                                            # again: replaced by name, not duplicated
+    assert [c.name for c in api.candidates_for(cand.TARGET, api.OP_MATMUL)] == ["gfx950_mfma_gemm"]
+    # a second host gets classes of its own base
+    other = host.CandidateHost()
 
-    class Fake(cand.Candidate):
-        target, op = "fake", cand.OP_MATMUL
-
-        def __init__(self, name, tier, err=0.0, tag="fake_kernel", ok=True):
-            self.name, self.tier, self.err, self.tag, self.ok = name, tier, err, tag, ok
-
-        def available(self):
-            return self.ok
-
-        def run(self, region, A, B, *a, **k):
-            return region.reference(A, B) + self.err, self.tag
-
-    for c in (Fake("slow_good", cand.Tier.SYNTHESIZED), Fake("lead_wrong", cand.Tier.HAND_TUNED, err=1.0),
-              Fake("lead_declines", cand.Tier.HAND_TUNED, tag="reference"), Fake("lead_absent", cand.Tier.HAND_TUNED, ok=False),
-              Fake("emitted_good", cand.Tier.EMITTED)):
-        cand.register_candidate(c)
-    region = cand.MatmulRegion("bfloat16")
-    assert cand.arbitrate(region, cand.OP_MATMUL, "fake").name == "emitted_good"      # wrong/declining leads dropped
-    assert cand.arbitrate(region, cand.OP_MATMUL, "fake", verify=False).name == "lead_wrong"
-    assert cand.arbitrate(region, cand.OP_MATMUL, "fake", measure=lambda c: {"slow_good": 1.0}.get(c.name, 5.0)).name == "slow_good"
-    with pytest.raises(cand.ArbiterError):
-        cand.arbitrate(region, cand.OP_MATMUL, "fake", force="lead_absent")
-    cand.reset_arbiter_dispatch_log()
-    A, B = np.ones((32, 32), np.float32), np.ones((32, 16), np.float32)
-    out, tag = cand.run_arbitrated(region, cand.OP_MATMUL, "fake", A, B)
-    assert tag == "fake_kernel" and np.all(out == 32)
-    assert cand.arbiter_dispatch_histogram()[("fake", cand.OP_MATMUL)] == {"won": 1, "degraded": 0, "no_candidate": 0}
-    with pytest.raises(ValueError):
-        cand.register_candidate(Fake("", cand.Tier.EMITTED))
+    class OtherBase(host.Candidate):
+        pass
+    other.Candidate = OtherBase
+    assert all(isinstance(c, OtherBase) for c in cand.build_candidates(other))
+    # region filters read attributes only
+    gemm, attn, fused, gated = by_op[api.OP_MATMUL], by_op[api.OP_ATTENTION], by_op[api.OP_FUSED_REGION], \
+        by_op[api.OP_GATED_MATMUL]
+    assert gemm.applies_to(host.MatmulRegion("float16")) and not gemm.applies_to(host.MatmulRegion("float32"))
+    assert gemm.mma_prefer_shape == (32, 32, 16) and gemm.mma_arch == "gfx950"
+    assert attn.applies_to(host.AttentionRegion(storage_dtype="bf16"))
+    assert fused.applies_to(host.FusedRegion(("bias", "gelu"))) and not fused.applies_to(host.FusedRegion(("relu", "bias")))
+    assert fused.mma_dtype(host.FusedRegion((), storage_dtype="bf16")) == "bf16"
+    assert gated.applies_to(host.GatedMatmulRegion("sigmoid"))
+    assert by_op[cand.OP_GROUPED_GEMM].applies_to(cand.GroupedGemmRegion((1, 2))) and \
+        not by_op[cand.OP_GROUPED_GEMM].applies_to(cand.GroupedGemmRegion((1, 2), "float16"))
 
 
-def test_region_references():
-    r = cand.MatmulRegion("bfloat16", transpose_b=True)
-    A = np.array([[1 + 2.0 ** -10, 2.0]], np.float32)
-    Bt = np.array([[1024.0, 1.0]], np.float32)                   # raw (N, K)
-    assert r.reference(A, Bt)[0, 0] == 1026.0                    # operand rounded to bf16 first
-    att = cand.AttentionRegion(scale=1.0, causal=True)
-    Q = K = np.eye(4, 16, dtype=np.float32)
-    V = np.arange(64, dtype=np.float32).reshape(4, 16)
-    assert np.allclose(att.reference(Q, K, V)[0], V[0])          # row 0 sees only key 0
+def test_install_registers_into_the_objects_it_is_given():
+    """One call plugs candidates, execution-matrix rows and executor functions into the
+    host's own objects (emit/candidate.py:81-87,206-236; execution_matrix.py:103,
+    2495-2537; runtime.py:30515), and the host's launch then reaches the lane."""
+    api, matrix = host.CandidateHost(), host.MatrixHost()
+    runtime = host.RuntimeHost(matrix)
+    report = inst.install(api, matrix, runtime)
+    assert len(report["candidates"]) == 5 and len(report["rows"]) == 5 and len(report["executors"]) == 5
+    row = matrix._MATRIX[("rocm_gfx950", "gfx950_flash_attn_bwd")]
+    assert isinstance(row, matrix.ExecutionRow) and row.direction == "backward" and row.op_family == "flash_attn"
+    assert row.executable and row.execution_kind == "native_gpu" and row.execution_mode == "hip_runtime"
+    assert ("cpu", "jit_cpu_numpy") in matrix._MATRIX                      # the host's own rows are untouched
+    assert set(report["executors"]) <= set(matrix.KNOWN_EXECUTORS)
+    table = runtime._executor_table()
+    assert "jit_cpu_numpy" in table and table["gfx950_gemm"] is ex.execute_gfx950_gemm
+    assert {r.executor_id for k, r in matrix._MATRIX.items() if k[0] == "rocm_gfx950"} == set(report["executors"])
+    inst.install(api, matrix, runtime)                                     # idempotent: wrapped once
+    assert runtime._executor_table()["gfx950_gemm"] is ex.execute_gfx950_gemm
+    plain: dict = {}
+    inst.install(executor_table=plain)
+    assert set(plain) == set(report["executors"])
+    with pytest.raises(TypeError):
+        inst.install(executor_table=object())
+    # the host's launch resolves the lane's executor and reports its errors in its envelope
+    art = ex.make_artifact("tessera.matmul", ["a", "b"], ["a", "b"], "gfx950_gemm", executable=True)
+    res = runtime.launch(art, (np.zeros((4, 5), np.float16), np.zeros((4, 4), np.float16)))
+    assert res["runtime_status"] == "invalid_artifact" and "matching K" in res["reason"]
+
+
+def test_grouped_gemm_region_definition():
+    r = cand.GroupedGemmRegion((1, 0, 2))
+    x = np.array([[1.0, 2.0], [1.0, 0.0], [0.0, 1 + 2.0 ** -10]], np.float32)
+    w = np.stack([np.eye(2), 7 * np.eye(2), np.array([[1.0, 2.0], [3.0, 4.0]])]).astype(np.float32)
+    want = np.array([[1.0, 2.0], [1.0, 2.0], [3.0, 4.0]], np.float32)     # last row: operand rounded to bf16 first
+    assert np.array_equal(r.reference(x, w), want)
 
 
 def test_tile_table():

@@ -5,6 +5,7 @@ import numpy as np
 import pytest
 import torch
 
+import standin_host as host
 import tessera_oracle as orc
 from tessera_amd import candidates as cand
 from tessera_amd import ops
@@ -18,7 +19,7 @@ def test_epilogue_vocabulary_matches_torch():
            "sigmoid": torch.sigmoid(t), "tanh": torch.tanh(t)}
     for name, want in lib.items():
         assert np.allclose(orc.EPILOGUE_REFS[name](x), want.numpy(), atol=1e-12), name
-        assert np.allclose(cand.EPILOGUE_REFS[name](x), want.numpy(), atol=1e-12), name
+        assert np.allclose(host.POINTWISE[name](x), want.numpy(), atol=1e-12), name
 
 
 def test_fused_epilogue_order_and_closed_forms():
@@ -39,29 +40,29 @@ def test_fused_epilogue_order_and_closed_forms():
     rng = np.random.default_rng(0)
     a, b = rng.standard_normal((8, 12)), rng.standard_normal((12, 16))
     bi = rng.standard_normal(16)
-    r = cand.FusedRegion(epilogue=("bias", "gelu"))
+    r = host.FusedRegion(epilogue=("bias", "gelu"))
     assert np.allclose(r.reference(a, b, bi), orc.fused_epilogue(a, b, bi, ("bias", "gelu")), atol=1e-5)
-    g = cand.GatedMatmulRegion("silu")
+    g = host.GatedMatmulRegion("silu")
     assert np.allclose(g.reference(a, b, b[:, ::-1]), orc.gated_matmul(a, b, b[:, ::-1], "silu"), atol=1e-5)
 
 
 def test_mfma_epilogue_representability():
-    R = cand.FusedRegion
-    assert cand.mfma_epilogue(R(epilogue=("bias",))) == (True, "none")
-    assert cand.mfma_epilogue(R(epilogue=("bias", "silu"))) == (True, "silu")
-    assert cand.mfma_epilogue(R(epilogue=("tanh",))) == (False, "tanh")
-    assert cand.mfma_epilogue(R(epilogue=("relu", "bias"))) is None          # bias after activation
-    assert cand.mfma_epilogue(R(epilogue=("relu", "gelu"))) is None          # two activations
-    assert cand.mfma_epilogue(R(epilogue=("relu",), residual=True)) is None
-    assert cand.mfma_epilogue(R(epilogue=("relu",), reduction="softmax")) is None
-    assert cand.mfma_epilogue(R(epilogue=("relu",), prologue=("gelu",))) is None
-    assert cand.mfma_epilogue(cand.MatmulRegion()) is None
+    R = host.FusedRegion
+    assert cand.fused_epilogue_plan(R(epilogue=("bias",))) == (True, "none")
+    assert cand.fused_epilogue_plan(R(epilogue=("bias", "silu"))) == (True, "silu")
+    assert cand.fused_epilogue_plan(R(epilogue=("tanh",))) == (False, "tanh")
+    assert cand.fused_epilogue_plan(R(epilogue=("relu", "bias"))) is None          # bias after activation
+    assert cand.fused_epilogue_plan(R(epilogue=("relu", "gelu"))) is None          # two activations
+    assert cand.fused_epilogue_plan(R(epilogue=("relu",), residual=True)) is None
+    assert cand.fused_epilogue_plan(R(epilogue=("relu",), reduction="softmax")) is None
+    assert cand.fused_epilogue_plan(R(epilogue=("relu",), prologue=("gelu",))) is None
+    assert cand.fused_epilogue_plan(host.MatmulRegion()) is None
     with pytest.raises(ValueError):
         R(epilogue=("swish",))
     with pytest.raises(ValueError):
         R(epilogue=("bias", "bias"))
     with pytest.raises(ValueError):
-        cand.GatedMatmulRegion("bias")
+        host.GatedMatmulRegion("bias")
 
 
 def test_host_argument_checks_need_no_device():

@@ -4,10 +4,12 @@ match the oracle."""
 import numpy as np
 import pytest
 
+import standin_host as host
 import tessera_oracle as orc
 from tessera_amd import bf16 as b16
 from tessera_amd import candidates as cand
 from tessera_amd import executors as ex
+from tessera_amd import install as inst
 from tessera_amd import ops
 
 pytestmark = pytest.mark.gpu
@@ -73,37 +75,58 @@ def test_launch_moe_transport_executor(lane):
 
 
 def test_arbiter_picks_and_runs_real_kernels(lane):
-    cand.reset_arbiter_dispatch_log()
+    """The candidates, registered into a host through install(), pass the host's gate
+    on real kernels and win its arbitration; nothing is ever tagged as a host-side run."""
+    api = host.CandidateHost()
+    inst.install(api)
     rng = np.random.default_rng(5)
+    gemm = api.candidates_for(cand.TARGET, api.OP_MATMUL)[0]
     for dtype in ("bfloat16", "float16"):
-        region = cand.MatmulRegion(dtype)
-        assert cand.verify_candidate(cand.Gfx950MfmaGemmCandidate(), region)
+        region = host.MatmulRegion(dtype)
+        assert api.verify_candidate(gemm, region)
         A = (rng.standard_normal((64, 96)) * .4).astype(np.float32)
         B = (rng.standard_normal((96, 40)) * .4).astype(np.float32)
-        out, tag = cand.run_arbitrated(region, cand.OP_MATMUL, cand.TARGET, A, B)
-        assert tag == cand.GEMM_TAG and tag not in cand.REFERENCE_EXECUTIONS
-        assert np.allclose(out, region.reference(A, B), atol=1e-3)
-    region = cand.MatmulRegion("bfloat16", transpose_a=True, transpose_b=True)
+        out, tag = api.run(region, api.OP_MATMUL, cand.TARGET, A, B)
+        assert tag == cand.GEMM_TAG and np.allclose(out, region.reference(A, B), atol=1e-3)
+    region = host.MatmulRegion("bfloat16", transpose_a=True, transpose_b=True)
     A = (rng.standard_normal((96, 64)) * .4).astype(np.float32)       # raw (K, M)
     B = (rng.standard_normal((40, 96)) * .4).astype(np.float32)       # raw (N, K)
-    out, tag = cand.run_arbitrated(region, cand.OP_MATMUL, cand.TARGET, A, B)
+    out, tag = api.run(region, api.OP_MATMUL, cand.TARGET, A, B)
     assert tag == cand.GEMM_TAG and np.allclose(out, region.reference(A, B), atol=1e-3)
     for causal in (False, True):
-        att = cand.AttentionRegion(scale=0.25, causal=causal, storage_dtype="bf16")
+        att = host.AttentionRegion(scale=0.25, causal=causal, storage_dtype="bf16")
         Q, K, V = ((rng.standard_normal((48, 32)) * .5).astype(np.float32) for _ in range(3))
-        out, tag = cand.run_arbitrated(att, cand.OP_ATTENTION, cand.TARGET, Q, K, V)
+        out, tag = api.run(att, api.OP_ATTENTION, cand.TARGET, Q, K, V)
         assert tag == cand.ATTN_TAG and np.allclose(out, att.reference(Q, K, V), atol=5e-3)
     gg = cand.GroupedGemmRegion((10, 0, 30), "bfloat16")
     x = (rng.standard_normal((40, 64)) * .4).astype(np.float32)
     w = (rng.standard_normal((3, 64, 32)) * .4).astype(np.float32)
-    out, tag = cand.run_arbitrated(gg, cand.OP_GROUPED_GEMM, cand.TARGET, x, w)
+    out, tag = api.run(gg, cand.OP_GROUPED_GEMM, cand.TARGET, x, w)
     assert tag == cand.GROUPED_TAG and np.allclose(out, gg.reference(x, w), atol=1e-3)
-    hist = cand.arbiter_dispatch_histogram(target=cand.TARGET)
-    assert all(v["degraded"] == 0 and v["no_candidate"] == 0 for v in hist.values())
-    ms = cand.Gfx950MfmaGemmCandidate().measure_device_latency(cand.MatmulRegion("bfloat16"),
-                                                               np.ones((256, 256), np.float32),
-                                                               np.ones((256, 256), np.float32), reps=5, warmup=2)
+    fr = host.FusedRegion(("bias", "gelu"), storage_dtype="bf16")
+    a, b, bias = rng.standard_normal((40, 64)) * .3, rng.standard_normal((64, 48)) * .3, rng.standard_normal(48)
+    out, tag = api.run(fr, api.OP_FUSED_REGION, cand.TARGET, a, b, bias)
+    assert tag == cand.FUSED_TAG and np.allclose(out, fr.reference(a, b, bias), atol=2e-2)
+    gr = host.GatedMatmulRegion("silu", "bf16")
+    out, tag = api.run(gr, api.OP_GATED_MATMUL, cand.TARGET, a, b, b[:, ::-1].copy())
+    assert tag == cand.GATED_TAG and np.allclose(out, gr.reference(a, b, b[:, ::-1]), atol=2e-2)
+    assert len(api.log) == 9 and all(name is not None and t not in api.NOT_A_KERNEL for _, _, name, t in api.log)
+    ms = gemm.measure_device_latency(host.MatmulRegion("bfloat16"), np.ones((256, 256), np.float32),
+                                     np.ones((256, 256), np.float32), reps=5, warmup=2)
     assert ms is not None and 0 < ms < 50
+
+
+def test_installed_lane_is_reached_through_the_hosts_launch(lane):
+    matrix = host.MatrixHost()
+    runtime = host.RuntimeHost(matrix)
+    inst.install(execution_matrix=matrix, executor_table=runtime)
+    rng = np.random.default_rng(9)
+    A = (rng.standard_normal((70, 96)) * .5).astype(np.float16)
+    B = (rng.standard_normal((96, 50)) * .5).astype(np.float16)
+    art = ex.make_artifact("tessera.matmul", ["a", "b"], ["a", "b"], "gfx950_gemm")
+    res = runtime.launch(art, (A, B))
+    assert res["ok"] and res["execution_kind"] == "native_gpu" and res["compiler_path"] == "gfx950_gemm"
+    assert orc.max_rel_err(res["output"], A.astype(np.float64) @ B.astype(np.float64)) <= 1e-5
 
 
 def test_bench_abi(lane):
@@ -116,28 +139,30 @@ def test_bench_abi(lane):
     assert "gfx950" in lane.device_name() and lane.device_cus() > 0
 
 
-def test_measured_arbitration_on_device(lane):
-    """Measure-at-first-miss on the real candidates: the verdict is keyed by the
-    rocm:gfx950 device tag and reused from the cache on the second call."""
+def test_tuning_on_device(lane):
+    """Measure at the first miss on the real candidates: the verdict is keyed by the
+    rocm:gfx950 device tag and reused on the second call."""
     from tessera_amd import autotune as at
-    from tessera_amd import candidates as cand
-    cand.register_all()
+    api = host.CandidateHost()
+    cand.register(api)
     rng = np.random.default_rng(0)
     A = (rng.standard_normal((256, 128)) * .1).astype(np.float32)
     B = (rng.standard_normal((128, 192)) * .1).astype(np.float32)
-    region = cand.MatmulRegion(dtype="bfloat16")
-    cache = at.MeasureCache()
-    w = at.measured_arbitrate(region, cand.OP_MATMUL, cand.TARGET, A, B, dtype="bfloat16", cache=cache, reps=5,
-                              warmup=1, timing=at.TIMING_DEVICE)
+    region = host.MatmulRegion(dtype="bfloat16")
+    corpus = at.Corpus()
+    w = at.tune(api, region, api.OP_MATMUL, cand.TARGET, A, B, dtype="bfloat16", corpus=corpus, reps=5, warmup=1,
+                timing="device")
     assert w is not None and w.name == "gfx950_mfma_gemm"
-    (key, rec), = cache.items()
-    assert key[0] == "rocm:gfx950" and key[3] == (256, 256, 128) and rec.latency_ms > 0
-    hits = cache.hits
-    out, tag = at.run_measured_arbitrated(region, cand.OP_MATMUL, cand.TARGET, A, B, dtype="bfloat16", cache=cache,
-                                          timing=at.TIMING_DEVICE)
-    assert cache.hits == hits + 1 and tag == cand.GEMM_TAG
+    ((key, verdict),) = list(corpus)
+    assert key.device == "rocm:gfx950" and key.bucket == (256, 256, 128) and verdict.latency_ms > 0
+    found = corpus.found
+    out, tag = at.run_tuned(api, region, api.OP_MATMUL, cand.TARGET, A, B, dtype="bfloat16", corpus=corpus,
+                            timing="device")
+    assert corpus.found == found + 1 and tag == cand.GEMM_TAG
     assert np.allclose(out, region.reference(A, B), atol=5e-3)
     # the packaged corpus recommends the same winner for the headline GEMM bucket
     big = np.zeros((8192, 8192), np.float32)
-    assert at.corpus_winner(region, cand.OP_MATMUL, cand.TARGET, big, big, dtype="bfloat16",
-                            timing=at.TIMING_DEVICE) == "gfx950_mfma_gemm"
+    packaged = at.Corpus()
+    packaged.absorb_file(at.PACKAGED)
+    assert at.recommended(api, region, api.OP_MATMUL, cand.TARGET, big, big, corpus=packaged, dtype="bfloat16",
+                          timing="device") == "gfx950_mfma_gemm"
