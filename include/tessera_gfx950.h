@@ -184,6 +184,19 @@ int tessera_gfx950_gemm_bf16_bench_rotating(int M, int N, int K, int iters, int 
  * (tessera_rocm_bench_last_timer_source, tessera_rocm_gemm.cpp:567-580). */
 int tessera_gfx950_bench_last_timer_source(void);
 
+/* Register-only matrix-pipe probe for the bench: 1024 workgroups of 4 waves, each wave
+ * holding 16 independent 32x32x16 bf16 accumulators and issuing `rounds` rounds of those
+ * 16 MFMAs with no memory access inside the loop.  The rate it reaches is what the
+ * matrix pipes deliver on the given operand VALUES at the clock the board grants for them
+ * (operand toggling sets the power draw, the power limit sets the clock), i.e. the
+ * ceiling a GEMM on such data is priced against on this board.  No counterpart in the
+ * reference (its bench ABI times whole GEMMs, tessera_rocm_gemm.cpp:551-667).
+ * fragments: device memory, 16 wave patterns x 8 fragments x 64 lanes x 16 bytes =
+ * 131072 bytes of bf16 values (wave w of the grid uses pattern w % 16: fragments 0-3 as A,
+ * 4-7 as B operands); sink: device memory, 1024 * 256 floats; *flop (may be NULL) receives
+ * the floating-point operations of one launch. */
+int tessera_gfx950_mfma_probe_bf16_dev(const void* fragments, int rounds, void* sink, double* flop, void* stream);
+
 /* ---- quantisers ------------------------------------------------------------ */
 
 /* ops.quantize_fp8(format="e4m3") (python/tessera/__init__.py:3340-3374; grid as
@@ -327,6 +340,51 @@ int tessera_gfx950_moe_route_f32_noalloc_dev(const float* scores, int T, int E, 
                                              float* combine_weights, int32_t* group_sizes,
                                              int32_t* group_offsets, int32_t* num_slots, void* stream);
 
+/* The reference's second router and its packing plan
+ * (python/tessera/models/moe_routing.py:54-113, python/tessera/stdlib/moe.py:79-134).
+ * With router_logits (f32 [T,E]; k <= 64): route_top_k — the k largest LOGITS per token,
+ * descending, ties to the lowest expert id; weights = softmax over the k selected logits
+ * (normalize != 0) or 1/k each (normalize == 0); written to expert_ids / weights ([T,k],
+ * rank order).  With router_logits NULL the selection is given instead (given_expert_ids
+ * int32 [T,k] with values in [0,E) — anything else is rc 1 in the host form —
+ * given_weights f32 [T,k] or NULL): plan_packing / plan_dispatch on a caller's routing.
+ * Then the plan: slots are taken in token-major order, an expert keeps its first
+ * `capacity` slots (capacity <= 0: all), kept slots are stable-sorted by expert.
+ *   kept_mask     uint8 [T,k]   1 = kept
+ *   sort_perm     int32 [S]     kept token-major slot ids in packed order (S = *num_slots)
+ *   inverse_perm  int32 [T*k]   packed position of each slot, -1 for a dropped one
+ *                               (without a capacity: the inverse permutation of sort_perm)
+ *   token_of_slot / expert_of_slot / combine_weights / group_sizes / group_offsets: the
+ *   transport descriptor of the same plan, as tessera_gfx950_moe_route_f32.
+ * Every output except group_sizes / group_offsets may be NULL. */
+int tessera_gfx950_moe_plan_f32(const float* router_logits, const int32_t* given_expert_ids,
+                                const float* given_weights, int T, int E, int k, int normalize, int capacity,
+                                int32_t* expert_ids, float* weights, uint8_t* kept_mask, int32_t* sort_perm,
+                                int32_t* inverse_perm, int32_t* token_of_slot, int32_t* expert_of_slot,
+                                float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
+                                int32_t* num_slots);
+int tessera_gfx950_moe_plan_f32_dev(const float* router_logits, const int32_t* given_expert_ids,
+                                    const float* given_weights, int T, int E, int k, int normalize, int capacity,
+                                    int32_t* expert_ids, float* weights, uint8_t* kept_mask, int32_t* sort_perm,
+                                    int32_t* inverse_perm, int32_t* token_of_slot, int32_t* expert_of_slot,
+                                    float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
+                                    int32_t* num_slots, void* stream);
+/* unpack_combine (python/tessera/models/moe_routing.py:103-111): out[t,:] = sum over the
+ * token's k slots in rank order of y_packed[inverse_perm[t*k+j],:] * weights[t,j], each
+ * product rounded to f32 before the add (numpy's (y_slots * w).sum(axis=1)); a dropped
+ * slot (inverse_perm < 0) adds nothing, as in stdlib.moe.combine.  y_packed [S,N] bf16
+ * or f32, out f32 [T,N]. */
+int tessera_gfx950_moe_unpack_combine_bf16(const void* y_packed, const int32_t* inverse_perm, const float* weights,
+                                           float* out, int T, int k, int S, int N);
+int tessera_gfx950_moe_unpack_combine_f32(const void* y_packed, const int32_t* inverse_perm, const float* weights,
+                                          float* out, int T, int k, int S, int N);
+int tessera_gfx950_moe_unpack_combine_bf16_dev(const void* y_packed, const int32_t* inverse_perm,
+                                               const float* weights, float* out, int T, int k, int S, int N,
+                                               void* stream);
+int tessera_gfx950_moe_unpack_combine_f32_dev(const void* y_packed, const int32_t* inverse_perm,
+                                              const float* weights, float* out, int T, int k, int S, int N,
+                                              void* stream);
+
 /* tessera.moe_dispatch: x_perm[s,:] = x[token_of_slot[s],:]  (exact gather,
  * python/tessera/runtime.py:1791-1806).  elem_bytes = 2 (f16/bf16) or 4 (f32). */
 int tessera_gfx950_moe_dispatch(const void* x, const int32_t* token_of_slot, void* x_perm,
@@ -372,7 +430,8 @@ int tessera_gfx950_moe_swiglu_block_bf16_dev(const void* x, const void* wg, cons
  * input is x[token_of_slot[m]], x the unpermuted bf16 [T,K] activation, so
  * moe_dispatch (python/tessera/stdlib/moe.py:117-125) needs no pass and no x_perm
  * buffer of its own.  token_of_slot: device int32[S] with values in [0, T);
- * T * K * 2 must stay under 4 GiB. */
+ * T * K * 2 must not exceed 2 GiB - 17 (the range of the buffer load that fetches a
+ * token row: rows past it would read as zeros), else rc 1. */
 int tessera_gfx950_moe_swiglu_block_gather_bf16_dev(const void* x, const int32_t* token_of_slot,
                                                     const void* wg, const void* wu, const void* wd,
                                                     const int32_t* offsets, void* y, void* hidden,
@@ -380,13 +439,39 @@ int tessera_gfx950_moe_swiglu_block_gather_bf16_dev(const void* x, const int32_t
 /* The whole local layer nn.functional.moe_layer
  * (python/tessera/nn/functional.py:403-490) with the router logits given:
  * route -> swiglu block (reading x through the dispatch map) -> combine.  out f32
- * [T,N].  The five
- * metadata outputs may each be NULL. */
+ * [T,N].  The five metadata outputs may each be NULL. */
 int tessera_gfx950_moe_layer_bf16(const void* x, const float* router_logits, const void* wg, const void* wu,
                                   const void* wd, float* out, int T, int H, int F, int N, int E, int k,
                                   int normalize, int capacity,
                                   int32_t* token_of_slot, int32_t* expert_of_slot, float* combine_weights,
                                   int32_t* group_sizes, int32_t* group_offsets);
+/* The same layer starting from the router weight: scores = ops.gemm(x, w_router) stored
+ * in bf16 and read as f32 (nn/functional.py:453; w_router bf16 [H,E]), then as above,
+ * without a host hop between the router product and the routing.  router_logits_out
+ * (f32 [T,E], may be NULL) receives the logits the routing saw. */
+int tessera_gfx950_moe_layer_router_bf16(const void* x, const void* w_router, const void* wg, const void* wu,
+                                         const void* wd, float* out, int T, int H, int F, int N, int E, int k,
+                                         int normalize, int capacity,
+                                         int32_t* token_of_slot, int32_t* expert_of_slot, float* combine_weights,
+                                         int32_t* group_sizes, int32_t* group_offsets, float* router_logits_out);
+/* Device-resident form of the layer: router GEMM (when w_router is not NULL; else
+ * router_logits, f32 [T,E], is read) -> routing -> expert block -> combine, enqueued on
+ * one stream with no host synchronisation in between — the chained, resident-operand
+ * execution the device-operand lease of python/tessera/runtime.py:1549-1614 exists for.
+ * All pointers are device memory.  workspace: at least
+ * tessera_gfx950_moe_layer_workspace_bytes(...) bytes, 16-byte aligned (router scores and
+ * logits, the hidden activation [T k, F] and the expert output [T k, N]).  The six
+ * metadata outputs are required (later stages read them): token_of_slot /
+ * expert_of_slot / combine_weights hold T*k entries of which the first *num_slots are
+ * valid.  T * H * 2 must stay inside the 2 GiB buffer range (see the gather block above). */
+int tessera_gfx950_moe_layer_workspace_bytes(int T, int H, int F, int N, int E, int k, size_t* bytes);
+int tessera_gfx950_moe_layer_bf16_dev(const void* x, const void* w_router, const float* router_logits,
+                                      const void* wg, const void* wu, const void* wd, float* out,
+                                      void* workspace, size_t workspace_bytes,
+                                      int T, int H, int F, int N, int E, int k, int normalize, int capacity,
+                                      int32_t* token_of_slot, int32_t* expert_of_slot, float* combine_weights,
+                                      int32_t* group_sizes, int32_t* group_offsets, int32_t* num_slots,
+                                      void* stream);
 
 #ifdef __cplusplus
 }

@@ -27,6 +27,11 @@ flash_attn (+GQA, +LSE)    dense textbook softmax in f64; row 0 -> V[0];
                            ``tessera_x86_flash_attn_ext_lse_f32``
 route_tokens / moe_layer   brute force on tiny inputs; partition invariants;
                            agreement of the two routers' expert sets
+route_top_k / plan /       per-token python sort with (-logit, index) keys; softmax
+unpack_combine             of the selected logits against scipy.special.softmax;
+                           first-come capacity by an independent per-expert walk;
+                           inverse_perm . sort_perm = identity; k = 1 and equal-weight
+                           closed forms of the combine
 fused epilogue / gated     torch.nn.functional relu / gelu(tanh) / silu / sigmoid /
                            tanh library cross-check; relu and zero-bias closed forms
 grouped_gemm / swiglu      per-group matmul; E=1 reduces to dense SwiGLU
@@ -484,6 +489,63 @@ def route_top_k_stable(logits: np.ndarray, top_k: int, normalize: bool = True):
     else:
         w = np.ones_like(sel) / top_k
     return order.astype(np.int64), w.astype(np.float32)
+
+
+@dataclass
+class PackingPlan:
+    """Token-major view of a packing plan (``stdlib/moe.py:58-77``)."""
+    expert_ids: np.ndarray     # (T, k) int64
+    weights: np.ndarray        # (T, k) f32
+    kept_mask: np.ndarray      # (T, k) bool
+    sort_perm: np.ndarray      # (S,) int64 kept token-major slot ids, expert-sorted
+    inverse_perm: np.ndarray   # (T*k,) int64 packed position of each slot, -1 = dropped
+    group_sizes: np.ndarray    # (E,) int64
+
+
+def plan_dispatch_token_major(expert_ids, weights, num_experts: int, capacity: int | None = None) -> PackingPlan:
+    """``stdlib.moe.plan_dispatch`` (``stdlib/moe.py:79-115``): slots in token-major
+    order; once an expert has ``capacity`` slots the rest routed to it are dropped;
+    kept slots stable-sorted by expert.  Without a capacity this is
+    ``models.moe_routing.plan_packing`` (``models/moe_routing.py:80-99``), whose
+    ``inverse_perm`` (``inverse_perm[sort_perm] = arange``) is extended here with -1 for
+    dropped slots."""
+    eids = np.asarray(expert_ids, np.int64)
+    if eids.ndim != 2:
+        raise ValueError("expert_ids must be (T, k)")
+    T, k = eids.shape
+    if eids.size and (eids.min() < 0 or eids.max() >= num_experts):
+        raise ValueError("expert id out of range")
+    flat = eids.reshape(-1)
+    kept = np.ones(flat.shape[0], bool)
+    if capacity is not None:
+        seen = np.zeros(num_experts, np.int64)
+        for s_ in range(flat.shape[0]):
+            e = int(flat[s_])
+            if seen[e] >= capacity:
+                kept[s_] = False
+            else:
+                seen[e] += 1
+    kept_slots = np.nonzero(kept)[0]
+    order = np.argsort(flat[kept_slots], kind="stable")
+    sort_perm = kept_slots[order].astype(np.int64)
+    inverse = np.full(flat.shape[0], -1, np.int64)
+    inverse[sort_perm] = np.arange(sort_perm.shape[0], dtype=np.int64)
+    sizes = np.bincount(flat[sort_perm], minlength=num_experts).astype(np.int64)
+    return PackingPlan(eids, np.asarray(weights, np.float32).reshape(T, k), kept.reshape(T, k), sort_perm, inverse,
+                       sizes)
+
+
+def unpack_combine(y_packed, inverse_perm, weights) -> np.ndarray:
+    """``models.moe_routing.unpack_combine`` (``models/moe_routing.py:109-116``):
+    ``(y_packed[inverse_perm].reshape(T, k, H) * w[:, :, None]).sum(axis=1)`` in f32;
+    a dropped slot (``inverse_perm < 0``) contributes zero, the rule of
+    ``stdlib.moe.combine`` (``stdlib/moe.py:124-134``)."""
+    yp = np.asarray(y_packed, np.float32)
+    w = np.asarray(weights, np.float32)
+    T, k = w.shape
+    inv = np.asarray(inverse_perm, np.int64).reshape(T, k)
+    rows = np.where(inv[:, :, None] >= 0, yp[np.maximum(inv, 0)], np.float32(0))      # (T, k, H)
+    return (rows * w[:, :, None]).sum(axis=1, dtype=np.float32)
 
 
 def grouped_gemm(x, w, group_sizes, dtype: str = "bf16", store: bool = True):

@@ -79,6 +79,17 @@ constexpr float FA_NEG = -1.0e30f;
 __device__ __forceinline__ float swap_half(float v) {
   return __shfl_xor(v, 32, 64);
 }
+// max of a value and the one held by the lane 32 positions away: one
+// v_permlane32_swap (the upper 32 lanes of the first register change places with the
+// lower 32 of the second) leaves both halves' values side by side in every lane, with
+// no LDS round trip.  The operands are finite, so the raw maximum serves.
+__device__ __forceinline__ float max_with_other_half(float v) {
+  const unsigned u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  float d;
+  asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(__uint_as_float(r[0])), "v"(__uint_as_float(r[1])));
+  return d;
+}
 
 // max(a, b, c) in one instruction; the operands are finite MFMA results, so the
 // NaN canonicalisation fmaxf() would add per operand is not needed.
@@ -372,7 +383,7 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
 #pragma unroll
         for (int r = (kt == 0 ? 3 : 0); r < 16; r += 2)
           mx = (r + 1 < 16) ? max3_raw(mx, sc[qt][kt][r], sc[qt][kt][r + 1]) : fmaxf(mx, sc[qt][kt][r]);
-      mx = fmaxf(mx, swap_half(mx));
+      mx = max_with_other_half(mx);
       m_new[qt] = fmaxf(m_run[qt], mx);
       grow = grow || (m_new[qt] > m_run[qt]);
     }

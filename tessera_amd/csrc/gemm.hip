@@ -42,6 +42,46 @@ int gemm16_host(const void* A, const void* B, void* D, int batch, int M, int N, 
   return scope.download(D, dD, d_bytes) ? kOk : kDeviceFailed;
 }
 
+// Register-only MFMA rate probe: every wave keeps 16 independent 32x32x16 bf16
+// accumulators (4 A fragments x 4 B fragments, fetched once) and issues `rounds` rounds of
+// those 16 MFMAs with no memory access in the loop: the rate the matrix pipes reach on
+// the given operand values at the clock the board grants for them.
+constexpr int kProbeBlocks = 1024;
+constexpr int kProbeThreads = 256;
+__global__ __launch_bounds__(kProbeThreads, 1) void mfma_probe_kernel(const uint4* __restrict__ frags, int rounds,
+                                                                       float* __restrict__ sink) {
+  const int lane = threadIdx.x & 63;
+  const int wave = (blockIdx.x * (kProbeThreads / 64) + (threadIdx.x >> 6)) & 15;
+  // 8 fragments per wave pattern, 16 patterns: frags[((pattern * 8) + f) * 64 + lane]
+  uint4 a[4], b[4];
+#pragma unroll
+  for (int f = 0; f < 4; ++f) {
+    a[f] = frags[(wave * 8 + f) * 64 + lane];
+    b[f] = frags[(wave * 8 + 4 + f) * 64 + lane];
+  }
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  for (int it = 0; it < rounds; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x16<BF16>(a[i], b[j], acc[i][j]);
+  }
+  float total = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) total += acc[i][j][r];
+  sink[(size_t)blockIdx.x * kProbeThreads + threadIdx.x] = total;
+}
+
 bool bad_activation(int act) { return act < ACT_NONE || act > ACT_TANH; }
 
 // D f32 = act(A B + bias): the fused matmul epilogue.
@@ -279,5 +319,14 @@ int tessera_gfx950_gemm_bf16_bench_rotating(int M, int N, int K, int iters, int 
 }
 
 int tessera_gfx950_bench_last_timer_source(void) { return g_last_timer_source; }
+
+int tessera_gfx950_mfma_probe_bf16_dev(const void* fragments, int rounds, void* sink, double* flop, void* stream) {
+  if (!fragments || !sink || rounds <= 0 || (reinterpret_cast<uintptr_t>(fragments) & 15)) return kBadShape;
+  if (flop) *flop = (double)kProbeBlocks * (kProbeThreads / 64) * rounds * 16.0 * (2.0 * 32 * 32 * 16);
+  if (probe_device() != kOk) return kNoDevice;
+  hipLaunchKernelGGL(mfma_probe_kernel, dim3(kProbeBlocks), dim3(kProbeThreads), 0, as_stream(stream),
+                     static_cast<const uint4*>(fragments), rounds, static_cast<float*>(sink));
+  return launch_status();
+}
 
 }  // extern "C"

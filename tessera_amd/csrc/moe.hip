@@ -45,74 +45,100 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Selection key of a score: an unsigned integer ordered like the float, with every NaN
+// below every number (numpy's stable descending sort leaves NaNs last) and 0 kept free as
+// the "already taken" marker.  A row of NaN probabilities (a NaN or +inf logit, or a row of
+// -inf, turns the whole softmax into NaN, in numpy as here) is then a row of equal keys and
+// takes experts 0..k-1: every selected id stays inside [0, E).
+__device__ __forceinline__ uint32_t select_key(float v) {
+  if (v != v) return 1u;
+  const uint32_t u = __float_as_uint(v + 0.f);     // -0 and +0 are one key, as they compare equal
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Router variants.  kRouterSoftmaxAll: distributed.moe.route_tokens — softmax over all
+// experts, top-k of the probabilities, weights = those probabilities (renormalised over
+// the k when asked).  kRouterSoftmaxSelected / kRouterUniform: models.moe_routing.route_top_k
+// — top-k of the logits themselves, weights = softmax over the k selected logits, or 1/k.
+constexpr int kRouterSoftmaxAll = 0;
+constexpr int kRouterSoftmaxSelected = 1;
+constexpr int kRouterUniform = 2;
+
 // One wavefront per token.  Lane l owns experts l, l+64, ... (EPL of them).
 template <int EPL>
-__global__ __launch_bounds__(256) void topk_kernel(const float* scores, int T, int E, int k, int normalize,
+__global__ __launch_bounds__(256) void topk_kernel(const float* scores, int T, int E, int k, int normalize, int router,
                                                    int32_t* expert_ids, float* weights) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
   const float* row = scores + (long)t * E;
-  float s[EPL], pr[EPL];
-  float mx = -INFINITY;
+  float pr[EPL];                 // the values the selection ranks: probabilities or logits
 #pragma unroll
   for (int i = 0; i < EPL; ++i) {
     const int e = lane + 64 * i;
-    s[i] = e < E ? row[e] : -INFINITY;
-    mx = fmaxf(mx, s[i]);
+    pr[i] = e < E ? row[e] : -INFINITY;
   }
-  mx = wave_max(mx);
-  float sum = 0.f;
+  if (router == kRouterSoftmaxAll) {
+    float mx = -INFINITY;
 #pragma unroll
-  for (int i = 0; i < EPL; ++i) {
-    const int e = lane + 64 * i;
-    pr[i] = e < E ? expf(s[i] - mx) : 0.f;
-    sum += pr[i];
-  }
-  sum = wave_sum(sum);
-  // A NaN or +inf logit, or a row of -inf, makes the sum (the same value in every lane)
-  // and with it every probability of the row NaN, in numpy as here.  NaN compares false
-  // with everything, so such a row is selected on equal keys instead: it takes experts
-  // 0..k-1 (ties go to the lowest id) with NaN weights, and every id stays inside [0, E).
-  const bool nan_row = !(sum == sum);
-#pragma unroll
-  for (int i = 0; i < EPL; ++i) {
-    const int e = lane + 64 * i;
-    pr[i] = e < E ? (nan_row ? 0.f : __fdiv_rn(pr[i], sum)) : -1.f;    // -1 never wins a selection
-  }
-  float wsum = 0.f;
-  float my_w = 0.f;       // lane j keeps the j-th selected weight
-  int my_e = -1;
-  for (int j = 0; j < k; ++j) {
-    // best (value desc, index asc) among this lane's experts, then across lanes
-    float bv = -2.f;
-    int be = 0x7fffffff;
+    for (int i = 0; i < EPL; ++i) mx = fmaxf(mx, pr[i]);
+    mx = wave_max(mx);
+    float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < EPL; ++i) {
       const int e = lane + 64 * i;
-      if (pr[i] > bv) { bv = pr[i]; be = e; }      // ascending e inside a lane: first max wins
+      pr[i] = e < E ? expf(pr[i] - mx) : 0.f;
+      sum += pr[i];
     }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) pr[i] = __fdiv_rn(pr[i], sum);
+  }
+  uint32_t key[EPL];
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) key[i] = lane + 64 * i < E ? select_key(pr[i]) : 0u;
+  float wsum = 0.f;
+  float my_w = 0.f;       // lane j keeps the j-th selected value
+  int my_e = -1;
+  for (int j = 0; j < k; ++j) {
+    // best (key desc, index asc) among this lane's experts, then across lanes
+    uint32_t bk = 0u;
+    int be = 0x7fffffff;
+    float bv = 0.f;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i)
+      if (key[i] > bk) { bk = key[i]; be = lane + 64 * i; bv = pr[i]; }   // ascending e inside a lane: first max wins
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(bv, o, 64);
+      const uint32_t ok = __shfl_xor(bk, o, 64);
       const int oe = __shfl_xor(be, o, 64);
-      if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
+      const float ov = __shfl_xor(bv, o, 64);
+      if (ok > bk || (ok == bk && oe < be)) { bk = ok; be = oe; bv = ov; }
     }
 #pragma unroll
     for (int i = 0; i < EPL; ++i)
-      if (lane + 64 * i == be) pr[i] = -1.f;       // remove the winner
-    if (lane == (j & 63)) { my_w = nan_row ? __builtin_nanf("") : bv; my_e = be; }
+      if (lane + 64 * i == be) key[i] = 0u;        // remove the winner
+    if (lane == (j & 63)) { my_w = bv; my_e = be; }
     wsum += bv;
     if ((j & 63) == 63 || j == k - 1) {
       // flush up to 64 selections (k <= 64 in practice; the loop form keeps it general)
       const int base = j - (j & 63);
+      float w_out = my_w;
+      if (router != kRouterSoftmaxAll) {
+        // (the launcher admits these routers for k <= 64 only: one flush holds the whole row)
+        const bool mine = lane < k;
+        const float top = wave_max(mine ? my_w : -INFINITY);
+        const float ex = mine ? expf(my_w - top) : 0.f;
+        const float tot = wave_sum(ex);
+        w_out = router == kRouterUniform ? __fdiv_rn(1.0f, (float)k) : __fdiv_rn(ex, tot);
+      }
       if (lane <= (j & 63)) {
         expert_ids[(long)t * k + base + lane] = my_e;
-        weights[(long)t * k + base + lane] = my_w;
+        weights[(long)t * k + base + lane] = w_out;
       }
     }
   }
-  if (normalize && k > 1) {
+  if (router == kRouterSoftmaxAll && normalize && k > 1) {
     const float d = wsum > 0.f ? wsum : 1.f;
     for (int j = lane; j < k; j += 64) weights[(long)t * k + j] = __fdiv_rn(weights[(long)t * k + j], d);
   }
@@ -186,7 +212,8 @@ __global__ __launch_bounds__(256) void scan_kernel(int32_t* chunk_counts, int ch
 __global__ __launch_bounds__(64) void place_kernel(const int32_t* expert_ids, const float* weights, int S, int E,
                                                    int k, int capacity, const int32_t* chunk_base,
                                                    const int32_t* group_offsets, int32_t* token_of_slot,
-                                                   int32_t* expert_of_slot, float* combine_weights) {
+                                                   int32_t* expert_of_slot, float* combine_weights,
+                                                   int32_t* sort_perm, int32_t* inverse_perm, uint8_t* kept_mask) {
   __shared__ int cursor[kMaxExperts];
   const int lane = threadIdx.x;
   for (int e = lane; e < E; e += 64) cursor[e] = chunk_base[(long)blockIdx.x * E + e];
@@ -215,11 +242,19 @@ __global__ __launch_bounds__(64) void place_kernel(const int32_t* expert_ids, co
     if (valid && (same >> lane) == 1ull) cursor[e] += __popcll(same);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    if (valid && (capacity <= 0 || rank < capacity)) {
-      const int pos = group_offsets[e] + rank;
-      token_of_slot[pos] = s / k;
-      expert_of_slot[pos] = e;
-      combine_weights[pos] = weights[s];
+    const bool kept = valid && (capacity <= 0 || rank < capacity);
+    int pos = -1;
+    if (kept) {
+      pos = group_offsets[e] + rank;
+      if (token_of_slot) token_of_slot[pos] = s / k;
+      if (expert_of_slot) expert_of_slot[pos] = e;
+      if (combine_weights) combine_weights[pos] = weights[s];
+      if (sort_perm) sort_perm[pos] = s;
+    }
+    // the packing plan in the token-major view: where a slot went (-1 = dropped)
+    if (s < S) {
+      if (inverse_perm) inverse_perm[s] = pos;
+      if (kept_mask) kept_mask[s] = kept ? 1 : 0;
     }
   }
 }
@@ -239,29 +274,49 @@ bool bad_route(const float* scores, int T, int E, int k, const int32_t* token_of
   return (long)T * k > 0x7fffffffL;      // int32 device ABI
 }
 
-// The four routing kernels on stream `s`, their temporaries in `ws` (device memory of at
+// Extra outputs of the packing plan in the token-major view (stdlib.moe.plan_dispatch,
+// models.moe_routing.plan_packing); each may be null.
+struct PlanOutputs {
+  int32_t* expert_ids = nullptr;     // (T, k) selected experts, rank order
+  float* weights = nullptr;          // (T, k) route weights, rank order
+  uint8_t* kept_mask = nullptr;      // (T, k) 1 = kept, 0 = dropped over capacity
+  int32_t* sort_perm = nullptr;      // [S] kept token-major slot ids, expert-sorted
+  int32_t* inverse_perm = nullptr;   // [T k] position of a slot in the packed order, -1 = dropped
+};
+
+// The routing kernels on stream `s`, their temporaries in `ws` (device memory of at
 // least route_workspace_bytes(T * k, E) bytes; every byte a kernel reads is written by an
-// earlier kernel of the same call, so `ws` needs no clearing).
-int route_launch(const float* scores, int T, int E, int k, int normalize, int capacity, int32_t* token_of_slot,
-                 int32_t* expert_of_slot, float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
-                 int32_t* num_slots, char* ws, hipStream_t s) {
+// earlier kernel of the same call, so `ws` needs no clearing).  `scores` null: the
+// selection is given (given_ids / given_weights, (T, k)) and only the plan is built.
+int route_launch(const float* scores, int T, int E, int k, int normalize, int capacity, int router,
+                 int32_t* token_of_slot, int32_t* expert_of_slot, float* combine_weights, int32_t* group_sizes,
+                 int32_t* group_offsets, int32_t* num_slots, char* ws, hipStream_t s,
+                 const PlanOutputs& plan = PlanOutputs{}, const int32_t* given_ids = nullptr,
+                 const float* given_weights = nullptr) {
   const int S = T * k;
   const int chunks = ceil_div(S, kSlotsPerChunk);
   const size_t slot_bytes = ((size_t)S * 4 + 255) & ~(size_t)255;
-  int32_t* ids = reinterpret_cast<int32_t*>(ws);
-  float* w = reinterpret_cast<float*>(ws + slot_bytes);
+  // the token-major selection goes straight to the caller's arrays when it wants them
+  int32_t* ids = plan.expert_ids ? plan.expert_ids : reinterpret_cast<int32_t*>(ws);
+  float* w = plan.weights ? plan.weights : reinterpret_cast<float*>(ws + slot_bytes);
   int32_t* counts = reinterpret_cast<int32_t*>(ws + 2 * slot_bytes);
-  const dim3 tgrid(ceil_div(T, 4));
-  const int epl = ceil_div(E, 64);
-  if (epl <= 1) hipLaunchKernelGGL((topk_kernel<1>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, ids, w);
-  else if (epl <= 2) hipLaunchKernelGGL((topk_kernel<2>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, ids, w);
-  else if (epl <= 4) hipLaunchKernelGGL((topk_kernel<4>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, ids, w);
-  else hipLaunchKernelGGL((topk_kernel<16>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, ids, w);
+  if (scores) {
+    const dim3 tgrid(ceil_div(T, 4));
+    const int epl = ceil_div(E, 64);
+    if (epl <= 1) hipLaunchKernelGGL((topk_kernel<1>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, router, ids, w);
+    else if (epl <= 2) hipLaunchKernelGGL((topk_kernel<2>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, router, ids, w);
+    else if (epl <= 4) hipLaunchKernelGGL((topk_kernel<4>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, router, ids, w);
+    else hipLaunchKernelGGL((topk_kernel<16>), tgrid, dim3(256), 0, s, scores, T, E, k, normalize, router, ids, w);
+  } else {
+    ids = const_cast<int32_t*>(given_ids);
+    w = const_cast<float*>(given_weights);
+  }
   hipLaunchKernelGGL(count_kernel, dim3(chunks), dim3(64), 0, s, ids, S, E, counts);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(256), 0, s, counts, chunks, E, capacity, group_sizes, group_offsets,
                      num_slots);
   hipLaunchKernelGGL(place_kernel, dim3(chunks), dim3(64), 0, s, ids, w, S, E, k, capacity, counts, group_offsets,
-                     token_of_slot, expert_of_slot, combine_weights);
+                     token_of_slot, expert_of_slot, combine_weights, plan.sort_perm, plan.inverse_perm,
+                     plan.kept_mask);
   return launch_status();
 }
 
@@ -276,8 +331,25 @@ int route_dev(const float* scores, int T, int E, int k, int normalize, int capac
   // and three stream-ordered allocate / free pairs less on the host side of a call.
   char* ws = static_cast<char*>(stream_workspace(s, route_workspace_bytes(T * k, E)));
   if (!ws) return kDeviceFailed;
-  return route_launch(scores, T, E, k, normalize, capacity, token_of_slot, expert_of_slot, combine_weights,
-                      group_sizes, group_offsets, num_slots, ws, s);
+  return route_launch(scores, T, E, k, normalize, capacity, kRouterSoftmaxAll, token_of_slot, expert_of_slot,
+                      combine_weights, group_sizes, group_offsets, num_slots, ws, s);
+}
+
+// route_top_k (or a given selection) + the packing plan with its token-major outputs.
+int plan_dev(const float* logits, const int32_t* given_ids, const float* given_weights, int T, int E, int k,
+             int router, int capacity, const PlanOutputs& plan, int32_t* token_of_slot, int32_t* expert_of_slot,
+             float* combine_weights, int32_t* group_sizes, int32_t* group_offsets, int32_t* num_slots, hipStream_t s) {
+  if (T <= 0 || E <= 0 || k <= 0 || k > E || E > kMaxExperts || (long)T * k > 0x7fffffffL || !group_sizes ||
+      !group_offsets)
+    return kBadShape;
+  if (logits ? (router != kRouterSoftmaxSelected && router != kRouterUniform) || k > 64
+             : (!given_ids || (combine_weights && !given_weights)))
+    return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  char* ws = static_cast<char*>(stream_workspace(s, route_workspace_bytes(T * k, E)));
+  if (!ws) return kDeviceFailed;
+  return route_launch(logits, T, E, k, 0, capacity, router, token_of_slot, expert_of_slot, combine_weights,
+                      group_sizes, group_offsets, num_slots, ws, s, plan, given_ids, given_weights);
 }
 
 // Device address of `scratch` on the current device, looked up once per device.
@@ -322,9 +394,11 @@ __global__ __launch_bounds__(256) void dispatch_kernel(const char* x, const int3
 // The slots of a token are found by sorting slot ids by token (count, scan,
 // fill); each token then adds its slots in ascending slot order — the order of
 // the reference's unbuffered scatter-add — so the f32 result is reproducible.
-__global__ void combine_count_kernel(const int32_t* token_of_slot, int S, int T, int32_t* cnt) {
+// (n_dev, when given, is the device-side number of valid slots: the host then only
+// knows the upper bound S)
+__global__ void combine_count_kernel(const int32_t* token_of_slot, int S, int T, int32_t* cnt, const int32_t* n_dev) {
   const int s = blockIdx.x * blockDim.x + threadIdx.x;
-  if (s >= S) return;
+  if (s >= S || (n_dev && s >= *n_dev)) return;
   const int t = token_of_slot[s];
   if (t >= 0 && t < T) atomicAdd(&cnt[t], 1);
 }
@@ -372,9 +446,9 @@ __global__ __launch_bounds__(1024) void combine_scan_kernel(int32_t* cnt, int T,
   }
 }
 __global__ void combine_fill_kernel(const int32_t* token_of_slot, int S, int T, const int32_t* off, int32_t* cursor,
-                                    int32_t* list) {
+                                    int32_t* list, const int32_t* n_dev) {
   const int s = blockIdx.x * blockDim.x + threadIdx.x;
-  if (s >= S) return;
+  if (s >= S || (n_dev && s >= *n_dev)) return;
   const int t = token_of_slot[s];
   if (t >= 0 && t < T) list[off[t] + atomicAdd(&cursor[t], 1)] = s;
 }
@@ -476,9 +550,69 @@ __global__ __launch_bounds__(256) void combine_kernel(const YT* y, const float* 
   }
 }
 
+// models.moe_routing.unpack_combine: out[t, :] = sum over the token's k slots, in rank
+// order j = 0..k-1, of y[inverse_perm[t k + j], :] * w[t, j]; the product is rounded before
+// the add, like numpy's (y_slots * w).sum(axis=1).  A dropped slot (inverse_perm < 0)
+// adds nothing.  One workgroup per token, 16-byte loads when the rows allow.
+template <class YT, bool VEC>
+__global__ __launch_bounds__(256) void unpack_combine_kernel(const YT* y, const int32_t* inverse_perm, const float* w,
+                                                             float* out, int k, int N, int S) {
+  constexpr int RUN = VEC ? 16 / (int)sizeof(YT) : 1;
+  const int t = blockIdx.x;
+  for (int n = threadIdx.x * RUN; n < N; n += 256 * RUN) {
+    float acc[RUN];
+#pragma unroll
+    for (int e = 0; e < RUN; ++e) acc[e] = 0.f;
+    for (int j = 0; j < k; ++j) {
+      const int pos = inverse_perm[(long)t * k + j];
+      if (pos < 0 || pos >= S) continue;
+      const float wt = w[(long)t * k + j];
+      const YT* src = y + (long)pos * N + n;
+      if constexpr (VEC) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(src);
+        const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int e = 0; e < RUN; ++e) {
+          float v;
+          if constexpr (sizeof(YT) == 2) v = __uint_as_float((e & 1) ? (u[e >> 1] & 0xffff0000u) : (u[e >> 1] << 16));
+          else v = __uint_as_float(u[e]);
+          acc[e] = add_rounded_product(acc[e], v, wt);
+        }
+      } else {
+        float v;
+        if constexpr (sizeof(YT) == 2) v = bf16_bits_to_f32(src[0]);
+        else v = src[0];
+        acc[0] = add_rounded_product(acc[0], v, wt);
+      }
+    }
+    if constexpr (VEC) {
+#pragma unroll
+      for (int e = 0; e < RUN; e += 4)
+        *reinterpret_cast<float4*>(out + (long)t * N + n + e) = make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
+    } else {
+      out[(long)t * N + n] = acc[0];
+    }
+  }
+}
+
+template <class YT>
+int unpack_combine_dev(const void* y, const int32_t* inverse_perm, const float* w, float* out, int T, int k, int S,
+                       int N, hipStream_t s) {
+  if (T <= 0 || k <= 0 || S < 0 || N <= 0 || !out || !inverse_perm || !w || (S > 0 && !y)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const bool vec = N % (16 / (int)sizeof(YT)) == 0 && aligned16(y) && aligned16(out);
+  if (vec)
+    hipLaunchKernelGGL((unpack_combine_kernel<YT, true>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y),
+                       inverse_perm, w, out, k, N, S);
+  else
+    hipLaunchKernelGGL((unpack_combine_kernel<YT, false>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y),
+                       inverse_perm, w, out, k, N, S);
+  return launch_status();
+}
+
 template <class YT>
 int combine_dev(const void* y, const int32_t* token_of_slot, const float* w, float* out, int T, int S, int N,
-                hipStream_t s) {
+                hipStream_t s, const int32_t* n_dev = nullptr) {
   if (T <= 0 || S < 0 || N <= 0 || !out || (S > 0 && (!y || !token_of_slot || !w))) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
   // the per-token slot lists live in the stream's own workspace (the combine kernel below
@@ -490,9 +624,9 @@ int combine_dev(const void* y, const int32_t* token_of_slot, const float* w, flo
   int32_t* off = reinterpret_cast<int32_t*>(ws + tok_bytes);
   int32_t* list = reinterpret_cast<int32_t*>(ws + 2 * tok_bytes);
   zero_words(cnt, (size_t)T, s);
-  if (S > 0) hipLaunchKernelGGL(combine_count_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, cnt);
+  if (S > 0) hipLaunchKernelGGL(combine_count_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, cnt, n_dev);
   hipLaunchKernelGGL(combine_scan_kernel, dim3(1), dim3(1024), 0, s, cnt, T, off);
-  if (S > 0) hipLaunchKernelGGL(combine_fill_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, off, cnt, list);
+  if (S > 0) hipLaunchKernelGGL(combine_fill_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, off, cnt, list, n_dev);
   const bool vec = N % (16 / (int)sizeof(YT)) == 0 && aligned16(y) && aligned16(out);
   if (vec)
     hipLaunchKernelGGL((combine_kernel<YT, true>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, off, list, out, N);
@@ -569,6 +703,136 @@ int swiglu_dev(const void* x, const void* wg, const void* wu, const void* wd, co
   return rc;
 }
 
+// bf16 bit patterns -> f32 (exact widening), 8 per thread.
+__global__ __launch_bounds__(256) void widen_bf16_kernel(const uint16_t* __restrict__ in, float* __restrict__ out, long n) {
+  const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i + 8 <= n) {
+    const uint4 v = *reinterpret_cast<const uint4*>(in + i);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+    float4 lo, hi;
+    lo.x = __uint_as_float(u[0] << 16); lo.y = __uint_as_float(u[0] & 0xffff0000u);
+    lo.z = __uint_as_float(u[1] << 16); lo.w = __uint_as_float(u[1] & 0xffff0000u);
+    hi.x = __uint_as_float(u[2] << 16); hi.y = __uint_as_float(u[2] & 0xffff0000u);
+    hi.z = __uint_as_float(u[3] << 16); hi.w = __uint_as_float(u[3] & 0xffff0000u);
+    *reinterpret_cast<float4*>(out + i) = lo;
+    *reinterpret_cast<float4*>(out + i + 4) = hi;
+  } else {
+    for (long j = i; j < n; ++j) out[j] = bf16_bits_to_f32(in[j]);
+  }
+}
+
+inline size_t round256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+// Device scratch of the whole layer: router scores (bf16) and logits (f32), the hidden
+// activation h [T k, F] and the expert output y [T k, N] (both bf16).
+struct LayerScratch {
+  size_t scores, logits, hidden, y, total;
+};
+LayerScratch layer_scratch(int T, int F, int N, int E, int k) {
+  LayerScratch w{};
+  const size_t S = (size_t)T * k;
+  w.scores = 0;
+  w.logits = w.scores + round256((size_t)T * E * 2);
+  w.hidden = w.logits + round256((size_t)T * E * 4);
+  w.y = w.hidden + round256(S * F * 2);
+  w.total = w.y + round256(S * N * 2);
+  return w;
+}
+
+bool bad_layer(int T, int H, int F, int N, int E, int k) {
+  return T <= 0 || H <= 0 || F <= 0 || N <= 0 || E <= 0 || k <= 0 || k > E || E > kMaxExperts ||
+         (long)T * k > 0x7fffffffL;
+}
+
+// nn.functional.moe_layer on one stream, no host hop: (router GEMM ->) route -> expert
+// block reading x through the dispatch map -> combine.  With a capacity the number of
+// kept slots is only known on the device (*num_slots): every later stage is launched
+// for the upper bound T k and takes its real extent from the device-side offsets / count.
+int moe_layer_dev(const void* x, const void* w_router, const float* router_logits, const void* wg, const void* wu,
+                  const void* wd, float* out, void* workspace, size_t workspace_bytes, int T, int H, int F, int N,
+                  int E, int k, int normalize, int capacity, int32_t* token_of_slot, int32_t* expert_of_slot,
+                  float* combine_weights, int32_t* group_sizes, int32_t* group_offsets, int32_t* num_slots,
+                  hipStream_t s) {
+  if (bad_layer(T, H, F, N, E, k) || !x || (!w_router && !router_logits) || !wg || !wu || !wd || !out ||
+      !workspace || !token_of_slot || !expert_of_slot || !combine_weights || !group_sizes || !group_offsets ||
+      !num_slots || !aligned16(workspace))
+    return kBadShape;
+  const LayerScratch w = layer_scratch(T, F, N, E, k);
+  if (workspace_bytes < w.total) return kBadShape;
+  if (gather_out_of_buffer_range(T, H)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  char* ws = static_cast<char*>(workspace);
+  const float* logits = router_logits;
+  if (w_router) {
+    // scores = ops.gemm(x, W_router): stored in bf16 like every reduced-precision
+    // product, then read as f32 (nn/functional.py:453)
+    Gemm16Params g{};
+    g.A = static_cast<const uint16_t*>(x);
+    g.B = static_cast<const uint16_t*>(w_router);
+    g.D = ws + w.scores;
+    g.M = T; g.N = E; g.K = H;
+    g.lda = H; g.ldb = E; g.ldd = E;
+    g.strideA = (long)T * H; g.strideB = (long)H * E; g.strideD = (long)T * E;
+    g.groups = 1;
+    if (const int rc = launch_gemm16<BF16, EPI_STORE16>(g, s); rc != kOk) return rc;
+    const long n = (long)T * E;
+    hipLaunchKernelGGL(widen_bf16_kernel, dim3((unsigned)((n + 2047) / 2048)), dim3(256), 0, s,
+                       reinterpret_cast<const uint16_t*>(ws + w.scores), reinterpret_cast<float*>(ws + w.logits), n);
+    logits = reinterpret_cast<const float*>(ws + w.logits);
+  }
+  int rc = route_dev(logits, T, E, k, normalize, capacity, token_of_slot, expert_of_slot, combine_weights,
+                     group_sizes, group_offsets, num_slots, s);
+  if (rc != kOk) return rc;
+  const int S = T * k;
+  rc = swiglu_dev(x, wg, wu, wd, group_offsets, ws + w.y, ws + w.hidden, S, H, F, N, E, s, token_of_slot, T);
+  if (rc != kOk) return rc;
+  return combine_dev<uint16_t>(ws + w.y, token_of_slot, combine_weights, out, T, S, N, s, num_slots);
+}
+
+// Host-pointer form of the layer: upload, run moe_layer_dev, download.
+int moe_layer_host(const void* x, const void* w_router, const float* router_logits, const void* wg, const void* wu,
+                   const void* wd, float* out, int T, int H, int F, int N, int E, int k, int normalize, int capacity,
+                   int32_t* token_of_slot, int32_t* expert_of_slot, float* combine_weights, int32_t* group_sizes,
+                   int32_t* group_offsets, float* logits_out) {
+  if (bad_layer(T, H, F, N, E, k) || !x || (!w_router && !router_logits) || !wg || !wu || !wd || !out)
+    return kBadShape;
+  if (gather_out_of_buffer_range(T, H)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t S = (size_t)T * k;
+  const LayerScratch w = layer_scratch(T, F, N, E, k);
+  DeviceScope scope;
+  void* dx = scope.alloc((size_t)T * H * 2, x);
+  void* dr = w_router ? scope.alloc((size_t)H * E * 2, w_router) : nullptr;
+  float* dl = router_logits && !w_router ? static_cast<float*>(scope.alloc((size_t)T * E * 4, router_logits)) : nullptr;
+  void* dg = scope.alloc((size_t)E * H * F * 2, wg);
+  void* du = scope.alloc((size_t)E * H * F * 2, wu);
+  void* dd = scope.alloc((size_t)E * F * N * 2, wd);
+  int32_t* dt = static_cast<int32_t*>(scope.alloc(S * 4));
+  int32_t* de = static_cast<int32_t*>(scope.alloc(S * 4));
+  float* dw = static_cast<float*>(scope.alloc(S * 4));
+  int32_t* dgs = static_cast<int32_t*>(scope.alloc((size_t)E * 4));
+  int32_t* dof = static_cast<int32_t*>(scope.alloc((size_t)(E + 1) * 4));
+  int32_t* dn = static_cast<int32_t*>(scope.alloc(4));
+  void* dws = scope.alloc(w.total);
+  float* dout = static_cast<float*>(scope.alloc((size_t)T * N * 4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = moe_layer_dev(dx, dr, dl, dg, du, dd, dout, dws, w.total, T, H, F, N, E, k, normalize, capacity, dt, de,
+                         dw, dgs, dof, dn, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  int32_t n = 0;                       // kept slots (a capacity may drop some)
+  if (!scope.download(&n, dn, 4) || !scope.download(out, dout, (size_t)T * N * 4)) return kDeviceFailed;
+  if (token_of_slot && !scope.download(token_of_slot, dt, (size_t)n * 4)) return kDeviceFailed;
+  if (expert_of_slot && !scope.download(expert_of_slot, de, (size_t)n * 4)) return kDeviceFailed;
+  if (combine_weights && !scope.download(combine_weights, dw, (size_t)n * 4)) return kDeviceFailed;
+  if (group_sizes && !scope.download(group_sizes, dgs, (size_t)E * 4)) return kDeviceFailed;
+  if (group_offsets && !scope.download(group_offsets, dof, (size_t)(E + 1) * 4)) return kDeviceFailed;
+  if (logits_out && w_router &&
+      !scope.download(logits_out, static_cast<char*>(dws) + w.logits, (size_t)T * E * 4))
+    return kDeviceFailed;
+  return kOk;
+}
+
 int combine_host(const void* y_perm, const int32_t* token_of_slot, const float* weights, float* out, int T,
                         int S, int N, int ysz) {
   if (T <= 0 || S < 0 || N <= 0 || !out || (S > 0 && (!y_perm || !token_of_slot || !weights))) return kBadShape;
@@ -638,8 +902,8 @@ int tessera_gfx950_moe_route_f32_noalloc_dev(const float* scores, int T, int E, 
   if (probe_device() != kOk) return kNoDevice;
   char* ws = nullptr;
   if (const int rc = route_scratch(&ws); rc != kOk) return rc;
-  return route_launch(scores, T, E, k, normalize, capacity, token_of_slot, expert_of_slot, combine_weights,
-                      group_sizes, group_offsets, num_slots, ws, as_stream(stream));
+  return route_launch(scores, T, E, k, normalize, capacity, kRouterSoftmaxAll, token_of_slot, expert_of_slot,
+                      combine_weights, group_sizes, group_offsets, num_slots, ws, as_stream(stream));
 }
 
 int tessera_gfx950_moe_route_f32(const float* scores, int T, int E, int k, int normalize, int capacity,
@@ -670,6 +934,112 @@ int tessera_gfx950_moe_route_f32(const float* scores, int T, int E, int k, int n
     return kDeviceFailed;
   if (num_slots) *num_slots = n;
   return kOk;
+}
+
+int tessera_gfx950_moe_plan_f32_dev(const float* router_logits, const int32_t* given_expert_ids,
+                                    const float* given_weights, int T, int E, int k, int normalize, int capacity,
+                                    int32_t* expert_ids, float* weights, uint8_t* kept_mask, int32_t* sort_perm,
+                                    int32_t* inverse_perm, int32_t* token_of_slot, int32_t* expert_of_slot,
+                                    float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
+                                    int32_t* num_slots, void* stream) {
+  PlanOutputs plan;
+  plan.expert_ids = router_logits ? expert_ids : nullptr;
+  plan.weights = router_logits ? weights : nullptr;
+  plan.kept_mask = kept_mask;
+  plan.sort_perm = sort_perm;
+  plan.inverse_perm = inverse_perm;
+  return plan_dev(router_logits, given_expert_ids, given_weights, T, E, k,
+                  normalize ? kRouterSoftmaxSelected : kRouterUniform, capacity, plan, token_of_slot, expert_of_slot,
+                  combine_weights, group_sizes, group_offsets, num_slots, as_stream(stream));
+}
+
+int tessera_gfx950_moe_plan_f32(const float* router_logits, const int32_t* given_expert_ids,
+                                const float* given_weights, int T, int E, int k, int normalize, int capacity,
+                                int32_t* expert_ids, float* weights, uint8_t* kept_mask, int32_t* sort_perm,
+                                int32_t* inverse_perm, int32_t* token_of_slot, int32_t* expert_of_slot,
+                                float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
+                                int32_t* num_slots) {
+  if (T <= 0 || E <= 0 || k <= 0 || k > E || E > kMaxExperts || (long)T * k > 0x7fffffffL || !group_sizes ||
+      !group_offsets)
+    return kBadShape;
+  if (router_logits ? k > 64 : !given_expert_ids) return kBadShape;
+  const size_t S = (size_t)T * k;
+  if (!router_logits)
+    for (size_t i = 0; i < S; ++i)
+      if (given_expert_ids[i] < 0 || given_expert_ids[i] >= E) return kBadShape;     // "expert id out of range"
+  if (probe_device() != kOk) return kNoDevice;
+  DeviceScope scope;
+  float* dl = router_logits ? static_cast<float*>(scope.alloc((size_t)T * E * 4, router_logits)) : nullptr;
+  int32_t* dgi = router_logits ? nullptr : static_cast<int32_t*>(scope.alloc(S * 4, given_expert_ids));
+  // (a plan built from ids alone carries no weights: zeros, as plan_packing's placeholder)
+  float* dgw = router_logits ? nullptr : static_cast<float*>(scope.alloc(S * 4, given_weights));
+  if (dgw && !given_weights && hipMemset(dgw, 0, S * 4) != hipSuccess) return kDeviceFailed;
+  int32_t* dids = static_cast<int32_t*>(scope.alloc(S * 4));
+  float* dw = static_cast<float*>(scope.alloc(S * 4));
+  uint8_t* dkm = static_cast<uint8_t*>(scope.alloc(S));
+  int32_t* dsp = static_cast<int32_t*>(scope.alloc(S * 4));
+  int32_t* dip = static_cast<int32_t*>(scope.alloc(S * 4));
+  int32_t* dt = static_cast<int32_t*>(scope.alloc(S * 4));
+  int32_t* de = static_cast<int32_t*>(scope.alloc(S * 4));
+  float* dcw = static_cast<float*>(scope.alloc(S * 4));
+  int32_t* dg = static_cast<int32_t*>(scope.alloc((size_t)E * 4));
+  int32_t* dof = static_cast<int32_t*>(scope.alloc((size_t)(E + 1) * 4));
+  int32_t* dn = static_cast<int32_t*>(scope.alloc(4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = tessera_gfx950_moe_plan_f32_dev(dl, dgi, dgw, T, E, k, normalize, capacity, dids, dw, dkm, dsp, dip, dt,
+                                           de, dcw, dg, dof, dn, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  int32_t n = 0;
+  if (!scope.download(&n, dn, 4)) return kDeviceFailed;
+  const size_t kept = (size_t)n * 4;
+  if ((expert_ids && router_logits && !scope.download(expert_ids, dids, S * 4)) ||
+      (weights && router_logits && !scope.download(weights, dw, S * 4)) ||
+      (kept_mask && !scope.download(kept_mask, dkm, S)) || (sort_perm && !scope.download(sort_perm, dsp, kept)) ||
+      (inverse_perm && !scope.download(inverse_perm, dip, S * 4)) ||
+      (token_of_slot && !scope.download(token_of_slot, dt, kept)) ||
+      (expert_of_slot && !scope.download(expert_of_slot, de, kept)) ||
+      (combine_weights && !scope.download(combine_weights, dcw, kept)) ||
+      !scope.download(group_sizes, dg, (size_t)E * 4) || !scope.download(group_offsets, dof, (size_t)(E + 1) * 4))
+    return kDeviceFailed;
+  if (num_slots) *num_slots = n;
+  return kOk;
+}
+
+int tessera_gfx950_moe_unpack_combine_bf16_dev(const void* y_packed, const int32_t* inverse_perm,
+                                               const float* weights, float* out, int T, int k, int S, int N,
+                                               void* stream) {
+  return unpack_combine_dev<uint16_t>(y_packed, inverse_perm, weights, out, T, k, S, N, as_stream(stream));
+}
+int tessera_gfx950_moe_unpack_combine_f32_dev(const void* y_packed, const int32_t* inverse_perm,
+                                              const float* weights, float* out, int T, int k, int S, int N,
+                                              void* stream) {
+  return unpack_combine_dev<float>(y_packed, inverse_perm, weights, out, T, k, S, N, as_stream(stream));
+}
+static int unpack_combine_host(const void* y_packed, const int32_t* inverse_perm, const float* weights, float* out,
+                               int T, int k, int S, int N, int ysz) {
+  if (T <= 0 || k <= 0 || S < 0 || N <= 0 || !out || !inverse_perm || !weights || (S > 0 && !y_packed))
+    return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  DeviceScope scope;
+  void* dy = scope.alloc((size_t)S * N * ysz, y_packed);
+  int32_t* dip = static_cast<int32_t*>(scope.alloc((size_t)T * k * 4, inverse_perm));
+  float* dw = static_cast<float*>(scope.alloc((size_t)T * k * 4, weights));
+  float* dout = static_cast<float*>(scope.alloc((size_t)T * N * 4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = ysz == 2 ? unpack_combine_dev<uint16_t>(dy, dip, dw, dout, T, k, S, N, nullptr)
+                    : unpack_combine_dev<float>(dy, dip, dw, dout, T, k, S, N, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  return scope.download(out, dout, (size_t)T * N * 4) ? kOk : kDeviceFailed;
+}
+int tessera_gfx950_moe_unpack_combine_bf16(const void* y_packed, const int32_t* inverse_perm, const float* weights,
+                                           float* out, int T, int k, int S, int N) {
+  return unpack_combine_host(y_packed, inverse_perm, weights, out, T, k, S, N, 2);
+}
+int tessera_gfx950_moe_unpack_combine_f32(const void* y_packed, const int32_t* inverse_perm, const float* weights,
+                                          float* out, int T, int k, int S, int N) {
+  return unpack_combine_host(y_packed, inverse_perm, weights, out, T, k, S, N, 4);
 }
 
 int tessera_gfx950_moe_dispatch_dev(const void* x, const int32_t* token_of_slot, void* x_perm, int T, int S, int H,
@@ -773,44 +1143,37 @@ int tessera_gfx950_moe_layer_bf16(const void* x, const float* router_logits, con
                                   const void* wd, float* out, int T, int H, int F, int N, int E, int k,
                                   int normalize, int capacity, int32_t* token_of_slot, int32_t* expert_of_slot,
                                   float* combine_weights, int32_t* group_sizes, int32_t* group_offsets) {
-  if (T <= 0 || H <= 0 || F <= 0 || N <= 0 || E <= 0 || k <= 0 || k > E || E > kMaxExperts || !x ||
-      !router_logits || !wg || !wu || !wd || !out)
-    return kBadShape;
-  if ((long)T * k > 0x7fffffffL) return kBadShape;
-  if (probe_device() != kOk) return kNoDevice;
-  const size_t S = (size_t)T * k;
-  DeviceScope scope;
-  void* dx = scope.alloc((size_t)T * H * 2, x);
-  float* dl = static_cast<float*>(scope.alloc((size_t)T * E * 4, router_logits));
-  void* dg = scope.alloc((size_t)E * H * F * 2, wg);
-  void* du = scope.alloc((size_t)E * H * F * 2, wu);
-  void* dd = scope.alloc((size_t)E * F * N * 2, wd);
-  int32_t* dt = static_cast<int32_t*>(scope.alloc(S * 4));
-  int32_t* de = static_cast<int32_t*>(scope.alloc(S * 4));
-  float* dw = static_cast<float*>(scope.alloc(S * 4));
-  int32_t* dgs = static_cast<int32_t*>(scope.alloc((size_t)E * 4));
-  int32_t* dof = static_cast<int32_t*>(scope.alloc((size_t)(E + 1) * 4));
-  int32_t* dn = static_cast<int32_t*>(scope.alloc(4));
-  void* dh = scope.alloc(S * F * 2);
-  void* dy = scope.alloc(S * N * 2);
-  float* dout = static_cast<float*>(scope.alloc((size_t)T * N * 4));
-  if (scope.failed()) return kDeviceFailed;
-  int rc = route_dev(dl, T, E, k, normalize, capacity, dt, de, dw, dgs, dof, dn, nullptr);
-  if (rc != kOk) return rc;
-  int32_t n = 0;                       // kept slots (capacity may drop some)
-  if (hipDeviceSynchronize() != hipSuccess || !scope.download(&n, dn, 4)) return kDeviceFailed;
-  // the dispatch x[token_of_slot] is the first GEMM's operand load
-  rc = swiglu_dev(dx, dg, du, dd, dof, dy, dh, n, H, F, N, E, nullptr, dt, T);
-  if (rc == kOk) rc = combine_dev<uint16_t>(dy, dt, dw, dout, T, n, N, nullptr);
-  if (rc != kOk) return rc;
-  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
-  if (!scope.download(out, dout, (size_t)T * N * 4)) return kDeviceFailed;
-  if (token_of_slot && !scope.download(token_of_slot, dt, (size_t)n * 4)) return kDeviceFailed;
-  if (expert_of_slot && !scope.download(expert_of_slot, de, (size_t)n * 4)) return kDeviceFailed;
-  if (combine_weights && !scope.download(combine_weights, dw, (size_t)n * 4)) return kDeviceFailed;
-  if (group_sizes && !scope.download(group_sizes, dgs, (size_t)E * 4)) return kDeviceFailed;
-  if (group_offsets && !scope.download(group_offsets, dof, (size_t)(E + 1) * 4)) return kDeviceFailed;
+  if (!router_logits) return kBadShape;
+  return moe_layer_host(x, nullptr, router_logits, wg, wu, wd, out, T, H, F, N, E, k, normalize, capacity,
+                        token_of_slot, expert_of_slot, combine_weights, group_sizes, group_offsets, nullptr);
+}
+
+int tessera_gfx950_moe_layer_router_bf16(const void* x, const void* w_router, const void* wg, const void* wu,
+                                         const void* wd, float* out, int T, int H, int F, int N, int E, int k,
+                                         int normalize, int capacity, int32_t* token_of_slot,
+                                         int32_t* expert_of_slot, float* combine_weights, int32_t* group_sizes,
+                                         int32_t* group_offsets, float* router_logits_out) {
+  if (!w_router) return kBadShape;
+  return moe_layer_host(x, w_router, nullptr, wg, wu, wd, out, T, H, F, N, E, k, normalize, capacity,
+                        token_of_slot, expert_of_slot, combine_weights, group_sizes, group_offsets,
+                        router_logits_out);
+}
+
+int tessera_gfx950_moe_layer_workspace_bytes(int T, int H, int F, int N, int E, int k, size_t* bytes) {
+  if (bad_layer(T, H, F, N, E, k) || !bytes) return kBadShape;
+  *bytes = layer_scratch(T, F, N, E, k).total;
   return kOk;
+}
+
+int tessera_gfx950_moe_layer_bf16_dev(const void* x, const void* w_router, const float* router_logits,
+                                      const void* wg, const void* wu, const void* wd, float* out,
+                                      void* workspace, size_t workspace_bytes, int T, int H, int F, int N, int E,
+                                      int k, int normalize, int capacity, int32_t* token_of_slot,
+                                      int32_t* expert_of_slot, float* combine_weights, int32_t* group_sizes,
+                                      int32_t* group_offsets, int32_t* num_slots, void* stream) {
+  return moe_layer_dev(x, w_router, router_logits, wg, wu, wd, out, workspace, workspace_bytes, T, H, F, N, E, k,
+                       normalize, capacity, token_of_slot, expert_of_slot, combine_weights, group_sizes,
+                       group_offsets, num_slots, as_stream(stream));
 }
 
 }  // extern "C"

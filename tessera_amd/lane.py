@@ -107,6 +107,7 @@ _SIGNATURES = {
     "tessera_gfx950_gemm_bf16_bench": [_c_int, _c_int, _c_int, _c_int, _P(ctypes.c_double)],
     "tessera_gfx950_gemm_bf16_bench_rotating": [_c_int, _c_int, _c_int, _c_int, _c_int, _P(ctypes.c_double)],
     "tessera_gfx950_bench_last_timer_source": [],
+    "tessera_gfx950_mfma_probe_bf16_dev": [_c_vp, _c_int, _c_vp, _P(ctypes.c_double), _c_vp],
     "tessera_gfx950_quantize_e4m3_f32": [_c_vp, _c_i64, _c_f, _c_vp, _P(_c_f)],
     "tessera_gfx950_quantize_i8_f32": [_c_vp, _c_int, _c_int, _c_int, _c_vp, _c_vp],
     "tessera_gfx950_quantize_e4m3_f32_dev": [_c_vp, _c_i64, _c_f, _c_vp, _c_vp, _c_vp],
@@ -132,6 +133,12 @@ _SIGNATURES = {
     "tessera_gfx950_moe_route_f32": [_c_vp] + [_c_int] * 5 + [_c_vp] * 6,
     "tessera_gfx950_moe_route_f32_dev": [_c_vp] + [_c_int] * 5 + [_c_vp] * 6 + [_c_vp],
     "tessera_gfx950_moe_route_f32_noalloc_dev": [_c_vp] + [_c_int] * 5 + [_c_vp] * 6 + [_c_vp],
+    "tessera_gfx950_moe_plan_f32": [_c_vp] * 3 + [_c_int] * 5 + [_c_vp] * 11,
+    "tessera_gfx950_moe_plan_f32_dev": [_c_vp] * 3 + [_c_int] * 5 + [_c_vp] * 11 + [_c_vp],
+    "tessera_gfx950_moe_unpack_combine_bf16": [_c_vp] * 4 + [_c_int] * 4,
+    "tessera_gfx950_moe_unpack_combine_f32": [_c_vp] * 4 + [_c_int] * 4,
+    "tessera_gfx950_moe_unpack_combine_bf16_dev": [_c_vp] * 4 + [_c_int] * 4 + [_c_vp],
+    "tessera_gfx950_moe_unpack_combine_f32_dev": [_c_vp] * 4 + [_c_int] * 4 + [_c_vp],
     "tessera_gfx950_moe_dispatch": [_c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int],
     "tessera_gfx950_moe_dispatch_dev": [_c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_moe_combine_bf16": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int],
@@ -146,6 +153,9 @@ _SIGNATURES = {
     "tessera_gfx950_moe_swiglu_block_bf16_dev": [_c_vp] * 7 + [_c_int] * 5 + [_c_vp],
     "tessera_gfx950_moe_swiglu_block_gather_bf16_dev": [_c_vp] * 8 + [_c_int] * 6 + [_c_vp],
     "tessera_gfx950_moe_layer_bf16": [_c_vp] * 6 + [_c_int] * 8 + [_c_vp] * 5,
+    "tessera_gfx950_moe_layer_router_bf16": [_c_vp] * 6 + [_c_int] * 8 + [_c_vp] * 6,
+    "tessera_gfx950_moe_layer_workspace_bytes": [_c_int] * 6 + [_P(_c_sz)],
+    "tessera_gfx950_moe_layer_bf16_dev": [_c_vp] * 8 + [_c_sz] + [_c_int] * 8 + [_c_vp] * 6 + [_c_vp],
 }
 
 

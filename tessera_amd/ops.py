@@ -515,6 +515,143 @@ def route_tokens(scores, num_experts: int, top_k: int, *, normalize_weights: boo
     return MoETransport(T, top_k, E, cap or None, tos[:k].copy(), eos[:k].copy(), cw[:k].copy(), gs, go)
 
 
+@dataclass
+class DispatchPlan:
+    """The reference's packing plan in its token-major view
+    (``stdlib/moe.py:58-77`` ``DispatchPlan``; ``models/moe_routing.py:33-51``
+    ``RoutingPlan`` is the no-capacity case): which routed slots survive and the
+    contiguous per-expert order of the survivors."""
+    expert_ids: np.ndarray       # (T, k) int64 selected experts
+    weights: np.ndarray          # (T, k) f32 route weights
+    kept_mask: np.ndarray        # (T, k) bool, False = dropped over capacity
+    sort_perm: np.ndarray        # (S,) int64 kept token-major slot ids, expert-sorted
+    inverse_perm: np.ndarray     # (T*k,) int64 packed position of each slot, -1 = dropped
+    group_sizes: np.ndarray      # (E,) int64 kept slots per expert
+    num_tokens: int
+    top_k: int
+    capacity: Optional[int]
+    transport: MoETransport      # the same plan as the int32 transport descriptor
+
+    @property
+    def num_kept(self) -> int:
+        return int(self.sort_perm.shape[0])
+
+    @property
+    def drop_fraction(self) -> float:
+        total = self.num_tokens * self.top_k
+        return 0.0 if total == 0 else 1.0 - self.num_kept / total
+
+    def round_trips(self) -> bool:
+        """True iff nothing was dropped and ``sort_perm[inverse_perm]`` is the identity."""
+        n = self.num_tokens * self.top_k
+        return self.num_kept == n and bool(np.array_equal(self.sort_perm[self.inverse_perm], np.arange(n)))
+
+
+def _plan_call(logits, given_ids, given_weights, T: int, E: int, k: int, normalize: bool,
+               capacity: Optional[int]) -> DispatchPlan:
+    S = T * k
+    cap = 0 if capacity is None else int(capacity)
+    ids = np.empty((T, k), np.int32)
+    w = np.empty((T, k), np.float32)
+    kept = np.empty((T, k), np.uint8)
+    sp = np.empty(S, np.int32)
+    ip = np.empty(S, np.int32)
+    tos = np.empty(S, np.int32)
+    eos = np.empty(S, np.int32)
+    cw = np.empty(S, np.float32)
+    gs = np.empty(E, np.int32)
+    go = np.empty(E + 1, np.int32)
+    n = np.zeros(1, np.int32)
+    rc = _lane.load().tessera_gfx950_moe_plan_f32(
+        _lane.ptr(logits), _lane.ptr(given_ids), _lane.ptr(given_weights), T, E, k, 1 if normalize else 0, cap,
+        ids.ctypes.data, w.ctypes.data, kept.ctypes.data, sp.ctypes.data, ip.ctypes.data, tos.ctypes.data,
+        eos.ctypes.data, cw.ctypes.data, gs.ctypes.data, go.ctypes.data, n.ctypes.data)
+    _lane.check(rc, "moe plan")
+    m = int(n[0])
+    if logits is None:
+        ids = np.asarray(given_ids, np.int32).reshape(T, k)
+        w = (np.zeros((T, k), np.float32) if given_weights is None
+             else np.asarray(given_weights, np.float32).reshape(T, k))
+    transport = MoETransport(T, k, E, capacity, tos[:m].copy(), eos[:m].copy(), cw[:m].copy(), gs, go)
+    return DispatchPlan(ids.astype(np.int64), w, kept.astype(bool), sp[:m].astype(np.int64), ip.astype(np.int64),
+                        gs.astype(np.int64), T, k, capacity, transport)
+
+
+def route_top_k(router_logits, top_k: int, *, normalize: bool = True):
+    """Exact top-k routing on the LOGITS → ``(expert_ids (T,k) int64, weights (T,k) f32)``:
+    descending by logit, ties to the lowest expert id; ``normalize`` makes the weights a
+    softmax over the selected logits, else each is ``1/k`` (``models/moe_routing.py:54-77``)."""
+    lg = np.ascontiguousarray(_unbox(router_logits), np.float32)
+    if lg.ndim != 2:
+        raise ValueError("router_logits must be (T, num_experts)")
+    T, E = lg.shape
+    if not (1 <= top_k <= E):
+        raise ValueError(f"top_k={top_k} out of [1, num_experts={E}]")
+    plan = _plan_call(lg, None, None, T, E, int(top_k), normalize, None)
+    return plan.expert_ids, plan.weights
+
+
+def _check_ids(expert_ids, num_experts: int) -> np.ndarray:
+    ids = np.asarray(_unbox(expert_ids))
+    if ids.ndim != 2:
+        raise ValueError("expert_ids must be (T, k)")
+    if ids.size and (ids.min() < 0 or ids.max() >= num_experts):
+        raise ValueError("expert id out of range")
+    return np.ascontiguousarray(ids, np.int32)
+
+
+def plan_packing(expert_ids, num_experts: int) -> DispatchPlan:
+    """The per-expert packing plan of a routing, nothing dropped
+    (``models/moe_routing.py:80-99``); ``weights`` is the reference's zero placeholder."""
+    ids = _check_ids(expert_ids, num_experts)
+    T, k = ids.shape
+    return _plan_call(None, ids, None, T, num_experts, k, True, None)
+
+
+def plan_dispatch(expert_ids, weights, num_experts: int, *, capacity: Optional[int] = None) -> DispatchPlan:
+    """Capacity-aware plan from routing decisions: slots in token-major order, an expert
+    keeps its first ``capacity`` (``None``: all), kept slots stable-sorted by expert
+    (``stdlib/moe.py:79-115``)."""
+    ids = _check_ids(expert_ids, num_experts)
+    w = np.ascontiguousarray(_unbox(weights), np.float32)
+    if w.shape != ids.shape:
+        raise ValueError("weights must match expert_ids")
+    T, k = ids.shape
+    if capacity is not None and capacity < 1:
+        raise ValueError("capacity must be >= 1 (or None)")
+    return _plan_call(None, ids, w, T, num_experts, k, True, capacity)
+
+
+def pack_tokens(x, plan: DispatchPlan):
+    """Gather ``x`` (T, H) into packed per-expert slot order → ``(S, H)``
+    (``models/moe_routing.py:102-106``, ``stdlib/moe.py:117-121``)."""
+    return moe_dispatch(x, plan.transport)
+
+
+def unpack_combine(y_packed, plan: DispatchPlan, weights) -> np.ndarray:
+    """Scatter packed expert rows back to token order and sum each token's k slots in
+    rank order with their route weights → ``(T, H)`` f32; dropped slots add nothing
+    (``models/moe_routing.py:109-116``)."""
+    y = _unbox(y_packed)
+    w = np.ascontiguousarray(_unbox(weights), np.float32)
+    T, k = plan.num_tokens, plan.top_k
+    if w.shape != (T, k):
+        raise ValueError(f"weights must be (T, k)=({T}, {k}); got {w.shape}")
+    lib = _lane.load()
+    if _bf16.is_bf16(y):
+        ya, fn = _bf16.as_bits(y), lib.tessera_gfx950_moe_unpack_combine_bf16
+    else:
+        ya, fn = np.ascontiguousarray(y, np.float32), lib.tessera_gfx950_moe_unpack_combine_f32
+    S = plan.num_kept
+    if ya.ndim != 2 or ya.shape[0] != S:
+        raise ValueError(f"packed rows must be (S, H) with S={S}; got {ya.shape}")
+    ip = np.ascontiguousarray(plan.inverse_perm, np.int32)
+    out = np.empty((T, ya.shape[1]), np.float32)
+    _lane.check(fn(ya.ctypes.data, ip.ctypes.data, w.ctypes.data, out.ctypes.data, T, k, S, ya.shape[1]),
+                "unpack_combine")
+    return out
+
+
 def moe_dispatch(x, plan: MoETransport):
     """Gather the token row of every kept, expert-sorted slot → ``(S, H)``."""
     x = _unbox(x)
@@ -586,14 +723,7 @@ def moe_layer(x, W_router, W_gate, W_up, W_down, *, top_k: int = 1, normalize_we
     if top_k < 1 or top_k > E:
         raise ValueError(f"top_k must be in [1, num_experts={E}], got {top_k}")
     N = wd.shape[2]
-    if router_logits is None:
-        scores = gemm(x, W_router)                       # storage-rounded, as ops.gemm
-        logits = scores.to_float32() if isinstance(scores, BF16Array) else np.asarray(scores, np.float32)
-    else:
-        logits = np.ascontiguousarray(router_logits, np.float32)
-    if logits.shape != (T, E):
-        raise ValueError(f"router logits must be (T, E)=({T}, {E}); got {logits.shape}")
-    logits = np.ascontiguousarray(logits, np.float32)
+    lib = _lane.load()
     cap = 0
     if capacity_factor > 0:
         cap = _capacity_arg(int(math.ceil(capacity_factor * T / E)), T, top_k)
@@ -604,10 +734,27 @@ def moe_layer(x, W_router, W_gate, W_up, W_down, *, top_k: int = 1, normalize_we
     cw = np.empty(S, np.float32)
     gs = np.empty(E, np.int32)
     go = np.empty(E + 1, np.int32)
-    rc = _lane.load().tessera_gfx950_moe_layer_bf16(
-        xa.ctypes.data, logits.ctypes.data, wg.ctypes.data, wu.ctypes.data, wd.ctypes.data, outp.ctypes.data,
-        T, H, F, N, E, top_k, 1 if normalize_weights else 0, cap,
-        tos.ctypes.data, eos.ctypes.data, cw.ctypes.data, gs.ctypes.data, go.ctypes.data)
+    tail = (T, H, F, N, E, top_k, 1 if normalize_weights else 0, cap,
+            tos.ctypes.data, eos.ctypes.data, cw.ctypes.data, gs.ctypes.data, go.ctypes.data)
+    if router_logits is None:
+        # scores = ops.gemm(x, W_router) on the device, stored in bf16 and read as f32 like every
+        # reduced-precision product; the routing follows on the same stream without a host hop
+        W_router = _unbox(W_router)
+        if _storage(W_router) != "bf16":
+            raise ValueError("moe_layer on the gfx950 lane takes a bf16 W_router")
+        wr = _bits(W_router)
+        if wr.shape != (H, E):
+            raise ValueError(f"W_router must be (K, E)=({H}, {E}); got {wr.shape}")
+        rc = lib.tessera_gfx950_moe_layer_router_bf16(
+            xa.ctypes.data, wr.ctypes.data, wg.ctypes.data, wu.ctypes.data, wd.ctypes.data, outp.ctypes.data,
+            *tail, None)
+    else:
+        logits = np.ascontiguousarray(router_logits, np.float32)
+        if logits.shape != (T, E):
+            raise ValueError(f"router logits must be (T, E)=({T}, {E}); got {logits.shape}")
+        rc = lib.tessera_gfx950_moe_layer_bf16(
+            xa.ctypes.data, logits.ctypes.data, wg.ctypes.data, wu.ctypes.data, wd.ctypes.data, outp.ctypes.data,
+            *tail)
     _lane.check(rc, "moe_layer")
     if not return_plan:
         return outp

@@ -5,6 +5,7 @@ the same 16-bit operands (f32 accumulate, f32 output)."""
 import numpy as np
 import pytest
 
+import standin_host as host
 import tessera_oracle as orc
 from tessera_amd import bf16 as b16
 from tessera_amd import candidates as cand
@@ -93,23 +94,24 @@ def test_gated_gemm_equals_two_products(lane):
 
 
 def test_fused_and_gated_candidates_pass_the_gate(lane):
-    cand.register_all()
+    api = host.CandidateHost()
+    cand.register(api)
     for epi in [("bias", "relu"), ("gelu",), ("bias",), ("bias", "silu")]:
-        region = cand.FusedRegion(epilogue=epi, storage_dtype="bf16")
-        winner = cand.arbitrate(region, cand.OP_FUSED_REGION, cand.TARGET)
+        region = host.FusedRegion(epilogue=epi, storage_dtype="bf16")
+        winner = api.arbitrate(region, api.OP_FUSED_REGION, cand.TARGET)
         assert winner is not None and winner.name == "gfx950_mfma_fused_gemm"
     # not representable: activation before bias, residual
-    assert cand.arbitrate(cand.FusedRegion(epilogue=("relu", "bias")), cand.OP_FUSED_REGION, cand.TARGET) is None
-    assert cand.arbitrate(cand.FusedRegion(epilogue=("relu",), residual=True), cand.OP_FUSED_REGION,
-                          cand.TARGET) is None
-    g = cand.GatedMatmulRegion("silu", "f16")
-    winner = cand.arbitrate(g, cand.OP_GATED_MATMUL, cand.TARGET)
+    assert api.arbitrate(host.FusedRegion(epilogue=("relu", "bias")), api.OP_FUSED_REGION, cand.TARGET) is None
+    assert api.arbitrate(host.FusedRegion(epilogue=("relu",), residual=True), api.OP_FUSED_REGION,
+                         cand.TARGET) is None
+    g = host.GatedMatmulRegion("silu", "f16")
+    winner = api.arbitrate(g, api.OP_GATED_MATMUL, cand.TARGET)
     assert winner is not None and winner.name == "gfx950_mfma_gated_gemm"
     rng = np.random.default_rng(0)
     A = (rng.standard_normal((64, 32)) * .3).astype(np.float32)
     Wg = (rng.standard_normal((32, 48)) * .3).astype(np.float32)
     Wu = (rng.standard_normal((32, 48)) * .3).astype(np.float32)
-    out, tag = cand.run_arbitrated(g, cand.OP_GATED_MATMUL, cand.TARGET, A, Wg, Wu)
+    out, tag = api.run(g, api.OP_GATED_MATMUL, cand.TARGET, A, Wg, Wu)
     assert tag == cand.GATED_TAG
     assert np.allclose(out, g.reference(A, Wg, Wu), atol=5e-3)
 

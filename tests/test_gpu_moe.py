@@ -91,6 +91,62 @@ def test_routing_non_finite_rows_stay_in_range(lane):
     assert int(np.isnan(plan.combine_weights).sum()) == 4 * k
 
 
+@pytest.mark.parametrize("T,E,k", [(257, 64, 8), (1000, 40, 6), (64, 8, 1), (33, 5, 5)])
+@pytest.mark.parametrize("normalize", [True, False])
+def test_route_top_k_and_packing_plan(lane, T, E, k, normalize):
+    """The reference's second router (top-k of the logits, softmax over the selected
+    ones or 1/k) and its packing plan: expert ids, sort_perm, inverse_perm, kept_mask and
+    group sizes bit for bit against the oracle, weights to f32 rounding."""
+    lg = np.random.default_rng(900 + T).standard_normal((T, E)).astype(np.float32)
+    lg[T // 2, 1] = lg[T // 2, 3] = 9.0                   # a tie at the top: lower id first
+    lg[T // 3, :] = -0.5                                   # a row of ties takes experts 0..k-1
+    ids, w = ops.route_top_k(lg, k, normalize=normalize)
+    rids, rw = orc.route_top_k_stable(lg, k, normalize=normalize)
+    assert ids.dtype == np.int64 and np.array_equal(ids, rids)
+    np.testing.assert_allclose(w, rw, rtol=3e-6, atol=1e-9)
+    if k >= 2:
+        assert list(ids[T // 2][:2]) == [1, 3]
+    assert list(ids[T // 3]) == list(range(k))
+    for cap in (None, max(1, (T * k) // (2 * E))):
+        plan = ops.plan_dispatch(ids, w, E, capacity=cap)
+        want = orc.plan_dispatch_token_major(rids, w, E, capacity=cap)
+        assert np.array_equal(plan.kept_mask, want.kept_mask)
+        assert np.array_equal(plan.sort_perm, want.sort_perm)
+        assert np.array_equal(plan.inverse_perm, want.inverse_perm)
+        assert np.array_equal(plan.group_sizes, want.group_sizes)
+        assert np.array_equal(plan.transport.token_of_slot, want.sort_perm // k)
+        assert np.array_equal(plan.transport.combine_weights, w.reshape(-1)[want.sort_perm])
+        assert (cap is None) == plan.round_trips()
+        if cap is not None:
+            assert plan.num_kept < T * k and plan.drop_fraction > 0
+    pk = ops.plan_packing(ids, E)
+    assert pk.round_trips() and np.array_equal(pk.sort_perm, orc.plan_dispatch_token_major(rids, w, E).sort_perm)
+    with pytest.raises(ValueError):
+        ops.plan_packing(np.full((4, 2), E), E)
+
+
+def test_pack_and_unpack_combine(lane):
+    """pack_tokens / unpack_combine (models/moe_routing.py:102-116): the packed rows are
+    an exact gather, and the token-major k-sum equals the oracle's bit for bit in f32."""
+    T, E, k, H = 300, 16, 4, 72
+    rng = np.random.default_rng(77)
+    lg = rng.standard_normal((T, E)).astype(np.float32)
+    ids, w = ops.route_top_k(lg, k)
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    for cap in (None, 50):
+        plan = ops.plan_dispatch(ids, w, E, capacity=cap)
+        packed = ops.pack_tokens(x, plan)
+        assert np.array_equal(packed, x[plan.sort_perm // k])
+        y = rng.standard_normal(packed.shape).astype(np.float32)
+        got = ops.unpack_combine(y, plan, w)
+        assert np.array_equal(got, orc.unpack_combine(y, plan.inverse_perm, w))
+        yb = b16.from_float32(y)
+        assert np.array_equal(ops.unpack_combine(yb, plan, w), orc.unpack_combine(yb.to_float32(), plan.inverse_perm, w))
+    H2 = 37                                                # rows that are not 16-byte multiples
+    y2 = rng.standard_normal((plan.num_kept, H2)).astype(np.float32)
+    assert np.array_equal(ops.unpack_combine(y2, plan, w), orc.unpack_combine(y2, plan.inverse_perm, w))
+
+
 def test_dispatch_and_combine(lane):
     T, H, E, k = 300, 96, 8, 2
     lg = _logits(T, E, 1, k)
@@ -287,6 +343,60 @@ def test_moe_layer_with_router_gemm(lane):
     out, plan = ops.moe_layer(xb, rb, *(b16.from_float32(a) for a in (wg, wu, wd)), top_k=k, return_plan=True)
     _check_plan(plan, desc)
     assert orc.max_rel_err(out, ref) <= TOL + 2.0 ** -8
+
+
+@pytest.mark.parametrize("cf,use_router", [(0.0, True), (0.75, False), (0.0, False)])
+def test_moe_layer_device_resident_entry(lane, cf, use_router):
+    """tessera_gfx950_moe_layer_bf16_dev through the C ABI: router product, routing,
+    expert block and combine on one stream with every operand resident; a capacity
+    leaves the number of kept slots on the device.  Checked against the oracle and,
+    bit for bit, against the host-pointer layer (the same kernels)."""
+    import ctypes
+    T, H, F, N, E, k = 320, 128, 192, 96, 8, 2
+    for seed in range(900, 1300):
+        rng = np.random.default_rng(seed)
+        x = rng.standard_normal((T, H)).astype(np.float32)
+        wr = rng.standard_normal((H, E)).astype(np.float32)
+        lg = orc.gemm_storage(x, wr, "bf16") if use_router else rng.standard_normal((T, E)).astype(np.float32)
+        if not orc.has_routing_ties(orc.router_probs(lg), k):
+            break
+    else:
+        pytest.fail("no tie-free seed found")
+    wg, wu = ((rng.standard_normal((E, H, F)) * 0.1).astype(np.float32) for _ in range(2))
+    wd = (rng.standard_normal((E, F, N)) * 0.1).astype(np.float32)
+    lib = lane.load()
+    bits = lambda a: np.ascontiguousarray(np.asarray(b16.from_float32(a), np.uint16))
+    dx, dr, dg, du, dd = (lane.DeviceBuffer.from_host(bits(a)) for a in (x, wr, wg, wu, wd))
+    dl = lane.DeviceBuffer.from_host(np.ascontiguousarray(lg, np.float32))
+    S = T * k
+    need = ctypes.c_size_t(0)
+    assert lib.tessera_gfx950_moe_layer_workspace_bytes(T, H, F, N, E, k, ctypes.byref(need)) == 0
+    dws = lane.DeviceBuffer(need.value)
+    dout = lane.DeviceBuffer(T * N * 4)
+    dtos, deos, dcw = (lane.DeviceBuffer(S * 4) for _ in range(3))
+    dgs, dgo, dn = lane.DeviceBuffer(E * 4), lane.DeviceBuffer((E + 1) * 4), lane.DeviceBuffer(4)
+    cap = int(np.ceil(cf * T / E)) if cf > 0 else 0
+    rc = lib.tessera_gfx950_moe_layer_bf16_dev(
+        dx.ptr, dr.ptr if use_router else None, None if use_router else dl.ptr, dg.ptr, du.ptr, dd.ptr, dout.ptr,
+        dws.ptr, need.value, T, H, F, N, E, k, 1, cap, dtos.ptr, deos.ptr, dcw.ptr, dgs.ptr, dgo.ptr, dn.ptr, None)
+    lane.check(rc, "moe_layer_dev")
+    lane.synchronize()
+    n = int(dn.download((1,), np.int32)[0])
+    got = dout.download((T, N), np.float32)
+    ref, desc = orc.moe_layer(x, lg, wg, wu, wd, k, capacity_factor=cf)
+    assert n == desc.token_of_slot.size and (cf == 0.0) == (n == S)
+    assert np.array_equal(dtos.download((S,), np.int32)[:n], desc.token_of_slot)
+    assert np.array_equal(deos.download((S,), np.int32)[:n], desc.expert_of_slot)
+    assert np.array_equal(dgo.download((E + 1,), np.int32), desc.group_offsets)
+    assert orc.max_rel_err(got, ref) <= TOL + 2.0 ** -8
+    host = ops.moe_layer(b16.from_float32(x), b16.from_float32(wr) if use_router else None,
+                         *(b16.from_float32(a) for a in (wg, wu, wd)), top_k=k, capacity_factor=cf,
+                         router_logits=None if use_router else lg)
+    assert np.array_equal(got.view(np.uint32), np.asarray(host, np.float32).view(np.uint32))
+    # a workspace that is too small is refused before anything is launched
+    assert lib.tessera_gfx950_moe_layer_bf16_dev(
+        dx.ptr, None, dl.ptr, dg.ptr, du.ptr, dd.ptr, dout.ptr, dws.ptr, need.value - 256, T, H, F, N, E, k, 1, 0,
+        dtos.ptr, deos.ptr, dcw.ptr, dgs.ptr, dgo.ptr, dn.ptr, None) == lane.BAD_SHAPE
 
 
 def test_moe_headline_config(lane):

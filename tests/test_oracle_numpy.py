@@ -327,3 +327,74 @@ def test_route_tokens_non_finite_rows_keep_indices_in_range():
     with np.errstate(invalid="ignore"):
         d = orc.plan_dispatch(r.assignment, r.weights, 8)
     assert d.group_offsets[-1] == 18 and np.array_equal(np.sort(d.token_of_slot), np.repeat(np.arange(6), 3))
+
+
+def test_route_top_k_against_a_per_token_sort_and_library_softmax():
+    """models/moe_routing.py:54-77: top-k of the LOGITS, descending, ties to the lowest
+    id; weights = softmax over the selected logits (scipy's) or 1/k."""
+    from scipy.special import softmax
+    rng = np.random.default_rng(5)
+    lg = rng.standard_normal((40, 12)).astype(np.float32)
+    lg[3, 4] = lg[3, 9] = lg[3].max() + 1.0          # a tie at the top: lower id first
+    lg[7, :] = 0.25                                   # a whole row of ties
+    ids, w = orc.route_top_k_stable(lg, 3)
+    for t in range(40):
+        want = sorted(range(12), key=lambda e: (-float(lg[t, e]), e))[:3]
+        assert list(ids[t]) == want
+        np.testing.assert_allclose(w[t], softmax(lg[t, want].astype(np.float64)), rtol=1e-6)
+    assert list(ids[3][:2]) == [4, 9] and list(ids[7]) == [0, 1, 2]
+    _, wu = orc.route_top_k_stable(lg, 4, normalize=False)
+    assert np.all(wu == np.float32(0.25))
+
+
+def test_packing_plan_against_an_independent_walk():
+    """stdlib/moe.py:79-115 and models/moe_routing.py:80-99, checked by walking each
+    expert's slots separately (not the oracle's own argsort)."""
+    rng = np.random.default_rng(6)
+    T, k, E, cap = 50, 3, 7, 15
+    ids = np.stack([rng.permutation(E)[:k] for _ in range(T)])
+    w = rng.random((T, k)).astype(np.float32)
+    plan = orc.plan_dispatch_token_major(ids, w, E, capacity=cap)
+    flat = ids.reshape(-1)
+    pos = 0
+    for e in range(E):
+        slots = [s for s in range(T * k) if flat[s] == e]           # token-major order
+        keep, drop = slots[:cap], slots[cap:]
+        assert plan.group_sizes[e] == len(keep)
+        assert list(plan.sort_perm[pos:pos + len(keep)]) == keep
+        assert all(plan.inverse_perm[s] == pos + i for i, s in enumerate(keep))
+        assert all(plan.inverse_perm[s] == -1 and not plan.kept_mask.reshape(-1)[s] for s in drop)
+        pos += len(keep)
+    assert pos == plan.sort_perm.size == int(plan.kept_mask.sum()) < T * k
+    full = orc.plan_dispatch_token_major(ids, w, E)
+    assert np.array_equal(full.sort_perm[full.inverse_perm], np.arange(T * k)) and full.kept_mask.all()
+    # the transport descriptor of route_tokens' plan is the same permutation
+    d = orc.plan_dispatch(np.where(plan.kept_mask, ids, -1), w, E)
+    assert np.array_equal(d.sort_perm, plan.sort_perm) and np.array_equal(d.token_of_slot, plan.sort_perm // k)
+    with pytest.raises(ValueError):
+        orc.plan_dispatch_token_major(np.array([[0, 7]]), np.ones((1, 2)), 7)
+
+
+def test_unpack_combine_closed_forms():
+    """models/moe_routing.py:109-116.  k = 1 with weight 1 undoes the packing; equal
+    weights 1/k over identical rows give the row back; dropped slots add nothing."""
+    rng = np.random.default_rng(8)
+    T, k, E, H = 30, 2, 5, 6
+    ids = np.stack([rng.permutation(E)[:k] for _ in range(T)])
+    plan = orc.plan_dispatch_token_major(ids, np.ones((T, k)), E)
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    packed = x[plan.sort_perm // k]                                  # every slot carries its token's row
+    half = np.full((T, k), 0.5, np.float32)
+    assert np.array_equal(orc.unpack_combine(packed, plan.inverse_perm, half), x)
+    one = orc.plan_dispatch_token_major(ids[:, :1], np.ones((T, 1)), E)
+    assert np.array_equal(orc.unpack_combine(x[one.sort_perm], one.inverse_perm, np.ones((T, 1), np.float32)), x)
+    capped = orc.plan_dispatch_token_major(ids, np.ones((T, k)), E, capacity=4)
+    got = orc.unpack_combine(x[capped.sort_perm // k], capped.inverse_perm, np.ones((T, k), np.float32))
+    assert np.array_equal(got, x * capped.kept_mask.sum(axis=1, keepdims=True).astype(np.float32))
+    # against the reference's own slot-order combine (stdlib/moe.py:124-134) on a random case
+    y = rng.standard_normal((capped.sort_perm.size, H)).astype(np.float32)
+    wts = rng.random((T, k)).astype(np.float32)
+    ref = np.zeros((T, H), np.float64)
+    for i, slot in enumerate(capped.sort_perm):
+        ref[slot // k] += float(wts.reshape(-1)[slot]) * y[i]
+    np.testing.assert_allclose(orc.unpack_combine(y, capped.inverse_perm, wts), ref, rtol=1e-5, atol=1e-6)
