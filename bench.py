@@ -667,6 +667,41 @@ def clock_and_power_trace(lane, seconds=4.0):
     return out
 
 
+def operand_residency_trace(lane, seconds=2.0):
+    """What the operand traffic of the headline GEMM costs at the board's power limit.
+
+    The same 256 x 256 tile kernel runs the same number of MFMAs (2 * 8192^3 FLOP per
+    launch) on problems whose operands do or do not have to come through the fabric:
+    one 8192^3 product; 64 products of 2048^3 on 64 distinct operand pairs; the same 64
+    products all reading ONE operand pair (stride 0: 16 MB, resident in the memory-side
+    cache and largely in the L2s); and likewise 512 products of 1024^3 (4 MB shared).
+    Shared against distinct operands at equal K-loop length is the cost of the traffic:
+    TFLOP/s, and the clock and power the board settles at."""
+    lib = lane.load()
+    rng = np.random.default_rng(0)
+    fn = lib.tessera_gfx950_batched_gemm_strided_bf16_dev
+    rows = []
+    for tag, batch, n, shared in (("1 x 8192^3", 1, 8192, False), ("64 x 2048^3, distinct operands", 64, 2048, False),
+                                  ("64 x 2048^3, one shared operand pair (16 MB)", 64, 2048, True),
+                                  ("512 x 1024^3, distinct operands", 512, 1024, False),
+                                  ("512 x 1024^3, one shared operand pair (4 MB)", 512, 1024, True)):
+        cnt = 1 if shared else batch
+        a = _bf16(rng.standard_normal((cnt, n, n), dtype=np.float32) / np.sqrt(n))
+        b = _bf16(rng.standard_normal((cnt, n, n), dtype=np.float32) / np.sqrt(n))
+        da, db, dd = lane.DeviceBuffer.from_host(a), lane.DeviceBuffer.from_host(b), lane.DeviceBuffer(batch * n * n * 2)
+        st = 0 if shared else n * n
+        launch = lambda: lane.check(fn(da.ptr, db.ptr, dd.ptr, batch, n, n, n, st, st, n * n, 1, None), "strided gemm")
+        _, ev = _timed(lane, launch, 20, 5)
+        held = _sustained(lane, launch, seconds)
+        flop = 2.0 * batch * n ** 3
+        rows.append({"case": tag, "ms": ev, "tflops": flop / ev / 1e9,
+                     "tflops_sustained": flop / held["ms"] / 1e9 if "ms" in held else None,
+                     "gfx_clock_mhz": held.get("gfx_clock_mhz"), "socket_power_w": held.get("socket_power_w")})
+        for buf in (da, db, dd):
+            buf.close()
+    return rows
+
+
 def cpu_baseline(A, B):
     """The reference's CPU path for this config is ``np.matmul`` on f32-promoted
     operands; the oracle restates it.  Timed once on the full workload."""
@@ -723,6 +758,8 @@ def main() -> int:
                     help="also launch a 1 GiB copy kernel (counter calibration for profiled runs)")
     ap.add_argument("--no-clock", action="store_true",
                     help="skip the clock / power readings (headline kernel and MFMA ceiling probe)")
+    ap.add_argument("--residency", action="store_true",
+                    help="instead of the bench line: the headline kernel on streamed against cache-resident operands")
     ap.add_argument("--clocks", action="store_true",
                     help="instead of the bench line: shader clock and socket power under each kernel")
     args = ap.parse_args()
@@ -738,6 +775,9 @@ def main() -> int:
     _RAMP["foreign"] = bool(args.profile)
     if args.clocks:
         print(json.dumps(clock_and_power_trace(lane), indent=1))
+        return 0
+    if args.residency:
+        print(json.dumps(operand_residency_trace(lane), indent=1))
         return 0
     if args.only:
         if args.only == "mfma_ceiling":

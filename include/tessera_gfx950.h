@@ -126,6 +126,18 @@ int tessera_gfx950_gemm_f16_f16_dev(const void* A, const void* B, void* D, int M
 int tessera_gfx950_gemm_bf16_bf16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream);
 int tessera_gfx950_batched_gemm_f16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K, void* stream);
 int tessera_gfx950_batched_gemm_bf16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K, void* stream);
+/* Strided batch: product z of `batch` reads A + z*stride_a and B + z*stride_b and writes
+ * D + z*stride_d (strides in elements).  A stride of 0 shares that operand between all
+ * products — np.matmul's broadcast of a 2-D weight over a stacked activation, which is
+ * what ops.batched_gemm is (python/tessera/__init__.py:250-254) — in one launch and
+ * without materialising the copies.  stride_d >= M*N.  out_dtype: 0 = f32 D, 1 = D in the
+ * operand storage dtype. */
+int tessera_gfx950_batched_gemm_strided_f16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K,
+                                                int64_t stride_a, int64_t stride_b, int64_t stride_d, int out_dtype,
+                                                void* stream);
+int tessera_gfx950_batched_gemm_strided_bf16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K,
+                                                 int64_t stride_a, int64_t stride_b, int64_t stride_d, int out_dtype,
+                                                 void* stream);
 int tessera_gfx950_gemm_i8_i32_dev(const void* A, const void* B, void* C, int M, int N, int K, void* stream);
 int tessera_gfx950_gemm_w8a8_f32_dev(const void* A, const void* B, const float* row_scale,
                                      const float* col_scale, void* D, void* acc_out,

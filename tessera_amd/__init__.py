@@ -6,6 +6,7 @@ Modules
 -------
 ``lane``        ctypes binding of ``lib/libtessera_gfx950.so``
 ``ops``         the ``tessera.ops`` / ``nn.functional`` surface of the path
+``resident``    the same ops on device-resident handles, for chains without host round trips
 ``executors``   the ``runtime.launch`` executor seam (execution-matrix rows)
 ``candidates``  gfx950 candidates for the host's measured arbiter (host API injected)
 ``install``     one call that registers candidates, matrix rows and executors with a host
@@ -15,4 +16,4 @@ Modules
 """
 from . import bf16, lane  # noqa: F401
 
-__all__ = ["bf16", "lane", "ops", "executors", "candidates", "install", "autotune", "tile_table", "build"]
+__all__ = ["bf16", "lane", "ops", "resident", "executors", "candidates", "install", "autotune", "tile_table", "build"]

@@ -24,6 +24,25 @@ int gemm16_dev(const void* A, const void* B, void* D, int batch, int M, int N, i
   return launch_gemm16<T, EPI>(p, s);
 }
 
+// Strided batch: product z reads A + z strideA, B + z strideB and writes D + z strideD
+// (strides in elements; 0 shares an operand between the products of the batch).
+template <class T, int EPI>
+int gemm16_strided_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K, long sA, long sB, long sD,
+                       hipStream_t s) {
+  if (bad_dims(batch, M, N, K) || !A || !B || !D || sA < 0 || sB < 0) return kBadShape;
+  if (batch > 1 && sD < (long)M * N) return kBadShape;      // outputs must not overlap
+  if (probe_device() != kOk) return kNoDevice;
+  Gemm16Params p{};
+  p.A = static_cast<const uint16_t*>(A);
+  p.B = static_cast<const uint16_t*>(B);
+  p.D = D;
+  p.M = M; p.N = N; p.K = K;
+  p.lda = K; p.ldb = N; p.ldd = N;
+  p.strideA = sA; p.strideB = sB; p.strideD = sD;
+  p.groups = batch;
+  return launch_gemm16<T, EPI>(p, s);
+}
+
 template <class T, int EPI>
 int gemm16_host(const void* A, const void* B, void* D, int batch, int M, int N, int K) {
   if (bad_dims(batch, M, N, K) || !A || !B || !D) return kBadShape;
@@ -194,6 +213,18 @@ int tessera_gfx950_gemm_f16_f16_dev(const void* A, const void* B, void* D, int M
 }
 int tessera_gfx950_gemm_bf16_bf16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream) {
   return gemm16_dev<BF16, EPI_STORE16>(A, B, D, 1, M, N, K, as_stream(stream));
+}
+int tessera_gfx950_batched_gemm_strided_f16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K,
+                                                int64_t stride_a, int64_t stride_b, int64_t stride_d, int out_dtype,
+                                                void* stream) {
+  return out_dtype ? gemm16_strided_dev<F16, EPI_STORE16>(A, B, D, batch, M, N, K, stride_a, stride_b, stride_d, as_stream(stream))
+                   : gemm16_strided_dev<F16, EPI_F32>(A, B, D, batch, M, N, K, stride_a, stride_b, stride_d, as_stream(stream));
+}
+int tessera_gfx950_batched_gemm_strided_bf16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K,
+                                                 int64_t stride_a, int64_t stride_b, int64_t stride_d, int out_dtype,
+                                                 void* stream) {
+  return out_dtype ? gemm16_strided_dev<BF16, EPI_STORE16>(A, B, D, batch, M, N, K, stride_a, stride_b, stride_d, as_stream(stream))
+                   : gemm16_strided_dev<BF16, EPI_F32>(A, B, D, batch, M, N, K, stride_a, stride_b, stride_d, as_stream(stream));
 }
 int tessera_gfx950_batched_gemm_f16_dev(const void* A, const void* B, void* D, int batch, int M, int N, int K,
                                         void* stream) {
