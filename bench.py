@@ -48,8 +48,9 @@ PEAK_HBM_GBS = 8000.0
 PEAK_CLOCK_MHZ = 2400.0         # shader clock the MFMA peaks are quoted at
 # HBM-side bytes one launch of the headline kernel moves: FETCH_SIZE + WRITE_SIZE per
 # dispatch from two counter runs of this script, each scaled by the same counter's
-# reading for the 1 GiB copy kernel (profiles/bench_all_kernels_hbm_bytes.txt).
-TRAFFIC_BYTES_GEMM_BF16_8192 = 1.7497e9
+# reading for the 1 GiB copy kernel (profiles/bench_all_kernels_hbm_bytes.txt).  A
+# profiler figure carried into the line, not something this run measures.
+TRAFFIC_BYTES_GEMM_BF16_8192 = 1.7452e9
 
 
 RAMP_SECONDS = 0.1
@@ -798,8 +799,8 @@ def main() -> int:
                    "device": lane.device_name()},
         "roofline": {"bound": "mfma", "achieved": flop / ev / 1e9, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": flop / ev / 1e9 / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BYTES_GEMM_BF16_8192,
-                     "traffic_source": "profiles/gemm_bf16_8192_hbm_bytes.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
-                                       "scaled by the copy kernel's readings)",
+                     "traffic_source": "profiles/bench_all_kernels_hbm_bytes.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an "
+                                       "earlier run, scaled by the copy kernel's readings; not measured by this run)",
                      "kernel": "gemm16_kernel<BF16,256,256,2,2,STORE16>", "avg_launch_ms": ev},
     }
     if copy_cal:

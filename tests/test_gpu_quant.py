@@ -142,3 +142,40 @@ def test_fp8_headline_shape_properties(lane):
     rows = rng.choice(M, 8, replace=False)
     ref = orc.gemm_e4m3(ac[rows], bc, 0.5, 0.25)
     assert orc.max_rel_err(got[rows], ref) <= 2e-3
+
+
+def test_config5_chain_at_full_size_on_normal_data(lane):
+    """The quantised-GEMM configuration end to end on its own data path: N(0,1)
+    operands (M = 4096, N = K = 8192) quantised by the lane's quantisers, multiplied,
+    rescaled; checked against the oracle's chain on sampled rows — (b) W8A8: codes,
+    scales and int32 accumulators bit-exact, y equal to f32 rounding; (a) e4m3: codes
+    equal as values (-0 and +0 are two codes of one value), result within 2e-3 of the
+    f32 product of the dequantised operands and within the format's own error of the
+    unquantised product."""
+    M, N, K = 4096, 8192, 8192
+    rng = np.random.default_rng(55)
+    X = rng.standard_normal((M, K), dtype=np.float32)
+    W = rng.standard_normal((K, N), dtype=np.float32)
+    rows = np.sort(rng.choice(M, 12, replace=False))
+    # (b) int8 W8A8
+    xq, a_scale = ops.quantize_int8_per_channel(X, axis=1)
+    wq, w_scale = ops.quantize_int8_per_channel(W, axis=0)
+    y, acc = ops.w8a8_gemm(xq, wq, a_scale, w_scale, return_acc=True)
+    ry, racc, rxq, ras, rwq, rws = orc.w8a8_matmul(X[rows], W)
+    assert np.array_equal(xq[rows], rxq) and np.array_equal(wq, rwq)
+    assert np.array_equal(a_scale[rows], ras) and np.array_equal(w_scale.reshape(-1), rws)
+    assert np.array_equal(acc[rows], racc)
+    assert np.array_equal(y[rows], ry)
+    # (a) fp8 e4m3 with per-tensor scales
+    xc, sx = ops.quantize_fp8_codes(X)
+    wc, sw = ops.quantize_fp8_codes(W)
+    oxc, _, osx = orc.quantize_fp8_e4m3(X)
+    owc, _, osw = orc.quantize_fp8_e4m3(W)
+    table = orc.e4m3_decode_table()
+    assert sx == osx and sw == osw
+    assert np.array_equal(table[xc], table[oxc]) and np.array_equal(table[wc], table[owc])
+    got = ops.gemm_fp8(xc, wc, sx, sw, out="f32")[rows]
+    assert orc.max_rel_err(got, orc.gemm_e4m3(oxc[rows], owc, osx, osw)) <= 2e-3
+    assert orc.max_rel_err(got, X[rows].astype(np.float64) @ W.astype(np.float64)) <= 5e-2
+    stored = ops.gemm_fp8(xc, wc, sx, sw, out="bf16")[rows]
+    assert np.array_equal(stored.to_float32(), orc.round_to_storage(got, "bf16"))
