@@ -297,6 +297,11 @@ def bench_quant(lane, steps, warmup, check=True):
                                                         "(includes quantising the whole 8192 x 8192 weight); "
                                                         "the full workload has 64x the rows"}
     out["gemm_w8a8_scaled_4096x8192x8192"] = w8
+    # the int8 matrix pipes' own rate on such codes, no memory access: the ceiling of both rows above
+    c8 = mfma_ceiling(lane, _OPTS["ceiling_seconds"], "int8")
+    out["mfma_ceiling_int8"] = c8
+    for key in ("gemm_int8_4096x8192x8192", "gemm_w8a8_scaled_4096x8192x8192"):
+        out[key].update(_ceiling_fields(c8, out[key]["tops"]))
 
     # ---- (a) fp8 e4m3, per-tensor scales ---------------------------------------------------
     sx, sw = lane.DeviceBuffer(4), lane.DeviceBuffer(4)
@@ -337,6 +342,9 @@ def bench_quant(lane, steps, warmup, check=True):
         f8["cpu_baseline"] = {"value": 2.0 * len(sample) * N * K / dt / 1e12, "unit": "TFLOP/s", "cores": _blas_threads(),
                               "kind": "port", "sample": f"quantise both tensors + f64 product of 64 dequantised rows in "
                                                         f"numpy, {dt:.2f} s; the full workload has 64x the rows"}
+    cf = mfma_ceiling(lane, _OPTS["ceiling_seconds"], "fp8")
+    out["mfma_ceiling_fp8"] = cf
+    f8.update(_ceiling_fields(cf, f8["tflops"]))
     out["gemm_fp8_e4m3_4096x8192x8192"] = f8
     for buf in (xf, wf, xq, wq, rs, cs, dd, sx, sw):
         buf.close()
@@ -503,37 +511,68 @@ def bench_moe(lane, steps, warmup, check=True):
     return out
 
 
-def mfma_ceiling(lane, seconds=2.0):
-    """The rate a register-only loop of independent 32x32x16 bf16 MFMAs reaches on this
-    board (tessera_gfx950_mfma_probe_bf16_dev: no memory access inside the loop), on
-    operands distributed like the headline GEMM's (N(0,1)/sqrt(8192)) and on constant ones,
-    with the shader clock and socket power sampled while it runs.  The matrix pipes draw
-    more power on toggling operands, the board holds its power limit by lowering the clock,
-    and the published peak assumes PEAK_CLOCK_MHZ: the random-operand figure is the ceiling a
-    GEMM on such data is up against on this board."""
+def mfma_ceiling(lane, seconds=2.0, kind="bf16"):
+    """The rate a register-only loop of independent matrix instructions reaches on this board
+    (tessera_gfx950_mfma_probe_dev: no memory access inside the loop; 32x32x16 bf16, 32x32x32
+    int8 or 32x32x64 fp8), on operands distributed like the workload's and on constant ones,
+    with the shader clock and socket power sampled while it runs.  The matrix pipes draw more
+    power on toggling operands, the board holds its power limit by lowering the clock, and the
+    published peak assumes PEAK_CLOCK_MHZ: the random-operand figure is the ceiling a GEMM on
+    such data is up against on this board.  bf16: N(0,1)/sqrt(8192) values; int8 and fp8: the
+    codes the lane's own quantisers give N(0,1) data (per-row absmax / per-tensor amax)."""
     import ctypes
     lib = lane.load()
     rng = np.random.default_rng(7)
-    n16 = 16 * 8 * 64 * 8                                   # bf16 values in the fragment buffer
+    nbytes = 16 * 8 * 64 * 16                               # the probe's fragment buffer
+    code = {"bf16": 0, "int8": 1, "fp8": 2}[kind]
     sink = lane.DeviceBuffer(1024 * 256 * 4)
-    flop = ctypes.c_double(0.0)
-    rounds = 600
+    ops = ctypes.c_double(0.0)
+    rounds = 600 if kind == "bf16" else 300
+    if kind == "bf16":
+        random_frags = lane.DeviceBuffer.from_host(_bf16(rng.standard_normal(nbytes // 2, dtype=np.float32) / np.sqrt(8192.0)))
+        constant = np.full(nbytes // 2, 0x3C3C, np.uint16)
+    else:
+        xf = lane.DeviceBuffer.from_host(rng.standard_normal(nbytes, dtype=np.float32))
+        random_frags, scales = lane.DeviceBuffer(nbytes), lane.DeviceBuffer(16 * 4)
+        if kind == "int8":
+            lane.check(lib.tessera_gfx950_quantize_i8_f32_dev(xf.ptr, 16, nbytes // 16, 1, random_frags.ptr, scales.ptr, None),
+                       "quantize_i8")
+            constant = np.full(nbytes, 1, np.int8)
+        else:
+            lane.check(lib.tessera_gfx950_quantize_e4m3_f32_dev(xf.ptr, nbytes, 0.0, random_frags.ptr, scales.ptr, None),
+                       "quantize_e4m3")
+            constant = np.full(nbytes, 0x38, np.uint8)       # 1.0 in e4m3
+        lane.synchronize()
+        xf.close()
+        scales.close()
     out = {}
-    for tag, vals in (("random", _bf16(rng.standard_normal(n16, dtype=np.float32) / np.sqrt(8192.0))),
-                      ("constant", np.full(n16, 0x3C3C, np.uint16))):
-        frags = lane.DeviceBuffer.from_host(vals)
-        launch = lambda: lane.check(lib.tessera_gfx950_mfma_probe_bf16_dev(frags.ptr, rounds, sink.ptr,
-                                                                           ctypes.byref(flop), None), "mfma_probe")
+    for tag, frags in (("random", random_frags), ("constant", lane.DeviceBuffer.from_host(constant))):
+        launch = lambda: lane.check(lib.tessera_gfx950_mfma_probe_dev(code, frags.ptr, rounds, sink.ptr,
+                                                                      ctypes.byref(ops), None), "mfma_probe")
         _, ev = _timed(lane, launch, 20, 5)
-        r = {"tflops": flop.value / ev / 1e9, "ms": ev}
-        held = _sustained(lane, launch, seconds)
-        if "ms" in held:
-            r.update({"tflops_sustained": flop.value / held["ms"] / 1e9, "gfx_clock_mhz": held["gfx_clock_mhz"],
-                      "socket_power_w": held["socket_power_w"]})
+        r = {"tflops": ops.value / ev / 1e9, "ms": ev}
+        if seconds > 0:
+            held = _sustained(lane, launch, seconds)
+            if "ms" in held:
+                r.update({"tflops_sustained": ops.value / held["ms"] / 1e9, "gfx_clock_mhz": held["gfx_clock_mhz"],
+                          "socket_power_w": held["socket_power_w"]})
         out[tag] = r
         frags.close()
     sink.close()
     return out
+
+
+def _ceiling_fields(ceil, rate):
+    """What a roofline entry says about the measured matrix-pipe ceiling."""
+    rnd, cst = ceil["random"], ceil["constant"]
+    top = rnd.get("tflops_sustained", rnd["tflops"])
+    return {"ceiling_random_tflops": top, "ceiling_constant_tflops": cst.get("tflops_sustained", cst["tflops"]),
+            "ceiling_random_clock_mhz": rnd.get("gfx_clock_mhz"), "ceiling_random_power_w": rnd.get("socket_power_w"),
+            "ceiling_constant_clock_mhz": cst.get("gfx_clock_mhz"), "ceiling_constant_power_w": cst.get("socket_power_w"),
+            "frac_of_random_ceiling": rate / top}
+
+
+_OPTS = {"ceiling_seconds": 1.5}      # 0: time the ceiling probes without sampling clock and power
 
 
 _VENDOR_SNIPPET = r"""
@@ -774,6 +813,8 @@ def main() -> int:
         return 3
 
     _RAMP["foreign"] = bool(args.profile)
+    if args.no_clock or args.profile:
+        _OPTS["ceiling_seconds"] = 0.0
     if args.clocks:
         print(json.dumps(clock_and_power_trace(lane), indent=1))
         return 0
@@ -782,7 +823,8 @@ def main() -> int:
         return 0
     if args.only:
         if args.only == "mfma_ceiling":
-            print(json.dumps({"mfma_ceiling": mfma_ceiling(lane, 0.0 if args.no_clock else 2.0)}))
+            print(json.dumps({"mfma_ceiling": {k: mfma_ceiling(lane, 0.0 if args.no_clock else 2.0, k)
+                                                for k in ("bf16", "int8", "fp8")}}))
         else:
             print(json.dumps(run_also(lane, args.only, args.steps, args.warmup, not args.no_cpu)))
         return 0
@@ -810,14 +852,7 @@ def main() -> int:
         # like the workload's and on constant ones, clock and power sampled under each
         ceil = mfma_ceiling(lane)
         result["mfma_ceiling"] = ceil
-        rnd, cst = ceil["random"], ceil["constant"]
-        result["roofline"].update({
-            "ceiling_random_tflops": rnd.get("tflops_sustained", rnd["tflops"]),
-            "ceiling_constant_tflops": cst.get("tflops_sustained", cst["tflops"]),
-            "ceiling_random_clock_mhz": rnd.get("gfx_clock_mhz"), "ceiling_random_power_w": rnd.get("socket_power_w"),
-            "ceiling_constant_clock_mhz": cst.get("gfx_clock_mhz"),
-            "ceiling_constant_power_w": cst.get("socket_power_w"),
-            "frac_of_random_ceiling": flop / ev / 1e9 / rnd.get("tflops_sustained", rnd["tflops"])})
+        result["roofline"].update(_ceiling_fields(ceil, flop / ev / 1e9))
         # the same launches kept up for 2 s: what clock the board grants this kernel on this
         # data (the peak is quoted at PEAK_CLOCK_MHZ), and the busy fraction at that clock
         lib = lane.load()

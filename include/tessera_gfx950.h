@@ -208,6 +208,12 @@ int tessera_gfx950_bench_last_timer_source(void);
  * 4-7 as B operands); sink: device memory, 1024 * 256 floats; *flop (may be NULL) receives
  * the floating-point operations of one launch. */
 int tessera_gfx950_mfma_probe_bf16_dev(const void* fragments, int rounds, void* sink, double* flop, void* stream);
+/* The same probe for the other matrix instructions of the lane: kind 0 = 32x32x16 bf16 (the
+ * call above), 1 = 32x32x32 int8 (int32 accumulate; the fragments are int8 values), 2 =
+ * 32x32x64 fp8 e4m3 in its unscaled form (the fragments are e4m3 codes; a 32-byte operand is
+ * two neighbouring 16-byte fragments).  *ops receives the operations of one launch
+ * (2 * 32 * 32 * k per instruction).  No counterpart in the reference. */
+int tessera_gfx950_mfma_probe_dev(int kind, const void* fragments, int rounds, void* sink, double* ops, void* stream);
 
 /* ---- quantisers ------------------------------------------------------------ */
 

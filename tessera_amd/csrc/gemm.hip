@@ -67,6 +67,8 @@ int gemm16_host(const void* A, const void* B, void* D, int batch, int M, int N, 
 // the given operand values at the clock the board grants for them.
 constexpr int kProbeBlocks = 1024;
 constexpr int kProbeThreads = 256;
+// KIND 0: 32x32x16 bf16; 1: 32x32x32 int8; 2: 32x32x64 fp8 (e4m3, unscaled form)
+template <int KIND>
 __global__ __launch_bounds__(kProbeThreads, 1) void mfma_probe_kernel(const uint4* __restrict__ frags, int rounds,
                                                                        float* __restrict__ sink) {
   const int lane = threadIdx.x & 63;
@@ -78,18 +80,33 @@ __global__ __launch_bounds__(kProbeThreads, 1) void mfma_probe_kernel(const uint
     a[f] = frags[(wave * 8 + f) * 64 + lane];
     b[f] = frags[(wave * 8 + 4 + f) * 64 + lane];
   }
-  f32x16 acc[4][4];
+  using acc_t = std::conditional_t<KIND == 1, i32x16, f32x16>;
+  acc_t acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
   for (int it = 0; it < rounds; ++it) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x16<BF16>(a[i], b[j], acc[i][j]);
+      for (int j = 0; j < 4; ++j) {
+        if constexpr (KIND == 0) {
+          acc[i][j] = mfma_32x32x16<BF16>(a[i], b[j], acc[i][j]);
+        } else if constexpr (KIND == 1) {
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a[i]),
+                                                            __builtin_bit_cast(i32x4, b[j]), acc[i][j], 0, 0, 0);
+        } else {
+          // a 32-byte operand is two of the 16-byte fragments
+          const i32x4 a0 = __builtin_bit_cast(i32x4, a[i]), a1 = __builtin_bit_cast(i32x4, a[(i + 1) & 3]);
+          const i32x4 b0 = __builtin_bit_cast(i32x4, b[j]), b1 = __builtin_bit_cast(i32x4, b[(j + 1) & 3]);
+          const i32x8 a8 = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+          const i32x8 b8 = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[i][j], 0, 0, 0, 0, 0, 0);
+        }
+      }
   }
   float total = 0.f;
 #pragma unroll
@@ -97,7 +114,7 @@ __global__ __launch_bounds__(kProbeThreads, 1) void mfma_probe_kernel(const uint
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) total += acc[i][j][r];
+      for (int r = 0; r < 16; ++r) total += (float)acc[i][j][r];
   sink[(size_t)blockIdx.x * kProbeThreads + threadIdx.x] = total;
 }
 
@@ -351,13 +368,23 @@ int tessera_gfx950_gemm_bf16_bench_rotating(int M, int N, int K, int iters, int 
 
 int tessera_gfx950_bench_last_timer_source(void) { return g_last_timer_source; }
 
-int tessera_gfx950_mfma_probe_bf16_dev(const void* fragments, int rounds, void* sink, double* flop, void* stream) {
-  if (!fragments || !sink || rounds <= 0 || (reinterpret_cast<uintptr_t>(fragments) & 15)) return kBadShape;
-  if (flop) *flop = (double)kProbeBlocks * (kProbeThreads / 64) * rounds * 16.0 * (2.0 * 32 * 32 * 16);
+int tessera_gfx950_mfma_probe_dev(int kind, const void* fragments, int rounds, void* sink, double* ops, void* stream) {
+  if (kind < 0 || kind > 2 || !fragments || !sink || rounds <= 0 || (reinterpret_cast<uintptr_t>(fragments) & 15))
+    return kBadShape;
+  const int depth = kind == 0 ? 16 : kind == 1 ? 32 : 64;     // k of one instruction
+  if (ops) *ops = (double)kProbeBlocks * (kProbeThreads / 64) * rounds * 16.0 * (2.0 * 32 * 32 * depth);
   if (probe_device() != kOk) return kNoDevice;
-  hipLaunchKernelGGL(mfma_probe_kernel, dim3(kProbeBlocks), dim3(kProbeThreads), 0, as_stream(stream),
-                     static_cast<const uint4*>(fragments), rounds, static_cast<float*>(sink));
+  const dim3 grid(kProbeBlocks), block(kProbeThreads);
+  const uint4* f = static_cast<const uint4*>(fragments);
+  float* out = static_cast<float*>(sink);
+  if (kind == 0) hipLaunchKernelGGL(mfma_probe_kernel<0>, grid, block, 0, as_stream(stream), f, rounds, out);
+  else if (kind == 1) hipLaunchKernelGGL(mfma_probe_kernel<1>, grid, block, 0, as_stream(stream), f, rounds, out);
+  else hipLaunchKernelGGL(mfma_probe_kernel<2>, grid, block, 0, as_stream(stream), f, rounds, out);
   return launch_status();
+}
+
+int tessera_gfx950_mfma_probe_bf16_dev(const void* fragments, int rounds, void* sink, double* flop, void* stream) {
+  return tessera_gfx950_mfma_probe_dev(0, fragments, rounds, sink, flop, stream);
 }
 
 }  // extern "C"

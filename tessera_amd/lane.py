@@ -110,6 +110,7 @@ _SIGNATURES = {
     "tessera_gfx950_gemm_bf16_bench_rotating": [_c_int, _c_int, _c_int, _c_int, _c_int, _P(ctypes.c_double)],
     "tessera_gfx950_bench_last_timer_source": [],
     "tessera_gfx950_mfma_probe_bf16_dev": [_c_vp, _c_int, _c_vp, _P(ctypes.c_double), _c_vp],
+    "tessera_gfx950_mfma_probe_dev": [_c_int, _c_vp, _c_int, _c_vp, _P(ctypes.c_double), _c_vp],
     "tessera_gfx950_quantize_e4m3_f32": [_c_vp, _c_i64, _c_f, _c_vp, _P(_c_f)],
     "tessera_gfx950_quantize_i8_f32": [_c_vp, _c_int, _c_int, _c_int, _c_vp, _c_vp],
     "tessera_gfx950_quantize_e4m3_f32_dev": [_c_vp, _c_i64, _c_f, _c_vp, _c_vp, _c_vp],
