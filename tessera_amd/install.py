@@ -11,7 +11,9 @@ registrations, each into an object the host owns:
   ``:2495-2537``) and their catalogue entries (``KNOWN_EXECUTORS``, ``:103``);
 * executor functions under the ids those rows name (``runtime._executor_table()``,
   ``python/tessera/runtime.py:30515``; ``launch`` resolves a row's ``executor_id``
-  through it, ``:31008-31020``).
+  through it, ``:31008-31020``);
+* optionally, the submit hook for typed native artifacts
+  (``runtime.register_native_launcher``, ``python/tessera/runtime.py:279-306``).
 
 :func:`install` does those registrations into whatever objects it is handed, and
 nothing else: it owns no registry and restates none of the host's machinery.
@@ -22,6 +24,7 @@ from typing import Any, Callable, MutableMapping, Optional
 
 from . import candidates as _cand
 from . import executors as _ex
+from . import native_launcher as _native
 
 
 def _rows_into(matrix_owner: Any) -> list:
@@ -67,22 +70,27 @@ def _executors_into(table_owner: Any) -> list:
     return sorted(ours)
 
 
-def install(candidate_api: Any = None, execution_matrix: Any = None, executor_table: Any = None) -> dict:
+def install(candidate_api: Any = None, execution_matrix: Any = None, executor_table: Any = None,
+            native_launchers: Any = None) -> dict:
     """Register the lane with a host; every argument is optional and independent.
 
     ``candidate_api``     the host's candidate module / namespace -> op kind + five candidates
     ``execution_matrix``  the host's execution-matrix module / namespace -> five rows + catalogue
     ``executor_table``    a mapping, or the host's runtime module -> five executor functions
+    ``native_launchers``  the host's runtime module (``register_native_launcher``) -> the typed-descriptor
+                          submit hook for target ``rocm_gfx950``
 
     Returns what was registered: ``{"candidates": [names], "rows": [(target, path)],
-    "executors": [ids]}``.  Safe to call again (everything is keyed by name)."""
-    report: dict = {"candidates": [], "rows": [], "executors": []}
+    "executors": [ids], "native_launcher": target or None}``.  Safe to call again (everything is keyed by name)."""
+    report: dict = {"candidates": [], "rows": [], "executors": [], "native_launcher": None}
     if candidate_api is not None:
         report["candidates"] = [c.name for c in _cand.register(candidate_api)]
     if execution_matrix is not None:
         report["rows"] = _rows_into(execution_matrix)
     if executor_table is not None:
         report["executors"] = _executors_into(executor_table)
+    if native_launchers is not None:
+        report["native_launcher"] = _native.register(native_launchers, replace=True)
     return report
 
 
@@ -92,4 +100,4 @@ def install_into_tessera() -> dict:
     from tessera import runtime
     from tessera.compiler import execution_matrix
     from tessera.compiler.emit import candidate
-    return install(candidate, execution_matrix, runtime)
+    return install(candidate, execution_matrix, runtime, runtime)

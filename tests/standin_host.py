@@ -320,3 +320,49 @@ class RuntimeHost:
             out, kind = out
         return {"ok": True, "runtime_status": "success", "execution_kind": kind, "output": out,
                 "compiler_path": row.compiler_path}
+
+
+# ---- typed native artifacts (stand-ins for the host's descriptor types) ---------------------
+
+@dataclass(frozen=True)
+class Binding:
+    """A descriptor's buffer binding: a name and its position among the arguments."""
+    name: str
+    ordinal: int
+
+
+@dataclass(frozen=True)
+class Descriptor:
+    abi_id: str
+    entry_symbol: str
+    buffers: tuple
+    provenance: dict = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class Image:
+    target: str
+    binary_format: str
+
+
+class NativeLauncherHost:
+    """Keeps one submit hook per exact target and drives it like the host's descriptor launch:
+    a raise from the hook becomes a ``device_error`` result."""
+
+    def __init__(self):
+        self.hooks = {}
+
+    def register_native_launcher(self, target, *, binary_formats, submit, replace=False):
+        if target in self.hooks and not replace:
+            raise ValueError(f"native launcher already registered for {target}")
+        self.hooks[target] = (tuple(binary_formats), submit)
+
+    def launch_descriptor(self, image, descriptor, buffers, scalars):
+        hook = self.hooks.get(image.target)
+        if hook is None or image.binary_format not in hook[0]:
+            return {"ok": False, "runtime_status": "unimplemented"}
+        try:
+            out = hook[1](image, descriptor, buffers, scalars, None)
+        except Exception as exc:                              # noqa: BLE001 - the envelope reports it
+            return {"ok": False, "runtime_status": "device_error", "reason": str(exc)}
+        return {"ok": True, "runtime_status": "success", "execution_kind": "native_gpu", "output": out}

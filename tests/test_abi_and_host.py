@@ -317,3 +317,39 @@ def test_gemm_schedule_query_needs_no_device():
         sel(8, 8, 8, arch="gfx1151")
     with pytest.raises(ValueError):
         sel(8, 8, 8, dtype="f64")
+
+
+def test_typed_descriptor_hook_validates_before_the_device():
+    """The native-launcher hook refuses what its descriptor does not cover with RuntimeError,
+    before any device call (nothing here needs a GPU)."""
+    from tessera_amd import native_launcher as nl
+    runtime = host.NativeLauncherHost()
+    assert inst.install(native_launchers=runtime)["native_launcher"] == nl.TARGET
+    assert runtime.hooks[nl.TARGET][0] == ("shared_object",)
+    inst.install(native_launchers=runtime)                                 # replace=True: no duplicate error
+    bind = lambda *names: tuple(host.Binding(n, i) for i, n in enumerate(names))
+    A = np.zeros((4, 8), np.float16)
+    B = np.zeros((8, 6), np.float16)
+    O = np.zeros((4, 6), np.float32)
+    image = host.Image(nl.TARGET, "shared_object")
+    cases = [
+        (host.Descriptor("tessera.rocm.softmax.x_o_rows_k.f32.v1", "tessera_gfx950_gemm_f16", bind("A", "B", "O")),
+         {"M": 4, "N": 6, "K": 8}, "unsupported"),
+        (host.Descriptor(nl.MATMUL_F16_F32_ABI, "tessera_gfx950_gemm_bf16", bind("A", "B", "O")),
+         {"M": 4, "N": 6, "K": 8}, "cannot launch"),
+        (host.Descriptor(nl.MATMUL_F16_F32_ABI, "tessera_gfx950_gemm_f16", bind("A", "B")),
+         {"M": 4, "N": 6, "K": 8}, "requires 3 buffers"),
+        (host.Descriptor(nl.MATMUL_F16_F32_ABI, "tessera_gfx950_gemm_f16", bind("A", "B", "O")),
+         {"M": 4, "N": 6, "K": 7}, "disagree"),
+        (host.Descriptor(nl.MATMUL_BF16_F32_ABI, "tessera_gfx950_gemm_bf16", bind("A", "B", "O")),
+         {"M": 4, "N": 6, "K": 8}, "disagree"),                            # f16 arrays under a bf16 ABI
+    ]
+    for desc, scalars, needle in cases:
+        res = runtime.launch_descriptor(image, desc, {"A": A, "B": B, "O": O}, scalars)
+        assert not res["ok"] and res["runtime_status"] == "device_error" and needle in res["reason"], (needle, res)
+    x = np.zeros((3, 4), np.float32)
+    res = runtime.launch_descriptor(
+        image, host.Descriptor(nl.MOE_DISPATCH_F32_ABI, "tessera_gfx950_moe_dispatch", bind("X", "T", "O")),
+        {"X": x, "T": np.array([0, 3], np.int32), "O": np.zeros((2, 4), np.float32)}, {"T": 3, "S": 2, "H": 4})
+    assert not res["ok"] and "disagree" in res["reason"]                   # token id 3 is out of range
+    assert set(nl.supported_abis()) >= {nl.MATMUL_F16_F32_ABI, nl.ATTN_BF16_ABI, nl.MOE_DISPATCH_F32_ABI}

@@ -10,6 +10,7 @@ from tessera_amd import bf16 as b16
 from tessera_amd import candidates as cand
 from tessera_amd import executors as ex
 from tessera_amd import install as inst
+from tessera_amd import native_launcher as nl
 from tessera_amd import ops
 
 pytestmark = pytest.mark.gpu
@@ -127,6 +128,59 @@ def test_installed_lane_is_reached_through_the_hosts_launch(lane):
     res = runtime.launch(art, (A, B))
     assert res["ok"] and res["execution_kind"] == "native_gpu" and res["compiler_path"] == "gfx950_gemm"
     assert orc.max_rel_err(res["output"], A.astype(np.float64) @ B.astype(np.float64)) <= 1e-5
+
+
+def _typed(abi, entry, names, provenance=None):
+    return host.Descriptor(abi, entry, tuple(host.Binding(n, i) for i, n in enumerate(names)), provenance or {})
+
+
+def test_typed_descriptor_launches(lane):
+    """The third seam: artifacts with a native image and a launch descriptor reach the lane
+    through the hook install() registers for the exact target."""
+    runtime = host.NativeLauncherHost()
+    assert inst.install(native_launchers=runtime)["native_launcher"] == "rocm_gfx950"
+    image = host.Image("rocm_gfx950", "shared_object")
+    rng = np.random.default_rng(11)
+    # matmul, f16 and bf16 -> f32
+    A = (rng.standard_normal((70, 96)) * .5).astype(np.float16)
+    B = (rng.standard_normal((96, 50)) * .5).astype(np.float16)
+    out = np.zeros((70, 50), np.float32)
+    res = runtime.launch_descriptor(image, _typed(nl.MATMUL_F16_F32_ABI, "tessera_gfx950_gemm_f16", ("A", "B", "O")),
+                                    {"A": A, "B": B, "O": out}, {"M": 70, "N": 50, "K": 96})
+    assert res["ok"] and res["output"] is out
+    assert orc.max_rel_err(out, A.astype(np.float64) @ B.astype(np.float64)) <= 1e-5
+    Ab, Bb = b16.from_float32(A.astype(np.float32)), b16.from_float32(B.astype(np.float32))
+    res = runtime.launch_descriptor(image, _typed(nl.MATMUL_BF16_F32_ABI, "tessera_gfx950_gemm_bf16", ("A", "B", "O")),
+                                    {"A": Ab, "B": Bb, "O": out}, {"M": 70, "N": 50, "K": 96})
+    assert res["ok"]
+    assert orc.max_rel_err(out, Ab.to_float32().astype(np.float64) @ Bb.to_float32().astype(np.float64)) <= 1e-5
+    # a descriptor whose scalars disagree with the arrays is refused before the device is touched
+    res = runtime.launch_descriptor(image, _typed(nl.MATMUL_F16_F32_ABI, "tessera_gfx950_gemm_f16", ("A", "B", "O")),
+                                    {"A": A, "B": B, "O": out}, {"M": 70, "N": 50, "K": 95})
+    assert not res["ok"] and res["runtime_status"] == "device_error" and "disagree" in res["reason"]
+    # attention: GQA, causal, a left window of 23 keys (band width 24)
+    b_, hq, hkv, sq, sk, d = 1, 4, 2, 80, 112, 64
+    Q = (rng.standard_normal((b_, hq, sq, d)) * .5).astype(np.float16)
+    K = (rng.standard_normal((b_, hkv, sk, d)) * .5).astype(np.float16)
+    V = (rng.standard_normal((b_, hkv, sk, d)) * .5).astype(np.float16)
+    O = np.zeros((b_, hq, sq, d), np.float32)
+    prov = {"shape": [b_, hq, hkv, sq, sk, d, d], "scale": 0.125, "causal": True, "gqa": True, "kv_ratio": 2,
+            "window_left": 23, "softcap": 0.0, "dropout_p": 0.0, "bias": False}
+    res = runtime.launch_descriptor(image, _typed(nl.ATTN_F16_ABI, "tessera_gfx950_flash_attn_ext_f16",
+                                                  ("Q", "K", "V", "O"), prov), {"Q": Q, "K": K, "V": V, "O": O}, {})
+    assert res["ok"], res
+    ref, _ = orc.flash_attn_dense(Q, K, V, 0.125, True, window=24)
+    assert orc.max_rel_err(O, ref) <= 2e-3
+    # MoE dispatch: an exact f32 gather
+    x = rng.standard_normal((33, 40)).astype(np.float32)
+    token = rng.integers(0, 33, 57).astype(np.int32)
+    y = np.zeros((57, 40), np.float32)
+    res = runtime.launch_descriptor(image, _typed(nl.MOE_DISPATCH_F32_ABI, "tessera_gfx950_moe_dispatch", ("X", "Token", "O")),
+                                    {"X": x, "Token": token, "O": y}, {"T": 33, "S": 57, "H": 40})
+    assert res["ok"] and np.array_equal(y, x[token])
+    # another target's image, or another format, is not this lane's
+    assert runtime.launch_descriptor(host.Image("rocm_gfx1151", "hsaco"), _typed(nl.MATMUL_F16_F32_ABI, "k", ("A",)),
+                                     {}, {})["runtime_status"] == "unimplemented"
 
 
 def test_bench_abi(lane):
