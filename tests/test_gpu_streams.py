@@ -1,0 +1,156 @@
+"""The `_dev` entry points on caller-owned HIP streams, from several host threads.
+
+Every `_dev` entry point takes a `hipStream_t`, enqueues and returns; the kernels that need
+scratch memory take it from a workspace the library keeps per (device, stream).  The other GPU
+tests pass the null stream.  Here the streams are the caller's (created through the HIP
+runtime, default priority), two host threads drive one stream each at the same time (ctypes
+drops the GIL during a call), and every result must equal, bit for bit, what the same call
+gives on the null stream: a workspace shared between streams, or a launch that ignored its
+stream argument, shows up as a mismatch.
+"""
+import ctypes
+import threading
+
+import numpy as np
+import pytest
+
+from tessera_amd import bf16 as b16
+
+pytestmark = pytest.mark.gpu
+
+
+class _Hip:
+    """The three runtime calls a caller needs to own a stream."""
+
+    def __init__(self):
+        self.lib = ctypes.CDLL("libamdhip64.so", mode=ctypes.RTLD_LOCAL)
+        self.lib.hipStreamCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.lib.hipStreamSynchronize.argtypes = [ctypes.c_void_p]
+        self.lib.hipStreamDestroy.argtypes = [ctypes.c_void_p]
+
+    def stream(self):
+        s = ctypes.c_void_p()
+        assert self.lib.hipStreamCreate(ctypes.byref(s)) == 0
+        return s
+
+    def sync(self, s):
+        assert self.lib.hipStreamSynchronize(s) == 0
+
+    def destroy(self, s):
+        assert self.lib.hipStreamDestroy(s) == 0
+
+
+@pytest.fixture(scope="module")
+def hip():
+    return _Hip()
+
+
+def _splitk_case(lane, seed, M=16, N=1024, K=4096):
+    """A decode-shaped product: the K-split form, whose partials live in the stream's workspace."""
+    rng = np.random.default_rng(seed)
+    a = b16.from_float32(rng.standard_normal((M, K)).astype(np.float32) * 0.5)
+    b = b16.from_float32(rng.standard_normal((K, N)).astype(np.float32) * 0.5)
+    da = lane.DeviceBuffer.from_host(np.asarray(a, np.uint16))
+    db = lane.DeviceBuffer.from_host(np.asarray(b, np.uint16))
+    dd = lane.DeviceBuffer(M * N * 4)
+    return da, db, dd, (M, N, K)
+
+
+def _route_case(lane, seed, T=700, E=64, k=8):
+    rng = np.random.default_rng(seed)
+    lg = rng.standard_normal((T, E)).astype(np.float32)
+    S = T * k
+    bufs = dict(lg=lane.DeviceBuffer.from_host(lg), tos=lane.DeviceBuffer(S * 4), eos=lane.DeviceBuffer(S * 4),
+                cw=lane.DeviceBuffer(S * 4), gs=lane.DeviceBuffer(E * 4), go=lane.DeviceBuffer((E + 1) * 4),
+                n=lane.DeviceBuffer(4))
+    return bufs, (T, E, k)
+
+
+def _gemm(lane, case, stream):
+    da, db, dd, (M, N, K) = case
+    dd.zero()
+    lane.check(lane.load().tessera_gfx950_gemm_bf16_dev(da.ptr, db.ptr, dd.ptr, M, N, K, stream), "gemm")
+
+
+def _route(lane, case, stream):
+    b, (T, E, k) = case
+    for name in ("tos", "eos", "cw", "gs", "go", "n"):
+        b[name].zero()
+    lane.check(lane.load().tessera_gfx950_moe_route_f32_dev(b["lg"].ptr, T, E, k, 1, 0, b["tos"].ptr, b["eos"].ptr,
+                                                            b["cw"].ptr, b["gs"].ptr, b["go"].ptr, b["n"].ptr, stream),
+               "route")
+
+
+def _read_gemm(case):
+    _, _, dd, (M, N, _) = case
+    return dd.download((M, N), np.float32)
+
+
+def _read_route(case):
+    b, (T, E, k) = case
+    S = T * k
+    return [b["tos"].download((S,), np.int32), b["eos"].download((S,), np.int32), b["cw"].download((S,), np.float32),
+            b["gs"].download((E,), np.int32), b["go"].download((E + 1,), np.int32)]
+
+
+def test_caller_streams_give_the_null_stream_results(lane, hip):
+    assert lane.load().tessera_gfx950_probe() == 0
+    g, r = _splitk_case(lane, 1), _route_case(lane, 2)
+    _gemm(lane, g, None)
+    _route(lane, r, None)
+    lane.synchronize()
+    want_g, want_r = _read_gemm(g), _read_route(r)
+    s = hip.stream()
+    try:
+        for _ in range(3):
+            _gemm(lane, g, s)
+            _route(lane, r, s)
+            hip.sync(s)
+            assert np.array_equal(_read_gemm(g), want_g)
+            for got, want in zip(_read_route(r), want_r):
+                assert np.array_equal(got, want)
+    finally:
+        hip.destroy(s)
+
+
+def test_two_threads_two_streams_at_once(lane, hip):
+    """Each thread owns a stream, its own operands and outputs, and alternates the K-split
+    product and the routing 40 times; the other thread does the same with different data at the
+    same time.  Every round must reproduce the thread's null-stream reference."""
+    cases = []
+    for t in range(2):
+        g, r = _splitk_case(lane, 10 + t, M=16 + 16 * t), _route_case(lane, 20 + t, T=500 + 300 * t)
+        _gemm(lane, g, None)
+        _route(lane, r, None)
+        lane.synchronize()
+        cases.append((g, r, _read_gemm(g), _read_route(r)))
+    streams = [hip.stream(), hip.stream()]
+    errors = []
+
+    def work(i):
+        g, r, want_g, want_r = cases[i]
+        try:
+            for round_ in range(40):
+                _gemm(lane, g, streams[i])
+                _route(lane, r, streams[i])
+                hip.sync(streams[i])
+                if not np.array_equal(_read_gemm(g), want_g):
+                    errors.append((i, round_, "gemm"))
+                for got, want in zip(_read_route(r), want_r):
+                    if not np.array_equal(got, want):
+                        errors.append((i, round_, "route"))
+        except Exception as exc:                          # noqa: BLE001 - reported by the main thread
+            errors.append((i, "raised", repr(exc)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    try:
+        for th in threads:
+            th.start()
+        for th in threads:
+            th.join(timeout=100)
+        assert not any(th.is_alive() for th in threads), "a stream thread did not finish"
+        assert not errors, errors[:5]
+    finally:
+        for s in streams:
+            hip.sync(s)
+            hip.destroy(s)
