@@ -154,3 +154,91 @@ def test_two_threads_two_streams_at_once(lane, hip):
         for s in streams:
             hip.sync(s)
             hip.destroy(s)
+
+
+def test_dev_entry_points_under_stream_capture(lane, hip):
+    """The `_dev` calls record into a HIP graph (they clear their counters with a fill kernel,
+    not a memset node, and take scratch from a workspace that already has its size after one
+    eager call).  The graph is replayed several times with eager work and synchronisations in
+    between; every replay must reproduce the eager results bit for bit."""
+    L = hip.lib
+    L.hipStreamBeginCapture.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    L.hipStreamEndCapture.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]
+    L.hipGraphInstantiate.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_void_p,
+                                      ctypes.c_void_p, ctypes.c_size_t]
+    L.hipGraphLaunch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    L.hipGraphExecDestroy.argtypes = [ctypes.c_void_p]
+    L.hipGraphDestroy.argtypes = [ctypes.c_void_p]
+    lib = lane.load()
+    g, r = _splitk_case(lane, 31), _route_case(lane, 32)
+    da, db, dd, (M, N, K) = g
+    rb, (T, E, k) = r
+    # attention operands
+    rng = np.random.default_rng(33)
+    B, Hq, Hkv, Sq, Sk, D = 1, 4, 2, 200, 264, 128
+    q, kk, v = (lane.DeviceBuffer.from_host(np.asarray(b16.from_float32(
+        rng.standard_normal(shape).astype(np.float32)), np.uint16)) for shape in
+        ((B, Hq, Sq, D), (B, Hkv, Sk, D), (B, Hkv, Sk, D)))
+    o, lse = lane.DeviceBuffer(B * Hq * Sq * D * 4), lane.DeviceBuffer(B * Hq * Sq * 4)
+    # a whole MoE layer with its router product (caller-provided workspace)
+    mT, mH, mF, mE, mk = 300, 256, 384, 8, 2
+    bits = lambda a: np.asarray(b16.from_float32(a.astype(np.float32)), np.uint16)
+    mx = lane.DeviceBuffer.from_host(bits(rng.standard_normal((mT, mH))))
+    mwr = lane.DeviceBuffer.from_host(bits(rng.standard_normal((mH, mE)) / 16))
+    mwg, mwu = (lane.DeviceBuffer.from_host(bits(rng.standard_normal((mE, mH, mF)) / 16)) for _ in range(2))
+    mwd = lane.DeviceBuffer.from_host(bits(rng.standard_normal((mE, mF, mH)) / 20))
+    need = ctypes.c_size_t(0)
+    lane.check(lib.tessera_gfx950_moe_layer_workspace_bytes(mT, mH, mF, mH, mE, mk, ctypes.byref(need)), "workspace")
+    mws, mout = lane.DeviceBuffer(need.value), lane.DeviceBuffer(mT * mH * 4)
+    mS = mT * mk
+    mplan = [lane.DeviceBuffer(mS * 4), lane.DeviceBuffer(mS * 4), lane.DeviceBuffer(mS * 4), lane.DeviceBuffer(mE * 4),
+             lane.DeviceBuffer((mE + 1) * 4), lane.DeviceBuffer(4)]
+
+    def enqueue(s):
+        lane.check(lib.tessera_gfx950_moe_layer_bf16_dev(
+            mx.ptr, mwr.ptr, None, mwg.ptr, mwu.ptr, mwd.ptr, mout.ptr, mws.ptr, need.value, mT, mH, mF, mH, mE, mk, 1, 0,
+            *(b.ptr for b in mplan), s), "moe_layer")
+        lane.check(lib.tessera_gfx950_gemm_bf16_dev(da.ptr, db.ptr, dd.ptr, M, N, K, s), "gemm")
+        lane.check(lib.tessera_gfx950_moe_route_f32_dev(rb["lg"].ptr, T, E, k, 1, 0, rb["tos"].ptr, rb["eos"].ptr,
+                                                        rb["cw"].ptr, rb["gs"].ptr, rb["go"].ptr, rb["n"].ptr, s), "route")
+        lane.check(lib.tessera_gfx950_flash_attn_gqa_bf16_dev(q.ptr, kk.ptr, v.ptr, o.ptr, lse.ptr, B, Hq, Hkv, Sq, Sk, D,
+                                                              ctypes.c_float(D ** -0.5), 1, 0, s), "flash_attn")
+
+    def read():
+        return [_read_gemm(g)] + _read_route(r) + [o.download((B, Hq, Sq, D), np.float32),
+                                                  lse.download((B, Hq, Sq), np.float32),
+                                                  mout.download((mT, mH), np.float32),
+                                                  mplan[0].download((mS,), np.int32)]
+
+    def clear():
+        for buf in (dd, o, lse, rb["tos"], rb["eos"], rb["cw"], rb["gs"], rb["go"], rb["n"], mout, mws, *mplan):
+            buf.zero()
+
+    s = hip.stream()
+    graph, exe = ctypes.c_void_p(), ctypes.c_void_p()
+    try:
+        enqueue(s)                                   # eager: sizes the stream's workspace, gives the reference
+        hip.sync(s)
+        want = read()
+        assert L.hipStreamBeginCapture(s, 0) == 0
+        enqueue(s)
+        assert L.hipStreamEndCapture(s, ctypes.byref(graph)) == 0 and graph.value
+        assert L.hipGraphInstantiate(ctypes.byref(exe), graph, None, None, 0) == 0
+        for replay in range(4):
+            clear()
+            # the program's own eager work between replays, on the same and on the null stream
+            _gemm(lane, _splitk_case(lane, 40 + replay, M=8), s)
+            hip.sync(s)
+            lane.synchronize()
+            clear()
+            assert L.hipGraphLaunch(exe, s) == 0
+            hip.sync(s)
+            for idx, (got, ref) in enumerate(zip(read(), want)):
+                assert np.array_equal(got, ref, equal_nan=True), (replay, idx)
+    finally:
+        if exe.value:
+            L.hipGraphExecDestroy(exe)
+        if graph.value:
+            L.hipGraphDestroy(graph)
+        hip.sync(s)
+        hip.destroy(s)
