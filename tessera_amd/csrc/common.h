@@ -71,6 +71,16 @@ template <> __device__ __forceinline__ f32x16 mfma_32x32x16<F16>(const uint4& a,
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
+// 16x16x32 MFMA on 16-bit operands (four accumulator registers per lane).  Per FLOP it moves
+// half the accumulator data of the 32x32x16 form through the register file.
+template <class T> __device__ __forceinline__ f32x4 mfma_16x16x32(const uint4& a, const uint4& b, f32x4 c);
+template <> __device__ __forceinline__ f32x4 mfma_16x16x32<BF16>(const uint4& a, const uint4& b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ f32x4 mfma_16x16x32<F16>(const uint4& a, const uint4& b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
 // LDS accessors on a byte offset into the dynamic LDS window.
 __device__ __forceinline__ uint4 lds_read_b128(const char* base, uint32_t byte_off) {
   return *reinterpret_cast<const uint4*>(base + byte_off);

@@ -130,16 +130,29 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
   tn = r / rows;
 }
 
+}  // namespace tsr950
+#include "gemm16_dl.h"
+namespace tsr950 {
+
 // One BM x BN output tile: rows [m_begin, min(m_begin + BM, m_end)), column tile tn, of
 // the product whose operand and output bases are Ab / Bb / B2b / Db.  All threads of the
 // workgroup call it with the same arguments.
-template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED>
+template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32, bool DL = false>
 __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, const int m_begin, const int m_end,
                                             const int tn, const uint16_t* Ab, const uint16_t* Bb,
                                             const uint16_t* B2b, char* Db) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN;     // wave tile
-  constexpr int MI = TM / 32, NJ = TN / 32;     // 32x32 MFMA tiles per wave
+  // MS: side of the MFMA tile.  32: v_mfma_f32_32x32x16 (16 accumulator registers per lane and
+  // tile, k = 16 per instruction); 16: v_mfma_f32_16x16x32 (4 registers, k = 32).  Per FLOP the
+  // 16-wide form reads and writes half the accumulator data, and a register-only loop of it runs
+  // 14 % faster under the board's power limit on random operands (2010 against 1760 TFLOP/s):
+  // the big tiles, which sit on that limit, use it.
+  static_assert(MS == 32 || MS == 16, "MFMA tile side");
+  constexpr int KD = 512 / MS;                  // k per MFMA instruction
+  constexpr int AE = MS * MS / 64;              // accumulator registers per MFMA tile
+  constexpr int MI = TM / MS, NJ = TN / MS;     // MFMA tiles per wave
+  using acc_t = std::conditional_t<MS == 32, f32x16, f32x4>;
   constexpr bool SWIGLU = (EPI == EPI_SWIGLU16 || EPI == EPI_GATED_F32);   // two-source B tile
   // SwiGLU: the BN columns of the LDS B tile are [gate n0..n0+BN/2) | up n0..n0+BN/2);
   // a wave's first NJ/2 column tiles are gate columns and the rest the matching up
@@ -158,15 +171,35 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
   constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;   // output columns per tile
   const int n_begin = tn * BN_OUT;
   const int K = p.K;
+  using std::true_type;
+  using std::false_type;
+  // A lane supplies row / column lm of an MFMA tile and the 8 k of group lk (KD / 8 groups).
+  const int lm = lane % MS, lk = lane / MS;
+  acc_t acc[MI][NJ];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int r = 0; r < AE; ++r) acc[i][j][r] = 0.f;
 
+  if constexpr (DL) {
+    gemm16_mainloop_dl<T, BM, BN, WM, WN, SWIGLU, GROUPED>(p, smem, acc, m_begin, m_end, n_begin, Ab, Bb, B2b);
+  } else {
   // ---- global load addressing ----------------------------------------------------
   // Buffer loads: a wave-uniform tile base (advanced along K on the scalar unit) plus
   // a fixed 32-bit per-lane byte offset, one address register per chunk.
   // A: chunk v = tid + NT*q  -> row v/8, 16-byte chunk v%8.
   const bool gathered = GROUPED && p.gather != nullptr;
   const uint16_t* a_base = gathered ? Ab : Ab + (long)m_begin * p.lda;
-  uint32_t a_off[A_CHUNKS], a_lds[A_CHUNKS];
+  // A thread's chunks are NT / 8 rows apart, a multiple of 16 rows, so the LDS swizzle is the
+  // same for all of them: one LDS address, the others a constant apart.  (The global offsets
+  // stay one register each: rows are clamped at the edge and may be gathered.)
+  static_assert((NT / 8) % 16 == 0, "a thread's A chunks must share their swizzle");
+  uint32_t a_off[A_CHUNKS];
   const int a_chunk = tid & 7;
+  const uint32_t a_lds0 = (tid >> 3) * G16_APITCH + ((a_chunk ^ g16_aswz(tid >> 3)) << 4);
+  auto a_lds = [&](int q) { return a_lds0 + q * (NT / 8) * G16_APITCH; };
 #pragma unroll
   for (int q = 0; q < A_CHUNKS; ++q) {
     const int row = (tid >> 3) + (NT / 8) * q;
@@ -176,32 +209,28 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
       if (gathered) gr = p.gather[m_begin + gr];            // source row (the launcher bounds rows * lda)
     }
     a_off[q] = ((uint32_t)gr * (uint32_t)p.lda + a_chunk * 8) * 2;
-    a_lds[q] = row * G16_APITCH + ((a_chunk ^ g16_aswz(row)) << 4);
   }
   // B: the tile's columns come from one matrix, or (SwiGLU) half from the gate and
   // half from the up matrix; the first B_CHUNKS / HALVES chunks of a thread belong to
-  // the first source.  Within a source: chunk v = tid + NT*q' -> k row v/CPR, n chunk v%CPR.
+  // the first source.  Within a source: chunk v = tid + NT*q' -> k row v/CPR, n chunk v%CPR:
+  // a thread's chunks share their n chunk and are NT / CPR k rows apart, so one global
+  // offset and one LDS address serve them all (the k rows enter the scalar tile base).
   constexpr int HALVES = SWIGLU ? 2 : 1;
   constexpr int CPR = BN / HALVES / 8;           // 16-byte chunks per row and source
   constexpr int B_PER = B_CHUNKS / HALVES;
+  constexpr int B_KSTRIDE = NT / CPR;            // k rows between a thread's chunks
   static_assert(B_CHUNKS % HALVES == 0, "B chunks must split over the sources");
+  static_assert(NT % CPR == 0, "a thread's B chunks must share their column");
   const uint16_t* b_base[HALVES];
   b_base[0] = Bb + n_begin;
   if constexpr (SWIGLU) b_base[1] = B2b + n_begin;
-  uint32_t b_off[B_CHUNKS], b_lds[B_CHUNKS];
-  int b_krow[B_CHUNKS];
-#pragma unroll
-  for (int q = 0; q < B_CHUNKS; ++q) {
-    const int half = q / B_PER;
-    const int v = tid + NT * (q % B_PER);
-    const int krow = v / CPR;
-    const int nch = v % CPR;
-    int col = nch * 8;
-    col = n_begin + col < p.N ? col : p.N - 8 - n_begin;    // clamp: columns past the edge are never stored
-    b_off[q] = ((uint32_t)krow * (uint32_t)p.ldb + col) * 2;
-    b_lds[q] = S::kAStage + krow * S::kBPitch + (half * CPR + nch) * 16;
-    b_krow[q] = krow;
-  }
+  const int b_krow0 = tid / CPR, b_nch = tid % CPR;
+  int b_col0 = b_nch * 8;
+  b_col0 = n_begin + b_col0 < p.N ? b_col0 : p.N - 8 - n_begin;   // clamp: columns past the edge are never stored
+  const uint32_t b_off0 = ((uint32_t)b_krow0 * (uint32_t)p.ldb + b_col0) * 2;
+  const uint32_t b_lds0 = S::kAStage + b_krow0 * S::kBPitch + b_nch * 16;
+  auto b_krow = [&](int qb) { return b_krow0 + (qb % B_PER) * B_KSTRIDE; };
+  auto b_lds = [&](int qb) { return b_lds0 + (qb % B_PER) * B_KSTRIDE * S::kBPitch + (qb / B_PER) * CPR * 16; };
 
   // ---- staging registers ------------------------------------------------------
   // st[q] holds one 16-byte chunk on its way from global memory to LDS:
@@ -209,7 +238,7 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
   // split into KS groups; a group is written to LDS and immediately refilled with
   // the same chunks of the K step two ahead, so every global load has a full K
   // step of MFMA time to land and loads / LDS writes are spread evenly over it.
-  constexpr int KS = G16_BK / 16;
+  constexpr int KS = G16_BK / KD;                // MFMA k steps per K step
   constexpr int NC = A_CHUNKS + B_CHUNKS;
   constexpr int CPG = (NC + KS - 1) / KS;       // (the last group is short when KS does not divide NC)
   uint4 st[NC];
@@ -226,16 +255,16 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
       return buffer_load_b128(a_base + k0, off);
     } else {
       const int qb = q - A_CHUNKS;
-      uint32_t off = b_off[qb];
-      if constexpr (GUARD) off = (k0 + b_krow[qb] < K) ? off : kOutOfRange;
-      return buffer_load_b128(b_base[qb / B_PER] + (long)k0 * p.ldb, off);
+      uint32_t off = b_off0;
+      if constexpr (GUARD) off = (k0 + b_krow(qb) < K) ? off : kOutOfRange;
+      return buffer_load_b128(b_base[qb / B_PER] + (long)(k0 + (qb % B_PER) * B_KSTRIDE) * p.ldb, off);
     }
   };
   auto gload1 = [&](int q, int k0, auto guarded_c) { st[q] = gfetch(q, k0, guarded_c); };
   auto lstore1 = [&](int q, int buf) {
     char* base = smem + buf * S::kStage;
-    if (q < A_CHUNKS) lds_write_b128(base, a_lds[q], st[q]);
-    else lds_write_b128(base, b_lds[q - A_CHUNKS], st[q]);
+    if (q < A_CHUNKS) lds_write_b128(base, a_lds(q), st[q]);
+    else lds_write_b128(base, b_lds(q - A_CHUNKS), st[q]);
   };
   // Group g: write its chunks (K step `write` done by the caller's choice of
   // buffer) and refill them.  MODE 0 = no refill, 1 = full step, 2 = guarded.
@@ -252,33 +281,25 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
   };
 
   // ---- operand read addressing --------------------------------------------
-  const int l32 = lane & 31, lh = lane >> 5;
   uint32_t a_rd[MI];       // byte offset of this lane's row; chunk applied per k step
   int a_sw[MI];
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
-    const int row = wm * TM + i * 32 + l32;
+    const int row = wm * TM + i * MS + lm;
     a_rd[i] = row * G16_APITCH;
     a_sw[i] = g16_aswz(row);
   }
-  // transposing read: lane supplies row (k) = 8*lh + r/4 (+4 for the second
-  // half), columns n = 32j + 16*((lane>>4)&1) + 4*(r%4), r = lane & 15.
+  // transposing read: lane supplies row (k) = 8*lk + r/4 (+4 for the second half), columns
+  // n = MS j + 16*((lane % MS) >> 4) + 4*(r%4), r = lane & 15.
   const int r16 = lane & 15;
-  const uint32_t b_rd0 = S::kAStage + (8 * lh + (r16 >> 2)) * S::kBPitch +
-                         (wn * (SWIGLU ? TN / 2 : TN) + 16 * ((lane >> 4) & 1) + 4 * (r16 & 3)) * 2;
+  const uint32_t b_rd0 = S::kAStage + (8 * lk + (r16 >> 2)) * S::kBPitch +
+                         (wn * (SWIGLU ? TN / 2 : TN) + 16 * (lm >> 4) + 4 * (r16 & 3)) * 2;
   // byte offset of the wave's j-th column tile inside its B rows (SwiGLU: the up
   // columns start BN/2 columns after the gate columns)
   auto b_col = [](int j) constexpr -> int {
-    return (SWIGLU && j >= NJ / 2) ? (BN / 2 + (j - NJ / 2) * 32) * 2 : j * 64;
+    return (SWIGLU && j >= NJ / 2) ? (BN / 2 + (j - NJ / 2) * MS) * 2 : j * MS * 2;
   };
 
-  f32x16 acc[MI][NJ];
-#pragma unroll
-  for (int i = 0; i < MI; ++i)
-#pragma unroll
-    for (int j = 0; j < NJ; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   // Operand fragments are double buffered in registers: the LDS reads of k
   // step s+1 are issued before the MFMAs of step s, which hide their latency.
@@ -287,10 +308,10 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
     const char* base = smem + buf * S::kStage;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
-      af[slot][i] = lds_read_b128(base, a_rd[i] + ((((ks << 1) | lh) ^ a_sw[i]) << 4));
+      af[slot][i] = lds_read_b128(base, a_rd[i] + (((ks * (KD / 8) + lk) ^ a_sw[i]) << 4));
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      const char* pb = base + b_rd0 + ks * 16 * S::kBPitch + b_col(j);
+      const char* pb = base + b_rd0 + ks * KD * S::kBPitch + b_col(j);
       const uint2 lo = lds_read_tr16_b64(pb);
       const uint2 hi = lds_read_tr16_b64(pb + 4 * S::kBPitch);
       bf[slot][j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
@@ -300,7 +321,10 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) acc[i][j] = mfma_32x32x16<T>(bf[slot][j], af[slot][i], acc[i][j]);
+      for (int j = 0; j < NJ; ++j) {
+        if constexpr (MS == 32) acc[i][j] = mfma_32x32x16<T>(bf[slot][j], af[slot][i], acc[i][j]);
+        else acc[i][j] = mfma_16x16x32<T>(bf[slot][j], af[slot][i], acc[i][j]);
+      }
   };
   // Scheduling hint for one k step of NM MFMAs that carries RD operand reads and
   // (when `stream`) CPG LDS writes + CPG global loads.  The writes cannot pass
@@ -388,27 +412,111 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
     if constexpr (HAS1) hint_step(std::integral_constant<bool, (L2 != 0)>{}, std::integral_constant<bool, (L3 != 0)>{});
     __builtin_amdgcn_sched_barrier(0);
   };
+  // The 16-wide MFMA form has twice the operand fragments per k step (8 + 8 of them for a
+  // 128 x 128 wave tile).  Double-buffering both sets would not fit the 256 ordinary registers
+  // next to the staging registers, so only the B fragments are: the step walks the wave tile
+  // row by row, and as soon as a row's MFMAs are issued its A fragment register takes the
+  // same row's fragment of the next k step; the next B fragments, the LDS writes and the
+  // global loads of the step are dealt out over the rows in the same way.
+  auto a_frag = [&](int buf, int ks, int i) __attribute__((always_inline)) -> uint4 {
+    return lds_read_b128(smem + buf * S::kStage, a_rd[i] + (((ks * (KD / 8) + lk) ^ a_sw[i]) << 4));
+  };
+  auto b_frag = [&](int buf, int ks, int j) __attribute__((always_inline)) -> uint4 {
+    const char* pb = smem + buf * S::kStage + b_rd0 + ks * KD * S::kBPitch + b_col(j);
+    const uint2 lo = lds_read_tr16_b64(pb);
+    const uint2 hi = lds_read_tr16_b64(pb + 4 * S::kBPitch);
+    return make_uint4(lo.x, lo.y, hi.x, hi.y);
+  };
+  auto kstep16 = [&](int kt, auto has1_c, auto l2_c, auto l3_c) __attribute__((always_inline)) {
+    constexpr bool HAS1 = decltype(has1_c)::value;
+    constexpr int L2 = decltype(l2_c)::value;
+    constexpr int L3 = decltype(l3_c)::value;
+    static_assert(MS != 16 || KS == 2, "two MFMA k steps per K step");
+    const int buf = kt & 1;
+    // one row of the wave tile: its MFMAs, then the row's share of the fragment reads for
+    // the next k step and of the chunk group `g` (written to LDS buffer `wbuf`, refilled from
+    // K offset k0_load in mode `mode_c`)
+    auto row = [&](int slot, int i, bool next_frags, int fbuf, int fks, auto stream_c, int g, int wbuf, int k0_load,
+                   auto mode_c) __attribute__((always_inline)) {
+      constexpr bool STREAM = decltype(stream_c)::value;
+      constexpr int MODE = decltype(mode_c)::value;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        if constexpr (MS == 16) acc[i][j] = mfma_16x16x32<T>(bf[slot][j], af[0][i], acc[i][j]);
+      }
+      int reads = 0, writes = 0;
+      if (next_frags) {
+        af[0][i] = a_frag(fbuf, fks, i);
+        ++reads;
+#pragma unroll
+        for (int j = i * NJ / MI; j < (i + 1) * NJ / MI; ++j) {
+          bf[slot ^ 1][j] = b_frag(fbuf, fks, j);
+          reads += 2;
+        }
+      }
+      if constexpr (STREAM) {
+#pragma unroll
+        for (int q = g * CPG + i * CPG / MI; q < g * CPG + (i + 1) * CPG / MI; ++q) {
+          if (q < NC) {
+            lstore1(q, wbuf);
+            if constexpr (MODE == 1) gload1(q, k0_load, false_type{});
+            if constexpr (MODE == 2) gload1(q, k0_load, true_type{});
+            ++writes;
+          }
+        }
+      }
+      // every memory instruction in the shadow of an MFMA of its row
+#pragma unroll
+      for (int x = 0; x < NJ; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (x < reads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        else if (x - reads < writes) {
+          __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+          if constexpr (MODE != 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // first k step of the K step (fragments in hand); the second's come from the same buffer,
+    // and chunk group 1 of K step kt+1 goes to the other buffer
+#pragma unroll
+    for (int i = 0; i < MI; ++i) row(0, i, true, buf, 1, std::integral_constant<bool, HAS1>{}, 1, buf ^ 1, (kt + 2) * G16_BK, l2_c);
+    // Every wave has issued all its reads of this buffer and all its writes of the other one;
+    // past the barrier the other buffer is complete and this one is free to take group 0 of
+    // step kt+2.
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < MI; ++i) row(1, i, HAS1, buf ^ 1, 0, std::integral_constant<bool, (L2 != 0)>{}, 0, buf, (kt + 3) * G16_BK, l3_c);
+  };
+  auto kstep_any = [&](int kt, auto has1_c, auto l2_c, auto l3_c) __attribute__((always_inline)) {
+    if constexpr (MS == 16) kstep16(kt, has1_c, l2_c, l3_c);
+    else kstep(kt, has1_c, l2_c, l3_c);
+  };
   int kt = 0;
-  for (; kt + 4 < ktiles; ++kt) kstep(kt, true_type{}, mode1{}, mode1{});
-  if (kt + 3 < ktiles) { kstep(kt, true_type{}, mode1{}, mode2{}); ++kt; }
-  if (kt + 2 < ktiles) { kstep(kt, true_type{}, mode2{}, mode0{}); ++kt; }
-  if (kt + 1 < ktiles) { kstep(kt, true_type{}, mode0{}, mode0{}); ++kt; }
-  kstep(kt, false_type{}, mode0{}, mode0{});
+  for (; kt + 4 < ktiles; ++kt) kstep_any(kt, true_type{}, mode1{}, mode1{});
+  if (kt + 3 < ktiles) { kstep_any(kt, true_type{}, mode1{}, mode2{}); ++kt; }
+  if (kt + 2 < ktiles) { kstep_any(kt, true_type{}, mode2{}, mode0{}); ++kt; }
+  if (kt + 1 < ktiles) { kstep_any(kt, true_type{}, mode0{}, mode0{}); ++kt; }
+  kstep_any(kt, false_type{}, mode0{}, mode0{});
+  }  // !DL
 
   // ---- epilogue -------------------------------------------------------------
-  // acc[i][j][r]: row m = 32i + l32, col n = 32j + 8*(r/4) + 4*lh + (r%4): a lane owns
-  // runs of four columns of 32 different rows.  Stored like that, every store
+  // acc[i][j][r]: row m = MS i + lm, col n = MS j + 8*(r/4) + 4*lk + (r%4): a lane owns
+  // runs of four columns of MS different rows.  Stored like that, every store
   // instruction would touch 32 cache lines with 16 bytes each, and the output write
   // would cost a tenth of a long-K product and half of a short-K one.  The wave
   // therefore stages its tile through its share of the (now free) LDS and writes
   // whole row segments: 16 bytes per lane, consecutive lanes along a row.
   constexpr int NJ_OUT = SWIGLU ? NJ / 2 : NJ;
-  constexpr int ROWB = NJ_OUT * 32 * DSZ;              // bytes of one row of the wave's output tile
+  constexpr int ROWB = NJ_OUT * MS * DSZ;              // bytes of one row of the wave's output tile
   constexpr int PITCH = ROWB + 16;
   constexpr int WAVE_LDS = S::kBytes / (WM * WN);
+  constexpr int MB = TM / 32;                          // 32-row blocks of the wave's tile
   constexpr int IB_FIT = WAVE_LDS / (32 * PITCH);      // 32-row blocks that fit the wave's share
-  constexpr int IB = IB_FIT >= MI ? MI : (IB_FIT >= 2 ? 2 : 1);
-  static_assert(IB_FIT >= 1 && MI % IB == 0, "epilogue staging does not fit");
+  constexpr int IB = IB_FIT >= MB ? MB : (IB_FIT >= 2 ? 2 : 1);
+  static_assert(IB_FIT >= 1 && MB % IB == 0, "epilogue staging does not fit");
+  constexpr int TPB = 32 / MS;                         // MFMA tiles per 32-row block
+  constexpr int QG = AE / 4;                           // runs of four columns per MFMA tile
   constexpr int LPR = ROWB / 16;                       // lanes per row
   constexpr int RPI = 64 / LPR;                        // rows per store instruction
   static_assert(LPR <= 64 && (IB * 32) % RPI == 0, "epilogue row mapping");
@@ -427,15 +535,15 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
     constexpr int ACT = decltype(act_c)::value;
     constexpr bool HAS_BIAS = decltype(bias_c)::value;
 #pragma unroll
-    for (int i0 = 0; i0 < MI; i0 += IB) {
+    for (int b0 = 0; b0 < MB; b0 += IB) {
 #pragma unroll
-      for (int ii = 0; ii < IB; ++ii) {
-        const int i = i0 + ii;
+      for (int ii = 0; ii < IB * TPB; ++ii) {
+        const int i = b0 * TPB + ii;
 #pragma unroll
         for (int j = 0; j < NJ_OUT; ++j) {
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int n = nw0 + j * 32 + q * 8 + lh * 4;
+          for (int q = 0; q < QG; ++q) {
+            const int n = nw0 + j * MS + q * 8 + lk * 4;
             float v0 = acc[i][j][q * 4 + 0], v1 = acc[i][j][q * 4 + 1];
             float v2 = acc[i][j][q * 4 + 2], v3 = acc[i][j][q * 4 + 3];
             if constexpr (EPI == EPI_F32_FUSED) {
@@ -448,16 +556,16 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
               v2 = activate_as<ACT>(v2); v3 = activate_as<ACT>(v3);
             }
             if constexpr (EPI == EPI_GATED_F32) {
-              const f32x16& u = acc[i][j + NJ / 2];
+              const acc_t& u = acc[i][j + NJ / 2];
               v0 = activate_as<ACT>(v0) * u[q * 4 + 0]; v1 = activate_as<ACT>(v1) * u[q * 4 + 1];
               v2 = activate_as<ACT>(v2) * u[q * 4 + 2]; v3 = activate_as<ACT>(v3) * u[q * 4 + 3];
             }
-            char* dst = stg + (ii * 32 + l32) * PITCH + (j * 32 + q * 8 + lh * 4) * DSZ;
+            char* dst = stg + (ii * MS + lm) * PITCH + (j * MS + q * 8 + lk * 4) * DSZ;
             if constexpr (DSZ == 4) {
               *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
             } else {
               if constexpr (EPI == EPI_SWIGLU16) {
-                const f32x16& u = acc[i][j + NJ / 2];
+                const acc_t& u = acc[i][j + NJ / 2];
                 float g[4] = {v0, v1, v2, v3};
                 float o[4];
 #pragma unroll
@@ -482,7 +590,7 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
       for (int it = 0; it < IB * 32 / RPI; ++it) {
         const int row = it * RPI + st_row;
         const uint4 v = lds_read_b128(stg, row * PITCH + st_chunk * 16);
-        const int m = m_begin + wm * TM + i0 * 32 + row;
+        const int m = m_begin + wm * TM + b0 * 32 + row;
         // N % 8 == 0 on this path: a 16-byte chunk is inside or outside as a whole
         if (m < m_end && st_n < p.N)
           *reinterpret_cast<uint4*>(Db + ((long)m * p.ldd + st_n) * DSZ) = v;
@@ -511,7 +619,7 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
   }
 }
 
-template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED>
+template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32, bool DL = false>
 __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Params p) {
   constexpr bool SWIGLU = (EPI == EPI_SWIGLU16 || EPI == EPI_GATED_F32);
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -607,11 +715,11 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     // share the columns of a 64-row tile instead: a quarter of the matrix work of the
     // full tile, whose other 192 rows would be computed and thrown away.
     if (m_end - m_begin <= 64) {
-      gemm16_tile<T, 64, BN, 1, 4, EPI, GROUPED>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db);
+      gemm16_tile<T, 64, BN, 1, 4, EPI, GROUPED, MS, DL>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db);
       return;
     }
   }
-  gemm16_tile<T, BM, BN, WM, WN, EPI, GROUPED>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db);
+  gemm16_tile<T, BM, BN, WM, WN, EPI, GROUPED, MS, DL>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db);
 }
 
 }  // namespace tsr950

@@ -61,12 +61,23 @@ __global__ void gemm16_grouped_generic_kernel(const Gemm16Params p) {
   else reinterpret_cast<uint16_t*>(p.D)[o] = to_storage<T>(acc);
 }
 
+// The 256 x 256 workgroup tiles use the 16-wide MFMA with operands loaded straight into LDS
+// (gemm16_dl.h); TSR_BIG_CLASSIC builds them on the register-staged 32-wide loop instead.
+#ifdef TSR_BIG_CLASSIC
+constexpr int kBigTileMfma = 32;
+constexpr bool kBigTileDirect = false;
+#else
+constexpr int kBigTileMfma = 16;
+constexpr bool kBigTileDirect = true;
+#endif
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED>
+template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32, bool DL = false>
 int launch_gemm16_tile(Gemm16Params p, hipStream_t s) {
   using S = Gemm16Smem<BM, BN>;
-  auto kern = gemm16_kernel<T, BM, BN, WM, WN, EPI, GROUPED>;
+  static_assert(!DL || Gemm16DlSmem<BM, BN>::kBytes <= S::kBytes, "the direct-load stages fit the same LDS window");
+  auto kern = gemm16_kernel<T, BM, BN, WM, WN, EPI, GROUPED, MS, DL>;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [&] {
@@ -203,9 +214,9 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
   }
   if (sch.tile == 256) {
     if constexpr (EPI == EPI_F32) {
-      if (fused) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI_F32_FUSED, false>(p, s);
+      if (fused) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI_F32_FUSED, false, kBigTileMfma, kBigTileDirect>(p, s);
     }
-    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false>(p, s);
+    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false, kBigTileMfma, kBigTileDirect>(p, s);
   }
   const bool t128 = sch.tile == 128;
   if (sch.skinny && sch.split_k == 1) return launch_gemm16_skinny<T, EPI>(p, p.K, 1, s);
