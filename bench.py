@@ -513,8 +513,9 @@ def bench_moe(lane, steps, warmup, check=True):
 
 def mfma_ceiling(lane, seconds=2.0, kind="bf16"):
     """The rate a register-only loop of independent matrix instructions reaches on this board
-    (tessera_gfx950_mfma_probe_dev: no memory access inside the loop; 32x32x16 bf16, 32x32x32
-    int8 or 32x32x64 fp8), on operands distributed like the workload's and on constant ones,
+    (tessera_gfx950_mfma_probe_dev: no memory access inside the loop; 16x16x32 bf16 -- the
+    instruction of the 256 x 256 GEMM tile --, 32x32x16 bf16 ("bf16_32x32x16": attention and the
+    MoE block), 32x32x32 int8 or 32x32x64 fp8), on operands distributed like the workload's and on constant ones,
     with the shader clock and socket power sampled while it runs.  The matrix pipes draw more
     power on toggling operands, the board holds its power limit by lowering the clock, and the
     published peak assumes PEAK_CLOCK_MHZ: the random-operand figure is the ceiling a GEMM on
@@ -524,11 +525,11 @@ def mfma_ceiling(lane, seconds=2.0, kind="bf16"):
     lib = lane.load()
     rng = np.random.default_rng(7)
     nbytes = 16 * 8 * 64 * 16                               # the probe's fragment buffer
-    code = {"bf16": 0, "int8": 1, "fp8": 2}[kind]
+    code = {"bf16": 3, "bf16_32x32x16": 0, "int8": 1, "fp8": 2}[kind]
     sink = lane.DeviceBuffer(1024 * 256 * 4)
     ops = ctypes.c_double(0.0)
-    rounds = 600 if kind == "bf16" else 300
-    if kind == "bf16":
+    rounds = 300 if kind == "bf16" else 600 if kind == "bf16_32x32x16" else 300
+    if kind.startswith("bf16"):
         random_frags = lane.DeviceBuffer.from_host(_bf16(rng.standard_normal(nbytes // 2, dtype=np.float32) / np.sqrt(8192.0)))
         constant = np.full(nbytes // 2, 0x3C3C, np.uint16)
     else:
@@ -824,7 +825,7 @@ def main() -> int:
     if args.only:
         if args.only == "mfma_ceiling":
             print(json.dumps({"mfma_ceiling": {k: mfma_ceiling(lane, 0.0 if args.no_clock else 2.0, k)
-                                                for k in ("bf16", "int8", "fp8")}}))
+                                                for k in ("bf16", "bf16_32x32x16", "int8", "fp8")}}))
         else:
             print(json.dumps(run_also(lane, args.only, args.steps, args.warmup, not args.no_cpu)))
         return 0
@@ -843,7 +844,7 @@ def main() -> int:
                      "frac": flop / ev / 1e9 / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BYTES_GEMM_BF16_8192,
                      "traffic_source": "profiles/bench_all_kernels_hbm_bytes.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an "
                                        "earlier run, scaled by the copy kernel's readings; not measured by this run)",
-                     "kernel": "gemm16_kernel<BF16,256,256,2,2,STORE16>", "avg_launch_ms": ev},
+                     "kernel": "gemm16_kernel<BF16,256,256,2,2,STORE16,mfma 16x16x32,direct-to-LDS>", "avg_launch_ms": ev},
     }
     if copy_cal:
         result["copy_calibration"] = copy_cal

@@ -211,8 +211,10 @@ int tessera_gfx950_mfma_probe_bf16_dev(const void* fragments, int rounds, void* 
 /* The same probe for the other matrix instructions of the lane: kind 0 = 32x32x16 bf16 (the
  * call above), 1 = 32x32x32 int8 (int32 accumulate; the fragments are int8 values), 2 =
  * 32x32x64 fp8 e4m3 in its unscaled form (the fragments are e4m3 codes; a 32-byte operand is
- * two neighbouring 16-byte fragments).  *ops receives the operations of one launch
- * (2 * 32 * 32 * k per instruction).  No counterpart in the reference. */
+ * two neighbouring 16-byte fragments), 3 = 16x16x32 bf16 (the instruction of the 256 x 256
+ * GEMM tile; a quarter of the accumulator registers per instruction, 64 accumulators and
+ * MFMAs per round).  *ops receives the operations of one launch (2 * m * n * k per
+ * instruction).  No counterpart in the reference. */
 int tessera_gfx950_mfma_probe_dev(int kind, const void* fragments, int rounds, void* sink, double* ops, void* stream);
 
 /* ---- quantisers ------------------------------------------------------------ */

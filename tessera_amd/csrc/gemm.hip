@@ -61,13 +61,13 @@ int gemm16_host(const void* A, const void* B, void* D, int batch, int M, int N, 
   return scope.download(D, dD, d_bytes) ? kOk : kDeviceFailed;
 }
 
-// Register-only MFMA rate probe: every wave keeps 16 independent 32x32x16 bf16
-// accumulators (4 A fragments x 4 B fragments, fetched once) and issues `rounds` rounds of
-// those 16 MFMAs with no memory access in the loop: the rate the matrix pipes reach on
-// the given operand values at the clock the board grants for them.
+// Register-only MFMA rate probe: every wave keeps the accumulators of a 128 x 128 tile (4 A
+// fragments x 4 B fragments, fetched once) and issues `rounds` rounds of one MFMA per
+// accumulator (16, or 64 of the 16 x 16 form) with no memory access in the loop: the rate the matrix pipes reach on the given operand values
+// at the clock the board grants for them.
 constexpr int kProbeBlocks = 1024;
 constexpr int kProbeThreads = 256;
-// KIND 0: 32x32x16 bf16; 1: 32x32x32 int8; 2: 32x32x64 fp8 (e4m3, unscaled form)
+// KIND 0: 32x32x16 bf16; 1: 32x32x32 int8; 2: 32x32x64 fp8 (e4m3, unscaled form); 3: 16x16x32 bf16
 template <int KIND>
 __global__ __launch_bounds__(kProbeThreads, 1) void mfma_probe_kernel(const uint4* __restrict__ frags, int rounds,
                                                                        float* __restrict__ sink) {
@@ -80,21 +80,26 @@ __global__ __launch_bounds__(kProbeThreads, 1) void mfma_probe_kernel(const uint
     a[f] = frags[(wave * 8 + f) * 64 + lane];
     b[f] = frags[(wave * 8 + 4 + f) * 64 + lane];
   }
-  using acc_t = std::conditional_t<KIND == 1, i32x16, f32x16>;
-  acc_t acc[4][4];
+  using acc_t = std::conditional_t<KIND == 1, i32x16, std::conditional_t<KIND == 3, f32x4, f32x16>>;
+  // the same 128 x 128 wave tile either way: 4 x 4 accumulators of 32 x 32, or 8 x 8 of 16 x 16
+  constexpr int AE = KIND == 3 ? 4 : 16;
+  constexpr int NI = KIND == 3 ? 8 : 4;
+  acc_t acc[NI][NI];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < NI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NI; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+      for (int r = 0; r < AE; ++r) acc[i][j][r] = 0;
   for (int it = 0; it < rounds; ++it) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < NI; ++j) {
         if constexpr (KIND == 0) {
           acc[i][j] = mfma_32x32x16<BF16>(a[i], b[j], acc[i][j]);
+        } else if constexpr (KIND == 3) {
+          acc[i][j] = mfma_16x16x32<BF16>(a[i & 3], b[j & 3], acc[i][j]);
         } else if constexpr (KIND == 1) {
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, a[i]),
                                                             __builtin_bit_cast(i32x4, b[j]), acc[i][j], 0, 0, 0);
@@ -110,11 +115,11 @@ __global__ __launch_bounds__(kProbeThreads, 1) void mfma_probe_kernel(const uint
   }
   float total = 0.f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < NI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NI; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) total += (float)acc[i][j][r];
+      for (int r = 0; r < AE; ++r) total += (float)acc[i][j][r];
   sink[(size_t)blockIdx.x * kProbeThreads + threadIdx.x] = total;
 }
 
@@ -369,16 +374,19 @@ int tessera_gfx950_gemm_bf16_bench_rotating(int M, int N, int K, int iters, int 
 int tessera_gfx950_bench_last_timer_source(void) { return g_last_timer_source; }
 
 int tessera_gfx950_mfma_probe_dev(int kind, const void* fragments, int rounds, void* sink, double* ops, void* stream) {
-  if (kind < 0 || kind > 2 || !fragments || !sink || rounds <= 0 || (reinterpret_cast<uintptr_t>(fragments) & 15))
+  if (kind < 0 || kind > 3 || !fragments || !sink || rounds <= 0 || (reinterpret_cast<uintptr_t>(fragments) & 15))
     return kBadShape;
-  const int depth = kind == 0 ? 16 : kind == 1 ? 32 : 64;     // k of one instruction
-  if (ops) *ops = (double)kProbeBlocks * (kProbeThreads / 64) * rounds * 16.0 * (2.0 * 32 * 32 * depth);
+  const int depth = kind == 0 ? 16 : kind == 1 ? 32 : kind == 2 ? 64 : 32;     // k of one instruction
+  const int side = kind == 3 ? 16 : 32;
+  const double per_round = kind == 3 ? 64.0 : 16.0;           // MFMAs per wave and round
+  if (ops) *ops = (double)kProbeBlocks * (kProbeThreads / 64) * rounds * per_round * (2.0 * side * side * depth);
   if (probe_device() != kOk) return kNoDevice;
   const dim3 grid(kProbeBlocks), block(kProbeThreads);
   const uint4* f = static_cast<const uint4*>(fragments);
   float* out = static_cast<float*>(sink);
   if (kind == 0) hipLaunchKernelGGL(mfma_probe_kernel<0>, grid, block, 0, as_stream(stream), f, rounds, out);
   else if (kind == 1) hipLaunchKernelGGL(mfma_probe_kernel<1>, grid, block, 0, as_stream(stream), f, rounds, out);
+  else if (kind == 3) hipLaunchKernelGGL(mfma_probe_kernel<3>, grid, block, 0, as_stream(stream), f, rounds, out);
   else hipLaunchKernelGGL(mfma_probe_kernel<2>, grid, block, 0, as_stream(stream), f, rounds, out);
   return launch_status();
 }

@@ -21,9 +21,10 @@
 // Pipeline (two LDS stages, one barrier per K step, KS = 2 MFMA k steps per K step).  The
 // barrier sits between the two k steps: before it every wave has read all fragments of the
 // current stage (those of the second k step are fetched during the first), after it the stage
-// is free and takes the loads of K step kt+2, which are dealt out over the rows of the next
-// two k steps and have a whole K step to land before the next barrier (s_waitcnt vmcnt(0)
-// just ahead of it).  The B fragments are double buffered in registers; the A fragment of a
+// is free and takes the loads of K step kt+2, which are dealt out over the rows of the k step
+// that follows the barrier and so have most of a K step to land before the next barrier
+// (s_waitcnt vmcnt(0) just ahead of it; loads issued in the k step before that barrier would
+// have no time left, and cost a quarter of the rate when tried).  The B fragments are double buffered in registers; the A fragment of a
 // row is replaced by the same row's fragment of the next k step as soon as the row's MFMAs
 // are issued.
 #pragma once
@@ -168,10 +169,7 @@ __device__ __forceinline__ void gemm16_mainloop_dl(const Params& p, char* smem, 
   // The loads of a K step go out over the SPREAD rows that follow the barrier which frees their
   // stage.  The stage is free for exactly one K step (2 MI rows), and what is issued late in
   // it has no time to land before the next barrier.
-#ifndef TSR_DL_SPREAD
-#define TSR_DL_SPREAD 8
-#endif
-  constexpr int SPREAD = TSR_DL_SPREAD < 2 * MI ? TSR_DL_SPREAD : 2 * MI;
+  constexpr int SPREAD = 8 < 2 * MI ? 8 : 2 * MI;
   constexpr int H_RAW = (MI * NL + SPREAD - 1) / SPREAD;
   constexpr int H = H_RAW < NL ? H_RAW : NL;    // loads that go out in the first of the two k steps (l SPREAD / NL < MI)
   // one row of the wave tile: its MFMAs, then its share of the fragment reads for the next
@@ -200,11 +198,7 @@ __device__ __forceinline__ void gemm16_mainloop_dl(const Params& p, char* smem, 
       // stage (rows MI and up are rows of the following k step)
 #pragma unroll
       for (int l = L0; l < L1; ++l)
-#ifndef TSR_DL_NOLOADS
         if (l * SPREAD / NL == i + (L0 == 0 ? 0 : MI)) load(l, lkt, lstage);
-#else
-        (void)lkt, (void)lstage;
-#endif
     }
     // the reads in the shadow of the row's first MFMAs
 #pragma unroll
@@ -242,9 +236,7 @@ __device__ __forceinline__ void gemm16_mainloop_dl(const Params& p, char* smem, 
     for (int i = 0; i < MI; ++i) row(0, i, yes{}, stage, 1, cH{}, cN{}, more1_c, kt + 1, stage ^ 1);
     // Every wave has read all it needs from this stage, and its own loads into the other one
     // have landed; past the barrier the other stage is complete and this one is free.
-#ifndef TSR_DL_NOWAIT
     wait_direct_loads();
-#endif
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < MI; ++i) row(1, i, has1_c, stage ^ 1, 0, c0{}, cH{}, has2_c, kt + 2, stage);
