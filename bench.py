@@ -844,7 +844,7 @@ def main() -> int:
                      "frac": flop / ev / 1e9 / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BYTES_GEMM_BF16_8192,
                      "traffic_source": "profiles/bench_all_kernels_hbm_bytes.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an "
                                        "earlier run, scaled by the copy kernel's readings; not measured by this run)",
-                     "kernel": "gemm16_kernel<BF16,256,256,2,2,STORE16,mfma 16x16x32,direct-to-LDS>", "avg_launch_ms": ev},
+                     "kernel": "gemm16_kernel<BF16,256,256,2,2,STORE16,mfma 16x16x32>", "avg_launch_ms": ev},
     }
     if copy_cal:
         result["copy_calibration"] = copy_cal

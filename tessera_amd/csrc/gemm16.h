@@ -155,10 +155,8 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
   // 16-wide form reads and writes half the accumulator data, and a register-only loop of it runs
   // 14 % faster under the board's power limit on random operands (2010 against 1760 TFLOP/s):
   // the big tiles, which sit on that limit, use it.
-  // The 16-wide form needs twice the operand fragments per k step, which do not fit the 256
-  // ordinary registers next to the registers that stage a K step: it comes with the main loop
-  // that loads straight into LDS (gemm16_dl.h).
-  static_assert((MS == 32 && !DL) || (MS == 16 && DL), "MFMA tile side / main loop pairs");
+  static_assert(MS == 32 || MS == 16, "MFMA tile side");
+  static_assert(!DL || MS == 16, "the direct-to-LDS main loop is written for the 16-wide MFMA");
   constexpr int KD = 512 / MS;                  // k per MFMA instruction
   constexpr int AE = MS * MS / 64;              // accumulator registers per MFMA tile
   constexpr int MI = TM / MS, NJ = TN / MS;     // MFMA tiles per wave
@@ -421,12 +419,96 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
     if constexpr (HAS1) hint_step(std::integral_constant<bool, (L2 != 0)>{}, std::integral_constant<bool, (L3 != 0)>{});
     __builtin_amdgcn_sched_barrier(0);
   };
+  // The 16-wide MFMA form has twice the operand fragments per k step (8 + 8 of them for a
+  // 128 x 128 wave tile).  Double-buffering both sets would not fit the 256 ordinary registers
+  // next to the staging registers, so only the B fragments are: the step walks the wave tile
+  // row by row, and as soon as a row's MFMAs are issued its A fragment register takes the
+  // same row's fragment of the next k step; the next B fragments, the LDS writes and the
+  // global loads of the step are dealt out over the rows in the same way.
+  auto a_frag = [&](int buf, int ks, int i) __attribute__((always_inline)) -> uint4 {
+    return lds_read_b128(smem + buf * S::kStage, a_rd[i] + (((ks * (KD / 8) + lk) ^ a_sw[i]) << 4));
+  };
+  auto b_frag = [&](int buf, int ks, int j) __attribute__((always_inline)) -> uint4 {
+    const char* pb = smem + buf * S::kStage + b_rd0 + ks * KD * S::kBPitch + b_col(j);
+    const uint2 lo = lds_read_tr16_b64(pb);
+    const uint2 hi = lds_read_tr16_b64(pb + 4 * S::kBPitch);
+    return make_uint4(lo.x, lo.y, hi.x, hi.y);
+  };
+  auto kstep16 = [&](int kt, auto has1_c, auto l2_c, auto l3_c) __attribute__((always_inline)) {
+    constexpr bool HAS1 = decltype(has1_c)::value;
+    constexpr int L2 = decltype(l2_c)::value;
+    constexpr int L3 = decltype(l3_c)::value;
+    static_assert(MS != 16 || KS == 2, "two MFMA k steps per K step");
+    const int buf = kt & 1;
+    // one row of the wave tile: its MFMAs, then the row's share of the fragment reads for
+    // the next k step and of the chunk group `g` (written to LDS buffer `wbuf`, refilled from
+    // K offset k0_load in mode `mode_c`)
+    auto row = [&](int slot, int i, bool next_frags, int fbuf, int fks, auto stream_c, int g, int wbuf, int k0_load,
+                   auto mode_c) __attribute__((always_inline)) {
+      constexpr bool STREAM = decltype(stream_c)::value;
+      constexpr int MODE = decltype(mode_c)::value;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        if constexpr (MS == 16) acc[i][j] = mfma_16x16x32<T>(bf[slot][j], af[0][i], acc[i][j]);
+      }
+      int reads = 0, writes = 0;
+      if (next_frags) {
+        af[0][i] = a_frag(fbuf, fks, i);
+        ++reads;
+#pragma unroll
+        for (int j = i * NJ / MI; j < (i + 1) * NJ / MI; ++j) {
+          bf[slot ^ 1][j] = b_frag(fbuf, fks, j);
+          reads += 2;
+        }
+      }
+      if constexpr (STREAM) {
+#pragma unroll
+        for (int q = g * CPG + i * CPG / MI; q < g * CPG + (i + 1) * CPG / MI; ++q) {
+          if (q < NC) {
+            lstore1(q, wbuf);
+            if constexpr (MODE == 1) gload1(q, k0_load, false_type{});
+            if constexpr (MODE == 2) gload1(q, k0_load, true_type{});
+            ++writes;
+          }
+        }
+      }
+      // every memory instruction in the shadow of an MFMA of its row
+#pragma unroll
+      for (int x = 0; x < NJ; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (x < reads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        else if (x - reads < writes) {
+          __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+          if constexpr (MODE != 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // first k step of the K step (fragments in hand); the second's come from the same buffer,
+    // and chunk group 1 of K step kt+1 goes to the other buffer
+#pragma unroll
+    for (int i = 0; i < MI; ++i) row(0, i, true, buf, 1, std::integral_constant<bool, HAS1>{}, 1, buf ^ 1, (kt + 2) * G16_BK, l2_c);
+    // Every wave has issued all its reads of this buffer and all its writes of the other one;
+    // past the barrier the other buffer is complete and this one is free to take group 0 of
+    // step kt+2.
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < MI; ++i) row(1, i, HAS1, buf ^ 1, 0, std::integral_constant<bool, (L2 != 0)>{}, 0, buf, (kt + 3) * G16_BK, l3_c);
+  };
+  auto kstep_any = [&](int kt, auto has1_c, auto l2_c, auto l3_c) __attribute__((always_inline)) {
+    if constexpr (MS == 16) kstep16(kt, has1_c, l2_c, l3_c);
+    else kstep(kt, has1_c, l2_c, l3_c);
+  };
   int kt = 0;
-  for (; kt + 4 < ktiles; ++kt) kstep(kt, true_type{}, mode1{}, mode1{});
-  if (kt + 3 < ktiles) { kstep(kt, true_type{}, mode1{}, mode2{}); ++kt; }
-  if (kt + 2 < ktiles) { kstep(kt, true_type{}, mode2{}, mode0{}); ++kt; }
-  if (kt + 1 < ktiles) { kstep(kt, true_type{}, mode0{}, mode0{}); ++kt; }
-  kstep(kt, false_type{}, mode0{}, mode0{});
+  // The first K step stands outside the loop: its MFMAs start from the zero accumulators, and
+  // with the loop entered directly the compiler rotates the 16-wide form's accumulators through
+  // ordinary registers (hundreds of register moves per K step) instead of updating them in place.
+  if (ktiles > 4) { kstep_any(0, true_type{}, mode1{}, mode1{}); kt = 1; }
+  for (; kt + 4 < ktiles; ++kt) kstep_any(kt, true_type{}, mode1{}, mode1{});
+  if (kt + 3 < ktiles) { kstep_any(kt, true_type{}, mode1{}, mode2{}); ++kt; }
+  if (kt + 2 < ktiles) { kstep_any(kt, true_type{}, mode2{}, mode0{}); ++kt; }
+  if (kt + 1 < ktiles) { kstep_any(kt, true_type{}, mode0{}, mode0{}); ++kt; }
+  kstep_any(kt, false_type{}, mode0{}, mode0{});
   }  // !DL
 
   // ---- epilogue -------------------------------------------------------------

@@ -61,14 +61,24 @@ __global__ void gemm16_grouped_generic_kernel(const Gemm16Params p) {
   else reinterpret_cast<uint16_t*>(p.D)[o] = to_storage<T>(acc);
 }
 
-// The 256 x 256 workgroup tiles use the 16-wide MFMA with operands loaded straight into LDS
-// (gemm16_dl.h); TSR_BIG_CLASSIC builds them on the register-staged 32-wide loop instead.
-#ifdef TSR_BIG_CLASSIC
+// The 256 x 256 workgroup tiles use the 16-wide MFMA in the register-staged main loop.
+// TSR_BIG_CLASSIC builds them on the 32-wide MFMA, TSR_BIG_DIRECT on the 16-wide one with
+// operands loaded straight into LDS (gemm16_dl.h): the two forms this one was measured against.
+#if defined(TSR_BIG_CLASSIC)
 constexpr int kBigTileMfma = 32;
 constexpr bool kBigTileDirect = false;
-#else
+#elif defined(TSR_BIG_DIRECT)
 constexpr int kBigTileMfma = 16;
 constexpr bool kBigTileDirect = true;
+#else
+constexpr int kBigTileMfma = 16;
+constexpr bool kBigTileDirect = false;
+#endif
+// The grouped (per-expert) 256 x 256 tiles likewise; TSR_GROUPED_CLASSIC keeps them 32-wide.
+#ifdef TSR_GROUPED_CLASSIC
+constexpr int kGroupedTileMfma = 32;
+#else
+constexpr int kGroupedTileMfma = 16;
 #endif
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -295,9 +305,9 @@ int launch_gemm16_grouped(Gemm16Params p, hipStream_t s) {
     return launch_status();
   }
   if constexpr (EPI == EPI_SWIGLU16) {
-    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true>(p, s);
+    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true, kGroupedTileMfma, false>(p, s);
   } else {
-    if ((long)p.M >= 64L * p.groups) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true>(p, s);
+    if ((long)p.M >= 64L * p.groups) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true, kGroupedTileMfma, false>(p, s);
     return launch_gemm16_tile<T, 128, 128, 2, 2, EPI, true>(p, s);
   }
 }

@@ -69,7 +69,7 @@ MFMA_BY_DTYPE = {
 
 KERNEL_TABLE: tuple = (
     KernelEntry("tessera.matmul", ("tile.matmul", "tile.mma"), "tessera_rocm.mfma_gemm", "m32n32k16",
-                "v_mfma_f32_32x32x16_{f16,bf16}; the 256x256 tile: v_mfma_f32_16x16x32_{f16,bf16}", ("f16", "bf16"),
+                "v_mfma_f32_16x16x32_{f16,bf16} (256x256 tiles); v_mfma_f32_32x32x16_{f16,bf16} (smaller tiles)", ("f16", "bf16"),
                 ("tessera_gfx950_gemm_f16", "tessera_gfx950_gemm_bf16", "tessera_gfx950_gemm_f16_f16",
                  "tessera_gfx950_gemm_bf16_bf16", "tessera_gfx950_batched_gemm_f16",
                  "tessera_gfx950_batched_gemm_bf16"),
