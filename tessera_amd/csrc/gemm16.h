@@ -9,12 +9,14 @@
 // budget — which needs 512 B of LDS operand reads per 32 MFMA cycles, half of the
 // 128 B/clk the LDS sustains.
 //
-// Two main loops share the tile body (addressing of the output, epilogues, the grouped and
-// SwiGLU forms).  The one in this file runs v_mfma_f32_32x32x16_{bf16,f16} and stages a K
-// step in registers on its way from global memory to LDS; it serves every tile shape.  The
-// dense 256x256 tile runs v_mfma_f32_16x16x32 with operands loaded straight into LDS
-// (gemm16_dl.h), which is the faster of the two on operands that toggle the matrix pipes.
-// What follows describes the register-staged loop.
+// The main loop stages a K step in registers on its way from global memory to LDS and comes
+// in two MFMA forms (template parameter MS): v_mfma_f32_32x32x16_{bf16,f16} (4 x 4 tiles per
+// wave) and v_mfma_f32_16x16x32 (8 x 8 tiles).  The 256x256 tiles run the 16-wide form, which
+// spends less power per FLOP: on operands that toggle the matrix pipes the board then grants
+// a higher clock.  A second main loop that loads operands straight into LDS (gemm16_dl.h,
+// DL = true) is the form this one was measured against; it is kept behind a build switch.
+// What follows describes the 32-wide step; the 16-wide one (kstep16) differs in how the
+// fragment reads are dealt out, see there.
 //
 // The tile body is a device function (gemm16_tile); the grouped kernel also holds a
 // 64 x BN instantiation of it with the four waves side by side along the columns, used

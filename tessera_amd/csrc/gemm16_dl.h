@@ -1,12 +1,11 @@
 // Main loop of the 16-bit GEMM tile on v_mfma_f32_16x16x32 with operands loaded from
 // global memory STRAIGHT INTO LDS (buffer_load ... lds, 16 bytes per lane).
 //
-// Why a second main loop.  Per FLOP the 16x16x32 MFMA moves half the accumulator data of the
-// 32x32x16 one through the register file, and a register-only loop of it runs 14 % faster
-// under the board's power limit on random operands.  It needs twice the operand fragments per
-// k step, though, and next to the 64 registers that stage a K step on its way from global
-// memory to LDS they do not fit the 256 ordinary registers of a wave.  Loading straight into
-// LDS takes the staging registers (and the LDS write instructions) away.
+// An alternative to the register-staged 16-wide step of gemm16.h, selected at build time
+// (TSR_BIG_DIRECT): no staging registers and no LDS write instructions.  It spends less power
+// per FLOP than the 32-wide staged loop and beat it by 5-6 % on random operands, but a stage
+// is free for exactly one K step, so its loads have at most that long to land, the matrix
+// pipes idle a third of the time, and the staged 16-wide step measures 2 % faster still.
 //
 // LDS stage = A tile [BM][64] 16-bit (128-byte rows, 16-byte chunks XOR-swizzled by
 // (row >> 1) & 7, as in the register-staged loop) + B tile(s) [64][cols] in natural row-major
