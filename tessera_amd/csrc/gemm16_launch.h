@@ -287,7 +287,7 @@ int launch_gemm16_gated(Gemm16Params p, hipStream_t s) {
     hipLaunchKernelGGL((gemm16_generic_kernel<T, EPI_GATED_F32>), grid, block, 0, s, p);
     return launch_status();
   }
-  return launch_gemm16_tile<T, 256, 256, 4, 1, EPI_GATED_F32, false>(p, s);
+  return launch_gemm16_tile<T, 256, 256, 4, 1, EPI_GATED_F32, false, kBigTileMfma, false>(p, s);
 }
 
 // Grouped.  p.M = total rows S, p.groups = E, p.offsets = device int32[E+1].
