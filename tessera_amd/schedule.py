@@ -86,6 +86,8 @@ def select_gfx950_gemm_schedule(m: int, n: int, k: int, *, dtype: str = "bf16", 
         int(m), int(n), int(k), int(batch), nbytes, ctypes.byref(tm), ctypes.byref(tn), ctypes.byref(tk),
         ctypes.byref(sk)), "gemm_schedule")
     inst = _INSTRUCTION_TILE[name]
+    if name in ("f16", "bf16") and tm.value == 256:
+        inst = (16, 16, 32)       # the 256 x 256 tiles run v_mfma_f32_16x16x32 (less power per FLOP)
     return Gfx950ScheduleDescriptor(
         arch="gfx950", dtype=name, instruction_tile=inst,
         macro_tile=(tm.value // inst[0], tn.value // inst[1]),

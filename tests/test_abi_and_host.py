@@ -297,8 +297,8 @@ def test_gemm_schedule_query_needs_no_device():
     """The schedule descriptor reads the launcher's own tile / split-K decision."""
     from tessera_amd.schedule import select_gfx950_gemm_schedule as sel
     big = sel(8192, 8192, 8192, dtype="bf16")
-    assert big.workgroup_tile == (256, 256, 64) and big.macro_tile == (8, 8) and big.split_k == 1
-    assert big.instruction_tile == (32, 32, 16) and big.target_ir_attrs()["schedule_arch"] == "gfx950"
+    assert big.workgroup_tile == (256, 256, 64) and big.macro_tile == (16, 16) and big.split_k == 1
+    assert big.instruction_tile == (16, 16, 32) and big.target_ir_attrs()["schedule_arch"] == "gfx950"
     dec = sel(4, 8192, 8192, dtype="bf16")                              # a few rows: the streaming kernel
     assert dec.workgroup_tile == (32, 64, 32) and dec.split_k == 2 and dec.waves_per_cu == 8
     assert sel(4, 32768, 8192).split_k == 1                             # enough column strips to fill the chip

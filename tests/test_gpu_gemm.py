@@ -63,6 +63,27 @@ def test_gemm_storage_out(lane, M, N, K, st):
     assert orc.max_rel_err(gf, ref) <= TOL + U_STORE[st]
 
 
+# The 256 x 256 tile (16-wide MFMA step: first K step peeled, main loop, peeled tails with and
+# without a guarded last step): every count of K steps from 1 to 6, whole and partial last
+# steps, K below one MFMA step, and row / column edges that leave part of a tile empty.
+BIG_TILE_EDGES = [(4096, 4096, k) for k in (8, 32, 40, 64, 72, 128, 136, 192, 200, 256, 264, 320, 328, 384)] + [
+    (4000, 3080, 264), (4096, 3072, 8), (3585, 3592, 1000), (8192, 2048, 520)]
+
+
+@pytest.mark.parametrize("M,N,K", BIG_TILE_EDGES)
+def test_big_tile_k_and_edge_shapes(lane, M, N, K):
+    from tessera_amd.schedule import select_gfx950_gemm_schedule
+    assert select_gfx950_gemm_schedule(M, N, K, dtype="bf16").workgroup_tile[:2] == (256, 256)
+    rng = np.random.default_rng(K * 7 + M)
+    a = b16.from_float32((rng.standard_normal((M, K)) * 0.5).astype(np.float32))
+    b = b16.from_float32((rng.standard_normal((K, N)) * 0.5).astype(np.float32))
+    ref = a.to_float32().astype(np.float64) @ b.to_float32().astype(np.float64)
+    acc = ops.gemm(a, b, out="f32")
+    assert orc.max_rel_err(acc, ref) <= 1e-5
+    stored = ops.gemm(a, b)
+    assert np.array_equal(np.asarray(stored).view(np.uint16), np.asarray(b16.from_float32(acc)).view(np.uint16))
+
+
 def test_readme_batched_gemm_config(lane):
     """A[4,128,64] f16 x W[4,64,256] f16 -> f32 accumulate (README step())."""
     rng = np.random.default_rng(0)
