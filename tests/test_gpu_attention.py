@@ -1,6 +1,6 @@
 """Flash-attention forward parity on the MI355X (through the C ABI) vs the oracle.
 
-Tolerances (written here as the north star states them): O max relative error
+Tolerances (as stated for this path): O max relative error
 <= 2e-3 normwise against an fp32-or-better reference of the same 16-bit inputs;
 LSE absolute error <= 2e-3.  The reference's own test budgets are looser
 (f16 2e-2, bf16 6e-2 absolute, tests/unit/test_rocm_flash_attn_runtime_symbol.py:90-132).

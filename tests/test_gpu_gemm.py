@@ -1,6 +1,6 @@
 """GEMM parity on the MI355X: HIP kernels (through the C ABI) vs the oracle.
 
-Tolerance: north-star bound max relative error <= 2e-3 for f16/bf16 against an
+Tolerance: the bound stated for this path is max relative error <= 2e-3 for f16/bf16 against an
 fp32-or-better reference (normwise: max|x-ref| / max|ref|).  The f32-output
 entry points are far inside it; the bound is binding for the 16-bit-output
 forms, whose final rounding alone is up to 2^-9 = 1.95e-3.
@@ -179,7 +179,7 @@ def test_full_size_bf16_gemm_properties(lane):
     lhs = float(got.astype(np.float64).sum())
     rhs = float(Aq.sum(axis=0) @ Bq.sum(axis=1))
     assert abs(lhs - rhs) <= 1e-6 * max(1.0, np.abs(Aq).sum(axis=0) @ np.abs(Bq).sum(axis=1))
-    # stored bf16 result within the north-star bound on the sampled rows
+    # stored bf16 result within that bound on the sampled rows
     stored = ops.gemm(ab, bb)
     assert np.array_equal(stored.to_float32(), orc.round_to_storage(got, "bf16"))
 
