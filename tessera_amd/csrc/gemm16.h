@@ -104,6 +104,7 @@ struct Gemm16Params {
 constexpr int G16_BK = 64;          // K step, elements
 constexpr int G16_APITCH = 128;     // bytes per A row in LDS
 constexpr int G16_BPAD = 32;        // B row pad, elements
+constexpr int kTailPace = 24;       // s_sleep units a paced short tile waits per K step
 // A-tile chunk swizzle: 16 consecutive rows of one chunk column hit 16 different
 // 16-byte slots of the 256-byte bank line.
 __device__ __forceinline__ int g16_aswz(int row) { return (row >> 1) & 7; }
@@ -149,7 +150,7 @@ namespace tsr950 {
 template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32, bool DL = false>
 __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, const int m_begin, const int m_end,
                                             const int tn, const uint16_t* Ab, const uint16_t* Bb,
-                                            const uint16_t* B2b, char* Db) {
+                                            const uint16_t* B2b, char* Db, const bool paced = false) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN;     // wave tile
   // MS: side of the MFMA tile.  32: v_mfma_f32_32x32x16 (16 accumulator registers per lane and
@@ -494,6 +495,14 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
     // past the barrier the other buffer is complete and this one is free to take group 0 of
     // step kt+2.
     __syncthreads();
+    // A short last row tile of a group issues a quarter of the MFMAs per K step and would run
+    // ahead of the full tiles of its column, which started with it on the same XCD: the weight
+    // panel they share would then pass through that XCD's L2 twice.  It waits here instead
+    // (kTailPace x 64 cycles per K step, about what the full tiles take longer), stays within
+    // reach of them, and the panel is fetched once.
+#ifndef TSR_NO_TAIL_PACE
+    if (paced) __builtin_amdgcn_s_sleep(kTailPace);
+#endif
 #pragma unroll
     for (int i = 0; i < MI; ++i) row(1, i, HAS1, buf ^ 1, 0, std::integral_constant<bool, (L2 != 0)>{}, 0, buf, (kt + 3) * G16_BK, l3_c);
   };
@@ -728,7 +737,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     // share the columns of a 64-row tile instead: a quarter of the matrix work of the
     // full tile, whose other 192 rows would be computed and thrown away.
     if (m_end - m_begin <= 64) {
-      gemm16_tile<T, 64, BN, 1, 4, EPI, GROUPED, MS, DL>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db);
+      // (paced when full tiles of the same group and column run beside it; 16-wide step only)
+      gemm16_tile<T, 64, BN, 1, 4, EPI, GROUPED, MS, DL>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db, MS == 16 && tm > 0);
       return;
     }
   }
