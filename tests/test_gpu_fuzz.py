@@ -53,6 +53,26 @@ def test_gemm_random_shapes(lane, seed):
         assert np.array_equal(np.asarray(stored).view(np.uint16), np.asarray(want).view(np.uint16)), (seed, M, N, K, st)
 
 
+@pytest.mark.parametrize("seed", range(2))
+def test_big_tile_gemm_random_shapes(lane, seed):
+    """Shapes large enough for the 256 x 256 tile (its 16-wide MFMA step, peeled first and last
+    K steps, ragged rows and columns), both storage types, short and odd K."""
+    from tessera_amd.schedule import select_gfx950_gemm_schedule
+    rng = np.random.default_rng(1500 + seed)
+    for _ in range(6):
+        M, N = (int(rng.integers(440, 560)) * 8 for _ in range(2))          # 3520 .. 4472, multiples of 8
+        K = int(rng.integers(1, 90)) * 8
+        st = "bf16" if rng.integers(0, 2) else "f16"
+        assert select_gfx950_gemm_schedule(M, N, K, dtype=st).workgroup_tile[:2] == (256, 256)
+        A = _store(rng.standard_normal((M, K)).astype(np.float32) * 0.5, st)
+        B = _store(rng.standard_normal((K, N)).astype(np.float32) * 0.5, st)
+        ref = _f32(A).astype(np.float64) @ _f32(B).astype(np.float64)
+        got = ops.gemm(A, B, out="f32")
+        assert orc.max_rel_err(got, ref) <= 1e-5, (seed, M, N, K, st)
+        stored = ops.gemm(A, B)
+        assert np.array_equal(np.asarray(stored).view(np.uint16), np.asarray(_store(got, st)).view(np.uint16)), (seed, M, N, K, st)
+
+
 @pytest.mark.parametrize("seed", range(3))
 def test_batched_gemm_random_shapes(lane, seed):
     rng = np.random.default_rng(2000 + seed)
