@@ -493,6 +493,35 @@ int tessera_gfx950_moe_layer_bf16_dev(const void* x, const void* w_router, const
                                       int32_t* group_sizes, int32_t* group_offsets, int32_t* num_slots,
                                       void* stream);
 
+/* ---- C-level launch bridge --------------------------------------------------- */
+
+/* A launcher for the reference's C runtime: a backend registers one function that maps a
+ * kernel NAME on a target to a native launch over ordered host buffers and scalar dims
+ * (tsrGpuLauncherFn / tsrRegisterGpuLauncher, src/runtime/include/tessera/
+ * tessera_runtime.h:81-99; params = tsrGpuLaunchParams, tsr_types.h:83-89: the struct
+ * below has the same layout, and the return values are the reference's TsrStatus codes,
+ * tsr_status.h:7-14).  tessera_gfx950_gpu_launcher has exactly the tsrGpuLauncherFn
+ * signature, so `tsrRegisterGpuLauncher(tessera_gfx950_gpu_launcher, NULL)` is the whole
+ * registration.  Targets: "rocm_gfx950" or "rocm".  Kernel names are this library's
+ * host-pointer entry points, each with its own buffer / dim order:
+ *   tessera_gfx950_gemm_{f16,bf16}, tessera_gfx950_gemm_{f16_f16,bf16_bf16},
+ *   tessera_gfx950_gemm_i8_i32                    buffers {A,B,D}      dims {M,N,K}
+ *   tessera_gfx950_batched_gemm_{f16,bf16}        buffers {A,B,D}      dims {batch,M,N,K}
+ *   tessera_gfx950_flash_attn_{f16,bf16}          buffers {Q,K,V,O}    dims {B,H,Sq,Sk,D,causal}
+ *                                                 (scale = 1/sqrt(D), the reference's default)
+ * Returns 0 success; 2 (not found) for another target or a name it does not handle, so
+ * the runtime reports an unbridged kernel honestly; 1 (invalid argument) for a wrong
+ * buffer / dim count, a NULL buffer or dims the entry point rejects; 7 (device error)
+ * when no gfx950 device is usable or the launch failed. */
+typedef struct {
+  void** buffers;
+  size_t num_buffers;
+  const int64_t* dims;
+  size_t num_dims;
+} tessera_gfx950_launch_params;
+int tessera_gfx950_gpu_launcher(const char* target, const char* kernel_name,
+                                const tessera_gfx950_launch_params* params, void* user);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,5 +1,6 @@
 // Device management half of the C ABI: probe, raw buffers, event timers.
 #include <atomic>
+#include <cmath>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -174,3 +175,65 @@ int tessera_gfx950_timer_destroy(void* timer) {
 }
 
 }  // extern "C"
+
+// ---- the reference C runtime's launch bridge ------------------------------------------
+namespace {
+constexpr int kTsrSuccess = 0, kTsrInvalidArgument = 1, kTsrNotFound = 2, kTsrDeviceError = 7;
+int tsr_status_of(int rc) {
+  return rc == tsr950::kOk ? kTsrSuccess : rc == tsr950::kBadShape ? kTsrInvalidArgument : kTsrDeviceError;
+}
+// every dim must fit the C int the entry points take
+bool dims_fit(const int64_t* d, size_t n) {
+  for (size_t i = 0; i < n; ++i)
+    if (d[i] < 0 || d[i] > 0x7fffffff) return false;
+  return true;
+}
+}  // namespace
+
+extern "C" int tessera_gfx950_gpu_launcher(const char* target, const char* kernel_name,
+                                           const tessera_gfx950_launch_params* params, void* user) {
+  (void)user;
+  if (!target || !kernel_name) return kTsrInvalidArgument;
+  if (std::strcmp(target, "rocm") != 0 && std::strcmp(target, "rocm_gfx950") != 0) return kTsrNotFound;
+  using Gemm = int (*)(const void*, const void*, void*, int, int, int);
+  using Batched = int (*)(const void*, const void*, void*, int, int, int, int);
+  using Attn = int (*)(const void*, const void*, const void*, void*, int, int, int, int, int, float, int);
+  struct { const char* name; Gemm fn; } const gemms[] = {
+      {"tessera_gfx950_gemm_f16", tessera_gfx950_gemm_f16},         {"tessera_gfx950_gemm_bf16", tessera_gfx950_gemm_bf16},
+      {"tessera_gfx950_gemm_f16_f16", tessera_gfx950_gemm_f16_f16}, {"tessera_gfx950_gemm_bf16_bf16", tessera_gfx950_gemm_bf16_bf16},
+      {"tessera_gfx950_gemm_i8_i32", tessera_gfx950_gemm_i8_i32}};
+  struct { const char* name; Batched fn; } const batched[] = {
+      {"tessera_gfx950_batched_gemm_f16", tessera_gfx950_batched_gemm_f16},
+      {"tessera_gfx950_batched_gemm_bf16", tessera_gfx950_batched_gemm_bf16}};
+  struct { const char* name; Attn fn; } const attns[] = {
+      {"tessera_gfx950_flash_attn_f16", tessera_gfx950_flash_attn_f16},
+      {"tessera_gfx950_flash_attn_bf16", tessera_gfx950_flash_attn_bf16}};
+  auto shaped = [&](size_t nbuf, size_t ndim) {
+    if (!params || params->num_buffers != nbuf || params->num_dims != ndim || !params->buffers || !params->dims) return false;
+    for (size_t i = 0; i < nbuf; ++i)
+      if (!params->buffers[i]) return false;
+    return dims_fit(params->dims, ndim);
+  };
+  for (const auto& g : gemms) {
+    if (std::strcmp(kernel_name, g.name) != 0) continue;
+    if (!shaped(3, 3)) return kTsrInvalidArgument;
+    const int64_t* d = params->dims;
+    return tsr_status_of(g.fn(params->buffers[0], params->buffers[1], params->buffers[2], (int)d[0], (int)d[1], (int)d[2]));
+  }
+  for (const auto& g : batched) {
+    if (std::strcmp(kernel_name, g.name) != 0) continue;
+    if (!shaped(3, 4)) return kTsrInvalidArgument;
+    const int64_t* d = params->dims;
+    return tsr_status_of(g.fn(params->buffers[0], params->buffers[1], params->buffers[2], (int)d[0], (int)d[1], (int)d[2], (int)d[3]));
+  }
+  for (const auto& a : attns) {
+    if (std::strcmp(kernel_name, a.name) != 0) continue;
+    if (!shaped(4, 6)) return kTsrInvalidArgument;
+    const int64_t* d = params->dims;
+    if (d[4] <= 0) return kTsrInvalidArgument;
+    const float scale = 1.0f / std::sqrt((float)d[4]);
+    return tsr_status_of(a.fn(params->buffers[0], params->buffers[1], params->buffers[2], params->buffers[3], (int)d[0],
+                              (int)d[1], (int)d[2], (int)d[3], (int)d[4], scale, d[5] != 0));
+  }
+  return kTsrNotFound;
+}

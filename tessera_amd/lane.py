@@ -59,6 +59,7 @@ def library_path() -> Path:
 # symbol -> argtypes; every entry point returns int.
 _GEMM = [_c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int]
 _SIGNATURES = {
+    "tessera_gfx950_gpu_launcher": [ctypes.c_char_p, ctypes.c_char_p, _c_vp, _c_vp],
     "tessera_gfx950_abi_version": [],
     "tessera_gfx950_probe": [],
     "tessera_gfx950_device_name": [ctypes.c_char_p, _c_int],

@@ -353,3 +353,51 @@ def test_typed_descriptor_hook_validates_before_the_device():
         {"X": x, "T": np.array([0, 3], np.int32), "O": np.zeros((2, 4), np.float32)}, {"T": 3, "S": 2, "H": 4})
     assert not res["ok"] and "disagree" in res["reason"]                   # token id 3 is out of range
     assert set(nl.supported_abis()) >= {nl.MATMUL_F16_F32_ABI, nl.ATTN_BF16_ABI, nl.MOE_DISPATCH_F32_ABI}
+
+
+class _LaunchParams(ctypes.Structure):
+    """tsrGpuLaunchParams (src/runtime/include/tessera/tsr_types.h:83-89)."""
+    _fields_ = [("buffers", ctypes.POINTER(ctypes.c_void_p)), ("num_buffers", ctypes.c_size_t),
+                ("dims", ctypes.POINTER(ctypes.c_int64)), ("num_dims", ctypes.c_size_t)]
+
+
+def launch_params(arrays, dims):
+    bufs = (ctypes.c_void_p * len(arrays))(*[a.ctypes.data if a is not None else None for a in arrays])
+    d = (ctypes.c_int64 * len(dims))(*dims)
+    keep = (bufs, d, arrays)
+    return _LaunchParams(bufs, len(arrays), d, len(dims)), keep
+
+
+def test_c_level_launcher_answers_like_the_runtime_expects():
+    """The tsrGpuLauncherFn entry point: TsrStatus codes (tsr_status.h:7-14) for everything
+    that is decided before a device is touched."""
+    SUCCESS, INVALID, NOT_FOUND, DEVICE_ERROR = 0, 1, 2, 7
+    lib = lane.load()
+    fn = lib.tessera_gfx950_gpu_launcher
+    a = np.zeros((4, 8), np.uint16)
+    b = np.zeros((8, 4), np.uint16)
+    d = np.zeros((4, 4), np.float32)
+    ok, keep = launch_params([a, b, d], [4, 4, 8])
+    assert fn(b"apple_gpu", b"tessera_gfx950_gemm_bf16", ctypes.byref(ok), None) == NOT_FOUND
+    assert fn(b"rocm_gfx1151", b"tessera_gfx950_gemm_bf16", ctypes.byref(ok), None) == NOT_FOUND
+    assert fn(b"rocm", b"tessera_rocm_gemm_f32", ctypes.byref(ok), None) == NOT_FOUND            # a name it does not bridge
+    assert fn(b"rocm", b"tessera_gfx950_gemm_bf16", None, None) == INVALID
+    assert fn(None, b"tessera_gfx950_gemm_bf16", ctypes.byref(ok), None) == INVALID
+    two, keep2 = launch_params([a, b], [4, 4, 8])
+    assert fn(b"rocm", b"tessera_gfx950_gemm_bf16", ctypes.byref(two), None) == INVALID          # buffer count
+    four, keep4 = launch_params([a, b, d], [4, 4, 8, 1])
+    assert fn(b"rocm", b"tessera_gfx950_gemm_bf16", ctypes.byref(four), None) == INVALID         # dim count
+    assert fn(b"rocm", b"tessera_gfx950_batched_gemm_bf16", ctypes.byref(ok), None) == INVALID   # wants {batch,M,N,K}
+    null, keepn = launch_params([a, None, d], [4, 4, 8])
+    assert fn(b"rocm_gfx950", b"tessera_gfx950_gemm_bf16", ctypes.byref(null), None) == INVALID
+    zero, keepz = launch_params([a, b, d], [0, 4, 8])
+    assert fn(b"rocm_gfx950", b"tessera_gfx950_gemm_bf16", ctypes.byref(zero), None) == INVALID  # rc 1 of the entry point
+    huge, keeph = launch_params([a, b, d], [4, 4, 1 << 40])
+    assert fn(b"rocm_gfx950", b"tessera_gfx950_gemm_bf16", ctypes.byref(huge), None) == INVALID  # does not fit a C int
+    attn, keepa = launch_params([a, a, a, d], [1, 1, 4, 4, 0, 1])
+    assert fn(b"rocm", b"tessera_gfx950_flash_attn_bf16", ctypes.byref(attn), None) == INVALID
+    if not lane.available():
+        assert fn(b"rocm", b"tessera_gfx950_gemm_bf16", ctypes.byref(ok), None) == DEVICE_ERROR  # no gfx950 here
+    else:
+        assert fn(b"rocm", b"tessera_gfx950_gemm_bf16", ctypes.byref(ok), None) == SUCCESS
+

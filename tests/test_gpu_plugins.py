@@ -220,3 +220,42 @@ def test_tuning_on_device(lane):
     packaged.absorb_file(at.PACKAGED)
     assert at.recommended(api, region, api.OP_MATMUL, cand.TARGET, big, big, corpus=packaged, dtype="bfloat16",
                           timing="device") == "gfx950_mfma_gemm"
+
+
+def test_c_level_launcher_runs_the_kernels(lane):
+    """The tsrGpuLauncherFn entry point (the C runtime's launch bridge,
+    src/runtime/include/tessera/tessera_runtime.h:81-99): kernel names on target
+    `rocm_gfx950` over ordered host buffers and dims; results equal the direct calls."""
+    import ctypes
+    from test_abi_and_host import launch_params
+    lib = lane.load()
+    fn = lib.tessera_gfx950_gpu_launcher
+    rng = np.random.default_rng(77)
+    M, N, K = 200, 328, 264
+    a = np.asarray(b16.from_float32((rng.standard_normal((M, K)) * 0.5).astype(np.float32)), np.uint16)
+    b = np.asarray(b16.from_float32((rng.standard_normal((K, N)) * 0.5).astype(np.float32)), np.uint16)
+    d = np.zeros((M, N), np.float32)
+    prm, keep = launch_params([a, b, d], [M, N, K])
+    assert fn(b"rocm_gfx950", b"tessera_gfx950_gemm_bf16", ctypes.byref(prm), None) == 0
+    want = ops.gemm(a.view(b16.BF16Array), b.view(b16.BF16Array), out="f32")
+    assert np.array_equal(d, want)
+    ref = a.view(b16.BF16Array).to_float32().astype(np.float64) @ b.view(b16.BF16Array).to_float32().astype(np.float64)
+    assert orc.max_rel_err(d, ref) <= 1e-5
+    # batched, f16
+    Bt = 3
+    af = (rng.standard_normal((Bt, 64, 40)) * 0.5).astype(np.float16)
+    bf = (rng.standard_normal((Bt, 40, 72)) * 0.5).astype(np.float16)
+    df = np.zeros((Bt, 64, 72), np.float32)
+    prm, keep = launch_params([af, bf, df], [Bt, 64, 72, 40])
+    assert fn(b"rocm", b"tessera_gfx950_batched_gemm_f16", ctypes.byref(prm), None) == 0
+    assert orc.max_rel_err(df, af.astype(np.float64) @ bf.astype(np.float64)) <= 1e-5
+    # attention with the default scale 1/sqrt(D), causal
+    B, H, Sq, Sk, D = 1, 2, 96, 160, 64
+    q, k, v = (np.asarray(b16.from_float32(rng.standard_normal(s).astype(np.float32)), np.uint16)
+               for s in ((B, H, Sq, D), (B, H, Sk, D), (B, H, Sk, D)))
+    o = np.zeros((B, H, Sq, D), np.float32)
+    prm, keep = launch_params([q, k, v, o], [B, H, Sq, Sk, D, 1])
+    assert fn(b"rocm_gfx950", b"tessera_gfx950_flash_attn_bf16", ctypes.byref(prm), None) == 0
+    want = ops.flash_attn(q.view(b16.BF16Array), k.view(b16.BF16Array), v.view(b16.BF16Array), causal=True, out="f32")
+    assert np.array_equal(o, np.asarray(want, np.float32))
+
