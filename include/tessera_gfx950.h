@@ -192,6 +192,14 @@ int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_m
  * as the layers of a decode step are.  No counterpart in the reference. */
 int tessera_gfx950_gemm_bf16_bench_rotating(int M, int N, int K, int iters, int weights,
                                             double* avg_ms);
+/* The bench ABI for the attention forward (the reference has it for the GEMM only): the
+ * same warm-up / HIP-event / wall-clock loop over tessera_gfx950_flash_attn_gqa_bf16_dev
+ * with bf16 output, scale 1/sqrt(D), on library-owned buffers filled with one constant
+ * (on this part a kernel's rate depends on its operand values; this figure is the one for
+ * operands that toggle nothing).  tessera_gfx950_bench_last_timer_source() answers for it
+ * as well. */
+int tessera_gfx950_flash_attn_bf16_bench(int B, int Hq, int Hkv, int Sq, int Sk, int D, int causal, int iters,
+                                         double* avg_ms);
 /* 0 = device events, 1 = host wall clock, -1 = no measurement yet
  * (tessera_rocm_bench_last_timer_source, tessera_rocm_gemm.cpp:567-580). */
 int tessera_gfx950_bench_last_timer_source(void);

@@ -233,6 +233,28 @@ int tessera_gfx950_flash_attn_gqa_f16_dev(const void* Q, const void* K, const vo
                                           int causal, int out_dtype, void* stream) {
   return flash_dev<F16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, out_dtype, as_stream(stream));
 }
+int tessera_gfx950_flash_attn_bf16_bench(int B, int Hq, int Hkv, int Sq, int Sk, int D, int causal, int iters,
+                                         double* avg_ms) {
+  g_last_timer_source = -1;
+  if (bad_attn(B, Hq, Hkv, Sq, Sk, D) || iters <= 0 || !avg_ms) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  DeviceScope scope;
+  const size_t q_bytes = (size_t)B * Hq * Sq * D * 2, kv_bytes = (size_t)B * Hkv * Sk * D * 2;
+  void* dQ = scope.alloc(q_bytes);
+  void* dK = scope.alloc(kv_bytes);
+  void* dV = scope.alloc(kv_bytes);
+  void* dO = scope.alloc(q_bytes);
+  void* dL = scope.alloc((size_t)B * Hq * Sq * 4);
+  if (scope.failed()) return kDeviceFailed;
+  // 0x3c3c: finite, non-trivial bf16 values
+  if (hipMemset(dQ, 0x3c, q_bytes) != hipSuccess || hipMemset(dK, 0x3c, kv_bytes) != hipSuccess ||
+      hipMemset(dV, 0x3c, kv_bytes) != hipSuccess)
+    return kDeviceFailed;
+  const float scale = 1.0f / std::sqrt((float)D);
+  return bench_loop([&](int) { return flash_dev<BF16>(dQ, dK, dV, dO, dL, B, Hq, Hkv, Sq, Sk, D, scale, causal, 1, nullptr); },
+                    iters, avg_ms);
+}
+
 int tessera_gfx950_flash_attn_gqa_bf16_dev(const void* Q, const void* K, const void* V, void* O, void* LSE,
                                            int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
                                            int causal, int out_dtype, void* stream) {

@@ -196,8 +196,6 @@ int gated_host(const void* A, const void* Wg, const void* Wu, int act, void* D, 
   return scope.download(D, dD, d_bytes) ? kOk : kDeviceFailed;
 }
 
-thread_local int g_last_timer_source = -1;
-
 }  // namespace
 }  // namespace tsr950
 
@@ -331,37 +329,8 @@ static int bench_gemm_bf16(int M, int N, int K, int iters, int weights, double* 
   if (hipMemset(dA, 0x3c, a_bytes) != hipSuccess) return kDeviceFailed;
   for (int i = 0; i < weights; ++i)
     if (hipMemset(dBs[i], 0x3c, b_bytes) != hipSuccess) return kDeviceFailed;
-  // Warm-up: at least five launches, and at least 60 ms of them, so that the clocks
-  // (which ramp up over tens of milliseconds after idle) are steady when timing starts.
-  const auto warm0 = std::chrono::steady_clock::now();
-  for (int w = 0; w < 5 || std::chrono::steady_clock::now() - warm0 < std::chrono::milliseconds(60); ++w) {
-    int rc = gemm16_dev<BF16, EPI_STORE16>(dA, dBs[w % weights], dD, 1, M, N, K, nullptr);
-    if (rc != kOk) return rc;
-    if ((w & 15) == 15 && hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
-  }
-  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
-  hipEvent_t e0, e1;
-  if (hipEventCreate(&e0) != hipSuccess) return kDeviceFailed;
-  if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return kDeviceFailed; }
-  int rc = kOk;
-  const auto t0 = std::chrono::steady_clock::now();
-  (void)hipEventRecord(e0, nullptr);
-  for (int it = 0; it < iters && rc == kOk; ++it)
-    rc = gemm16_dev<BF16, EPI_STORE16>(dA, dBs[it % weights], dD, 1, M, N, K, nullptr);
-  (void)hipEventRecord(e1, nullptr);
-  const bool synced = hipEventSynchronize(e1) == hipSuccess;
-  const double wall_ms =
-      std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
-  float ev_ms = 0.f;
-  const bool ev_ok = synced && hipEventElapsedTime(&ev_ms, e0, e1) == hipSuccess && std::isfinite(ev_ms) &&
-                     ev_ms > 0.f && ev_ms <= 2.0 * wall_ms && ev_ms >= 0.5 * wall_ms;
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
-  if (rc != kOk) return rc;
-  if (!synced) return kDeviceFailed;
-  g_last_timer_source = ev_ok ? 0 : 1;
-  *avg_ms = (ev_ok ? (double)ev_ms : wall_ms) / iters;
-  return kOk;
+  return bench_loop([&](int i) { return gemm16_dev<BF16, EPI_STORE16>(dA, dBs[i % weights], dD, 1, M, N, K, nullptr); },
+                    iters, avg_ms);
 }
 
 int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_ms) {

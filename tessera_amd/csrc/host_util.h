@@ -1,6 +1,8 @@
 // Host-side helpers shared by the C-ABI translation units: the cached device
 // probe, RAII device buffers for the host-pointer entry points, error mapping.
 #pragma once
+#include <cmath>
+#include <chrono>
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <vector>
@@ -42,6 +44,48 @@ class DeviceScope {
   std::vector<void*> ptrs_;
   bool failed_ = false;
 };
+
+// Which clock the last bench-ABI call on this thread reported: 0 HIP events, 1 wall clock,
+// -1 none yet / the call failed (tessera_gfx950_bench_last_timer_source).
+extern thread_local int g_last_timer_source;
+
+// The timing loop of the bench ABI (after tessera_rocm_gemm.cpp:551-667): warm-up of at
+// least five launches and 60 ms, so that the clocks, which ramp up over tens of
+// milliseconds after idle, are steady; then `iters` launches between two HIP events on the
+// null stream, cross-checked against the wall clock (the event figure is used when it lies
+// within a factor of two of it, otherwise the wall-clock one, and the source says which).
+// `launch(i)` enqueues launch i and returns a status code.
+template <class Launch>
+int bench_loop(Launch&& launch, int iters, double* avg_ms) {
+  const auto warm0 = std::chrono::steady_clock::now();
+  for (int w = 0; w < 5 || std::chrono::steady_clock::now() - warm0 < std::chrono::milliseconds(60); ++w) {
+    const int rc = launch(w);
+    if (rc != kOk) return rc;
+    if ((w & 15) == 15 && hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  }
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess) return kDeviceFailed;
+  if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return kDeviceFailed; }
+  int rc = kOk;
+  const auto t0 = std::chrono::steady_clock::now();
+  (void)hipEventRecord(e0, nullptr);
+  for (int it = 0; it < iters && rc == kOk; ++it) rc = launch(it);
+  (void)hipEventRecord(e1, nullptr);
+  const bool synced = hipEventSynchronize(e1) == hipSuccess;
+  const double wall_ms =
+      std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+  float ev_ms = 0.f;
+  const bool ev_ok = synced && hipEventElapsedTime(&ev_ms, e0, e1) == hipSuccess && std::isfinite(ev_ms) &&
+                     ev_ms > 0.f && ev_ms <= 2.0 * wall_ms && ev_ms >= 0.5 * wall_ms;
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc != kOk) return rc;
+  if (!synced) return kDeviceFailed;
+  g_last_timer_source = ev_ok ? 0 : 1;
+  *avg_ms = (ev_ok ? (double)ev_ms : wall_ms) / iters;
+  return kOk;
+}
 
 // Device scratch for kernels that need it between two launches of one call (split-K
 // partials, routing and combine lists, quantiser maxima): one buffer per (device,

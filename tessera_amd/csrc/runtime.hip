@@ -11,6 +11,8 @@
 
 namespace tsr950 {
 
+thread_local int g_last_timer_source = -1;
+
 int probe_device() {
   static std::once_flag once;
   static int cached = kNoDevice;

@@ -60,6 +60,7 @@ def library_path() -> Path:
 _GEMM = [_c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int]
 _SIGNATURES = {
     "tessera_gfx950_gpu_launcher": [ctypes.c_char_p, ctypes.c_char_p, _c_vp, _c_vp],
+    "tessera_gfx950_flash_attn_bf16_bench": [_c_int] * 8 + [_P(ctypes.c_double)],
     "tessera_gfx950_abi_version": [],
     "tessera_gfx950_probe": [],
     "tessera_gfx950_device_name": [ctypes.c_char_p, _c_int],

@@ -60,6 +60,9 @@ def test_shape_validation_precedes_the_device():
     tos = np.array([0, 9], np.int32)                           # token index out of range
     assert lib.tessera_gfx950_moe_dispatch(p(z), p(tos), p(z), 4, 2, 8, 2) == 1
     assert lib.tessera_gfx950_quantize_i8_f32(p(d), 4, 4, 2, p(z), p(d)) == 1
+    ms = ctypes.c_double(0)
+    assert lib.tessera_gfx950_flash_attn_bf16_bench(1, 4, 2, 64, 64, 24, 1, 3, ctypes.byref(ms)) == 1    # head dim
+    assert lib.tessera_gfx950_flash_attn_bf16_bench(1, 4, 2, 64, 64, 128, 1, 0, ctypes.byref(ms)) == 1   # no launches
     assert lib.tessera_gfx950_bench_last_timer_source() == -1
 
 

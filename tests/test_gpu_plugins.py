@@ -191,6 +191,11 @@ def test_bench_abi(lane):
     assert 0 < ms.value < 100
     assert lib.tessera_gfx950_bench_last_timer_source() in (0, 1)
     assert "gfx950" in lane.device_name() and lane.device_cus() > 0
+    # the attention forward's bench entry: a failed call resets the timer source, a good one sets it
+    assert lib.tessera_gfx950_flash_attn_bf16_bench(1, 4, 3, 64, 64, 128, 1, 3, ctypes.byref(ms)) == 1     # Hq % Hkv
+    assert lib.tessera_gfx950_bench_last_timer_source() == -1
+    assert lib.tessera_gfx950_flash_attn_bf16_bench(2, 8, 2, 1024, 1024, 128, 1, 5, ctypes.byref(ms)) == 0
+    assert 0 < ms.value < 100 and lib.tessera_gfx950_bench_last_timer_source() in (0, 1)
 
 
 def test_tuning_on_device(lane):
