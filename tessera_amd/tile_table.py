@@ -58,17 +58,18 @@ class KernelEntry:
     lds_bytes: int
 
 
-#: MFMA instruction per storage dtype on gfx950 (K doubles at each halving of the
-#: element size; the f8f6f4 form is the full-rate fp8 path).
+#: MFMA instruction of the 256 x 256 workgroup tile per storage dtype on gfx950 (the 16-bit
+#: tiles run the 16-wide form, which spends less power per FLOP; their smaller tiles and the
+#: attention kernels run m32n32k16; the f8f6f4 form is the full-rate fp8 path).
 MFMA_BY_DTYPE = {
-    "f16": ("m32n32k16", "v_mfma_f32_32x32x16_f16"),
-    "bf16": ("m32n32k16", "v_mfma_f32_32x32x16_bf16"),
+    "f16": ("m16n16k32", "v_mfma_f32_16x16x32_f16"),
+    "bf16": ("m16n16k32", "v_mfma_f32_16x16x32_bf16"),
     "int8": ("m32n32k32", "v_mfma_i32_32x32x32_i8"),
     "fp8_e4m3": ("m32n32k64", "v_mfma_f32_32x32x64_f8f6f4"),
 }
 
 KERNEL_TABLE: tuple = (
-    KernelEntry("tessera.matmul", ("tile.matmul", "tile.mma"), "tessera_rocm.mfma_gemm", "m32n32k16",
+    KernelEntry("tessera.matmul", ("tile.matmul", "tile.mma"), "tessera_rocm.mfma_gemm", "m16n16k32",
                 "v_mfma_f32_16x16x32_{f16,bf16} (256x256 tiles); v_mfma_f32_32x32x16_{f16,bf16} (smaller tiles)", ("f16", "bf16"),
                 ("tessera_gfx950_gemm_f16", "tessera_gfx950_gemm_bf16", "tessera_gfx950_gemm_f16_f16",
                  "tessera_gfx950_gemm_bf16_bf16", "tessera_gfx950_batched_gemm_f16",
@@ -78,8 +79,8 @@ KERNEL_TABLE: tuple = (
                 "v_mfma_i32_32x32x32_i8", ("int8",),
                 ("tessera_gfx950_gemm_i8_i32", "tessera_gfx950_gemm_w8a8_f32"),
                 "gfx950_gemm", "256x256x128, 2x2 waves of 128x128", 135168),
-    KernelEntry("tessera.fused_epilogue", ("tile.matmul", "tile.mma"), "tessera_rocm.mfma_gemm", "m32n32k16",
-                "v_mfma_f32_32x32x16_{f16,bf16}", ("f16", "bf16"),
+    KernelEntry("tessera.fused_epilogue", ("tile.matmul", "tile.mma"), "tessera_rocm.mfma_gemm", "m16n16k32",
+                "v_mfma_f32_16x16x32_{f16,bf16} (256x256 tiles); v_mfma_f32_32x32x16_{f16,bf16} (smaller tiles)", ("f16", "bf16"),
                 ("tessera_gfx950_gemm_bias_act_f16", "tessera_gfx950_gemm_bias_act_bf16",
                  "tessera_gfx950_gated_gemm_f16", "tessera_gfx950_gated_gemm_bf16"),
                 "gfx950_gemm", "256x256x64, bias + activation (or gate * up) in the epilogue", 135168),
@@ -96,8 +97,8 @@ KERNEL_TABLE: tuple = (
                 "v_mfma_f32_32x32x16_{f16,bf16}", ("f16", "bf16"),
                 ("tessera_gfx950_flash_attn_bwd_f16", "tessera_gfx950_flash_attn_bwd_bf16"),
                 "gfx950_flash_attn_bwd", "dQ: 256 q rows x 64 keys; dK/dV: 128 keys x 64 q rows", 66560),
-    KernelEntry("tessera.grouped_gemm", ("tile.matmul", "tile.mma"), "tessera_rocm.grouped_gemm", "m32n32k16",
-                "v_mfma_f32_32x32x16_bf16", ("bf16",),
+    KernelEntry("tessera.grouped_gemm", ("tile.matmul", "tile.mma"), "tessera_rocm.grouped_gemm", "m16n16k32",
+                "v_mfma_f32_16x16x32_bf16", ("bf16",),
                 ("tessera_gfx950_grouped_gemm_bf16", "tessera_gfx950_grouped_gemm_bf16_f32",
                  "tessera_gfx950_moe_swiglu_block_bf16"),
                 "gfx950_moe_transport", "256x256x64 per (expert, row tile), one launch", 135168),
@@ -125,7 +126,7 @@ def lower_tile_op(op: TileOp, *, arch: str = ARCH) -> list:
         return [TargetOp("tessera_rocm.grouped_gemm", {
             **base, "name": "grouped_gemm", "arch": arch, "status": "device_verified_abi",
             "runtime_lane": "gfx950_moe_transport", "argument_layout": "device_offsets[E+1]", "dispatches": 1,
-            "shape": "m32n32k16", "symbol": "tessera_gfx950_grouped_gemm_bf16"})]
+            "shape": "m16n16k32", "symbol": "tessera_gfx950_grouped_gemm_bf16"})]
     if source == "tessera.flash_attn" or op.op_name in ATTN_OPS:
         dtype = _norm_dtype(op.attrs.get("dtype", "bf16"))
         if dtype not in ("f16", "bf16"):

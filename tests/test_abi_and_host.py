@@ -282,12 +282,14 @@ def test_grouped_gemm_region_definition():
 def test_tile_table():
     ops_ = tile_table.lower_tile_op(tile_table.TileOp("tile.matmul", {"dtype": "bf16"}, 3))
     assert [o.name for o in ops_] == ["tessera_rocm.mfma", "tessera_rocm.mfma_gemm"]
-    assert ops_[0].attrs["shape"] == "m32n32k16" and ops_[1].attrs["symbol"] == "tessera_gfx950_gemm_bf16"
+    assert ops_[0].attrs["shape"] == "m16n16k32" and ops_[0].attrs["instr"] == "v_mfma_f32_16x16x32_bf16"
+    assert ops_[1].attrs["symbol"] == "tessera_gfx950_gemm_bf16" and ops_[1].attrs["block_m"] == 256
     assert tile_table.lower_tile_op(tile_table.TileOp("tile.mma", {"dtype": "int8"}))[0].attrs["shape"] == "m32n32k32"
     fa = tile_table.lower_tile_op(tile_table.TileOp("tessera_attn.online_softmax", {"source": "tessera.flash_attn", "causal": True}))
     assert fa[0].name == "tessera_rocm.mfma_flash_attn" and fa[0].attrs["runtime_lane"] == "gfx950_flash_attn"
     gg = tile_table.lower_tile_op(tile_table.TileOp("tile.matmul", {"source": "tessera.grouped_gemm"}))
     assert gg[0].attrs["argument_layout"] == "device_offsets[E+1]" and gg[0].attrs["dispatches"] == 1
+    assert gg[0].attrs["shape"] == "m16n16k32" and fa[0].attrs["shape"] == "m32n32k16"
     assert tile_table.lower_tile_op(tile_table.TileOp("tile.kv_cache"))[0].name == "tessera.target.diagnostic"
     lanes = set(ex.executor_table())
     declared = set(_header_symbols())
