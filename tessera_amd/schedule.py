@@ -25,7 +25,7 @@ _DTYPES = {
 }
 _INSTRUCTION_TILE = {"f16": (32, 32, 16), "bf16": (32, 32, 16), "int8": (32, 32, 32), "fp8_e4m3": (32, 32, 64)}
 # accumulators + operand fragments + staging of one wave, from the assembler's report
-_VGPRS = {256: 456, 128: 170, 64: 96, 32: 137}
+_VGPRS = {256: 508, 128: 170, 64: 96, 32: 137}
 
 
 @dataclass(frozen=True)
