@@ -440,7 +440,6 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
   auto kstep16 = [&](int kt, auto has1_c, auto l2_c, auto l3_c) __attribute__((always_inline)) {
     constexpr bool HAS1 = decltype(has1_c)::value;
     constexpr int L2 = decltype(l2_c)::value;
-    constexpr int L3 = decltype(l3_c)::value;
     static_assert(MS != 16 || KS == 2, "two MFMA k steps per K step");
     const int buf = kt & 1;
     // one row of the wave tile: its MFMAs, then the row's share of the fragment reads for
