@@ -50,7 +50,7 @@ PEAK_CLOCK_MHZ = 2400.0         # shader clock the MFMA peaks are quoted at
 # dispatch from two counter runs of this script, each scaled by the same counter's
 # reading for the 1 GiB copy kernel (profiles/bench_all_kernels_hbm_bytes.txt).  A
 # profiler figure carried into the line, not something this run measures.
-TRAFFIC_BYTES_GEMM_BF16_8192 = 2.0265e9
+TRAFFIC_BYTES_GEMM_BF16_8192 = 1.7454e9
 
 
 RAMP_SECONDS = 0.1
