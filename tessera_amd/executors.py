@@ -118,30 +118,29 @@ def lane_default_available() -> bool:
     return _lane.available()
 
 
-# ---- argument plumbing (runtime.py:44363-44384) --------------------------------------
+# ---- argument plumbing -----------------------------------------------------------------
+# What the reference's launch does with its ``args`` (runtime.py:44363-44384): a mapping is
+# taken by name, a bare value is one positional argument, positions follow ``arg_names``,
+# and a short argument list is a ValueError naming what is absent.
 
-def _bind_launch_args(args: Any, arg_names: list) -> dict:
+def _named_args(args: Any, arg_names: list) -> dict:
     if isinstance(args, Mapping):
-        return dict(args)
-    if args is None:
-        args = ()
-    if not isinstance(args, (list, tuple)):
-        args = (args,)
-    values = {name: value for name, value in zip(arg_names, args)}
-    if len(values) < len(arg_names):
-        missing = ", ".join(arg_names[len(values):])
-        raise ValueError(f"launch args missing value(s): {missing}")
-    return values
+        return {key: args[key] for key in args}
+    positional = [] if args is None else list(args) if isinstance(args, (list, tuple)) else [args]
+    absent = arg_names[len(positional):]
+    if absent:
+        raise ValueError("launch args missing value(s): " + ", ".join(absent))
+    return dict(zip(arg_names, positional))
 
 
-def _as_array(value: Any):
-    if hasattr(value, "numpy") and callable(value.numpy):
-        return np.asarray(value.numpy())
-    if hasattr(value, "_data"):
-        value = value._data
-    if _bf16.is_bf16(value):
-        return value
-    return np.asarray(value)
+def _host_array(value: Any):
+    """The numpy view of an operand: tensor wrappers are unwrapped (a ``numpy()`` method,
+    else a ``_data`` payload), bf16 arrays pass through as they are."""
+    to_numpy = getattr(value, "numpy", None)
+    if callable(to_numpy):
+        return np.asarray(to_numpy())
+    payload = getattr(value, "_data", value)
+    return payload if _bf16.is_bf16(payload) else np.asarray(payload)
 
 
 def _single_op(artifact: RuntimeArtifact, allowed: tuple, who: str) -> dict:
@@ -162,7 +161,7 @@ def execute_gfx950_gemm(artifact: RuntimeArtifact, args: Any):
     activation — float only (``runtime.py:6603-6660``)."""
     md = artifact.metadata or {}
     op = _single_op(artifact, ("tessera.matmul", "tessera.gemm", "tessera.fused_epilogue"), "gfx950_gemm")
-    values = _bind_launch_args(args, list(md.get("arg_names") or []))
+    values = _named_args(args, list(md.get("arg_names") or []))
     names = [str(n) for n in op.get("operands", [])]
     kwargs = op.get("kwargs") or {}
     activation = str(kwargs.get("activation") or "none")
@@ -171,7 +170,7 @@ def execute_gfx950_gemm(artifact: RuntimeArtifact, args: Any):
     if len(names) not in (2, 3):
         raise ValueError(f"matmul takes two operands (a, b) plus an optional third bias operand; got {len(names)}")
     has_bias = len(names) == 3
-    a, b = _as_array(values[names[0]]), _as_array(values[names[1]])
+    a, b = _host_array(values[names[0]]), _host_array(values[names[1]])
     if a.ndim != 2 or b.ndim != 2 or a.shape[1] != b.shape[0]:
         raise ValueError(f"gfx950 matmul needs rank-2 operands with matching K; got {a.shape} @ {b.shape}")
     if a.dtype == np.int8 and b.dtype == np.int8:
@@ -182,7 +181,7 @@ def execute_gfx950_gemm(artifact: RuntimeArtifact, args: Any):
         return _ops.gemm(a, b, out="f32")
     bias = None
     if has_bias:
-        bias = np.ascontiguousarray(np.asarray(_as_array(values[names[2]])), dtype=np.float32)
+        bias = np.ascontiguousarray(np.asarray(_host_array(values[names[2]])), dtype=np.float32)
         if bias.shape != (b.shape[1],):
             raise ValueError(f"bias must have shape ({b.shape[1]},) (one per output column); got {bias.shape}")
     return _ops.fused_gemm(a, b, bias, activation)
@@ -205,9 +204,9 @@ def execute_gfx950_flash_attn(artifact: RuntimeArtifact, args: Any):
         raise ValueError("flash_attn requires Q, K, V operands")
     if len(names) > 4:
         raise ValueError(f"flash_attn takes Q, K, V plus an optional attn_bias operand; got {len(names)}")
-    values = _bind_launch_args(args, list(md.get("arg_names") or []))
-    q, k, v = (_as_array(values[n]) for n in names[:3])
-    bias = np.asarray(_as_array(values[names[3]])) if len(names) == 4 else None
+    values = _named_args(args, list(md.get("arg_names") or []))
+    q, k, v = (_host_array(values[n]) for n in names[:3])
+    bias = np.asarray(_host_array(values[names[3]])) if len(names) == 4 else None
     kwargs = op.get("kwargs") or {}
     if kwargs.get("dropout_p"):
         raise ValueError("gfx950 flash_attn lane does not implement `dropout_p`")
@@ -239,8 +238,8 @@ def execute_gfx950_flash_attn_bwd(artifact: RuntimeArtifact, args: Any):
     names = [str(n) for n in op.get("operands", [])]
     if len(names) != 4:
         raise ValueError("gfx950 flash_attn backward requires exactly the (dO, Q, K, V) operands")
-    values = _bind_launch_args(args, list(md.get("arg_names") or []))
-    do, q, k, v = (_as_array(values[n]) for n in names)
+    values = _named_args(args, list(md.get("arg_names") or []))
+    do, q, k, v = (_host_array(values[n]) for n in names)
     kwargs = op.get("kwargs") or {}
     if kwargs.get("window") or kwargs.get("logit_softcap") or kwargs.get("attn_bias") is not None:
         raise ValueError("gfx950 flash_attn backward handles scale + causal only (no bias / window / soft-cap)")
@@ -286,7 +285,7 @@ def execute_gfx950_moe_transport(artifact: RuntimeArtifact, args: Any):
     """``tessera.moe_dispatch`` / ``moe_combine`` / ``grouped_gemm`` /
     ``grouped_swiglu`` → ``(output, "native_gpu")``."""
     md = artifact.metadata or {}
-    values = dict(args) if isinstance(args, Mapping) else _bind_launch_args(args, list(md.get("arg_names") or ["x", "plan"]))
+    values = dict(args) if isinstance(args, Mapping) else _named_args(args, list(md.get("arg_names") or ["x", "plan"]))
     ops = list(md.get("ops") or [])
     name = str(ops[0].get("op_name", "")) if len(ops) == 1 else ""
 
@@ -298,16 +297,16 @@ def execute_gfx950_moe_transport(artifact: RuntimeArtifact, args: Any):
 
     if name == "tessera.moe_dispatch":
         x, plan = need("x", "plan")
-        return (_ops.moe_dispatch(_as_array(x), _plan_to_transport(plan)), "native_gpu")
+        return (_ops.moe_dispatch(_host_array(x), _plan_to_transport(plan)), "native_gpu")
     if name == "tessera.moe_combine":
         partials, plan = need("partials", "plan")
-        return (_ops.moe_combine(_as_array(partials), _plan_to_transport(plan)), "native_gpu")
+        return (_ops.moe_combine(_host_array(partials), _plan_to_transport(plan)), "native_gpu")
     if name == "tessera.grouped_gemm":
         x, w, gs = need("x", "weights", "group_sizes")
-        return (_ops.grouped_gemm(_as_array(x), _as_array(w), gs, out="f32"), "native_gpu")
+        return (_ops.grouped_gemm(_host_array(x), _host_array(w), gs, out="f32"), "native_gpu")
     if name == "tessera.grouped_swiglu":
         x, wg, wu, wd, gs = need("x_packed", "w_gate", "w_up", "w_down", "group_sizes")
-        return (_ops.moe_swiglu_block(*map(_as_array, (x, wg, wu, wd)), gs), "native_gpu")
+        return (_ops.moe_swiglu_block(*map(_host_array, (x, wg, wu, wd)), gs), "native_gpu")
     raise ValueError("gfx950_moe_transport executor handles tessera.moe_dispatch, tessera.moe_combine, "
                      f"tessera.grouped_gemm, or tessera.grouped_swiglu; got {name!r}")
 
@@ -317,7 +316,7 @@ def execute_gfx950_quant_gemm(artifact: RuntimeArtifact, args: Any):
     ``tessera.w8a8_gemm``: operands (x_q, w_q, a_scale, w_scale)."""
     md = artifact.metadata or {}
     op = _single_op(artifact, ("tessera.fp8_gemm", "tessera.w8a8_gemm"), "gfx950_quant_gemm")
-    values = _bind_launch_args(args, list(md.get("arg_names") or []))
+    values = _named_args(args, list(md.get("arg_names") or []))
     names = [str(n) for n in op.get("operands", [])]
     kwargs = op.get("kwargs") or {}
     if op["op_name"] == "tessera.fp8_gemm":
