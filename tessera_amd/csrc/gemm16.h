@@ -13,8 +13,7 @@
 // in two MFMA forms (template parameter MS): v_mfma_f32_32x32x16_{bf16,f16} (4 x 4 tiles per
 // wave) and v_mfma_f32_16x16x32 (8 x 8 tiles).  The 256x256 tiles run the 16-wide form, which
 // spends less power per FLOP: on operands that toggle the matrix pipes the board then grants
-// a higher clock.  A second main loop that loads operands straight into LDS (gemm16_dl.h,
-// DL = true) is the form this one was measured against; it is kept behind a build switch.
+// a higher clock.
 // What follows describes the 32-wide step; the 16-wide one (kstep16) differs in how the
 // fragment reads are dealt out, see there.
 //
@@ -140,14 +139,10 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
   tn = r / rows;
 }
 
-}  // namespace tsr950
-#include "gemm16_dl.h"
-namespace tsr950 {
-
 // One BM x BN output tile: rows [m_begin, min(m_begin + BM, m_end)), column tile tn, of
 // the product whose operand and output bases are Ab / Bb / B2b / Db.  All threads of the
 // workgroup call it with the same arguments.
-template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32, bool DL = false>
+template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32>
 __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, const int m_begin, const int m_end,
                                             const int tn, const uint16_t* Ab, const uint16_t* Bb,
                                             const uint16_t* B2b, char* Db, const bool paced = false) {
@@ -159,7 +154,6 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
   // 14 % faster under the board's power limit on random operands (2010 against 1760 TFLOP/s):
   // the big tiles, which sit on that limit, use it.
   static_assert(MS == 32 || MS == 16, "MFMA tile side");
-  static_assert(!DL || MS == 16, "the direct-to-LDS main loop is written for the 16-wide MFMA");
   constexpr int KD = 512 / MS;                  // k per MFMA instruction
   constexpr int AE = MS * MS / 64;              // accumulator registers per MFMA tile
   constexpr int MI = TM / MS, NJ = TN / MS;     // MFMA tiles per wave
@@ -194,9 +188,6 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
 #pragma unroll
       for (int r = 0; r < AE; ++r) acc[i][j][r] = 0.f;
 
-  if constexpr (DL) {
-    gemm16_mainloop_dl<T, BM, BN, WM, WN, SWIGLU, GROUPED>(p, smem, acc, m_begin, m_end, n_begin, Ab, Bb, B2b);
-  } else {
   // ---- global load addressing ----------------------------------------------------
   // Buffer loads: a wave-uniform tile base (advanced along K on the scalar unit) plus
   // a fixed 32-bit per-lane byte offset, one address register per chunk.
@@ -499,9 +490,7 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
     // panel they share would then pass through that XCD's L2 twice.  It waits here instead
     // (kTailPace x 64 cycles per K step, about what the full tiles take longer), stays within
     // reach of them, and the panel is fetched once.
-#ifndef TSR_NO_TAIL_PACE
     if (paced) __builtin_amdgcn_s_sleep(kTailPace);
-#endif
 #pragma unroll
     for (int i = 0; i < MI; ++i) row(1, i, HAS1, buf ^ 1, 0, std::integral_constant<bool, (L2 != 0)>{}, 0, buf, (kt + 3) * G16_BK, l3_c);
   };
@@ -519,7 +508,6 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
   if (kt + 2 < ktiles) { kstep_any(kt, true_type{}, mode2{}, mode0{}); ++kt; }
   if (kt + 1 < ktiles) { kstep_any(kt, true_type{}, mode0{}, mode0{}); ++kt; }
   kstep_any(kt, false_type{}, mode0{}, mode0{});
-  }  // !DL
 
   // ---- epilogue -------------------------------------------------------------
   // acc[i][j][r]: row m = MS i + lm, col n = MS j + 8*(r/4) + 4*lk + (r%4): a lane owns
@@ -640,7 +628,7 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
   }
 }
 
-template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32, bool DL = false>
+template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32>
 __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Params p) {
   constexpr bool SWIGLU = (EPI == EPI_SWIGLU16 || EPI == EPI_GATED_F32);
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -737,11 +725,11 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     // full tile, whose other 192 rows would be computed and thrown away.
     if (m_end - m_begin <= 64) {
       // (paced when full tiles of the same group and column run beside it; 16-wide step only)
-      gemm16_tile<T, 64, BN, 1, 4, EPI, GROUPED, MS, DL>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db, MS == 16 && tm > 0);
+      gemm16_tile<T, 64, BN, 1, 4, EPI, GROUPED, MS>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db, MS == 16 && tm > 0);
       return;
     }
   }
-  gemm16_tile<T, BM, BN, WM, WN, EPI, GROUPED, MS, DL>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db);
+  gemm16_tile<T, BM, BN, WM, WN, EPI, GROUPED, MS>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db);
 }
 
 }  // namespace tsr950

@@ -61,33 +61,17 @@ __global__ void gemm16_grouped_generic_kernel(const Gemm16Params p) {
   else reinterpret_cast<uint16_t*>(p.D)[o] = to_storage<T>(acc);
 }
 
-// The 256 x 256 workgroup tiles use the 16-wide MFMA in the register-staged main loop.
-// TSR_BIG_CLASSIC builds them on the 32-wide MFMA, TSR_BIG_DIRECT on the 16-wide one with
-// operands loaded straight into LDS (gemm16_dl.h): the two forms this one was measured against.
-#if defined(TSR_BIG_CLASSIC)
-constexpr int kBigTileMfma = 32;
-constexpr bool kBigTileDirect = false;
-#elif defined(TSR_BIG_DIRECT)
+// The 256 x 256 workgroup tiles, dense and grouped (per expert), use the 16-wide MFMA in the
+// register-staged main loop; the smaller tiles use the 32-wide one.
 constexpr int kBigTileMfma = 16;
-constexpr bool kBigTileDirect = true;
-#else
-constexpr int kBigTileMfma = 16;
-constexpr bool kBigTileDirect = false;
-#endif
-// The grouped (per-expert) 256 x 256 tiles likewise; TSR_GROUPED_CLASSIC keeps them 32-wide.
-#ifdef TSR_GROUPED_CLASSIC
-constexpr int kGroupedTileMfma = 32;
-#else
 constexpr int kGroupedTileMfma = 16;
-#endif
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32, bool DL = false>
+template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32>
 int launch_gemm16_tile(Gemm16Params p, hipStream_t s) {
   using S = Gemm16Smem<BM, BN>;
-  static_assert(!DL || Gemm16DlSmem<BM, BN>::kBytes <= S::kBytes, "the direct-load stages fit the same LDS window");
-  auto kern = gemm16_kernel<T, BM, BN, WM, WN, EPI, GROUPED, MS, DL>;
+  auto kern = gemm16_kernel<T, BM, BN, WM, WN, EPI, GROUPED, MS>;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [&] {
@@ -224,9 +208,9 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
   }
   if (sch.tile == 256) {
     if constexpr (EPI == EPI_F32) {
-      if (fused) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI_F32_FUSED, false, kBigTileMfma, kBigTileDirect>(p, s);
+      if (fused) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI_F32_FUSED, false, kBigTileMfma>(p, s);
     }
-    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false, kBigTileMfma, kBigTileDirect>(p, s);
+    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false, kBigTileMfma>(p, s);
   }
   const bool t128 = sch.tile == 128;
   if (sch.skinny && sch.split_k == 1) return launch_gemm16_skinny<T, EPI>(p, p.K, 1, s);
@@ -287,7 +271,7 @@ int launch_gemm16_gated(Gemm16Params p, hipStream_t s) {
     hipLaunchKernelGGL((gemm16_generic_kernel<T, EPI_GATED_F32>), grid, block, 0, s, p);
     return launch_status();
   }
-  return launch_gemm16_tile<T, 256, 256, 4, 1, EPI_GATED_F32, false, kBigTileMfma, false>(p, s);
+  return launch_gemm16_tile<T, 256, 256, 4, 1, EPI_GATED_F32, false, kBigTileMfma>(p, s);
 }
 
 // Grouped.  p.M = total rows S, p.groups = E, p.offsets = device int32[E+1].
@@ -305,9 +289,9 @@ int launch_gemm16_grouped(Gemm16Params p, hipStream_t s) {
     return launch_status();
   }
   if constexpr (EPI == EPI_SWIGLU16) {
-    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true, kGroupedTileMfma, false>(p, s);
+    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true, kGroupedTileMfma>(p, s);
   } else {
-    if ((long)p.M >= 64L * p.groups) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true, kGroupedTileMfma, false>(p, s);
+    if ((long)p.M >= 64L * p.groups) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true, kGroupedTileMfma>(p, s);
     return launch_gemm16_tile<T, 128, 128, 2, 2, EPI, true>(p, s);
   }
 }
