@@ -398,13 +398,20 @@ def has_routing_ties(p: np.ndarray, k: int) -> bool:
     return bool(np.any(srt[:, : kk - 1] == srt[:, 1:kk]))
 
 
+def compute_capacity(capacity_factor, num_tokens, num_experts):
+    """MoEConfig.compute_capacity (distributed/moe.py:79-92) on one rank: the tokens-per-expert
+    quotient is formed first, then scaled, then rounded up (numpy float64 throughout)."""
+    tokens_per_expert = num_tokens / max(1, num_experts)
+    return int(np.ceil(capacity_factor * tokens_per_expert))
+
+
 def route_tokens(scores: np.ndarray, num_experts: int, top_k: int,
                  normalize_weights: bool = True,
                  capacity_factor: float = 1e9,
                  capacity: int | None = None) -> Routing:
     """``distributed/moe.py:119-206`` without jitter.
 
-    capacity = ``ceil(capacity_factor * T / E)`` when not given
+    capacity = ``ceil(capacity_factor * (T / E))`` when not given
     (``distributed/moe.py:79-92``).  Over-capacity slots are dropped in
     token-major, slot-minor order: assignment -1, weight 0.
     """
@@ -423,7 +430,7 @@ def route_tokens(scores: np.ndarray, num_experts: int, top_k: int,
         w = w / ws
     load = np.bincount(idx.reshape(-1), minlength=E).astype(np.int64)
     if capacity is None:
-        capacity = int(math.ceil(capacity_factor * T / E))
+        capacity = compute_capacity(capacity_factor, T, E)
     assignment = idx.astype(np.int64).copy()
     weights = w.astype(np.float32).copy()
     overflow = 0

@@ -473,6 +473,14 @@ class MoETransport:
         return int(self.token_of_slot.shape[0])
 
 
+def expert_capacity(capacity_factor: float, num_tokens: int, num_experts: int) -> int:
+    """Slots per expert, ``ceil(capacity_factor * (T / E))`` evaluated in that order
+    (``MoEConfig.compute_capacity``, ``distributed/moe.py:79-92``): the quotient first,
+    then the factor — ``(cf * T) / E`` rounds differently on a few (cf, T, E) triples
+    (cf=1.1, T=540, E=3: 199, not 198) and one slot of capacity changes which slots drop."""
+    return int(math.ceil(capacity_factor * (num_tokens / max(1, num_experts))))
+
+
 def _capacity_arg(capacity: Optional[int], T: int, k: int) -> int:
     if capacity is None or capacity >= T * k:
         return 0            # cannot overflow
@@ -484,7 +492,7 @@ def _capacity_arg(capacity: Optional[int], T: int, k: int) -> int:
 def route_tokens(scores, num_experts: int, top_k: int, *, normalize_weights: bool = True,
                  capacity_factor: float = 1.25, capacity: Optional[int] = None) -> MoETransport:
     """Top-k routing + packing plan.  ``scores`` ``(T, E)`` f32 gate logits.
-    capacity defaults to ``ceil(capacity_factor * T / E)``; over-capacity slots are
+    capacity defaults to ``ceil(capacity_factor * (T / E))``; over-capacity slots are
     dropped first-come in token-major order.  Ties between equal probabilities go
     to the lowest expert id."""
     s = np.ascontiguousarray(_unbox(scores), np.float32)
@@ -498,7 +506,7 @@ def route_tokens(scores, num_experts: int, top_k: int, *, normalize_weights: boo
     if capacity is None:
         if capacity_factor <= 0:
             raise ValueError(f"capacity_factor must be > 0, got {capacity_factor}")
-        capacity = int(math.ceil(capacity_factor * T / E))
+        capacity = expert_capacity(capacity_factor, T, E)
     cap = _capacity_arg(capacity, T, top_k)
     S = T * top_k
     tos = np.empty(S, np.int32)
@@ -726,7 +734,7 @@ def moe_layer(x, W_router, W_gate, W_up, W_down, *, top_k: int = 1, normalize_we
     lib = _lane.load()
     cap = 0
     if capacity_factor > 0:
-        cap = _capacity_arg(int(math.ceil(capacity_factor * T / E)), T, top_k)
+        cap = _capacity_arg(expert_capacity(capacity_factor, T, E), T, top_k)
     S = T * top_k
     outp = np.zeros((T, N), np.float32)
     tos = np.empty(S, np.int32)

@@ -29,6 +29,7 @@ import numpy as np
 
 from . import bf16 as _bf16
 from . import lane as _lane
+from . import ops as _ops
 
 _ITEMSIZE = {"bf16": 2, "f16": 2, "f32": 4, "i32": 4, "i8": 1, "u8": 1}
 _NUMPY = {"f16": np.float16, "f32": np.float32, "i32": np.int32, "i8": np.int8, "u8": np.uint8}
@@ -209,7 +210,7 @@ def moe_layer(x: DeviceArray, W_router: Optional[DeviceArray], W_gate: DeviceArr
         raise ValueError(f"W_router must be bf16 (K, E)=({H}, {E})")
     if router_logits is not None and (router_logits.dtype != "f32" or router_logits.shape != (T, E)):
         raise ValueError(f"router_logits must be f32 (T, E)=({T}, {E})")
-    cap = int(math.ceil(capacity_factor * T / E)) if capacity_factor > 0 else 0
+    cap = _ops.expert_capacity(capacity_factor, T, E) if capacity_factor > 0 else 0
     lib = _lane.load()
     need = ctypes.c_size_t(0)
     _lane.check(lib.tessera_gfx950_moe_layer_workspace_bytes(T, H, F, N, E, top_k, ctypes.byref(need)), "moe_layer")

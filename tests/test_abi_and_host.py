@@ -406,3 +406,26 @@ def test_c_level_launcher_answers_like_the_runtime_expects():
     else:
         assert fn(b"rocm", b"tessera_gfx950_gemm_bf16", ctypes.byref(ok), None) == SUCCESS
 
+
+
+def test_expert_capacity_follows_the_reference_order():
+    """capacity = ceil(cf * (T / E)) (distributed/moe.py:79-92).  (cf * T) / E rounds
+    differently on about 0.04 % of triples; the known one is cf=1.1, T=540, E=3 -> 199."""
+    import math
+    from fractions import Fraction
+
+    import tessera_oracle as orc
+    from tessera_amd import ops
+    assert ops.expert_capacity(1.1, 540, 3) == 199 == orc.compute_capacity(1.1, 540, 3)
+    assert int(math.ceil(1.1 * 540 / 3)) == 198          # the other order, for the record
+    differ = 0
+    for cf in (1.0, 1.05, 1.1, 1.25, 1.3, 1.7, 2.0, 2.2):
+        for T in range(1, 700, 7):
+            for E in (1, 3, 6, 7, 8, 12, 48, 64):
+                got = ops.expert_capacity(cf, T, E)
+                assert got == orc.compute_capacity(cf, T, E)
+                # never below the exact rational value's ceiling minus the float slack of one slot
+                exact = math.ceil(Fraction(cf) * Fraction(T, E))
+                assert abs(got - exact) <= 1
+                differ += got != int(math.ceil(cf * T / E))
+    assert differ > 0
