@@ -597,35 +597,51 @@ print(json.dumps({"ms": ms, "tflops": 2.0 * M * N * K / ms / 1e9, "library": "to
 """
 
 
+def _run_child(cmd, timeout_s):
+    """Run `cmd` in a process group of its own, wait for it, and make sure nothing it started
+    outlives this call (the group is ended and reaped whichever way the child finished)."""
+    import signal
+    import subprocess
+    p = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, start_new_session=True)
+    try:
+        out, err = p.communicate(timeout=timeout_s)
+    except subprocess.TimeoutExpired:
+        out, err = "", f"timed out after {timeout_s} s"
+    finally:
+        try:
+            os.killpg(p.pid, signal.SIGKILL)          # the group this call created, by its exact id
+        except (ProcessLookupError, PermissionError):
+            pass
+        p.wait()
+    return p.returncode, out, err
+
+
 def vendor_gemm_same_box(timeout_s=240):
     """The vendor library's GEMM of the same shape, layout and data distribution on the
     same box, in a child process (PyTorch is not part of this package): a yardstick for
     what a production kernel reaches under the same power limit.  Any failure is reported,
     not raised."""
-    import subprocess
     try:
-        r = subprocess.run([sys.executable, "-c", _VENDOR_SNIPPET], capture_output=True, text=True, timeout=timeout_s)
-        line = [l for l in r.stdout.splitlines() if l.startswith("{")]
-        if r.returncode != 0 or not line:
-            return {"error": (r.stderr or r.stdout).strip().splitlines()[-1:] or ["no output"]}
+        rc, out, err = _run_child([sys.executable, "-c", _VENDOR_SNIPPET], timeout_s)
+        line = [l for l in out.splitlines() if l.startswith("{")]
+        if rc != 0 or not line:
+            return {"error": (err or out).strip().splitlines()[-1:] or ["no output"]}
         d = json.loads(line[-1])
         d["frac_mfma_peak"] = d["tflops"] / PEAK_BF16_TFLOPS
         return d
-    except (OSError, subprocess.SubprocessError, ValueError) as exc:
+    except (OSError, ValueError) as exc:
         return {"error": str(exc)}
 
 
 def _smi_sample():
     """(mean shader clock over the XCDs in MHz, socket power in W) from amd-smi, or None."""
-    import subprocess
     try:
-        r = subprocess.run(["/opt/rocm/bin/amd-smi", "metric", "-p", "-c", "--json"], capture_output=True, text=True,
-                           timeout=20)
-        j = json.loads(r.stdout)
+        _, out, _ = _run_child(["/opt/rocm/bin/amd-smi", "metric", "-p", "-c", "--json"], 20)
+        j = json.loads(out)
         g = j[0] if isinstance(j, list) else j["gpu_data"][0]
         clk = [v["clk"]["value"] for k, v in g["clock"].items() if k.startswith("gfx_")]
         return float(np.mean(clk)), float(g["power"]["socket_power"]["value"])
-    except (OSError, ValueError, KeyError, IndexError, TypeError, subprocess.SubprocessError):
+    except (OSError, ValueError, KeyError, IndexError, TypeError):
         return None
 
 
@@ -741,6 +757,18 @@ def operand_residency_trace(lane, seconds=2.0):
         for buf in (da, db, dd):
             buf.close()
     return rows
+
+
+def gemm_f32_accumulators(lane, a_bits, b_bits, M, N, K):
+    """A . B through the f32-output entry point (the accumulators before any storage rounding)."""
+    lib = lane.load()
+    da, db, dd = lane.DeviceBuffer.from_host(a_bits), lane.DeviceBuffer.from_host(b_bits), lane.DeviceBuffer(M * N * 4)
+    lane.check(lib.tessera_gfx950_gemm_bf16_dev(da.ptr, db.ptr, dd.ptr, M, N, K, None), "gemm f32")
+    lane.synchronize()
+    acc = dd.download((M, N), np.float32)
+    for buf in (da, db, dd):
+        buf.close()
+    return acc
 
 
 def cpu_baseline(A, B):
@@ -873,6 +901,17 @@ def main() -> int:
         got = (out.astype(np.uint32) << 16).view(np.float32)
         err = float(np.max(np.abs(got - ref)) / np.max(np.abs(ref)))
         result["parity_max_rel_vs_cpu"] = err                 # includes the bf16 store (<= 2^-8)
+        # The same product with the f32 epilogue: the kernel's own error, without the store's
+        # rounding, and whether the stored output is exactly the RNE of those accumulators.
+        acc = gemm_f32_accumulators(lane, a, b, M, N, K)
+        result["parity_f32_accumulators_max_rel_vs_cpu"] = float(np.max(np.abs(acc - ref)) / np.max(np.abs(ref)))
+        result["stored_output_is_rne_of_accumulators"] = bool(np.array_equal(_bf16(acc), out))
+        result["parity_bounds"] = {"f32_accumulators": 2e-3, "bf16_stored": 2e-3 + 2.0 ** -8}
+        if result["parity_f32_accumulators_max_rel_vs_cpu"] > 2e-3 or err > 2e-3 + 2.0 ** -8:
+            print("bench: parity bound exceeded", file=sys.stderr)
+            print(json.dumps(result))
+            return 4
+        del acc
     del A, B, a, b, out
     if not args.only_headline:
         also = {}
