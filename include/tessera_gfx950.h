@@ -27,14 +27,31 @@
  *                               synchronising.  This is the resident-buffer form
  *                               used for chained ops and for timing.
  *
+ * Threads.  The host-pointer entry points (and tessera_gfx950_gpu_launcher, which calls
+ * them) are re-entrant, like the reference's, which allocate per call: the library
+ * serialises them internally (one lock from a call's first allocation to its last
+ * download), so any number of host threads may be inside them at once and each gets the
+ * result the call gives alone.  They do not overlap with each other on the device.
+ *
  * Temporaries of the _dev entry points (split-K partials, routing and combine lists,
  * quantiser maxima) come from one workspace per (device, stream) that the library
  * grows on demand: a call that needs more than any earlier call on its stream makes
  * one hipMalloc (no free, no synchronisation; the outgrown buffer is kept for the
  * work still queued on it), every other call allocates nothing.  All calls on one
  * stream share that workspace from its first byte, so the host threads that enqueue
- * on one stream must be serialised by the caller; under stream capture run the call
- * once beforehand so the workspace already has its size.
+ * on one stream must be serialised by the caller.  The workspace lives until
+ * tessera_gfx950_stream_release(stream) or the end of the process; release a stream's
+ * workspace before destroying the stream (a new stream may be given the old handle).
+ *
+ * HIP graphs.  A _dev call that uses the workspace must have been made once EAGERLY on the
+ * stream, with arguments at least as large, before it is recorded into a stream capture:
+ * the first call (or a larger one) allocates, which a capture does not allow, and the
+ * recorded kernels hold the workspace's address.  Replay such a graph on the stream it was
+ * captured on (launched elsewhere it shares that stream's workspace with eager calls on it
+ * and races with them), and do not release the stream's workspace while the graph is in
+ * use.  tessera_gfx950_moe_layer_bf16_dev takes a caller-owned workspace instead and has
+ * neither restriction.  Any entry point (tessera_gfx950_probe is the cheapest) must have
+ * been called once before the first capture: the first call initialises the device.
  */
 #ifndef TESSERA_GFX950_H
 #define TESSERA_GFX950_H
@@ -59,6 +76,10 @@ int tessera_gfx950_abi_version(void);
  * reference's lanes expose through their 16x16x16 zero-GEMM
  * (python/tessera/runtime.py:1992-2033). */
 int tessera_gfx950_probe(void);
+/* Waits for `stream` (a hipStream_t; NULL = the default stream) and frees the workspace the
+ * library keeps for it on the current device.  A later _dev call on the stream allocates a
+ * new one.  No counterpart in the reference (its entry points allocate per call). */
+int tessera_gfx950_stream_release(void* stream);
 /* Writes the gcnArchName / marketing name (NUL-terminated, truncated). */
 int tessera_gfx950_device_name(char* buf, int buflen);
 int tessera_gfx950_device_cus(int* cus);
@@ -187,6 +208,12 @@ int tessera_gfx950_gemm_schedule(int M, int N, int K, int batch, int elem_bytes,
  * launches between HIP events, cross-checked against wall clock
  * (tessera_rocm_gemm.cpp:551-667).  *avg_ms = mean per-launch ms. */
 int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_ms);
+/* The f16 form with the parameter list of tessera_rocm_wmma_gemm_f16_bench
+ * (tessera_rocm_gemm.cpp:861-866), so a caller of that symbol binds this one unchanged.
+ * There mt / nt choose the register blocking of the benchmarked variant; here the
+ * launcher picks the tile from the shape (tessera_gfx950_gemm_schedule tells which), so
+ * they are validated (> 0, else 1) and otherwise unused.  f16 in, f16 out. */
+int tessera_gfx950_gemm_f16_bench(int M, int N, int K, int iters, int mt, int nt, double* avg_ms);
 /* The same loop cycling over `weights` (1..64) distinct B matrices: a weight matrix
  * that would fit the memory-side cache is then streamed from HBM on every launch,
  * as the layers of a decode step are.  No counterpart in the reference. */
@@ -362,7 +389,10 @@ int tessera_gfx950_moe_route_f32_dev(const float* scores, int T, int E, int k, i
  * ceil(T*k / 512) * E * 4 <= 4 MiB (T*k up to about 490,000 slots at E = 64), else
  * rc 1.  Every call on one GPU shares that array, so two such calls that overlap on
  * one GPU (different streams, or different host threads) race; calls on one stream
- * are safe back to back.  All pointers are device memory. */
+ * are safe back to back.  The array's device address is looked up when the library first
+ * touches the device (any entry point; tessera_gfx950_probe does it), so make one library
+ * call before the first stream capture; after that this entry point records into a capture
+ * and replays like any kernel launch.  All pointers are device memory. */
 int tessera_gfx950_moe_route_f32_noalloc_dev(const float* scores, int T, int E, int k, int normalize, int capacity,
                                              int32_t* token_of_slot, int32_t* expert_of_slot,
                                              float* combine_weights, int32_t* group_sizes,

@@ -196,6 +196,31 @@ int gated_host(const void* A, const void* Wg, const void* Wu, int act, void* D, 
   return scope.download(D, dD, d_bytes) ? kOk : kDeviceFailed;
 }
 
+// Kernel-only timing on resident buffers.  The device-event figure is accepted
+// only when it lies within 0.5x..2x of the wall clock around the same launches;
+// otherwise the wall-clock figure is reported and the source says so.
+// `weights` > 1 cycles the launches over that many distinct B matrices, so that a
+// weight matrix smaller than the 256 MB memory-side cache is still read from HBM.
+template <class T>
+int bench_gemm16(int M, int N, int K, int iters, int weights, double* avg_ms) {
+  g_last_timer_source = -1;
+  if (bad_dims(1, M, N, K) || iters <= 0 || weights <= 0 || weights > 64 || !avg_ms) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  DeviceScope scope;
+  const size_t a_bytes = (size_t)M * K * 2, b_bytes = (size_t)K * N * 2, d_bytes = (size_t)M * N * 2;
+  void* dA = scope.alloc(a_bytes);
+  void* dBs[64];
+  for (int i = 0; i < weights; ++i) dBs[i] = scope.alloc(b_bytes);
+  void* dD = scope.alloc(d_bytes);
+  if (scope.failed()) return kDeviceFailed;
+  // 0x3c3c in every element: a finite, non-trivial value in bf16 (0.0115) and in f16 (1.06).
+  if (hipMemset(dA, 0x3c, a_bytes) != hipSuccess) return kDeviceFailed;
+  for (int i = 0; i < weights; ++i)
+    if (hipMemset(dBs[i], 0x3c, b_bytes) != hipSuccess) return kDeviceFailed;
+  return bench_loop([&](int i) { return gemm16_dev<T, EPI_STORE16>(dA, dBs[i % weights], dD, 1, M, N, K, nullptr); },
+                    iters, avg_ms);
+}
+
 }  // namespace
 }  // namespace tsr950
 
@@ -309,35 +334,15 @@ int tessera_gfx950_gemm_schedule(int M, int N, int K, int batch, int elem_bytes,
   return kBadShape;
 }
 
-// Kernel-only timing on resident buffers.  The device-event figure is accepted
-// only when it lies within 0.5x..2x of the wall clock around the same launches;
-// otherwise the wall-clock figure is reported and the source says so.
-// `weights` > 1 cycles the launches over that many distinct B matrices, so that a
-// weight matrix smaller than the 256 MB memory-side cache is still read from HBM.
-static int bench_gemm_bf16(int M, int N, int K, int iters, int weights, double* avg_ms) {
-  g_last_timer_source = -1;
-  if (bad_dims(1, M, N, K) || iters <= 0 || weights <= 0 || weights > 64 || !avg_ms) return kBadShape;
-  if (probe_device() != kOk) return kNoDevice;
-  DeviceScope scope;
-  const size_t a_bytes = (size_t)M * K * 2, b_bytes = (size_t)K * N * 2, d_bytes = (size_t)M * N * 2;
-  void* dA = scope.alloc(a_bytes);
-  void* dBs[64];
-  for (int i = 0; i < weights; ++i) dBs[i] = scope.alloc(b_bytes);
-  void* dD = scope.alloc(d_bytes);
-  if (scope.failed()) return kDeviceFailed;
-  // 0x3c00 pattern bytes: finite, non-trivial bf16 values.
-  if (hipMemset(dA, 0x3c, a_bytes) != hipSuccess) return kDeviceFailed;
-  for (int i = 0; i < weights; ++i)
-    if (hipMemset(dBs[i], 0x3c, b_bytes) != hipSuccess) return kDeviceFailed;
-  return bench_loop([&](int i) { return gemm16_dev<BF16, EPI_STORE16>(dA, dBs[i % weights], dD, 1, M, N, K, nullptr); },
-                    iters, avg_ms);
-}
-
 int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_ms) {
-  return bench_gemm_bf16(M, N, K, iters, 1, avg_ms);
+  return bench_gemm16<BF16>(M, N, K, iters, 1, avg_ms);
+}
+int tessera_gfx950_gemm_f16_bench(int M, int N, int K, int iters, int mt, int nt, double* avg_ms) {
+  if (mt <= 0 || nt <= 0) { g_last_timer_source = -1; return kBadShape; }
+  return bench_gemm16<F16>(M, N, K, iters, 1, avg_ms);
 }
 int tessera_gfx950_gemm_bf16_bench_rotating(int M, int N, int K, int iters, int weights, double* avg_ms) {
-  return bench_gemm_bf16(M, N, K, iters, weights, avg_ms);
+  return bench_gemm16<BF16>(M, N, K, iters, weights, avg_ms);
 }
 
 int tessera_gfx950_bench_last_timer_source(void) { return g_last_timer_source; }

@@ -4,6 +4,7 @@
 #include <cmath>
 #include <chrono>
 #include <hip/hip_runtime.h>
+#include <mutex>
 #include <stddef.h>
 #include <vector>
 #include "common.h"
@@ -15,11 +16,20 @@ int probe_device();
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// Serialises the host-pointer entry points.  Each of them uploads, runs its device-pointer
+// twin on the null stream, synchronises and downloads; the twin takes its scratch (split-K
+// partials, routing lists, quantiser maxima) from the null stream's workspace at offset 0.
+// Two host threads inside such calls at once would share those bytes, so every
+// host-pointer call holds this lock from its first allocation to its last download.
+// Recursive: a host-pointer entry point may be reached through another (the launcher).
+std::recursive_mutex& host_call_mutex();
+
 // Owns device allocations made on behalf of a host-pointer entry point and frees
-// them on scope exit, whichever way the call ends.
+// them on scope exit, whichever way the call ends.  Holds host_call_mutex() for its
+// lifetime, which makes the host-pointer ABI safe to call from several threads.
 class DeviceScope {
  public:
-  DeviceScope() = default;
+  DeviceScope() : lock_(host_call_mutex()) {}
   DeviceScope(const DeviceScope&) = delete;
   DeviceScope& operator=(const DeviceScope&) = delete;
   ~DeviceScope() {
@@ -41,6 +51,7 @@ class DeviceScope {
   bool failed() const { return failed_; }
 
  private:
+  std::unique_lock<std::recursive_mutex> lock_;   // declared first: released after the frees
   std::vector<void*> ptrs_;
   bool failed_ = false;
 };
@@ -98,6 +109,11 @@ int bench_loop(Launch&& launch, int iters, double* avg_ms) {
 // buffer must already have its final size (run the call once outside the capture).
 // Returns null on failure.
 void* stream_workspace(hipStream_t s, size_t bytes);
+// Synchronises `s` and frees its workspace; a later call on the stream allocates afresh.
+int stream_workspace_release(hipStream_t s);
+// Looks up the device address of the allocation-free routing entry's scratch array for the
+// current device (idempotent); called from the device probe.
+int route_scratch_warm();
 
 // Clears `words` 32-bit words on the stream with a fill kernel.  (A memset node recorded
 // into a captured graph has given wrong results on replays after the first, so nothing a

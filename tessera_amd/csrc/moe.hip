@@ -373,6 +373,13 @@ int route_scratch(char** out) {
   return kOk;
 }
 
+}  // namespace
+int route_scratch_warm() {
+  char* unused = nullptr;
+  return route_scratch(&unused);
+}
+namespace {
+
 // ---- dispatch: exact row gather, 16 bytes per lane -------------------------------
 __global__ __launch_bounds__(256) void dispatch_kernel(const char* x, const int32_t* token_of_slot, char* x_perm,
                                                        int T, int S, long row_bytes) {

@@ -13,6 +13,11 @@ namespace tsr950 {
 
 thread_local int g_last_timer_source = -1;
 
+std::recursive_mutex& host_call_mutex() {
+  static std::recursive_mutex mu;
+  return mu;
+}
+
 int probe_device() {
   static std::once_flag once;
   static int cached = kNoDevice;
@@ -24,19 +29,29 @@ int probe_device() {
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) return;
     if (hipSetDevice(0) != hipSuccess) { (void)hipGetLastError(); return; }
     cached = kOk;
+    // Device addresses of the library's own device arrays are looked up here, once, so that no
+    // entry point does it inside a caller's stream capture.  A failure is reported by the entry
+    // point that needs the array.
+    (void)route_scratch_warm();
   });
   return cached;
 }
 
+namespace {
+struct WorkspaceSlot {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+  std::vector<void*> retired;      // outgrown buffers: work queued before the growth may still use them
+};
+std::mutex g_ws_mu;
+std::map<std::pair<int, hipStream_t>, WorkspaceSlot> g_ws_slots;
+}  // namespace
+
 void* stream_workspace(hipStream_t s, size_t bytes) {
-  struct Slot { void* ptr; size_t bytes; };
-  static std::mutex mu;
-  static std::map<std::pair<int, hipStream_t>, Slot> slots;
-  static std::vector<void*> retired;      // outgrown buffers: kept until the process ends
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-  std::lock_guard<std::mutex> lock(mu);
-  Slot& slot = slots[{dev, s}];
+  std::lock_guard<std::mutex> lock(g_ws_mu);
+  WorkspaceSlot& slot = g_ws_slots[{dev, s}];
   if (slot.bytes >= bytes && slot.ptr) return slot.ptr;
   // Work already queued on the stream may still use the old buffer, so it is neither
   // freed nor waited for: it is set aside, and the new one is at least twice its size,
@@ -45,9 +60,31 @@ void* stream_workspace(hipStream_t s, size_t bytes) {
   if (want < 2 * slot.bytes) want = 2 * slot.bytes;
   void* p = nullptr;
   if (hipMalloc(&p, want) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-  if (slot.ptr) retired.push_back(slot.ptr);
-  slot = Slot{p, want};
+  if (slot.ptr) slot.retired.push_back(slot.ptr);
+  slot.ptr = p;
+  slot.bytes = want;
   return p;
+}
+
+// Waits for the stream, then frees its workspace (the buffer in use and the outgrown ones).
+int stream_workspace_release(hipStream_t s) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return kDeviceFailed; }
+  if (hipStreamSynchronize(s) != hipSuccess) { (void)hipGetLastError(); return kDeviceFailed; }
+  WorkspaceSlot gone;
+  {
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    auto it = g_ws_slots.find({dev, s});
+    if (it == g_ws_slots.end()) return kOk;
+    gone = std::move(it->second);
+    g_ws_slots.erase(it);
+  }
+  int rc = kOk;
+  if (gone.ptr && hipFree(gone.ptr) != hipSuccess) rc = kDeviceFailed;
+  for (void* p : gone.retired)
+    if (hipFree(p) != hipSuccess) rc = kDeviceFailed;
+  if (rc != kOk) (void)hipGetLastError();
+  return rc;
 }
 
 struct Timer {
@@ -69,6 +106,11 @@ extern "C" {
 int tessera_gfx950_abi_version(void) { return 1; }
 
 int tessera_gfx950_probe(void) { return probe_device(); }
+
+int tessera_gfx950_stream_release(void* stream) {
+  if (probe_device() != kOk) return kNoDevice;
+  return stream_workspace_release(as_stream(stream));
+}
 
 int tessera_gfx950_device_name(char* buf, int buflen) {
   if (!buf || buflen <= 0) return kBadShape;

@@ -108,7 +108,9 @@ _SIGNATURES = {
     "tessera_gfx950_gemm_w8a8_f32_dev": [_c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_gemm_e4m3_bf16_dev": [_c_vp, _c_vp, _c_f, _c_f, _c_vp, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_gemm_e4m3_f32_dev": [_c_vp, _c_vp, _c_f, _c_f, _c_vp, _c_int, _c_int, _c_int, _c_vp],
+    "tessera_gfx950_stream_release": [_c_vp],
     "tessera_gfx950_gemm_bf16_bench": [_c_int, _c_int, _c_int, _c_int, _P(ctypes.c_double)],
+    "tessera_gfx950_gemm_f16_bench": [_c_int] * 6 + [_P(ctypes.c_double)],
     "tessera_gfx950_gemm_bf16_bench_rotating": [_c_int, _c_int, _c_int, _c_int, _c_int, _P(ctypes.c_double)],
     "tessera_gfx950_bench_last_timer_source": [],
     "tessera_gfx950_mfma_probe_bf16_dev": [_c_vp, _c_int, _c_vp, _P(ctypes.c_double), _c_vp],

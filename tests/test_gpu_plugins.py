@@ -190,6 +190,11 @@ def test_bench_abi(lane):
     assert lib.tessera_gfx950_gemm_bf16_bench(1024, 1024, 1024, 5, ctypes.byref(ms)) == 0
     assert 0 < ms.value < 100
     assert lib.tessera_gfx950_bench_last_timer_source() in (0, 1)
+    # the f16 form carries the parameter list of tessera_rocm_wmma_gemm_f16_bench (mt, nt before avg_ms)
+    assert lib.tessera_gfx950_gemm_f16_bench(1024, 1024, 1024, 5, 4, 2, ctypes.byref(ms)) == 0
+    assert 0 < ms.value < 100 and lib.tessera_gfx950_bench_last_timer_source() in (0, 1)
+    assert lib.tessera_gfx950_gemm_f16_bench(1024, 1024, 1024, 5, 0, 2, ctypes.byref(ms)) == 1
+    assert lib.tessera_gfx950_bench_last_timer_source() == -1
     assert "gfx950" in lane.device_name() and lane.device_cus() > 0
     # the attention forward's bench entry: a failed call resets the timer source, a good one sets it
     assert lib.tessera_gfx950_flash_attn_bf16_bench(1, 4, 3, 64, 64, 128, 1, 3, ctypes.byref(ms)) == 1     # Hq % Hkv

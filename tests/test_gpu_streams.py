@@ -156,6 +156,78 @@ def test_two_threads_two_streams_at_once(lane, hip):
             hip.destroy(s)
 
 
+def test_stream_release_frees_and_a_later_call_reallocates(lane, hip):
+    """`tessera_gfx950_stream_release` waits for the stream and frees its workspace; the next
+    call on the stream sizes a new one and gives the same result.  Releasing a stream that has
+    no workspace is not an error."""
+    lib = lane.load()
+    g = _splitk_case(lane, 61)
+    _gemm(lane, g, None)
+    lane.synchronize()
+    want = _read_gemm(g)
+    s = hip.stream()
+    try:
+        assert lib.tessera_gfx950_stream_release(s) == 0           # nothing kept yet
+        for _ in range(2):
+            _gemm(lane, g, s)
+            assert lib.tessera_gfx950_stream_release(s) == 0       # synchronises, then frees
+            assert np.array_equal(_read_gemm(g), want)
+    finally:
+        hip.destroy(s)
+
+
+def test_host_pointer_entry_points_from_two_threads(lane):
+    """The host-pointer ABI is re-entrant like the reference's (which allocates per call): two
+    host threads inside `tessera_gfx950_gemm_bf16` (a K-split shape, partials in scratch memory)
+    and `tessera_gfx950_moe_route_f32` (routing lists in scratch memory) at the same time must
+    each get what the call gives when it runs alone."""
+    lib = lane.load()
+
+    def make(seed, M, T):
+        rng = np.random.default_rng(seed)
+        N, K, E, k = 1024, 4096, 64, 8
+        a = np.ascontiguousarray(np.asarray(b16.from_float32(rng.standard_normal((M, K)).astype(np.float32) * 0.5),
+                                            np.uint16))
+        b = np.ascontiguousarray(np.asarray(b16.from_float32(rng.standard_normal((K, N)).astype(np.float32) * 0.5),
+                                            np.uint16))
+        lg = rng.standard_normal((T, E)).astype(np.float32)
+        return dict(a=a, b=b, lg=lg, M=M, N=N, K=K, T=T, E=E, k=k)
+
+    def run(c):
+        d = np.zeros((c["M"], c["N"]), np.float32)
+        assert lib.tessera_gfx950_gemm_bf16(c["a"].ctypes.data, c["b"].ctypes.data, d.ctypes.data, c["M"], c["N"],
+                                            c["K"]) == 0
+        S = c["T"] * c["k"]
+        tos, eos = np.zeros(S, np.int32), np.zeros(S, np.int32)
+        cw = np.zeros(S, np.float32)
+        gs, go, n = np.zeros(c["E"], np.int32), np.zeros(c["E"] + 1, np.int32), np.zeros(1, np.int32)
+        assert lib.tessera_gfx950_moe_route_f32(c["lg"].ctypes.data, c["T"], c["E"], c["k"], 1, 0, tos.ctypes.data,
+                                                eos.ctypes.data, cw.ctypes.data, gs.ctypes.data, go.ctypes.data,
+                                                n.ctypes.data) == 0
+        return [d, tos, eos, cw, gs, go, n]
+
+    cases = [make(51, 16, 500), make(52, 32, 800)]
+    want = [run(c) for c in cases]
+    errors = []
+
+    def work(i):
+        try:
+            for round_ in range(25):
+                for idx, (got, ref) in enumerate(zip(run(cases[i]), want[i])):
+                    if not np.array_equal(got, ref):
+                        errors.append((i, round_, idx))
+        except Exception as exc:                          # noqa: BLE001 - reported by the main thread
+            errors.append((i, "raised", repr(exc)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not any(th.is_alive() for th in threads), "a host-pointer thread did not finish"
+    assert not errors, errors[:5]
+
+
 def test_dev_entry_points_under_stream_capture(lane, hip):
     """The `_dev` calls record into a HIP graph (they clear their counters with a fill kernel,
     not a memset node, and take scratch from a workspace that already has its size after one
