@@ -313,6 +313,27 @@ int tessera_gfx950_flash_attn_ext_bf16_dev(const void* Q, const void* K, const v
                                            int causal, int window, float softcap, int out_dtype,
                                            void* stream);
 
+/* Attention forward on strided operands, so that a projection GEMM's output feeds the
+ * kernel where it lies (the reference copies per op, tessera_rocm_gemm.cpp:450-475; its
+ * executor takes [..., H, S, D] only, python/tessera/runtime.py:7229-7475 — no counterpart
+ * for other layouts).  strides: 12 element strides, (batch, head, row) for Q, K, V, O in
+ * that order; element (b, h, s, d) of X lies at X[b*batch + h*head + s*row + d], the last
+ * dimension is contiguous.  [B,S,H,D] is (S*H*D, D, H*D); the Q / K / V column blocks of a
+ * fused (B*S) x ((Hq + 2 Hkv) * D) projection are (S*W, D, W) with W the row width and the
+ * pointers offset to the block's first column.  Strides must be >= 0 (row >= D); the MFMA
+ * kernel needs pointers and strides that are multiples of 8 elements, anything else takes
+ * the per-row kernel.  O (f32 for out_dtype 0, else the storage dtype) is written through
+ * its own strides; LSE is contiguous [B,Hq,Sq] f32 or NULL.  window / softcap as in the
+ * _ext entry points (0 = none). */
+int tessera_gfx950_flash_attn_strided_f16_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, int B,
+                                              int Hq, int Hkv, int Sq, int Sk, int D, const int64_t* strides,
+                                              float scale, int causal, int window, float softcap, int out_dtype,
+                                              void* stream);
+int tessera_gfx950_flash_attn_strided_bf16_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, int B,
+                                               int Hq, int Hkv, int Sq, int Sk, int D, const int64_t* strides,
+                                               float scale, int causal, int window, float softcap, int out_dtype,
+                                               void* stream);
+
 /* Additive attention bias: O = softmax(scale Q K^T + bias, ...) V with bias an f32
  * tensor [B, Hq, Sq, Sk] (the caller broadcasts, as the reference's executor does for
  * its fourth operand, python/tessera/runtime.py:7270-7274); NULL means none.  With a

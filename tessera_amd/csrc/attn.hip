@@ -16,38 +16,73 @@ bool bad_attn(int B, int Hq, int Hkv, int Sq, int Sk, int D) {
   return false;
 }
 
-template <class T, int D, bool EXT>
+template <class T, int DP, bool EXT, bool PAD>
 int launch_flash(const FlashParams& p, hipStream_t s) {
-  constexpr int kSmem = 2 * 2 * FA_BKV * D * 2;
-  auto kern = flash_fwd_kernel<T, D, EXT>;
+  using G = FlashGeom<DP>;
+  auto kern = flash_fwd_kernel<T, DP, EXT, PAD>;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [&] {
     attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, G::SMEM);
   });
   if (attr_err != hipSuccess) return kDeviceFailed;
-  const int qblocks = ceil_div(p.Sq, FA_BQ);
+  const int qblocks = ceil_div(p.Sq, G::BQ);
   const bool xcd_grouped = (p.B * p.Hkv) % 8 == 0;
   const dim3 grid = xcd_grouped ? dim3(8 * p.ratio, qblocks, p.B * p.Hkv / 8) : dim3(p.B * p.Hq, qblocks, 1);
-  hipLaunchKernelGGL(kern, grid, dim3(FA_THREADS), kSmem, s, p);
+  hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), G::SMEM, s, p);
   return launch_status();
 }
+
+// The kernel for head dimension p.D: compiled for DP = 64 / 128 / 256, exact when D == DP
+// (plain and extended forms), zero-padded otherwise (one form, the extended one, serves both).
+template <class T>
+int launch_flash_for(const FlashParams& p, bool ext, hipStream_t s) {
+  switch (p.D) {
+    case 64: return ext ? launch_flash<T, 64, true, false>(p, s) : launch_flash<T, 64, false, false>(p, s);
+    case 128: return ext ? launch_flash<T, 128, true, false>(p, s) : launch_flash<T, 128, false, false>(p, s);
+    case 256: return ext ? launch_flash<T, 256, true, false>(p, s) : launch_flash<T, 256, false, false>(p, s);
+    default: break;
+  }
+  if (p.D < 64) return launch_flash<T, 64, true, true>(p, s);
+  if (p.D < 128) return launch_flash<T, 128, true, true>(p, s);
+  return launch_flash<T, 256, true, true>(p, s);
+}
+
+// Contiguous [B, H, S, D].
+inline FlashStrides bhsd(int H, int S, int D) { return FlashStrides{(long)H * S * D, (long)S * D, (long)D}; }
+// [B, S, H, D]: the rows of a (B * S) x (H * D) matrix, one head's D columns at a time.
+inline FlashStrides bshd(int H, int S, int D) { return FlashStrides{(long)S * H * D, (long)D, (long)H * D}; }
+
+bool bad_strides(const FlashStrides& st) {
+  return st.batch < 0 || st.head < 0 || st.row <= 0;
+}
+bool aligned16(const FlashStrides& st) { return ((st.batch | st.head | st.row) & 7) == 0; }
 
 template <class T>
 int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, int B, int Hq, int Hkv,
               int Sq, int Sk, int D, float scale, int causal, int out_storage, hipStream_t s, int window = 0,
-              float softcap = 0.f, const float* bias = nullptr) {
+              float softcap = 0.f, const float* bias = nullptr, const FlashStrides* strides = nullptr) {
   if (bad_attn(B, Hq, Hkv, Sq, Sk, D) || !Q || !K || !V || !O) return kBadShape;
   if (window < 0 || !(softcap >= 0.f)) return kBadShape;
-  if (probe_device() != kOk) return kNoDevice;
   FlashParams p{};
+  if (strides) {
+    for (int i = 0; i < 4; ++i)
+      if (bad_strides(strides[i])) return kBadShape;
+    p.qs = strides[0]; p.ks = strides[1]; p.vs = strides[2]; p.os = strides[3];
+    if (p.qs.row < D || p.ks.row < D || p.vs.row < D || p.os.row < D) return kBadShape;
+    // per-lane byte offsets inside a 64-key tile are 32-bit
+    if (p.ks.row > (1L << 23) || p.vs.row > (1L << 23)) return kBadShape;
+  } else {
+    p.qs = bhsd(Hq, Sq, D); p.ks = bhsd(Hkv, Sk, D); p.vs = p.ks; p.os = p.qs;
+  }
+  if (probe_device() != kOk) return kNoDevice;
   p.Q = static_cast<const uint16_t*>(Q);
   p.K = static_cast<const uint16_t*>(K);
   p.V = static_cast<const uint16_t*>(V);
   p.O = O;
   p.LSE = static_cast<float*>(LSE);
-  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Sq = Sq; p.Sk = Sk;
+  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Sq = Sq; p.Sk = Sk; p.D = D;
   p.ratio = Hq / Hkv;
   p.scale = scale;
   p.causal = causal ? 1 : 0;
@@ -55,16 +90,29 @@ int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, i
   p.window = window;
   p.softcap = softcap;
   p.bias = bias;
+  // 16-byte accesses: pointers and strides must be multiples of 16 bytes (8 elements of the
+  // 16-bit operands; O in f32 is then aligned as well).
   const bool al = ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
-                    reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(O)) & 15) == 0;
+                    reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(O)) & 15) == 0 &&
+                  aligned16(p.qs) && aligned16(p.ks) && aligned16(p.vs) && aligned16(p.os);
   // The plain variant takes row maxima of the raw scores, which needs scale > 0; the
   // extended one scales first and serves every other scale.
   const bool ext = p.softcap > 0.f || p.bias != nullptr || !(scale > 0.f);
-  if (al && D == 128) return ext ? launch_flash<T, 128, true>(p, s) : launch_flash<T, 128, false>(p, s);
-  if (al && D == 64) return ext ? launch_flash<T, 64, true>(p, s) : launch_flash<T, 64, false>(p, s);
+  if (al) return launch_flash_for<T>(p, ext, s);
   const long rows = (long)B * Hq * Sq;
-  hipLaunchKernelGGL((flash_fwd_generic_kernel<T>), dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, p, D);
+  hipLaunchKernelGGL((flash_fwd_generic_kernel<T>), dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, p);
   return launch_status();
+}
+
+template <class T>
+int flash_strided(const void* Q, const void* K, const void* V, void* O, void* LSE, int B, int Hq, int Hkv, int Sq,
+                  int Sk, int D, const int64_t* strides, float scale, int causal, int window, float softcap,
+                  int out_dtype, void* stream) {
+  if (!strides) return kBadShape;
+  FlashStrides st[4];
+  for (int i = 0; i < 4; ++i) st[i] = FlashStrides{(long)strides[3 * i], (long)strides[3 * i + 1], (long)strides[3 * i + 2]};
+  return flash_dev<T>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, out_dtype, as_stream(stream), window,
+                      softcap, nullptr, st);
 }
 
 template <class T>
@@ -282,6 +330,21 @@ int tessera_gfx950_flash_attn_ext_bf16_dev(const void* Q, const void* K, const v
                                            int window, float softcap, int out_dtype, void* stream) {
   return flash_dev<BF16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, scale, causal, out_dtype, as_stream(stream), window,
                          softcap);
+}
+
+int tessera_gfx950_flash_attn_strided_f16_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, int B,
+                                              int Hq, int Hkv, int Sq, int Sk, int D, const int64_t* strides,
+                                              float scale, int causal, int window, float softcap, int out_dtype,
+                                              void* stream) {
+  return flash_strided<F16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, strides, scale, causal, window, softcap, out_dtype,
+                            stream);
+}
+int tessera_gfx950_flash_attn_strided_bf16_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, int B,
+                                               int Hq, int Hkv, int Sq, int Sk, int D, const int64_t* strides,
+                                               float scale, int causal, int window, float softcap, int out_dtype,
+                                               void* stream) {
+  return flash_strided<BF16>(Q, K, V, O, LSE, B, Hq, Hkv, Sq, Sk, D, strides, scale, causal, window, softcap,
+                             out_dtype, stream);
 }
 
 int tessera_gfx950_flash_attn_bias_f16(const void* Q, const void* K, const void* V, const float* bias, void* O,

@@ -1,8 +1,17 @@
 // Flash-attention forward for gfx950: O = softmax(scale * Q K^T, causal) V with
 // GQA and the per-row log-sum-exp, 16-bit storage, f32 softmax and accumulate.
 //
+// The kernel is compiled for a padded head dimension DP in {64, 128, 256} and serves every
+// head dimension D <= DP that is a multiple of 16 (the matrix path of the reference's
+// kernel, tessera_rocm_flash_attn.cpp:47-144): with D < DP the missing columns of Q, K and
+// V are zeros (registers set to zero, LDS columns cleared once and never loaded), which
+// leaves the scores unchanged and yields output columns that are not stored.  Q, K, V and O
+// are addressed through (batch, head, row) strides, so [B,H,S,D], [B,S,H,D] and column
+// slices of a fused projection output are all served without a copy.
+//
 // One workgroup of 8 waves (two per SIMD) owns 256 query rows of one (batch, q
-// head); each wave owns 32 of them as one MFMA tile.  K/V are walked in 64-key
+// head) (DP = 256: 4 waves, one per SIMD with the whole register file each, 128 rows);
+// each wave owns 32 of them as one MFMA tile.  K/V are walked in 64-key
 // tiles that stream from global memory straight into LDS (two stages each, one
 // barrier per tile).  The loop is software-pipelined: the score MFMAs of tile
 // t+1 are issued under the softmax arithmetic of tile t, and the exponentials of
@@ -35,13 +44,19 @@
 
 namespace tsr950 {
 
+// Element (b, h, s, d) of a strided operand X is X[b * batch + h * head + s * row + d].
+struct FlashStrides {
+  long batch, head, row;
+};
 struct FlashParams {
-  const uint16_t* Q;   // [B, Hq, Sq, D]
-  const uint16_t* K;   // [B, Hkv, Sk, D]
-  const uint16_t* V;   // [B, Hkv, Sk, D]
-  void* O;             // [B, Hq, Sq, D]  f32 or storage dtype
-  float* LSE;          // [B, Hq, Sq] or null
+  const uint16_t* Q;   // (B, Hq, Sq, D) through qs
+  const uint16_t* K;   // (B, Hkv, Sk, D) through ks
+  const uint16_t* V;   // (B, Hkv, Sk, D) through vs
+  void* O;             // (B, Hq, Sq, D) through os, f32 or storage dtype
+  float* LSE;          // [B, Hq, Sq] contiguous, or null
+  FlashStrides qs, ks, vs, os;
   int B, Hq, Hkv, Sq, Sk;
+  int D;               // head dimension, a multiple of 16, <= the kernel's DP
   float scale;
   int causal;
   int out_storage;     // 0: f32 O, 1: O in the storage dtype
@@ -67,12 +82,20 @@ __host__ __device__ inline void key_bounds(int i, int Sq, int Sk, int causal, in
   hi = hi < Sk - 1 ? hi : Sk - 1;
 }
 
-constexpr int FA_BQ = 256;             // query rows per workgroup
 constexpr int FA_QT = 1;               // 32-row query tiles per wave
-constexpr int FA_WAVES = FA_BQ / (32 * FA_QT);
-constexpr int FA_THREADS = FA_WAVES * 64;
 constexpr int FA_BKV = 64;             // keys per LDS tile
-constexpr int FA_KT = FA_BKV / 32;     // 32-key MFMA tiles per LDS tile
+// Per padded head dimension: waves per workgroup (two per SIMD while a wave's accumulators,
+// Q fragments and score tiles fit 256 registers, else one per SIMD), query rows per
+// workgroup, 16-byte chunks per LDS row, bytes of one K (or V) stage, LDS bytes.
+template <int DP> struct FlashGeom {
+  static constexpr int WAVES = DP > 128 ? 4 : 8;
+  static constexpr int THREADS = WAVES * 64;
+  static constexpr int BQ = WAVES * 32 * FA_QT;
+  static constexpr int CHUNKS = DP / 8;
+  static constexpr int TILE = FA_BKV * DP * 2;
+  static constexpr int STAGE_PITCH = DP * 4 + 16;              // epilogue staging row, f32
+  static constexpr int SMEM = 4 * TILE > WAVES * 32 * FA_QT * STAGE_PITCH ? 4 * TILE : WAVES * 32 * FA_QT * STAGE_PITCH;
+};
 constexpr float FA_NEG = -1.0e30f;
 
 // Exchange a value with the lane 32 positions away.
@@ -124,8 +147,12 @@ __device__ __forceinline__ float scale_acc(float acc, float corr) {
   return acc;
 }
 
-template <class T, int D, bool EXT>
-__global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashParams p) {
+template <class T, int DP, bool EXT, bool PAD>
+__global__ __launch_bounds__(FlashGeom<DP>::THREADS, 1) void flash_fwd_kernel(const FlashParams p) {
+  using G = FlashGeom<DP>;
+  constexpr int D = DP;                  // extent the loops are unrolled for
+  constexpr int FA_WAVES = G::WAVES, FA_THREADS = G::THREADS, FA_BQ = G::BQ;
+  constexpr int FA_KT = FA_BKV / 32;     // 32-key MFMA tiles per LDS tile
   constexpr int QT = FA_QT;
   constexpr int KSTEPS = D / 16;         // MFMA k steps of the score product
   constexpr int KA = (KSTEPS + 3) / 4;   // score k steps issued under the row-max phase
@@ -138,8 +165,10 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
   static_assert(FA_BKV * CHUNKS % FA_THREADS == 0, "tile/thread mismatch");
   // K swizzle: the 16 rows an LDS cycle serves must hit 16 different 16-byte slots
   // of the 256-byte bank line.  V swizzle: the 4 rows of a patch, 64 bytes each.
-  auto kswz = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
-  auto vswz = [](int key) { return D == 128 ? ((key & 3) << 2) : (((key >> 1) & 1) << 2); };
+  // (Rows of 256 or 512 bytes start in the same bank: 16 different chunks, and four keys a
+  // 64-byte step apart; rows of 128 bytes alternate between the two halves of the banks.)
+  auto kswz = [](int row) { return CHUNKS % 16 == 0 ? (row & 15) : ((row >> 1) & 7); };
+  auto vswz = [](int key) { return CHUNKS % 16 == 0 ? ((key & 3) << 2) : (((key >> 1) & 1) << 2); };
 
   // LDS: K stages at 0 and TILE, V stages at 2 TILE and 3 TILE.
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -170,6 +199,8 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
     qlin = blockIdx.x;
     kvlin = qlin / p.ratio;
   }
+  const int batch = kvlin / p.Hkv;
+  const int hkv = kvlin - batch * p.Hkv, hq = qlin - batch * p.Hq;
 
   const int q0 = qb * FA_BQ;                  // first query row of the workgroup
   // Waves w and w + 4 share a SIMD.  Under a causal mask a wave's key range grows with
@@ -177,9 +208,10 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
   // gets one of the blocks 0-3 and its mirror image 7-4, the same work on all four.
   const int rblk = wave < FA_WAVES / 2 ? wave : FA_WAVES + FA_WAVES / 2 - 1 - wave;
   const int qw = q0 + rblk * (32 * QT);       // first query row of the wave
-  const uint16_t* Qb = p.Q + ((long)qlin * p.Sq) * D;
-  const uint16_t* Kb = p.K + ((long)kvlin * p.Sk) * D;
-  const uint16_t* Vb = p.V + ((long)kvlin * p.Sk) * D;
+  const uint16_t* Qb = p.Q + batch * p.qs.batch + hq * p.qs.head;
+  const uint16_t* Kb = p.K + batch * p.ks.batch + hkv * p.ks.head;
+  const uint16_t* Vb = p.V + batch * p.vs.batch + hkv * p.vs.head;
+  const int ksteps_real = PAD ? p.D / 16 : KSTEPS;      // k steps that hold data; the rest is zero padding
 
   // Key tiles this workgroup needs: from the first visible key of its first row to
   // the last visible key of its last row (bounds are monotone in the row index).
@@ -206,43 +238,55 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
   for (int qt = 0; qt < QT; ++qt) {
     int row = qw + 32 * qt + l32;
     row = row < p.Sq ? row : p.Sq - 1;
-    const uint16_t* src = Qb + (long)row * D + 8 * lh;
+    const uint16_t* src = Qb + (long)row * p.qs.row + 8 * lh;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qf[qt][ks] = *reinterpret_cast<const uint4*>(src + 16 * ks);
+    for (int ks = 0; ks < KSTEPS; ++ks)
+      qf[qt][ks] = (!PAD || ks < ksteps_real) ? *reinterpret_cast<const uint4*>(src + 16 * ks) : make_uint4(0u, 0u, 0u, 0u);
   }
 
   // ---- K/V tile loaders: straight from global memory into LDS ----------------------
   // One wave instruction fills 64 consecutive 16-byte LDS slots; slot P is (row
   // P / CHUNKS, physical chunk P % CHUNKS) and holds the row's logical chunk
   // (physical ^ swizzle(row)), so the swizzle is applied on the global address.
+  // With D < DP the chunks past the row's end are never loaded (those lanes sit out): their
+  // LDS slots keep the zeros written below.
   int ld_row[LD_PER_THREAD];
   uint32_t ld_koff[LD_PER_THREAD], ld_voff[LD_PER_THREAD];   // byte offsets inside a full tile
+  bool ld_kok[LD_PER_THREAD], ld_vok[LD_PER_THREAD];
+  const uint32_t krow_bytes = (uint32_t)p.ks.row * 2, vrow_bytes = (uint32_t)p.vs.row * 2;
 #pragma unroll
   for (int q = 0; q < LD_PER_THREAD; ++q) {
     const int P = (wave * LD_PER_THREAD + q) * 64 + lane;
     const int row = P / CHUNKS, chp = P % CHUNKS;
     ld_row[q] = row;
-    ld_koff[q] = row * ROWB + ((chp ^ kswz(row)) << 4);
-    ld_voff[q] = row * ROWB + ((chp ^ vswz(row)) << 4);
+    ld_koff[q] = row * krow_bytes + ((chp ^ kswz(row)) << 4);
+    ld_voff[q] = row * vrow_bytes + ((chp ^ vswz(row)) << 4);
+    ld_kok[q] = !PAD || (chp ^ kswz(row)) < 2 * ksteps_real;
+    ld_vok[q] = !PAD || (chp ^ vswz(row)) < 2 * ksteps_real;
+  }
+  if constexpr (PAD) {
+    for (int o = tid * 16; o < 4 * TILE; o += FA_THREADS * 16) lds_write_b128(smem, o, make_uint4(0u, 0u, 0u, 0u));
+    __syncthreads();
   }
   // Full tiles use the precomputed per-lane offsets on a uniform tile base; the
   // ragged last tile clamps its rows (rows past the end are masked in the scores
   // and meet P = 0 in the second product).
-  auto load_tile = [&](const uint16_t* base, const uint32_t (&offs)[LD_PER_THREAD], int tile, int lds_stage) {
-    const uint16_t* tb = base + (long)tile * FA_BKV * D;
+  auto load_tile = [&](const uint16_t* base, long row_elems, uint32_t row_bytes, const uint32_t (&offs)[LD_PER_THREAD],
+                       const bool (&ok)[LD_PER_THREAD], int tile, int lds_stage) {
+    const uint16_t* tb = base + (long)tile * FA_BKV * row_elems;
     const bool full = (tile + 1) * FA_BKV <= p.Sk;
 #pragma unroll
     for (int q = 0; q < LD_PER_THREAD; ++q) {
       uint32_t o = offs[q];
       if (!full) {
         const int last = p.Sk - 1 - tile * FA_BKV;        // last valid row of this tile
-        if (ld_row[q] > last) o -= (uint32_t)(ld_row[q] - last) * ROWB;
+        if (ld_row[q] > last) o -= (uint32_t)(ld_row[q] - last) * row_bytes;
       }
-      load16_to_lds(tb, o, lds0 + lds_stage * TILE + (wave * LD_PER_THREAD + q) * 1024);
+      if (!PAD || ok[q]) load16_to_lds(tb, o, lds0 + lds_stage * TILE + (wave * LD_PER_THREAD + q) * 1024);
     }
   };
-  auto load_k = [&](int tile, int stage) { load_tile(Kb, ld_koff, tile, stage); };
-  auto load_v = [&](int tile, int stage) { load_tile(Vb, ld_voff, tile, 2 + stage); };
+  auto load_k = [&](int tile, int stage) { load_tile(Kb, p.ks.row, krow_bytes, ld_koff, ld_kok, tile, stage); };
+  auto load_v = [&](int tile, int stage) { load_tile(Vb, p.vs.row, vrow_bytes, ld_voff, ld_vok, tile, 2 + stage); };
 
   // ---- state -----------------------------------------------------------------
   f32x16 o_acc[QT][DT];
@@ -510,16 +554,22 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
   for (; t < ntiles; ++t) idle_step(t);
 
   // ---- epilogue -------------------------------------------------------------------
+  // A lane owns 4-column pieces of ONE output row: stored from the registers, a wave
+  // instruction would touch 32 rows with 16 or 32 bytes each.  Every wave therefore passes its
+  // 32 x D tile through its own slice of the (now idle) LDS and writes whole rows, 16 bytes per
+  // lane with consecutive lanes along a row.  The last loop barrier has passed, so no wave
+  // reads K or V any more.
+  const int dreal = PAD ? p.D : D;
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     const int qi = qw + 32 * qt + l32;
     float l = l_run[qt] + swap_half(l_run[qt]);
-    if (qi >= p.Sq) continue;
     if (khi[qt] < klo[qt]) l = 0.f;                      // no visible key: O = 0, LSE = -inf
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     const long row = (long)qlin * p.Sq + qi;
-    if (p.LSE && lh == 0)
+    if (p.LSE && lh == 0 && qi < p.Sq)
       p.LSE[row] = l > 0.f ? (m_run[qt] * cs + __log2f(l)) * 0.69314718055994530942f : -INFINITY;
+    char* stage = smem + (wave * QT + qt) * 32 * G::STAGE_PITCH;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -531,18 +581,30 @@ __global__ __launch_bounds__(FA_THREADS, 1) void flash_fwd_kernel(const FlashPar
           uint2 pk;
           pk.x = pack2<T>(v0, v1);
           pk.y = pack2<T>(v2, v3);
-          *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.O) + row * D + d) = pk;
+          *reinterpret_cast<uint2*>(stage + l32 * G::STAGE_PITCH + d * 2) = pk;
         } else {
-          *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.O) + row * D + d) = make_float4(v0, v1, v2, v3);
+          *reinterpret_cast<float4*>(stage + l32 * G::STAGE_PITCH + d * 4) = make_float4(v0, v1, v2, v3);
         }
       }
+    // rows of dreal elements, 16 bytes per lane
+    const int esz = p.out_storage ? 2 : 4;
+    const int per_row = dreal * esz / 16;                  // 16-byte pieces per output row
+    const int rows_here = min(32, p.Sq - (qw + 32 * qt));
+    char* Ob = reinterpret_cast<char*>(p.O) + (batch * p.os.batch + hq * p.os.head) * esz;
+    for (int idx = lane; idx < rows_here * per_row; idx += 64) {
+      const int r = idx / per_row, c = idx - r * per_row;
+      const uint4 v = *reinterpret_cast<const uint4*>(stage + r * G::STAGE_PITCH + c * 16);
+      *reinterpret_cast<uint4*>(Ob + ((long)(qw + 32 * qt + r) * p.os.row) * esz + c * 16) = v;
+    }
   }
 }
 
-// Any head dimension: one thread per query row, streaming online softmax in f32.
-// Serves the shapes the MFMA kernel does not (D not 64 or 128).
+// Any head dimension and any alignment: one thread per query row, streaming online softmax
+// in f32.  Serves only operands the MFMA kernel cannot address (pointers or strides that are
+// not multiples of 16 bytes).
 template <class T>
-__global__ void flash_fwd_generic_kernel(const FlashParams p, int D) {
+__global__ void flash_fwd_generic_kernel(const FlashParams p) {
+  const int D = p.D;
   const long row = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const long total = (long)p.B * p.Hq * p.Sq;
   if (row >= total) return;
@@ -550,9 +612,9 @@ __global__ void flash_fwd_generic_kernel(const FlashParams p, int D) {
   const int hq = (int)((row / p.Sq) % p.Hq);
   const int b = (int)(row / ((long)p.Sq * p.Hq));
   const int hkv = (int)(((long)hq * p.Hkv) / p.Hq);
-  const uint16_t* q = p.Q + row * D;
-  const uint16_t* Kb = p.K + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
-  const uint16_t* Vb = p.V + ((long)(b * p.Hkv + hkv) * p.Sk) * D;
+  const uint16_t* q = p.Q + b * p.qs.batch + hq * p.qs.head + qi * p.qs.row;
+  const uint16_t* Kb = p.K + b * p.ks.batch + hkv * p.ks.head;
+  const uint16_t* Vb = p.V + b * p.vs.batch + hkv * p.vs.head;
   float acc[256];
   for (int d = 0; d < D; ++d) acc[d] = 0.f;
   float m = -INFINITY, l = 0.f;
@@ -560,7 +622,7 @@ __global__ void flash_fwd_generic_kernel(const FlashParams p, int D) {
   key_bounds(qi, p.Sq, p.Sk, p.causal, p.window, jmin, jmax);
   for (int j = jmin; j <= jmax; ++j) {
     float s = 0.f;
-    for (int d = 0; d < D; ++d) s += from_storage<T>(q[d]) * from_storage<T>(Kb[(long)j * D + d]);
+    for (int d = 0; d < D; ++d) s += from_storage<T>(q[d]) * from_storage<T>(Kb[(long)j * p.ks.row + d]);
     s *= p.scale;
     if (p.softcap > 0.f) s = p.softcap * tanhf(s / p.softcap);
     if (p.bias) s += p.bias[row * p.Sk + j];
@@ -568,15 +630,16 @@ __global__ void flash_fwd_generic_kernel(const FlashParams p, int D) {
     const float cr = __expf(m - mn);       // exp(-inf) = 0 on the first key
     const float e = __expf(s - mn);
     l = l * cr + e;
-    for (int d = 0; d < D; ++d) acc[d] = acc[d] * cr + e * from_storage<T>(Vb[(long)j * D + d]);
+    for (int d = 0; d < D; ++d) acc[d] = acc[d] * cr + e * from_storage<T>(Vb[(long)j * p.vs.row + d]);
     m = mn;
   }
   const float inv = l > 0.f ? 1.0f / l : 0.f;
   if (p.LSE) p.LSE[row] = l > 0.f ? m + __logf(l) : -INFINITY;
+  const long o_at = b * p.os.batch + hq * p.os.head + qi * p.os.row;
   for (int d = 0; d < D; ++d) {
     const float v = acc[d] * inv;
-    if (p.out_storage) reinterpret_cast<uint16_t*>(p.O)[row * D + d] = to_storage<T>(v);
-    else reinterpret_cast<float*>(p.O)[row * D + d] = v;
+    if (p.out_storage) reinterpret_cast<uint16_t*>(p.O)[o_at + d] = to_storage<T>(v);
+    else reinterpret_cast<float*>(p.O)[o_at + d] = v;
   }
 }
 

@@ -129,6 +129,8 @@ _SIGNATURES = {
     "tessera_gfx950_flash_attn_ext_bf16": [_c_vp] * 5 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f],
     "tessera_gfx950_flash_attn_ext_f16_dev": [_c_vp] * 5 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f, _c_int, _c_vp],
     "tessera_gfx950_flash_attn_ext_bf16_dev": [_c_vp] * 5 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f, _c_int, _c_vp],
+    "tessera_gfx950_flash_attn_strided_f16_dev": [_c_vp] * 5 + [_c_int] * 6 + [_c_vp, _c_f, _c_int, _c_int, _c_f, _c_int, _c_vp],
+    "tessera_gfx950_flash_attn_strided_bf16_dev": [_c_vp] * 5 + [_c_int] * 6 + [_c_vp, _c_f, _c_int, _c_int, _c_f, _c_int, _c_vp],
     "tessera_gfx950_flash_attn_bias_f16": [_c_vp] * 6 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f],
     "tessera_gfx950_flash_attn_bias_bf16": [_c_vp] * 6 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f],
     "tessera_gfx950_flash_attn_bias_f16_dev": [_c_vp] * 6 + [_c_int] * 6 + [_c_f, _c_int, _c_int, _c_f, _c_int, _c_vp],

@@ -11,7 +11,7 @@ stream, and nothing synchronises until :meth:`DeviceArray.to_host`.
 
     x = DeviceArray.from_host(x_bf16);  wq = DeviceArray.from_host(wq_bf16)  # once
     q = gemm(x, wq)                                  # stays on the device
-    o = flash_attn(q4, k4, v4, causal=True)          # consumes device handles
+    o = flash_attn(q.reshape(B, S, H, D), k4, v4, causal=True, layout="bshd")   # reads the projections in place
     y = moe_layer(h, w_router, wg, wu, wd, top_k=8)  # router product -> routing -> experts -> combine
     y.to_host()
 
@@ -129,24 +129,66 @@ matmul = gemm
 batched_gemm = gemm
 
 
+def _attention_call(st, q_ptr, k_ptr, v_ptr, O, L, B, Hq, Hkv, Sq, Sk, D, strides, sc, causal, window, softcap, out):
+    arr = (ctypes.c_int64 * 12)(*strides)
+    fn = getattr(_lane.load(), f"tessera_gfx950_flash_attn_strided_{st}_dev")
+    _lane.check(fn(q_ptr, k_ptr, v_ptr, O.ptr, L.ptr if L else None, B, Hq, Hkv, Sq, Sk, D, arr, ctypes.c_float(sc),
+                   1 if causal else 0, int(window), ctypes.c_float(softcap), 0 if out == "f32" else 1, None),
+                "flash_attn")
+
+
 def flash_attn(Q: DeviceArray, K: DeviceArray, V: DeviceArray, *, scale: Optional[float] = None,
-               causal: bool = False, return_lse: bool = False, out: str = "storage"):
-    """Attention forward on ``[B, Hq, Sq, D]`` / ``[B, Hkv, Sk, D]`` handles (GQA when
-    ``Hq != Hkv``); ``out`` ``"storage"`` or ``"f32"``; the log-sum-exp ``[B, Hq, Sq]`` f32
-    on request."""
+               causal: bool = False, return_lse: bool = False, out: str = "storage", layout: str = "bhsd",
+               window: int = 0, logit_softcap: float = 0.0):
+    """Attention forward on device handles (GQA when ``Hq != Hkv``); ``out`` ``"storage"`` or
+    ``"f32"``; the log-sum-exp ``[B, Hq, Sq]`` f32 on request.
+
+    ``layout="bhsd"``: ``Q [B, Hq, Sq, D]``, ``K, V [B, Hkv, Sk, D]`` (the reference's layout).
+    ``layout="bshd"``: ``Q [B, Sq, Hq, D]``, ``K, V [B, Sk, Hkv, D]`` — what a projection
+    ``x[B, S, E] @ W[E, H * D]`` leaves in memory (reshape the handle, no copy); the output
+    comes back in the same layout, ready for the output projection."""
     st = _storage(Q, K, V)
+    if layout not in ("bhsd", "bshd"):
+        raise ValueError("layout must be 'bhsd' or 'bshd'")
     if Q.ndim != 4 or K.ndim != 4 or V.shape != K.shape or K.shape[0] != Q.shape[0] or K.shape[3] != Q.shape[3]:
         raise ValueError(f"flash_attn: Q {Q.shape}, K {K.shape}, V {V.shape}")
-    B, Hq, Sq, D = Q.shape
-    Hkv, Sk = K.shape[1], K.shape[2]
+    if layout == "bhsd":
+        B, Hq, Sq, D = Q.shape
+        Hkv, Sk = K.shape[1], K.shape[2]
+        qst, kst = (Hq * Sq * D, Sq * D, D), (Hkv * Sk * D, Sk * D, D)
+    else:
+        B, Sq, Hq, D = Q.shape
+        Sk, Hkv = K.shape[1], K.shape[2]
+        qst, kst = (Sq * Hq * D, D, Hq * D), (Sk * Hkv * D, D, Hkv * D)
     if Hq % Hkv:
         raise ValueError("the number of query heads must be a multiple of the KV heads")
     sc = float(scale) if scale is not None else 1.0 / math.sqrt(D)
     O = DeviceArray(Q.shape, "f32" if out == "f32" else st)
     L = DeviceArray((B, Hq, Sq), "f32") if return_lse else None
-    fn = getattr(_lane.load(), f"tessera_gfx950_flash_attn_gqa_{st}_dev")
-    _lane.check(fn(Q.ptr, K.ptr, V.ptr, O.ptr, L.ptr if L else None, B, Hq, Hkv, Sq, Sk, D, ctypes.c_float(sc),
-                   1 if causal else 0, 0 if out == "f32" else 1, None), "flash_attn")
+    _attention_call(st, Q.ptr, K.ptr, V.ptr, O, L, B, Hq, Hkv, Sq, Sk, D, qst + kst + kst + qst, sc, causal, window,
+                    logit_softcap, out)
+    return (O, L) if return_lse else O
+
+
+def flash_attn_fused_qkv(QKV: DeviceArray, num_q_heads: int, num_kv_heads: int, *, scale: Optional[float] = None,
+                         causal: bool = False, return_lse: bool = False, out: str = "storage"):
+    """Attention forward on the output of ONE fused projection ``x[B, S, E] @ Wqkv[E, (Hq + 2 Hkv) * D]``:
+    ``QKV [B, S, (Hq + 2 Hkv) * D]`` holds, per token, the query heads, then the key heads, then
+    the value heads.  The kernel reads the three column blocks in place through row strides;
+    returns ``O [B, S, Hq, D]`` (and ``LSE [B, Hq, S]``)."""
+    st = _storage(QKV)
+    if QKV.ndim != 3 or QKV.shape[2] % (num_q_heads + 2 * num_kv_heads) or num_q_heads % num_kv_heads:
+        raise ValueError(f"flash_attn_fused_qkv: QKV {QKV.shape} for {num_q_heads} + 2 x {num_kv_heads} heads")
+    B, S, W = QKV.shape
+    D = W // (num_q_heads + 2 * num_kv_heads)
+    sc = float(scale) if scale is not None else 1.0 / math.sqrt(D)
+    O = DeviceArray((B, S, num_q_heads, D), "f32" if out == "f32" else st)
+    L = DeviceArray((B, num_q_heads, S), "f32") if return_lse else None
+    inb, outb = (S * W, D, W), (S * num_q_heads * D, D, num_q_heads * D)
+    k_ptr = QKV.ptr + num_q_heads * D * 2
+    v_ptr = k_ptr + num_kv_heads * D * 2
+    _attention_call(st, QKV.ptr, k_ptr, v_ptr, O, L, B, num_q_heads, num_kv_heads, S, S, D, inb + inb + inb + outb, sc,
+                    causal, 0, 0.0, out)
     return (O, L) if return_lse else O
 
 

@@ -128,6 +128,55 @@ def test_headline_config_properties(lane):
         assert np.max(np.abs(lse[b, h] - ref_lse[b, h])) <= TOL
 
 
+HEAD_DIMS = [16, 32, 48, 64, 80, 96, 112, 128, 144, 160, 192, 208, 256]
+
+
+@pytest.mark.parametrize("D", HEAD_DIMS)
+@pytest.mark.parametrize("st", ["bf16", "f16"])
+def test_every_head_dim_on_the_matrix_path(lane, D, st):
+    """Every head dimension that is a multiple of 16 runs the MFMA kernel (zero-padded to the
+    next compiled width, as the reference's kernel serves every D % 16 == 0 on its matrix
+    path, tessera_rocm_flash_attn.cpp:47-144): causal GQA with a ragged last tile, plus the
+    soft-capped, windowed form."""
+    B, Hq, Hkv, Sq, Sk = 1, 4, 2, 150, 203
+    q, k, v = _qkv(B, Hq, Hkv, Sq, Sk, D, 100 + D, st)
+    ref_o, ref_lse = orc.flash_attn_dense(_f32(q), _f32(k), _f32(v), causal=True)
+    o, lse = ops.gqa_attention(q, k, v, causal=True, return_lse=True, out="f32")
+    assert not np.isnan(o).any()
+    assert orc.max_rel_err(o, ref_o) <= TOL
+    assert np.max(np.abs(lse - ref_lse)) <= TOL
+    o16 = ops.gqa_attention(q, k, v, causal=True)
+    want16 = b16.from_float32(o) if st == "bf16" else o.astype(np.float16)
+    assert np.array_equal(np.asarray(o16, np.uint16) if st == "bf16" else o16.view(np.uint16),
+                          np.asarray(want16, np.uint16) if st == "bf16" else want16.view(np.uint16))
+    ref_o, ref_lse = orc.flash_attn_dense(_f32(q), _f32(k), _f32(v), causal=True, window=70, softcap=4.0)
+    o, lse = ops.gqa_attention(q, k, v, causal=True, return_lse=True, out="f32", window=70, logit_softcap=4.0)
+    assert orc.max_rel_err(o, ref_o) <= TOL
+    assert np.max(np.abs(lse - ref_lse)) <= TOL
+
+
+def test_mfma_kernel_is_the_one_that_runs_for_padded_head_dims(lane):
+    """The per-row kernel serves unaligned operands only: at S = 2048 it would take tens of
+    milliseconds per launch, the MFMA kernel well under one."""
+    import ctypes, time
+    B, Hq, Hkv, S, D = 1, 16, 4, 2048, 96
+    q, k, v = _qkv(B, Hq, Hkv, S, S, D, 5, "bf16")
+    dq, dk, dv = (lane.DeviceBuffer.from_host(np.asarray(x, np.uint16)) for x in (q, k, v))
+    do = lane.DeviceBuffer(B * Hq * S * D * 2)
+    fn = lane.load().tessera_gfx950_flash_attn_gqa_bf16_dev
+    run = lambda: fn(dq.ptr, dk.ptr, dv.ptr, do.ptr, None, B, Hq, Hkv, S, S, D, ctypes.c_float(D ** -0.5), 1, 1, None)
+    for _ in range(3):
+        assert run() == 0
+    lane.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        run()
+    lane.synchronize()
+    ms = (time.perf_counter() - t0) / 10 * 1e3
+    flop = 4.0 * B * Hq * (S * (S + 1) / 2) * D
+    assert flop / ms / 1e9 > 20.0, f"{ms:.3f} ms per launch: not the matrix path"
+
+
 def test_attention_rejects_bad_shapes(lane):
     lib = lane.load()
     z = np.zeros(1024, np.uint16)

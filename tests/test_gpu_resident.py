@@ -12,8 +12,16 @@ from tessera_amd import resident as rs
 pytestmark = pytest.mark.gpu
 
 
+def _heads_first(t, B, S, h, D):
+    """[B, S, h*D] bits -> [B, h, S, D] BF16Array (host-side head split, for the reference chain)."""
+    return b16.from_bits(np.ascontiguousarray(np.asarray(t, np.uint16).reshape(B, S, h, D).transpose(0, 2, 1, 3)))
+
+
 def test_projection_then_attention_chain(lane):
-    """x @ Wq / Wk / Wv -> attention -> @ Wo with no host hop in between."""
+    """x @ Wq / Wk / Wv -> attention -> @ Wo with NO host hop: the attention kernel reads the
+    projections where the GEMMs left them ([B, S, H, D] through row strides) and writes its
+    output in the layout the output projection consumes.  Nothing is downloaded before the
+    chain's result; the intermediates are fetched afterwards only to check them."""
     B, S, Hq, Hkv, D, E = 2, 192, 4, 2, 64, 256
     rng = np.random.default_rng(3)
     x = (rng.standard_normal((B, S, E)) * 0.5).astype(np.float32)
@@ -25,27 +33,66 @@ def test_projection_then_attention_chain(lane):
     q = rs.gemm(dx, dwq)                                           # (B, S, Hq*D) bf16, resident
     k, v = rs.gemm(dx, dwk), rs.gemm(dx, dwv)
     assert q.shape == (B, S, Hq * D) and q.dtype == "bf16"
-    # head split: the host-side reference does the same transposition on downloaded copies
-    heads = lambda t, h: b16.from_bits(np.ascontiguousarray(
-        np.asarray(t.to_host(), np.uint16).reshape(B, S, h, D).transpose(0, 2, 1, 3)))
-    q4, k4, v4 = (rs.DeviceArray.from_host(heads(t, h)) for t, h in ((q, Hq), (k, Hkv), (v, Hkv)))
-    o, lse = rs.flash_attn(q4, k4, v4, causal=True, return_lse=True)
-    merged = rs.DeviceArray.from_host(b16.from_bits(np.ascontiguousarray(
-        np.asarray(o.to_host(), np.uint16).transpose(0, 2, 1, 3).reshape(B, S, Hq * D))))
-    y = rs.gemm(merged, dwo, out="f32").to_host()
-    # the same chain through the host-pointer ops: identical bits
+    o, lse = rs.flash_attn(q.reshape(B, S, Hq, D), k.reshape(B, S, Hkv, D), v.reshape(B, S, Hkv, D), causal=True,
+                           return_lse=True, layout="bshd")
+    assert o.shape == (B, S, Hq, D)
+    y = rs.gemm(o.reshape(B, S, Hq * D), dwo, out="f32").to_host()  # the first download of the chain
+    # the same chain through the host-pointer ops (which copy and transpose on the host): identical bits
     hq, hk, hv = ops.gemm(xb, wqb), ops.gemm(xb, wkb), ops.gemm(xb, wvb)
     assert np.array_equal(np.asarray(hq, np.uint16), np.asarray(q.to_host(), np.uint16))
-    t4 = lambda t, h: b16.from_bits(np.ascontiguousarray(np.asarray(t, np.uint16).reshape(B, S, h, D).transpose(0, 2, 1, 3)))
-    ho, hl = ops.gqa_attention(t4(hq, Hq), t4(hk, Hkv), t4(hv, Hkv), causal=True, return_lse=True)
-    assert np.array_equal(np.asarray(ho, np.uint16), np.asarray(o.to_host(), np.uint16))
+    q4, k4, v4 = _heads_first(hq, B, S, Hq, D), _heads_first(hk, B, S, Hkv, D), _heads_first(hv, B, S, Hkv, D)
+    ho, hl = ops.gqa_attention(q4, k4, v4, causal=True, return_lse=True)
+    o_bits = np.asarray(o.to_host(), np.uint16)                    # [B, S, Hq, D]
+    assert np.array_equal(np.asarray(ho, np.uint16), o_bits.transpose(0, 2, 1, 3))
     assert np.array_equal(hl, lse.to_host())
-    # and the oracle on the attention stage
-    ro, rl = orc.flash_attn_dense(t4(hq, Hq).to_float32(), t4(hk, Hkv).to_float32(), t4(hv, Hkv).to_float32(), causal=True)
-    assert orc.max_rel_err(o.to_host().to_float32(), ro) <= 2e-3 + 2.0 ** -8
+    # and the oracle on the attention stage and on the output projection
+    ro, rl = orc.flash_attn_dense(q4.to_float32(), k4.to_float32(), v4.to_float32(), causal=True)
+    got_o = b16.from_bits(np.ascontiguousarray(o_bits.transpose(0, 2, 1, 3))).to_float32()
+    assert orc.max_rel_err(got_o, ro) <= 2e-3 + 2.0 ** -8
+    assert np.max(np.abs(lse.to_host() - rl)) <= 2e-3
     assert y.shape == (B, S, E) and np.isfinite(y).all()
-    ref_y = orc.gemm_f64(merged.to_host().to_float32().reshape(B * S, -1), wob.to_float32())
+    ref_y = orc.gemm_f64(b16.from_bits(o_bits).to_float32().reshape(B * S, -1), wob.to_float32())
     assert orc.max_rel_err(y.reshape(B * S, E), ref_y) <= 1e-5
+    host_y = ops.gemm(b16.from_bits(np.ascontiguousarray(o_bits.reshape(B * S, Hq * D))), wob, out="f32")
+    assert np.array_equal(host_y.view(np.uint32), y.reshape(B * S, E).view(np.uint32))
+
+
+def test_fused_qkv_projection_feeds_attention_in_place(lane):
+    """ONE projection x @ [Wq | Wk | Wv]; the attention kernel reads its three column blocks
+    through row strides (pointers offset to each block), f16 storage, D = 128."""
+    B, S, Hq, Hkv, D, E = 1, 300, 4, 1, 128, 192
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((B, S, E)) * 0.5).astype(np.float16)
+    w = (rng.standard_normal((E, (Hq + 2 * Hkv) * D)) / 12).astype(np.float16)
+    qkv = rs.gemm(rs.DeviceArray.from_host(x), rs.DeviceArray.from_host(w))
+    o, lse = rs.flash_attn_fused_qkv(qkv, Hq, Hkv, causal=True, return_lse=True, out="f32")
+    h = np.asarray(qkv.to_host()).reshape(B, S, Hq + 2 * Hkv, D).transpose(0, 2, 1, 3).astype(np.float32)
+    ro, rl = orc.flash_attn_dense(h[:, :Hq], h[:, Hq:Hq + Hkv], h[:, Hq + Hkv:], causal=True)
+    assert orc.max_rel_err(o.to_host().transpose(0, 2, 1, 3), ro) <= 2e-3
+    assert np.max(np.abs(lse.to_host() - rl)) <= 2e-3
+    # the contiguous entry point on host-transposed copies gives the same bits
+    c = np.ascontiguousarray
+    o2, l2 = ops.gqa_attention(c(h[:, :Hq]).astype(np.float16), c(h[:, Hq:Hq + Hkv]).astype(np.float16),
+                               c(h[:, Hq + Hkv:]).astype(np.float16), causal=True, return_lse=True, out="f32")
+    assert np.array_equal(o2, o.to_host().transpose(0, 2, 1, 3)) and np.array_equal(l2, lse.to_host())
+
+
+def test_strided_attention_rejects_bad_strides(lane):
+    import ctypes
+    lib = lane.load()
+    z = lane.DeviceBuffer(1 << 16)
+    def call(strides, D=64):
+        arr = (ctypes.c_int64 * 12)(*strides)
+        return lib.tessera_gfx950_flash_attn_strided_bf16_dev(z.ptr, z.ptr, z.ptr, z.ptr, None, 1, 2, 2, 16, 16, D, arr,
+                                                              ctypes.c_float(0.125), 1, 0, ctypes.c_float(0.0), 1, None)
+    good = (2 * 16 * 64, 64, 128) * 4
+    assert call(good) == 0
+    lane.synchronize()
+    assert call((2 * 16 * 64, 64, 32) + good[3:]) == lane.BAD_SHAPE          # row stride shorter than a row
+    assert call((-1, 64, 128) + good[3:]) == lane.BAD_SHAPE
+    assert lib.tessera_gfx950_flash_attn_strided_bf16_dev(z.ptr, z.ptr, z.ptr, z.ptr, None, 1, 2, 2, 16, 16, 64, None,
+                                                          ctypes.c_float(0.125), 1, 0, ctypes.c_float(0.0), 1,
+                                                          None) == lane.BAD_SHAPE
 
 
 def test_batched_and_shared_weight_gemm(lane):
