@@ -3,7 +3,7 @@
 
 A "step" is one pass of the hot path over one batch of synthetic input: one
 ``D = A . B`` with A, B bf16 8192 x 8192 (entries N(0,1)/sqrt(K), seeded), f32
-accumulate, bf16 output — BASELINE.json's configs[1].  Inputs are resident in
+accumulate, bf16 output — the configuration the headline metric is quoted on.  Inputs are resident in
 HBM before the timed region; the timed region is K launches through the C ABI's
 device-pointer entry point, bracketed by a device synchronise on both sides.
 
