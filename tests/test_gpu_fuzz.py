@@ -6,7 +6,12 @@ kernel family behind each entry point (square-tile, skinny, split-K, generic fal
 with the same bounds: bit-exact for integer and index results, <= 2e-3 (normwise) for 16-bit
 floating point with f32 accumulation, exact RNE of the f32 accumulators for stored results.
 Every draw prints nothing and is reproducible from its seed.
+
+``TESSERA_FUZZ_SCALE=n`` in the environment multiplies the number of seeds of every sweep
+(default 1: the suite's normal run; a soak run uses 8 or more).
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -16,6 +21,7 @@ from tessera_amd import ops
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-3
+SCALE = max(1, int(os.environ.get("TESSERA_FUZZ_SCALE", "1")))
 
 
 def _store(x, st):
@@ -32,7 +38,7 @@ def _dim(rng, hi, aligned):
     return max(8, n // 8 * 8) if aligned else n
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(6 * SCALE))
 def test_gemm_random_shapes(lane, seed):
     rng = np.random.default_rng(1000 + seed)
     for _ in range(60):
@@ -53,7 +59,7 @@ def test_gemm_random_shapes(lane, seed):
         assert np.array_equal(np.asarray(stored).view(np.uint16), np.asarray(want).view(np.uint16)), (seed, M, N, K, st)
 
 
-@pytest.mark.parametrize("seed", range(2))
+@pytest.mark.parametrize("seed", range(2 * SCALE))
 def test_big_tile_gemm_random_shapes(lane, seed):
     """Shapes large enough for the 256 x 256 tile (its 16-wide MFMA step, peeled first and last
     K steps, ragged rows and columns), both storage types, short and odd K."""
@@ -73,7 +79,7 @@ def test_big_tile_gemm_random_shapes(lane, seed):
         assert np.array_equal(np.asarray(stored).view(np.uint16), np.asarray(_store(got, st)).view(np.uint16)), (seed, M, N, K, st)
 
 
-@pytest.mark.parametrize("seed", range(3))
+@pytest.mark.parametrize("seed", range(3 * SCALE))
 def test_batched_gemm_random_shapes(lane, seed):
     rng = np.random.default_rng(2000 + seed)
     for _ in range(30):
@@ -89,7 +95,7 @@ def test_batched_gemm_random_shapes(lane, seed):
         assert orc.max_rel_err(got, ref) <= 1e-5, (seed, Bt, M, N, K, st)
 
 
-@pytest.mark.parametrize("seed", range(3))
+@pytest.mark.parametrize("seed", range(3 * SCALE))
 def test_int8_gemm_random_shapes_bit_exact(lane, seed):
     rng = np.random.default_rng(3000 + seed)
     for _ in range(40):
@@ -102,7 +108,7 @@ def test_int8_gemm_random_shapes_bit_exact(lane, seed):
         assert np.array_equal(got, orc.gemm_i8_i32(a, b)), (seed, M, N, K)
 
 
-@pytest.mark.parametrize("seed", range(3))
+@pytest.mark.parametrize("seed", range(3 * SCALE))
 def test_quantised_chains_random_shapes(lane, seed):
     """quantise -> GEMM -> dequantise on random shapes: int8 accumulators, codes and scales
     bit-exact; e4m3 codes equal as values, product within 2e-3 of the dequantised product."""
@@ -132,7 +138,7 @@ def test_quantised_chains_random_shapes(lane, seed):
         assert orc.max_rel_err(got, ref) <= TOL, (seed, M, N, K)
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(6 * SCALE))
 def test_attention_random_shapes(lane, seed):
     rng = np.random.default_rng(5000 + seed)
     for _ in range(30):
@@ -141,7 +147,7 @@ def test_attention_random_shapes(lane, seed):
         ratio = int(rng.choice([1, 1, 2, 4]))
         if rng.integers(0, 4) == 0:                       # the XCD-grouped workgroup order: B * Hkv % 8 == 0
             B, Hkv = 1, 8
-        D = int(rng.choice([16, 32, 48, 64, 64, 80, 128, 128, 128, 256]))
+        D = int(rng.choice([16, 32, 48, 64, 64, 80, 96, 128, 128, 128, 160, 192, 256]))
         Sq, Sk = int(rng.integers(1, 420)), int(rng.integers(1, 420))
         causal = bool(rng.integers(0, 2))
         window = int(rng.choice([0, 0, 0, 1, 7, 64, 130]))
@@ -168,6 +174,57 @@ def test_attention_random_shapes(lane, seed):
         assert np.max(np.abs(lse[live] - ref_lse[live]), initial=0.0) <= TOL, case
 
 
+@pytest.mark.parametrize("seed", range(3 * SCALE))
+def test_strided_attention_random_layouts(lane, seed):
+    """The strided entry point on operands that live inside wider rows (a fused projection's
+    column blocks, with random gaps between the heads' blocks) gives the bits the contiguous
+    entry point gives on compacted copies: only the addressing differs."""
+    import ctypes
+    lib = lane.load()
+    rng = np.random.default_rng(5500 + seed)
+    for _ in range(12):
+        B, Hkv = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+        Hq = Hkv * int(rng.choice([1, 2, 4]))
+        D = int(rng.choice([16, 48, 64, 96, 128, 256]))
+        Sq, Sk = int(rng.integers(1, 300)), int(rng.integers(1, 300))
+        causal = int(rng.integers(0, 2))
+        f32_out = int(rng.integers(0, 2))
+        st = "bf16" if rng.integers(0, 2) else "f16"
+        # rows of width W hold [gap | q heads | gap | k heads | v heads | gap], gaps multiples of 8 elements
+        g0, g1, g2 = (8 * int(rng.integers(0, 3)) for _ in range(3))
+        Wq, Wk = g0 + Hq * D + g1, Hkv * D * 2 + g2
+        q_rows = _store(rng.standard_normal((B, Sq, Wq)).astype(np.float32), st)
+        kv_rows = _store(rng.standard_normal((B, Sk, Wk)).astype(np.float32), st)
+        bits = lambda a: np.ascontiguousarray(np.asarray(a).view(np.uint16) if st == "f16" else np.asarray(a, np.uint16))
+        qb, kvb = bits(q_rows), bits(kv_rows)
+        dq, dkv = lane.DeviceBuffer.from_host(qb), lane.DeviceBuffer.from_host(kvb)
+        esz = 4 if f32_out else 2
+        Wo = Hq * D + g1
+        do, dl = lane.DeviceBuffer(B * Sq * Wo * esz), lane.DeviceBuffer(B * Hq * Sq * 4)
+        do.zero()
+        strides = (ctypes.c_int64 * 12)(Sq * Wq, D, Wq, Sk * Wk, D, Wk, Sk * Wk, D, Wk, Sq * Wo, D, Wo)
+        fn = getattr(lib, f"tessera_gfx950_flash_attn_strided_{st}_dev")
+        rc = fn(dq.ptr + g0 * 2, dkv.ptr, dkv.ptr + Hkv * D * 2, do.ptr, dl.ptr, B, Hq, Hkv, Sq, Sk, D, strides,
+                ctypes.c_float(D ** -0.5), causal, 0, ctypes.c_float(0.0), 0 if f32_out else 1, None)
+        case = (seed, B, Hq, Hkv, Sq, Sk, D, causal, f32_out, st, g0, g1, g2)
+        assert rc == 0, case
+        lane.synchronize()
+        got = do.download((B, Sq, Wo), np.float32 if f32_out else np.uint16)[:, :, :Hq * D].reshape(B, Sq, Hq, D)
+        got_lse = dl.download((B, Hq, Sq), np.float32)
+        # compacted [B, H, S, D] copies through the contiguous entry point
+        q4 = np.ascontiguousarray(qb[:, :, g0:g0 + Hq * D].reshape(B, Sq, Hq, D).transpose(0, 2, 1, 3))
+        k4 = np.ascontiguousarray(kvb[:, :, :Hkv * D].reshape(B, Sk, Hkv, D).transpose(0, 2, 1, 3))
+        v4 = np.ascontiguousarray(kvb[:, :, Hkv * D:2 * Hkv * D].reshape(B, Sk, Hkv, D).transpose(0, 2, 1, 3))
+        wrap = (lambda a: b16.from_bits(a)) if st == "bf16" else (lambda a: a.view(np.float16))
+        ref, ref_lse = ops.gqa_attention(wrap(q4), wrap(k4), wrap(v4), causal=bool(causal), return_lse=True,
+                                         out="f32" if f32_out else "storage")
+        ref_bits = np.asarray(ref, np.float32) if f32_out else bits(ref)
+        assert np.array_equal(got.transpose(0, 2, 1, 3), ref_bits), case
+        assert np.array_equal(got_lse, ref_lse), case
+        for buf in (dq, dkv, do, dl):
+            buf.close()
+
+
 def _tie_free_logits(rng, T, E, k):
     for _ in range(50):
         lg = rng.standard_normal((T, E)).astype(np.float32)
@@ -176,7 +233,7 @@ def _tie_free_logits(rng, T, E, k):
     raise AssertionError("could not draw tie-free logits")
 
 
-@pytest.mark.parametrize("seed", range(4))
+@pytest.mark.parametrize("seed", range(4 * SCALE))
 def test_routing_random_shapes_bit_exact(lane, seed):
     rng = np.random.default_rng(6000 + seed)
     for _ in range(40):
@@ -203,7 +260,7 @@ def test_routing_random_shapes_bit_exact(lane, seed):
         np.testing.assert_allclose(w, rw, rtol=2e-6, atol=1e-9)
 
 
-@pytest.mark.parametrize("seed", range(3))
+@pytest.mark.parametrize("seed", range(3 * SCALE))
 def test_grouped_gemm_random_groups(lane, seed):
     rng = np.random.default_rng(7000 + seed)
     for _ in range(15):
@@ -224,7 +281,7 @@ def test_grouped_gemm_random_groups(lane, seed):
         assert np.array_equal(np.asarray(stored).view(np.uint16), np.asarray(b16.from_float32(got)).view(np.uint16))
 
 
-@pytest.mark.parametrize("seed", range(4))
+@pytest.mark.parametrize("seed", range(4 * SCALE))
 def test_attention_backward_random_shapes(lane, seed):
     """dQ, dK, dV against the f64 gradients of the same 16-bit inputs; bounds as in the
     hand-picked backward tests (2e-3 f16, 5e-3 bf16: P and dS are rounded to the storage dtype
@@ -253,7 +310,7 @@ def test_attention_backward_random_shapes(lane, seed):
             assert orc.max_rel_err(g, r) <= bound[st], (name, case)
 
 
-@pytest.mark.parametrize("seed", range(3))
+@pytest.mark.parametrize("seed", range(3 * SCALE))
 def test_moe_layer_random_shapes(lane, seed):
     """The whole layer (router product, routing, expert block, combine) on random sizes: the
     plan's indices bit-exact, the output within the bf16 stage-rounding bound of the layer tests."""
