@@ -103,7 +103,12 @@ struct Gemm16Params {
 constexpr int G16_BK = 64;          // K step, elements
 constexpr int G16_APITCH = 128;     // bytes per A row in LDS
 constexpr int G16_BPAD = 32;        // B row pad, elements
-constexpr int kTailPace = 24;       // s_sleep units a paced short tile waits per K step
+// s_sleep units (64 shader clocks each) a paced short last tile waits per K step.  Per K step a
+// wave of a full 256-row tile issues 128 MFMAs of 16 cycles (2048 cycles), a wave of the 64-row
+// tile 32 (512 cycles): the difference, (2048 - 512) / 64 = 24 units, keeps the short tile in step
+// with the full tiles of its column.  Both terms are fixed by the tile shapes; the unit is shader
+// clocks, so the figure does not depend on K or on the clock the board grants.
+constexpr int kTailPace = (2048 - 512) / 64;
 // A-tile chunk swizzle: 16 consecutive rows of one chunk column hit 16 different
 // 16-byte slots of the 256-byte bank line.
 __device__ __forceinline__ int g16_aswz(int row) { return (row >> 1) & 7; }

@@ -177,6 +177,33 @@ def test_mfma_kernel_is_the_one_that_runs_for_padded_head_dims(lane):
     assert flop / ms / 1e9 > 20.0, f"{ms:.3f} ms per launch: not the matrix path"
 
 
+def test_strided_operands_that_are_not_16_byte_aligned_take_the_per_row_kernel(lane):
+    """Row strides that are not multiples of 8 elements cannot be read 16 bytes at a time: the
+    per-row kernel serves them through the same strides, to the same bounds."""
+    import ctypes
+    B, Hq, Hkv, Sq, Sk, D = 1, 2, 1, 40, 55, 32
+    q, k, v = _qkv(B, Hq, Hkv, Sq, Sk, D, 41, "f16")
+    ref_o, ref_lse = orc.flash_attn_dense(_f32(q), _f32(k), _f32(v), causal=True)
+    pad = 4                                                           # rows of D + 4 elements
+    def rows(x):
+        out = np.zeros(x.shape[:-1] + (D + pad,), np.float16)
+        out[..., :D] = x
+        return lane.DeviceBuffer.from_host(np.ascontiguousarray(out.view(np.uint16)))
+    dq, dk, dv = rows(q), rows(k), rows(v)
+    do, dl = lane.DeviceBuffer(B * Hq * Sq * (D + pad) * 4), lane.DeviceBuffer(B * Hq * Sq * 4)
+    W = D + pad
+    strides = (ctypes.c_int64 * 12)(Hq * Sq * W, Sq * W, W, Hkv * Sk * W, Sk * W, W, Hkv * Sk * W, Sk * W, W,
+                                    Hq * Sq * W, Sq * W, W)
+    rc = lane.load().tessera_gfx950_flash_attn_strided_f16_dev(dq.ptr, dk.ptr, dv.ptr, do.ptr, dl.ptr, B, Hq, Hkv, Sq, Sk, D,
+                                                               strides, ctypes.c_float(D ** -0.5), 1, 0, ctypes.c_float(0.0),
+                                                               0, None)
+    assert rc == 0
+    lane.synchronize()
+    o = do.download((B, Hq, Sq, W), np.float32)[..., :D]
+    assert orc.max_rel_err(o, ref_o) <= TOL
+    assert np.max(np.abs(dl.download((B, Hq, Sq), np.float32) - ref_lse)) <= TOL
+
+
 def test_attention_rejects_bad_shapes(lane):
     lib = lane.load()
     z = np.zeros(1024, np.uint16)
