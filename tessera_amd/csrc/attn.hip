@@ -163,6 +163,81 @@ int launch_bwd(const FlashBwdParams& p, hipStream_t s) {
   return launch_status();
 }
 
+// Rows of `src_chunks` 16-byte chunks copied into rows of `dst_chunks`: a wider destination is
+// zero-filled behind the source's columns, a narrower one takes the leading columns.
+__global__ void __launch_bounds__(256) repitch_rows_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src,
+                                                           long rows, int src_chunks, int dst_chunks) {
+  const long total = rows * dst_chunks;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+    const long r = i / dst_chunks;
+    const int c = (int)(i - r * dst_chunks);
+    dst[i] = c < src_chunks ? src[r * src_chunks + c] : make_uint4(0u, 0u, 0u, 0u);
+  }
+}
+inline void repitch_rows(void* dst, const void* src, long rows, int src_bytes, int dst_bytes, hipStream_t s) {
+  const long total = rows * (dst_bytes / 16);
+  const long blocks = (total + 255) / 256;
+  hipLaunchKernelGGL(repitch_rows_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, s,
+                     static_cast<uint4*>(dst), static_cast<const uint4*>(src), rows, src_bytes / 16, dst_bytes / 16);
+}
+
+template <class T>
+int flash_bwd_dev(const void* dO, const void* Q, const void* K, const void* V, const float* O, const float* LSE,
+                  float* dQ, float* dK, float* dV, int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                  int causal, hipStream_t s);
+
+// Head dimensions below 128 other than 64: the MFMA kernels are compiled for 64 and 128, so the
+// operands are copied into zero-padded rows of the next compiled width (zero columns of Q, K, V
+// and dO change no score, no dP and no Delta, and yield zero gradient columns), the kernels run
+// at that width, and the leading D columns of the gradients are copied out.  The forward's O
+// and log-sum-exp are taken from the caller or recomputed at the real width.
+template <class T>
+int flash_bwd_padded_dev(const void* dO, const void* Q, const void* K, const void* V, const float* O,
+                         const float* LSE, float* dQ, float* dK, float* dV, int B, int Hq, int Hkv, int Sq, int Sk,
+                         int D, float scale, int causal, hipStream_t s) {
+  const int DP = D < 64 ? 64 : 128;
+  const size_t rows = (size_t)B * Hq * Sq, kvrows = (size_t)B * Hkv * Sk;
+  const bool recompute = !O || !LSE;
+  // 16-bit: Qp dOp (rows) Kp Vp (kvrows); f32: Op dQp (rows) dKp dVp (kvrows) [+ O, LSE at the real width]
+  const size_t b16q = rows * DP * 2, b16k = kvrows * DP * 2, f32q = rows * DP * 4, f32k = kvrows * DP * 4;
+  const size_t extra = recompute ? rows * D * 4 + rows * 4 : 0;
+  char* ws = nullptr;
+  if (hipMallocAsync(reinterpret_cast<void**>(&ws), 2 * b16q + 2 * b16k + 2 * f32q + 2 * f32k + extra, s) != hipSuccess) {
+    (void)hipGetLastError();
+    return kDeviceFailed;
+  }
+  char* Qp = ws; char* dOp = Qp + b16q; char* Kp = dOp + b16q; char* Vp = Kp + b16k;
+  char* Op = Vp + b16k; char* dQp = Op + f32q; char* dKp = dQp + f32q; char* dVp = dKp + f32k;
+  int rc = kOk;
+  if (recompute) {
+    float* o_ws = reinterpret_cast<float*>(dVp + f32k);
+    float* lse_ws = o_ws + rows * D;
+    rc = flash_dev<T>(Q, K, V, o_ws, lse_ws, B, Hq, Hkv, Sq, Sk, D, scale, causal, 0, s);
+    O = o_ws;
+    LSE = lse_ws;
+  }
+  if (rc == kOk) {
+    repitch_rows(Qp, Q, (long)rows, D * 2, DP * 2, s);
+    repitch_rows(dOp, dO, (long)rows, D * 2, DP * 2, s);
+    repitch_rows(Kp, K, (long)kvrows, D * 2, DP * 2, s);
+    repitch_rows(Vp, V, (long)kvrows, D * 2, DP * 2, s);
+    repitch_rows(Op, O, (long)rows, D * 4, DP * 4, s);
+    rc = launch_status();
+  }
+  if (rc == kOk)
+    rc = flash_bwd_dev<T>(dOp, Qp, Kp, Vp, reinterpret_cast<const float*>(Op), LSE, reinterpret_cast<float*>(dQp),
+                          reinterpret_cast<float*>(dKp), reinterpret_cast<float*>(dVp), B, Hq, Hkv, Sq, Sk, DP, scale,
+                          causal, s);
+  if (rc == kOk) {
+    repitch_rows(dQ, dQp, (long)rows, DP * 4, D * 4, s);
+    repitch_rows(dK, dKp, (long)kvrows, DP * 4, D * 4, s);
+    repitch_rows(dV, dVp, (long)kvrows, DP * 4, D * 4, s);
+    rc = launch_status();
+  }
+  if (hipFreeAsync(ws, s) != hipSuccess) { (void)hipGetLastError(); rc = rc == kOk ? kDeviceFailed : rc; }
+  return rc;
+}
+
 // (dQ, dK, dV) from (dO, Q, K, V).  O and LSE may be passed in (saved by the forward
 // call); when either is null the forward kernel is run first to recompute both.
 template <class T>
@@ -177,6 +252,13 @@ int flash_bwd_dev(const void* dO, const void* Q, const void* K, const void* V, c
   // The MFMA kernels fold -LSE / scale into their accumulators: they need a scale it
   // can be divided by; anything else takes the generic kernels.
   const bool scale_ok = std::isfinite(scale) && std::fabs(scale) >= 1e-20f;
+  {
+    const bool al_in = ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) | reinterpret_cast<uintptr_t>(V) |
+                         reinterpret_cast<uintptr_t>(dO) | reinterpret_cast<uintptr_t>(dQ) | reinterpret_cast<uintptr_t>(dK) |
+                         reinterpret_cast<uintptr_t>(dV) | reinterpret_cast<uintptr_t>(O)) & 15) == 0;
+    if (al_in && scale_ok && D < 128 && D != 64)
+      return flash_bwd_padded_dev<T>(dO, Q, K, V, O, LSE, dQ, dK, dV, B, Hq, Hkv, Sq, Sk, D, scale, causal, s);
+  }
   const size_t ws_floats = 2 * rows + (recompute ? rows * D + rows : 0);
   if (hipMallocAsync(reinterpret_cast<void**>(&ws), ws_floats * sizeof(float), s) != hipSuccess) {
     (void)hipGetLastError();

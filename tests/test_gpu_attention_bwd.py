@@ -40,7 +40,9 @@ CASES = [
     (2, 4, 2, 300, 300, 128, True), (1, 8, 2, 257, 511, 128, True),
     (1, 2, 2, 100, 77, 64, False), (1, 2, 1, 200, 333, 64, True), (1, 2, 2, 333, 200, 64, True),
     (1, 4, 4, 513, 129, 128, False), (1, 2, 2, 1, 129, 128, True),
-    (1, 3, 3, 40, 40, 48, False), (1, 2, 1, 50, 60, 32, True),      # generic head dims
+    (1, 3, 3, 40, 40, 48, False), (1, 2, 1, 50, 60, 32, True),      # head dims served zero-padded to 64 / 128
+    (1, 2, 1, 150, 203, 80, True), (1, 4, 2, 130, 130, 96, True), (2, 2, 2, 70, 90, 16, False),
+    (1, 2, 2, 64, 64, 112, True), (1, 2, 1, 40, 70, 160, True),      # 160: above the compiled widths, per-row kernels
     # B * Hkv a multiple of 8: the XCD-aware workgroup order
     (2, 8, 4, 200, 264, 128, True), (1, 16, 8, 130, 130, 64, True), (2, 24, 8, 70, 330, 128, False),
 ]
@@ -115,6 +117,31 @@ def test_backward_headline_shape_properties(lane):
     do2 = b16.from_float32(2.0 * do.to_float32())
     dq2, dk2, dv2 = ops.flash_attn_backward(do2, q, k, v, causal=True)
     assert np.array_equal(dq2, 2 * dq) and np.array_equal(dk2, 2 * dk) and np.array_equal(dv2, 2 * dv)
+
+
+@pytest.mark.parametrize("D", [48, 80, 128])
+def test_backward_with_saved_forward_results_equals_recompute(lane, D):
+    """The device entry point fed the forward's own O and log-sum-exp gives the bits the
+    recomputing host entry gives (the padded widths take the same path either way)."""
+    import ctypes
+    B, Hq, Hkv, Sq, Sk = 1, 4, 2, 150, 170
+    do, q, k, v = _inputs(B, Hq, Hkv, Sq, Sk, D, 77, "bf16")
+    want = ops.flash_attn_backward(do, q, k, v, causal=True)
+    lib = lane.load()
+    up = lambda a: lane.DeviceBuffer.from_host(np.ascontiguousarray(np.asarray(a, np.uint16)))
+    ddo, dq_, dk_, dv_ = up(do), up(q), up(k), up(v)
+    o, lse = lane.DeviceBuffer(B * Hq * Sq * D * 4), lane.DeviceBuffer(B * Hq * Sq * 4)
+    gq, gk, gv = lane.DeviceBuffer(B * Hq * Sq * D * 4), lane.DeviceBuffer(B * Hkv * Sk * D * 4), lane.DeviceBuffer(B * Hkv * Sk * D * 4)
+    sc = ctypes.c_float(D ** -0.5)
+    lane.check(lib.tessera_gfx950_flash_attn_gqa_bf16_dev(dq_.ptr, dk_.ptr, dv_.ptr, o.ptr, lse.ptr, B, Hq, Hkv, Sq, Sk, D,
+                                                          sc, 1, 0, None), "fwd")
+    lane.check(lib.tessera_gfx950_flash_attn_bwd_bf16_dev(ddo.ptr, dq_.ptr, dk_.ptr, dv_.ptr, o.ptr, lse.ptr, gq.ptr, gk.ptr,
+                                                          gv.ptr, B, Hq, Hkv, Sq, Sk, D, sc, 1, None), "bwd")
+    lane.synchronize()
+    got = (gq.download((B, Hq, Sq, D), np.float32), gk.download((B, Hkv, Sk, D), np.float32),
+           gv.download((B, Hkv, Sk, D), np.float32))
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
 
 
 def test_backward_executor_and_bad_shapes(lane):
