@@ -35,7 +35,7 @@ int launch_flash(const FlashParams& p, hipStream_t s) {
 }
 
 // The kernel for head dimension p.D: compiled for DP = 64 / 128 / 256, exact when D == DP
-// (plain and extended forms), zero-padded otherwise (one form, the extended one, serves both).
+// or zero-padded to it, each in the plain and the extended form.
 template <class T>
 int launch_flash_for(const FlashParams& p, bool ext, hipStream_t s) {
   switch (p.D) {
@@ -44,9 +44,9 @@ int launch_flash_for(const FlashParams& p, bool ext, hipStream_t s) {
     case 256: return ext ? launch_flash<T, 256, true, false>(p, s) : launch_flash<T, 256, false, false>(p, s);
     default: break;
   }
-  if (p.D < 64) return launch_flash<T, 64, true, true>(p, s);
-  if (p.D < 128) return launch_flash<T, 128, true, true>(p, s);
-  return launch_flash<T, 256, true, true>(p, s);
+  if (p.D < 64) return ext ? launch_flash<T, 64, true, true>(p, s) : launch_flash<T, 64, false, true>(p, s);
+  if (p.D < 128) return ext ? launch_flash<T, 128, true, true>(p, s) : launch_flash<T, 128, false, true>(p, s);
+  return ext ? launch_flash<T, 256, true, true>(p, s) : launch_flash<T, 256, false, true>(p, s);
 }
 
 // Contiguous [B, H, S, D].
