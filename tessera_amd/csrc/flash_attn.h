@@ -10,8 +10,9 @@
 // slices of a fused projection output are all served without a copy.
 //
 // One workgroup of 8 waves (two per SIMD) owns 256 query rows of one (batch, q
-// head) (DP = 256: 4 waves, one per SIMD with the whole register file each, 128 rows);
-// each wave owns 32 of them as one MFMA tile.  K/V are walked in 64-key
+// head); each wave owns 32 of them as one MFMA tile.  (DP = 256: 128 query rows; two waves
+// share each 32-row block, both computing its scores, each accumulating one half of the
+// output columns — see FlashGeom.)  K/V are walked in 64-key
 // tiles that stream from global memory straight into LDS (two stages each, one
 // barrier per tile).  The loop is software-pipelined: the score MFMAs of tile
 // t+1 are issued under the softmax arithmetic of tile t, and the exponentials of
@@ -84,16 +85,21 @@ __host__ __device__ inline void key_bounds(int i, int Sq, int Sk, int causal, in
 
 constexpr int FA_QT = 1;               // 32-row query tiles per wave
 constexpr int FA_BKV = 64;             // keys per LDS tile
-// Per padded head dimension: waves per workgroup (two per SIMD while a wave's accumulators,
-// Q fragments and score tiles fit 256 registers, else one per SIMD), query rows per
-// workgroup, 16-byte chunks per LDS row, bytes of one K (or V) stage, LDS bytes.
+// Per padded head dimension: waves per workgroup (always two per SIMD), how many waves share
+// one 32-row block by output columns, query rows per workgroup, 16-byte chunks per LDS row,
+// bytes of one K (or V) stage, LDS bytes.
 template <int DP> struct FlashGeom {
-  static constexpr int WAVES = DP > 128 ? 4 : 8;
+  static constexpr int WAVES = 8;
   static constexpr int THREADS = WAVES * 64;
-  static constexpr int BQ = WAVES * 32 * FA_QT;
+  // DP = 256: a wave's 32 rows x 256 output columns would be 128 accumulator registers, which
+  // does not fit next to 64 Q and 64 score registers in the 256 a wave has at two per SIMD.
+  // Two waves therefore share each 32-row block: both compute its scores and softmax (the same
+  // bits), each accumulates one half of the output columns.
+  static constexpr int DSPLIT = DP > 128 ? 2 : 1;
+  static constexpr int BQ = WAVES / DSPLIT * 32 * FA_QT;
   static constexpr int CHUNKS = DP / 8;
   static constexpr int TILE = FA_BKV * DP * 2;
-  static constexpr int STAGE_PITCH = DP * 4 + 16;              // epilogue staging row, f32
+  static constexpr int STAGE_PITCH = DP / DSPLIT * 4 + 16;     // epilogue staging row, f32
   static constexpr int SMEM = 4 * TILE > WAVES * 32 * FA_QT * STAGE_PITCH ? 4 * TILE : WAVES * 32 * FA_QT * STAGE_PITCH;
 };
 constexpr float FA_NEG = -1.0e30f;
@@ -157,7 +163,8 @@ __global__ __launch_bounds__(FlashGeom<DP>::THREADS, 1) void flash_fwd_kernel(co
   constexpr int KSTEPS = D / 16;         // MFMA k steps of the score product
   constexpr int KA = (KSTEPS + 3) / 4;   // score k steps issued under the row-max phase
   constexpr int KB = (KSTEPS + KA) / 2;  // ... and up to here under the first exponentials
-  constexpr int DT = D / 32;             // 32-wide d tiles of the output
+  constexpr int DS = G::DSPLIT;          // waves that share a row block, splitting the output columns
+  constexpr int DT = D / 32 / DS;        // 32-wide d tiles of the output this wave accumulates
   constexpr int ROWB = D * 2;            // bytes per K/V row
   constexpr int CHUNKS = D / 8;          // 16-byte chunks per row
   constexpr int TILE = FA_BKV * ROWB;    // bytes per K (or V) tile
@@ -206,7 +213,10 @@ __global__ __launch_bounds__(FlashGeom<DP>::THREADS, 1) void flash_fwd_kernel(co
   // Waves w and w + 4 share a SIMD.  Under a causal mask a wave's key range grows with
   // its row block, so the upper four waves take the row blocks in reverse: every SIMD
   // gets one of the blocks 0-3 and its mirror image 7-4, the same work on all four.
-  const int rblk = wave < FA_WAVES / 2 ? wave : FA_WAVES + FA_WAVES / 2 - 1 - wave;
+  constexpr int RB = FA_WAVES / DS;            // row blocks of the workgroup
+  const int dsel = wave / RB;                  // which part of the output columns this wave accumulates
+  const int wrow = wave - dsel * RB;
+  const int rblk = wrow < RB / 2 ? wrow : RB + RB / 2 - 1 - wrow;
   const int qw = q0 + rblk * (32 * QT);       // first query row of the wave
   const uint16_t* Qb = p.Q + batch * p.qs.batch + hq * p.qs.head;
   const uint16_t* Kb = p.K + batch * p.ks.batch + hkv * p.ks.head;
@@ -334,7 +344,7 @@ __global__ __launch_bounds__(FlashGeom<DP>::THREADS, 1) void flash_fwd_kernel(co
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
     const int key = 4 * lh + (r16 >> 2);
-    const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (r16 & 3);
+    const int col = (dsel * DT + dt) * 32 + 16 * ((lane >> 4) & 1) + 4 * (r16 & 3);
     v_rd[dt] = 2 * TILE + key * ROWB + (((col >> 3) ^ vswz(key)) << 4) + (col & 7) * 2;
   }
 
@@ -567,7 +577,7 @@ __global__ __launch_bounds__(FlashGeom<DP>::THREADS, 1) void flash_fwd_kernel(co
     if (khi[qt] < klo[qt]) l = 0.f;                      // no visible key: O = 0, LSE = -inf
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     const long row = (long)qlin * p.Sq + qi;
-    if (p.LSE && lh == 0 && qi < p.Sq)
+    if (p.LSE && lh == 0 && dsel == 0 && qi < p.Sq)
       p.LSE[row] = l > 0.f ? (m_run[qt] * cs + __log2f(l)) * 0.69314718055994530942f : -INFINITY;
     char* stage = smem + (wave * QT + qt) * 32 * G::STAGE_PITCH;
 #pragma unroll
@@ -586,15 +596,17 @@ __global__ __launch_bounds__(FlashGeom<DP>::THREADS, 1) void flash_fwd_kernel(co
           *reinterpret_cast<float4*>(stage + l32 * G::STAGE_PITCH + d * 4) = make_float4(v0, v1, v2, v3);
         }
       }
-    // rows of dreal elements, 16 bytes per lane
+    // rows of this wave's share of the dreal columns, 16 bytes per lane
     const int esz = p.out_storage ? 2 : 4;
-    const int per_row = dreal * esz / 16;                  // 16-byte pieces per output row
+    const int dcol0 = dsel * DT * 32;                      // first output column of this wave
+    const int dcols = min(dreal - dcol0, DT * 32);
+    const int per_row = dcols > 0 ? dcols * esz / 16 : 0;  // 16-byte pieces per output row
     const int rows_here = min(32, p.Sq - (qw + 32 * qt));
     char* Ob = reinterpret_cast<char*>(p.O) + (batch * p.os.batch + hq * p.os.head) * esz;
     for (int idx = lane; idx < rows_here * per_row; idx += 64) {
       const int r = idx / per_row, c = idx - r * per_row;
       const uint4 v = *reinterpret_cast<const uint4*>(stage + r * G::STAGE_PITCH + c * 16);
-      *reinterpret_cast<uint4*>(Ob + ((long)(qw + 32 * qt + r) * p.os.row) * esz + c * 16) = v;
+      *reinterpret_cast<uint4*>(Ob + ((long)(qw + 32 * qt + r) * p.os.row + dcol0) * esz + c * 16) = v;
     }
   }
 }
