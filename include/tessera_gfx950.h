@@ -204,6 +204,14 @@ int tessera_gfx950_gated_gemm_bf16_dev(const void* A, const void* Wg, const void
 int tessera_gfx950_gemm_schedule(int M, int N, int K, int batch, int elem_bytes,
                                  int* tile_m, int* tile_n, int* tile_k, int* split_k);
 
+/* A product on 256 x 256 tiles whose tile count is a little over a multiple of the 256 compute
+ * units: the tiles beyond the last full round (*rest_tiles of them) are split along K into
+ * *rest_split parts each by a second launch and summed by a third, so that round fills the chip.
+ * *rest_split == 1: every tile is computed whole by one launch (*rest_tiles is then 0).
+ * Host-only query beside tessera_gfx950_gemm_schedule; 16-bit operands.  No counterpart in the
+ * reference, whose schedule has no such step. */
+int tessera_gfx950_gemm_rest_split(int M, int N, int K, int batch, int* rest_tiles, int* rest_split);
+
 /* Kernel-only benchmark with resident, library-owned buffers: warm-up, `iters`
  * launches between HIP events, cross-checked against wall clock
  * (tessera_rocm_gemm.cpp:551-667).  *avg_ms = mean per-launch ms. */

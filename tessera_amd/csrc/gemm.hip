@@ -334,6 +334,15 @@ int tessera_gfx950_gemm_schedule(int M, int N, int K, int batch, int elem_bytes,
   return kBadShape;
 }
 
+int tessera_gfx950_gemm_rest_split(int M, int N, int K, int batch, int* rest_tiles, int* rest_split) {
+  if (bad_dims(batch, M, N, K) || !rest_tiles || !rest_split) return kBadShape;
+  const Gemm16Schedule sch = select_gemm16_schedule(M, N, K, batch);
+  const bool on = sch.tile == 256 && sch.split_k == 1 && !sch.skinny && sch.rest_split > 1;
+  *rest_split = on ? sch.rest_split : 1;
+  *rest_tiles = on ? (int)(((long)ceil_div(M, 256) * ceil_div(N, 256)) % 256) : 0;
+  return kOk;
+}
+
 int tessera_gfx950_gemm_bf16_bench(int M, int N, int K, int iters, double* avg_ms) {
   return bench_gemm16<BF16>(M, N, K, iters, 1, avg_ms);
 }

@@ -737,4 +737,67 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
   gemm16_tile<T, BM, BN, WM, WN, EPI, GROUPED, MS>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db);
 }
 
+// The tiles that are left when the tile count is not a multiple of the 256 compute units would
+// run as a last, mostly empty round.  This kernel takes those tiles (ids first_tile .. in the
+// order of tile_of_block) and splits each along K over gridDim.y workgroups, so the round fills
+// the chip: workgroup (r, z) computes K range [z ksplit, (z + 1) ksplit) of tile first_tile + r
+// and writes the f32 partial tile, row-major 256 x 256, to ws[(z * gridDim.x + r)]; a second
+// kernel sums the partials in split order.  Dense, unbatched products only.
+template <class T, int MS>
+__global__ __launch_bounds__(256, 1) void gemm16_rest_splitk_kernel(const Gemm16Params p, int first_tile, int ksplit,
+                                                                    float* __restrict__ ws) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  int tm, tn;
+  tile_of_block(first_tile + (int)blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  const int z = blockIdx.y;
+  const int k0 = z * ksplit;
+  Gemm16Params q = p;
+  q.K = min(ksplit, p.K - k0);
+  q.ldd = 256;
+  q.bias = nullptr;
+  q.act = ACT_NONE;
+  const int m_begin = tm * 256;
+  float* tile_ws = ws + ((long)z * gridDim.x + blockIdx.x) * (256 * 256);
+  // the tile function stores element (m, n) at Db + (m ldd + n): shift the base so that the
+  // tile's first element lands on tile_ws
+  char* Db = reinterpret_cast<char*>(tile_ws - ((long)m_begin * 256 + (long)tn * 256));
+  gemm16_tile<T, 256, 256, 2, 2, EPI_F32, false, MS>(q, smem, m_begin, p.M, tn, p.A + k0, p.B + (long)k0 * p.ldb, nullptr,
+                                                      Db);
+}
+
+// D tile = sum over the splits (in split order) of the partial tiles written by the kernel above,
+// then bias / activation, stored as f32 or in the storage dtype; four columns per thread.
+template <class T, int EPI>
+__global__ __launch_bounds__(256) void gemm16_rest_sum_kernel(const float* __restrict__ ws, void* __restrict__ D, int M,
+                                                              int N, long ldd, int tiles_m, int tiles_n, int first_tile,
+                                                              int splits, const float* __restrict__ bias, int act) {
+  int tm, tn;
+  tile_of_block(first_tile + (int)blockIdx.y, tiles_m, tiles_n, tm, tn);
+  const int quad = blockIdx.x * 256 + threadIdx.x;     // 64 quads of four columns per row
+  const int row = quad >> 6, col = (quad & 63) * 4;
+  const int m = tm * 256 + row, n = tn * 256 + col;
+  if (m >= M || n >= N) return;
+  const long tile_elems = 256 * 256;
+  const float* src = ws + (long)blockIdx.y * tile_elems + row * 256 + col;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int z = 0; z < splits; ++z) {
+    const float4 v = *reinterpret_cast<const float4*>(src + (long)z * gridDim.y * tile_elems);
+    acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+  }
+  if (bias) {
+    const float4 bv = *reinterpret_cast<const float4*>(bias + n);
+    acc.x += bv.x; acc.y += bv.y; acc.z += bv.z; acc.w += bv.w;
+  }
+  acc.x = activate(acc.x, act); acc.y = activate(acc.y, act);
+  acc.z = activate(acc.z, act); acc.w = activate(acc.w, act);
+  if constexpr (EPI == EPI_F32 || EPI == EPI_F32_FUSED) {
+    *reinterpret_cast<float4*>(reinterpret_cast<float*>(D) + (long)m * ldd + n) = acc;
+  } else {
+    uint2 pk;
+    pk.x = pack2<T>(acc.x, acc.y);
+    pk.y = pack2<T>(acc.z, acc.w);
+    *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(D) + (long)m * ldd + n) = pk;
+  }
+}
+
 }  // namespace tsr950

@@ -68,8 +68,10 @@ constexpr int kGroupedTileMfma = 16;
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// wg_limit > 0: only the first wg_limit workgroups of a dense product's tile order are launched
+// (the caller serves the remaining tiles itself).
 template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32>
-int launch_gemm16_tile(Gemm16Params p, hipStream_t s) {
+int launch_gemm16_tile(Gemm16Params p, hipStream_t s, int wg_limit = 0) {
   using S = Gemm16Smem<BM, BN>;
   auto kern = gemm16_kernel<T, BM, BN, WM, WN, EPI, GROUPED, MS>;
   static std::once_flag once;
@@ -89,7 +91,7 @@ int launch_gemm16_tile(Gemm16Params p, hipStream_t s) {
     grid = dim3(p.tiles_n * p.tiles_m + 8, 1, 1);
   } else {
     p.tiles_m = ceil_div(p.M, BM);
-    grid = dim3(p.tiles_m * p.tiles_n, 1, p.groups);
+    grid = dim3(wg_limit > 0 ? wg_limit : p.tiles_m * p.tiles_n, 1, p.groups);
   }
   hipLaunchKernelGGL(kern, grid, dim3(WM * WN * 64), S::kBytes, s, p);
   return launch_status();
@@ -135,16 +137,37 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, void* __restr
 
 // Tile and split-K choice of the dense 16-bit GEMM for an aligned problem — the one
 // place the decision lives (the launcher below and the schedule query of the C ABI
-// both call it).  256x256 when that alone fills the chip; else 128x128 or 64x64
-// tiles, and for a single product with few tiles and a long K (decode-shaped: the
-// weight matrix streams from HBM once) K is split over about 768 workgroups.
+// both call it).
 struct Gemm16Schedule {
   int tile;      // square workgroup tile edge: 256, 128 or 64
   int split_k;   // number of K splits (1 = none)
   bool skinny;   // M <= 8: the streaming kernel (32 x 64 workgroup tile, K slices of 32)
+  int rest_split = 1;   // 256 tiles, split_k 1: K splits of the tiles beyond the last full round of 256
 };
 constexpr int kSkinnyMaxM = 8;
 constexpr long kSplitTargetWgs = 768;
+constexpr int kWeightStreamMaxM = 128;   // up to here a product is bound by reading B once
+
+// Time estimates (microseconds) behind the choice for products with more than kWeightStreamMaxM
+// rows, fitted to timings of forced (tile, split) pairs on this part over products from 1024^3
+// to 7168^3: a 256 x 256 tile spends 9.6 us outside its K loop and 1.09 us per 64-deep K step
+// while at most 144 of the 256 compute units are busy, rising to 1.43 us with all of them busy
+// (the board's power limit sets the clock); a 128 x 128 tile 5 us and 0.52 us per step, two
+// of them sharing a compute unit at half that rate each (512 run at a time); the sum over K splits reads the f32
+// partials and writes the result at about 4.4 TB/s.
+inline double est_tiles256_us(long tiles, int ksteps) {
+  const long full = tiles / 256, rem = tiles % 256;
+  double t = (double)full * (9.6 + ksteps * 1.43);
+  if (rem) t += 9.6 + ksteps * (1.09 + 0.34 * std::min(1.0, std::max(0.0, (rem - 144) / 112.0)));
+  return t;
+}
+inline double est_tiles128_us(long tiles, int ksteps) {
+  return 5.0 * (double)((tiles + 511) / 512) + ksteps * 0.52 * (double)((tiles + 255) / 256);
+}
+inline double est_split_sum_us(long mn, int splits) {
+  return splits > 1 ? 2.0 + (double)mn * (4.0 * splits + 2.0) / 4.4e6 : 0.0;
+}
+
 inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
   if (batch == 1 && M <= kSkinnyMaxM && K % 32 == 0 && K >= 512) {
     // one workgroup per 64-column strip and K split; about one workgroup per CU, and
@@ -155,6 +178,42 @@ inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
   }
   const long tiles256 = (long)ceil_div(M, 256) * ceil_div(N, 256) * batch;
   const long tiles128 = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch;
+  if (M > kWeightStreamMaxM && N >= 128) {
+    // the cheapest of: either tile, K in 1, 2, 3, 4 or 8 parts (a single product only; every
+    // part a whole number of K steps and at least 512 deep)
+    const int ksteps = ceil_div(K, G16_BK);
+    Gemm16Schedule best{256, 1, false};
+    double best_us = est_tiles256_us(tiles256, ksteps);
+    auto consider = [&](int tile, int splits, double us) {
+      if (us < best_us) { best_us = us; best = Gemm16Schedule{tile, splits, false}; }
+    };
+    consider(128, 1, est_tiles128_us(tiles128, ksteps));
+    if (batch == 1) {
+      for (int splits : {2, 3, 4, 8}) {
+        if (K % (splits * G16_BK) != 0 || K / splits < 512) continue;
+        const double sum_us = est_split_sum_us((long)M * N, splits);
+        consider(256, splits, est_tiles256_us(tiles256 * splits, ksteps / splits) + sum_us);
+        consider(128, splits, est_tiles128_us(tiles128 * splits, ksteps / splits) + sum_us);
+      }
+    }
+    // A tile count a little over a multiple of 256 leaves a last round with most compute units
+    // idle: those tiles can be split along K among them (one more launch and a sum over the
+    // partial tiles).
+    const long full = tiles256 / 256, rest = tiles256 % 256;
+    if (batch == 1 && full >= 1 && rest > 0 && rest <= 128) {
+      const double main_us = (double)full * (9.6 + ksteps * 1.43);
+      for (int splits : {2, 3, 4, 6, 8, 12, 16}) {
+        const int per = ceil_div(ksteps, splits);
+        if (rest * splits > 256 || per < 2 || (long)per * (splits - 1) >= ksteps) continue;
+        const double us = main_us + 3.0 + est_tiles256_us(rest * splits, per) +
+                          est_split_sum_us(rest * 65536L, splits);
+        if (us < best_us) { best_us = us; best = Gemm16Schedule{256, 1, false, splits}; }
+      }
+    }
+    return best;
+  }
+  // Few rows: the weight matrix streams from HBM once and the tiles are small; for a single
+  // product with few tiles and a long K, K is split over about 768 workgroups.
   if (tiles256 >= 192) return {256, 1, false};
   const bool t128 = tiles128 >= 192 || (M > 64 && N >= 128);
   int splits = 1;
@@ -185,6 +244,165 @@ int launch_gemm16_skinny(const Gemm16Params& p, int kps, int splits, hipStream_t
   return launch_status();
 }
 
+// Copies between a matrix of any pitch and alignment and a 16-byte aligned one whose pitch is a
+// multiple of 16 bytes, for operands the vector loads of the tile kernels cannot take as they are.
+// A thread moves one 16-byte chunk: blockIdx.x / threadIdx.x run along a row, blockIdx.y /
+// threadIdx.y over rows, blockIdx.z over the batch.  The side of any alignment is accessed with one
+// 16-byte instruction where the whole chunk is inside the row (global memory takes accesses off
+// their natural alignment), element by element at the row's end.
+template <class E> struct __attribute__((packed, aligned(sizeof(E)))) LooseChunk { uint4 v; };
+constexpr int kCopyRowsPerBlock = 4;
+
+// dst[b][r][c] (rows_dst x ld_dst, 16-byte aligned) = src[b][r][c] inside rows_src x cols_src, else 0.
+template <class E>
+__global__ void __launch_bounds__(64 * kCopyRowsPerBlock)
+pad_rows_kernel(E* __restrict__ dst, long ld_dst, long stride_dst, const E* __restrict__ src, long ld_src,
+                long stride_src, int rows_src, int cols_src, int rows_dst) {
+  constexpr int V = 16 / sizeof(E);
+  const int c0 = (blockIdx.x * 64 + threadIdx.x) * V;
+  if (c0 >= ld_dst) return;
+  const long b = blockIdx.z;
+  for (int r = blockIdx.y * kCopyRowsPerBlock + threadIdx.y; r < rows_dst; r += gridDim.y * kCopyRowsPerBlock) {
+    uint4 out = make_uint4(0u, 0u, 0u, 0u);
+    if (r < rows_src && c0 < cols_src) {
+      const E* sp = src + b * stride_src + (long)r * ld_src + c0;
+      if (c0 + V <= cols_src) {
+        out = reinterpret_cast<const LooseChunk<E>*>(sp)->v;
+      } else {
+        alignas(16) E v[V];
+#pragma unroll
+        for (int u = 0; u < V; ++u) v[u] = c0 + u < cols_src ? sp[u] : E(0);
+        out = *reinterpret_cast<const uint4*>(v);
+      }
+    }
+    *reinterpret_cast<uint4*>(dst + b * stride_dst + (long)r * ld_dst + c0) = out;
+  }
+}
+// dst[b][r][c] = src[b][r][c] for r < rows, c < cols; src 16-byte aligned with pitch ld_src, dst any.
+template <class E>
+__global__ void __launch_bounds__(64 * kCopyRowsPerBlock)
+unpad_rows_kernel(E* __restrict__ dst, long ld_dst, long stride_dst, const E* __restrict__ src, long ld_src,
+                  long stride_src, int rows, int cols) {
+  constexpr int V = 16 / sizeof(E);
+  const int c0 = (blockIdx.x * 64 + threadIdx.x) * V;
+  if (c0 >= cols) return;
+  const long b = blockIdx.z;
+  for (int r = blockIdx.y * kCopyRowsPerBlock + threadIdx.y; r < rows; r += gridDim.y * kCopyRowsPerBlock) {
+    const uint4 in = *reinterpret_cast<const uint4*>(src + b * stride_src + (long)r * ld_src + c0);
+    E* dp = dst + b * stride_dst + (long)r * ld_dst + c0;
+    if (c0 + V <= cols) {
+      reinterpret_cast<LooseChunk<E>*>(dp)->v = in;
+    } else {
+      alignas(16) E v[V];
+      *reinterpret_cast<uint4*>(v) = in;
+#pragma unroll
+      for (int u = 0; u < V; ++u)
+        if (c0 + u < cols) dp[u] = v[u];
+    }
+  }
+}
+inline dim3 copy_grid(long rows, long ld, int vec, int batch) {
+  const long bx = (ld / vec + 63) / 64, by = (rows + kCopyRowsPerBlock - 1) / kCopyRowsPerBlock;
+  return dim3((unsigned)bx, (unsigned)std::max<long>(1, std::min<long>(by, 16384)), (unsigned)batch);
+}
+inline dim3 copy_block() { return dim3(64, kCopyRowsPerBlock, 1); }
+
+template <class T, int EPI>
+int launch_gemm16(Gemm16Params p, hipStream_t s);
+
+// A product whose operands the tile kernels cannot load as they are (K, N or a pitch not a
+// multiple of 8 elements, or a pointer off a 16-byte boundary): the offending operands are
+// copied into aligned, zero-padded buffers (K and N rounded up to multiples of 8: zero columns
+// of A, zero rows and columns of B), the tile kernels run on those, and the leading N columns
+// of the result are copied out.  The buffers live from here to the end of this call's work on
+// the stream (stream-ordered allocation).
+template <class T, int EPI>
+int launch_gemm16_repitched(const Gemm16Params& p, hipStream_t s) {
+  constexpr int dsz = (EPI == EPI_F32) ? 4 : 2;
+  const int K8 = (p.K + 7) & ~7, N8 = (p.N + 7) & ~7, G = p.groups;
+  const bool a_ok = p.K % 8 == 0 && p.lda % 8 == 0 && p.strideA % 8 == 0 && aligned16(p.A) && p.lda < (1L << 21);
+  const bool b_ok = p.K % 8 == 0 && p.N % 8 == 0 && p.ldb % 8 == 0 && p.strideB % 8 == 0 && aligned16(p.B) &&
+                    p.ldb < (1L << 21);
+  const bool d_ok = p.N % 8 == 0 && (p.ldd * dsz) % 16 == 0 && (p.strideD * dsz) % 16 == 0 && aligned16(p.D);
+  const bool bias_ok = !p.bias || (p.N % 8 == 0 && aligned16(p.bias));
+  const size_t a_bytes = a_ok ? 0 : (size_t)G * p.M * K8 * 2, b_bytes = b_ok ? 0 : (size_t)G * K8 * N8 * 2;
+  const size_t d_bytes = d_ok ? 0 : (size_t)G * p.M * N8 * dsz, bias_bytes = bias_ok ? 0 : (size_t)N8 * 4;
+  char* ws = nullptr;
+  if (hipMallocAsync(reinterpret_cast<void**>(&ws), a_bytes + b_bytes + d_bytes + bias_bytes + 16, s) != hipSuccess) {
+    (void)hipGetLastError();
+    return kDeviceFailed;
+  }
+  Gemm16Params q = p;
+  q.K = K8;
+  q.N = N8;
+  char* at = ws;
+  if (!a_ok) {
+    uint16_t* a2 = reinterpret_cast<uint16_t*>(at);
+    at += a_bytes;
+    hipLaunchKernelGGL(pad_rows_kernel<uint16_t>, copy_grid(p.M, K8, 8, G), copy_block(), 0, s, a2, (long)K8,
+                       (long)p.M * K8, p.A, p.lda, p.strideA, p.M, p.K, p.M);
+    q.A = a2; q.lda = K8; q.strideA = (long)p.M * K8;
+  }
+  if (!b_ok) {
+    uint16_t* b2 = reinterpret_cast<uint16_t*>(at);
+    at += b_bytes;
+    hipLaunchKernelGGL(pad_rows_kernel<uint16_t>, copy_grid(K8, N8, 8, G), copy_block(), 0, s, b2, (long)N8,
+                       (long)K8 * N8, p.B, p.ldb, p.strideB, p.K, p.N, K8);
+    q.B = b2; q.ldb = N8; q.strideB = (long)K8 * N8;
+  }
+  void* d2 = nullptr;
+  if (!d_ok) {
+    d2 = at;
+    at += d_bytes;
+    q.D = d2; q.ldd = N8; q.strideD = (long)p.M * N8;
+  }
+  if (!bias_ok) {
+    float* bias2 = reinterpret_cast<float*>(at);
+    hipLaunchKernelGGL(pad_rows_kernel<float>, copy_grid(1, N8, 4, 1), copy_block(), 0, s, bias2, (long)N8, (long)N8,
+                       p.bias, (long)p.N, (long)p.N, 1, p.N, 1);
+    q.bias = bias2;
+  }
+  int rc = launch_status();
+  if (rc == kOk) rc = launch_gemm16<T, EPI>(q, s);
+  if (rc == kOk && !d_ok) {
+    if constexpr (dsz == 4)
+      hipLaunchKernelGGL(unpad_rows_kernel<float>, copy_grid(p.M, N8, 4, G), copy_block(), 0, s, static_cast<float*>(p.D),
+                         p.ldd, p.strideD, static_cast<const float*>(d2), (long)N8, (long)p.M * N8, p.M, p.N);
+    else
+      hipLaunchKernelGGL(unpad_rows_kernel<uint16_t>, copy_grid(p.M, N8, 8, G), copy_block(), 0, s,
+                         static_cast<uint16_t*>(p.D), p.ldd, p.strideD, static_cast<const uint16_t*>(d2), (long)N8,
+                         (long)p.M * N8, p.M, p.N);
+    rc = launch_status();
+  }
+  if (hipFreeAsync(ws, s) != hipSuccess) { (void)hipGetLastError(); rc = rc == kOk ? kDeviceFailed : rc; }
+  return rc;
+}
+
+// The tiles first_tile .. first_tile + rest - 1 of a dense product on 256 x 256 tiles, each split
+// along K over `splits` workgroups, then summed (with the bias / activation of the product).
+template <class T, int EPI>
+int launch_gemm16_rest(Gemm16Params p, int first_tile, int rest, int splits, hipStream_t s) {
+  using S = Gemm16Smem<256, 256>;
+  auto kern = gemm16_rest_splitk_kernel<T, kBigTileMfma>;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, S::kBytes);
+  });
+  if (attr_err != hipSuccess) return kDeviceFailed;
+  float* ws = static_cast<float*>(stream_workspace(s, (size_t)rest * splits * 256 * 256 * sizeof(float)));
+  if (!ws) return kDeviceFailed;
+  p.tiles_m = ceil_div(p.M, 256);
+  p.tiles_n = ceil_div(p.N, 256);
+  const int ksplit = ceil_div(ceil_div(p.K, G16_BK), splits) * G16_BK;
+  hipLaunchKernelGGL(kern, dim3(rest, splits), dim3(256), S::kBytes, s, p, first_tile, ksplit, ws);
+  if (int rc = launch_status(); rc != kOk) return rc;
+  hipLaunchKernelGGL((gemm16_rest_sum_kernel<T, EPI>), dim3(64, rest), dim3(256), 0, s, ws, p.D, p.M, p.N, p.ldd,
+                     p.tiles_m, p.tiles_n, first_tile, splits, p.bias, p.act);
+  return launch_status();
+}
+
 // Dense / batched.  p.groups = batch count (>= 1).
 template <class T, int EPI>
 int launch_gemm16(Gemm16Params p, hipStream_t s) {
@@ -196,6 +414,11 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
                    ((p.strideD * dsz) % 16 == 0) && aligned16(p.A) && aligned16(p.B) && aligned16(p.D) &&
                    (!p.bias || aligned16(p.bias));
   if (!vec) {
+    // small products go one thread per output element; above about 2^24 multiply-adds the
+    // copies into aligned buffers cost less than that kernel loses
+    if ((double)p.M * p.N * p.K * p.groups >= (double)(1L << 24) && p.M >= 16 && p.N >= 16 &&
+        p.K + 8 < (1L << 21) && p.N + 8 < (1L << 21))
+      return launch_gemm16_repitched<T, EPI>(p, s);
     dim3 block(32, 8), grid(ceil_div(p.N, 32), ceil_div(p.M, 8), p.groups);
     hipLaunchKernelGGL((gemm16_generic_kernel<T, EPI>), grid, block, 0, s, p);
     return launch_status();
@@ -206,11 +429,18 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
   if constexpr (EPI != EPI_F32) {
     if (fused) return kBadShape;
   }
-  if (sch.tile == 256) {
-    if constexpr (EPI == EPI_F32) {
-      if (fused) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI_F32_FUSED, false, kBigTileMfma>(p, s);
+  if (sch.tile == 256 && sch.split_k == 1) {
+    const int tiles = ceil_div(p.M, 256) * ceil_div(p.N, 256);
+    const int main_wgs = sch.rest_split > 1 ? tiles / 256 * 256 : 0;     // 0: every tile in one launch
+    int rc = kOk;
+    if (EPI == EPI_F32 && fused) {
+      if constexpr (EPI == EPI_F32)
+        rc = launch_gemm16_tile<T, 256, 256, 2, 2, EPI_F32_FUSED, false, kBigTileMfma>(p, s, main_wgs);
+    } else {
+      rc = launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false, kBigTileMfma>(p, s, main_wgs);
     }
-    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, false, kBigTileMfma>(p, s);
+    if (rc != kOk || sch.rest_split <= 1) return rc;
+    return launch_gemm16_rest<T, EPI>(p, main_wgs, tiles - main_wgs, sch.rest_split, s);
   }
   const bool t128 = sch.tile == 128;
   if (sch.skinny && sch.split_k == 1) return launch_gemm16_skinny<T, EPI>(p, p.K, 1, s);
@@ -238,8 +468,9 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
         q.K = p.K;
         rc = launch_gemm16_skinny<T, EPI_F32>(q, ceil_div(ceil_div(p.K, splits), 32) * 32, splits, s);
       } else {
-        rc = t128 ? launch_gemm16_tile<T, 128, 128, 2, 2, EPI_F32, false>(q, s)
-                  : launch_gemm16_tile<T, 64, 64, 2, 2, EPI_F32, false>(q, s);
+        rc = sch.tile == 256 ? launch_gemm16_tile<T, 256, 256, 2, 2, EPI_F32, false, kBigTileMfma>(q, s)
+             : t128      ? launch_gemm16_tile<T, 128, 128, 2, 2, EPI_F32, false>(q, s)
+                         : launch_gemm16_tile<T, 64, 64, 2, 2, EPI_F32, false>(q, s);
       }
       if (rc == kOk) {
         const long quads = (long)p.M * (p.N / 4);

@@ -44,6 +44,8 @@ class Gfx950ScheduleDescriptor:
     source: str
     raster_order: str = "xcd_banded"
     raster_group: int = 4
+    rest_tiles: int = 0               # tiles beyond the last full round of 256 workgroups that are ...
+    rest_split_k: int = 1             # ... split along K into this many parts (1: none are)
 
     @property
     def mt(self) -> int:
@@ -65,6 +67,8 @@ class Gfx950ScheduleDescriptor:
             "schedule_raster_order": self.raster_order,
             "schedule_raster_group": self.raster_group,
             "schedule_split_k": self.split_k,
+            "schedule_rest_tiles": self.rest_tiles,
+            "schedule_rest_split_k": self.rest_split_k,
         }
 
     def cache_key(self) -> tuple:
@@ -85,6 +89,10 @@ def select_gfx950_gemm_schedule(m: int, n: int, k: int, *, dtype: str = "bf16", 
     _lane.check(_lane.load().tessera_gfx950_gemm_schedule(
         int(m), int(n), int(k), int(batch), nbytes, ctypes.byref(tm), ctypes.byref(tn), ctypes.byref(tk),
         ctypes.byref(sk)), "gemm_schedule")
+    rest_tiles, rest_split = ctypes.c_int(0), ctypes.c_int(1)
+    if nbytes == 2:
+        _lane.check(_lane.load().tessera_gfx950_gemm_rest_split(
+            int(m), int(n), int(k), int(batch), ctypes.byref(rest_tiles), ctypes.byref(rest_split)), "gemm_rest_split")
     inst = _INSTRUCTION_TILE[name]
     if name in ("f16", "bf16") and tm.value == 256:
         inst = (16, 16, 32)       # the 256 x 256 tiles run v_mfma_f32_16x16x32 (less power per FLOP)
@@ -96,7 +104,8 @@ def select_gfx950_gemm_schedule(m: int, n: int, k: int, *, dtype: str = "bf16", 
         lds_layout=("A from global in operand order; B wave-private [k][n] slices + transposing ds_read"
                     if tm.value == 32 else "A xor-swizzled 16B chunks; B natural [k][n] + transposing ds_read"),
         ownership="wave", vgpr_estimate=_VGPRS[tm.value], split_k=sk.value,
-        source="tessera_gfx950_gemm_schedule (the launcher's own decision)")
+        source="tessera_gfx950_gemm_schedule (the launcher's own decision)",
+        rest_tiles=rest_tiles.value, rest_split_k=rest_split.value)
 
 
 __all__ = ["Gfx950ScheduleDescriptor", "select_gfx950_gemm_schedule"]

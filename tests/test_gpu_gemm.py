@@ -84,6 +84,70 @@ def test_big_tile_k_and_edge_shapes(lane, M, N, K):
     assert np.array_equal(np.asarray(stored).view(np.uint16), np.asarray(b16.from_float32(acc)).view(np.uint16))
 
 
+# Products the launcher splits along K on the 256 x 256 tile (few tiles, long K), with the sum
+# over the splits by a second kernel, and ones it serves with 128 x 128 tiles unsplit.
+@pytest.mark.parametrize("M,N,K,tile,split", [
+    (1024, 8192, 8192, 256, 2), (8192, 1024, 8192, 256, 2), (900, 7992, 8192, 256, 2),
+    (2048, 2048, 2048, 128, 1), (2560, 2560, 2560, 128, 1), (1024, 1024, 8192, 128, 4)])
+def test_mid_size_schedules(lane, M, N, K, tile, split):
+    from tessera_amd.schedule import select_gfx950_gemm_schedule
+    sch = select_gfx950_gemm_schedule(M, N, K, dtype="bf16")
+    assert sch.workgroup_tile[:2] == (tile, tile) and sch.split_k == split
+    rng = np.random.default_rng(M + N + K)
+    a = b16.from_float32((rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32))
+    b = b16.from_float32(rng.standard_normal((K, N)).astype(np.float32))
+    ref = a.to_float32().astype(np.float64) @ b.to_float32().astype(np.float64)
+    acc = ops.gemm(a, b, out="f32")
+    assert orc.max_rel_err(acc, ref) <= 1e-5
+    stored = ops.gemm(a, b)
+    assert np.array_equal(np.asarray(stored).view(np.uint16), np.asarray(b16.from_float32(acc)).view(np.uint16))
+    bias = rng.standard_normal(N).astype(np.float32)
+    fused = ops.fused_gemm(a, b, bias=bias, activation="relu")
+    assert orc.max_rel_err(fused, np.maximum(ref + bias, 0.0)) <= 1e-5
+
+
+# Tile counts a little over a multiple of 256: the tiles beyond the last full round are split along
+# K by a second launch and summed by a third (ragged edges, K that the splits do not divide, the
+# fused epilogue on both kinds of tile).
+@pytest.mark.parametrize("M,N,K", [(4096, 4104, 4096), (4352, 4096, 1000), (4350, 4088, 2056), (4100, 4360, 2000), (6140, 6136, 2048)])
+def test_rest_round_split_along_k(lane, M, N, K):
+    from tessera_amd.schedule import select_gfx950_gemm_schedule
+    sch = select_gfx950_gemm_schedule(M, N, K, dtype="bf16")
+    assert sch.workgroup_tile[:2] == (256, 256) and sch.split_k == 1 and sch.rest_split_k > 1
+    assert sch.rest_tiles == (-(-M // 256) * -(-N // 256)) % 256
+    rng = np.random.default_rng(M + 2 * N + 3 * K)
+    a = b16.from_float32((rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32))
+    b = b16.from_float32(rng.standard_normal((K, N)).astype(np.float32))
+    ref = a.to_float32().astype(np.float64) @ b.to_float32().astype(np.float64)
+    acc = ops.gemm(a, b, out="f32")
+    assert orc.max_rel_err(acc, ref) <= 1e-5
+    stored = ops.gemm(a, b)
+    assert np.array_equal(np.asarray(stored).view(np.uint16), np.asarray(b16.from_float32(acc)).view(np.uint16))
+    bias = rng.standard_normal(N).astype(np.float32)
+    fused = ops.fused_gemm(a, b, bias=bias, activation="silu")
+    x = ref + bias
+    assert orc.max_rel_err(fused, x / (1.0 + np.exp(-x))) <= 1e-5
+
+
+# K or N not a multiple of 8 (rows off the 16-byte grid): large products are copied into aligned,
+# zero-padded buffers and run on the tile kernels; small ones take the one-thread-per-element kernel.
+@pytest.mark.parametrize("M,N,K", [(517, 1003, 771), (2050, 4100, 1028), (4100, 2052, 4100), (300, 50257, 768),
+                                   (1000, 1000, 1001), (64, 515, 520), (40, 41, 42)])
+@pytest.mark.parametrize("st", ["bf16", "f16"])
+def test_unaligned_shapes(lane, M, N, K, st):
+    rng = np.random.default_rng(M * 3 + N * 5 + K)
+    A = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    ref = orc.gemm_f64(A, B, st)
+    a = b16.from_float32(A) if st == "bf16" else A.astype(np.float16)
+    b = b16.from_float32(B) if st == "bf16" else B.astype(np.float16)
+    acc = ops.gemm(a, b, out="f32")
+    assert acc.shape == (M, N) and orc.max_rel_err(acc, ref) <= 1e-5
+    stored = ops.gemm(a, b)
+    sf = stored.to_float32() if st == "bf16" else stored.astype(np.float32)
+    assert np.array_equal(sf, orc.round_to_storage(acc, st))
+
+
 def test_readme_batched_gemm_config(lane):
     """A[4,128,64] f16 x W[4,64,256] f16 -> f32 accumulate (README step())."""
     rng = np.random.default_rng(0)
