@@ -212,6 +212,46 @@ def bench_attention(lane, steps, warmup, check=True):
     return out
 
 
+def bench_attention_decode(lane, steps, warmup, check=True):
+    """One query row per head against a long key range (a decode step with a KV cache): bound by
+    reading K and V once, 537 MB here (more than the memory-side cache holds).  The rows of a GQA
+    group share one MFMA tile and the key range is split over the chip (the decode kernel)."""
+    B, Hq, Hkv, Sk, D = 64, 32, 8, 2048, 128
+    rng = np.random.default_rng(2)
+    q = _bf16(rng.standard_normal((B, Hq, 1, D), dtype=np.float32))
+    # eight distinct batches of K / V, repeated: the bytes streamed are what matters for the timing
+    k8 = _bf16(rng.standard_normal((8, Hkv, Sk, D), dtype=np.float32))
+    v8 = _bf16(rng.standard_normal((8, Hkv, Sk, D), dtype=np.float32))
+    k, v = np.tile(k8, (B // 8, 1, 1, 1)), np.tile(v8, (B // 8, 1, 1, 1))
+    dq, dk, dv = (lane.DeviceBuffer.from_host(x) for x in (q, k, v))
+    do = lane.DeviceBuffer(q.size * 4)
+    dl = lane.DeviceBuffer(B * Hq * 4)
+    fn = lane.load().tessera_gfx950_flash_attn_gqa_bf16_dev
+    scale = 1.0 / np.sqrt(D)
+
+    def launch():
+        lane.check(fn(dq.ptr, dk.ptr, dv.ptr, do.ptr, dl.ptr, B, Hq, Hkv, 1, Sk, D, scale, 0, 0, None), "flash_attn")
+
+    wall, ev = _timed(lane, launch, max(steps, 50), warmup)
+    nbytes = 2 * k.size * 2 + q.size * 2 + q.size * 4
+    out = {"workload": f"flash_attn_decode_bf16_B{B}_Hq{Hq}_Hkv{Hkv}_Sq1_Sk{Sk}_D{D}", "ms": ev,
+           "gbs": nbytes / ev / 1e6, "frac_hbm_peak": nbytes / ev / 1e6 / PEAK_HBM_GBS}
+    if check:
+        orc = _oracle()
+        lane.synchronize()
+        got_o = do.download((B, Hq, 1, D), np.float32)
+        got_l = dl.download((B, Hq, 1), np.float32)
+        f32 = lambda bits: (bits.astype(np.uint32) << 16).view(np.float32)
+        sample = [0, 9, 63]
+        ro, rl = orc.flash_attn_dense(f32(q[sample]), f32(k[sample]), f32(v[sample]), scale=scale, causal=False)
+        out["parity"] = {"o_max_rel": orc.max_rel_err(got_o[sample], ro),
+                         "lse_max_abs": float(np.max(np.abs(got_l[sample] - rl))), "bound": 2e-3,
+                         "sample": f"{len(sample)} of {B} batches, all heads, dense f64 oracle"}
+    for buf in (dq, dk, dv, do, dl):
+        buf.close()
+    return out
+
+
 def bench_attention_bwd(lane, steps, warmup):
     """Backward of the same attention configuration with the forward's O and LSE
     saved (dQ, dK, dV kernels + the Delta pass), and with the forward recomputed."""
@@ -786,14 +826,16 @@ def cpu_baseline(A, B):
                  "sample": f"full {M}x{N}x{K} product once, numpy f32 matmul of the bf16-rounded operands, {dt:.2f} s"}
 
 
-ALSO = ("flash_attn", "flash_attn_bwd", "quant", "gemm_constant", "batched", "decode", "moe", "mfma_ceiling",
-        "vendor_gemm")
+ALSO = ("flash_attn", "flash_attn_decode", "flash_attn_bwd", "quant", "gemm_constant", "batched", "decode", "moe",
+        "mfma_ceiling", "vendor_gemm")
 
 
 def run_also(lane, name, steps, warmup, check):
     """One of the `also` workloads -> dict of result entries."""
     if name == "flash_attn":
         return {"flash_attn": bench_attention(lane, steps, warmup, check)}
+    if name == "flash_attn_decode":
+        return {"flash_attn_decode": bench_attention_decode(lane, steps, warmup, check)}
     if name == "flash_attn_bwd":
         return {"flash_attn_bwd": bench_attention_bwd(lane, steps, warmup)}
     if name == "quant":

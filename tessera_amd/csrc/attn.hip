@@ -3,6 +3,7 @@
 #include <mutex>
 #include "../../include/tessera_gfx950.h"
 #include "flash_attn.h"
+#include "flash_decode.h"
 #include "flash_bwd.h"
 #include "host_util.h"
 
@@ -47,6 +48,56 @@ int launch_flash_for(const FlashParams& p, bool ext, hipStream_t s) {
   if (p.D < 64) return ext ? launch_flash<T, 64, true, true>(p, s) : launch_flash<T, 64, false, true>(p, s);
   if (p.D < 128) return ext ? launch_flash<T, 128, true, true>(p, s) : launch_flash<T, 128, false, true>(p, s);
   return ext ? launch_flash<T, 256, true, true>(p, s) : launch_flash<T, 256, false, true>(p, s);
+}
+
+// Few query rows per KV head (decode, short speculative steps): the rows of a whole GQA group
+// share one MFMA tile and the key range is split over workgroups (flash_decode.h).  Returns
+// false when the problem is not of that kind (the general kernel then serves it).
+template <class T, int DP>
+int launch_decode(const FlashParams& p, hipStream_t s) {
+  using G = DecodeGeom<DP>;
+  auto kern = flash_decode_kernel<T, DP>;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, G::SMEM);
+  });
+  if (attr_err != hipSuccess) return kDeviceFailed;
+  FlashDecodeParams dp{};
+  dp.f = p;
+  dp.rows = p.ratio * p.Sq;
+  int lo0, hi0, lo1, hi1;
+  key_bounds(0, p.Sq, p.Sk, p.causal, p.window, lo0, hi0);
+  key_bounds(p.Sq - 1, p.Sq, p.Sk, p.causal, p.window, lo1, hi1);
+  dp.tile_lo = lo0 / G::BK;
+  dp.tile_end = hi1 / G::BK + 1;
+  const int tiles = dp.tile_end - dp.tile_lo;
+  // about two workgroups per compute unit, and at least two tiles for every wave of a split
+  const int kvheads = p.B * p.Hkv;
+  int nsplit = std::max(1, std::min(ceil_div(512, kvheads), tiles / (2 * G::WAVES)));
+  dp.tiles_per_split = ceil_div(ceil_div(tiles, nsplit), G::WAVES) * G::WAVES;
+  nsplit = ceil_div(tiles, dp.tiles_per_split);
+  if (nsplit > 1) {
+    const size_t rows = (size_t)p.B * p.Hq * p.Sq;
+    float* ws = static_cast<float*>(stream_workspace(s, (size_t)nsplit * rows * (DP + 1) * sizeof(float)));
+    if (!ws) return kDeviceFailed;
+    dp.part_o = ws;
+    dp.part_lse = ws + (size_t)nsplit * rows * DP;
+  }
+  hipLaunchKernelGGL(kern, dim3(kvheads, nsplit), dim3(G::THREADS), G::SMEM, s, dp);
+  if (int rc = launch_status(); rc != kOk || nsplit == 1) return rc;
+  const long quads = (long)p.B * p.Hq * p.Sq * (DP / 4);
+  hipLaunchKernelGGL((flash_decode_merge_kernel<T>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p,
+                     dp.part_o, dp.part_lse, nsplit);
+  return launch_status();
+}
+inline bool decode_shaped(const FlashParams& p) {
+  if ((long)p.ratio * p.Sq > 32 || !(p.D == 64 || p.D == 128 || p.D == 256)) return false;
+  int lo0, hi0, lo1, hi1;
+  key_bounds(0, p.Sq, p.Sk, p.causal, p.window, lo0, hi0);
+  key_bounds(p.Sq - 1, p.Sq, p.Sk, p.causal, p.window, lo1, hi1);
+  return hi1 >= lo0;                                   // some row sees some key
 }
 
 // Contiguous [B, H, S, D].
@@ -98,6 +149,11 @@ int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, i
   // The plain variant takes row maxima of the raw scores, which needs scale > 0; the
   // extended one scales first and serves every other scale.
   const bool ext = p.softcap > 0.f || p.bias != nullptr || !(scale > 0.f);
+  if (al && !ext && decode_shaped(p)) {
+    if (p.D == 64) return launch_decode<T, 64>(p, s);
+    if (p.D == 128) return launch_decode<T, 128>(p, s);
+    return launch_decode<T, 256>(p, s);
+  }
   if (al) return launch_flash_for<T>(p, ext, s);
   const long rows = (long)B * Hq * Sq;
   hipLaunchKernelGGL((flash_fwd_generic_kernel<T>), dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, p);

@@ -57,6 +57,58 @@ def test_attention_matches_oracle(lane, B, Hq, Hkv, Sq, Sk, D, causal, st):
     assert np.max(np.abs(lse - ref_lse)) <= TOL
 
 
+# Few query rows per KV head — (Hq / Hkv) * Sq <= 32 with D in {64, 128, 256} — take the decode
+# kernel: the rows of a GQA group share one MFMA tile, the key range is split over workgroups
+# and waves, partials are merged.  One and many key splits, ratio 1 to 16, rows that fill the
+# tile and that do not, ragged last tile, causal steps of several rows, a sliding window.
+DECODE_CASES = [
+    # B, Hq, Hkv, Sq, Sk, D, causal, window
+    (2, 8, 2, 1, 777, 128, False, 0), (1, 32, 8, 1, 8192, 128, False, 0), (3, 16, 16, 1, 300, 64, False, 0),
+    (2, 8, 1, 4, 1000, 128, True, 0), (1, 4, 4, 7, 129, 256, True, 0), (2, 6, 2, 3, 64, 64, True, 0),
+    (1, 16, 1, 2, 4100, 128, True, 0), (1, 8, 2, 1, 5000, 128, True, 1024), (1, 2, 2, 16, 31, 128, False, 0),
+    (40, 8, 2, 1, 2048, 128, False, 0), (1, 8, 8, 1, 33000, 64, False, 0), (2, 4, 1, 8, 20, 256, True, 0),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,window", DECODE_CASES)
+@pytest.mark.parametrize("st", ["bf16", "f16"])
+def test_decode_shapes_match_oracle(lane, B, Hq, Hkv, Sq, Sk, D, causal, window, st):
+    q, k, v = _qkv(B, Hq, Hkv, Sq, Sk, D, 23, st)
+    ref_o, ref_lse = orc.flash_attn_dense(_f32(q), _f32(k), _f32(v), causal=causal, window=window)
+    o, lse = ops.gqa_attention(q, k, v, causal=causal, return_lse=True, out="f32", window=window)
+    assert not np.isnan(o).any()
+    assert orc.max_rel_err(o, ref_o) <= TOL
+    assert np.max(np.abs(lse - ref_lse)) <= TOL
+    stored = ops.gqa_attention(q, k, v, causal=causal, window=window)
+    assert orc.max_rel_err(_f32(stored), ref_o) <= TOL + (2.0 ** -8 if st == "bf16" else 2.0 ** -11)
+
+
+def test_decode_kernel_reads_k_and_v_about_once(lane):
+    """What the decode kernel is for: one query row per head against a long key range runs
+    near the rate at which K and V can be read once, not once per query head."""
+    import ctypes
+    import time
+    B, Hq, Hkv, Sk, D = 16, 32, 8, 4096, 128
+    rng = np.random.default_rng(1)
+    mk = lambda *shape: lane.DeviceBuffer.from_host((rng.standard_normal(shape).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16))
+    q, k, v = mk(B, Hq, 1, D), mk(B, Hkv, Sk, D), mk(B, Hkv, Sk, D)
+    o = lane.DeviceBuffer(B * Hq * D * 2)
+    fn = lane.load().tessera_gfx950_flash_attn_gqa_bf16_dev
+    call = lambda: lane.check(fn(q.ptr, k.ptr, v.ptr, o.ptr, None, B, Hq, Hkv, 1, Sk, D, ctypes.c_float(D ** -0.5), 0, 1, None), "decode")
+    for _ in range(5):
+        call()
+    lane.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(20):
+        call()
+    lane.synchronize()
+    per_call = (time.perf_counter() - t0) / 20
+    kv_bytes = 2 * B * Hkv * Sk * D * 2
+    for b in (q, k, v, o):
+        b.close()
+    assert kv_bytes / per_call > 1.5e12, f"{kv_bytes / per_call / 1e12:.2f} TB/s"     # the general kernel: 2.1e12 / 4 heads
+
+
 @pytest.mark.parametrize("scale", [0.3, 1e-3, 0.0, -0.07])
 def test_attention_scales(lane, scale):
     """Any finite scale: a negative one turns the row maximum of the raw scores into
