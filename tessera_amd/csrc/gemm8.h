@@ -41,6 +41,8 @@ struct Gemm8Params {
   float scale_a, scale_b;    // FP8
   int M, N, K;
   int tiles_m, tiles_n;
+  int ksplit;                // > 0: workgroup (tile, z = blockIdx.y) computes K range [z ksplit, (z + 1) ksplit)
+                             // and stores at D + z M N (partial results, summed by gemm8_split_sum_kernel)
 };
 
 constexpr int G8_BK = 128;       // K step in bytes (= elements)
@@ -86,12 +88,15 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
   int tm, tn;
   tile_of_block8(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
   const int m_begin = tm * G8_BM, n_begin = tn * G8_BN;
-  const int K = p.K;
+  // K range of this workgroup: all of it, or slice blockIdx.y of a split product.  (`K` below is the
+  // length of the range; rows of A are p.K bytes apart either way.)
+  const int kz = p.ksplit > 0 ? (int)blockIdx.y * p.ksplit : 0;
+  const int K = p.ksplit > 0 ? min(p.ksplit, p.K - kz) : p.K;
 
   // Global addressing: a wave-uniform tile base (advanced along K on the scalar unit)
   // plus a fixed 32-bit per-lane offset, so a chunk costs one address register.
-  const uint8_t* a_base = p.A + (long)m_begin * K;
-  const uint8_t* b_base = p.B + n_begin;
+  const uint8_t* a_base = p.A + (long)m_begin * p.K + kz;
+  const uint8_t* b_base = p.B + (long)kz * p.N + n_begin;
   uint32_t a_off[A_CHUNKS], a_lds[A_CHUNKS];
   const int a_chunk = tid & 7;
 #pragma unroll
@@ -99,7 +104,7 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
     const int row = (tid >> 3) + 32 * q;
     int gr = row;
     gr = m_begin + gr < p.M ? gr : p.M - 1 - m_begin;          // clamp: rows past the edge are never stored
-    a_off[q] = (uint32_t)gr * (uint32_t)K + a_chunk * 16;
+    a_off[q] = (uint32_t)gr * (uint32_t)p.K + a_chunk * 16;
     a_lds[q] = row * G8_APITCH + ((a_chunk ^ ((row >> 1) & 7)) << 4);
   }
   uint32_t b_off[B_CHUNKS], b_lds[B_CHUNKS];
@@ -389,10 +394,12 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
       __builtin_amdgcn_wave_barrier();
     }
   };
+  char* out_base = reinterpret_cast<char*>(p.D);
+  if (p.ksplit > 0) out_base += (long)blockIdx.y * p.M * p.N * DSZ;   // this slice's partial result
   if constexpr (EPI == EPI8_I32) {
-    pass(reinterpret_cast<char*>(p.D), true_type{});
+    pass(out_base, true_type{});
   } else {
-    pass(reinterpret_cast<char*>(p.D), false_type{});
+    pass(out_base, false_type{});
     if constexpr (EPI == EPI8_W8A8_F32) {
       if (p.acc_out) pass(reinterpret_cast<char*>(p.acc_out), true_type{});
     }
@@ -408,6 +415,54 @@ __device__ __forceinline__ float e4m3_to_f32(uint8_t c) {
   else if (e == 15 && m == 7) v = __builtin_nanf("");
   else v = __builtin_bit_cast(float, ((e + 120u) << 23) | (m << 20));
   return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) | s);
+}
+
+// A product split along K: the slices' partial results (int32 accumulators, or f32 ones of the fp8
+// form computed with unit scales), [splits][M][N], are summed in slice order and passed through
+// the product's epilogue.  int32 sums are exact, so the int8 forms give the bits of the unsplit
+// kernel; the f32 sum of the fp8 form is one fixed order.  Four columns per thread.
+template <class T, int EPI>
+__global__ __launch_bounds__(256) void gemm8_split_sum_kernel(const void* __restrict__ part, int splits, const Gemm8Params p) {
+  constexpr bool IS_I8 = std::is_same<T, I8>::value;
+  const long quad = (long)blockIdx.x * 256 + threadIdx.x;
+  const int nq = p.N / 4;
+  if (quad >= (long)p.M * nq) return;
+  const int m = (int)(quad / nq), n = (int)(quad - (long)m * nq) * 4;
+  const long o = (long)m * p.N + n, mn = (long)p.M * p.N;
+  float v[4];
+  if constexpr (IS_I8) {
+    int4 acc = make_int4(0, 0, 0, 0);
+    for (int z = 0; z < splits; ++z) {
+      const int4 a = *reinterpret_cast<const int4*>(reinterpret_cast<const int32_t*>(part) + z * mn + o);
+      acc.x += a.x; acc.y += a.y; acc.z += a.z; acc.w += a.w;
+    }
+    if constexpr (EPI == EPI8_I32) {
+      *reinterpret_cast<int4*>(reinterpret_cast<int32_t*>(p.D) + o) = acc;
+      return;
+    } else {
+      if (p.acc_out) *reinterpret_cast<int4*>(p.acc_out + o) = acc;
+      const float rs = p.row_scale[m];
+      const float4 cs = *reinterpret_cast<const float4*>(p.col_scale + n);
+      v[0] = ((float)acc.x * rs) * cs.x; v[1] = ((float)acc.y * rs) * cs.y;
+      v[2] = ((float)acc.z * rs) * cs.z; v[3] = ((float)acc.w * rs) * cs.w;
+    }
+  } else {
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int z = 0; z < splits; ++z) {
+      const float4 a = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(part) + z * mn + o);
+      acc.x += a.x; acc.y += a.y; acc.z += a.z; acc.w += a.w;
+    }
+    v[0] = (acc.x * p.scale_a) * p.scale_b; v[1] = (acc.y * p.scale_a) * p.scale_b;
+    v[2] = (acc.z * p.scale_a) * p.scale_b; v[3] = (acc.w * p.scale_a) * p.scale_b;
+  }
+  if constexpr (EPI == EPI8_SCALED_BF16) {
+    uint2 pk;
+    pk.x = pack2<BF16>(v[0], v[1]);
+    pk.y = pack2<BF16>(v[2], v[3]);
+    *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.D) + o) = pk;
+  } else if constexpr (EPI != EPI8_I32) {
+    *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.D) + o) = make_float4(v[0], v[1], v[2], v[3]);
+  }
 }
 
 // Any-shape fallback, one thread per output element, k in order.

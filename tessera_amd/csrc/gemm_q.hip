@@ -10,6 +10,18 @@ namespace {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// The tile kernel needs more dynamic LDS than the default limit: raised once per instantiation.
+template <class T, int EPI>
+int gemm8_attr() {
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_kernel<T, EPI>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, G8_SMEM);
+  });
+  return attr_err == hipSuccess ? kOk : kDeviceFailed;
+}
+
 template <class T, int EPI>
 int gemm8_dev(Gemm8Params p, hipStream_t s) {
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || !p.A || !p.B || !p.D) return kBadShape;
@@ -23,17 +35,45 @@ int gemm8_dev(Gemm8Params p, hipStream_t s) {
     hipLaunchKernelGGL((gemm8_generic_kernel<T, EPI>), grid, block, 0, s, p);
     return launch_status();
   }
-  auto kern = gemm8_kernel<T, EPI>;
-  static std::once_flag once;
-  static hipError_t attr_err = hipSuccess;
-  std::call_once(once, [&] {
-    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, G8_SMEM);
-  });
-  if (attr_err != hipSuccess) return kDeviceFailed;
   p.tiles_m = ceil_div(p.M, G8_BM);
   p.tiles_n = ceil_div(p.N, G8_BN);
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(256), G8_SMEM, s, p);
+  p.ksplit = 0;
+  // Few tiles and a long K (few rows against a big weight matrix): K is split over the idle compute
+  // units, the slices write raw accumulators to the stream workspace and a second kernel sums them
+  // and applies the epilogue.  The number of slices (a power of two, tiles x slices within the 256
+  // compute units, every slice at least 512 deep) is the one with the least estimated time: a tile
+  // costs 9.6 us plus 1.2 us per 128-deep K step, the sum kernel reads the partials and writes the
+  // result at about 4.4 TB/s (figures fitted to timings on this part).
+  const int tiles = p.tiles_m * p.tiles_n;
+  int splits = 1;
+  if (tiles <= 128) {
+    const int ksteps = ceil_div(p.K, G8_BK);
+    double best_us = 9.6 + 1.2 * ksteps;
+    for (int sp = 2; sp <= 16 && tiles * sp <= 256 && p.K / sp >= 512; sp *= 2) {
+      const double us = 9.6 + 1.2 * ceil_div(ksteps, sp) + 2.0 + (double)p.M * p.N * (4.0 * sp + 4.0) / 4.4e6;
+      if (us < best_us) { best_us = us; splits = sp; }
+    }
+  }
+  if (splits > 1) {
+    // raw accumulators: int32 for int8 operands, f32 with unit scales for fp8
+    constexpr int RAW_EPI = std::is_same<T, I8>::value ? EPI8_I32 : EPI8_SCALED_F32;
+    if (int rc = gemm8_attr<T, RAW_EPI>(); rc != kOk) return rc;
+    void* ws = stream_workspace(s, (size_t)splits * p.M * p.N * 4);
+    if (!ws) return kDeviceFailed;
+    Gemm8Params q = p;
+    q.D = ws;
+    q.acc_out = nullptr;
+    q.scale_a = q.scale_b = 1.f;
+    q.ksplit = ceil_div(ceil_div(p.K, G8_BK), splits) * G8_BK;
+    hipLaunchKernelGGL((gemm8_kernel<T, RAW_EPI>), dim3(tiles, splits), dim3(256), G8_SMEM, s, q);
+    if (int rc = launch_status(); rc != kOk) return rc;
+    const long quads = (long)p.M * (p.N / 4);
+    hipLaunchKernelGGL((gemm8_split_sum_kernel<T, EPI>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, ws,
+                       splits, p);
+    return launch_status();
+  }
+  if (int rc = gemm8_attr<T, EPI>(); rc != kOk) return rc;
+  hipLaunchKernelGGL((gemm8_kernel<T, EPI>), dim3(tiles), dim3(256), G8_SMEM, s, p);
   return launch_status();
 }
 
