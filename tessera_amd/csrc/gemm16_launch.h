@@ -491,9 +491,53 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
   return launch_gemm16_tile<T, 64, 64, 2, 2, EPI, false>(p, s);
 }
 
+// D[i] = act(G[i]) * U[i], four elements per thread (n % 4 == 0, 16-byte aligned pointers).
+template <int ACT_DYNAMIC = 1>   // (a template so that every translation unit may include this header)
+__global__ __launch_bounds__(256) void gate_mul_kernel(float* __restrict__ D, const float* __restrict__ G,
+                                                       const float* __restrict__ U, long n4, int act) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n4) return;
+  const float4 g = reinterpret_cast<const float4*>(G)[i], u = reinterpret_cast<const float4*>(U)[i];
+  reinterpret_cast<float4*>(D)[i] =
+      make_float4(activate(g.x, act) * u.x, activate(g.y, act) * u.y, activate(g.z, act) * u.z, activate(g.w, act) * u.w);
+}
+
 // Dense gated product D f32 = act(A Wg) * (A Wu); p.B = Wg, p.B2 = Wu, p.N = H.
 template <class T>
 int launch_gemm16_gated(Gemm16Params p, hipStream_t s) {
+  // Few rows: both products are bound by reading their weight matrix once, which the dense
+  // launcher's decode schedules (small tiles, K split over the chip) do at several times the rate
+  // of one 256-row tile per 128 output columns.  Two products into stream-ordered scratch, then
+  // the gate.
+  if (p.M <= kWeightStreamMaxM && p.N % 8 == 0 && p.K % 8 == 0 && p.ldd == p.N && aligned16(p.D) &&
+      (long)p.M * p.N >= 128L * 128L) {
+    const size_t mn = (size_t)p.M * p.N;
+    float* tmp = nullptr;
+    if (hipMallocAsync(reinterpret_cast<void**>(&tmp), 2 * mn * sizeof(float), s) != hipSuccess) {
+      (void)hipGetLastError();
+      return kDeviceFailed;
+    }
+    Gemm16Params q = p;
+    q.B2 = nullptr;
+    q.act = ACT_NONE;
+    q.bias = nullptr;
+    q.groups = 1;
+    q.strideA = q.strideB = q.strideD = 0;
+    q.D = tmp;
+    int rc = launch_gemm16<T, EPI_F32>(q, s);
+    if (rc == kOk) {
+      q.B = p.B2;
+      q.D = tmp + mn;
+      rc = launch_gemm16<T, EPI_F32>(q, s);
+    }
+    if (rc == kOk) {
+      hipLaunchKernelGGL(gate_mul_kernel<1>, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, s,
+                         static_cast<float*>(p.D), tmp, tmp + mn, (long)(mn / 4), p.act);
+      rc = launch_status();
+    }
+    if (hipFreeAsync(tmp, s) != hipSuccess) { (void)hipGetLastError(); rc = rc == kOk ? kDeviceFailed : rc; }
+    return rc;
+  }
   const bool vec = (p.K % 8 == 0) && (p.N % 8 == 0) && (p.lda % 8 == 0) && (p.ldb % 8 == 0) &&
                    (p.lda < (1L << 21)) && (p.ldb < (1L << 21)) && (p.ldd % 4 == 0) && aligned16(p.A) &&
                    aligned16(p.B) && aligned16(p.B2) && aligned16(p.D);

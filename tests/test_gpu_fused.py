@@ -59,7 +59,9 @@ def test_fused_gemm_closed_forms(lane):
     assert np.array_equal(ops.fused_gemm(a, b, np.full(256, 1.5, np.float32), "none"), plain + np.float32(1.5))
 
 
-@pytest.mark.parametrize("M,H,K", [(512, 640, 256), (8, 16, 12), (130, 264, 72), (256, 128, 1024)])
+@pytest.mark.parametrize("M,H,K", [(512, 640, 256), (8, 16, 12), (130, 264, 72), (256, 128, 1024),
+                                   # few rows: two weight-streaming products and a gate kernel
+                                   (16, 2048, 4096), (128, 1024, 520), (1, 16384, 1024), (100, 264, 72)])
 @pytest.mark.parametrize("act", ["silu", "gelu", "relu", "sigmoid", "tanh"])
 def test_gated_gemm_matches_oracle(lane, M, H, K, act):
     rng = np.random.default_rng(H + K)
