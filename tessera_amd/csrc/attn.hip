@@ -294,6 +294,137 @@ int flash_bwd_padded_dev(const void* dO, const void* Q, const void* K, const voi
   return rc;
 }
 
+// ---- backward for head dimensions above 128, as dense products ------------------------------
+// The flash kernels hold a query (or key) block's accumulators and operand fragments in
+// registers, which stops at D = 128.  Above it the backward of one (batch, KV head) group is five
+// dense products on the GEMM kernels around one elementwise kernel, with S and dP of the group
+// written out (rows = (Hq / Hkv) Sq query rows of the group's heads, one after the other):
+//   S  = Qg K^T, dP = dOg V^T                     [rows, Sk] f32   (K^T, V^T: transposed copies)
+//   P  = exp(scale S - LSE),  dS = scale P (dP - Delta), masked  -> dS [rows, Sk], P^T, dS^T [Sk, rows]
+//   dQg = dS K,   dV = P^T dOg,   dK = dS^T Qg    (the sums over the group's heads are part of
+//                                                  the last two contractions)
+// At D = 256 a score costs 2 D = 512 multiply-adds per product against 14 bytes of S, dP, P and
+// dS traffic, so the dense form stays within a small factor of a fused kernel; it does not skip
+// the masked half of a causal problem.  Groups are processed in chunks that bound the scratch.
+
+// dst[z][c][r] = src[z][r][c], 16-bit elements, 64 x 64 tiles through LDS.
+__global__ __launch_bounds__(256) void transpose16_kernel(uint16_t* __restrict__ dst, const uint16_t* __restrict__ src,
+                                                          int R, int C) {
+  __shared__ uint16_t tile[64][66];
+  const long z = blockIdx.z;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4)
+    if (r0 + i < R && c0 + tx < C) tile[i][tx] = src[(z * R + r0 + i) * C + c0 + tx];
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4)
+    if (c0 + i < C && r0 + tx < R) dst[(z * C + c0 + i) * R + r0 + tx] = tile[tx][i];
+}
+
+// One 64 x 64 tile of (rows, keys) per workgroup: P and dS from S and dP (see above).  Row r of
+// group z is query r % Sq of the group's head r / Sq; lse / delta are indexed [z][r].
+template <class T>
+__global__ __launch_bounds__(256) void bwd_dense_softmax_kernel(const float* __restrict__ S, const float* __restrict__ dP,
+                                                                const float* __restrict__ lse,
+                                                                const float* __restrict__ delta, uint16_t* __restrict__ dS,
+                                                                uint16_t* __restrict__ PT, uint16_t* __restrict__ dST,
+                                                                int rows, int Sq, int Sk, float scale, int causal) {
+  __shared__ uint16_t pt[64][66], dst[64][66];
+  const long z = blockIdx.z;
+  const int r0 = blockIdx.y * 64, k0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int off = Sk > Sq ? Sk - Sq : 0;
+  const int key = k0 + tx;
+  for (int i = ty; i < 64; i += 4) {
+    const int r = r0 + i;
+    uint16_t pb = 0, db = 0;
+    if (r < rows && key < Sk) {
+      const long at = (z * rows + r) * Sk + key;
+      const int q = r % Sq;
+      const bool seen = !causal || key <= q + off;
+      float pv = 0.f, dv = 0.f;
+      if (seen) {
+        pv = __expf(scale * S[at] - lse[z * rows + r]);
+        dv = scale * pv * (dP[at] - delta[z * rows + r]);
+      }
+      pb = to_storage<T>(pv);
+      db = to_storage<T>(dv);
+      dS[at] = db;
+    }
+    pt[i][tx] = pb;
+    dst[i][tx] = db;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int k = k0 + i, r = r0 + tx;
+    if (k < Sk && r < rows) {
+      const long at = (z * Sk + k) * rows + r;
+      PT[at] = pt[tx][i];
+      dST[at] = dst[tx][i];
+    }
+  }
+}
+
+template <class T>
+int gemm_f32_batched(const void* A, const void* B, void* D, int batch, int M, int N, int K, long sa, long sb, long sd,
+                     hipStream_t s) {
+  if constexpr (std::is_same<T, BF16>::value)
+    return tessera_gfx950_batched_gemm_strided_bf16_dev(A, B, D, batch, M, N, K, sa, sb, sd, 0, s);
+  else
+    return tessera_gfx950_batched_gemm_strided_f16_dev(A, B, D, batch, M, N, K, sa, sb, sd, 0, s);
+}
+
+// O and LSE as saved by the forward (not null), Delta scratch [B Hq Sq] from the caller.
+template <class T>
+int flash_bwd_dense_dev(const void* dO, const void* Q, const void* K, const void* V, const float* LSE, const float* Delta,
+                        float* dQ, float* dK, float* dV, int B, int Hq, int Hkv, int Sq, int Sk, int D, float scale,
+                        int causal, hipStream_t s) {
+  const int ratio = Hq / Hkv, groups = B * Hkv;
+  const long rows = (long)ratio * Sq;
+  // per group: S, dP f32; dS, P^T, dS^T 16-bit; K^T, V^T 16-bit
+  const size_t per_group = (size_t)rows * Sk * (4 + 4 + 2 + 2 + 2) + (size_t)2 * Sk * D * 2;
+  const size_t budget = (size_t)2 << 30;                                      // aim for 2 GiB of scratch per chunk
+  const int gpc = (int)std::max<size_t>(1, std::min<size_t>(groups, budget / per_group));
+  char* ws = nullptr;
+  if (hipMallocAsync(reinterpret_cast<void**>(&ws), per_group * gpc + 256, s) != hipSuccess) {
+    (void)hipGetLastError();
+    return kDeviceFailed;
+  }
+  const size_t e = (size_t)rows * Sk;
+  float* Sb = reinterpret_cast<float*>(ws);
+  float* dPb = Sb + e * gpc;
+  uint16_t* dSb = reinterpret_cast<uint16_t*>(dPb + e * gpc);
+  uint16_t* PTb = dSb + e * gpc;
+  uint16_t* dSTb = PTb + e * gpc;
+  uint16_t* KTb = dSTb + e * gpc;
+  uint16_t* VTb = KTb + (size_t)Sk * D * gpc;
+  const uint16_t* Qp = static_cast<const uint16_t*>(Q);
+  const uint16_t* Kp = static_cast<const uint16_t*>(K);
+  const uint16_t* Vp = static_cast<const uint16_t*>(V);
+  const uint16_t* dOp = static_cast<const uint16_t*>(dO);
+  int rc = kOk;
+  for (int g0 = 0; g0 < groups && rc == kOk; g0 += gpc) {
+    const int n = std::min(gpc, groups - g0);
+    const long qo = (long)g0 * rows * D, ko = (long)g0 * Sk * D;
+    const dim3 tgrid(ceil_div(D, 64), ceil_div(Sk, 64), n);
+    hipLaunchKernelGGL(transpose16_kernel, tgrid, dim3(256), 0, s, KTb, Kp + ko, Sk, D);
+    hipLaunchKernelGGL(transpose16_kernel, tgrid, dim3(256), 0, s, VTb, Vp + ko, Sk, D);
+    rc = launch_status();
+    if (rc == kOk) rc = gemm_f32_batched<T>(Qp + qo, KTb, Sb, n, (int)rows, Sk, D, rows * D, (long)D * Sk, (long)e, s);
+    if (rc == kOk) rc = gemm_f32_batched<T>(dOp + qo, VTb, dPb, n, (int)rows, Sk, D, rows * D, (long)D * Sk, (long)e, s);
+    if (rc != kOk) break;
+    hipLaunchKernelGGL((bwd_dense_softmax_kernel<T>), dim3(ceil_div(Sk, 64), (unsigned)ceil_div((int)rows, 64), n), dim3(256), 0,
+                       s, Sb, dPb, LSE + (long)g0 * rows, Delta + (long)g0 * rows, dSb, PTb, dSTb, (int)rows, Sq, Sk, scale,
+                       causal);
+    rc = launch_status();
+    if (rc == kOk) rc = gemm_f32_batched<T>(dSb, Kp + ko, dQ + qo, n, (int)rows, D, Sk, (long)e, (long)Sk * D, rows * D, s);
+    if (rc == kOk) rc = gemm_f32_batched<T>(PTb, dOp + qo, dV + ko, n, Sk, D, (int)rows, (long)e, rows * D, (long)Sk * D, s);
+    if (rc == kOk) rc = gemm_f32_batched<T>(dSTb, Qp + qo, dK + ko, n, Sk, D, (int)rows, (long)e, rows * D, (long)Sk * D, s);
+  }
+  if (hipFreeAsync(ws, s) != hipSuccess) { (void)hipGetLastError(); rc = rc == kOk ? kDeviceFailed : rc; }
+  return rc;
+}
+
 // (dQ, dK, dV) from (dO, Q, K, V).  O and LSE may be passed in (saved by the forward
 // call); when either is null the forward kernel is run first to recompute both.
 template <class T>
@@ -352,6 +483,8 @@ int flash_bwd_dev(const void* dO, const void* Q, const void* K, const void* V, c
     if (rc == kOk) {
       if (mfma && D == 128) rc = launch_bwd<T, 128>(p, s);
       else if (mfma) rc = launch_bwd<T, 64>(p, s);
+      else if (al && D > 128 && std::isfinite(scale) && (long)(Hq / Hkv) * Sq * Sk <= (1L << 33))   // (else: 112 GiB of scratch a group)
+        rc = flash_bwd_dense_dev<T>(dO, Q, K, V, LSE, delta, dQ, dK, dV, B, Hq, Hkv, Sq, Sk, D, scale, causal, s);
       else {
         const long kvrows = (long)B * Hkv * Sk;
         hipLaunchKernelGGL((flash_bwd_generic_dq_kernel<T>), dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, s, p, D);

@@ -42,7 +42,10 @@ CASES = [
     (1, 4, 4, 513, 129, 128, False), (1, 2, 2, 1, 129, 128, True),
     (1, 3, 3, 40, 40, 48, False), (1, 2, 1, 50, 60, 32, True),      # head dims served zero-padded to 64 / 128
     (1, 2, 1, 150, 203, 80, True), (1, 4, 2, 130, 130, 96, True), (2, 2, 2, 70, 90, 16, False),
-    (1, 2, 2, 64, 64, 112, True), (1, 2, 1, 40, 70, 160, True),      # 160: above the compiled widths, per-row kernels
+    (1, 2, 2, 64, 64, 112, True),
+    # above 128: dense products around an elementwise softmax kernel, per (batch, KV head) group
+    (1, 2, 1, 40, 70, 160, True), (2, 4, 2, 200, 264, 256, True), (1, 6, 2, 130, 77, 192, False), (3, 2, 2, 65, 129, 256, True),
+    (1, 8, 8, 333, 200, 144, True), (1, 4, 1, 1, 300, 256, True),
     # B * Hkv a multiple of 8: the XCD-aware workgroup order
     (2, 8, 4, 200, 264, 128, True), (1, 16, 8, 130, 130, 64, True), (2, 24, 8, 70, 330, 128, False),
 ]
@@ -119,7 +122,7 @@ def test_backward_headline_shape_properties(lane):
     assert np.array_equal(dq2, 2 * dq) and np.array_equal(dk2, 2 * dk) and np.array_equal(dv2, 2 * dv)
 
 
-@pytest.mark.parametrize("D", [48, 80, 128])
+@pytest.mark.parametrize("D", [48, 80, 128, 256])
 def test_backward_with_saved_forward_results_equals_recompute(lane, D):
     """The device entry point fed the forward's own O and log-sum-exp gives the bits the
     recomputing host entry gives (the padded widths take the same path either way)."""
