@@ -5,6 +5,7 @@
 #include "gemm16.h"
 #include "gemm16_skinny.h"
 #include "host_util.h"
+#include "pitch_copy.h"
 
 namespace tsr950 {
 
@@ -243,69 +244,6 @@ int launch_gemm16_skinny(const Gemm16Params& p, int kps, int splits, hipStream_t
   hipLaunchKernelGGL(kern, dim3(ceil_div(p.N, 32 * NJ), splits), dim3(NW * 64), lds, s, p, kps);
   return launch_status();
 }
-
-// Copies between a matrix of any pitch and alignment and a 16-byte aligned one whose pitch is a
-// multiple of 16 bytes, for operands the vector loads of the tile kernels cannot take as they are.
-// A thread moves one 16-byte chunk: blockIdx.x / threadIdx.x run along a row, blockIdx.y /
-// threadIdx.y over rows, blockIdx.z over the batch.  The side of any alignment is accessed with one
-// 16-byte instruction where the whole chunk is inside the row (global memory takes accesses off
-// their natural alignment), element by element at the row's end.
-template <class E> struct __attribute__((packed, aligned(sizeof(E)))) LooseChunk { uint4 v; };
-constexpr int kCopyRowsPerBlock = 4;
-
-// dst[b][r][c] (rows_dst x ld_dst, 16-byte aligned) = src[b][r][c] inside rows_src x cols_src, else 0.
-template <class E>
-__global__ void __launch_bounds__(64 * kCopyRowsPerBlock)
-pad_rows_kernel(E* __restrict__ dst, long ld_dst, long stride_dst, const E* __restrict__ src, long ld_src,
-                long stride_src, int rows_src, int cols_src, int rows_dst) {
-  constexpr int V = 16 / sizeof(E);
-  const int c0 = (blockIdx.x * 64 + threadIdx.x) * V;
-  if (c0 >= ld_dst) return;
-  const long b = blockIdx.z;
-  for (int r = blockIdx.y * kCopyRowsPerBlock + threadIdx.y; r < rows_dst; r += gridDim.y * kCopyRowsPerBlock) {
-    uint4 out = make_uint4(0u, 0u, 0u, 0u);
-    if (r < rows_src && c0 < cols_src) {
-      const E* sp = src + b * stride_src + (long)r * ld_src + c0;
-      if (c0 + V <= cols_src) {
-        out = reinterpret_cast<const LooseChunk<E>*>(sp)->v;
-      } else {
-        alignas(16) E v[V];
-#pragma unroll
-        for (int u = 0; u < V; ++u) v[u] = c0 + u < cols_src ? sp[u] : E(0);
-        out = *reinterpret_cast<const uint4*>(v);
-      }
-    }
-    *reinterpret_cast<uint4*>(dst + b * stride_dst + (long)r * ld_dst + c0) = out;
-  }
-}
-// dst[b][r][c] = src[b][r][c] for r < rows, c < cols; src 16-byte aligned with pitch ld_src, dst any.
-template <class E>
-__global__ void __launch_bounds__(64 * kCopyRowsPerBlock)
-unpad_rows_kernel(E* __restrict__ dst, long ld_dst, long stride_dst, const E* __restrict__ src, long ld_src,
-                  long stride_src, int rows, int cols) {
-  constexpr int V = 16 / sizeof(E);
-  const int c0 = (blockIdx.x * 64 + threadIdx.x) * V;
-  if (c0 >= cols) return;
-  const long b = blockIdx.z;
-  for (int r = blockIdx.y * kCopyRowsPerBlock + threadIdx.y; r < rows; r += gridDim.y * kCopyRowsPerBlock) {
-    const uint4 in = *reinterpret_cast<const uint4*>(src + b * stride_src + (long)r * ld_src + c0);
-    E* dp = dst + b * stride_dst + (long)r * ld_dst + c0;
-    if (c0 + V <= cols) {
-      reinterpret_cast<LooseChunk<E>*>(dp)->v = in;
-    } else {
-      alignas(16) E v[V];
-      *reinterpret_cast<uint4*>(v) = in;
-#pragma unroll
-      for (int u = 0; u < V; ++u)
-        if (c0 + u < cols) dp[u] = v[u];
-    }
-  }
-}
-inline dim3 copy_grid(long rows, long ld, int vec, int batch) {
-  const long bx = (ld / vec + 63) / 64, by = (rows + kCopyRowsPerBlock - 1) / kCopyRowsPerBlock;
-  return dim3((unsigned)bx, (unsigned)std::max<long>(1, std::min<long>(by, 16384)), (unsigned)batch);
-}
-inline dim3 copy_block() { return dim3(64, kCopyRowsPerBlock, 1); }
 
 template <class T, int EPI>
 int launch_gemm16(Gemm16Params p, hipStream_t s);

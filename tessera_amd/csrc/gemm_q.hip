@@ -4,6 +4,7 @@
 #include "../../include/tessera_gfx950.h"
 #include "gemm8.h"
 #include "host_util.h"
+#include "pitch_copy.h"
 
 namespace tsr950 {
 namespace {
@@ -23,6 +24,75 @@ int gemm8_attr() {
 }
 
 template <class T, int EPI>
+int gemm8_dev(Gemm8Params p, hipStream_t s);
+
+// K or N not a multiple of 16, or a pointer off a 16-byte boundary: the operands concerned are
+// copied into aligned buffers with K and N rounded up to multiples of 16 (zero columns of A, zero
+// rows and columns of B: they add exact zeros), the tile kernel runs on those, and the leading N
+// columns of the results are copied out.  Stream-ordered scratch.
+template <class T, int EPI>
+int gemm8_repitched(const Gemm8Params& p, hipStream_t s) {
+  constexpr int dsz = EPI == EPI8_SCALED_BF16 ? 2 : 4;
+  const int K16 = (p.K + 15) & ~15, N16 = (p.N + 15) & ~15;
+  const bool a_ok = p.K % 16 == 0 && aligned16(p.A);
+  const bool b_ok = p.K % 16 == 0 && p.N % 16 == 0 && aligned16(p.B);
+  const bool d_ok = p.N % 16 == 0 && aligned16(p.D);
+  const bool acc_ok = !p.acc_out || (p.N % 16 == 0 && aligned16(p.acc_out));
+  const bool cs_ok = !p.col_scale || (p.N % 16 == 0 && aligned16(p.col_scale));
+  const size_t a_bytes = a_ok ? 0 : (size_t)p.M * K16, b_bytes = b_ok ? 0 : (size_t)K16 * N16;
+  const size_t d_bytes = d_ok ? 0 : (size_t)p.M * N16 * dsz, acc_bytes = acc_ok ? 0 : (size_t)p.M * N16 * 4;
+  const size_t cs_bytes = cs_ok ? 0 : (size_t)N16 * 4;
+  char* ws = nullptr;
+  if (hipMallocAsync(reinterpret_cast<void**>(&ws), a_bytes + b_bytes + d_bytes + acc_bytes + cs_bytes + 16, s) != hipSuccess) {
+    (void)hipGetLastError();
+    return kDeviceFailed;
+  }
+  Gemm8Params q = p;
+  q.K = K16;
+  q.N = N16;
+  char* at = ws;
+  if (!a_ok) {
+    hipLaunchKernelGGL(pad_rows_kernel<uint8_t>, copy_grid(p.M, K16, 16, 1), copy_block(), 0, s, reinterpret_cast<uint8_t*>(at),
+                       (long)K16, 0L, p.A, (long)p.K, 0L, p.M, p.K, p.M);
+    q.A = reinterpret_cast<const uint8_t*>(at);
+    at += a_bytes;
+  }
+  if (!b_ok) {
+    hipLaunchKernelGGL(pad_rows_kernel<uint8_t>, copy_grid(K16, N16, 16, 1), copy_block(), 0, s, reinterpret_cast<uint8_t*>(at),
+                       (long)N16, 0L, p.B, (long)p.N, 0L, p.K, p.N, K16);
+    q.B = reinterpret_cast<const uint8_t*>(at);
+    at += b_bytes;
+  }
+  void* d2 = nullptr;
+  if (!d_ok) { d2 = at; q.D = d2; at += d_bytes; }
+  int32_t* acc2 = nullptr;
+  if (!acc_ok) { acc2 = reinterpret_cast<int32_t*>(at); q.acc_out = acc2; at += acc_bytes; }
+  if (!cs_ok) {
+    hipLaunchKernelGGL(pad_rows_kernel<float>, copy_grid(1, N16, 4, 1), copy_block(), 0, s, reinterpret_cast<float*>(at),
+                       (long)N16, 0L, p.col_scale, (long)p.N, 0L, 1, p.N, 1);
+    q.col_scale = reinterpret_cast<const float*>(at);
+  }
+  int rc = launch_status();
+  if (rc == kOk) rc = gemm8_dev<T, EPI>(q, s);
+  if (rc == kOk && !d_ok) {
+    if constexpr (dsz == 4)
+      hipLaunchKernelGGL(unpad_rows_kernel<uint32_t>, copy_grid(p.M, N16, 4, 1), copy_block(), 0, s, static_cast<uint32_t*>(p.D),
+                         (long)p.N, 0L, static_cast<const uint32_t*>(d2), (long)N16, 0L, p.M, p.N);
+    else
+      hipLaunchKernelGGL(unpad_rows_kernel<uint16_t>, copy_grid(p.M, N16, 8, 1), copy_block(), 0, s, static_cast<uint16_t*>(p.D),
+                         (long)p.N, 0L, static_cast<const uint16_t*>(d2), (long)N16, 0L, p.M, p.N);
+    rc = launch_status();
+  }
+  if (rc == kOk && !acc_ok) {
+    hipLaunchKernelGGL(unpad_rows_kernel<int32_t>, copy_grid(p.M, N16, 4, 1), copy_block(), 0, s, p.acc_out, (long)p.N, 0L,
+                       static_cast<const int32_t*>(acc2), (long)N16, 0L, p.M, p.N);
+    rc = launch_status();
+  }
+  if (hipFreeAsync(ws, s) != hipSuccess) { (void)hipGetLastError(); rc = rc == kOk ? kDeviceFailed : rc; }
+  return rc;
+}
+
+template <class T, int EPI>
 int gemm8_dev(Gemm8Params p, hipStream_t s) {
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || !p.A || !p.B || !p.D) return kBadShape;
   if (EPI == EPI8_W8A8_F32 && (!p.row_scale || !p.col_scale)) return kBadShape;
@@ -31,6 +101,10 @@ int gemm8_dev(Gemm8Params p, hipStream_t s) {
   const bool vec = (p.K % 16 == 0) && (p.N % 16 == 0) && (p.K < (1 << 22)) && (p.N < (1 << 22)) && aligned16(p.A) && aligned16(p.B) && aligned16(p.D) &&
                    (!p.acc_out || aligned16(p.acc_out)) && (!p.col_scale || aligned16(p.col_scale));
   if (!vec) {
+    // small products go one thread per output element; above about 2^24 multiply-adds the copies
+    // into aligned, zero-padded buffers cost less than that kernel loses
+    if ((double)p.M * p.N * p.K >= (double)(1L << 24) && p.M >= 16 && p.N >= 16 && p.K + 16 < (1 << 22) && p.N + 16 < (1 << 22))
+      return gemm8_repitched<T, EPI>(p, s);
     dim3 block(32, 8), grid(ceil_div(p.N, 32), ceil_div(p.M, 8), 1);
     hipLaunchKernelGGL((gemm8_generic_kernel<T, EPI>), grid, block, 0, s, p);
     return launch_status();

@@ -14,7 +14,9 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("M,N,K", [(16, 16, 16), (32, 48, 64), (256, 256, 128), (300, 528, 400),
                                    (7, 13, 5), (100, 36, 1000), (512, 1024, 2048),
                                    # few tiles, long K: split along K (2, 4, 8, 16 slices; a ragged last slice)
-                                   (16, 2048, 4096), (300, 1024, 8192), (128, 512, 16384), (1, 256, 40000), (40, 528, 2304)])
+                                   (16, 2048, 4096), (300, 1024, 8192), (128, 512, 16384), (1, 256, 40000), (40, 528, 2304),
+                                   # K or N off the 16-byte grid, large: aligned zero-padded copies and the tile kernel
+                                   (517, 1003, 771), (300, 2050, 4100), (64, 5000, 1001)])
 def test_int8_gemm_bit_exact(lane, M, N, K):
     rng = np.random.default_rng(K + M)
     a = rng.integers(-127, 128, (M, K)).astype(np.int8)
@@ -51,7 +53,8 @@ def test_quantize_int8_matches_oracle(lane, M, N, K):
     assert np.array_equal(wq, owq) and np.array_equal(ws, ows)
 
 
-@pytest.mark.parametrize("M,K,N", [(320, 512, 272), (48, 4096, 2048), (200, 8192, 512)])   # the last two: K split
+@pytest.mark.parametrize("M,K,N", [(320, 512, 272), (48, 4096, 2048), (200, 8192, 512),    # the last two: K split
+                                   (333, 1001, 1030)])                                       # unaligned, large
 def test_w8a8_matmul(lane, M, K, N):
     rng = np.random.default_rng(8)
     X = rng.standard_normal((M, K)).astype(np.float32)
@@ -112,7 +115,8 @@ def test_e4m3_quantiser_matches_oracle(lane):
 
 
 @pytest.mark.parametrize("M,N,K", [(64, 64, 64), (256, 512, 1024), (130, 272, 208), (9, 21, 13),
-                                   (16, 2048, 4096), (300, 1024, 8192), (128, 512, 16400)])   # the last three: K split
+                                   (16, 2048, 4096), (300, 1024, 8192), (128, 512, 16400),    # these three: K split
+                                   (517, 1003, 771), (300, 2050, 4100)])                      # unaligned, large
 def test_fp8_gemm(lane, M, N, K):
     rng = np.random.default_rng(6)
     A = rng.standard_normal((M, K)).astype(np.float32)
