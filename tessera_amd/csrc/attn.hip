@@ -30,6 +30,35 @@ int launch_flash(const FlashParams& p, hipStream_t s) {
   if (attr_err != hipSuccess) return kDeviceFailed;
   const int qblocks = ceil_div(p.Sq, G::BQ);
   const bool xcd_grouped = (p.B * p.Hkv) % 8 == 0;
+  // Few workgroups against a long key range (a chunk of queries against a long context): the key
+  // tiles are split over gridDim.y, each split writes a normalised partial O and its log-sum-exp
+  // to the stream workspace, and the merge kernel of the decode path combines them.  About two
+  // workgroups per compute unit, at least 8 tiles (512 keys) a split.
+  const long wgs = (long)p.B * p.Hq * qblocks;
+  const int tiles = ceil_div(p.Sk, FA_BKV);
+  int nsplit = 1;
+  if (wgs < 192 && !p.bias) nsplit = (int)std::max<long>(1, std::min<long>(std::min<long>(ceil_div(512, (int)wgs), tiles / 8), 64));
+  if (nsplit > 1) {
+    FlashParams q = p;
+    q.tiles_per_split = ceil_div(tiles, nsplit);
+    q.nsplit = ceil_div(tiles, q.tiles_per_split);
+    const size_t rows = (size_t)p.B * p.Hq * p.Sq;
+    float* ws = static_cast<float*>(stream_workspace(s, (size_t)q.nsplit * rows * (p.D + 1) * sizeof(float)));
+    if (!ws) return kDeviceFailed;
+    q.O = ws;
+    q.LSE = ws + (size_t)q.nsplit * rows * p.D;
+    q.os = FlashStrides{(long)p.Hq * p.Sq * p.D, (long)p.Sq * p.D, (long)p.D};
+    q.out_storage = 0;
+    q.split_o_elems = (long)rows * p.D;
+    const dim3 grid = xcd_grouped ? dim3(8 * p.ratio, qblocks * q.nsplit, p.B * p.Hkv / 8)
+                                  : dim3(p.B * p.Hq, qblocks * q.nsplit, 1);
+    hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), G::SMEM, s, q);
+    if (int rc = launch_status(); rc != kOk) return rc;
+    const long quads = (long)rows * (p.D / 4);
+    hipLaunchKernelGGL((flash_decode_merge_kernel<T>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p,
+                       static_cast<const float*>(q.O), static_cast<const float*>(q.LSE), q.nsplit);
+    return launch_status();
+  }
   const dim3 grid = xcd_grouped ? dim3(8 * p.ratio, qblocks, p.B * p.Hkv / 8) : dim3(p.B * p.Hq, qblocks, 1);
   hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), G::SMEM, s, p);
   return launch_status();

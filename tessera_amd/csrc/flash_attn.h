@@ -65,6 +65,13 @@ struct FlashParams {
   float softcap;       // > 0: scaled scores pass through cap * tanh(s / cap); 0: none
   int ratio;           // Hq / Hkv
   const float* bias;   // additive bias [B, Hq, Sq, Sk] f32 added to the (capped) scaled scores, or null
+  // Key splits (few workgroups against a long key range): gridDim.y = query blocks x nsplit;
+  // split s of a workgroup covers the 64-key tiles [s tiles_per_split, (s + 1) tiles_per_split)
+  // of its key range and writes a normalised partial O (f32, contiguous [B, Hq, Sq, D]) and its
+  // log-sum-exp at O + s split_o_elems and LSE + s B Hq Sq; flash_decode_merge_kernel merges them.
+  int nsplit;          // 0 or 1: none
+  int tiles_per_split;
+  long split_o_elems;  // B Hq Sq D
 };
 
 // Visible keys [lo, hi] of query row i — the reference's attention_bounds
@@ -196,7 +203,9 @@ __global__ __launch_bounds__(FlashGeom<DP>::THREADS, 1) void flash_fwd_kernel(co
   // the grid is (B * Hq, query blocks, 1), heaviest blocks first.  No index needs a
   // division either way.
   // qlin / kvlin: linear (batch, head) index of the query head / of its KV head.
-  const int qb = (int)gridDim.y - 1 - (int)blockIdx.y;
+  const int nsplit = p.nsplit > 1 ? p.nsplit : 1;
+  const int split = p.nsplit > 1 ? (int)blockIdx.y % nsplit : 0;
+  const int qb = (int)gridDim.y / nsplit - 1 - (int)blockIdx.y / nsplit;
   int qlin, kvlin;
   if (gridDim.z > 1 || (int)gridDim.x == 8 * p.ratio) {
     const int w = blockIdx.x;
@@ -229,8 +238,14 @@ __global__ __launch_bounds__(FlashGeom<DP>::THREADS, 1) void flash_fwd_kernel(co
   int lo_first, hi_first, lo_last, hi_last;
   key_bounds(q0, p.Sq, p.Sk, p.causal, p.window, lo_first, hi_first);
   key_bounds(min(q0 + FA_BQ, p.Sq) - 1, p.Sq, p.Sk, p.causal, p.window, lo_last, hi_last);
-  const int tile_base = lo_first / FA_BKV;
-  const int ntiles = max((hi_last + FA_BKV) / FA_BKV - tile_base, 0);
+  int tile_base = lo_first / FA_BKV;
+  int ntiles = max((hi_last + FA_BKV) / FA_BKV - tile_base, 0);
+  if (p.nsplit > 1) {                         // this split's share of the tile range (possibly none)
+    const int lo = max(tile_base, split * p.tiles_per_split);
+    const int hi = min(tile_base + ntiles, (split + 1) * p.tiles_per_split);
+    tile_base = lo;
+    ntiles = max(hi - lo, 0);
+  }
   // Tiles this wave computes on: from (an even number of tiles before) its first
   // row's first key to its last row's last key.
   int nt_w = 0, t_w0 = 0;
@@ -576,7 +591,7 @@ __global__ __launch_bounds__(FlashGeom<DP>::THREADS, 1) void flash_fwd_kernel(co
     float l = l_run[qt] + swap_half(l_run[qt]);
     if (khi[qt] < klo[qt]) l = 0.f;                      // no visible key: O = 0, LSE = -inf
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    const long row = (long)qlin * p.Sq + qi;
+    const long row = (long)qlin * p.Sq + qi + (long)split * p.B * p.Hq * p.Sq;
     if (p.LSE && lh == 0 && dsel == 0 && qi < p.Sq)
       p.LSE[row] = l > 0.f ? (m_run[qt] * cs + __log2f(l)) * 0.69314718055994530942f : -INFINITY;
     char* stage = smem + (wave * QT + qt) * 32 * G::STAGE_PITCH;
@@ -602,7 +617,7 @@ __global__ __launch_bounds__(FlashGeom<DP>::THREADS, 1) void flash_fwd_kernel(co
     const int dcols = min(dreal - dcol0, DT * 32);
     const int per_row = dcols > 0 ? dcols * esz / 16 : 0;  // 16-byte pieces per output row
     const int rows_here = min(32, p.Sq - (qw + 32 * qt));
-    char* Ob = reinterpret_cast<char*>(p.O) + (batch * p.os.batch + hq * p.os.head) * esz;
+    char* Ob = reinterpret_cast<char*>(p.O) + (batch * p.os.batch + hq * p.os.head + split * p.split_o_elems) * esz;
     for (int idx = lane; idx < rows_here * per_row; idx += 64) {
       const int r = idx / per_row, c = idx - r * per_row;
       const uint4 v = *reinterpret_cast<const uint4*>(stage + r * G::STAGE_PITCH + c * 16);

@@ -109,6 +109,30 @@ def test_decode_kernel_reads_k_and_v_about_once(lane):
     assert kv_bytes / per_call > 1.5e12, f"{kv_bytes / per_call / 1e12:.2f} TB/s"     # the general kernel: 2.1e12 / 4 heads
 
 
+# Few workgroups against a long key range (a chunk of queries against a long context): the general
+# kernel splits the key tiles over the grid and the partials are merged.  Causal (bottom-right
+# aligned), non-causal, a window, GQA, head dims on the padded and the column-split kernels.
+SPLIT_CASES = [
+    # B, Hq, Hkv, Sq, Sk, D, causal, window
+    (1, 8, 2, 128, 8192, 128, True, 0), (1, 4, 4, 300, 5000, 64, True, 0), (1, 16, 2, 16, 4100, 128, True, 0),
+    (1, 2, 1, 257, 6000, 256, True, 0), (2, 4, 2, 64, 3000, 96, False, 0), (1, 8, 8, 200, 9000, 128, True, 2048),
+    (1, 6, 2, 40, 2049, 160, True, 0),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,window", SPLIT_CASES)
+@pytest.mark.parametrize("st", ["bf16", "f16"])
+def test_key_split_shapes_match_oracle(lane, B, Hq, Hkv, Sq, Sk, D, causal, window, st):
+    q, k, v = _qkv(B, Hq, Hkv, Sq, Sk, D, 29, st)
+    ref_o, ref_lse = orc.flash_attn_dense(_f32(q), _f32(k), _f32(v), causal=causal, window=window)
+    o, lse = ops.gqa_attention(q, k, v, causal=causal, return_lse=True, out="f32", window=window)
+    assert not np.isnan(o).any()
+    assert orc.max_rel_err(o, ref_o) <= TOL
+    assert np.max(np.abs(lse - ref_lse)) <= TOL
+    stored = ops.gqa_attention(q, k, v, causal=causal, window=window)
+    assert orc.max_rel_err(_f32(stored), ref_o) <= TOL + (2.0 ** -8 if st == "bf16" else 2.0 ** -11)
+
+
 @pytest.mark.parametrize("scale", [0.3, 1e-3, 0.0, -0.07])
 def test_attention_scales(lane, scale):
     """Any finite scale: a negative one turns the row maximum of the raw scores into
