@@ -82,10 +82,10 @@ int launch_flash_for(const FlashParams& p, bool ext, hipStream_t s) {
 // Few query rows per KV head (decode, short speculative steps): the rows of a whole GQA group
 // share one MFMA tile and the key range is split over workgroups (flash_decode.h).  Returns
 // false when the problem is not of that kind (the general kernel then serves it).
-template <class T, int DP>
+template <class T, int DP, int NQ>
 int launch_decode(const FlashParams& p, hipStream_t s) {
   using G = DecodeGeom<DP>;
-  auto kern = flash_decode_kernel<T, DP>;
+  auto kern = flash_decode_kernel<T, DP, NQ>;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [&] {
@@ -121,8 +121,15 @@ int launch_decode(const FlashParams& p, hipStream_t s) {
                      dp.part_o, dp.part_lse, nsplit);
   return launch_status();
 }
+// (up to 32 rows per KV head at D = 256, 64 at D = 128, 128 at D = 64: one, two or four query
+// tiles per wave, what the register file holds of their accumulators)
+inline int decode_row_limit(int D) { return D == 64 ? 128 : D == 128 ? 64 : D == 256 ? 32 : 0; }
 inline bool decode_shaped(const FlashParams& p) {
-  if ((long)p.ratio * p.Sq > 32 || !(p.D == 64 || p.D == 128 || p.D == 256)) return false;
+  const long rows = (long)p.ratio * p.Sq;
+  if (rows > decode_row_limit(p.D)) return false;
+  // beyond one query tile the gain is the shared read of K and V by the group's heads (measured: up to
+  // 6x with 8 heads a group, a tie or a loss with one)
+  if (rows > 32 && p.ratio == 1) return false;
   int lo0, hi0, lo1, hi1;
   key_bounds(0, p.Sq, p.Sk, p.causal, p.window, lo0, hi0);
   key_bounds(p.Sq - 1, p.Sq, p.Sk, p.causal, p.window, lo1, hi1);
@@ -179,9 +186,11 @@ int flash_dev(const void* Q, const void* K, const void* V, void* O, void* LSE, i
   // extended one scales first and serves every other scale.
   const bool ext = p.softcap > 0.f || p.bias != nullptr || !(scale > 0.f);
   if (al && !ext && decode_shaped(p)) {
-    if (p.D == 64) return launch_decode<T, 64>(p, s);
-    if (p.D == 128) return launch_decode<T, 128>(p, s);
-    return launch_decode<T, 256>(p, s);
+    const int rows = p.ratio * p.Sq;
+    if (p.D == 64) return rows <= 32 ? launch_decode<T, 64, 1>(p, s) : rows <= 64 ? launch_decode<T, 64, 2>(p, s)
+                                                                                  : launch_decode<T, 64, 4>(p, s);
+    if (p.D == 128) return rows <= 32 ? launch_decode<T, 128, 1>(p, s) : launch_decode<T, 128, 2>(p, s);
+    return launch_decode<T, 256, 1>(p, s);
   }
   if (al) return launch_flash_for<T>(p, ext, s);
   const long rows = (long)B * Hq * Sq;

@@ -4,8 +4,8 @@
 // The general kernel (flash_attn.h) gives a workgroup 256 query rows of ONE query head.  With
 // one query row per head that is one useful row in 256, one workgroup per head however long
 // the key range is, and every query head of a GQA group streams the group's K and V again.
-// Here the rows of a whole GQA group — (Hq / Hkv) heads x Sq rows, at most 32 — are the 32
-// columns of ONE MFMA tile, so K and V of a KV head are read once for the group; the key
+// Here the rows of a whole GQA group — (Hq / Hkv) heads x Sq rows, at most 32 NQ — are the
+// columns of NQ MFMA tiles that share every K / V fragment, so K and V of a KV head are read once for the group; the key
 // range of a (batch, KV head) is split over gridDim.y workgroups and, inside a workgroup, over
 // its waves (wave w takes the 32-key tiles w, w + WAVES, ...), so the read of K and V — the
 // bound of this problem — is spread over the whole chip.  Every wave runs the online softmax
@@ -36,13 +36,13 @@ struct FlashDecodeParams {
   FlashParams f;
   float* part_o;          // [nsplit][B * Hq * Sq][D] normalised partial O, or null when nsplit == 1
   float* part_lse;        // [nsplit][B * Hq * Sq] natural-log LSE of each partial
-  int rows;               // (Hq / Hkv) * Sq <= 32: the query rows of one KV head
+  int rows;               // (Hq / Hkv) * Sq <= 32 NQ: the query rows of one KV head
   int tile_lo;            // first 32-key tile any row sees
   int tile_end;           // one past the last
   int tiles_per_split;
 };
 
-template <class T, int DP>
+template <class T, int DP, int NQ>
 __global__ __launch_bounds__(DecodeGeom<DP>::THREADS) void flash_decode_kernel(const FlashDecodeParams dp) {
   using G = DecodeGeom<DP>;
   const FlashParams& p = dp.f;
@@ -62,23 +62,26 @@ __global__ __launch_bounds__(DecodeGeom<DP>::THREADS) void flash_decode_kernel(c
 
   const int kvlin = blockIdx.x, split = blockIdx.y;
   const int batch = kvlin / p.Hkv, hkv = kvlin - batch * p.Hkv;
-  // Row i of the MFMA tile: query row i % Sq of query head hkv * ratio + i / Sq.
-  const bool valid = l32 < dp.rows;
-  const int hsel = valid ? l32 / p.Sq : 0;
-  const int qi = valid ? l32 - hsel * p.Sq : 0;
-  const int hq = hkv * p.ratio + hsel;
+  // Row i of the group (tile i / 32, column i % 32): query row i % Sq of query head hkv * ratio + i / Sq.
   const uint16_t* Kb = p.K + batch * p.ks.batch + hkv * p.ks.head;
   const uint16_t* Vb = p.V + batch * p.vs.batch + hkv * p.vs.head;
 
-  uint4 qf[KSTEPS];
-  {
-    const uint16_t* src = p.Q + batch * p.qs.batch + hq * p.qs.head + (long)qi * p.qs.row + 8 * lh;
+  uint4 qf[NQ][KSTEPS];
+  int klo[NQ], khi[NQ];                                // a row past dp.rows sees no key
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) {
+    const int i = 32 * qt + l32;
+    const bool valid = i < dp.rows;
+    const int hsel = valid ? i / p.Sq : 0;
+    const int qi = valid ? i - hsel * p.Sq : 0;
+    const uint16_t* src = p.Q + batch * p.qs.batch + (hkv * p.ratio + hsel) * p.qs.head + (long)qi * p.qs.row + 8 * lh;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks)
-      qf[ks] = valid ? *reinterpret_cast<const uint4*>(src + 16 * ks) : make_uint4(0u, 0u, 0u, 0u);
+      qf[qt][ks] = valid ? *reinterpret_cast<const uint4*>(src + 16 * ks) : make_uint4(0u, 0u, 0u, 0u);
+    klo[qt] = 0;
+    khi[qt] = -1;
+    if (valid) key_bounds(qi, p.Sq, p.Sk, p.causal, p.window, klo[qt], khi[qt]);
   }
-  int klo = 0, khi = -1;                               // a row past dp.rows sees no key
-  if (valid) key_bounds(qi, p.Sq, p.Sk, p.causal, p.window, klo, khi);
   int lo0, hi0, lo1, hi1;                              // bounds of the first and the last query row
   key_bounds(0, p.Sq, p.Sk, p.causal, p.window, lo0, hi0);
   key_bounds(p.Sq - 1, p.Sq, p.Sk, p.causal, p.window, lo1, hi1);
@@ -126,12 +129,17 @@ __global__ __launch_bounds__(DecodeGeom<DP>::THREADS) void flash_decode_kernel(c
   }
 
   // ---- state ----
-  f32x16 o_acc[DT];
+  f32x16 o_acc[NQ][DT];
+  float m_run[NQ], l_run[NQ];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+  for (int qt = 0; qt < NQ; ++qt) {
+    m_run[qt] = FA_NEG;
+    l_run[qt] = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.f;
-  float m_run = FA_NEG, l_run = 0.f;
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o_acc[qt][dt][r] = 0.f;
+  }
   const float cs = p.scale * 1.44269504088896340736f;  // scale * log2(e); scale > 0 on this path
 
   const int t0 = dp.tile_lo + split * dp.tiles_per_split;
@@ -146,56 +154,63 @@ __global__ __launch_bounds__(DecodeGeom<DP>::THREADS) void flash_decode_kernel(c
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    // S^T = K . Q^T for the tile's 32 keys
-    f32x16 sc;
+    // S^T = K . Q^T for the tile's 32 keys; a K fragment serves the NQ query tiles
+    f32x16 sc[NQ];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+    for (int qt = 0; qt < NQ; ++qt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[qt][r] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       const uint4 kf = lds_read_b128(wsm, k_rd[ks] + stage * TILE);
-      sc = mfma_32x32x16<T>(kf, qf[ks], sc);
+#pragma unroll
+      for (int qt = 0; qt < NQ; ++qt) sc[qt] = mfma_32x32x16<T>(kf, qf[qt][ks], sc[qt]);
     }
     const int kv0 = t * G::BK;
-    if (kv0 + G::BK - 1 > hi0 || kv0 < lo1) {
+    const bool need_mask = kv0 + G::BK - 1 > hi0 || kv0 < lo1;
+    uint4 pf[NQ][2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-        if (key > khi || key < klo) sc[r] = FA_NEG;
+    for (int qt = 0; qt < NQ; ++qt) {
+      if (need_mask) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kv0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+          if (key > khi[qt] || key < klo[qt]) sc[qt][r] = FA_NEG;
+        }
       }
-    }
-    float mx = max3_raw(sc[0], sc[1], sc[2]);
+      float mx = max3_raw(sc[qt][0], sc[qt][1], sc[qt][2]);
 #pragma unroll
-    for (int r = 3; r < 16; r += 2) mx = (r + 1 < 16) ? max3_raw(mx, sc[r], sc[r + 1]) : fmaxf(mx, sc[r]);
-    mx = max_with_other_half(mx);
-    const float m_new = fmaxf(m_run, mx);
-    if (__any(m_new > m_run)) {
-      const float corr = fast_exp2((m_run - m_new) * cs);
-      l_run *= corr;
+      for (int r = 3; r < 16; r += 2) mx = (r + 1 < 16) ? max3_raw(mx, sc[qt][r], sc[qt][r + 1]) : fmaxf(mx, sc[qt][r]);
+      mx = max_with_other_half(mx);
+      const float m_new = fmaxf(m_run[qt], mx);
+      if (__any(m_new > m_run[qt])) {
+        const float corr = fast_exp2((m_run[qt] - m_new) * cs);
+        l_run[qt] *= corr;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o_acc[dt][r] *= corr;
-      m_run = m_new;
-    }
-    // (a row that has met no visible key keeps the sentinel: reference 0, so masked entries give P = 0)
-    const float mc = m_new > 0.5f * FA_NEG ? m_new * cs : 0.f;
-    uint4 pf[2];
-    float sum = 0.f;
-#pragma unroll
-    for (int g = 0; g < 2; ++g) {
-#pragma unroll
-      for (int r = 8 * g; r < 8 * g + 8; ++r) {
-        const float e = fast_exp2(fmaf(sc[r], cs, -mc));
-        sc[r] = e;
-        sum += e;
+          for (int r = 0; r < 16; ++r) o_acc[qt][dt][r] *= corr;
+        m_run[qt] = m_new;
       }
-      pf[g].x = pack2<T>(sc[8 * g + 0], sc[8 * g + 1]);
-      pf[g].y = pack2<T>(sc[8 * g + 2], sc[8 * g + 3]);
-      pf[g].z = pack2<T>(sc[8 * g + 4], sc[8 * g + 5]);
-      pf[g].w = pack2<T>(sc[8 * g + 6], sc[8 * g + 7]);
+      // (a row that has met no visible key keeps the sentinel: reference 0, so masked entries give P = 0)
+      const float mc = m_new > 0.5f * FA_NEG ? m_new * cs : 0.f;
+      float sum = 0.f;
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+#pragma unroll
+        for (int r = 8 * g; r < 8 * g + 8; ++r) {
+          const float e = fast_exp2(fmaf(sc[qt][r], cs, -mc));
+          sc[qt][r] = e;
+          sum += e;
+        }
+        pf[qt][g].x = pack2<T>(sc[qt][8 * g + 0], sc[qt][8 * g + 1]);
+        pf[qt][g].y = pack2<T>(sc[qt][8 * g + 2], sc[qt][8 * g + 3]);
+        pf[qt][g].z = pack2<T>(sc[qt][8 * g + 4], sc[qt][8 * g + 5]);
+        pf[qt][g].w = pack2<T>(sc[qt][8 * g + 6], sc[qt][8 * g + 7]);
+      }
+      l_run[qt] += sum;
     }
-    l_run += sum;
-    // O^T += V^T . P^T, 16 keys per step
+    // O^T += V^T . P^T, 16 keys per step; a V fragment serves the NQ query tiles
 #pragma unroll
     for (int g = 0; g < 2; ++g)
 #pragma unroll
@@ -203,76 +218,83 @@ __global__ __launch_bounds__(DecodeGeom<DP>::THREADS) void flash_decode_kernel(c
         const uint32_t a = v_rd[dt] + stage * TILE + g * 16 * ROWB;
         const uint2 lo = lds_read_tr16_b64(wsm + a);
         const uint2 hi = lds_read_tr16_b64(wsm + a + 8 * ROWB);
-        o_acc[dt] = mfma_32x32x16<T>(make_uint4(lo.x, lo.y, hi.x, hi.y), pf[g], o_acc[dt]);
+        const uint4 vf = make_uint4(lo.x, lo.y, hi.x, hi.y);
+#pragma unroll
+        for (int qt = 0; qt < NQ; ++qt) o_acc[qt][dt] = mfma_32x32x16<T>(vf, pf[qt][g], o_acc[qt][dt]);
       }
     stage ^= 1;
   }
 
-  // ---- merge the waves' partials through LDS ----
+  // ---- merge the waves' partials through LDS, one 32-row query tile at a time ----
   float* ml = reinterpret_cast<float*>(smem + G::ML_AT);     // m[WAVES][32] | l[WAVES][32] | m_tot[32] | l_tot[32]
-  __syncthreads();                                           // every wave is done with its tiles
-  const float l_wave = l_run + swap_half(l_run);
-  if (lh == 0) {
-    ml[wave * 32 + l32] = m_run;
-    ml[(G::WAVES + wave) * 32 + l32] = l_wave;
-  }
-  __syncthreads();
-  float m_tot = FA_NEG;
-#pragma unroll
-  for (int w = 0; w < G::WAVES; ++w) m_tot = fmaxf(m_tot, ml[w * 32 + l32]);
-  float l_tot = 0.f;
-#pragma unroll
-  for (int w = 0; w < G::WAVES; ++w) l_tot += ml[(G::WAVES + w) * 32 + l32] * fast_exp2((ml[w * 32 + l32] - m_tot) * cs);
-  const float mine = fast_exp2((m_run - m_tot) * cs);        // both sentinels: 1, on accumulators that are 0
-  if (wave == 0 && lh == 0) {
-    ml[2 * G::WAVES * 32 + l32] = m_tot;
-    ml[(2 * G::WAVES + 1) * 32 + l32] = l_tot;
-  }
-  {
-    char* stg = wsm;                                         // [32 rows][STAGE_PITCH], f32
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        const int d = dt * 32 + 8 * a + 4 * lh;
-        *reinterpret_cast<float4*>(stg + l32 * G::STAGE_PITCH + d * 4) =
-            make_float4(o_acc[dt][4 * a + 0] * mine, o_acc[dt][4 * a + 1] * mine, o_acc[dt][4 * a + 2] * mine,
-                        o_acc[dt][4 * a + 3] * mine);
-      }
-  }
-  __syncthreads();
-  // every thread sums four columns of one row over the waves and stores them
   const bool final_out = dp.part_o == nullptr;
   const long total_rows = (long)p.B * p.Hq * p.Sq;
-  for (int idx = tid; idx < dp.rows * (D / 4); idx += G::THREADS) {
-    const int i = idx / (D / 4), d = (idx - i * (D / 4)) * 4;
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-    for (int w = 0; w < G::WAVES; ++w) {
-      const float4 v = *reinterpret_cast<const float4*>(smem + w * G::WAVE_LDS + i * G::STAGE_PITCH + d * 4);
-      acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+  for (int qt = 0; qt < NQ; ++qt) {
+    __syncthreads();                                         // every wave is done with its tiles / the last pass
+    const float l_wave = l_run[qt] + swap_half(l_run[qt]);
+    if (lh == 0) {
+      ml[wave * 32 + l32] = m_run[qt];
+      ml[(G::WAVES + wave) * 32 + l32] = l_wave;
     }
-    const float mt = ml[2 * G::WAVES * 32 + i], lt = ml[(2 * G::WAVES + 1) * 32 + i];
-    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-    acc.x *= inv; acc.y *= inv; acc.z *= inv; acc.w *= inv;
-    const int hs = i / p.Sq, q = i - hs * p.Sq;
-    const int hq_i = hkv * p.ratio + hs;
-    const long rowlin = ((long)batch * p.Hq + hq_i) * p.Sq + q;
-    const float lse = lt > 0.f ? (mt * cs + __log2f(lt)) * 0.69314718055994530942f : -INFINITY;
-    if (final_out) {
-      const long o_at = batch * p.os.batch + hq_i * p.os.head + (long)q * p.os.row + d;
-      if (p.out_storage) {
-        uint2 pk;
-        pk.x = pack2<T>(acc.x, acc.y);
-        pk.y = pack2<T>(acc.z, acc.w);
-        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.O) + o_at) = pk;
-      } else {
-        *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.O) + o_at) = acc;
+    __syncthreads();
+    float m_tot = FA_NEG;
+#pragma unroll
+    for (int w = 0; w < G::WAVES; ++w) m_tot = fmaxf(m_tot, ml[w * 32 + l32]);
+    float l_tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < G::WAVES; ++w) l_tot += ml[(G::WAVES + w) * 32 + l32] * fast_exp2((ml[w * 32 + l32] - m_tot) * cs);
+    const float mine = fast_exp2((m_run[qt] - m_tot) * cs);  // both sentinels: 1, on accumulators that are 0
+    if (wave == 0 && lh == 0) {
+      ml[2 * G::WAVES * 32 + l32] = m_tot;
+      ml[(2 * G::WAVES + 1) * 32 + l32] = l_tot;
+    }
+    {
+      char* stg = wsm;                                       // [32 rows][STAGE_PITCH], f32
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          const int d = dt * 32 + 8 * a + 4 * lh;
+          *reinterpret_cast<float4*>(stg + l32 * G::STAGE_PITCH + d * 4) =
+              make_float4(o_acc[qt][dt][4 * a + 0] * mine, o_acc[qt][dt][4 * a + 1] * mine, o_acc[qt][dt][4 * a + 2] * mine,
+                          o_acc[qt][dt][4 * a + 3] * mine);
+        }
+    }
+    __syncthreads();
+    // every thread sums four columns of one row over the waves and stores them
+    const int rows_here = min(32, dp.rows - 32 * qt);
+    for (int idx = tid; idx < rows_here * (D / 4); idx += G::THREADS) {
+      const int il = idx / (D / 4), d = (idx - il * (D / 4)) * 4;
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int w = 0; w < G::WAVES; ++w) {
+        const float4 v = *reinterpret_cast<const float4*>(smem + w * G::WAVE_LDS + il * G::STAGE_PITCH + d * 4);
+        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
       }
-      if (p.LSE && d == 0) p.LSE[rowlin] = lse;
-    } else {
-      *reinterpret_cast<float4*>(dp.part_o + ((long)split * total_rows + rowlin) * D + d) = acc;
-      if (d == 0) dp.part_lse[(long)split * total_rows + rowlin] = lse;
+      const float mt = ml[2 * G::WAVES * 32 + il], lt = ml[(2 * G::WAVES + 1) * 32 + il];
+      const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+      acc.x *= inv; acc.y *= inv; acc.z *= inv; acc.w *= inv;
+      const int i = 32 * qt + il;
+      const int hs = i / p.Sq, q = i - hs * p.Sq;
+      const int hq_i = hkv * p.ratio + hs;
+      const long rowlin = ((long)batch * p.Hq + hq_i) * p.Sq + q;
+      const float lse = lt > 0.f ? (mt * cs + __log2f(lt)) * 0.69314718055994530942f : -INFINITY;
+      if (final_out) {
+        const long o_at = batch * p.os.batch + hq_i * p.os.head + (long)q * p.os.row + d;
+        if (p.out_storage) {
+          uint2 pk;
+          pk.x = pack2<T>(acc.x, acc.y);
+          pk.y = pack2<T>(acc.z, acc.w);
+          *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.O) + o_at) = pk;
+        } else {
+          *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.O) + o_at) = acc;
+        }
+        if (p.LSE && d == 0) p.LSE[rowlin] = lse;
+      } else {
+        *reinterpret_cast<float4*>(dp.part_o + ((long)split * total_rows + rowlin) * D + d) = acc;
+        if (d == 0) dp.part_lse[(long)split * total_rows + rowlin] = lse;
+      }
     }
   }
 }

@@ -57,7 +57,7 @@ def test_attention_matches_oracle(lane, B, Hq, Hkv, Sq, Sk, D, causal, st):
     assert np.max(np.abs(lse - ref_lse)) <= TOL
 
 
-# Few query rows per KV head — (Hq / Hkv) * Sq <= 32 with D in {64, 128, 256} — take the decode
+# Few query rows per KV head — (Hq / Hkv) * Sq <= 32 at D = 256, 64 at 128, 128 at 64 — take the decode
 # kernel: the rows of a GQA group share one MFMA tile, the key range is split over workgroups
 # and waves, partials are merged.  One and many key splits, ratio 1 to 16, rows that fill the
 # tile and that do not, ragged last tile, causal steps of several rows, a sliding window.
@@ -67,6 +67,9 @@ DECODE_CASES = [
     (2, 8, 1, 4, 1000, 128, True, 0), (1, 4, 4, 7, 129, 256, True, 0), (2, 6, 2, 3, 64, 64, True, 0),
     (1, 16, 1, 2, 4100, 128, True, 0), (1, 8, 2, 1, 5000, 128, True, 1024), (1, 2, 2, 16, 31, 128, False, 0),
     (40, 8, 2, 1, 2048, 128, False, 0), (1, 8, 8, 1, 33000, 64, False, 0), (2, 4, 1, 8, 20, 256, True, 0),
+    # two and four query tiles per wave: up to 64 rows per KV head at D = 128, 128 at D = 64
+    (1, 64, 8, 5, 3000, 128, True, 0), (2, 16, 2, 8, 777, 128, True, 0), (1, 8, 1, 7, 2100, 128, False, 0),
+    (1, 16, 1, 8, 1500, 64, True, 0), (2, 12, 4, 33, 500, 64, True, 0), (1, 4, 2, 20, 4097, 64, False, 0),
 ]
 
 
