@@ -319,7 +319,7 @@ int tessera_gfx950_gemm_schedule(int M, int N, int K, int batch, int elem_bytes,
   if (bad_dims(batch, M, N, K) || !tile_m || !tile_n || !tile_k || !split_k) return kBadShape;
   if (elem_bytes == 2) {
     const Gemm16Schedule sch = select_gemm16_schedule(M, N, K, batch);
-    *tile_m = sch.skinny ? 32 : sch.tile;
+    *tile_m = sch.skinny ? 32 : sch.tile_m ? sch.tile_m : sch.tile;
     *tile_n = sch.tile;
     *tile_k = sch.skinny ? 32 : G16_BK;
     *split_k = sch.split_k;

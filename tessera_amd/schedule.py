@@ -25,7 +25,7 @@ _DTYPES = {
 }
 _INSTRUCTION_TILE = {"f16": (32, 32, 16), "bf16": (32, 32, 16), "int8": (32, 32, 32), "fp8_e4m3": (32, 32, 64)}
 # accumulators + operand fragments + staging of one wave, from the assembler's report
-_VGPRS = {256: 508, 128: 170, 64: 96, 32: 137}
+_VGPRS = {(256, 256): 508, (128, 256): 360, (128, 128): 170, (64, 64): 96, (32, 64): 137}
 
 
 @dataclass(frozen=True)
@@ -94,8 +94,8 @@ def select_gfx950_gemm_schedule(m: int, n: int, k: int, *, dtype: str = "bf16", 
         _lane.check(_lane.load().tessera_gfx950_gemm_rest_split(
             int(m), int(n), int(k), int(batch), ctypes.byref(rest_tiles), ctypes.byref(rest_split)), "gemm_rest_split")
     inst = _INSTRUCTION_TILE[name]
-    if name in ("f16", "bf16") and tm.value == 256:
-        inst = (16, 16, 32)       # the 256 x 256 tiles run v_mfma_f32_16x16x32 (less power per FLOP)
+    if name in ("f16", "bf16") and max(tm.value, tn.value) == 256:
+        inst = (16, 16, 32)       # the 256-wide tiles run v_mfma_f32_16x16x32 (less power per FLOP)
     return Gfx950ScheduleDescriptor(
         arch="gfx950", dtype=name, instruction_tile=inst,
         macro_tile=(tm.value // inst[0], tn.value // inst[1]),
@@ -103,7 +103,7 @@ def select_gfx950_gemm_schedule(m: int, n: int, k: int, *, dtype: str = "bf16", 
         waves_per_cu=8 if tm.value == 32 else 4, pipeline_stages=2,
         lds_layout=("A from global in operand order; B wave-private [k][n] slices + transposing ds_read"
                     if tm.value == 32 else "A xor-swizzled 16B chunks; B natural [k][n] + transposing ds_read"),
-        ownership="wave", vgpr_estimate=_VGPRS[tm.value], split_k=sk.value,
+        ownership="wave", vgpr_estimate=_VGPRS.get((tm.value, tn.value), 508), split_k=sk.value,
         source="tessera_gfx950_gemm_schedule (the launcher's own decision)",
         rest_tiles=rest_tiles.value, rest_split_k=rest_split.value)
 

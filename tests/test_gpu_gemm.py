@@ -87,12 +87,15 @@ def test_big_tile_k_and_edge_shapes(lane, M, N, K):
 # Products the launcher splits along K on the 256 x 256 tile (few tiles, long K), with the sum
 # over the splits by a second kernel, and ones it serves with 128 x 128 tiles unsplit.
 @pytest.mark.parametrize("M,N,K,tile,split", [
-    (1024, 8192, 8192, 256, 2), (8192, 1024, 8192, 256, 2), (900, 7992, 8192, 256, 2),
-    (2048, 2048, 2048, 128, 1), (2560, 2560, 2560, 128, 1), (1024, 1024, 8192, 128, 4)])
+    (512, 8192, 16384, (256, 256), 4), (8192, 512, 16384, (256, 256), 4), (500, 7992, 16384, (256, 256), 4),
+    (2048, 2048, 2048, (128, 128), 1), (1024, 1024, 8192, (128, 128), 4),
+    # 128 x 256 tiles: twice the tiles of the square form when that is what fills the chip
+    (2560, 2560, 2560, (128, 256), 1), (2048, 4096, 4096, (128, 256), 1), (1000, 8000, 4104, (128, 256), 1),
+    (1280, 5120, 2000, (128, 256), 1)])
 def test_mid_size_schedules(lane, M, N, K, tile, split):
     from tessera_amd.schedule import select_gfx950_gemm_schedule
     sch = select_gfx950_gemm_schedule(M, N, K, dtype="bf16")
-    assert sch.workgroup_tile[:2] == (tile, tile) and sch.split_k == split
+    assert sch.workgroup_tile[:2] == tile and sch.split_k == split
     rng = np.random.default_rng(M + N + K)
     a = b16.from_float32((rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32))
     b = b16.from_float32(rng.standard_normal((K, N)).astype(np.float32))
