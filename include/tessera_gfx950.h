@@ -270,6 +270,17 @@ int tessera_gfx950_quantize_e4m3_f32(const float* x, int64_t n, float scale, voi
 /* _quantize_int8_per_channel (python/tessera/compiler/smoothquant.py:79-84):
  * axis=1 -> one scale per row (scales[M]); axis=0 -> one per column (scales[N]). */
 int tessera_gfx950_quantize_i8_f32(const float* x, int M, int N, int axis, void* q, float* scales);
+/* ops.quantize_nvfp4 followed by ops.dequantize_nvfp4 (python/tessera/__init__.py:3472-3504, i.e.
+ * compiler/microscaling.py:317-384 with the nvfp4 format): x f32 [rows, cols] rounded onto the
+ * NVFP4 grid in blocks of 16 along the last axis — block scale = max(amax / 6, 1e-30) rounded to
+ * e4m3fn, codes on the E2M1 grid {0, .5, 1, 1.5, 2, 3, 4, 6}, nearest even.  dq (f32) and / or
+ * dq_bf16 (the same values as bf16 bit patterns, exact) receive the dequantised values, scales
+ * (optional) the block scales, [rows, ceil(cols / 16)].  This is what the reference's
+ * grouped_gemm(quant="nvfp4") applies to x and to each expert's weight before its f32 product
+ * (compiler/grouped_layout.py:353-392). */
+int tessera_gfx950_fake_quantize_nvfp4_f32(const float* x, int rows, int cols, float* dq, void* dq_bf16, float* scales);
+int tessera_gfx950_fake_quantize_nvfp4_f32_dev(const float* x, int rows, int cols, float* dq, void* dq_bf16,
+                                               float* scales, void* stream);
 int tessera_gfx950_quantize_e4m3_f32_dev(const float* x, int64_t n, float scale, void* codes, float* scale_out_dev, void* stream);
 int tessera_gfx950_quantize_i8_f32_dev(const float* x, int M, int N, int axis, void* q, float* scales, void* stream);
 

@@ -706,6 +706,49 @@ def quantize_fp8_e4m3(x: np.ndarray, scale: float | None = None):
     return e4m3_encode(grid), grid, np.float32(scale)
 
 
+def quantize_nvfp4(x: np.ndarray, block_size: int = 16):
+    """``ops.quantize_nvfp4`` (``__init__.py:3472-3500``), i.e. ``microscaling.quantize`` with
+    the ``nvfp4`` format followed by ``dequantize`` (``compiler/microscaling.py:317-384``):
+    blocks of ``block_size`` along the last axis (zero-padded to a whole block);
+    ``raw = max(amax / 6, 1e-30)``; the block scale is ``raw`` cast to e4m3fn (round to
+    nearest even; a scale that rounds to zero is replaced by 1); codes are
+    ``block / scale`` cast to the E2M1 grid {0, .5, 1, 1.5, 2, 3, 4, 6} (round to nearest
+    even, saturating); the dequantised value is ``code * scale`` in f32.  Returns
+    ``(dequantised f32, scales f32)`` with ``scales.shape == x.shape[:-1] + (blocks,)``.
+    (The reference's casts go through ``ml_dtypes``; a raw scale above 448, which that
+    cast turns into NaN, saturates here.)"""
+    x = np.asarray(x, np.float32)
+    n = x.shape[-1]
+    nb = -(-n // block_size)
+    xp = np.zeros(x.shape[:-1] + (nb * block_size,), np.float32)
+    xp[..., :n] = x
+    blocks = xp.reshape(x.shape[:-1] + (nb, block_size))
+    amax = np.abs(blocks).max(axis=-1)
+    raw = np.maximum(amax / np.float32(6.0), np.float32(1e-30)).astype(np.float32)
+    scale = fpquant_grid(raw)                                   # e4m3fn grid, RNE, gradual underflow
+    sf = np.where(scale == 0.0, np.float32(1.0), scale).astype(np.float32)[..., None]
+    codes = fpquant_grid((blocks / sf).astype(np.float32), max_normal=6.0, mantissa_bits=1, min_exp=0)
+    dq = (codes * sf).astype(np.float32).reshape(x.shape[:-1] + (nb * block_size,))[..., :n]
+    return np.ascontiguousarray(dq), scale.astype(np.float32)
+
+
+def grouped_gemm_nvfp4(x, w, group_sizes):
+    """``ops.grouped_gemm(..., quant="nvfp4")`` (``__init__.py:340-351``,
+    ``compiler/grouped_layout.py:353-392``): x ``(T, K)`` and every expert's weight
+    ``(K, N)`` are rounded onto the NVFP4 grid along their last axis, then the grouped
+    product runs on the dequantised values (f64 here).  Returns ``(T, N)`` f64."""
+    xq, _ = quantize_nvfp4(np.asarray(x, np.float32))
+    w = np.asarray(w, np.float32)
+    wq = np.stack([quantize_nvfp4(w[e])[0] for e in range(w.shape[0])])
+    out = np.zeros((xq.shape[0], w.shape[2]), np.float64)
+    off = 0
+    for e, n in enumerate(np.asarray(group_sizes).astype(np.int64)):
+        if n:
+            out[off:off + n] = xq[off:off + n].astype(np.float64) @ wq[e].astype(np.float64)
+        off += int(n)
+    return out
+
+
 def gemm_e4m3(a_codes, b_codes, scale_a, scale_b, out_dtype: str = "bf16"):
     """fp8 GEMM config: ``f32acc(Aq.Bq) * sA * sB`` stored in ``out_dtype``
     (f64 accumulate here).  Returns the f64 value before the final store; the

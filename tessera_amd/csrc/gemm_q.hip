@@ -426,6 +426,67 @@ int quantize_i8_dev(const float* x, int M, int N, int axis, void* q, float* scal
   return launch_status();
 }
 
+// ---- NVFP4 (block-scaled E2M1) rounding -------------------------------------------------------
+// ops.quantize_nvfp4 followed by dequantize_nvfp4 (python/tessera/__init__.py:3472-3504;
+// compiler/microscaling.py:317-384): blocks of 16 along the last axis (a short last block counts
+// its missing elements as zeros); raw = max(amax / 6, 1e-30); block scale = raw rounded to e4m3fn
+// (a scale that rounds to zero becomes 1); code = x / scale rounded to the E2M1 grid
+// {0, .5, 1, 1.5, 2, 3, 4, 6} (nearest even, saturating); value = code * scale.  A value has at
+// most 2 + 4 significant bits, so its bf16 form is exact.  One thread per block.
+__device__ __forceinline__ float e2m1_round(float v) {
+  const float a = fminf(fabsf(v), 6.0f);
+  const float ulp = a < 2.0f ? 0.5f : (a < 4.0f ? 1.0f : 2.0f);
+  const float r = fminf(__builtin_rintf(__fdiv_rn(a, ulp)) * ulp, 6.0f);
+  return copysignf(r, v);
+}
+
+__global__ __launch_bounds__(256) void fake_quantize_nvfp4_kernel(const float* __restrict__ x, int rows, int cols,
+                                                                  float* __restrict__ dq, uint16_t* __restrict__ dq16,
+                                                                  float* __restrict__ scales) {
+  const int nb = (cols + 15) / 16;
+  const long id = (long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (long)rows * nb) return;
+  const long r = id / nb;
+  const int b = (int)(id - r * nb);
+  const int c0 = b * 16, n = min(16, cols - c0);
+  const float* src = x + r * cols + c0;
+  float v[16];
+  if (n == 16 && ((reinterpret_cast<uintptr_t>(src) & 15) == 0)) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 t = reinterpret_cast<const float4*>(src)[q];
+      v[4 * q] = t.x; v[4 * q + 1] = t.y; v[4 * q + 2] = t.z; v[4 * q + 3] = t.w;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = i < n ? src[i] : 0.f;
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
+  const float raw = fmaxf(__fdiv_rn(amax, 6.0f), 1e-30f);
+  const float scale = e4m3_to_f32(f32_to_e4m3(fminf(raw, 448.0f)));
+  const float sf = scale == 0.f ? 1.0f : scale;
+  if (scales) scales[id] = scale;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    if (i < n) {
+      const float o = e2m1_round(__fdiv_rn(v[i], sf)) * sf;
+      if (dq) dq[r * cols + c0 + i] = o;
+      if (dq16) dq16[r * cols + c0 + i] = (uint16_t)(__builtin_bit_cast(uint32_t, o) >> 16);
+    }
+  }
+}
+
+int fake_quantize_nvfp4_dev(const float* x, int rows, int cols, float* dq, void* dq16, float* scales, hipStream_t s) {
+  if (rows <= 0 || cols <= 0 || !x || (!dq && !dq16)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const long blocks = (long)rows * ((cols + 15) / 16);
+  hipLaunchKernelGGL(fake_quantize_nvfp4_kernel, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0, s, x, rows, cols, dq,
+                     static_cast<uint16_t*>(dq16), scales);
+  return launch_status();
+}
+
 Gemm8Params make_params(const void* A, const void* B, void* D, int M, int N, int K) {
   Gemm8Params p{};
   p.A = static_cast<const uint8_t*>(A);
@@ -517,6 +578,30 @@ int tessera_gfx950_quantize_e4m3_f32_dev(const float* x, int64_t n, float scale,
 int tessera_gfx950_quantize_i8_f32_dev(const float* x, int M, int N, int axis, void* q, float* scales,
                                        void* stream) {
   return quantize_i8_dev(x, M, N, axis, q, scales, as_stream(stream));
+}
+
+int tessera_gfx950_fake_quantize_nvfp4_f32_dev(const float* x, int rows, int cols, float* dq, void* dq_bf16,
+                                               float* scales, void* stream) {
+  return fake_quantize_nvfp4_dev(x, rows, cols, dq, dq_bf16, scales, as_stream(stream));
+}
+
+int tessera_gfx950_fake_quantize_nvfp4_f32(const float* x, int rows, int cols, float* dq, void* dq_bf16, float* scales) {
+  if (rows <= 0 || cols <= 0 || !x || (!dq && !dq_bf16)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t n = (size_t)rows * cols, ns = (size_t)rows * ((cols + 15) / 16);
+  DeviceScope scope;
+  float* dx = static_cast<float*>(scope.alloc(n * 4, x));
+  float* dd = dq ? static_cast<float*>(scope.alloc(n * 4)) : nullptr;
+  void* d16 = dq_bf16 ? scope.alloc(n * 2) : nullptr;
+  float* ds = scales ? static_cast<float*>(scope.alloc(ns * 4)) : nullptr;
+  if (scope.failed()) return kDeviceFailed;
+  int rc = fake_quantize_nvfp4_dev(dx, rows, cols, dd, d16, ds, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  if (dq && !scope.download(dq, dd, n * 4)) return kDeviceFailed;
+  if (dq_bf16 && !scope.download(dq_bf16, d16, n * 2)) return kDeviceFailed;
+  if (scales && !scope.download(scales, ds, ns * 4)) return kDeviceFailed;
+  return kOk;
 }
 
 int tessera_gfx950_quantize_e4m3_f32(const float* x, int64_t n, float scale, void* codes, float* scale_out) {

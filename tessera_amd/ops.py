@@ -359,6 +359,8 @@ def grouped_gemm(x, weights, group_sizes, *, kind: str = "contiguous", alignment
     xa, w = _bits(x), _bits(weights)
     gs = np.asarray(group_sizes).astype(np.int64).reshape(-1)
     if quant is not None:
+        if str(quant).lower() == "nvfp4":
+            return _grouped_gemm_nvfp4(x, weights, xa, w, gs, alignment, out)
         return _grouped_gemm_fp8(x, weights, xa, w, gs, quant, alignment, out)
     if alignment is not None:
         al = int(alignment)
@@ -381,6 +383,73 @@ def grouped_gemm(x, weights, group_sizes, *, kind: str = "contiguous", alignment
     return y if f32 else y.view(BF16Array)
 
 
+def _nvfp4_round(x32: np.ndarray, want_scales: bool = False):
+    """x f32 (..., n) rounded onto the NVFP4 grid on the device → (dequantised f32,
+    dequantised bf16 bits, scales or None)."""
+    x32 = np.ascontiguousarray(x32, np.float32)
+    n = x32.shape[-1]
+    rows = int(x32.size // n) if n else 0
+    if rows <= 0 or n <= 0:
+        raise ValueError("quantize_nvfp4 needs a non-empty array")
+    dq = np.empty(x32.shape, np.float32)
+    dq16 = np.empty(x32.shape, np.uint16)
+    scales = np.empty(x32.shape[:-1] + (-(-n // 16),), np.float32) if want_scales else None
+    _lane.check(_lane.load().tessera_gfx950_fake_quantize_nvfp4_f32(
+        x32.ctypes.data, rows, n, dq.ctypes.data, dq16.ctypes.data, scales.ctypes.data if want_scales else None),
+        "quantize_nvfp4")
+    return dq, dq16, scales
+
+
+def quantize_nvfp4(x, *, block_size: int = 16):
+    """NVFP4 — block-scaled E2M1 with one e4m3 scale per 16 elements of the last axis
+    (``__init__.py:3472-3500``).  Returns ``(x_q_as_fp32, scales)`` like the reference:
+    the values already dequantised, and the block scales as f32."""
+    if int(block_size) != 16:
+        raise NotImplementedError("the gfx950 lane rounds to NVFP4 in blocks of 16 (the format's block size)")
+    x = _unbox(x)
+    x32 = x.to_float32() if isinstance(x, BF16Array) else np.asarray(x, np.float32)
+    if x32.shape[-1] % 16 != 0:
+        raise ValueError(f"last dim {x32.shape[-1]} must be divisible by block_size 16 for NVFP4")
+    dq, _, scales = _nvfp4_round(x32, want_scales=True)
+    return dq, scales
+
+
+def dequantize_nvfp4(x_q, scales=None, *, block_size: int = 16):
+    """Inverse of :func:`quantize_nvfp4`, which already returns dequantised values
+    (``__init__.py:3502-3504``)."""
+    return np.asarray(x_q, np.float32)
+
+
+def _grouped_gemm_nvfp4(x, weights, xa, w, gs, alignment, out):
+    """``quant="nvfp4"``: x and every expert's weight are rounded onto the NVFP4 grid along
+    their last axis (``compiler/grouped_layout.py:353-392``) on the device, and the grouped
+    product runs on the rounded values — which are exact in bf16 (at most six significant
+    bits), so the bf16 MFMA kernel with f32 accumulation computes the reference's f32
+    product of the dequantised operands up to summation order."""
+    if alignment is not None:
+        al = int(alignment)
+        if al <= 0 or np.any(gs % al != 0):
+            raise ValueError(f"grouped_gemm: every group size must be a multiple of alignment={alignment}")
+    if xa.ndim != 2 or w.ndim != 3 or w.shape[0] != gs.shape[0] or w.shape[1] != xa.shape[1]:
+        raise ValueError(f"grouped_gemm: x {xa.shape} / weights {w.shape} / group_sizes {gs.shape} disagree")
+    T, K = xa.shape
+    E, _, N = w.shape
+    for n_last in (K, N):                              # x is blocked along K, a weight along N
+        if n_last % 16 != 0:
+            raise ValueError(f"last dim {n_last} must be divisible by block_size 16 for NVFP4")
+    off = _offsets(gs, T, "grouped_gemm")
+    xf = x.to_float32() if isinstance(x, BF16Array) else _bf16.from_bits(xa).to_float32()
+    wf = weights.to_float32() if isinstance(weights, BF16Array) else _bf16.from_bits(w).to_float32()
+    _, xq16, _ = _nvfp4_round(xf)
+    _, wq16, _ = _nvfp4_round(wf)                      # (E, K, N): blocks run along N, per expert row
+    f32 = out == "f32"
+    y = np.zeros((T, N), np.float32 if f32 else np.uint16)
+    name = "tessera_gfx950_grouped_gemm_bf16" + ("_f32" if f32 else "")
+    _lane.check(getattr(_lane.load(), name)(xq16.ctypes.data, wq16.ctypes.data, off.ctypes.data, y.ctypes.data, T, K, N, E),
+                "grouped_gemm")
+    return y if f32 else y.view(BF16Array)
+
+
 #: quant schemes of the reference's grouped GEMM that map onto the lane's e4m3 operand format
 _FP8_GROUPED_QUANT = ("fp8_e4m3", "fp8")
 
@@ -395,7 +464,7 @@ def _grouped_gemm_fp8(x, weights, xa, w, gs, quant, alignment, out):
     if q not in _FP8_GROUPED_QUANT:
         raise NotImplementedError(
             f"grouped_gemm: quant={quant!r} is not implemented on the gfx950 lane — supported: "
-            f"{', '.join(_FP8_GROUPED_QUANT)}")
+            f"{', '.join(_FP8_GROUPED_QUANT)}, nvfp4")
     if alignment is not None:
         al = int(alignment)
         if al <= 0 or np.any(gs % al != 0):

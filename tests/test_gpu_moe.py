@@ -288,7 +288,7 @@ def test_grouped_gemm_fp8_quant(lane):
     stored = ops.grouped_gemm(x, w, sizes, quant="fp8")
     assert np.array_equal(np.asarray(stored, np.uint16), np.asarray(b16.from_float32(got), np.uint16))
     with pytest.raises(NotImplementedError):
-        ops.grouped_gemm(x, w, sizes, quant="nvfp4")
+        ops.grouped_gemm(x, w, sizes, quant="fp8_e5m2")          # the lane's fp8 operand format is e4m3
 
 
 def test_single_expert_reduces_to_dense_swiglu(lane):

@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 import tessera_oracle as orc
+from tessera_amd import bf16 as b16
 from tessera_amd import ops
 
 pytestmark = pytest.mark.gpu
@@ -187,3 +188,59 @@ def test_config5_chain_at_full_size_on_normal_data(lane):
     assert orc.max_rel_err(got, X[rows].astype(np.float64) @ W.astype(np.float64)) <= 5e-2
     stored = ops.gemm_fp8(xc, wc, sx, sw, out="bf16")[rows]
     assert np.array_equal(stored.to_float32(), orc.round_to_storage(got, "bf16"))
+
+
+def test_nvfp4_rounding_matches_oracle_bit_for_bit(lane):
+    """Device NVFP4 rounding (block scale in e4m3, E2M1 codes) against the oracle: dequantised
+    values and scales bit for bit, on data spanning 12 orders of magnitude, exact ties, zero
+    blocks, a short last block and an unaligned row length."""
+    from tessera_amd import lane as ln
+    lib = ln.load()
+    rng = np.random.default_rng(41)
+    cases = [(rng.standard_normal((300, 256)) * np.exp(rng.standard_normal((300, 1)) * 6)).astype(np.float32),
+             np.tile(np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0, -0.25, -0.75, -1.25, -1.75, -2.5, -3.5, -5.0, -6.0],
+                              np.float32), (4, 3)),
+             np.zeros((3, 48), np.float32),
+             rng.standard_normal((7, 40)).astype(np.float32),             # 2.5 blocks a row
+             rng.standard_normal((5, 19)).astype(np.float32) * 1e-8]       # scales in the e4m3 subnormals / zero
+    for x in cases:
+        rows, cols = x.shape
+        dq = np.empty_like(x)
+        dq16 = np.empty(x.shape, np.uint16)
+        sc = np.empty((rows, -(-cols // 16)), np.float32)
+        ln.check(lib.tessera_gfx950_fake_quantize_nvfp4_f32(x.ctypes.data, rows, cols, dq.ctypes.data, dq16.ctypes.data,
+                                                            sc.ctypes.data), "nvfp4")
+        odq, osc = orc.quantize_nvfp4(x)
+        assert np.array_equal(dq.view(np.uint32), odq.view(np.uint32))
+        assert np.array_equal(sc.view(np.uint32), osc.view(np.uint32))
+        assert np.array_equal((dq16.astype(np.uint32) << 16).view(np.float32), odq)     # the bf16 form is exact
+    dq, scales = ops.quantize_nvfp4(cases[0])
+    assert np.array_equal(dq, orc.quantize_nvfp4(cases[0])[0]) and scales.shape == (300, 16)
+    with pytest.raises(ValueError):
+        ops.quantize_nvfp4(cases[3])                                        # 40 % 16 != 0, as the reference
+
+
+@pytest.mark.parametrize("gs", [[5, 3, 4], [16, 16, 32], [300, 0, 77, 1000]])
+def test_grouped_gemm_nvfp4(lane, gs):
+    """quant="nvfp4": the product of the NVFP4-rounded operands (the reference rounds on the host
+    and multiplies in f32).  Against the oracle's f64 product of the same rounded operands, and
+    inside the reference's own 20 % budget against the unquantised product."""
+    rng = np.random.default_rng(sum(gs))
+    small = sum(gs) < 100
+    T, K, N, E = sum(gs), (64 if small else 512), (16 if small else 256), len(gs)
+    x = b16.from_float32(rng.standard_normal((T, K)).astype(np.float32))
+    w = b16.from_float32(rng.standard_normal((E, K, N)).astype(np.float32))
+    ref = orc.grouped_gemm_nvfp4(x.to_float32(), w.to_float32(), gs)
+    got = ops.grouped_gemm(x, w, gs, quant="nvfp4", out="f32")
+    assert got.shape == (T, N) and orc.max_rel_err(got, ref) <= 1e-5
+    stored = ops.grouped_gemm(x, w, gs, quant="nvfp4")
+    assert np.array_equal(stored.to_float32(), orc.round_to_storage(got, "bf16"))
+    full = np.zeros((T, N))
+    off = 0
+    for e, n in enumerate(gs):
+        full[off:off + n] = x.to_float32()[off:off + n].astype(np.float64) @ w.to_float32()[e].astype(np.float64)
+        off += n
+    assert np.linalg.norm(got - full) / np.linalg.norm(full) < 0.20
+    with pytest.raises(ValueError):
+        ops.grouped_gemm(b16.from_float32(np.zeros((T, 24), np.float32)),        # K = 24 is not whole blocks
+                         b16.from_float32(np.zeros((E, 24, N), np.float32)), gs, quant="nvfp4")

@@ -247,6 +247,62 @@ def test_quantize_fp8_scale_and_saturation():
     assert list(c) == [0x7E, 0xFE]                                     # tests/unit/test_phase_e_f.py:498-511
 
 
+def test_nvfp4_grid_scales_and_error_bound():
+    """The NVFP4 rounding (block-scaled E2M1) pinned by the format itself and by the bound the
+    reference's own tests hold it to: the E2M1 grid by brute force (nearest value, ties to the
+    even code), the block scale against torch's e4m3fn cast, closed forms for a zero block
+    and a short last block, and the 20 % relative-error budget of
+    tests/unit/test_grouped_gemm_contract.py:158-169 on a grouped product."""
+    grid = np.array([0, 0.5, 1, 1.5, 2, 3, 4, 6], np.float64)          # E2M1: codes 0..7 in order
+    xs = np.concatenate([np.linspace(-7, 7, 56001), (grid[:-1] + grid[1:]) / 2, -(grid[:-1] + grid[1:]) / 2])
+    want = np.empty_like(xs)
+    for i, v in enumerate(np.abs(xs)):
+        d = np.abs(grid - v)
+        near = np.flatnonzero(d == d.min())
+        code = near[0] if near.size == 1 else (near[0] if near[0] % 2 == 0 else near[1])   # tie: even code
+        want[i] = grid[code]
+    want = np.copysign(want, xs)
+    got = orc.fpquant_grid(xs.astype(np.float32), max_normal=6.0, mantissa_bits=1, min_exp=0)
+    exact = xs.astype(np.float32).astype(np.float64) == xs              # only points f32 holds exactly are ties
+    assert np.array_equal(got[exact], want[exact].astype(np.float32))
+    assert np.max(np.abs(got - want)) <= 1.0                            # (a point f32 rounds across a midpoint lands on the neighbour)
+    assert np.mean(got == want.astype(np.float32)) > 0.9999
+    # a block whose amax is 6 * s for an e4m3-exact s quantises with scale s: values on the grid come back exactly
+    blk = np.array([6, -4, 3, 2, 1.5, 1, 0.5, 0, -0.5, -1, -1.5, -2, -3, 4, -6, 0], np.float32)
+    for sc in (1.0, 0.375, 2.0 ** -9, 448.0 / 8):
+        dq, scales = orc.quantize_nvfp4((blk * np.float32(sc))[None])
+        assert scales.shape == (1, 1) and scales[0, 0] == np.float32(sc)
+        assert np.array_equal(dq[0], blk * np.float32(sc))
+    # the block scale is the e4m3fn cast of amax / 6
+    rng = np.random.default_rng(12)
+    X = (rng.standard_normal((500, 64)) * np.exp(rng.standard_normal((500, 1)) * 3)).astype(np.float32)
+    dq, scales = orc.quantize_nvfp4(X)
+    raw = np.maximum(np.abs(X.reshape(500, 4, 16)).max(-1) / np.float32(6.0), np.float32(1e-30)).astype(np.float32)
+    tq = torch.from_numpy(np.minimum(raw, np.float32(448.0))).to(torch.float8_e4m3fn).to(torch.float32).numpy()
+    assert np.array_equal(scales, tq)
+    # every value is code * scale with the code on the grid
+    sf = np.where(scales == 0, 1, scales)[..., None]
+    codes = np.abs(dq.reshape(500, 4, 16) / sf)
+    assert np.isin(codes, grid.astype(np.float32)).all()
+    # zero block -> zeros, scale as the cast of the floor (0 in e4m3); short last block == zero-padded block
+    z, zs = orc.quantize_nvfp4(np.zeros((2, 32), np.float32))
+    assert not z.any() and not zs.any()
+    a, sa = orc.quantize_nvfp4(X[:, :40])
+    b, sb = orc.quantize_nvfp4(np.concatenate([X[:, :40], np.zeros((500, 8), np.float32)], 1))
+    assert np.array_equal(a, b[:, :40]) and np.array_equal(sa, sb)
+    # the reference's budget for the grouped product on its own test's shapes
+    for gs in ([5, 3, 4], [16, 16, 32]):
+        r = np.random.default_rng(9)
+        T = sum(gs)
+        x = r.standard_normal((T, 64)).astype(np.float32)
+        w = r.standard_normal((len(gs), 64, 16)).astype(np.float32)
+        full = np.zeros((T, 16)); off = 0
+        for e, n in enumerate(gs):
+            full[off:off + n] = x[off:off + n].astype(np.float64) @ w[e].astype(np.float64); off += n
+        got = orc.grouped_gemm_nvfp4(x, w, gs)
+        assert np.linalg.norm(got - full) / np.linalg.norm(full) < 0.20
+
+
 def test_int8_quantiser_and_w8a8():
     M = np.array([[1.0, -2.0, 0.5], [0.0, 0.0, 0.0], [127.0, 63.5, -64.5]], np.float32)
     q, s = orc.quantize_int8_per_channel(M, axis=1)
