@@ -513,6 +513,14 @@ int tessera_gfx950_grouped_gemm_bf16_dev(const void* x, const void* w, const int
                                          int S, int K, int N, int E, void* stream);
 int tessera_gfx950_grouped_gemm_bf16_f32_dev(const void* x, const void* w, const int32_t* offsets, void* y,
                                              int S, int K, int N, int E, void* stream);
+/* ops.silu_mul (python/tessera/__init__.py:559-574): out = silu(a) * b elementwise, silu(a) =
+ * a / (1 + exp(-a)); 16-bit storage in and out, f32 arithmetic, n elements.  The stand-alone
+ * form of the step the fused block below applies in its epilogue (the reference's quantised
+ * block composes grouped_gemm, silu_mul and grouped_gemm: python/tessera/__init__.py:610-616). */
+int tessera_gfx950_silu_mul_bf16(const void* a, const void* b, void* out, int64_t n);
+int tessera_gfx950_silu_mul_f16(const void* a, const void* b, void* out, int64_t n);
+int tessera_gfx950_silu_mul_bf16_dev(const void* a, const void* b, void* out, int64_t n, void* stream);
+int tessera_gfx950_silu_mul_f16_dev(const void* a, const void* b, void* out, int64_t n, void* stream);
 /* tessera.grouped_swiglu / ops.moe_swiglu_block
  * (python/tessera/runtime.py:20353-20368; python/tessera/__init__.py:592-616):
  * y = gg(bf16(silu(bf16(gg(x,Wg))) * bf16(gg(x,Wu))), Wd), every intermediate

@@ -884,12 +884,70 @@ int grouped_host(const void* x, const void* w, const int32_t* offsets, void* y, 
   if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
   return scope.download(y, dy, (size_t)S * N * dsz) ? kOk : kDeviceFailed;
 }
+// out = storage(silu(a) * b) elementwise on 16-bit storage, eight elements per thread in the body.
+template <class T>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
+                                                       uint16_t* __restrict__ out, long n) {
+  auto one = [](uint16_t ga, uint16_t ub) -> uint16_t {
+    const float g = from_storage<T>(ga), u = from_storage<T>(ub);
+    return to_storage<T>((g / (1.0f + __expf(-g))) * u);
+  };
+  const long tid = (long)blockIdx.x * 256 + threadIdx.x, nth = (long)gridDim.x * 256;
+  const bool vec = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  const long n8 = vec ? n / 8 : 0;
+  for (long i = tid; i < n8; i += nth) {
+    const uint4 va = reinterpret_cast<const uint4*>(a)[i], vb = reinterpret_cast<const uint4*>(b)[i];
+    const uint32_t wa[4] = {va.x, va.y, va.z, va.w}, wb[4] = {vb.x, vb.y, vb.z, vb.w};
+    uint32_t wo[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      wo[e] = (uint32_t)one((uint16_t)(wa[e] & 0xffff), (uint16_t)(wb[e] & 0xffff)) |
+              ((uint32_t)one((uint16_t)(wa[e] >> 16), (uint16_t)(wb[e] >> 16)) << 16);
+    reinterpret_cast<uint4*>(out)[i] = make_uint4(wo[0], wo[1], wo[2], wo[3]);
+  }
+  for (long i = n8 * 8 + tid; i < n; i += nth) out[i] = one(a[i], b[i]);
+}
+
+template <class T>
+int silu_mul_dev(const void* a, const void* b, void* out, int64_t n, hipStream_t s) {
+  if (n <= 0 || !a || !b || !out) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const long blocks = std::min<long>((n / 8 + 255) / 256 + 1, 8192);
+  hipLaunchKernelGGL(silu_mul_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const uint16_t*>(a),
+                     static_cast<const uint16_t*>(b), static_cast<uint16_t*>(out), (long)n);
+  return launch_status();
+}
+
+template <class T>
+int silu_mul_host(const void* a, const void* b, void* out, int64_t n) {
+  if (n <= 0 || !a || !b || !out) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  DeviceScope scope;
+  void* da = scope.alloc((size_t)n * 2, a);
+  void* db = scope.alloc((size_t)n * 2, b);
+  void* dout = scope.alloc((size_t)n * 2);
+  if (scope.failed()) return kDeviceFailed;
+  int rc = silu_mul_dev<T>(da, db, dout, n, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  return scope.download(out, dout, (size_t)n * 2) ? kOk : kDeviceFailed;
+}
 }  // namespace
 }  // namespace tsr950
 
 using namespace tsr950;
 
 extern "C" {
+
+int tessera_gfx950_silu_mul_bf16(const void* a, const void* b, void* out, int64_t n) { return silu_mul_host<BF16>(a, b, out, n); }
+int tessera_gfx950_silu_mul_f16(const void* a, const void* b, void* out, int64_t n) { return silu_mul_host<F16>(a, b, out, n); }
+int tessera_gfx950_silu_mul_bf16_dev(const void* a, const void* b, void* out, int64_t n, void* stream) {
+  return silu_mul_dev<BF16>(a, b, out, n, as_stream(stream));
+}
+int tessera_gfx950_silu_mul_f16_dev(const void* a, const void* b, void* out, int64_t n, void* stream) {
+  return silu_mul_dev<F16>(a, b, out, n, as_stream(stream));
+}
+
 
 int tessera_gfx950_moe_route_f32_dev(const float* scores, int T, int E, int k, int normalize, int capacity,
                                      int32_t* token_of_slot, int32_t* expert_of_slot, float* combine_weights,

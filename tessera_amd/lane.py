@@ -97,6 +97,10 @@ _SIGNATURES = {
     "tessera_gfx950_batched_gemm_strided_bf16_dev": [_c_vp] * 3 + [_c_int] * 4 + [_c_i64] * 3 + [_c_int, _c_vp],
     "tessera_gfx950_fake_quantize_nvfp4_f32": [_c_vp, _c_int, _c_int, _c_vp, _c_vp, _c_vp],
     "tessera_gfx950_fake_quantize_nvfp4_f32_dev": [_c_vp, _c_int, _c_int, _c_vp, _c_vp, _c_vp, _c_vp],
+    "tessera_gfx950_silu_mul_bf16": [_c_vp, _c_vp, _c_vp, _c_i64],
+    "tessera_gfx950_silu_mul_bf16_dev": [_c_vp, _c_vp, _c_vp, _c_i64, _c_vp],
+    "tessera_gfx950_silu_mul_f16": [_c_vp, _c_vp, _c_vp, _c_i64],
+    "tessera_gfx950_silu_mul_f16_dev": [_c_vp, _c_vp, _c_vp, _c_i64, _c_vp],
     "tessera_gfx950_gemm_schedule": [_c_int] * 5 + [_c_vp] * 4,
     "tessera_gfx950_gemm_rest_split": [_c_int] * 4 + [_c_vp] * 2,
     "tessera_gfx950_gemm_bias_act_f16": [_c_vp, _c_vp, _c_vp, _c_int, _c_vp, _c_int, _c_int, _c_int],

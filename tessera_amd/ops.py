@@ -490,14 +490,35 @@ def _grouped_gemm_fp8(x, weights, xa, w, gs, quant, alignment, out):
     return y if f32 else y.view(BF16Array)
 
 
+def silu_mul(a, b):
+    """``silu(a) * b`` elementwise (``__init__.py:559-574``) on 16-bit storage arrays of one
+    shape; the result is rounded to the same storage dtype."""
+    a, b = _unbox(a), _unbox(b)
+    st = _storage(a, b)
+    ab, bb = _bits(a), _bits(b)
+    if ab.shape != bb.shape:
+        raise ValueError(f"silu_mul: shapes differ — {ab.shape} vs {bb.shape}")
+    outb = np.empty(ab.shape, np.uint16)
+    if ab.size:
+        _lane.check(getattr(_lane.load(), f"tessera_gfx950_silu_mul_{st}")(
+            np.ascontiguousarray(ab).ctypes.data, np.ascontiguousarray(bb).ctypes.data, outb.ctypes.data, ab.size), "silu_mul")
+    return _wrap(outb, st)
+
+
 def moe_swiglu_block(x, w_gate, w_up, w_down, group_sizes, *, kind: str = "contiguous", alignment=None,
                      quant=None):
     """``gg(silu_mul(gg(x, Wg), gg(x, Wu)), Wd)`` over contiguous expert groups,
-    every intermediate rounded to bf16 as the reference's storage rule does."""
+    every intermediate rounded to bf16 as the reference's storage rule does.  With
+    ``quant`` every grouped product quantises its operands as ``grouped_gemm(quant=)``
+    does, and the block is the reference's composition of the three products around
+    ``silu_mul`` (``__init__.py:610-616``) instead of the fused kernel."""
     if kind not in GROUPED_KINDS:
         raise ValueError(f"moe_swiglu_block: unknown kind {kind!r}")
-    if kind not in _SUPPORTED_GROUPED_KINDS or quant is not None:
-        raise NotImplementedError("moe_swiglu_block: only contiguous/dense, unquantised on the gfx950 lane")
+    if kind not in _SUPPORTED_GROUPED_KINDS:
+        raise NotImplementedError("moe_swiglu_block: only contiguous/dense on the gfx950 lane")
+    if quant is not None:
+        gg = lambda a, w: grouped_gemm(a, w, group_sizes, kind=kind, alignment=alignment, quant=quant)
+        return gg(silu_mul(gg(x, w_gate), gg(x, w_up)), w_down)
     x, w_gate, w_up, w_down = map(_unbox, (x, w_gate, w_up, w_down))
     for a in (x, w_gate, w_up, w_down):
         if _storage(a) != "bf16":
@@ -776,6 +797,28 @@ def moe_combine(y_packed, plan: MoETransport) -> np.ndarray:
     return outp
 
 
+def _moe_layer_staged(x, W_router, W_gate, W_up, W_down, top_k, normalize_weights, capacity_factor, kind, alignment,
+                      quant, router_logits, return_plan):
+    """The layer as the reference composes it (``nn/functional.py:447-490``) — router product,
+    routing, dispatch, expert block, combine — each stage one device op with host arrays in
+    between: the form that carries ``quant`` and ``alignment`` into the expert block."""
+    xa = _unbox(x)
+    T = _bits(xa).shape[0]
+    E = _bits(_unbox(W_gate)).shape[0]
+    if router_logits is None:
+        scores = gemm(xa, W_router)
+        scores = scores.to_float32() if isinstance(scores, BF16Array) else np.asarray(scores, np.float32)
+    else:
+        scores = np.ascontiguousarray(router_logits, np.float32)
+    plan = route_tokens(scores, E, top_k, normalize_weights=normalize_weights,
+                        capacity_factor=capacity_factor if capacity_factor > 0 else 1e9)
+    x_perm = moe_dispatch(xa, plan)
+    y_perm = moe_swiglu_block(x_perm, W_gate, W_up, W_down, np.asarray(plan.group_sizes, np.int64), kind=kind,
+                              alignment=alignment, quant=quant)
+    out = moe_combine(y_perm, plan)
+    return (out, plan) if return_plan else out
+
+
 def moe_layer(x, W_router, W_gate, W_up, W_down, *, top_k: int = 1, normalize_weights: bool = True,
               capacity_factor: float = 0.0, kind: str = "contiguous", alignment=None, quant=None,
               router_logits=None, return_plan: bool = False):
@@ -784,8 +827,11 @@ def moe_layer(x, W_router, W_gate, W_up, W_down, *, top_k: int = 1, normalize_we
     ``(E, K, F)``, ``W_down`` ``(E, F, N)`` in bf16; returns ``(T, N)`` f32.
     ``capacity_factor <= 0`` disables capacity drops.  ``router_logits``
     ``(T, E)`` f32 may be given instead of ``W_router``."""
-    if kind not in _SUPPORTED_GROUPED_KINDS or quant is not None or alignment is not None:
-        raise NotImplementedError("moe_layer: contiguous, unquantised, unaligned form only on the gfx950 lane")
+    if kind not in _SUPPORTED_GROUPED_KINDS:
+        raise NotImplementedError("moe_layer: contiguous / dense grouped layouts only on the gfx950 lane")
+    if quant is not None or alignment is not None:
+        return _moe_layer_staged(x, W_router, W_gate, W_up, W_down, top_k, normalize_weights, capacity_factor, kind,
+                                 alignment, quant, router_logits, return_plan)
     x, W_gate, W_up, W_down = map(_unbox, (x, W_gate, W_up, W_down))
     for a in (x, W_gate, W_up, W_down):
         if _storage(a) != "bf16":

@@ -441,3 +441,68 @@ def test_moe_headline_config(lane):
     np.add.at(ref, tok_of, y.astype(np.float64) * desc.combine_weights[slots][:, None].astype(np.float64))
     got = np.asarray(out, np.float32)[tokens]
     assert orc.max_rel_err(got, ref[tokens]) <= TOL + 2.0 ** -8
+
+
+def test_silu_mul_on_the_storage_grid(lane):
+    """ops.silu_mul: silu(a) * b on 16-bit storage, rounded to the same storage; odd length and
+    both dtypes; the unquantised block equals grouped products around it."""
+    rng = np.random.default_rng(61)
+    for n in (1, 7, 4096, 100003):
+        a = (rng.standard_normal(n) * 3).astype(np.float32)
+        b = rng.standard_normal(n).astype(np.float32)
+        for st in ("bf16", "f16"):
+            aa = b16.from_float32(a) if st == "bf16" else a.astype(np.float16)
+            bb = b16.from_float32(b) if st == "bf16" else b.astype(np.float16)
+            af = aa.to_float32() if st == "bf16" else aa.astype(np.float32)
+            bf = bb.to_float32() if st == "bf16" else bb.astype(np.float32)
+            got = ops.silu_mul(aa, bb)
+            gf = got.to_float32() if st == "bf16" else got.astype(np.float32)
+            ref = (af.astype(np.float64) / (1 + np.exp(-af.astype(np.float64)))) * bf
+            assert np.max(np.abs(gf - ref) / (np.abs(ref) + 1e-3)) <= (2.0 ** -8 if st == "bf16" else 2.0 ** -11) + 1e-5
+    sizes = [40, 0, 300, 7]
+    x, wg, wu, wd = _swiglu_inputs(sizes, 256, 384, 128, 3)
+    xb, g, u, d = (b16.from_float32(t) for t in (x, wg, wu, wd))
+    fused = ops.moe_swiglu_block(xb, g, u, d, sizes).to_float32()
+    staged = ops.grouped_gemm(ops.silu_mul(ops.grouped_gemm(xb, g, sizes), ops.grouped_gemm(xb, u, sizes)), d, sizes).to_float32()
+    assert orc.max_rel_err(staged, fused) <= 2.0 ** -7          # the same roundings; exp differs in its last bits
+
+
+@pytest.mark.parametrize("quant,budget", [("nvfp4", 0.30), ("fp8_e4m3", 0.10)])
+def test_quantised_swiglu_block_and_layer(lane, quant, budget):
+    """moe_swiglu_block(quant=) is the reference's composition — three quantised grouped products
+    around silu_mul — and moe_layer(quant=) carries it through routing, dispatch and combine.
+    Against the unquantised block inside a format budget, against the oracle's composition
+    normwise (a hidden value that sits on a rounding boundary may fall either way), and the
+    layer against its own stages."""
+    sizes = [48, 0, 304, 16]
+    x, wg, wu, wd = _swiglu_inputs(sizes, 256, 384, 128, 5)
+    xb, g, u, d = (b16.from_float32(t) for t in (x, wg, wu, wd))
+    full = ops.moe_swiglu_block(xb, g, u, d, sizes).to_float32()
+    got = ops.moe_swiglu_block(xb, g, u, d, sizes, quant=quant).to_float32()
+    assert got.shape == full.shape
+    assert np.linalg.norm(got - full) / np.linalg.norm(full) < budget
+    if quant == "nvfp4":
+        f = lambda t: t.to_float32()
+        st = lambda t: orc.round_to_storage(np.asarray(t, np.float32), "bf16")
+        gate = st(orc.grouped_gemm_nvfp4(f(xb), f(g), sizes))
+        up = st(orc.grouped_gemm_nvfp4(f(xb), f(u), sizes))
+        hid = st(orc.silu_mul(gate, up))
+        ref = st(orc.grouped_gemm_nvfp4(hid, f(d), sizes))
+        assert np.linalg.norm(got - ref) / np.linalg.norm(ref) < 2e-2
+    with pytest.raises(ValueError):
+        ops.moe_swiglu_block(xb, g, u, d, sizes, quant=quant, alignment=32)       # 48 and 304 are multiples of 16 only
+    assert ops.moe_swiglu_block(xb, g, u, d, sizes, quant=quant, alignment=16).shape == full.shape
+    # the layer
+    T, H, F, N, E, k = 200, 256, 384, 128, 4, 2
+    rng = np.random.default_rng(8)
+    xl = b16.from_float32(rng.standard_normal((T, H)).astype(np.float32))
+    lg = _logits(T, E, 41, k)
+    plain, plan0 = ops.moe_layer(xl, None, g, u, d, top_k=k, router_logits=lg, return_plan=True)
+    out, plan = ops.moe_layer(xl, None, g, u, d, top_k=k, router_logits=lg, quant=quant, return_plan=True)
+    assert np.array_equal(plan.token_of_slot, plan0.token_of_slot) and np.array_equal(plan.group_sizes, plan0.group_sizes)
+    assert np.linalg.norm(out - plain) / np.linalg.norm(plain) < budget
+    staged = ops.moe_combine(ops.moe_swiglu_block(ops.moe_dispatch(xl, plan), g, u, d, np.asarray(plan.group_sizes),
+                                                  quant=quant), plan)
+    assert np.array_equal(out, staged)
+    aligned = ops.moe_layer(xl, None, g, u, d, top_k=k, router_logits=lg, alignment=1)
+    assert orc.max_rel_err(aligned, plain) <= 2.0 ** -6         # the staged unquantised form against the fused layer
