@@ -281,6 +281,28 @@ int tessera_gfx950_quantize_i8_f32(const float* x, int M, int N, int axis, void*
 int tessera_gfx950_fake_quantize_nvfp4_f32(const float* x, int rows, int cols, float* dq, void* dq_bf16, float* scales);
 int tessera_gfx950_fake_quantize_nvfp4_f32_dev(const float* x, int rows, int cols, float* dq, void* dq_bf16,
                                                float* scales, void* stream);
+/* tessera_x86_avx512_fpquant_f32
+ * (src/compiler/codegen/tessera_x86_backend/src/kernels/avx512_fpquant_f32.cpp:45-83; the scalar
+ * definition at :28-41): out[i] = x[i] snapped to the float grid (max_normal, mantissa_bits,
+ * min_exp) — ax = min(|x|, max_normal); e = max(floor(log2 ax), min_exp); ulp = 2^(e - mantissa_bits);
+ * out = sign(x) min(rne(ax / ulp) ulp, max_normal); NaN propagates.  The reference's format table
+ * (python/tessera/runtime.py:16939-16946): e4m3 (448, 3, -6), e5m2 (57344, 2, -14), e2m3
+ * (7.5, 3, -126), e3m2 (28, 2, -126), e2m1 (6, 1, -126).  mantissa_bits in [0, 23], min_exp in
+ * [-126, 127], max_normal finite and positive, else TSR_BAD_SHAPE. */
+int tessera_gfx950_fpquant_f32(const float* x, int64_t n, float max_normal, int mantissa_bits, int min_exp, float* out);
+int tessera_gfx950_fpquant_f32_dev(const float* x, int64_t n, float max_normal, int mantissa_bits, int min_exp,
+                                   float* out, void* stream);
+/* ops.quantize_fp8 / quantize_fp6 / quantize_fp4 (python/tessera/__init__.py:3340-3374, 3411-3464):
+ * per-tensor scale = `scale` if > 0, else max(amax|x| / max_normal, 1e-12) found on the device;
+ * grid = fpquant(x / scale) as above; dq (f32, optional) receives grid * scale, the reference's
+ * return value; grid_bf16 (optional) the unscaled grid values as bf16 bit patterns, exact for
+ * every format of the table above, i.e. a ready operand for a 16-bit product that is scaled
+ * afterwards; scale_out (optional) the scale used.  With the automatic scale a NaN in x is
+ * skipped by the maximum (the reference's numpy maximum would return NaN for everything). */
+int tessera_gfx950_fake_quantize_fp_f32(const float* x, int64_t n, float max_normal, int mantissa_bits, int min_exp,
+                                        float scale, float* dq, void* grid_bf16, float* scale_out);
+int tessera_gfx950_fake_quantize_fp_f32_dev(const float* x, int64_t n, float max_normal, int mantissa_bits, int min_exp,
+                                            float scale, float* dq, void* grid_bf16, float* scale_out_dev, void* stream);
 int tessera_gfx950_quantize_e4m3_f32_dev(const float* x, int64_t n, float scale, void* codes, float* scale_out_dev, void* stream);
 int tessera_gfx950_quantize_i8_f32_dev(const float* x, int M, int N, int axis, void* q, float* scales, void* stream);
 
@@ -513,6 +535,16 @@ int tessera_gfx950_grouped_gemm_bf16_dev(const void* x, const void* w, const int
                                          int S, int K, int N, int E, void* stream);
 int tessera_gfx950_grouped_gemm_bf16_f32_dev(const void* x, const void* w, const int32_t* offsets, void* y,
                                              int S, int K, int N, int E, void* stream);
+/* The per-tensor scales of the reference's quantised grouped product
+ * (python/tessera/compiler/grouped_layout.py:373-392: x quantised as one tensor, each expert's
+ * weight on its own), applied after the product of the unscaled grid values:
+ * out[r, :] = y[r, :] * scale[e] for offsets[e] <= r < offsets[e+1].  y f32 [S, N]; scale f32 [E]
+ * (the activation's scale times expert e's); out f32, or bf16 when out_bf16 != 0 (may not alias y
+ * then). */
+int tessera_gfx950_scale_groups_f32(const float* y, const int32_t* offsets, const float* scale, void* out, int out_bf16,
+                                    int S, int N, int E);
+int tessera_gfx950_scale_groups_f32_dev(const float* y, const int32_t* offsets, const float* scale, void* out,
+                                        int out_bf16, int S, int N, int E, void* stream);
 /* ops.silu_mul (python/tessera/__init__.py:559-574): out = silu(a) * b elementwise, silu(a) =
  * a / (1 + exp(-a)); 16-bit storage in and out, f32 arithmetic, n elements.  The stand-alone
  * form of the step the fused block below applies in its epilogue (the reference's quantised

@@ -706,6 +706,29 @@ def quantize_fp8_e4m3(x: np.ndarray, scale: float | None = None):
     return e4m3_encode(grid), grid, np.float32(scale)
 
 
+#: (max_normal, mantissa_bits, min_exp) of the per-tensor float grids: the native lanes'
+#: format table (``runtime.py:16939-16946``).  The fp8 grids have IEEE gradual underflow;
+#: fp6 and fp4 keep the pure mantissa snap (exponent floor -126, i.e. none in practice).
+FP_FORMATS = {"e4m3": (448.0, 3, -6), "e5m2": (57344.0, 2, -14), "e2m3": (7.5, 3, -126), "e3m2": (28.0, 2, -126),
+              "e2m1": (6.0, 1, -126)}
+
+
+def quantize_fp(x: np.ndarray, fmt: str, scale: float | None = None):
+    """``ops.quantize_fp8`` / ``quantize_fp6`` / ``quantize_fp4`` (``__init__.py:3340-3374``,
+    ``3411-3464``): per-tensor ``scale = max(amax / max_normal, 1e-12)`` in f32 unless given,
+    ``grid = fpquant(clip(x / scale))``, result ``grid * f32(scale)``.  Returns
+    ``(dequantised f32, grid f32, scale np.float32)``."""
+    mx, mant, min_exp = FP_FORMATS[fmt]
+    x = np.asarray(x, np.float32)
+    if scale is None:
+        amax = np.max(np.abs(x)) if x.size else np.float32(0)
+        scale = float(np.maximum(amax / np.float32(mx), np.float32(1e-12)))
+    with np.errstate(invalid="ignore"):
+        scaled = np.clip(x / np.float32(scale), -mx, mx).astype(np.float32)
+    grid = fpquant_grid(scaled, mx, mant, min_exp)
+    return (grid * np.float32(scale)).astype(np.float32), grid, np.float32(scale)
+
+
 def quantize_nvfp4(x: np.ndarray, block_size: int = 16):
     """``ops.quantize_nvfp4`` (``__init__.py:3472-3500``), i.e. ``microscaling.quantize`` with
     the ``nvfp4`` format followed by ``dequantize`` (``compiler/microscaling.py:317-384``):
@@ -740,6 +763,40 @@ def grouped_gemm_nvfp4(x, w, group_sizes):
     xq, _ = quantize_nvfp4(np.asarray(x, np.float32))
     w = np.asarray(w, np.float32)
     wq = np.stack([quantize_nvfp4(w[e])[0] for e in range(w.shape[0])])
+    out = np.zeros((xq.shape[0], w.shape[2]), np.float64)
+    off = 0
+    for e, n in enumerate(np.asarray(group_sizes).astype(np.int64)):
+        if n:
+            out[off:off + n] = xq[off:off + n].astype(np.float64) @ wq[e].astype(np.float64)
+        off += int(n)
+    return out
+
+
+#: quant= spellings of the grouped product -> (activation format, weight format)
+#: (``compiler/grouped_layout.py:320-332``)
+GROUPED_QUANT_SCHEMES = {
+    "fp8_e4m3": ("fp8_e4m3", "fp8_e4m3"), "fp8": ("fp8_e4m3", "fp8_e4m3"), "fp8_e5m2": ("fp8_e5m2", "fp8_e5m2"),
+    "nvfp4": ("nvfp4", "nvfp4"), "fp8xfp4": ("fp8_e4m3", "nvfp4"), "fp8_e4m3xnvfp4": ("fp8_e4m3", "nvfp4"),
+    "fp8_e5m2xnvfp4": ("fp8_e5m2", "nvfp4"),
+}
+
+
+def _qdq(a: np.ndarray, dtype: str) -> np.ndarray:
+    """One 2-D operand quantised and dequantised (``compiler/grouped_layout.py:353-370``)."""
+    if dtype == "nvfp4":
+        return quantize_nvfp4(a)[0]
+    return quantize_fp(a, "e5m2" if dtype == "fp8_e5m2" else "e4m3")[0]
+
+
+def grouped_gemm_quant(x, w, group_sizes, quant: str):
+    """``ops.grouped_gemm(..., quant=)`` for every scheme of the reference
+    (``compiler/grouped_layout.py:373-392``): x ``(T, K)`` is quantised as one tensor with
+    the activation format, every expert's ``(K, N)`` weight on its own with the weight
+    format, and the grouped product runs on the dequantised values (f64 here)."""
+    act, wt = GROUPED_QUANT_SCHEMES[str(quant).lower()]
+    xq = _qdq(np.asarray(x, np.float32), act)
+    w = np.asarray(w, np.float32)
+    wq = np.stack([_qdq(w[e], wt) for e in range(w.shape[0])])
     out = np.zeros((xq.shape[0], w.shape[2]), np.float64)
     off = 0
     for e, n in enumerate(np.asarray(group_sizes).astype(np.int64)):

@@ -1,5 +1,6 @@
 // C ABI: quantised GEMMs (int8 -> int32, W8A8 with scales, fp8 e4m3 with
 // per-tensor scales) and the quantisers that produce their operands.
+#include <cmath>
 #include <mutex>
 #include "../../include/tessera_gfx950.h"
 #include "gemm8.h"
@@ -426,6 +427,81 @@ int quantize_i8_dev(const float* x, int M, int N, int axis, void* q, float* scal
   return launch_status();
 }
 
+// ---- per-tensor float grids (fp8 / fp6 / fp4) ---------------------------------------------------
+// The native lanes' grid rounding, tessera_x86_avx512_fpquant_f32
+// (src/compiler/codegen/tessera_x86_backend/src/kernels/avx512_fpquant_f32.cpp:28-41):
+//   ax = min(|v|, max_normal); e = max(floor(log2 ax), min_exp); ulp = 2^(e - mantissa_bits);
+//   out = sign(v) * min(rne(ax / ulp) * ulp, max_normal); NaN propagates; zero gives +0.
+// Both scalings are by powers of two, so ldexp is exact wherever the division and the product are.
+__device__ __forceinline__ float fp_grid(float v, float max_normal, int mant, int min_exp) {
+  if (v != v) return v;
+  const float ax = fminf(fabsf(v), max_normal);
+  if (!(ax > 0.f)) return 0.f;
+  int e;
+  (void)frexpf(ax, &e);                                   // ax = m 2^e with m in [0.5, 1), denormals included
+  e = max(e - 1, min_exp);
+  const float q = __builtin_rintf(ldexpf(ax, mant - e));
+  const float r = fminf(ldexpf(q, e - mant), max_normal);
+  return v < 0.f ? -r : r;
+}
+
+// ops.quantize_fp8 / quantize_fp6 / quantize_fp4 (python/tessera/__init__.py:3340-3374, 3411-3464):
+// scale = scale_in if > 0, else max(amax / max_normal, 1e-12); grid = fp_grid(x / scale) (the
+// reference clips x / scale to +-max_normal first, which the grid's own clamp already does);
+// dq = grid * scale.  grid16 receives the grid values as bf16 bits: exact for every format of at
+// most 7 mantissa bits whose range lies within bf16's.
+__global__ __launch_bounds__(256) void fake_quantize_fp_kernel(const float* __restrict__ x, long n, float max_normal,
+                                                               int mant, int min_exp, float scale_in,
+                                                               const unsigned* amax_bits, float* __restrict__ dq,
+                                                               uint16_t* __restrict__ grid16, float* scale_out) {
+  float scale = scale_in;
+  if (!(scale_in > 0.f)) scale = fmaxf(__fdiv_rn(__builtin_bit_cast(float, *amax_bits), max_normal), 1e-12f);
+  if (scale_out && blockIdx.x == 0 && threadIdx.x == 0) *scale_out = scale;
+  const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x, nthreads = (long)gridDim.x * blockDim.x;
+  const bool vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dq)) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(grid16) & 7) == 0;
+  const long n4 = vec ? n / 4 : 0;
+  auto bf16_bits = [](float g) { return (uint32_t)(__builtin_bit_cast(uint32_t, g) >> 16); };
+  for (long i = tid; i < n4; i += nthreads) {
+    const float4 v = reinterpret_cast<const float4*>(x)[i];
+    const float g0 = fp_grid(__fdiv_rn(v.x, scale), max_normal, mant, min_exp);
+    const float g1 = fp_grid(__fdiv_rn(v.y, scale), max_normal, mant, min_exp);
+    const float g2 = fp_grid(__fdiv_rn(v.z, scale), max_normal, mant, min_exp);
+    const float g3 = fp_grid(__fdiv_rn(v.w, scale), max_normal, mant, min_exp);
+    if (dq) reinterpret_cast<float4*>(dq)[i] = make_float4(g0 * scale, g1 * scale, g2 * scale, g3 * scale);
+    if (grid16)
+      reinterpret_cast<uint2*>(grid16)[i] = make_uint2(bf16_bits(g0) | (bf16_bits(g1) << 16), bf16_bits(g2) | (bf16_bits(g3) << 16));
+  }
+  for (long i = n4 * 4 + tid; i < n; i += nthreads) {
+    const float g = fp_grid(__fdiv_rn(x[i], scale), max_normal, mant, min_exp);
+    if (dq) dq[i] = g * scale;
+    if (grid16) grid16[i] = (uint16_t)bf16_bits(g);
+  }
+}
+
+// mantissa_bits 0..23 and min_exp -126..127 keep every power of two the rounding forms a normal
+// or denormal f32.
+bool bad_fp_format(float max_normal, int mant, int min_exp) {
+  return !(max_normal > 0.f) || !std::isfinite(max_normal) || mant < 0 || mant > 23 || min_exp < -126 || min_exp > 127;
+}
+
+int fake_quantize_fp_dev(const float* x, int64_t n, float max_normal, int mant, int min_exp, float scale, float* dq,
+                         void* grid16, float* scale_out_dev, hipStream_t s) {
+  if (n <= 0 || !x || (!dq && !grid16) || bad_fp_format(max_normal, mant, min_exp) || scale != scale) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const int blocks = (int)std::min<int64_t>((n / 4 + 255) / 256 + 1, 4096);
+  unsigned* amax = nullptr;
+  if (!(scale > 0.f)) {
+    amax = static_cast<unsigned*>(stream_workspace(s, 256));
+    if (!amax) return kDeviceFailed;
+    zero_words(amax, 1, s);
+    hipLaunchKernelGGL(absmax_kernel, dim3(std::min(blocks, 512)), dim3(256), 0, s, x, (long)n, amax);
+  }
+  hipLaunchKernelGGL(fake_quantize_fp_kernel, dim3(blocks), dim3(256), 0, s, x, (long)n, max_normal, mant, min_exp, scale,
+                     amax, dq, static_cast<uint16_t*>(grid16), scale_out_dev);
+  return launch_status();
+}
+
 // ---- NVFP4 (block-scaled E2M1) rounding -------------------------------------------------------
 // ops.quantize_nvfp4 followed by dequantize_nvfp4 (python/tessera/__init__.py:3472-3504;
 // compiler/microscaling.py:317-384): blocks of 16 along the last axis (a short last block counts
@@ -602,6 +678,41 @@ int tessera_gfx950_fake_quantize_nvfp4_f32(const float* x, int rows, int cols, f
   if (dq_bf16 && !scope.download(dq_bf16, d16, n * 2)) return kDeviceFailed;
   if (scales && !scope.download(scales, ds, ns * 4)) return kDeviceFailed;
   return kOk;
+}
+
+int tessera_gfx950_fake_quantize_fp_f32_dev(const float* x, int64_t n, float max_normal, int mantissa_bits, int min_exp,
+                                            float scale, float* dq, void* grid_bf16, float* scale_out_dev, void* stream) {
+  return fake_quantize_fp_dev(x, n, max_normal, mantissa_bits, min_exp, scale, dq, grid_bf16, scale_out_dev,
+                              as_stream(stream));
+}
+int tessera_gfx950_fpquant_f32_dev(const float* x, int64_t n, float max_normal, int mantissa_bits, int min_exp, float* out,
+                                   void* stream) {
+  if (!out) return kBadShape;
+  return fake_quantize_fp_dev(x, n, max_normal, mantissa_bits, min_exp, 1.0f, out, nullptr, nullptr, as_stream(stream));
+}
+
+int tessera_gfx950_fake_quantize_fp_f32(const float* x, int64_t n, float max_normal, int mantissa_bits, int min_exp,
+                                        float scale, float* dq, void* grid_bf16, float* scale_out) {
+  if (n <= 0 || !x || (!dq && !grid_bf16) || bad_fp_format(max_normal, mantissa_bits, min_exp) || scale != scale)
+    return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  DeviceScope scope;
+  float* dx = static_cast<float*>(scope.alloc((size_t)n * 4, x));
+  float* dd = dq ? static_cast<float*>(scope.alloc((size_t)n * 4)) : nullptr;
+  void* d16 = grid_bf16 ? scope.alloc((size_t)n * 2) : nullptr;
+  float* ds = static_cast<float*>(scope.alloc(4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = fake_quantize_fp_dev(dx, n, max_normal, mantissa_bits, min_exp, scale, dd, d16, ds, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  if (dq && !scope.download(dq, dd, (size_t)n * 4)) return kDeviceFailed;
+  if (grid_bf16 && !scope.download(grid_bf16, d16, (size_t)n * 2)) return kDeviceFailed;
+  if (scale_out && !scope.download(scale_out, ds, 4)) return kDeviceFailed;
+  return kOk;
+}
+int tessera_gfx950_fpquant_f32(const float* x, int64_t n, float max_normal, int mantissa_bits, int min_exp, float* out) {
+  if (!out) return kBadShape;
+  return tessera_gfx950_fake_quantize_fp_f32(x, n, max_normal, mantissa_bits, min_exp, 1.0f, out, nullptr, nullptr);
 }
 
 int tessera_gfx950_quantize_e4m3_f32(const float* x, int64_t n, float scale, void* codes, float* scale_out) {

@@ -654,6 +654,40 @@ int dispatch_dev(const void* x, const int32_t* token_of_slot, void* x_perm, int 
   return launch_status();
 }
 
+// out[r, :] = y[r, :] * scale[e] for the rows r of group e (offsets[e] <= r < offsets[e + 1]): the
+// per-tensor scales of a quantised grouped product, applied to the f32 result of the product of
+// the unscaled grid values.  One workgroup per row.  OUT16: the result is rounded to bf16.
+template <bool OUT16>
+__global__ __launch_bounds__(256) void scale_groups_kernel(const float* __restrict__ y, const int32_t* __restrict__ offsets,
+                                                           const float* __restrict__ scale, int E, int N,
+                                                           void* __restrict__ out) {
+  const int r = blockIdx.x;
+  int lo = 0, hi = E - 1;                                  // the last group whose first row is <= r
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (offsets[mid] <= r) lo = mid; else hi = mid - 1;
+  }
+  const float sc = scale[lo];
+  const float* src = y + (long)r * N;
+  for (int n = threadIdx.x; n < N; n += 256) {
+    const float v = src[n] * sc;
+    if constexpr (OUT16) static_cast<uint16_t*>(out)[(long)r * N + n] = f32_to_bf16_bits(v);
+    else static_cast<float*>(out)[(long)r * N + n] = v;
+  }
+}
+
+int scale_groups_dev(const float* y, const int32_t* offsets, const float* scale, void* out, int out_bf16, int S, int N,
+                     int E, hipStream_t s) {
+  if (S < 0 || N <= 0 || E <= 0 || !offsets || !scale || (S > 0 && (!y || !out))) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  if (S == 0) return kOk;
+  if (out_bf16)
+    hipLaunchKernelGGL((scale_groups_kernel<true>), dim3(S), dim3(256), 0, s, y, offsets, scale, E, N, out);
+  else
+    hipLaunchKernelGGL((scale_groups_kernel<false>), dim3(S), dim3(256), 0, s, y, offsets, scale, E, N, out);
+  return launch_status();
+}
+
 bool bad_grouped(int S, int K, int N, int E) { return S < 0 || K <= 0 || N <= 0 || E <= 0; }
 
 // A gathered row of the (rows, K) 16-bit activation is fetched by a buffer load whose
@@ -1167,6 +1201,29 @@ int tessera_gfx950_grouped_gemm_bf16(const void* x, const void* w, const int32_t
 int tessera_gfx950_grouped_gemm_bf16_f32(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K,
                                          int N, int E) {
   return grouped_host<EPI_F32>(x, w, offsets, y, S, K, N, E);
+}
+
+int tessera_gfx950_scale_groups_f32_dev(const float* y, const int32_t* offsets, const float* scale, void* out,
+                                        int out_bf16, int S, int N, int E, void* stream) {
+  return scale_groups_dev(y, offsets, scale, out, out_bf16, S, N, E, as_stream(stream));
+}
+int tessera_gfx950_scale_groups_f32(const float* y, const int32_t* offsets, const float* scale, void* out, int out_bf16,
+                                    int S, int N, int E) {
+  if (S < 0 || N <= 0 || E <= 0 || !offsets || !scale || (S > 0 && (!y || !out))) return kBadShape;
+  if (bad_offsets(offsets, E, S)) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  if (S == 0) return kOk;
+  const size_t ob = (size_t)S * N * (out_bf16 ? 2 : 4);
+  DeviceScope scope;
+  float* dy = static_cast<float*>(scope.alloc((size_t)S * N * 4, y));
+  int32_t* dof = static_cast<int32_t*>(scope.alloc((size_t)(E + 1) * 4, offsets));
+  float* dsc = static_cast<float*>(scope.alloc((size_t)E * 4, scale));
+  void* dout = scope.alloc(ob);
+  if (scope.failed()) return kDeviceFailed;
+  int rc = scale_groups_dev(dy, dof, dsc, dout, out_bf16, S, N, E, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  return scope.download(out, dout, ob) ? kOk : kDeviceFailed;
 }
 
 int tessera_gfx950_moe_swiglu_block_bf16_dev(const void* x, const void* wg, const void* wu, const void* wd,

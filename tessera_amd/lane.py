@@ -97,6 +97,12 @@ _SIGNATURES = {
     "tessera_gfx950_batched_gemm_strided_bf16_dev": [_c_vp] * 3 + [_c_int] * 4 + [_c_i64] * 3 + [_c_int, _c_vp],
     "tessera_gfx950_fake_quantize_nvfp4_f32": [_c_vp, _c_int, _c_int, _c_vp, _c_vp, _c_vp],
     "tessera_gfx950_fake_quantize_nvfp4_f32_dev": [_c_vp, _c_int, _c_int, _c_vp, _c_vp, _c_vp, _c_vp],
+    "tessera_gfx950_fpquant_f32": [_c_vp, _c_i64, _c_f, _c_int, _c_int, _c_vp],
+    "tessera_gfx950_fpquant_f32_dev": [_c_vp, _c_i64, _c_f, _c_int, _c_int, _c_vp, _c_vp],
+    "tessera_gfx950_fake_quantize_fp_f32": [_c_vp, _c_i64, _c_f, _c_int, _c_int, _c_f, _c_vp, _c_vp, _c_vp],
+    "tessera_gfx950_fake_quantize_fp_f32_dev": [_c_vp, _c_i64, _c_f, _c_int, _c_int, _c_f, _c_vp, _c_vp, _c_vp, _c_vp],
+    "tessera_gfx950_scale_groups_f32": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int],
+    "tessera_gfx950_scale_groups_f32_dev": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_silu_mul_bf16": [_c_vp, _c_vp, _c_vp, _c_i64],
     "tessera_gfx950_silu_mul_bf16_dev": [_c_vp, _c_vp, _c_vp, _c_i64, _c_vp],
     "tessera_gfx950_silu_mul_f16": [_c_vp, _c_vp, _c_vp, _c_i64],

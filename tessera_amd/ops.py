@@ -359,9 +359,13 @@ def grouped_gemm(x, weights, group_sizes, *, kind: str = "contiguous", alignment
     xa, w = _bits(x), _bits(weights)
     gs = np.asarray(group_sizes).astype(np.int64).reshape(-1)
     if quant is not None:
-        if str(quant).lower() == "nvfp4":
-            return _grouped_gemm_nvfp4(x, weights, xa, w, gs, alignment, out)
-        return _grouped_gemm_fp8(x, weights, xa, w, gs, quant, alignment, out)
+        scheme = GROUPED_QUANT_SCHEMES.get(str(quant).lower())
+        if scheme is None:
+            raise ValueError(f"grouped_gemm: quant {quant!r} has no grouped path; expected one of "
+                             f"{tuple(GROUPED_QUANT_SCHEMES)}")
+        if scheme == ("fp8_e4m3", "fp8_e4m3"):
+            return _grouped_gemm_fp8(x, weights, xa, w, gs, quant, alignment, out)
+        return _grouped_gemm_grid(x, weights, xa, w, gs, scheme, alignment, out)
     if alignment is not None:
         al = int(alignment)
         if al <= 0 or np.any(gs % al != 0):
@@ -420,12 +424,111 @@ def dequantize_nvfp4(x_q, scales=None, *, block_size: int = 16):
     return np.asarray(x_q, np.float32)
 
 
-def _grouped_gemm_nvfp4(x, weights, xa, w, gs, alignment, out):
-    """``quant="nvfp4"``: x and every expert's weight are rounded onto the NVFP4 grid along
-    their last axis (``compiler/grouped_layout.py:353-392``) on the device, and the grouped
-    product runs on the rounded values — which are exact in bf16 (at most six significant
-    bits), so the bf16 MFMA kernel with f32 accumulation computes the reference's f32
-    product of the dequantised operands up to summation order."""
+#: (max_normal, mantissa_bits, min_exp) of the per-tensor float grids
+#: (``runtime.py:16939-16946``): IEEE gradual underflow for fp8, the pure mantissa snap for
+#: fp6 and fp4.
+FP_FORMATS = {"e4m3": (448.0, 3, -6), "e5m2": (57344.0, 2, -14), "e2m3": (7.5, 3, -126), "e3m2": (28.0, 2, -126),
+              "e2m1": (6.0, 1, -126)}
+
+
+def _fp_round(x32: np.ndarray, fmt: str, scale=None, want_grid: bool = False):
+    """x f32 snapped to a per-tensor float grid on the device → (dequantised f32, grid values
+    as bf16 bits or None, scale f32)."""
+    mx, mant, min_exp = FP_FORMATS[fmt]
+    x32 = np.ascontiguousarray(x32, np.float32)
+    if x32.size == 0:
+        raise ValueError("quantize: empty array")
+    dq = np.empty(x32.shape, np.float32)
+    g16 = np.empty(x32.shape, np.uint16) if want_grid else None
+    s_out = np.zeros(1, np.float32)
+    _lane.check(_lane.load().tessera_gfx950_fake_quantize_fp_f32(
+        x32.ctypes.data, x32.size, mx, mant, min_exp, 0.0 if scale is None else float(scale), dq.ctypes.data,
+        g16.ctypes.data if want_grid else None, s_out.ctypes.data), "quantize_fp")
+    return dq, g16, np.float32(s_out[0])
+
+
+def fpquant(x, max_normal: float, mantissa_bits: int, min_exp: int) -> np.ndarray:
+    """x f32 snapped to the float grid ``(max_normal, mantissa_bits, min_exp)``: the native
+    lanes' grid kernel (``avx512_fpquant_f32.cpp:45-83``) on the device."""
+    x32 = np.ascontiguousarray(_unbox(x), np.float32)
+    out = np.empty(x32.shape, np.float32)
+    if x32.size:
+        _lane.check(_lane.load().tessera_gfx950_fpquant_f32(x32.ctypes.data, x32.size, float(max_normal), int(mantissa_bits),
+                                                            int(min_exp), out.ctypes.data), "fpquant")
+    return out
+
+
+def _quantize_per_tensor(x, fmt: str, formats, scale):
+    if fmt not in formats:
+        raise ValueError("format must be " + " or ".join(repr(f) for f in formats) + f"; got {fmt!r}")
+    x = _unbox(x)
+    x32 = x.to_float32() if isinstance(x, BF16Array) else np.asarray(x, np.float32)
+    dq, _, s = _fp_round(x32, fmt, scale)
+    return dq, s
+
+
+def quantize_fp6(x, *, format: str = "e3m2", scale=None):
+    """Per-tensor symmetric fp6 quantisation (``__init__.py:3411-3435``) →
+    ``(x_q_as_fp32, scale)``."""
+    return _quantize_per_tensor(x, format, ("e2m3", "e3m2"), scale)
+
+
+def quantize_fp4(x, *, format: str = "e2m1", scale=None):
+    """Per-tensor symmetric fp4 quantisation (``__init__.py:3446-3464``) →
+    ``(x_q_as_fp32, scale)``."""
+    return _quantize_per_tensor(x, format, ("e2m1",), scale)
+
+
+def dequantize_fp8(x_q, scale=None, *, format: str = "e4m3"):
+    """The quantisers already return rescaled values (``__init__.py:3376-3392``)."""
+    if format not in ("e4m3", "e5m2"):
+        raise ValueError(f"format must be 'e4m3' or 'e5m2'; got {format!r}")
+    return np.asarray(x_q, np.float32)
+
+
+def dequantize_fp6(x_q, scale=None, *, format: str = "e3m2"):
+    if format not in ("e2m3", "e3m2"):
+        raise ValueError(f"format must be 'e2m3' or 'e3m2'; got {format!r}")
+    return np.asarray(x_q, np.float32)
+
+
+def dequantize_fp4(x_q, scale=None, *, format: str = "e2m1"):
+    if format != "e2m1":
+        raise ValueError(f"format must be 'e2m1'; got {format!r}")
+    return np.asarray(x_q, np.float32)
+
+
+#: ``quant=`` spellings of the grouped product → (activation format, weight format)
+#: (``compiler/grouped_layout.py:320-332``)
+GROUPED_QUANT_SCHEMES = {
+    "fp8_e4m3": ("fp8_e4m3", "fp8_e4m3"), "fp8": ("fp8_e4m3", "fp8_e4m3"), "fp8_e5m2": ("fp8_e5m2", "fp8_e5m2"),
+    "nvfp4": ("nvfp4", "nvfp4"), "fp8xfp4": ("fp8_e4m3", "nvfp4"), "fp8_e4m3xnvfp4": ("fp8_e4m3", "nvfp4"),
+    "fp8_e5m2xnvfp4": ("fp8_e5m2", "nvfp4"),
+}
+
+
+def _grid_operand(a32: np.ndarray, dtype: str):
+    """One 2-D operand rounded as the reference's ``_qdq_2d`` does
+    (``compiler/grouped_layout.py:353-370``) → (values exact in bf16, as bits; the f32 factor
+    that turns them into the dequantised operand)."""
+    if dtype == "nvfp4":
+        if a32.shape[-1] % 16 != 0:
+            raise ValueError(f"last dim {a32.shape[-1]} must be divisible by block_size 16 for NVFP4")
+        return _nvfp4_round(a32)[1], np.float32(1.0)
+    _, g16, s = _fp_round(a32, "e5m2" if dtype == "fp8_e5m2" else "e4m3", want_grid=True)
+    return g16, s
+
+
+def _grouped_gemm_grid(x, weights, xa, w, gs, scheme, alignment, out):
+    """The quantised grouped product for every scheme but plain e4m3: x is rounded as one
+    tensor with the activation format and every expert's weight on its own with the weight
+    format (``compiler/grouped_layout.py:373-392``), on the device.  The rounded values
+    without their per-tensor scales are exact in bf16 (at most six significant bits), so one
+    launch of the bf16 grouped kernel with f32 accumulation forms their product, and the
+    scales (the activation's times expert e's) multiply the rows of group e afterwards: the
+    reference's f32 product of the dequantised operands up to summation order and one
+    rounding of the scale product."""
+    act, wt = scheme
     if alignment is not None:
         al = int(alignment)
         if al <= 0 or np.any(gs % al != 0):
@@ -434,24 +537,33 @@ def _grouped_gemm_nvfp4(x, weights, xa, w, gs, alignment, out):
         raise ValueError(f"grouped_gemm: x {xa.shape} / weights {w.shape} / group_sizes {gs.shape} disagree")
     T, K = xa.shape
     E, _, N = w.shape
-    for n_last in (K, N):                              # x is blocked along K, a weight along N
-        if n_last % 16 != 0:
-            raise ValueError(f"last dim {n_last} must be divisible by block_size 16 for NVFP4")
     off = _offsets(gs, T, "grouped_gemm")
     xf = x.to_float32() if isinstance(x, BF16Array) else _bf16.from_bits(xa).to_float32()
     wf = weights.to_float32() if isinstance(weights, BF16Array) else _bf16.from_bits(w).to_float32()
-    _, xq16, _ = _nvfp4_round(xf)
-    _, wq16, _ = _nvfp4_round(wf)                      # (E, K, N): blocks run along N, per expert row
+    xg, sx = _grid_operand(xf, act)
+    if wt == "nvfp4":                                   # blocks along N within one expert's row: one call
+        wg, sw = _grid_operand(wf, wt)[0], np.ones(E, np.float32)
+    else:
+        parts = [_grid_operand(wf[e], wt) for e in range(E)]
+        wg = np.stack([p[0] for p in parts])
+        sw = np.array([p[1] for p in parts], np.float32)
     f32 = out == "f32"
+    lib = _lane.load()
+    scales = (np.float32(sx) * sw).astype(np.float32)
+    if np.all(scales == np.float32(1.0)):
+        y = np.zeros((T, N), np.float32 if f32 else np.uint16)
+        name = "tessera_gfx950_grouped_gemm_bf16" + ("_f32" if f32 else "")
+        _lane.check(getattr(lib, name)(xg.ctypes.data, wg.ctypes.data, off.ctypes.data, y.ctypes.data, T, K, N, E),
+                    "grouped_gemm")
+        return y if f32 else y.view(BF16Array)
+    acc = np.zeros((T, N), np.float32)
+    _lane.check(lib.tessera_gfx950_grouped_gemm_bf16_f32(xg.ctypes.data, wg.ctypes.data, off.ctypes.data, acc.ctypes.data,
+                                                         T, K, N, E), "grouped_gemm")
     y = np.zeros((T, N), np.float32 if f32 else np.uint16)
-    name = "tessera_gfx950_grouped_gemm_bf16" + ("_f32" if f32 else "")
-    _lane.check(getattr(_lane.load(), name)(xq16.ctypes.data, wq16.ctypes.data, off.ctypes.data, y.ctypes.data, T, K, N, E),
-                "grouped_gemm")
+    if T:
+        _lane.check(lib.tessera_gfx950_scale_groups_f32(acc.ctypes.data, off.ctypes.data, scales.ctypes.data, y.ctypes.data,
+                                                        0 if f32 else 1, T, N, E), "grouped_gemm")
     return y if f32 else y.view(BF16Array)
-
-
-#: quant schemes of the reference's grouped GEMM that map onto the lane's e4m3 operand format
-_FP8_GROUPED_QUANT = ("fp8_e4m3", "fp8")
 
 
 def _grouped_gemm_fp8(x, weights, xa, w, gs, quant, alignment, out):
@@ -460,11 +572,6 @@ def _grouped_gemm_fp8(x, weights, xa, w, gs, quant, alignment, out):
     and each group is one e4m3 GEMM with f32 accumulation, scaled by both scales.
     The reference dequantises on the host and multiplies in f32; the products of two
     e4m3 values are exact in f32, so the two differ only in summation order."""
-    q = str(quant).lower()
-    if q not in _FP8_GROUPED_QUANT:
-        raise NotImplementedError(
-            f"grouped_gemm: quant={quant!r} is not implemented on the gfx950 lane — supported: "
-            f"{', '.join(_FP8_GROUPED_QUANT)}, nvfp4")
     if alignment is not None:
         al = int(alignment)
         if al <= 0 or np.any(gs % al != 0):
@@ -920,12 +1027,7 @@ def quantize_fp8_codes(x, *, scale=None):
 def quantize_fp8(x, *, format: str = "e4m3", scale=None):
     """Per-tensor symmetric fp8 quantisation → ``(x_q_as_fp32, scale)`` where
     ``x_q_as_fp32`` is the fp8-rounded value cast back to f32 (``grid * scale``)."""
-    if format not in ("e4m3", "e5m2"):
-        raise ValueError(f"format must be 'e4m3' or 'e5m2'; got {format!r}")
-    if format != "e4m3":
-        raise NotImplementedError("the gfx950 lane quantises to e4m3 (the GEMM operand format)")
-    codes, s = quantize_fp8_codes(x, scale=scale)
-    return e4m3_table()[codes] * np.float32(s), np.float32(s)
+    return _quantize_per_tensor(x, format, ("e4m3", "e5m2"), scale)
 
 
 def gemm_fp8(a_codes, b_codes, scale_a, scale_b, *, out: str = "bf16"):

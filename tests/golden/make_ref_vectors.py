@@ -62,6 +62,23 @@ def main() -> int:
                   -2.5 * 2.0 ** -9, 3.5 * 2.0 ** -9], np.float32),
     ])
     out["fpq_x"], out["fpq_y"] = x, co.ref_fpquant(x)
+    # the same kernel on the other grids of its format table (runtime.py:16939-16946):
+    # e5m2, the two fp6 grids and e2m1, each over magnitudes from far below the smallest
+    # step to beyond saturation, every grid point, every midpoint between neighbours (the
+    # ties), NaN and both zeros; plus E2M1 with the exponent floor at 0, the NVFP4 code grid
+    for tag, (mx, mant, min_exp) in {"e5m2": (57344.0, 2, -14), "e2m3": (7.5, 3, -126), "e3m2": (28.0, 2, -126),
+                                     "e2m1": (6.0, 1, -126), "e2m1_floor0": (6.0, 1, 0)}.items():
+        lo = max(min_exp, -20)
+        pts = [np.ldexp(1.0 + m / 2.0 ** mant, e) for e in range(lo - 2, int(np.log2(mx)) + 1) for m in range(2 ** mant)]
+        pts = np.array(sorted(p for p in pts if p <= mx), np.float64)
+        mids = (pts[1:] + pts[:-1]) / 2
+        mag = np.exp(rng.uniform(np.log(2.0 ** (lo - 6)), np.log(mx * 4), 768))
+        vals = np.concatenate([pts, mids, np.nextafter(mids.astype(np.float32), np.float32(0)),
+                               np.nextafter(mids.astype(np.float32), np.float32(np.inf)), mag,
+                               [0.0, -0.0, np.nan, mx, mx * 1.01, 1e30, np.ldexp(1.0, lo - 3), 1e-40, 2.0 ** -126]])
+        xs = (vals * rng.choice([-1.0, 1.0], vals.size)).astype(np.float32)
+        out[f"fpq_{tag}_x"], out[f"fpq_{tag}_y"] = xs, co.ref_fpquant(xs, mx, mant, min_exp)
+        out[f"fpq_{tag}_fmt"] = np.array([mx, mant, min_exp], np.float64)
     np.savez_compressed(Path(__file__).with_name("ref_vectors.npz"), **out)
     print("wrote", len(out), "arrays")
     return 0

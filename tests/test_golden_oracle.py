@@ -33,3 +33,15 @@ def test_flash_attn_golden(tag):
 
 def test_fpquant_golden():
     assert np.array_equal(orc.fpquant_grid(GOLD["fpq_x"]), GOLD["fpq_y"])
+
+
+FP_GRID_TAGS = ("e5m2", "e2m3", "e3m2", "e2m1", "e2m1_floor0")
+
+
+@pytest.mark.parametrize("tag", FP_GRID_TAGS)
+def test_fpquant_other_grids_golden(tag):
+    """e5m2, both fp6 grids and E2M1 (free exponent and the NVFP4 floor) against the
+    reference's compiled kernel: every grid point, every tie, subnormals, saturation, NaN."""
+    mx, mant, min_exp = GOLD[f"fpq_{tag}_fmt"]
+    got = orc.fpquant_grid(GOLD[f"fpq_{tag}_x"], float(mx), int(mant), int(min_exp))
+    assert np.array_equal(got, GOLD[f"fpq_{tag}_y"], equal_nan=True)

@@ -287,8 +287,8 @@ def test_grouped_gemm_fp8_quant(lane):
     assert orc.max_rel_err(got, orc.grouped_gemm(x.to_float32(), w.to_float32(), sizes, store=False)) <= 3e-2 * 4
     stored = ops.grouped_gemm(x, w, sizes, quant="fp8")
     assert np.array_equal(np.asarray(stored, np.uint16), np.asarray(b16.from_float32(got), np.uint16))
-    with pytest.raises(NotImplementedError):
-        ops.grouped_gemm(x, w, sizes, quant="fp8_e5m2")          # the lane's fp8 operand format is e4m3
+    with pytest.raises(ValueError):
+        ops.grouped_gemm(x, w, sizes, quant="fp9")                # not one of the reference's schemes
 
 
 def test_single_expert_reduces_to_dense_swiglu(lane):

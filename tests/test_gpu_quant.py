@@ -244,3 +244,92 @@ def test_grouped_gemm_nvfp4(lane, gs):
     with pytest.raises(ValueError):
         ops.grouped_gemm(b16.from_float32(np.zeros((T, 24), np.float32)),        # K = 24 is not whole blocks
                          b16.from_float32(np.zeros((E, 24, N), np.float32)), gs, quant="nvfp4")
+
+
+FP_FORMATS = {"e4m3": (448.0, 3, -6), "e5m2": (57344.0, 2, -14), "e2m3": (7.5, 3, -126), "e3m2": (28.0, 2, -126),
+              "e2m1": (6.0, 1, -126)}
+
+
+@pytest.mark.parametrize("fmt", sorted(FP_FORMATS))
+def test_float_grid_kernel_matches_oracle_bit_for_bit(lane, fmt):
+    """The device grid rounding against the oracle (itself pinned on the reference's compiled
+    kernel for every one of these formats): magnitudes from the denormals to beyond
+    saturation, every tie, NaN and both zeros; through the 16-byte path and the element tail."""
+    mx, mant, min_exp = FP_FORMATS[fmt]
+    rng = np.random.default_rng(mant * 100 - min_exp)
+    lo = max(min_exp, -20)
+    pts = np.array(sorted({np.ldexp(1.0 + m / 2.0 ** mant, e) for e in range(lo - 2, int(np.log2(mx)) + 1)
+                           for m in range(2 ** mant)}), np.float64)
+    pts = pts[pts <= mx]
+    mids = ((pts[1:] + pts[:-1]) / 2).astype(np.float32)
+    mag = np.exp(rng.uniform(np.log(1e-42), np.log(mx * 8), 1 << 16))
+    vals = np.concatenate([pts, mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(np.inf)), mag,
+                           [0.0, -0.0, np.nan, mx, mx * 1.01, 1e30, np.inf, 1e-40, 2.0 ** -126, 2.0 ** -149]])
+    x = (vals * rng.choice([-1.0, 1.0], vals.size)).astype(np.float32)
+    for xs in (x, x[1:], x[:7]):                                       # aligned, unaligned, tail only
+        got = ops.fpquant(xs, mx, mant, min_exp)
+        assert np.array_equal(got, orc.fpquant_grid(xs, mx, mant, min_exp), equal_nan=True)
+    # a snapped value is a fixed point
+    g = ops.fpquant(x, mx, mant, min_exp)
+    assert np.array_equal(ops.fpquant(g, mx, mant, min_exp), g, equal_nan=True)
+
+
+@pytest.mark.parametrize("tag", ["e5m2", "e2m3", "e3m2", "e2m1", "e2m1_floor0"])
+def test_float_grid_kernel_golden(lane, tag):
+    from pathlib import Path
+    gold = np.load(Path(__file__).parent / "golden" / "ref_vectors.npz")
+    mx, mant, min_exp = gold[f"fpq_{tag}_fmt"]
+    got = ops.fpquant(gold[f"fpq_{tag}_x"], float(mx), int(mant), int(min_exp))
+    assert np.array_equal(got, gold[f"fpq_{tag}_y"], equal_nan=True)
+
+
+@pytest.mark.parametrize("fmt", sorted(FP_FORMATS))
+def test_per_tensor_float_quantisers_match_oracle(lane, fmt):
+    """ops.quantize_fp8 / fp6 / fp4: automatic and given scale, values and scale bit for bit;
+    the bf16 form of the unscaled grid values is exact."""
+    from tessera_amd import lane as ln
+    q = {"e4m3": ops.quantize_fp8, "e5m2": ops.quantize_fp8, "e2m3": ops.quantize_fp6, "e3m2": ops.quantize_fp6,
+         "e2m1": ops.quantize_fp4}[fmt]
+    rng = np.random.default_rng(len(fmt) + FP_FORMATS[fmt][1])
+    x = (rng.standard_normal((257, 129)) * np.exp(rng.standard_normal((257, 1)) * 3)).astype(np.float32)
+    for scale in (None, 0.037):
+        dq, s = q(x, format=fmt, scale=scale)
+        odq, ogrid, os_ = orc.quantize_fp(x, fmt, scale)
+        assert s == os_ and dq.shape == x.shape
+        assert np.array_equal(dq.view(np.uint32) & 0x7FFFFFFF, odq.view(np.uint32) & 0x7FFFFFFF) and np.array_equal(dq, odq)
+        mx, mant, min_exp = FP_FORMATS[fmt]
+        g16 = np.empty(x.shape, np.uint16)
+        ln.check(ln.load().tessera_gfx950_fake_quantize_fp_f32(x.ctypes.data, x.size, mx, mant, min_exp, float(s), None,
+                                                               g16.ctypes.data, None), "grid")
+        assert np.array_equal((g16.astype(np.uint32) << 16).view(np.float32), ogrid)
+    assert np.array_equal(ops.quantize_fp8(np.zeros(5, np.float32), format="e5m2")[0], np.zeros(5, np.float32))
+    with pytest.raises(ValueError):
+        q(x, format="e9m9")
+
+
+@pytest.mark.parametrize("quant", ["fp8_e5m2", "fp8xfp4", "fp8_e4m3xnvfp4", "fp8_e5m2xnvfp4", "fp8", "nvfp4"])
+@pytest.mark.parametrize("gs", [[5, 3, 4], [300, 0, 77, 1000]])
+def test_grouped_gemm_quant_schemes(lane, quant, gs):
+    """Every quant= scheme of the reference's grouped product against the oracle's f64 product of
+    the same quantised operands."""
+    rng = np.random.default_rng(sum(gs) + len(quant))
+    small = sum(gs) < 100
+    T, K, N, E = sum(gs), (64 if small else 512), (16 if small else 256), len(gs)
+    x = b16.from_float32((rng.standard_normal((T, K)) * 3).astype(np.float32))
+    w = b16.from_float32((rng.standard_normal((E, K, N)) * np.array([0.1, 1.0, 7.0, 0.5][:E])[:, None, None]).astype(np.float32))
+    ref = orc.grouped_gemm_quant(x.to_float32(), w.to_float32(), gs, quant)
+    got = ops.grouped_gemm(x, w, gs, quant=quant, out="f32")
+    # (plain e4m3 runs on the fp8 matrix instruction, whose sum over one instruction's 64
+    # products keeps fewer bits than an f32 sum; the other schemes run on the bf16 one)
+    tol = 1e-4 if quant == "fp8" else 1e-5
+    assert got.shape == (T, N) and orc.max_rel_err(got, ref) <= tol
+    stored = ops.grouped_gemm(x, w, gs, quant=quant)
+    assert orc.max_rel_err(stored.to_float32(), ref) <= 2.0 ** -8 + tol
+    full = np.zeros((T, N))
+    off = 0
+    for e, n in enumerate(gs):
+        full[off:off + n] = x.to_float32()[off:off + n].astype(np.float64) @ w.to_float32()[e].astype(np.float64)
+        off += n
+    assert np.linalg.norm(got - full) / np.linalg.norm(full) < 0.25
+    with pytest.raises(ValueError):
+        ops.grouped_gemm(x, w, gs, quant="int3")
