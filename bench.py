@@ -350,6 +350,13 @@ def bench_quant(lane, steps, warmup, check=True):
     _, ev = _timed(lane, q_e4, steps, warmup)
     ebytes = 9.0 * M * K
     out["quantize_e4m3_tensor_4096x8192"] = {"ms": ev, "gbs": ebytes / ev / 1e6, "frac_hbm_peak": ebytes / ev / 1e6 / PEAK_HBM_GBS}
+    # the per-tensor float-grid kernel (e5m2 here): absmax pass, then read f32 / write the dequantised f32
+    _, ev = _timed(lane, lambda: lane.check(lib.tessera_gfx950_fake_quantize_fp_f32_dev(
+        xf.ptr, M * K, ctypes.c_float(57344.0), 2, -14, ctypes.c_float(0.0), dd.ptr, None, None, None), "quantize_fp"),
+        steps, warmup)
+    gbytes = 12.0 * M * K
+    out["fake_quantize_e5m2_tensor_4096x8192"] = {"ms": ev, "gbs": gbytes / ev / 1e6,
+                                                  "frac_hbm_peak": gbytes / ev / 1e6 / PEAK_HBM_GBS}
     lane.synchronize()
     scale_a = float(sx.download((1,), np.float32)[0])
     scale_b = float(sw.download((1,), np.float32)[0])

@@ -333,3 +333,51 @@ def test_grouped_gemm_quant_schemes(lane, quant, gs):
     assert np.linalg.norm(got - full) / np.linalg.norm(full) < 0.25
     with pytest.raises(ValueError):
         ops.grouped_gemm(x, w, gs, quant="int3")
+
+
+def test_float_grid_and_group_scaling_on_device_buffers(lane):
+    """The device-pointer forms: e5m2 with the automatic scale into f32 and bf16-grid outputs, the
+    bare grid kernel, and the per-group scaling with f32 and bf16 results."""
+    import ctypes
+    from tessera_amd import lane as ln
+    lib = ln.load()
+    rng = np.random.default_rng(77)
+    x = (rng.standard_normal(50003) * 11).astype(np.float32)
+    dx = ln.DeviceBuffer.from_host(x)
+    ddq, dg, dsc, dout = ln.DeviceBuffer(x.size * 4), ln.DeviceBuffer(x.size * 2), ln.DeviceBuffer(4), ln.DeviceBuffer(x.size * 4)
+    try:
+        ln.check(lib.tessera_gfx950_fake_quantize_fp_f32_dev(dx.ptr, x.size, ctypes.c_float(57344.0), 2, -14, ctypes.c_float(0.0),
+                                                             ddq.ptr, dg.ptr, dsc.ptr, None), "fake_quantize_fp")
+        ln.check(lib.tessera_gfx950_fpquant_f32_dev(dx.ptr, x.size, ctypes.c_float(6.0), 1, 0, dout.ptr, None), "fpquant")
+        ln.synchronize()
+        odq, ogrid, oscale = orc.quantize_fp(x, "e5m2")
+        assert dsc.download((1,), np.float32)[0] == oscale
+        assert np.array_equal(ddq.download(x.shape, np.float32), odq)
+        assert np.array_equal((dg.download(x.shape, np.uint16).astype(np.uint32) << 16).view(np.float32), ogrid)
+        assert np.array_equal(dout.download(x.shape, np.float32), orc.fpquant_grid(x, 6.0, 1, 0))
+        # bad formats are refused before anything is launched
+        assert lib.tessera_gfx950_fpquant_f32_dev(dx.ptr, x.size, ctypes.c_float(6.0), 24, 0, dout.ptr, None) == 1
+        assert lib.tessera_gfx950_fpquant_f32_dev(dx.ptr, x.size, ctypes.c_float(-1.0), 1, 0, dout.ptr, None) == 1
+        assert lib.tessera_gfx950_fpquant_f32_dev(dx.ptr, x.size, ctypes.c_float(6.0), 1, -127, dout.ptr, None) == 1
+    finally:
+        for b in (dx, ddq, dg, dsc, dout):
+            b.close()
+    S, N, E = 37, 24, 5
+    y = rng.standard_normal((S, N)).astype(np.float32)
+    off = np.array([0, 10, 10, 11, 30, 37], np.int32)
+    sc = rng.uniform(0.1, 3.0, E).astype(np.float32)
+    ref = y * np.repeat(sc, np.diff(off))[:, None]
+    dy, dof, dsc2 = ln.DeviceBuffer.from_host(y), ln.DeviceBuffer.from_host(off), ln.DeviceBuffer.from_host(sc)
+    d32, d16 = ln.DeviceBuffer(S * N * 4), ln.DeviceBuffer(S * N * 2)
+    try:
+        ln.check(lib.tessera_gfx950_scale_groups_f32_dev(dy.ptr, dof.ptr, dsc2.ptr, d32.ptr, 0, S, N, E, None), "scale_groups")
+        ln.check(lib.tessera_gfx950_scale_groups_f32_dev(dy.ptr, dof.ptr, dsc2.ptr, d16.ptr, 1, S, N, E, None), "scale_groups")
+        ln.synchronize()
+        assert np.array_equal(d32.download((S, N), np.float32), ref)
+        assert np.array_equal(d16.download((S, N), np.uint16), b16.from_float32(ref).view(np.uint16).reshape(S, N))
+    finally:
+        for b in (dy, dof, dsc2, d32, d16):
+            b.close()
+    out = np.empty((S, N), np.float32)
+    bad = off.copy(); bad[2] = 12                        # offsets must not decrease
+    assert lib.tessera_gfx950_scale_groups_f32(y.ctypes.data, bad.ctypes.data, sc.ctypes.data, out.ctypes.data, 0, S, N, E) == 1
