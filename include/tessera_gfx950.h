@@ -535,6 +535,16 @@ int tessera_gfx950_grouped_gemm_bf16_dev(const void* x, const void* w, const int
                                          int S, int K, int N, int E, void* stream);
 int tessera_gfx950_grouped_gemm_bf16_f32_dev(const void* x, const void* w, const int32_t* offsets, void* y,
                                              int S, int K, int N, int E, void* stream);
+/* The same on f16 storage (the reference's grouped product takes any float dtype and applies the
+ * storage rule: python/tessera/__init__.py:291-351, 5783-5855). */
+int tessera_gfx950_grouped_gemm_f16(const void* x, const void* w, const int32_t* offsets, void* y,
+                                    int S, int K, int N, int E);
+int tessera_gfx950_grouped_gemm_f16_f32(const void* x, const void* w, const int32_t* offsets, void* y,
+                                        int S, int K, int N, int E);
+int tessera_gfx950_grouped_gemm_f16_dev(const void* x, const void* w, const int32_t* offsets, void* y,
+                                        int S, int K, int N, int E, void* stream);
+int tessera_gfx950_grouped_gemm_f16_f32_dev(const void* x, const void* w, const int32_t* offsets, void* y,
+                                            int S, int K, int N, int E, void* stream);
 /* The per-tensor scales of the reference's quantised grouped product
  * (python/tessera/compiler/grouped_layout.py:373-392: x quantised as one tensor, each expert's
  * weight on its own), applied after the product of the unscaled grid values:

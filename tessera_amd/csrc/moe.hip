@@ -696,7 +696,7 @@ bool bad_grouped(int S, int K, int N, int E) { return S < 0 || K <= 0 || N <= 0 
 // activation has to lie inside it.
 bool gather_out_of_buffer_range(int rows, int K) { return (long)rows * K * 2 > (long)kBufferRange - 16; }
 
-template <int EPI>
+template <int EPI, class T = BF16>
 int grouped_dev(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K, int N, int E,
                 hipStream_t s) {
   if (bad_grouped(S, K, N, E) || !w || !offsets || (S > 0 && (!x || !y))) return kBadShape;
@@ -711,7 +711,7 @@ int grouped_dev(const void* x, const void* w, const int32_t* offsets, void* y, i
   p.strideB = (long)K * N;
   p.offsets = offsets;
   p.groups = E;
-  return launch_gemm16_grouped<BF16, EPI>(p, s);
+  return launch_gemm16_grouped<T, EPI>(p, s);
 }
 
 // `gather` (device int32[S], or null): row m of the block's input is x[gather[m]], i.e.
@@ -900,7 +900,7 @@ bool bad_offsets(const int32_t* offsets, int E, int S) {
   return false;
 }
 
-template <int EPI>
+template <int EPI, class T = BF16>
 int grouped_host(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K, int N, int E) {
   if (bad_grouped(S, K, N, E) || !w || !offsets || (S > 0 && (!x || !y))) return kBadShape;
   if (bad_offsets(offsets, E, S)) return kBadShape;
@@ -913,7 +913,7 @@ int grouped_host(const void* x, const void* w, const int32_t* offsets, void* y, 
   int32_t* dof = static_cast<int32_t*>(scope.alloc((size_t)(E + 1) * 4, offsets));
   void* dy = scope.alloc((size_t)S * N * dsz);
   if (scope.failed()) return kDeviceFailed;
-  int rc = grouped_dev<EPI>(dx, dw, dof, dy, S, K, N, E, nullptr);
+  int rc = grouped_dev<EPI, T>(dx, dw, dof, dy, S, K, N, E, nullptr);
   if (rc != kOk) return rc;
   if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
   return scope.download(y, dy, (size_t)S * N * dsz) ? kOk : kDeviceFailed;
@@ -1201,6 +1201,23 @@ int tessera_gfx950_grouped_gemm_bf16(const void* x, const void* w, const int32_t
 int tessera_gfx950_grouped_gemm_bf16_f32(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K,
                                          int N, int E) {
   return grouped_host<EPI_F32>(x, w, offsets, y, S, K, N, E);
+}
+
+int tessera_gfx950_grouped_gemm_f16_dev(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K,
+                                        int N, int E, void* stream) {
+  return grouped_dev<EPI_STORE16, F16>(x, w, offsets, y, S, K, N, E, as_stream(stream));
+}
+int tessera_gfx950_grouped_gemm_f16_f32_dev(const void* x, const void* w, const int32_t* offsets, void* y, int S,
+                                            int K, int N, int E, void* stream) {
+  return grouped_dev<EPI_F32, F16>(x, w, offsets, y, S, K, N, E, as_stream(stream));
+}
+int tessera_gfx950_grouped_gemm_f16(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K, int N,
+                                    int E) {
+  return grouped_host<EPI_STORE16, F16>(x, w, offsets, y, S, K, N, E);
+}
+int tessera_gfx950_grouped_gemm_f16_f32(const void* x, const void* w, const int32_t* offsets, void* y, int S, int K,
+                                        int N, int E) {
+  return grouped_host<EPI_F32, F16>(x, w, offsets, y, S, K, N, E);
 }
 
 int tessera_gfx950_scale_groups_f32_dev(const float* y, const int32_t* offsets, const float* scale, void* out,

@@ -171,6 +171,10 @@ _SIGNATURES = {
     "tessera_gfx950_grouped_gemm_bf16_f32": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int],
     "tessera_gfx950_grouped_gemm_bf16_dev": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_grouped_gemm_bf16_f32_dev": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_vp],
+    "tessera_gfx950_grouped_gemm_f16": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int],
+    "tessera_gfx950_grouped_gemm_f16_f32": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int],
+    "tessera_gfx950_grouped_gemm_f16_dev": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_vp],
+    "tessera_gfx950_grouped_gemm_f16_f32_dev": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_moe_swiglu_block_bf16": [_c_vp] * 6 + [_c_int] * 5,
     "tessera_gfx950_moe_swiglu_block_bf16_dev": [_c_vp] * 7 + [_c_int] * 5 + [_c_vp],
     "tessera_gfx950_moe_swiglu_block_gather_bf16_dev": [_c_vp] * 8 + [_c_int] * 6 + [_c_vp],

@@ -354,11 +354,12 @@ def grouped_gemm(x, weights, group_sizes, *, kind: str = "contiguous", alignment
             f"grouped_gemm: kind={kind!r} is not implemented — supported: "
             f"{', '.join(_SUPPORTED_GROUPED_KINDS)}")
     x, weights = _unbox(x), _unbox(weights)
-    if _storage(x, weights) != "bf16":
-        raise ValueError("grouped_gemm on the gfx950 lane takes bf16 storage")
+    st = _storage(x, weights)
     xa, w = _bits(x), _bits(weights)
     gs = np.asarray(group_sizes).astype(np.int64).reshape(-1)
     if quant is not None:
+        if st != "bf16":
+            raise ValueError("grouped_gemm(quant=) on the gfx950 lane takes bf16 storage")
         scheme = GROUPED_QUANT_SCHEMES.get(str(quant).lower())
         if scheme is None:
             raise ValueError(f"grouped_gemm: quant {quant!r} has no grouped path; expected one of "
@@ -381,10 +382,10 @@ def grouped_gemm(x, weights, group_sizes, *, kind: str = "contiguous", alignment
     off = _offsets(gs, T, "grouped_gemm")
     f32 = out == "f32"
     y = np.zeros((T, N), np.float32 if f32 else np.uint16)
-    name = "tessera_gfx950_grouped_gemm_bf16" + ("_f32" if f32 else "")
+    name = f"tessera_gfx950_grouped_gemm_{st}" + ("_f32" if f32 else "")
     _lane.check(getattr(_lane.load(), name)(xa.ctypes.data, w.ctypes.data, off.ctypes.data, y.ctypes.data, T, K, N, E),
                 "grouped_gemm")
-    return y if f32 else y.view(BF16Array)
+    return y if f32 else _wrap(y, st)
 
 
 def _nvfp4_round(x32: np.ndarray, want_scales: bool = False):

@@ -196,6 +196,29 @@ def test_grouped_gemm(lane, sizes, K, N):
         ops.grouped_gemm(b16.from_float32(x), b16.from_float32(w), sizes, kind="masked")
 
 
+@pytest.mark.parametrize("sizes,K,N", [
+    ([5, 0, 300, 1, 64, 0, 257, 13], 128, 256),
+    ([100, 200, 300, 400], 1408, 512),
+    ([3, 5], 24, 40),
+    ([2, 1, 4], 30, 18),                                  # off the 16-byte grid: the per-element kernel
+])
+def test_grouped_gemm_f16_storage(lane, sizes, K, N):
+    """The grouped product on f16 storage: f32 accumulation, result stored back as f16."""
+    E, T = len(sizes), int(sum(sizes))
+    rng = np.random.default_rng(K * N + 1)
+    x = rng.standard_normal((T, K)).astype(np.float16)
+    w = (rng.standard_normal((E, K, N)) / np.sqrt(K)).astype(np.float16)
+    ref = orc.grouped_gemm(x.astype(np.float32), w.astype(np.float32), sizes, dtype="f16", store=False)
+    got = ops.grouped_gemm(x, w, sizes, out="f32")
+    assert got.dtype == np.float32 and orc.max_rel_err(got, ref) <= 1e-5
+    stored = ops.grouped_gemm(x, w, sizes)
+    assert stored.dtype == np.float16 and np.array_equal(stored, got.astype(np.float16))
+    with pytest.raises(ValueError):
+        ops.grouped_gemm(x, b16.from_float32(w.astype(np.float32)), sizes)        # mixed storage
+    with pytest.raises(ValueError):
+        ops.grouped_gemm(x, w, sizes, quant="fp8")                                # the quantised paths take bf16
+
+
 def test_grouped_gemm_more_than_64_experts(lane):
     """The tile kernel looks its expert up 64 groups at a time: 150 experts of 0..300
     rows cross that boundary twice, with empty groups and short last tiles among them."""
