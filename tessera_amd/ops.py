@@ -81,13 +81,50 @@ def _unbox(x):
 # ---------------------------------------------------------------------------
 
 
-def gemm(A, B, *, out: str = "storage"):
+#: activations of ``ops.fused_epilogue`` (``__init__.py:2665-2670``; anything else is the identity there)
+_EPILOGUE_ACTIVATIONS = {"linear": "none", "none": "none", None: "none", "gelu": "gelu", "relu": "relu", "silu": "silu"}
+
+
+def _gemm_with_epilogue(A, B, epilogue: dict, out: str):
+    """``gemm(A, B, epilogue={...})`` (``__init__.py:239-248, 2658-2675``): bias add and
+    activation on the f32 product, inside the GEMM kernel, before the storage rule rounds."""
+    ep = dict(epilogue)
+    bias = ep.pop("bias", None)
+    act = ep.pop("activation", "linear")
+    for key in ("residual", "cast_dtype"):
+        if ep.pop(key, None) is not None:
+            raise NotImplementedError(f"gemm(epilogue=): {key!r} is not fused on the gfx950 lane")
+    if ep.pop("dropout_p", 0.0):
+        raise NotImplementedError("gemm(epilogue=): dropout is not fused on the gfx950 lane")
+    if act not in _EPILOGUE_ACTIVATIONS:
+        act = "linear"                                  # the reference applies no activation for other names
+    A, B = _unbox(A), _unbox(B)
+    st = _storage(A, B)
+    if _bits(B).ndim != 2:
+        raise NotImplementedError("gemm(epilogue=) with a batched B is not fused on the gfx950 lane")
+    a = _bits(A)
+    N = _bits(B).shape[1]
+    if bias is not None:
+        bias = np.ascontiguousarray(np.broadcast_to(np.asarray(_unbox(bias), np.float32), (N,)))
+    a2 = _wrap(np.ascontiguousarray(a.reshape(-1, a.shape[-1])), st)
+    d = fused_gemm(a2, B, bias, _EPILOGUE_ACTIVATIONS[act]).reshape(a.shape[:-1] + (N,))
+    if out == "f32":
+        return d
+    return _bf16.from_float32(d) if st == "bf16" else d.astype(np.float16)
+
+
+def gemm(A, B, epilogue=None, *, out: str = "storage"):
     """``A @ B`` with f32 accumulate.  16-bit operands; leading dims of ``A`` (and
     of ``B`` when it is not rank 2) are batch dims and must match.
 
     ``out="storage"`` stores the result in the operands' storage dtype (the
     ``ops.gemm`` rule for reduced-precision operands); ``out="f32"`` returns the
-    f32 accumulators (the executors' contract)."""
+    f32 accumulators (the executors' contract).  ``epilogue`` is the reference's
+    ``fused_epilogue`` dict (``bias``, ``activation``), applied to the f32 product."""
+    if out not in ("storage", "f32"):
+        raise ValueError("out must be 'storage' or 'f32'")
+    if epilogue:
+        return _gemm_with_epilogue(A, B, epilogue, out)
     A, B = _unbox(A), _unbox(B)
     st = _storage(A, B)
     a, b = _bits(A), _bits(B)

@@ -137,3 +137,22 @@ def test_executor_fused_epilogue_op(lane):
     res = ex.launch(ex.make_artifact("tessera.matmul", ["a", "b"], ["a", "b"], "gfx950_gemm",
                                      kwargs={"activation": "relu"}), (ai, np.ones((16, 8), np.int8)))
     assert not res["ok"] and "float-only" in res["reason"]
+
+
+@pytest.mark.parametrize("act", ["linear", "gelu", "relu", "silu"])
+def test_gemm_epilogue_keyword(lane, act):
+    """ops.gemm(A, B, epilogue={"bias", "activation"}): the reference applies the epilogue to the
+    f32 product and rounds to the storage dtype afterwards."""
+    rng = np.random.default_rng(len(act))
+    a = b16.from_float32(rng.standard_normal((3, 70, 96)).astype(np.float32))       # leading dims fold into M
+    b = b16.from_float32((rng.standard_normal((96, 136)) / 8).astype(np.float32))
+    bias = rng.standard_normal(136).astype(np.float32)
+    chain = ["bias"] + ([] if act == "linear" else [act])
+    ref = orc.fused_epilogue(a.to_float32().reshape(-1, 96), b.to_float32(), bias, chain).reshape(3, 70, 136)
+    got32 = ops.gemm(a, b, epilogue={"bias": bias, "activation": act}, out="f32")
+    assert got32.shape == (3, 70, 136) and orc.max_rel_err(got32, ref) <= 2e-5
+    got = ops.gemm(a, b, epilogue={"bias": bias, "activation": act})
+    assert np.array_equal(got.to_float32(), orc.round_to_storage(got32, "bf16"))
+    assert np.array_equal(np.asarray(ops.gemm(a, b, epilogue={}), np.uint16), np.asarray(ops.gemm(a, b), np.uint16))
+    with pytest.raises(NotImplementedError):
+        ops.gemm(a, b, epilogue={"residual": np.zeros((3, 70, 136), np.float32)})
