@@ -464,8 +464,13 @@ int tessera_gfx950_moe_route_f32_noalloc_dev(const float* scores, int T, int E, 
  * (python/tessera/models/moe_routing.py:54-113, python/tessera/stdlib/moe.py:79-134).
  * With router_logits (f32 [T,E]; k <= 64): route_top_k — the k largest LOGITS per token,
  * descending, ties to the lowest expert id; weights = softmax over the k selected logits
- * (normalize != 0) or 1/k each (normalize == 0); written to expert_ids / weights ([T,k],
- * rank order).  With router_logits NULL the selection is given instead (given_expert_ids
+ * (normalize == 1) or 1/k each (normalize == 0); written to expert_ids / weights ([T,k],
+ * rank order).  normalize == 2 / 3 select distributed.moe.route_tokens' router instead
+ * (python/tessera/distributed/moe.py:164-176): softmax over all E experts, the k largest
+ * probabilities, renormalised over the k (2; for k > 1) or as they are (3) — the token-major
+ * view (expert_ids, weights, kept_mask) of the routing tessera_gfx950_moe_route_f32 packs,
+ * which is what RoutingResult.assignment / weights are made of (any k <= E).  Other values
+ * of normalize are rc 1.  With router_logits NULL the selection is given instead (given_expert_ids
  * int32 [T,k] with values in [0,E) — anything else is rc 1 in the host form —
  * given_weights f32 [T,k] or NULL): plan_packing / plan_dispatch on a caller's routing.
  * Then the plan: slots are taken in token-major order, an expert keeps its first

@@ -338,18 +338,31 @@ int route_dev(const float* scores, int T, int E, int k, int normalize, int capac
 // route_top_k (or a given selection) + the packing plan with its token-major outputs.
 int plan_dev(const float* logits, const int32_t* given_ids, const float* given_weights, int T, int E, int k,
              int router, int capacity, const PlanOutputs& plan, int32_t* token_of_slot, int32_t* expert_of_slot,
-             float* combine_weights, int32_t* group_sizes, int32_t* group_offsets, int32_t* num_slots, hipStream_t s) {
+             float* combine_weights, int32_t* group_sizes, int32_t* group_offsets, int32_t* num_slots, hipStream_t s,
+             int renormalize = 0) {
   if (T <= 0 || E <= 0 || k <= 0 || k > E || E > kMaxExperts || (long)T * k > 0x7fffffffL || !group_sizes ||
       !group_offsets)
     return kBadShape;
-  if (logits ? (router != kRouterSoftmaxSelected && router != kRouterUniform) || k > 64
-             : (!given_ids || (combine_weights && !given_weights)))
+  if (logits ? (router != kRouterSoftmaxAll && k > 64) : (!given_ids || (combine_weights && !given_weights)))
     return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
   char* ws = static_cast<char*>(stream_workspace(s, route_workspace_bytes(T * k, E)));
   if (!ws) return kDeviceFailed;
-  return route_launch(logits, T, E, k, 0, capacity, router, token_of_slot, expert_of_slot, combine_weights,
+  return route_launch(logits, T, E, k, renormalize, capacity, router, token_of_slot, expert_of_slot, combine_weights,
                       group_sizes, group_offsets, num_slots, ws, s, plan, given_ids, given_weights);
+}
+
+// The `normalize` argument of the plan entry points: 0 = 1/k each, 1 = softmax over the selected
+// logits (both route_top_k), 2 / 3 = route_tokens' router (softmax over all experts, the k
+// largest probabilities), renormalised over the k (2) or as they are (3).
+bool plan_router(int normalize, int* router, int* renormalize) {
+  *renormalize = normalize == 2;
+  switch (normalize) {
+    case 0: *router = kRouterUniform; return true;
+    case 1: *router = kRouterSoftmaxSelected; return true;
+    case 2: case 3: *router = kRouterSoftmaxAll; return true;
+    default: return false;
+  }
 }
 
 // Device address of `scratch` on the current device, looked up once per device.
@@ -1047,9 +1060,10 @@ int tessera_gfx950_moe_plan_f32_dev(const float* router_logits, const int32_t* g
   plan.kept_mask = kept_mask;
   plan.sort_perm = sort_perm;
   plan.inverse_perm = inverse_perm;
-  return plan_dev(router_logits, given_expert_ids, given_weights, T, E, k,
-                  normalize ? kRouterSoftmaxSelected : kRouterUniform, capacity, plan, token_of_slot, expert_of_slot,
-                  combine_weights, group_sizes, group_offsets, num_slots, as_stream(stream));
+  int router = 0, renorm = 0;
+  if (!plan_router(normalize, &router, &renorm)) return kBadShape;
+  return plan_dev(router_logits, given_expert_ids, given_weights, T, E, k, router, capacity, plan, token_of_slot,
+                  expert_of_slot, combine_weights, group_sizes, group_offsets, num_slots, as_stream(stream), renorm);
 }
 
 int tessera_gfx950_moe_plan_f32(const float* router_logits, const int32_t* given_expert_ids,
@@ -1061,7 +1075,7 @@ int tessera_gfx950_moe_plan_f32(const float* router_logits, const int32_t* given
   if (T <= 0 || E <= 0 || k <= 0 || k > E || E > kMaxExperts || (long)T * k > 0x7fffffffL || !group_sizes ||
       !group_offsets)
     return kBadShape;
-  if (router_logits ? k > 64 : !given_expert_ids) return kBadShape;
+  if (router_logits ? (normalize < 0 || normalize > 3 || (normalize < 2 && k > 64)) : !given_expert_ids) return kBadShape;
   const size_t S = (size_t)T * k;
   if (!router_logits)
     for (size_t i = 0; i < S; ++i)

@@ -30,7 +30,7 @@ from __future__ import annotations
 import ctypes
 import math
 from dataclasses import dataclass
-from typing import Optional
+from typing import NamedTuple, Optional
 
 import numpy as np
 
@@ -347,21 +347,50 @@ def flash_attn_backward(dO, Q, K, V, scale=None, causal: bool = False):
     return dq, dk, dv
 
 
-def flash_attn(Q, K=None, V=None, scale=None, causal: bool = False, *, return_lse: bool = False,
-               out: str = "storage", window: int = 0, logit_softcap: float = 0.0, attn_bias=None):
+def flash_attn(Q, K=None, V=None, scale=None, causal: bool = False, cache=None, dropout_p: float = 0.0, params=None,
+               deterministic=None, seed=None, attn_bias=None, kv_state=None, *, return_lse: bool = False,
+               out: str = "storage", window: int = 0, logit_softcap: float = 0.0):
     """``softmax(scale * Q K^T, causal) V``.  Q/K/V ``[..., H, S, D]`` 16-bit; the
     causal mask is bottom-right aligned (key ``j`` visible to query ``i`` iff
     ``j <= i + max(Sk - Sq, 0)``).  Head counts must match (as in the reference).
     ``attn_bias`` (f32, broadcastable to ``[..., H, Sq, Sk]``) is added to the scaled
-    (and, with ``logit_softcap``, capped) scores before the softmax."""
+    (and, with ``logit_softcap``, capped) scores before the softmax.  The positional
+    parameters are the reference's (``__init__.py:1304-1317``); the kernel is
+    deterministic and has no dropout, and paged KV state is another lane's."""
+    if not 0.0 <= float(dropout_p) < 1.0:
+        raise ValueError("dropout_p must be in [0.0, 1.0)")
+    if dropout_p:
+        raise NotImplementedError("flash_attn: dropout is not implemented on the gfx950 lane")
+    if kv_state is not None or cache is not None:
+        raise NotImplementedError("flash_attn: paged KV state / cache objects are not served by the gfx950 lane")
+    if K is None or V is None:
+        raise ValueError("flash_attn needs K and V")
     return _attention(Q, K, V, scale, causal, return_lse, out, False, window, logit_softcap, attn_bias)
 
 
-def gqa_attention(Q, K, V, scale=None, causal: bool = False, *, return_lse: bool = False,
-                  out: str = "storage", window: int = 0, logit_softcap: float = 0.0, attn_bias=None):
-    """Grouped-query attention: kv head of query head ``h`` is ``h // (Hq / Hkv)``
-    — identical to repeating K/V along the head axis."""
+def gqa_attention(Q, K, V, num_query_heads=None, num_kv_heads=None, *, scale=None, causal: bool = False,
+                  return_lse: bool = False, out: str = "storage", window: int = 0, logit_softcap: float = 0.0,
+                  attn_bias=None):
+    """Grouped-query attention (``nn/functional.py:349-356``): kv head of query head ``h``
+    is ``h // (Hq / Hkv)`` — identical to repeating K/V along the head axis, which is what
+    the reference does with ``num_query_heads // num_kv_heads``.  The head counts may be left
+    out (they are read off the operands); when given they must agree with the operands."""
+    if num_query_heads is not None or num_kv_heads is not None:
+        if num_query_heads is None or num_kv_heads is None:
+            raise ValueError("gqa_attention: give both num_query_heads and num_kv_heads, or neither")
+        nq, nkv = int(num_query_heads), int(num_kv_heads)
+        if nkv <= 0 or nq % nkv != 0:
+            raise ValueError("num_query_heads must be divisible by num_kv_heads")
+        hq, hkv = _bits(_unbox(Q)).shape[-3], _bits(_unbox(K)).shape[-3]
+        if hkv * (nq // nkv) != hq:
+            raise ValueError(f"gqa_attention: K/V with {hkv} heads repeated {nq // nkv} times do not match "
+                             f"Q's {hq} heads")
     return _attention(Q, K, V, scale, causal, return_lse, out, True, window, logit_softcap, attn_bias)
+
+
+def mqa_attention(Q, K, V, **kwargs):
+    """Multi-query attention (``nn/functional.py:359-360``): one K/V head shared by every query head."""
+    return gqa_attention(Q, K, V, num_query_heads=_bits(_unbox(Q)).shape[-3], num_kv_heads=1, **kwargs)
 
 
 # ---------------------------------------------------------------------------
@@ -724,12 +753,80 @@ def _capacity_arg(capacity: Optional[int], T: int, k: int) -> int:
     return int(capacity)
 
 
-def route_tokens(scores, num_experts: int, top_k: int, *, normalize_weights: bool = True,
-                 capacity_factor: float = 1.25, capacity: Optional[int] = None) -> MoETransport:
+@dataclass(frozen=True)
+class MoEConfig:
+    """The reference's MoE configuration record (``distributed/moe.py:43-92``)."""
+    num_experts: int
+    top_k: int = 1
+    expert_capacity: Optional[int] = None
+    capacity_factor: float = 1.25
+    jitter_noise: float = 0.0
+    normalize_weights: bool = True
+
+    def __post_init__(self) -> None:
+        if self.num_experts < 1:
+            raise ValueError(f"num_experts must be >= 1, got {self.num_experts}")
+        if self.top_k < 1 or self.top_k > self.num_experts:
+            raise ValueError(f"top_k must be in [1, num_experts={self.num_experts}], got {self.top_k}")
+        if self.capacity_factor <= 0:
+            raise ValueError(f"capacity_factor must be > 0, got {self.capacity_factor}")
+        if not (0.0 <= self.jitter_noise < 1.0):
+            raise ValueError(f"jitter_noise must be in [0, 1), got {self.jitter_noise}")
+
+    def compute_capacity(self, num_tokens: int, num_ranks: int = 1) -> int:
+        if self.expert_capacity is not None:
+            return self.expert_capacity
+        return expert_capacity(self.capacity_factor, num_tokens, max(1, self.num_experts // num_ranks))
+
+
+class RoutingResult(NamedTuple):
+    """What the reference's ``route_tokens`` returns (``distributed/moe.py:98-113``)."""
+    assignment: np.ndarray   # (T, top_k) int64, -1 = dropped over capacity
+    weights: np.ndarray      # (T, top_k) f32, 0 for a dropped slot
+    load: np.ndarray         # (E,) int64, selections per expert before any drop
+    overflow: int
+
+
+def _route_tokens_result(scores, config, capacity) -> RoutingResult:
+    """``route_tokens(scores, config, capacity=None)`` as the reference spells it
+    (``distributed/moe.py:119-206``): the token-major view of the routing — selection, weights
+    and the first-come capacity drop run on the device; ties between bit-equal probabilities
+    go to the lowest expert id."""
+    s = np.ascontiguousarray(_unbox(scores), np.float32)
+    if s.ndim != 2:
+        raise ValueError(f"scores must be 2D (num_tokens, num_experts), got shape {s.shape}")
+    T, E = s.shape
+    if E != config.num_experts:
+        raise ValueError(f"scores has {E} expert columns but config.num_experts={config.num_experts}")
+    if getattr(config, "jitter_noise", 0.0) > 0.0:
+        raise NotImplementedError("route_tokens: jitter noise is not implemented on the gfx950 lane")
+    k = int(config.top_k)
+    if capacity is None:
+        capacity = config.compute_capacity(T)
+    capacity = int(capacity)
+    cap = min(capacity, T * k) if capacity > 0 else None          # (0 or less: every slot drops, below)
+    plan = _plan_call(s, None, None, T, E, k, 2 if config.normalize_weights else 3, cap)
+    kept = plan.kept_mask if capacity > 0 else np.zeros((T, k), bool)
+    assignment = np.where(kept, plan.expert_ids, -1).astype(np.int64)
+    weights = np.where(kept, plan.weights, np.float32(0.0)).astype(np.float32)
+    load = np.bincount(plan.expert_ids.reshape(-1), minlength=E).astype(np.int64)
+    return RoutingResult(assignment, weights, load, int(kept.size - int(kept.sum())))
+
+
+def route_tokens(scores, num_experts, top_k: Optional[int] = None, *, normalize_weights: bool = True,
+                 capacity_factor: float = 1.25, capacity: Optional[int] = None):
     """Top-k routing + packing plan.  ``scores`` ``(T, E)`` f32 gate logits.
     capacity defaults to ``ceil(capacity_factor * (T / E))``; over-capacity slots are
     dropped first-come in token-major order.  Ties between equal probabilities go
-    to the lowest expert id."""
+    to the lowest expert id.  Returns the transport descriptor of the kept slots.
+
+    Called as the reference spells it — ``route_tokens(scores, config, capacity=None)`` with
+    a :class:`MoEConfig` (or any object with its fields) — it returns a
+    :class:`RoutingResult` instead (assignment, weights, load, overflow)."""
+    if hasattr(num_experts, "num_experts"):
+        return _route_tokens_result(scores, num_experts, top_k if capacity is None else capacity)
+    if top_k is None:
+        raise TypeError("route_tokens(scores, num_experts, top_k) needs top_k")
     s = np.ascontiguousarray(_unbox(scores), np.float32)
     if s.ndim != 2:
         raise ValueError(f"scores must be 2D (num_tokens, num_experts), got shape {s.shape}")
@@ -806,7 +903,7 @@ def _plan_call(logits, given_ids, given_weights, T: int, E: int, k: int, normali
     go = np.empty(E + 1, np.int32)
     n = np.zeros(1, np.int32)
     rc = _lane.load().tessera_gfx950_moe_plan_f32(
-        _lane.ptr(logits), _lane.ptr(given_ids), _lane.ptr(given_weights), T, E, k, 1 if normalize else 0, cap,
+        _lane.ptr(logits), _lane.ptr(given_ids), _lane.ptr(given_weights), T, E, k, int(normalize), cap,
         ids.ctypes.data, w.ctypes.data, kept.ctypes.data, sp.ctypes.data, ip.ctypes.data, tos.ctypes.data,
         eos.ctypes.data, cw.ctypes.data, gs.ctypes.data, go.ctypes.data, n.ctypes.data)
     _lane.check(rc, "moe plan")

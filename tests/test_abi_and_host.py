@@ -98,9 +98,25 @@ def test_python_side_argument_errors():
     with pytest.raises(ValueError):
         ops.flash_attn(q, q, q)                                                    # head_dim % 16
     q = np.zeros((1, 4, 8, 16), np.float16)
+    # the reference's positional parameters (Q, K, V, scale, causal, cache, dropout_p, ...) are accepted
+    with pytest.raises(ValueError):
+        ops.flash_attn(q, q, q, None, False, None, 1.5)                            # dropout_p out of range
+    with pytest.raises(NotImplementedError):
+        ops.flash_attn(q, q, q, dropout_p=0.1)
+    with pytest.raises(NotImplementedError):
+        ops.flash_attn(q, kv_state=object())
+    with pytest.raises(ValueError):
+        ops.flash_attn(q)
     k = np.zeros((1, 3, 8, 16), np.float16)
     with pytest.raises(ValueError):
         ops.gqa_attention(q, k, k)                                                 # 4 % 3
+    with pytest.raises(ValueError):
+        ops.gqa_attention(q, k, k, 4, 3)                                           # the reference's own check
+    k2 = np.zeros((1, 2, 8, 16), np.float16)
+    with pytest.raises(ValueError):
+        ops.gqa_attention(q, k2, k2, 8, 2)                                         # 2 heads x 4 != 4 heads
+    with pytest.raises(ValueError):
+        ops.mqa_attention(q, k2, k2)                                               # MQA wants one K/V head
     x = b16.from_float32(np.zeros((6, 8)))
     w = b16.from_float32(np.zeros((2, 8, 8)))
     with pytest.raises(ValueError):

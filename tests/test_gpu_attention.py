@@ -394,3 +394,19 @@ def test_bias_executor_operand(lane):
     assert orc.max_rel_err(res["output"], ref) <= TOL
     bad = ex.launch(art, (q, k, v, np.zeros((7, 130), np.float32)))
     assert bad["runtime_status"] == "invalid_artifact"
+
+
+def test_gqa_and_mqa_take_the_reference_head_count_arguments(lane):
+    """nn.functional.gqa_attention(Q, K, V, num_query_heads, num_kv_heads, **kwargs) and mqa_attention."""
+    rng = np.random.default_rng(5)
+    q = b16.from_float32(rng.standard_normal((2, 8, 40, 64)).astype(np.float32))
+    k = b16.from_float32(rng.standard_normal((2, 2, 40, 64)).astype(np.float32))
+    v = b16.from_float32(rng.standard_normal((2, 2, 40, 64)).astype(np.float32))
+    a = ops.gqa_attention(q, k, v, 8, 2, causal=True, out="f32")
+    assert np.array_equal(a, ops.gqa_attention(q, k, v, causal=True, out="f32"))
+    ref, _ = orc.flash_attn_dense(q.to_float32(), k.to_float32(), v.to_float32(), causal=True)
+    assert orc.max_rel_err(a, ref) <= 2e-3
+    k1, v1 = b16.from_float32(k.to_float32()[:, :1]), b16.from_float32(v.to_float32()[:, :1])
+    m = ops.mqa_attention(q, k1, v1, out="f32")
+    ref1, _ = orc.flash_attn_dense(q.to_float32(), k1.to_float32(), v1.to_float32())
+    assert orc.max_rel_err(m, ref1) <= 2e-3

@@ -529,3 +529,35 @@ def test_quantised_swiglu_block_and_layer(lane, quant, budget):
     assert np.array_equal(out, staged)
     aligned = ops.moe_layer(xl, None, g, u, d, top_k=k, router_logits=lg, alignment=1)
     assert orc.max_rel_err(aligned, plain) <= 2.0 ** -6         # the staged unquantised form against the fused layer
+
+
+@pytest.mark.parametrize("T,E,k,normalize,capacity", [
+    (200, 8, 2, True, None), (200, 8, 2, False, None), (517, 64, 8, True, None), (517, 64, 8, True, 40),
+    (64, 4, 1, True, 3), (300, 160, 70, True, None), (50, 6, 3, True, 0),
+])
+def test_route_tokens_with_the_reference_signature(lane, T, E, k, normalize, capacity):
+    """route_tokens(scores, MoEConfig, capacity) -> RoutingResult(assignment, weights, load, overflow):
+    indices and drops bit-exact, weights to the last bit of the f32 softmax."""
+    rng = np.random.default_rng(T + E + k)
+    scores = rng.standard_normal((T, E)).astype(np.float32)
+    assert not orc.has_routing_ties(orc.router_probs(scores), k)
+    cfg = ops.MoEConfig(num_experts=E, top_k=k, normalize_weights=normalize)
+    got = ops.route_tokens(scores, cfg, capacity)
+    ref = orc.route_tokens(scores, E, k, normalize_weights=normalize, capacity_factor=cfg.capacity_factor, capacity=capacity)
+    assert got.assignment.dtype == np.int64 and got.weights.dtype == np.float32 and got.load.dtype == np.int64
+    assert np.array_equal(got.assignment, ref.assignment)
+    assert np.array_equal(got.load, ref.load) and got.overflow == ref.overflow
+    assert np.allclose(got.weights, ref.weights, rtol=2e-6, atol=1e-9)
+    assert np.array_equal(got.weights == 0, ref.weights == 0)
+    # the same routing as the packed form
+    if capacity != 0:
+        tr = ops.route_tokens(scores, E, k, normalize_weights=normalize, capacity_factor=cfg.capacity_factor,
+                              capacity=capacity)
+        assert tr.num_slots == T * k - got.overflow
+        assert np.array_equal(np.bincount(got.assignment[got.assignment >= 0], minlength=E), tr.group_sizes)
+    with pytest.raises(ValueError):
+        ops.route_tokens(scores, ops.MoEConfig(num_experts=E + 1, top_k=k))
+    with pytest.raises(ValueError):
+        ops.MoEConfig(num_experts=4, top_k=5)
+    with pytest.raises(NotImplementedError):
+        ops.route_tokens(scores, ops.MoEConfig(num_experts=E, top_k=k, jitter_noise=0.1))
