@@ -270,6 +270,12 @@ int tessera_gfx950_quantize_e4m3_f32(const float* x, int64_t n, float scale, voi
 /* _quantize_int8_per_channel (python/tessera/compiler/smoothquant.py:79-84):
  * axis=1 -> one scale per row (scales[M]); axis=0 -> one per column (scales[N]). */
 int tessera_gfx950_quantize_i8_f32(const float* x, int M, int N, int axis, void* q, float* scales);
+/* The activation side of smoothquant_matmul (python/tessera/compiler/smoothquant.py:60-62, 115-122):
+ * x_hat[m][n] = x[m][n] / smoothing[n] (f32 division), then the per-row quantiser above on x_hat,
+ * in one pass over x.  smoothing f32[N]; q int8 [M,N]; scales f32[M]. */
+int tessera_gfx950_quantize_i8_smoothed_f32(const float* x, int M, int N, const float* smoothing, void* q, float* scales);
+int tessera_gfx950_quantize_i8_smoothed_f32_dev(const float* x, int M, int N, const float* smoothing, void* q,
+                                                float* scales, void* stream);
 /* ops.quantize_nvfp4 followed by ops.dequantize_nvfp4 (python/tessera/__init__.py:3472-3504, i.e.
  * compiler/microscaling.py:317-384 with the nvfp4 format): x f32 [rows, cols] rounded onto the
  * NVFP4 grid in blocks of 16 along the last axis — block scale = max(amax / 6, 1e-30) rounded to

@@ -854,6 +854,31 @@ def w8a8_matmul(X: np.ndarray, W: np.ndarray):
     return y.astype(np.float32), acc, x_q, a_scale, w_q, w_scale.reshape(-1)
 
 
+def migrate_activation_scale(X_calib: np.ndarray, W: np.ndarray, alpha: float = 0.5, eps: float = 1e-5):
+    """``compiler/smoothquant.py:69-76, 87-112``: per input channel
+    ``s = max(max|X|^alpha / max|W|^(1-alpha), eps)`` (f64 powers of the eps-floored maxima,
+    stored f32), ``W_s = s[:, None] * W``, quantised per output column.
+    Returns ``(s f32 [C_in], w_q int8, w_scale f32 [C_out])``."""
+    X_calib = np.asarray(X_calib, np.float32)
+    W = np.asarray(W, np.float32)
+    a = np.maximum(np.abs(X_calib).max(axis=0).astype(np.float64), eps)
+    w = np.maximum(np.abs(W).max(axis=1).astype(np.float64), eps)
+    s = np.maximum((a ** alpha) / (w ** (1.0 - alpha)), eps).astype(np.float32)
+    w_q, w_scale = quantize_int8_per_channel(s[:, None] * W, axis=0)
+    return s, w_q, w_scale.reshape(-1)
+
+
+def smoothquant_matmul(X: np.ndarray, smoothing: np.ndarray, w_q: np.ndarray, w_scale: np.ndarray):
+    """``compiler/smoothquant.py:115-124``: ``X_hat = f32(X) / s``; per-row int8 codes of
+    ``X_hat``; exact integer product with the int8 weight; ``f32(acc) * a_scale * w_scale``.
+    Returns ``(y f32, acc i32, x_q, a_scale [M,1])``."""
+    X_hat = np.asarray(X, np.float32) / np.asarray(smoothing, np.float32)[None, :]
+    x_q, a_scale = quantize_int8_per_channel(X_hat, axis=1)
+    acc = gemm_i8_i32(x_q, np.asarray(w_q, np.int8))
+    y = acc.astype(np.float32) * a_scale * np.asarray(w_scale, np.float32).reshape(-1)[None, :]
+    return y.astype(np.float32), acc, x_q, a_scale
+
+
 # ---------------------------------------------------------------------------
 # error metrics used by the parity tests
 # ---------------------------------------------------------------------------

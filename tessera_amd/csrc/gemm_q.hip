@@ -247,13 +247,16 @@ __global__ void quantize_e4m3_kernel(const float* x, long n, float scale_in, con
 }
 
 // One workgroup per row: absmax, scale = max(absmax, 1e-12) / 127, q = rint(x / scale).
-__global__ void quantize_i8_rows_kernel(const float* x, int M, int N, int8_t* q, float* scales) {
+// `divisor` (f32[N] or null): x[m][n] / divisor[n] takes the place of x[m][n] — the smoothed
+// activation of the W8A8 direct-consume path (compiler/smoothquant.py:60-62, 121-122).
+__global__ void quantize_i8_rows_kernel(const float* x, int M, int N, int8_t* q, float* scales, const float* divisor) {
   __shared__ float red[4];
   const int m = blockIdx.x;
   if (m >= M) return;
   const float* row = x + (long)m * N;
+  auto at = [&](int n) { return divisor ? __fdiv_rn(row[n], divisor[n]) : row[n]; };
   float mx = 0.f;
-  for (int n = threadIdx.x; n < N; n += blockDim.x) mx = fmaxf(mx, fabsf(row[n]));
+  for (int n = threadIdx.x; n < N; n += blockDim.x) mx = fmaxf(mx, fabsf(at(n)));
   mx = warp_max(mx);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
   __syncthreads();
@@ -261,7 +264,7 @@ __global__ void quantize_i8_rows_kernel(const float* x, int M, int N, int8_t* q,
   const float scale = __fdiv_rn(fmaxf(mx, 1e-12f), 127.0f);
   if (threadIdx.x == 0) scales[m] = scale;
   for (int n = threadIdx.x; n < N; n += blockDim.x) {
-    float t = __builtin_rintf(__fdiv_rn(row[n], scale));
+    float t = __builtin_rintf(__fdiv_rn(at(n), scale));
     t = fminf(fmaxf(t, -127.f), 127.f);
     q[(long)m * N + n] = (int8_t)t;
   }
@@ -271,9 +274,10 @@ __global__ void quantize_i8_rows_kernel(const float* x, int M, int N, int8_t* q,
 // a thread keeps its runs of 16 elements in registers between the absmax pass and the
 // quantising pass, so x is read from memory once, with 16-byte loads, and every run of
 // 16 codes leaves as one 16-byte store.
-template <int GV>
+// (SMOOTH: every element is first divided by its column's entry of `divisor`, 16-byte aligned)
+template <int GV, bool SMOOTH = false>
 __global__ __launch_bounds__(256) void quantize_i8_rows_vec_kernel(const float* x, int M, int N, int8_t* q,
-                                                                   float* scales) {
+                                                                   float* scales, const float* divisor = nullptr) {
   __shared__ float red[4];
   const int m = blockIdx.x;
   if (m >= M) return;
@@ -288,6 +292,11 @@ __global__ __launch_bounds__(256) void quantize_i8_rows_vec_kernel(const float* 
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         v[u][c] = row[g * 4 + c];
+        if constexpr (SMOOTH) {
+          const float4 d = reinterpret_cast<const float4*>(divisor)[g * 4 + c];
+          v[u][c] = make_float4(__fdiv_rn(v[u][c].x, d.x), __fdiv_rn(v[u][c].y, d.y), __fdiv_rn(v[u][c].z, d.z),
+                                __fdiv_rn(v[u][c].w, d.w));
+        }
         mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v[u][c].x), fabsf(v[u][c].y)), fmaxf(fabsf(v[u][c].z), fabsf(v[u][c].w))));
       }
     }
@@ -395,21 +404,31 @@ int quantize_e4m3_dev(const float* x, int64_t n, float scale, void* codes, float
   return launch_status();
 }
 
-int quantize_i8_dev(const float* x, int M, int N, int axis, void* q, float* scales, hipStream_t s) {
-  if (M <= 0 || N <= 0 || !x || !q || !scales || (axis != 0 && axis != 1)) return kBadShape;
+int quantize_i8_dev(const float* x, int M, int N, int axis, void* q, float* scales, hipStream_t s,
+                    const float* divisor = nullptr) {
+  if (M <= 0 || N <= 0 || !x || !q || !scales || (axis != 0 && axis != 1) || (divisor && axis != 1)) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
   if (axis == 1) {
     int8_t* codes = static_cast<int8_t*>(q);
     const int groups = N / 16;
-    const bool vec = N % 16 == 0 && groups <= 4 * 256 && aligned16(x) && aligned16(q);
-    if (vec && groups <= 256)
-      hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<1>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales);
+    const bool vec = N % 16 == 0 && groups <= 4 * 256 && aligned16(x) && aligned16(q) && aligned16(divisor);
+    if (divisor) {
+      if (vec && groups <= 256)
+        hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<1, true>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales, divisor);
+      else if (vec && groups <= 512)
+        hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<2, true>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales, divisor);
+      else if (vec)
+        hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<4, true>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales, divisor);
+      else
+        hipLaunchKernelGGL(quantize_i8_rows_kernel, dim3(M), dim3(256), 0, s, x, M, N, codes, scales, divisor);
+    } else if (vec && groups <= 256)
+      hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<1>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales, nullptr);
     else if (vec && groups <= 512)
-      hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<2>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales);
+      hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<2>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales, nullptr);
     else if (vec)
-      hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<4>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales);
+      hipLaunchKernelGGL((quantize_i8_rows_vec_kernel<4>), dim3(M), dim3(256), 0, s, x, M, N, codes, scales, nullptr);
     else
-      hipLaunchKernelGGL(quantize_i8_rows_kernel, dim3(M), dim3(256), 0, s, x, M, N, codes, scales);
+      hipLaunchKernelGGL(quantize_i8_rows_kernel, dim3(M), dim3(256), 0, s, x, M, N, codes, scales, nullptr);
   } else if (N % 4 == 0 && aligned16(x) && aligned16(scales) && (reinterpret_cast<uintptr_t>(q) & 3) == 0 &&
              ceil_div(M, kColRows) <= 65535) {
     // the per-column running maxima live in the stream's own workspace
@@ -656,6 +675,12 @@ int tessera_gfx950_quantize_i8_f32_dev(const float* x, int M, int N, int axis, v
   return quantize_i8_dev(x, M, N, axis, q, scales, as_stream(stream));
 }
 
+int tessera_gfx950_quantize_i8_smoothed_f32_dev(const float* x, int M, int N, const float* smoothing, void* q,
+                                                float* scales, void* stream) {
+  if (!smoothing) return kBadShape;
+  return quantize_i8_dev(x, M, N, 1, q, scales, as_stream(stream), smoothing);
+}
+
 int tessera_gfx950_fake_quantize_nvfp4_f32_dev(const float* x, int rows, int cols, float* dq, void* dq_bf16,
                                                float* scales, void* stream) {
   return fake_quantize_nvfp4_dev(x, rows, cols, dq, dq_bf16, scales, as_stream(stream));
@@ -728,6 +753,23 @@ int tessera_gfx950_quantize_e4m3_f32(const float* x, int64_t n, float scale, voi
   if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
   if (!scope.download(codes, dc, (size_t)n)) return kDeviceFailed;
   if (scale_out && !scope.download(scale_out, ds, 4)) return kDeviceFailed;
+  return kOk;
+}
+
+int tessera_gfx950_quantize_i8_smoothed_f32(const float* x, int M, int N, const float* smoothing, void* q, float* scales) {
+  if (M <= 0 || N <= 0 || !x || !q || !scales || !smoothing) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const size_t n = (size_t)M * N;
+  DeviceScope scope;
+  float* dx = static_cast<float*>(scope.alloc(n * 4, x));
+  float* dsm = static_cast<float*>(scope.alloc((size_t)N * 4, smoothing));
+  void* dq = scope.alloc(n);
+  float* ds = static_cast<float*>(scope.alloc((size_t)M * 4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = quantize_i8_dev(dx, M, N, 1, dq, ds, nullptr, dsm);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  if (!scope.download(q, dq, n) || !scope.download(scales, ds, (size_t)M * 4)) return kDeviceFailed;
   return kOk;
 }
 

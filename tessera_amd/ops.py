@@ -1185,18 +1185,43 @@ def gemm_fp8(a_codes, b_codes, scale_a, scale_b, *, out: str = "bf16"):
     return d.view(BF16Array) if out == "bf16" else d
 
 
-def quantize_int8_per_channel(M, axis: int):
+def quantize_int8_per_channel(M, axis: int, *, smoothing=None):
     """Symmetric int8 quantise along the kept axis → ``(q int8, scale f32)`` with
-    ``scale`` shaped like numpy's ``keepdims`` reduction over ``axis``."""
+    ``scale`` shaped like numpy's ``keepdims`` reduction over ``axis``.  ``smoothing``
+    (f32 ``[C]``, ``axis=1`` only): every element is divided by its column's factor first,
+    in the same pass (the smoothed activation of ``smoothquant_matmul``)."""
     a = np.ascontiguousarray(_unbox(M), np.float32)
     if a.ndim != 2 or axis not in (0, 1):
         raise ValueError("quantize_int8_per_channel takes a 2-D array and axis 0 or 1")
     R, C = a.shape
     q = np.empty((R, C), np.int8)
     sc = np.empty(R if axis == 1 else C, np.float32)
+    if smoothing is not None:
+        sm = np.ascontiguousarray(smoothing, np.float32).reshape(-1)
+        if axis != 1 or sm.shape[0] != C:
+            raise ValueError(f"smoothing needs axis=1 and one factor per column ({C}); got axis={axis}, {sm.shape}")
+        _lane.check(_lane.load().tessera_gfx950_quantize_i8_smoothed_f32(a.ctypes.data, R, C, sm.ctypes.data, q.ctypes.data,
+                                                                         sc.ctypes.data), "quantize_int8_per_channel")
+        return q, sc.reshape(R, 1)
     _lane.check(_lane.load().tessera_gfx950_quantize_i8_f32(a.ctypes.data, R, C, axis, q.ctypes.data, sc.ctypes.data),
                 "quantize_int8_per_channel")
     return q, (sc.reshape(R, 1) if axis == 1 else sc.reshape(1, C))
+
+
+def smoothquant_matmul(X, migrated):
+    """The W8A8 direct-consume path (``compiler/smoothquant.py:115-124``): the activation is
+    smoothed (``X / migrated.smoothing``) and quantised per token on the device in one pass,
+    multiplied with the int8 weight ``migrated.w_q`` on the int8 matrix cores, and the int32
+    accumulators are rescaled by the token scales and ``migrated.w_scale``.  ``migrated`` is the
+    reference's ``MigratedLinear`` or any object with its ``smoothing``, ``w_q``, ``w_scale``."""
+    x = np.asarray(_unbox(X), np.float32)
+    w_q = np.asarray(migrated.w_q)
+    if x.ndim != 2 or w_q.ndim != 2 or x.shape[1] != w_q.shape[0]:
+        raise ValueError(f"shape mismatch: X {x.shape} @ w_q {w_q.shape}")
+    if w_q.dtype != np.int8:
+        raise ValueError("smoothquant_matmul consumes the int8 weight operand as it is")
+    x_q, a_scale = quantize_int8_per_channel(x, axis=1, smoothing=migrated.smoothing)
+    return w8a8_gemm(x_q, w_q, a_scale, migrated.w_scale)
 
 
 def w8a8_gemm(x_q, w_q, a_scale, w_scale, *, return_acc: bool = False):

@@ -381,3 +381,27 @@ def test_float_grid_and_group_scaling_on_device_buffers(lane):
     out = np.empty((S, N), np.float32)
     bad = off.copy(); bad[2] = 12                        # offsets must not decrease
     assert lib.tessera_gfx950_scale_groups_f32(y.ctypes.data, bad.ctypes.data, sc.ctypes.data, out.ctypes.data, 0, S, N, E) == 1
+
+
+@pytest.mark.parametrize("M,K,N", [(64, 256, 128), (33, 100, 72), (300, 4096, 512), (8, 16400, 64)])
+def test_smoothquant_matmul_bit_for_bit(lane, M, K, N):
+    """smoothquant_matmul on a migrated layer: smoothed activation codes, token scales and int32
+    accumulators bit for bit, the rescaled f32 result exactly as numpy's two multiplies give it."""
+    from types import SimpleNamespace
+    rng = np.random.default_rng(M + K + N)
+    X = (rng.standard_normal((M, K)) * np.exp(rng.standard_normal(K))).astype(np.float32)     # outlier channels
+    W = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
+    s, w_q, w_scale = orc.migrate_activation_scale(X, W)
+    x_q, a_scale = ops.quantize_int8_per_channel(X, 1, smoothing=s)
+    ry, racc, rxq, ras = orc.smoothquant_matmul(X, s, w_q, w_scale)
+    assert np.array_equal(x_q, rxq) and np.array_equal(a_scale, ras)
+    got = ops.smoothquant_matmul(X, SimpleNamespace(smoothing=s, w_q=w_q, w_scale=w_scale))
+    assert got.dtype == np.float32 and np.array_equal(got, ry)
+    # the point of the migration: closer to the f32 product than plain W8A8 on data with outlier channels
+    full = X.astype(np.float64) @ W.astype(np.float64)
+    plain = ops.w8a8_matmul(X, W)
+    assert np.linalg.norm(got - full) <= np.linalg.norm(plain - full) * 1.05
+    with pytest.raises(ValueError):
+        ops.quantize_int8_per_channel(X, 0, smoothing=s)
+    with pytest.raises(ValueError):
+        ops.smoothquant_matmul(X, SimpleNamespace(smoothing=s, w_q=w_q.astype(np.int32), w_scale=w_scale))

@@ -454,3 +454,39 @@ def test_unpack_combine_closed_forms():
     for i, slot in enumerate(capped.sort_perm):
         ref[slot // k] += float(wts.reshape(-1)[slot]) * y[i]
     np.testing.assert_allclose(orc.unpack_combine(y, capped.inverse_perm, wts), ref, rtol=1e-5, atol=1e-6)
+
+
+def test_smoothquant_restatement_closed_forms():
+    """migrate_activation_scale / smoothquant_matmul: hand-worked factors at alpha 0, 0.5 and 1, the
+    eps floor, reduction to the plain W8A8 path at s = 1, and the migration's defining identity
+    (X / s) (s W) = X W within the int8 error."""
+    X = np.array([[2.0, -8.0, 0.0], [1.0, 4.0, 0.0]], np.float32)
+    W = np.array([[1.0, -0.5], [4.0, 2.0], [0.25, 0.125]], np.float32)
+    s, w_q, w_scale = orc.migrate_activation_scale(X, W, alpha=0.5, eps=1e-5)
+    # channel maxima: activations (2, 8, 0 -> eps), weights (1, 4, 0.25)
+    want = np.array([np.sqrt(2.0 / 1.0), np.sqrt(8.0 / 4.0), np.sqrt(1e-5 / 0.25)])
+    assert np.allclose(s, want, rtol=1e-6)
+    assert np.allclose(orc.migrate_activation_scale(X, W, alpha=1.0)[0], [2.0, 8.0, 1e-5], rtol=1e-6)
+    assert np.allclose(orc.migrate_activation_scale(X, W, alpha=0.0)[0], [1.0, 0.25, 4.0], rtol=1e-6)
+    # the weight operand is the column-quantised smoothed weight
+    ws = s[:, None] * W
+    assert np.array_equal(w_q, np.rint(ws / (np.abs(ws).max(axis=0) / 127)).astype(np.int8))
+    assert np.allclose(w_scale, np.abs(ws).max(axis=0) / 127, rtol=1e-6)
+    rng = np.random.default_rng(3)
+    X = (rng.standard_normal((40, 96)) * np.exp(rng.standard_normal(96))).astype(np.float32)
+    W = (rng.standard_normal((96, 24)) / 10).astype(np.float32)
+    # s = 1: exactly the unsmoothed path
+    wq1, ws1 = orc.quantize_int8_per_channel(W, axis=0)
+    y1, acc1, xq1, as1 = orc.smoothquant_matmul(X, np.ones(96, np.float32), wq1, ws1)
+    ry, racc, rxq, ras, _, _ = orc.w8a8_matmul(X, W)
+    assert np.array_equal(y1, ry) and np.array_equal(acc1, racc) and np.array_equal(xq1, rxq) and np.array_equal(as1, ras)
+    # migrated: the product survives, and beats the unsmoothed path on outlier channels
+    s, w_q, w_scale = orc.migrate_activation_scale(X, W)
+    y, acc, x_q, a_scale = orc.smoothquant_matmul(X, s, w_q, w_scale)
+    full = X.astype(np.float64) @ W.astype(np.float64)
+    assert np.linalg.norm(y - full) / np.linalg.norm(full) < 0.02
+    assert np.linalg.norm(y - full) < np.linalg.norm(ry - full)
+    # codes are those of X / s, row scales its row maxima / 127
+    xh = X / s[None, :]
+    assert np.array_equal(a_scale.reshape(-1), np.abs(xh).max(axis=1) / np.float32(127.0))
+    assert np.array_equal(acc, x_q.astype(np.int64) @ w_q.astype(np.int64))
