@@ -270,6 +270,12 @@ int tessera_gfx950_quantize_e4m3_f32(const float* x, int64_t n, float scale, voi
 /* _quantize_int8_per_channel (python/tessera/compiler/smoothquant.py:79-84):
  * axis=1 -> one scale per row (scales[M]); axis=0 -> one per column (scales[N]). */
 int tessera_gfx950_quantize_i8_f32(const float* x, int M, int N, int axis, void* q, float* scales);
+/* quantization.quantize_int8, symmetric form (python/tessera/quantization.py:24-37): one scale for
+ * the whole tensor — `scale` if > 0, else max|x| / 127 found on the device (1 for an all-zero
+ * tensor) — and q = clip(rint(x / scale), -127, 127).  scale_out (optional) receives the scale. */
+int tessera_gfx950_quantize_i8_tensor_f32(const float* x, int64_t n, float scale, void* q, float* scale_out);
+int tessera_gfx950_quantize_i8_tensor_f32_dev(const float* x, int64_t n, float scale, void* q, float* scale_out_dev,
+                                              void* stream);
 /* The activation side of smoothquant_matmul (python/tessera/compiler/smoothquant.py:60-62, 115-122):
  * x_hat[m][n] = x[m][n] / smoothing[n] (f32 division), then the per-row quantiser above on x_hat,
  * in one pass over x.  smoothing f32[N]; q int8 [M,N]; scales f32[M]. */

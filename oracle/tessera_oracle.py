@@ -854,6 +854,19 @@ def w8a8_matmul(X: np.ndarray, W: np.ndarray):
     return y.astype(np.float32), acc, x_q, a_scale, w_q, w_scale.reshape(-1)
 
 
+def quantize_int8_tensor(x: np.ndarray, scale: float | None = None):
+    """``quantization.quantize_int8`` symmetric (``quantization.py:24-37``): one scale,
+    ``f32(max|x| / 127)`` (1 when the tensor is all zero) unless given;
+    ``q = clip(rint(x / scale), -127, 127)``.  Returns ``(q int8, scale np.float32)``."""
+    x = np.asarray(x, np.float32)
+    if scale is None:
+        m = float(np.max(np.abs(x))) if x.size else 0.0
+        s = np.float32(1.0) if m == 0.0 else np.float32(m / 127)
+    else:
+        s = np.float32(scale)
+    return np.round(x / s).clip(-127, 127).astype(np.int8), s
+
+
 def migrate_activation_scale(X_calib: np.ndarray, W: np.ndarray, alpha: float = 0.5, eps: float = 1e-5):
     """``compiler/smoothquant.py:69-76, 87-112``: per input channel
     ``s = max(max|X|^alpha / max|W|^(1-alpha), eps)`` (f64 powers of the eps-floored maxima,

@@ -446,6 +446,53 @@ int quantize_i8_dev(const float* x, int M, int N, int axis, void* q, float* scal
   return launch_status();
 }
 
+// quantization.quantize_int8, symmetric form (python/tessera/quantization.py:24-37): one scale for
+// the whole tensor, scale_in if > 0 else max|x| / 127 (1 for an all-zero tensor);
+// q = clip(rint(x / scale), -127, 127).  Runs of 16 elements per thread.
+__global__ __launch_bounds__(256) void quantize_i8_tensor_kernel(const float* __restrict__ x, long n, float scale_in,
+                                                                 const unsigned* amax_bits, int8_t* __restrict__ q,
+                                                                 float* scale_out) {
+  float scale = scale_in;
+  if (!(scale_in > 0.f)) {
+    const float amax = __builtin_bit_cast(float, *amax_bits);
+    scale = amax == 0.f ? 1.0f : __fdiv_rn(amax, 127.0f);
+  }
+  if (scale_out && blockIdx.x == 0 && threadIdx.x == 0) *scale_out = scale;
+  auto code = [&](float f) -> uint32_t {
+    float t = __builtin_rintf(__fdiv_rn(f, scale));
+    t = fminf(fmaxf(t, -127.f), 127.f);
+    return (uint32_t)(uint8_t)(int8_t)t;
+  };
+  auto pack = [&](const float4& f) -> uint32_t {
+    return code(f.x) | (code(f.y) << 8) | (code(f.z) << 16) | (code(f.w) << 24);
+  };
+  const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x, nthreads = (long)gridDim.x * blockDim.x;
+  const bool vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(q)) & 15) == 0;
+  const long n16 = vec ? n / 16 : 0;
+  for (long g = tid; g < n16; g += nthreads) {
+    const float4* src = reinterpret_cast<const float4*>(x) + g * 4;
+    const float4 v0 = src[0], v1 = src[1], v2 = src[2], v3 = src[3];
+    reinterpret_cast<uint4*>(q)[g] = make_uint4(pack(v0), pack(v1), pack(v2), pack(v3));
+  }
+  for (long i = n16 * 16 + tid; i < n; i += nthreads) q[i] = (int8_t)code(x[i]);
+}
+
+int quantize_i8_tensor_dev(const float* x, int64_t n, float scale, void* q, float* scale_out_dev, hipStream_t s) {
+  if (n <= 0 || !x || !q || scale != scale) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  const int blocks = (int)std::min<int64_t>((n / 16 + 255) / 256 + 1, 4096);
+  unsigned* amax = nullptr;
+  if (!(scale > 0.f)) {
+    amax = static_cast<unsigned*>(stream_workspace(s, 256));
+    if (!amax) return kDeviceFailed;
+    zero_words(amax, 1, s);
+    hipLaunchKernelGGL(absmax_kernel, dim3(std::min(blocks, 512)), dim3(256), 0, s, x, (long)n, amax);
+  }
+  hipLaunchKernelGGL(quantize_i8_tensor_kernel, dim3(blocks), dim3(256), 0, s, x, (long)n, scale, amax,
+                     static_cast<int8_t*>(q), scale_out_dev);
+  return launch_status();
+}
+
 // ---- per-tensor float grids (fp8 / fp6 / fp4) ---------------------------------------------------
 // The native lanes' grid rounding, tessera_x86_avx512_fpquant_f32
 // (src/compiler/codegen/tessera_x86_backend/src/kernels/avx512_fpquant_f32.cpp:28-41):
@@ -675,6 +722,10 @@ int tessera_gfx950_quantize_i8_f32_dev(const float* x, int M, int N, int axis, v
   return quantize_i8_dev(x, M, N, axis, q, scales, as_stream(stream));
 }
 
+int tessera_gfx950_quantize_i8_tensor_f32_dev(const float* x, int64_t n, float scale, void* q, float* scale_out_dev,
+                                              void* stream) {
+  return quantize_i8_tensor_dev(x, n, scale, q, scale_out_dev, as_stream(stream));
+}
 int tessera_gfx950_quantize_i8_smoothed_f32_dev(const float* x, int M, int N, const float* smoothing, void* q,
                                                 float* scales, void* stream) {
   if (!smoothing) return kBadShape;
@@ -752,6 +803,22 @@ int tessera_gfx950_quantize_e4m3_f32(const float* x, int64_t n, float scale, voi
   if (rc != kOk) return rc;
   if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
   if (!scope.download(codes, dc, (size_t)n)) return kDeviceFailed;
+  if (scale_out && !scope.download(scale_out, ds, 4)) return kDeviceFailed;
+  return kOk;
+}
+
+int tessera_gfx950_quantize_i8_tensor_f32(const float* x, int64_t n, float scale, void* q, float* scale_out) {
+  if (n <= 0 || !x || !q || scale != scale) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  DeviceScope scope;
+  float* dx = static_cast<float*>(scope.alloc((size_t)n * 4, x));
+  void* dq = scope.alloc((size_t)n);
+  float* ds = static_cast<float*>(scope.alloc(4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = quantize_i8_tensor_dev(dx, n, scale, dq, ds, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  if (!scope.download(q, dq, (size_t)n)) return kDeviceFailed;
   if (scale_out && !scope.download(scale_out, ds, 4)) return kDeviceFailed;
   return kOk;
 }

@@ -97,6 +97,8 @@ _SIGNATURES = {
     "tessera_gfx950_batched_gemm_strided_bf16_dev": [_c_vp] * 3 + [_c_int] * 4 + [_c_i64] * 3 + [_c_int, _c_vp],
     "tessera_gfx950_fake_quantize_nvfp4_f32": [_c_vp, _c_int, _c_int, _c_vp, _c_vp, _c_vp],
     "tessera_gfx950_fake_quantize_nvfp4_f32_dev": [_c_vp, _c_int, _c_int, _c_vp, _c_vp, _c_vp, _c_vp],
+    "tessera_gfx950_quantize_i8_tensor_f32": [_c_vp, _c_i64, _c_f, _c_vp, _c_vp],
+    "tessera_gfx950_quantize_i8_tensor_f32_dev": [_c_vp, _c_i64, _c_f, _c_vp, _c_vp, _c_vp],
     "tessera_gfx950_quantize_i8_smoothed_f32": [_c_vp, _c_int, _c_int, _c_vp, _c_vp, _c_vp],
     "tessera_gfx950_quantize_i8_smoothed_f32_dev": [_c_vp, _c_int, _c_int, _c_vp, _c_vp, _c_vp, _c_vp],
     "tessera_gfx950_fpquant_f32": [_c_vp, _c_i64, _c_f, _c_int, _c_int, _c_vp],

@@ -1208,6 +1208,30 @@ def quantize_int8_per_channel(M, axis: int, *, smoothing=None):
     return q, (sc.reshape(R, 1) if axis == 1 else sc.reshape(1, C))
 
 
+def quantize_int8(x, scale=None, zero_point: int = 0, *, symmetric: bool = True):
+    """Per-tensor int8 quantisation → ``(q, scale, zero_point)`` (``quantization.py:31-44``);
+    the symmetric form runs on the device."""
+    if not symmetric:
+        raise NotImplementedError("quantize_int8: only the symmetric form is implemented on the gfx950 lane")
+    a = np.ascontiguousarray(_unbox(x), np.float32)
+    q = np.empty(a.shape, np.int8)
+    s_out = np.ones(1, np.float32)
+    if scale is not None and not float(scale) > 0.0:
+        raise ValueError("quantize_int8: scale must be positive")
+    if a.size:
+        _lane.check(_lane.load().tessera_gfx950_quantize_i8_tensor_f32(
+            a.ctypes.data, a.size, 0.0 if scale is None else float(np.float32(scale)), q.ctypes.data, s_out.ctypes.data),
+            "quantize_int8")
+    elif scale is not None:
+        s_out[0] = np.float32(scale)
+    return q, np.float32(s_out[0]), 0
+
+
+def dequantize_int8(q, scale, zero_point: int = 0) -> np.ndarray:
+    """``(q - zero_point) * scale`` in f32 (``quantization.py:47-48``); a host-side view of codes."""
+    return (np.asarray(_unbox(q)).astype(np.float32) - float(zero_point)) * np.float32(scale)
+
+
 def smoothquant_matmul(X, migrated):
     """The W8A8 direct-consume path (``compiler/smoothquant.py:115-124``): the activation is
     smoothed (``X / migrated.smoothing``) and quantised per token on the device in one pass,

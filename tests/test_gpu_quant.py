@@ -405,3 +405,23 @@ def test_smoothquant_matmul_bit_for_bit(lane, M, K, N):
         ops.quantize_int8_per_channel(X, 0, smoothing=s)
     with pytest.raises(ValueError):
         ops.smoothquant_matmul(X, SimpleNamespace(smoothing=s, w_q=w_q.astype(np.int32), w_scale=w_scale))
+
+
+def test_per_tensor_int8_quantiser(lane):
+    """quantization.quantize_int8 (symmetric): codes and scale bit for bit; every half-way point of
+    the code grid rounds to the even code; an all-zero tensor gets scale 1."""
+    rng = np.random.default_rng(12)
+    x = (rng.standard_normal((513, 257)) * 3).astype(np.float32)
+    q, s, zp = ops.quantize_int8(x)
+    oq, os_ = orc.quantize_int8_tensor(x)
+    assert zp == 0 and s == os_ and q.dtype == np.int8 and np.array_equal(q, oq)
+    q2, s2, _ = ops.quantize_int8(x, scale=0.05)
+    assert s2 == np.float32(0.05) and np.array_equal(q2, orc.quantize_int8_tensor(x, 0.05)[0])
+    ties = (np.arange(-260, 261, dtype=np.float32) / 2)                      # scale 1: k + 0.5 -> even
+    qt, _, _ = ops.quantize_int8(ties, scale=1.0)
+    assert np.array_equal(qt, np.clip(np.rint(ties), -127, 127).astype(np.int8))
+    qz, sz, _ = ops.quantize_int8(np.zeros(40, np.float32))
+    assert sz == np.float32(1.0) and not qz.any()
+    assert np.allclose(ops.dequantize_int8(q, s), x, atol=float(s) / 2 * 1.0001)
+    with pytest.raises(NotImplementedError):
+        ops.quantize_int8(x, symmetric=False)

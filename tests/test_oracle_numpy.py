@@ -490,3 +490,15 @@ def test_smoothquant_restatement_closed_forms():
     xh = X / s[None, :]
     assert np.array_equal(a_scale.reshape(-1), np.abs(xh).max(axis=1) / np.float32(127.0))
     assert np.array_equal(acc, x_q.astype(np.int64) @ w_q.astype(np.int64))
+
+
+def test_per_tensor_int8_closed_forms():
+    """quantize_int8_tensor: a ramp of exact multiples of the scale maps to its own indices, half-way
+    points go to the even code, the scale is max|x| / 127, zeros get scale 1, saturation at +-127."""
+    ramp = np.arange(-127, 128, dtype=np.float32) * np.float32(0.25)
+    q, s = orc.quantize_int8_tensor(ramp)
+    assert s == np.float32(127 * 0.25 / 127) and np.array_equal(q, np.arange(-127, 128).astype(np.int8))
+    q, _ = orc.quantize_int8_tensor(np.array([0.5, 1.5, 2.5, -0.5, -1.5, 300.0, -300.0], np.float32), scale=1.0)
+    assert list(q) == [0, 2, 2, 0, -2, 127, -127]
+    q, s = orc.quantize_int8_tensor(np.zeros(5, np.float32))
+    assert s == np.float32(1.0) and not q.any()
