@@ -917,10 +917,12 @@ def _plan_call(logits, given_ids, given_weights, T: int, E: int, k: int, normali
                         gs.astype(np.int64), T, k, capacity, transport)
 
 
-def route_top_k(router_logits, top_k: int, *, normalize: bool = True):
+def route_top_k(router_logits, top_k: int, *, normalize: bool = True, compute_dtype=np.float32):
     """Exact top-k routing on the LOGITS → ``(expert_ids (T,k) int64, weights (T,k) f32)``:
     descending by logit, ties to the lowest expert id; ``normalize`` makes the weights a
     softmax over the selected logits, else each is ``1/k`` (``models/moe_routing.py:54-77``)."""
+    if np.dtype(compute_dtype) != np.float32:
+        raise NotImplementedError("route_top_k on the gfx950 lane computes in f32")
     lg = np.ascontiguousarray(_unbox(router_logits), np.float32)
     if lg.ndim != 2:
         raise ValueError("router_logits must be (T, num_experts)")
@@ -1037,6 +1039,55 @@ def moe_combine(y_packed, plan: MoETransport) -> np.ndarray:
     _lane.check(fn(ya.ctypes.data, tos.ctypes.data, w.ctypes.data, outp.ctypes.data, plan.num_tokens, S, N),
                 "moe_combine")
     return outp
+
+
+def _as_transport(plan) -> MoETransport:
+    """The int32 descriptor of a plan: a :class:`MoETransport`, this module's
+    :class:`DispatchPlan`, or any object with the fields of the reference's plans
+    (``stdlib/moe.py:55-67``, ``models/moe_routing.py:35-45``)."""
+    if isinstance(plan, MoETransport):
+        return plan
+    tr = getattr(plan, "transport", None)
+    if isinstance(tr, MoETransport):
+        return tr
+    ids = np.asarray(plan.expert_ids)
+    T, k = ids.shape
+    perm = np.asarray(plan.sort_perm, np.int64).reshape(-1)
+    groups = np.asarray(plan.group_sizes, np.int64).reshape(-1)
+    if perm.size and (perm.min() < 0 or perm.max() >= T * k):
+        raise ValueError("plan.sort_perm contains an invalid slot")
+    if int(groups.sum()) != perm.size:
+        raise ValueError("plan.group_sizes must sum to the number of kept slots")
+    w = getattr(plan, "weights", None)
+    w = np.zeros(T * k, np.float32) if w is None else np.asarray(w, np.float32).reshape(-1)
+    offsets = np.concatenate((np.zeros(1, np.int64), np.cumsum(groups))).astype(np.int32)
+    return MoETransport(int(T), int(k), int(groups.size), getattr(plan, "capacity", None), (perm // k).astype(np.int32),
+                        ids.reshape(-1)[perm].astype(np.int32), w[perm].astype(np.float32), groups.astype(np.int32), offsets)
+
+
+def compute_capacity(num_tokens: int, top_k: int, num_experts: int, capacity_factor: float) -> int:
+    """Per-expert capacity ``ceil(factor * T * k / E)``, at least 1 (``stdlib/moe.py:41-52``)."""
+    if num_tokens <= 0:
+        return 0
+    return max(1, int(math.ceil(capacity_factor * num_tokens * top_k / max(1, num_experts))))
+
+
+def dispatch(x, plan):
+    """``stdlib.moe.dispatch`` (``stdlib/moe.py:117-121``): token rows of the kept, expert-sorted
+    slots → ``(S, H)``, gathered on the device."""
+    return moe_dispatch(x, _as_transport(plan))
+
+
+def combine(y_packed, plan) -> np.ndarray:
+    """``stdlib.moe.combine`` (``stdlib/moe.py:124-134``): packed expert rows scattered back to
+    ``(T, H)``, each weighted by its slot's route weight, added in packed order (f32 here)."""
+    return moe_combine(y_packed, _as_transport(plan))
+
+
+def grouped_swiglu(x_packed, w_gate, w_up, w_down, group_sizes):
+    """``stdlib.moe.grouped_swiglu`` (``stdlib/moe.py:151-163``) on the fused expert-block
+    kernels: bf16 storage in and out, f32 accumulation."""
+    return moe_swiglu_block(x_packed, w_gate, w_up, w_down, group_sizes)
 
 
 def _moe_layer_staged(x, W_router, W_gate, W_up, W_down, top_k, normalize_weights, capacity_factor, kind, alignment,

@@ -561,3 +561,39 @@ def test_route_tokens_with_the_reference_signature(lane, T, E, k, normalize, cap
         ops.MoEConfig(num_experts=4, top_k=5)
     with pytest.raises(NotImplementedError):
         ops.route_tokens(scores, ops.MoEConfig(num_experts=E, top_k=k, jitter_noise=0.1))
+
+
+def test_stdlib_moe_spellings(lane):
+    """stdlib.moe's dispatch / combine / grouped_swiglu / compute_capacity on a plan object that only
+    has the reference's fields (no device descriptor attached)."""
+    from types import SimpleNamespace
+    rng = np.random.default_rng(21)
+    T, E, k, H, F = 96, 6, 2, 64, 48
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    ids, w = ops.route_top_k(logits, k, compute_dtype=np.float32)
+    cap = ops.compute_capacity(T, k, E, 1.0)
+    assert cap == 32 and ops.compute_capacity(0, k, E, 1.0) == 0 and ops.compute_capacity(3, 1, 64, 0.5) == 1
+    plan = ops.plan_dispatch(ids, w, E, capacity=cap)
+    bare = SimpleNamespace(expert_ids=plan.expert_ids, weights=plan.weights, kept_mask=plan.kept_mask,
+                           sort_perm=plan.sort_perm, group_sizes=plan.group_sizes, num_tokens=T, top_k=k, capacity=cap)
+    x = b16.from_float32(rng.standard_normal((T, H)).astype(np.float32))
+    xp = ops.dispatch(x, bare)
+    tok = plan.sort_perm // k
+    assert np.array_equal(np.asarray(xp, np.uint16), np.asarray(x, np.uint16)[tok])
+    assert np.array_equal(np.asarray(ops.dispatch(x, plan), np.uint16), np.asarray(xp, np.uint16))
+    wg, wu = (b16.from_float32((rng.standard_normal((E, H, F)) / 8).astype(np.float32)) for _ in range(2))
+    wd = b16.from_float32((rng.standard_normal((E, F, H)) / 7).astype(np.float32))
+    yp = ops.grouped_swiglu(xp, wg, wu, wd, plan.group_sizes)
+    ref = orc.moe_swiglu_block(xp.to_float32(), wg.to_float32(), wu.to_float32(), wd.to_float32(), plan.group_sizes)
+    assert orc.max_rel_err(yp.to_float32(), ref) <= 2e-3 + 2.0 ** -8
+    out = ops.combine(yp, bare)
+    want = np.zeros((T, H), np.float64)
+    flat_w = plan.weights.reshape(-1)
+    for i, slot in enumerate(plan.sort_perm):                        # stdlib.moe.combine, as written there
+        want[int(slot) // k] += float(flat_w[int(slot)]) * yp.to_float32()[i].astype(np.float64)
+    assert out.shape == (T, H) and np.allclose(out, want, rtol=1e-5, atol=1e-6)
+    with pytest.raises(NotImplementedError):
+        ops.route_top_k(logits, k, compute_dtype=np.float64)
+    with pytest.raises(ValueError):
+        bad = SimpleNamespace(**{**bare.__dict__, "group_sizes": plan.group_sizes + 1})
+        ops.dispatch(x, bad)
