@@ -597,3 +597,26 @@ def test_stdlib_moe_spellings(lane):
     with pytest.raises(ValueError):
         bad = SimpleNamespace(**{**bare.__dict__, "group_sizes": plan.group_sizes + 1})
         ops.dispatch(x, bad)
+
+
+def test_route_tokens_facts_the_reference_tests_hold(lane):
+    """The statements of the reference's own routing tests (tests/unit/test_moe.py:46-103)."""
+    rng = np.random.default_rng(0)
+    scores = rng.standard_normal((128, 8)).astype(np.float32)
+    res = ops.route_tokens(scores, ops.MoEConfig(num_experts=8, top_k=2))
+    assert res.assignment.shape == (128, 2) and res.weights.shape == (128, 2)
+    res = ops.route_tokens(scores[:64], ops.MoEConfig(num_experts=8, top_k=2, normalize_weights=True))
+    valid = (res.assignment >= 0).all(axis=1)
+    assert np.allclose(res.weights.sum(axis=1)[valid], 1.0, atol=1e-5)
+    res = ops.route_tokens(scores[:32], ops.MoEConfig(num_experts=8, top_k=1))
+    a = res.assignment[:, 0]
+    assert ((a[a >= 0] >= 0) & (a[a >= 0] < 8)).all() and res.load.sum() <= 32
+    with pytest.raises(ValueError, match="num_experts"):
+        ops.route_tokens(np.zeros((32, 4), np.float32), ops.MoEConfig(num_experts=8, top_k=1))
+    with pytest.raises(ValueError, match="2D"):
+        ops.route_tokens(np.zeros((32,), np.float32), ops.MoEConfig(num_experts=1, top_k=1))
+    # equal scores: every token ties; a capacity of one slot per expert overflows
+    res = ops.route_tokens(np.ones((16, 4), np.float32), ops.MoEConfig(num_experts=4, top_k=1, expert_capacity=1), capacity=1)
+    assert res.overflow > 0 and res.overflow == int((res.assignment < 0).sum())
+    assert ops.MoEConfig(num_experts=8, expert_capacity=50).compute_capacity(num_tokens=128) == 50
+    assert ops.MoEConfig(num_experts=8, capacity_factor=1.25).compute_capacity(num_tokens=128) == 20

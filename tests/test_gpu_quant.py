@@ -425,3 +425,23 @@ def test_per_tensor_int8_quantiser(lane):
     assert np.allclose(ops.dequantize_int8(q, s), x, atol=float(s) / 2 * 1.0001)
     with pytest.raises(NotImplementedError):
         ops.quantize_int8(x, symmetric=False)
+
+
+@pytest.mark.parametrize("fmt,bound", [("e4m3", 0.15), ("e5m2", 0.30)])
+def test_fp8_facts_the_reference_tests_hold(lane, fmt, bound):
+    """The statements of the reference's own fp8 tests (tests/unit/test_phase_e_f.py:474-516):
+    round-trip error bound per format, dequantize is the identity on x_q, an explicit scale
+    saturates at the format's max_normal, zeros stay zeros, an unknown format is a ValueError."""
+    rng = np.random.RandomState(0)
+    x = (rng.randn(64) * 50.0).astype(np.float32)
+    x_q, scale = ops.quantize_fp8(x, format=fmt)
+    assert float((np.abs(x - x_q) / (np.abs(x) + 1e-6)).max()) <= bound
+    assert np.array_equal(ops.dequantize_fp8(x_q, scale, format=fmt), x_q)
+    huge = np.array([1e6, -1e6], np.float32)
+    top = 448.0 if fmt == "e4m3" else 57344.0
+    assert np.array_equal(ops.quantize_fp8(huge, format=fmt, scale=1.0)[0], [top, -top])
+    assert np.array_equal(ops.quantize_fp8(np.zeros(4, np.float32), format=fmt)[0], np.zeros(4))
+    with pytest.raises(ValueError, match="format"):
+        ops.quantize_fp8(np.array([1.0], np.float32), format="e3m4")
+    with pytest.raises(ValueError, match="format"):
+        ops.dequantize_fp8(x_q, scale, format="e3m4")
