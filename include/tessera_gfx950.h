@@ -523,7 +523,7 @@ int tessera_gfx950_moe_unpack_combine_f32_dev(const void* y_packed, const int32_
                                               void* stream);
 
 /* tessera.moe_dispatch: x_perm[s,:] = x[token_of_slot[s],:]  (exact gather,
- * python/tessera/runtime.py:1791-1806).  elem_bytes = 2 (f16/bf16) or 4 (f32). */
+ * python/tessera/runtime.py:1791-1806).  elem_bytes = 1, 2 (f16/bf16), 4 (f32) or 8 (f64): rows are copied byte for byte. */
 int tessera_gfx950_moe_dispatch(const void* x, const int32_t* token_of_slot, void* x_perm,
                                 int T, int S, int H, int elem_bytes);
 int tessera_gfx950_moe_dispatch_dev(const void* x, const int32_t* token_of_slot, void* x_perm,

@@ -657,7 +657,7 @@ int combine_dev(const void* y, const int32_t* token_of_slot, const float* w, flo
 
 int dispatch_dev(const void* x, const int32_t* token_of_slot, void* x_perm, int T, int S, int H, int elem_bytes,
                  hipStream_t s) {
-  if (T <= 0 || S < 0 || H <= 0 || (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) || !x ||
+  if (T <= 0 || S < 0 || H <= 0 || (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8) || !x ||
       (S > 0 && (!token_of_slot || !x_perm)))
     return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
@@ -1162,7 +1162,7 @@ int tessera_gfx950_moe_dispatch_dev(const void* x, const int32_t* token_of_slot,
 
 int tessera_gfx950_moe_dispatch(const void* x, const int32_t* token_of_slot, void* x_perm, int T, int S, int H,
                                 int elem_bytes) {
-  if (T <= 0 || S < 0 || H <= 0 || (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) || !x ||
+  if (T <= 0 || S < 0 || H <= 0 || (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8) || !x ||
       (S > 0 && (!token_of_slot || !x_perm)))
     return kBadShape;
   for (int s = 0; s < S; ++s)

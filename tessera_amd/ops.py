@@ -1001,8 +1001,8 @@ def moe_dispatch(x, plan: MoETransport):
         xa, wrap = _bf16.as_bits(x), (lambda b: b.view(BF16Array))
     else:
         xa = np.ascontiguousarray(x)
-        if xa.dtype not in (np.float16, np.float32):
-            raise ValueError("moe_dispatch takes f16, bf16 or f32 rows")
+        if xa.dtype not in (np.float16, np.float32, np.float64):
+            raise ValueError("moe_dispatch takes f16, bf16, f32 or f64 rows")
         wrap = lambda b: b
     if xa.ndim != 2:
         raise ValueError(f"moe_dispatch x must be 2-D (T,H); got {xa.shape}")

@@ -620,3 +620,17 @@ def test_route_tokens_facts_the_reference_tests_hold(lane):
     assert res.overflow > 0 and res.overflow == int((res.assignment < 0).sum())
     assert ops.MoEConfig(num_experts=8, expert_capacity=50).compute_capacity(num_tokens=128) == 50
     assert ops.MoEConfig(num_experts=8, capacity_factor=1.25).compute_capacity(num_tokens=128) == 20
+
+
+def test_dispatch_combine_round_trip_with_unit_weights(lane):
+    """combine(dispatch(x)) with unit weights and no capacity is k times x
+    (tests/unit/test_stdlib_moe.py:68-79), on f64 rows as the reference's test feeds them."""
+    rng = np.random.default_rng(2)
+    H, E, k, T = 8, 5, 2, 10
+    x = rng.standard_normal((T, H)).astype(np.float64)
+    eids = rng.integers(0, E, size=(T, k)).astype(np.int64)
+    plan = ops.plan_dispatch(eids, np.ones((T, k), np.float32), E, capacity=None)
+    packed = ops.dispatch(x, plan)
+    assert packed.dtype == np.float64 and np.array_equal(packed, x[plan.sort_perm // k])
+    np.testing.assert_allclose(ops.combine(packed, plan), x * k, rtol=1e-6, atol=1e-6)
+    assert ops.compute_capacity(16, 2, 8, 1.5) == 6 and ops.compute_capacity(16, 2, 8, 1.0) == 4

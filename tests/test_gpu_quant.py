@@ -445,3 +445,18 @@ def test_fp8_facts_the_reference_tests_hold(lane, fmt, bound):
         ops.quantize_fp8(np.array([1.0], np.float32), format="e3m4")
     with pytest.raises(ValueError, match="format"):
         ops.dequantize_fp8(x_q, scale, format="e3m4")
+
+
+@pytest.mark.parametrize("quant,bound", [("fp8_e4m3", 0.06), ("fp8_e5m2", 0.30), ("nvfp4", 0.20), ("fp8xfp4", 0.20)])
+def test_quantised_grouped_gemm_inside_the_reference_budgets(lane, quant, bound):
+    """The normwise error budgets the reference's own tests give each scheme against the
+    unquantised grouped product (tests/unit/test_grouped_gemm_contract.py:223-229)."""
+    rng = np.random.default_rng(11)
+    gs = [16, 16, 32]
+    x32 = rng.standard_normal((sum(gs), 64)).astype(np.float32)
+    w32 = rng.standard_normal((len(gs), 64, 16)).astype(np.float32)
+    x, w = b16.from_float32(x32), b16.from_float32(w32)
+    ref = orc.grouped_gemm(x.to_float32(), w.to_float32(), gs, store=False)
+    got = ops.grouped_gemm(x, w, gs, quant=quant, out="f32")
+    rel = np.linalg.norm(got - ref) / (np.linalg.norm(ref) + 1e-9)
+    assert rel < bound, f"{quant}: {rel:.4f}"
