@@ -337,6 +337,24 @@ def bench_quant(lane, steps, warmup, check=True):
                                                         "(includes quantising the whole 8192 x 8192 weight); "
                                                         "the full workload has 64x the rows"}
     out["gemm_w8a8_scaled_4096x8192x8192"] = w8
+    # quantised decode: a few rows of int8 activations against the same 8192 x 8192 int8 weight, launches cycling
+    # over four copies of it so that the 67 MB do not sit in the memory-side cache (HBM-bound: one pass over B)
+    wcopies = [wq] + [lane.DeviceBuffer(K * N) for _ in range(3)]
+    for c in wcopies[1:]:
+        lane.check(lib.tessera_gfx950_memcpy_d2d_dev(c.ptr, wq.ptr, K * N, None), "copy")
+    lane.synchronize()
+    for Md in (1, 16, 32):
+        turn = [0]
+        def dec():
+            turn[0] += 1
+            lane.check(lib.tessera_gfx950_gemm_w8a8_f32_dev(xq.ptr, wcopies[turn[0] & 3].ptr, rs.ptr, cs.ptr, dd.ptr, None,
+                                                            Md, N, K, None), "gemm_w8a8")
+        _, ev = _timed(lane, dec, max(steps, 50), warmup)
+        dbytes = 1.0 * K * N + Md * K + 4.0 * Md * N
+        out[f"gemm_w8a8_decode_M{Md}_8192x8192"] = {"ms": ev, "gbs": dbytes / ev / 1e6,
+                                                    "frac_hbm_peak": dbytes / ev / 1e6 / PEAK_HBM_GBS, "weights_cycled": 4}
+    for c in wcopies[1:]:
+        c.close()
     # the int8 matrix pipes' own rate on such codes, no memory access: the ceiling of both rows above
     c8 = mfma_ceiling(lane, _OPTS["ceiling_seconds"], "int8")
     out["mfma_ceiling_int8"] = c8

@@ -16,6 +16,9 @@ pytestmark = pytest.mark.gpu
                                    (7, 13, 5), (100, 36, 1000), (512, 1024, 2048),
                                    # few tiles, long K: split along K (2, 4, 8, 16 slices; a ragged last slice)
                                    (16, 2048, 4096), (300, 1024, 8192), (128, 512, 16384), (1, 256, 40000), (40, 528, 2304),
+                                   # at most 32 rows, K a multiple of 64 from 2048 up: the streaming kernel (strips of 128
+                                   # columns, a ragged last strip and last K split, one row, 32 rows)
+                                   (1, 8192, 8192), (32, 144, 2048), (3, 8208, 4160), (31, 4096, 12352), (17, 272, 2112),
                                    # K or N off the 16-byte grid, large: aligned zero-padded copies and the tile kernel
                                    (517, 1003, 771), (300, 2050, 4100), (64, 5000, 1001)])
 def test_int8_gemm_bit_exact(lane, M, N, K):
@@ -55,6 +58,7 @@ def test_quantize_int8_matches_oracle(lane, M, N, K):
 
 
 @pytest.mark.parametrize("M,K,N", [(320, 512, 272), (48, 4096, 2048), (200, 8192, 512),    # the last two: K split
+                                   (1, 4096, 4096), (24, 2112, 400),                      # the few-row streaming kernel
                                    (333, 1001, 1030)])                                       # unaligned, large
 def test_w8a8_matmul(lane, M, K, N):
     rng = np.random.default_rng(8)
@@ -117,6 +121,7 @@ def test_e4m3_quantiser_matches_oracle(lane):
 
 @pytest.mark.parametrize("M,N,K", [(64, 64, 64), (256, 512, 1024), (130, 272, 208), (9, 21, 13),
                                    (16, 2048, 4096), (300, 1024, 8192), (128, 512, 16400),    # these three: K split
+                                   (1, 8192, 8192), (32, 144, 2048), (3, 8208, 4160), (17, 272, 2112),   # the few-row streaming kernel
                                    (517, 1003, 771), (300, 2050, 4100)])                      # unaligned, large
 def test_fp8_gemm(lane, M, N, K):
     rng = np.random.default_rng(6)
