@@ -114,26 +114,35 @@ int gemm8_dev(Gemm8Params p, hipStream_t s) {
   // At most 32 rows against a long K (quantised decode): the streaming kernel, one workgroup per
   // 128-column strip and K range, about one workgroup per compute unit and at least two 64-row
   // slices for each of its 8 waves; its raw accumulators go through the split sum below.
-  if (p.M <= G8S_MAX_M && p.K % G8S_ROWS == 0 && p.K >= 2048) {
-    // (8 waves and about 256 workgroups measured best: 4-wave workgroups, two per compute unit, and
-    // 384 or 512 workgroups were level or slower on M = 1 ... 32 against 4096 ... 28672 columns)
-    constexpr int NW = 8;
-    auto kern = gemm8_skinny_kernel<T, NW>;
+  if (p.M <= 64 && p.K % G8S_ROWS == 0 && p.K >= 2048) {
+    // (8 waves and about 256 workgroups measured best for up to 32 rows: 4-wave workgroups, two per
+    // compute unit, and 384 or 512 workgroups were level or slower on M = 1 ... 32 against 4096 ...
+    // 28672 columns.  33 to 64 rows double the accumulators: 4 waves, one per SIMD.)
+    const int nw = p.M <= 32 ? 8 : 4;
+    const int smem = p.M <= 32 ? g8s_smem(8, 1) : g8s_smem(4, 2);
+    const void* kern = p.M <= 32 ? reinterpret_cast<const void*>(gemm8_skinny_kernel<T, 8, 1>)
+                                 : reinterpret_cast<const void*>(gemm8_skinny_kernel<T, 4, 2>);
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [&] {
-      attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     g8s_smem(NW));
+      attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_skinny_kernel<T, 8, 1>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, g8s_smem(8, 1));
+      if (attr_err == hipSuccess)
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_skinny_kernel<T, 4, 2>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, g8s_smem(4, 2));
     });
     if (attr_err != hipSuccess) return kDeviceFailed;
     const int strips = ceil_div(p.N, G8S_COLS);
-    int splits = std::max(1, std::min((256 + strips / 2) / strips, p.K / (2 * NW * G8S_ROWS)));
+    int splits = std::max(1, std::min((256 + strips / 2) / strips, p.K / (2 * nw * G8S_ROWS)));
     const int kps = ceil_div(ceil_div(p.K, splits), G8S_ROWS) * G8S_ROWS;
     splits = ceil_div(p.K, kps);
     void* ws = stream_workspace(s, (size_t)splits * p.M * p.N * 4);
     if (!ws) return kDeviceFailed;
-    hipLaunchKernelGGL(kern, dim3(strips, splits), dim3(NW * 64), g8s_smem(NW), s, p.A, p.B, ws, p.M, p.N, p.K, kps);
-    if (int rc = launch_status(); rc != kOk) return rc;
+    void* args[] = {(void*)&p.A, (void*)&p.B, (void*)&ws, (void*)&p.M, (void*)&p.N, (void*)&p.K, (void*)&kps};
+    if (hipLaunchKernel(kern, dim3(strips, splits), dim3(nw * 64), args, smem, s) != hipSuccess) {
+      (void)hipGetLastError();
+      return kDeviceFailed;
+    }
     const long quads = (long)p.M * (p.N / 4);
     hipLaunchKernelGGL((gemm8_split_sum_kernel<T, EPI>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, ws,
                        splits, p);

@@ -19,6 +19,7 @@ pytestmark = pytest.mark.gpu
                                    # at most 32 rows, K a multiple of 64 from 2048 up: the streaming kernel (strips of 128
                                    # columns, a ragged last strip and last K split, one row, 32 rows)
                                    (1, 8192, 8192), (32, 144, 2048), (3, 8208, 4160), (31, 4096, 12352), (17, 272, 2112),
+                                   (33, 8208, 2112), (64, 272, 4096), (50, 1024, 8192),       # 33 to 64 rows: two row blocks a wave
                                    # K or N off the 16-byte grid, large: aligned zero-padded copies and the tile kernel
                                    (517, 1003, 771), (300, 2050, 4100), (64, 5000, 1001)])
 def test_int8_gemm_bit_exact(lane, M, N, K):
@@ -122,6 +123,7 @@ def test_e4m3_quantiser_matches_oracle(lane):
 @pytest.mark.parametrize("M,N,K", [(64, 64, 64), (256, 512, 1024), (130, 272, 208), (9, 21, 13),
                                    (16, 2048, 4096), (300, 1024, 8192), (128, 512, 16400),    # these three: K split
                                    (1, 8192, 8192), (32, 144, 2048), (3, 8208, 4160), (17, 272, 2112),   # the few-row streaming kernel
+                                   (33, 8208, 2112), (64, 272, 4096),
                                    (517, 1003, 771), (300, 2050, 4100)])                      # unaligned, large
 def test_fp8_gemm(lane, M, N, K):
     rng = np.random.default_rng(6)
