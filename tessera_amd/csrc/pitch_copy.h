@@ -10,7 +10,11 @@ namespace tsr950 {
 // threadIdx.y over rows, blockIdx.z over the batch.  The side of any alignment is accessed with one
 // 16-byte instruction where the whole chunk is inside the row (global memory takes accesses off
 // their natural alignment), element by element at the row's end.
-template <class E> struct __attribute__((packed, aligned(sizeof(E)))) LooseChunk { uint4 v; };
+// (the field is a plain vector type: a packed attribute is ignored on a field of class type, which would
+// leave the struct 16-byte aligned and the access free to assume it)
+template <class E> struct __attribute__((packed, aligned(sizeof(E)))) LooseChunk { u32x4 v; };
+static_assert(alignof(LooseChunk<uint8_t>) == 1 && alignof(LooseChunk<uint16_t>) == 2 && sizeof(LooseChunk<uint16_t>) == 16,
+              "LooseChunk must carry its element's alignment");
 constexpr int kCopyRowsPerBlock = 4;
 
 // dst[b][r][c] (rows_dst x ld_dst, 16-byte aligned) = src[b][r][c] inside rows_src x cols_src, else 0.
@@ -27,7 +31,8 @@ pad_rows_kernel(E* __restrict__ dst, long ld_dst, long stride_dst, const E* __re
     if (r < rows_src && c0 < cols_src) {
       const E* sp = src + b * stride_src + (long)r * ld_src + c0;
       if (c0 + V <= cols_src) {
-        out = reinterpret_cast<const LooseChunk<E>*>(sp)->v;
+        const u32x4 t = reinterpret_cast<const LooseChunk<E>*>(sp)->v;
+        out = make_uint4(t[0], t[1], t[2], t[3]);
       } else {
         alignas(16) E v[V];
 #pragma unroll
@@ -51,7 +56,7 @@ unpad_rows_kernel(E* __restrict__ dst, long ld_dst, long stride_dst, const E* __
     const uint4 in = *reinterpret_cast<const uint4*>(src + b * stride_src + (long)r * ld_src + c0);
     E* dp = dst + b * stride_dst + (long)r * ld_dst + c0;
     if (c0 + V <= cols) {
-      reinterpret_cast<LooseChunk<E>*>(dp)->v = in;
+      reinterpret_cast<LooseChunk<E>*>(dp)->v = u32x4{in.x, in.y, in.z, in.w};
     } else {
       alignas(16) E v[V];
       *reinterpret_cast<uint4*>(v) = in;
