@@ -138,8 +138,8 @@ inline bool decode_shaped(const FlashParams& p) {
 
 // Contiguous [B, H, S, D].
 inline FlashStrides bhsd(int H, int S, int D) { return FlashStrides{(long)H * S * D, (long)S * D, (long)D}; }
-// [B, S, H, D]: the rows of a (B * S) x (H * D) matrix, one head's D columns at a time.
-inline FlashStrides bshd(int H, int S, int D) { return FlashStrides{(long)S * H * D, (long)D, (long)H * D}; }
+// ([B, S, H, D], the rows of a (B * S) x (H * D) matrix one head's D columns at a time, is
+// {S * H * D, D, H * D}: callers of the strided entry points pass it themselves.)
 
 bool bad_strides(const FlashStrides& st) {
   return st.batch < 0 || st.head < 0 || st.row <= 0;
