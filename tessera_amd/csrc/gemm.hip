@@ -3,6 +3,7 @@
 #include <cmath>
 #include "../../include/tessera_gfx950.h"
 #include "gemm16_launch.h"
+#include "gemm8_schedule.h"
 
 namespace tsr950 {
 namespace {
@@ -325,10 +326,12 @@ int tessera_gfx950_gemm_schedule(int M, int N, int K, int batch, int elem_bytes,
     *split_k = sch.split_k;
     return kOk;
   }
-  if (elem_bytes == 1) {                     // int8 / fp8: one 256 x 256 x 128 tile shape
-    *tile_m = *tile_n = 256;
-    *tile_k = 128;
-    *split_k = 1;
+  if (elem_bytes == 1) {                     // int8 / fp8 (a single product: batch is not used)
+    const Gemm8Schedule sch = select_gemm8_schedule(M, N, K);
+    *tile_m = sch.tile_m;
+    *tile_n = sch.tile_n;
+    *tile_k = sch.tile_k;
+    *split_k = sch.split_k;
     return kOk;
   }
   return kBadShape;

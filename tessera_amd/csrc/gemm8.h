@@ -53,6 +53,7 @@ constexpr int G8_ASTAGE = G8_BM * G8_APITCH;
 constexpr int G8_BSTAGE = G8_BK * G8_BPITCH;
 constexpr int G8_STAGE = G8_ASTAGE + G8_BSTAGE;
 constexpr int G8_SMEM = 2 * G8_STAGE;
+constexpr int g8_smem(int bm) { return 2 * (bm * G8_APITCH + G8_BSTAGE); }   // LDS of a tile of bm rows
 
 __device__ __forceinline__ void tile_of_block8(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int total = tiles_m * tiles_n;
@@ -68,12 +69,16 @@ __device__ __forceinline__ void tile_of_block8(int bid, int tiles_m, int tiles_n
   tn = r / rows;
 }
 
-template <class T, int EPI>
+// BM: rows of the workgroup tile, 256 or 128 (the 2 x 2 waves then own 64 rows x 128 columns each: twice the
+// tiles to fill the chip with when a product has few of them).
+template <class T, int EPI, int BM = G8_BM>
 __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
+  static_assert(BM == 256 || BM == 128, "tile rows");
+  constexpr int ASTAGE = BM * G8_APITCH, STAGE = ASTAGE + G8_BSTAGE, SMEM = 2 * STAGE;
   constexpr bool IS_I8 = std::is_same<T, I8>::value;
-  constexpr int MI = 4, NJ = 4;
+  constexpr int MI = BM / 64, NJ = 4;
   constexpr int NT = 256;
-  constexpr int A_CHUNKS = G8_BM * 8 / NT;                 // 8
+  constexpr int A_CHUNKS = BM * 8 / NT;                 // 8
   constexpr int B_CHUNKS = G8_BK * (G8_BN / 16) / NT;      // 8
   // MFMA k steps per 128-byte tile: 4 x 32 (int8) or 2 x 64 (fp8).
   constexpr int KS = IS_I8 ? 4 : 2;
@@ -87,7 +92,7 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
 
   int tm, tn;
   tile_of_block8(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
-  const int m_begin = tm * G8_BM, n_begin = tn * G8_BN;
+  const int m_begin = tm * BM, n_begin = tn * G8_BN;
   // K range of this workgroup: all of it, or slice blockIdx.y of a split product.  (`K` below is the
   // length of the range; rows of A are p.K bytes apart either way.)
   const int kz = p.ksplit > 0 ? (int)blockIdx.y * p.ksplit : 0;
@@ -116,7 +121,7 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
     int gc = nch * 16;
     gc = n_begin + gc < p.N ? gc : p.N - 16 - n_begin;         // clamp: columns past the edge are never stored
     b_off[q] = (uint32_t)krow * (uint32_t)p.N + gc;
-    b_lds[q] = G8_ASTAGE + krow * G8_BPITCH + nch * 16;
+    b_lds[q] = ASTAGE + krow * G8_BPITCH + nch * 16;
     b_krow[q] = krow;
   }
 
@@ -149,7 +154,7 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
   };
   auto gload1 = [&](int q, int k0, auto guarded_c) { st[q] = gfetch(q, k0, guarded_c); };
   auto lstore1 = [&](int q, int buf) {
-    char* base = smem + buf * G8_STAGE;
+    char* base = smem + buf * STAGE;
     if (q < A_CHUNKS) lds_write_b128(base, a_lds[q], st[q]);
     else lds_write_b128(base, b_lds[q - A_CHUNKS], st[q]);
   };
@@ -169,14 +174,14 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
   int a_sw[MI];
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
-    const int row = wm * 128 + i * 32 + l32;
+    const int row = wm * (BM / 2) + i * 32 + l32;
     a_rd[i] = row * G8_APITCH;
     a_sw[i] = (row >> 1) & 7;
   }
   // Transposing byte read: lane r of a 16-lane block supplies row k0 + r/2 and
   // columns n0 + 8 (r % 2) .. +7; lane i receives column n0 + i, k0 .. k0+7.
   const int r16 = lane & 15;
-  const uint32_t b_rd0 = G8_ASTAGE + (16 * lh + (r16 >> 1)) * G8_BPITCH +
+  const uint32_t b_rd0 = ASTAGE + (16 * lh + (r16 >> 1)) * G8_BPITCH +
                          (wn * 128 + 16 * ((lane >> 4) & 1) + 8 * (r16 & 1));
 
   acc_t acc[MI][NJ];
@@ -191,7 +196,7 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
   // half its 16 bytes [32 f + 16 h, +16).
   uint4 af[2][MI][FR], bf[2][NJ][FR];
   auto frag_load = [&](int buf, int ks, int slot) {
-    const char* base = smem + buf * G8_STAGE;
+    const char* base = smem + buf * STAGE;
 #pragma unroll
     for (int x = 0; x < FR; ++x) {
       const int f = ks * FR + x;
@@ -324,8 +329,8 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
   constexpr int DSZ = EPI == EPI8_SCALED_BF16 ? 2 : 4;
   constexpr int ROWB = NJ * 32 * DSZ;                  // bytes of one row of the wave's 128-column tile
   constexpr int PITCH = ROWB + 16;
-  constexpr int WAVE_LDS = G8_SMEM / 4;
-  constexpr int IB = WAVE_LDS / (32 * PITCH) >= MI ? MI : 2;   // 32-row blocks staged per pass
+  constexpr int WAVE_LDS = SMEM / 4;
+  constexpr int IB = WAVE_LDS / (32 * PITCH) >= MI ? MI : (WAVE_LDS / (32 * PITCH) >= 2 ? 2 : 1);   // 32-row blocks staged per pass
   static_assert(IB * 32 * PITCH <= WAVE_LDS && MI % IB == 0, "epilogue staging does not fit");
   constexpr int LPR = ROWB / 16, RPI = 64 / LPR;       // lanes per row, rows per store instruction
   __syncthreads();                                     // nobody reads the operand tiles any more
@@ -345,7 +350,7 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
         const int i = i0 + ii;
         float rs = 1.f;
         if constexpr (EPI == EPI8_W8A8_F32 && !RAW) {
-          const int m = m_begin + wm * 128 + i * 32 + l32;
+          const int m = m_begin + wm * (BM / 2) + i * 32 + l32;
           rs = p.row_scale[m < p.M ? m : p.M - 1];
         }
 #pragma unroll
@@ -387,7 +392,7 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
       for (int it = 0; it < IB * 32 / RPI; ++it) {
         const int row = it * RPI + st_row;
         const uint4 v = lds_read_b128(stg, row * PITCH + st_chunk * 16);
-        const int m = m_begin + wm * 128 + i0 * 32 + row;
+        const int m = m_begin + wm * (BM / 2) + i0 * 32 + row;
         // N % 16 == 0 on this path: a 16-byte chunk is inside or outside as a whole
         if (m < p.M && st_n < p.N) *reinterpret_cast<uint4*>(out + ((long)m * p.N + st_n) * PDSZ) = v;
       }

@@ -5,6 +5,7 @@
 #include "../../include/tessera_gfx950.h"
 #include "gemm8.h"
 #include "gemm8_skinny.h"
+#include "gemm8_schedule.h"
 #include "host_util.h"
 #include "pitch_copy.h"
 
@@ -14,13 +15,13 @@ namespace {
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // The tile kernel needs more dynamic LDS than the default limit: raised once per instantiation.
-template <class T, int EPI>
+template <class T, int EPI, int BM = G8_BM>
 int gemm8_attr() {
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [&] {
-    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_kernel<T, EPI>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, G8_SMEM);
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_kernel<T, EPI, BM>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, g8_smem(BM));
   });
   return attr_err == hipSuccess ? kOk : kDeviceFailed;
 }
@@ -111,10 +112,8 @@ int gemm8_dev(Gemm8Params p, hipStream_t s) {
     hipLaunchKernelGGL((gemm8_generic_kernel<T, EPI>), grid, block, 0, s, p);
     return launch_status();
   }
-  // At most 32 rows against a long K (quantised decode): the streaming kernel, one workgroup per
-  // 128-column strip and K range, about one workgroup per compute unit and at least two 64-row
-  // slices for each of its 8 waves; its raw accumulators go through the split sum below.
-  if (p.M <= 64 && p.K % G8S_ROWS == 0 && p.K >= 2048) {
+  const Gemm8Schedule sch = select_gemm8_schedule(p.M, p.N, p.K);
+  if (sch.skinny) {
     // (8 waves and about 256 workgroups measured best for up to 32 rows: 4-wave workgroups, two per
     // compute unit, and 384 or 512 workgroups were level or slower on M = 1 ... 32 against 4096 ...
     // 28672 columns.  33 to 64 rows double the accumulators: 4 waves, one per SIMD.)
@@ -133,9 +132,8 @@ int gemm8_dev(Gemm8Params p, hipStream_t s) {
     });
     if (attr_err != hipSuccess) return kDeviceFailed;
     const int strips = ceil_div(p.N, G8S_COLS);
-    int splits = std::max(1, std::min((256 + strips / 2) / strips, p.K / (2 * nw * G8S_ROWS)));
+    const int splits = sch.split_k;
     const int kps = ceil_div(ceil_div(p.K, splits), G8S_ROWS) * G8S_ROWS;
-    splits = ceil_div(p.K, kps);
     void* ws = stream_workspace(s, (size_t)splits * p.M * p.N * 4);
     if (!ws) return kDeviceFailed;
     void* args[] = {(void*)&p.A, (void*)&p.B, (void*)&ws, (void*)&p.M, (void*)&p.N, (void*)&p.K, (void*)&kps};
@@ -148,46 +146,36 @@ int gemm8_dev(Gemm8Params p, hipStream_t s) {
                        splits, p);
     return launch_status();
   }
-  p.tiles_m = ceil_div(p.M, G8_BM);
+  const int bm = sch.tile_m, splits = sch.split_k;
+  p.tiles_m = ceil_div(p.M, bm);
   p.tiles_n = ceil_div(p.N, G8_BN);
   p.ksplit = 0;
-  // Few tiles and a long K (few rows against a big weight matrix): K is split over the idle compute
-  // units, the slices write raw accumulators to the stream workspace and a second kernel sums them
-  // and applies the epilogue.  The number of slices (a power of two, tiles x slices within the 256
-  // compute units, every slice at least 512 deep) is the one with the least estimated time: a tile
-  // costs 9.6 us plus 1.2 us per 128-deep K step, the sum kernel reads the partials and writes the
-  // result at about 4.4 TB/s (figures fitted to timings on this part).
   const int tiles = p.tiles_m * p.tiles_n;
-  int splits = 1;
-  if (tiles <= 128) {
-    const int ksteps = ceil_div(p.K, G8_BK);
-    double best_us = 9.6 + 1.2 * ksteps;
-    for (int sp = 2; sp <= 16 && tiles * sp <= 256 && p.K / sp >= 512; sp *= 2) {
-      const double us = 9.6 + 1.2 * ceil_div(ksteps, sp) + 2.0 + (double)p.M * p.N * (4.0 * sp + 4.0) / 4.4e6;
-      if (us < best_us) { best_us = us; splits = sp; }
+  auto launch = [&](auto bm_c) -> int {
+    constexpr int BM = decltype(bm_c)::value;
+    if (splits > 1) {
+      // raw accumulators: int32 for int8 operands, f32 with unit scales for fp8
+      constexpr int RAW_EPI = std::is_same<T, I8>::value ? EPI8_I32 : EPI8_SCALED_F32;
+      if (int rc = gemm8_attr<T, RAW_EPI, BM>(); rc != kOk) return rc;
+      void* ws = stream_workspace(s, (size_t)splits * p.M * p.N * 4);
+      if (!ws) return kDeviceFailed;
+      Gemm8Params q = p;
+      q.D = ws;
+      q.acc_out = nullptr;
+      q.scale_a = q.scale_b = 1.f;
+      q.ksplit = ceil_div(ceil_div(p.K, G8_BK), splits) * G8_BK;
+      hipLaunchKernelGGL((gemm8_kernel<T, RAW_EPI, BM>), dim3(tiles, splits), dim3(256), g8_smem(BM), s, q);
+      if (int rc = launch_status(); rc != kOk) return rc;
+      const long quads = (long)p.M * (p.N / 4);
+      hipLaunchKernelGGL((gemm8_split_sum_kernel<T, EPI>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, ws,
+                         splits, p);
+      return launch_status();
     }
-  }
-  if (splits > 1) {
-    // raw accumulators: int32 for int8 operands, f32 with unit scales for fp8
-    constexpr int RAW_EPI = std::is_same<T, I8>::value ? EPI8_I32 : EPI8_SCALED_F32;
-    if (int rc = gemm8_attr<T, RAW_EPI>(); rc != kOk) return rc;
-    void* ws = stream_workspace(s, (size_t)splits * p.M * p.N * 4);
-    if (!ws) return kDeviceFailed;
-    Gemm8Params q = p;
-    q.D = ws;
-    q.acc_out = nullptr;
-    q.scale_a = q.scale_b = 1.f;
-    q.ksplit = ceil_div(ceil_div(p.K, G8_BK), splits) * G8_BK;
-    hipLaunchKernelGGL((gemm8_kernel<T, RAW_EPI>), dim3(tiles, splits), dim3(256), G8_SMEM, s, q);
-    if (int rc = launch_status(); rc != kOk) return rc;
-    const long quads = (long)p.M * (p.N / 4);
-    hipLaunchKernelGGL((gemm8_split_sum_kernel<T, EPI>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, ws,
-                       splits, p);
+    if (int rc = gemm8_attr<T, EPI, BM>(); rc != kOk) return rc;
+    hipLaunchKernelGGL((gemm8_kernel<T, EPI, BM>), dim3(tiles), dim3(256), g8_smem(BM), s, p);
     return launch_status();
-  }
-  if (int rc = gemm8_attr<T, EPI>(); rc != kOk) return rc;
-  hipLaunchKernelGGL((gemm8_kernel<T, EPI>), dim3(tiles), dim3(256), G8_SMEM, s, p);
-  return launch_status();
+  };
+  return bm == 256 ? launch(std::integral_constant<int, 256>{}) : launch(std::integral_constant<int, 128>{});
 }
 
 // ---- quantisers ---------------------------------------------------------------

@@ -96,13 +96,15 @@ def select_gfx950_gemm_schedule(m: int, n: int, k: int, *, dtype: str = "bf16", 
     inst = _INSTRUCTION_TILE[name]
     if name in ("f16", "bf16") and max(tm.value, tn.value) == 256:
         inst = (16, 16, 32)       # the 256-wide tiles run v_mfma_f32_16x16x32 (less power per FLOP)
+    # the few-row streaming kernels: 32 x 64 strips (16-bit), 32 or 64 x 128 strips (8-bit)
+    streaming = tm.value == 32 or (nbytes == 1 and tn.value == 128)
     return Gfx950ScheduleDescriptor(
         arch="gfx950", dtype=name, instruction_tile=inst,
-        macro_tile=(tm.value // inst[0], tn.value // inst[1]),
+        macro_tile=(max(1, tm.value // inst[0]), tn.value // inst[1]),
         workgroup_tile=(tm.value, tn.value, tk.value),
         waves_per_cu=8 if tm.value == 32 else 4, pipeline_stages=2,
         lds_layout=("A from global in operand order; B wave-private [k][n] slices + transposing ds_read"
-                    if tm.value == 32 else "A xor-swizzled 16B chunks; B natural [k][n] + transposing ds_read"),
+                    if streaming else "A xor-swizzled 16B chunks; B natural [k][n] + transposing ds_read"),
         ownership="wave", vgpr_estimate=_VGPRS.get((tm.value, tn.value), 508), split_k=sk.value,
         source="tessera_gfx950_gemm_schedule (the launcher's own decision)",
         rest_tiles=rest_tiles.value, rest_split_k=rest_split.value)

@@ -330,6 +330,13 @@ def test_gemm_schedule_query_needs_no_device():
     q = sel(4096, 8192, 8192, dtype="int8")
     assert q.workgroup_tile == (256, 256, 128) and q.instruction_tile == (32, 32, 32)
     assert sel(4096, 8192, 8192, dtype="fp8_e4m3").instruction_tile == (32, 32, 64)
+    # 8-bit: fewer tiles take the 128-row tile, up to 64 rows the streaming kernel (K split over ~256 workgroups)
+    assert sel(1024, 8192, 8192, dtype="int8").workgroup_tile == (128, 256, 128)
+    assert sel(2048, 2048, 2048, dtype="int8").workgroup_tile[0] == 128
+    qd = sel(1, 8192, 8192, dtype="int8")
+    assert qd.workgroup_tile == (32, 128, 64) and qd.split_k == 4 and qd.waves_per_cu == 8 and "wave-private" in qd.lds_layout
+    assert sel(64, 8192, 8192, dtype="fp8_e4m3").workgroup_tile == (64, 128, 64)
+    assert sel(64, 8192, 1000, dtype="int8").workgroup_tile[2] == 128           # K off the slice grid: the tile kernel
     assert big.cache_key() != dec.cache_key()
     import pytest
     with pytest.raises(ValueError):
