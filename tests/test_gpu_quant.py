@@ -74,6 +74,22 @@ def test_w8a8_matmul(lane, M, K, N):
     assert orc.max_rel_err(y, X.astype(np.float64) @ W.astype(np.float64)) < 3e-2
 
 
+@pytest.mark.parametrize("M", [1, 48, 200, 1024])
+def test_int8_every_kernel_against_one_big_weight(lane, M):
+    """N = K = 8192 with 1, 48, 200 and 1024 rows — the streaming kernel with one and with two row blocks, the
+    128-row tile with K split and the 128-row tile on a full chip: sampled rows exact, and the checksum
+    of checksums of the whole result in exact integer arithmetic."""
+    N = K = 8192
+    rng = np.random.default_rng(M)
+    xq = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wq = rng.integers(-127, 128, (K, N)).astype(np.int8)
+    acc = ops.gemm_i8(xq, wq)
+    rows = rng.choice(M, min(M, 8), replace=False)
+    assert np.array_equal(acc[rows], orc.gemm_i8_i32(xq[rows], wq))
+    assert int(acc.astype(np.int64).sum()) == int(xq.astype(np.int64).sum(0) @ wq.astype(np.int64).sum(1))
+    assert np.array_equal(acc.astype(np.int64).sum(0), xq.astype(np.int64).sum(0) @ wq.astype(np.int64))
+
+
 def test_w8a8_headline_shape_properties(lane):
     """M=4096, N=K=8192: accumulators checked exactly on sampled rows/columns."""
     M, N, K = 4096, 8192, 8192
