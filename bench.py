@@ -407,6 +407,17 @@ def bench_quant(lane, steps, warmup, check=True):
         f8["cpu_baseline"] = {"value": 2.0 * len(sample) * N * K / dt / 1e12, "unit": "TFLOP/s", "cores": _blas_threads(),
                               "kind": "port", "sample": f"quantise both tensors + f64 product of 64 dequantised rows in "
                                                         f"numpy, {dt:.2f} s; the full workload has 64x the rows"}
+    # the same product on e5m2 codes (the matrix instruction's second fp8 operand format)
+    lane.check(lib.tessera_gfx950_quantize_e5m2_f32_dev(xf.ptr, M * K, 0.0, xq.ptr, sx.ptr, None), "quantize_e5m2")
+    lane.check(lib.tessera_gfx950_quantize_e5m2_f32_dev(wf.ptr, K * N, 0.0, wq.ptr, sw.ptr, None), "quantize_e5m2")
+    lane.synchronize()
+    s5a, s5b = float(sx.download((1,), np.float32)[0]), float(sw.download((1,), np.float32)[0])
+    _, ev = _timed(lane, lambda: lane.check(
+        lib.tessera_gfx950_gemm_e5m2_bf16_dev(xq.ptr, wq.ptr, ctypes.c_float(s5a), ctypes.c_float(s5b), dd.ptr,
+                                              M, N, K, None), "gemm_e5m2"), steps, warmup)
+    out["gemm_fp8_e5m2_4096x8192x8192"] = {"workload": "e5m2 codes of N(0,1) data, per-tensor scales amax/57344, bf16 out",
+                                           "ms": ev, "tflops": ops / ev / 1e9,
+                                           "frac_mfma_peak": ops / ev / 1e9 / PEAK_FP8_TFLOPS}
     cf = mfma_ceiling(lane, _OPTS["ceiling_seconds"], "fp8")
     out["mfma_ceiling_fp8"] = cf
     f8.update(_ceiling_fields(cf, f8["tflops"]))

@@ -140,6 +140,13 @@ int tessera_gfx950_gemm_e4m3_bf16(const void* A, const void* B, float scale_a, f
                                   void* D, int M, int N, int K);
 int tessera_gfx950_gemm_e4m3_f32(const void* A, const void* B, float scale_a, float scale_b,
                                  void* D, int M, int N, int K);
+/* The same over fp8 e5m2 (OCP) codes, the format table's second fp8 grid
+ * (python/tessera/runtime.py:16939-16940; GEMM over raw bytes as tessera_nvidia_mma_gemm_e5m2,
+ * compiler/codegen/tessera_gpu_backend_NVIDIA): the matrix instruction's operand format 1. */
+int tessera_gfx950_gemm_e5m2_bf16(const void* A, const void* B, float scale_a, float scale_b,
+                                  void* D, int M, int N, int K);
+int tessera_gfx950_gemm_e5m2_f32(const void* A, const void* B, float scale_a, float scale_b,
+                                 void* D, int M, int N, int K);
 
 int tessera_gfx950_gemm_f16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream);
 int tessera_gfx950_gemm_bf16_dev(const void* A, const void* B, void* D, int M, int N, int K, void* stream);
@@ -166,6 +173,10 @@ int tessera_gfx950_gemm_w8a8_f32_dev(const void* A, const void* B, const float* 
 int tessera_gfx950_gemm_e4m3_bf16_dev(const void* A, const void* B, float scale_a, float scale_b,
                                       void* D, int M, int N, int K, void* stream);
 int tessera_gfx950_gemm_e4m3_f32_dev(const void* A, const void* B, float scale_a, float scale_b,
+                                     void* D, int M, int N, int K, void* stream);
+int tessera_gfx950_gemm_e5m2_bf16_dev(const void* A, const void* B, float scale_a, float scale_b,
+                                      void* D, int M, int N, int K, void* stream);
+int tessera_gfx950_gemm_e5m2_f32_dev(const void* A, const void* B, float scale_a, float scale_b,
                                      void* D, int M, int N, int K, void* stream);
 
 /* Fused matmul epilogue  D f32 = act(A . B + bias[n]):  the bias operand and
@@ -267,6 +278,9 @@ int tessera_gfx950_mfma_probe_dev(int kind, const void* fragments, int rounds, v
  * byte of clip(x[i]/scale, +-448) rounded RNE.  scale <= 0 means "compute
  * max(amax/448, 1e-12)"; the scale used is written to *scale_out. */
 int tessera_gfx950_quantize_e4m3_f32(const float* x, int64_t n, float scale, void* codes, float* scale_out);
+/* The same to e5m2 codes: scale = max(amax / 57344, 1e-12), clip to +-57344, round to nearest even
+ * with gradual underflow below 2^-14 (the grid (57344, 2, -14) of the format table). */
+int tessera_gfx950_quantize_e5m2_f32(const float* x, int64_t n, float scale, void* codes, float* scale_out);
 /* _quantize_int8_per_channel (python/tessera/compiler/smoothquant.py:79-84):
  * axis=1 -> one scale per row (scales[M]); axis=0 -> one per column (scales[N]). */
 int tessera_gfx950_quantize_i8_f32(const float* x, int M, int N, int axis, void* q, float* scales);
@@ -316,6 +330,7 @@ int tessera_gfx950_fake_quantize_fp_f32(const float* x, int64_t n, float max_nor
 int tessera_gfx950_fake_quantize_fp_f32_dev(const float* x, int64_t n, float max_normal, int mantissa_bits, int min_exp,
                                             float scale, float* dq, void* grid_bf16, float* scale_out_dev, void* stream);
 int tessera_gfx950_quantize_e4m3_f32_dev(const float* x, int64_t n, float scale, void* codes, float* scale_out_dev, void* stream);
+int tessera_gfx950_quantize_e5m2_f32_dev(const float* x, int64_t n, float scale, void* codes, float* scale_out_dev, void* stream);
 int tessera_gfx950_quantize_i8_f32_dev(const float* x, int M, int N, int axis, void* q, float* scales, void* stream);
 
 /* ---- flash-attention forward ---------------------------------------------- */

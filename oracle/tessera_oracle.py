@@ -806,6 +806,44 @@ def grouped_gemm_quant(x, w, group_sizes, quant: str):
     return out
 
 
+def e5m2_decode_table() -> np.ndarray:
+    """All 256 OCP e5m2 codes -> f32 (bias 15, two mantissa bits, subnormal step 2^-16, exponent 31
+    = inf / NaN): the published format, i.e. the upper byte of IEEE half precision."""
+    t = np.zeros(256, np.float32)
+    for c in range(256):
+        s = -1.0 if c & 0x80 else 1.0
+        e = (c >> 2) & 0x1F
+        m = c & 3
+        if e == 0x1F:
+            t[c] = s * np.inf if m == 0 else np.nan
+        elif e == 0:
+            t[c] = s * m * 2.0 ** -16
+        else:
+            t[c] = s * (1.0 + m / 4.0) * 2.0 ** (e - 15)
+    return t
+
+
+def e5m2_encode(grid_values: np.ndarray) -> np.ndarray:
+    """f32 values that already lie on the e5m2 grid (finite) -> their byte codes."""
+    v = np.asarray(grid_values, np.float32)
+    h = v.astype(np.float16)                      # exact: every e5m2 value is a half
+    assert np.array_equal(h.astype(np.float32), v, equal_nan=True)
+    return (h.view(np.uint16) >> 8).astype(np.uint8)
+
+
+def quantize_fp8_e5m2(x: np.ndarray, scale: float | None = None):
+    """``ops.quantize_fp8(format="e5m2")`` (``__init__.py:3340-3374``) -> ``(codes uint8, grid f32,
+    scale np.float32)``: per-tensor ``scale = max(amax / 57344, 1e-12)``, clip, the (57344, 2, -14) grid."""
+    dq, grid, s = quantize_fp(x, "e5m2", scale)
+    return e5m2_encode(grid), grid, s
+
+
+def gemm_fp8_codes(a_codes, b_codes, scale_a, scale_b, fmt: str = "e4m3"):
+    """The fp8 GEMM on codes of either format, f64 accumulate: ``(A @ B) * sA * sB``."""
+    t = (e5m2_decode_table() if fmt == "e5m2" else e4m3_decode_table()).astype(np.float64)
+    return (t[np.asarray(a_codes, np.uint8)] @ t[np.asarray(b_codes, np.uint8)]) * float(np.float32(scale_a)) * float(np.float32(scale_b))
+
+
 def gemm_e4m3(a_codes, b_codes, scale_a, scale_b, out_dtype: str = "bf16"):
     """fp8 GEMM config: ``f32acc(Aq.Bq) * sA * sB`` stored in ``out_dtype``
     (f64 accumulate here).  Returns the f64 value before the final store; the

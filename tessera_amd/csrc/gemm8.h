@@ -22,7 +22,10 @@
 namespace tsr950 {
 
 struct I8 {};
-struct FP8 {};
+struct FP8 {};     // OCP e4m3fn
+struct BF8 {};     // OCP e5m2
+// operand format selector of the f8f6f4 matrix instruction: 0 = e4m3, 1 = e5m2
+template <class T> constexpr int f8_format() { return std::is_same<T, BF8>::value ? 1 : 0; }
 
 enum Gemm8Epilogue : int {
   EPI8_I32 = 0,        // I8: int32 accumulators
@@ -227,8 +230,9 @@ __global__ __launch_bounds__(256, 1) void gemm8_kernel(const Gemm8Params p) {
           const i32x4 a0 = __builtin_bit_cast(i32x4, af[slot][i][0]), a1 = __builtin_bit_cast(i32x4, af[slot][i][1]);
           b8 = (i32x8){b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
           a8 = (i32x8){a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-          // format selectors 0 = e4m3; zero scale operands select the unscaled form.
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, a8, acc[i][j], 0, 0, 0, 0, 0, 0);
+          // format selectors 0 = e4m3, 1 = e5m2; zero scale operands select the unscaled form.
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, a8, acc[i][j], f8_format<T>(), f8_format<T>(),
+                                                                      0, 0, 0, 0);
         }
       }
   };
@@ -422,6 +426,15 @@ __device__ __forceinline__ float e4m3_to_f32(uint8_t c) {
   return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) | s);
 }
 
+// e5m2 (OCP) byte -> f32: the byte is the upper half of the IEEE half-precision pattern.
+__device__ __forceinline__ float e5m2_to_f32(uint8_t c) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)((uint16_t)c << 8));
+}
+template <class T> __device__ __forceinline__ float f8_to_f32(uint8_t c) {
+  if constexpr (std::is_same<T, BF8>::value) return e5m2_to_f32(c);
+  else return e4m3_to_f32(c);
+}
+
 // A product split along K: the slices' partial results (int32 accumulators, or f32 ones of the fp8
 // form computed with unit scales), [splits][M][N], are summed in slice order and passed through
 // the product's epilogue.  int32 sums are exact, so the int8 forms give the bits of the unsplit
@@ -492,7 +505,7 @@ __global__ void gemm8_generic_kernel(const Gemm8Params p) {
     const uint8_t* A = p.A + (long)m * p.K;
     const uint8_t* B = p.B + n;
     float acc = 0.f;
-    for (int k = 0; k < p.K; ++k) acc += e4m3_to_f32(A[k]) * e4m3_to_f32(B[(long)k * p.N]);
+    for (int k = 0; k < p.K; ++k) acc += f8_to_f32<T>(A[k]) * f8_to_f32<T>(B[(long)k * p.N]);
     const float v = (acc * p.scale_a) * p.scale_b;
     if constexpr (EPI == EPI8_SCALED_F32) reinterpret_cast<float*>(p.D)[o] = v;
     else reinterpret_cast<uint16_t*>(p.D)[o] = f32_to_bf16_bits(v);

@@ -122,7 +122,8 @@ __global__ __launch_bounds__(G8S_NW * 64) void gemm8_skinny_kernel(const uint8_t
           const i32x4 x0 = __builtin_bit_cast(i32x4, af[mi][0]), x1 = __builtin_bit_cast(i32x4, af[mi][1]);
           const i32x8 b8 = (i32x8){b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
           const i32x8 a8 = (i32x8){x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-          acc[mi][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, a8, acc[mi][j], 0, 0, 0, 0, 0, 0);
+          acc[mi][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b8, a8, acc[mi][j], f8_format<T>(), f8_format<T>(),
+                                                                       0, 0, 0, 0);
         }
       }
   };

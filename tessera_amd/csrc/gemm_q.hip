@@ -237,19 +237,41 @@ __device__ __forceinline__ uint8_t f32_to_e4m3(float v) {
   return (uint8_t)(sign | code);
 }
 
-// scale_in > 0: use it; else scale = max(amax / 448, 1e-12) from *amax_bits.
-__global__ void quantize_e4m3_kernel(const float* x, long n, float scale_in, const unsigned* amax_bits,
-                                     uint8_t* codes, float* scale_out) {
+// f32 (already clipped to +-57344) -> e5m2 byte, round-to-nearest-even with gradual
+// underflow below 2^-14 (the IEEE half-precision pattern cut to two mantissa bits).
+__device__ __forceinline__ uint8_t f32_to_e5m2(float v) {
+  const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+  const uint8_t sign = (uint8_t)((bits >> 24) & 0x80);
+  const uint32_t ab = bits & 0x7fffffffu;
+  if (ab > 0x7f800000u) return (uint8_t)(sign | 0x7f);            // NaN
+  const float a = __builtin_bit_cast(float, ab);
+  uint32_t code;
+  if (a < 6.103515625e-05f) {                                     // below the smallest normal 2^-14
+    code = (uint32_t)__builtin_rintf(a * 65536.0f);               // multiples of 2^-16; 4 carries into 0x04
+  } else {
+    const uint32_t r = (ab + 0xfffffu + ((ab >> 21) & 1u)) >> 21; // (biased exp << 2) | 2-bit mantissa
+    code = r - (112u << 2);
+    if (code > 0x7bu) code = 0x7bu;                               // saturate at 57344
+  }
+  return (uint8_t)(sign | code);
+}
+
+// FMT 0: e4m3 (max 448), 1: e5m2 (max 57344).
+// scale_in > 0: use it; else scale = max(amax / max_normal, 1e-12) from *amax_bits.
+template <int FMT>
+__global__ void quantize_f8_kernel(const float* x, long n, float scale_in, const unsigned* amax_bits,
+                                   uint8_t* codes, float* scale_out) {
+  constexpr float MAXN = FMT == 0 ? 448.0f : 57344.0f;
   float scale = scale_in;
   if (!(scale_in > 0.f)) {
     const float amax = __builtin_bit_cast(float, *amax_bits);
-    scale = fmaxf(__fdiv_rn(amax, 448.0f), 1e-12f);
+    scale = fmaxf(__fdiv_rn(amax, MAXN), 1e-12f);
   }
   if (scale_out && blockIdx.x == 0 && threadIdx.x == 0) *scale_out = scale;
+  auto clip = [&](float f) { return fminf(fmaxf(__fdiv_rn(f, scale), -MAXN), MAXN); };
   auto code = [&](float f) -> uint32_t {
-    float t = __fdiv_rn(f, scale);
-    t = fminf(fmaxf(t, -448.0f), 448.0f);
-    return f32_to_e4m3(t);
+    if constexpr (FMT == 0) return f32_to_e4m3(clip(f));
+    else return f32_to_e5m2(clip(f));
   };
   const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x, nthreads = (long)gridDim.x * blockDim.x;
   // runs of 16 elements: four 16-byte loads, one 16-byte store (both pointers 16-byte aligned)
@@ -260,11 +282,16 @@ __global__ void quantize_e4m3_kernel(const float* x, long n, float scale_in, con
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const float4 v = reinterpret_cast<const float4*>(x)[g * 4 + c];
-      // the hardware conversion (OCP e4m3, round to nearest even, gradual underflow) on
-      // values already clipped to +-448 gives the codes of f32_to_e4m3
-      auto clip = [&](float f) { return fminf(fmaxf(__fdiv_rn(f, scale), -448.0f), 448.0f); };
-      int pk = __builtin_amdgcn_cvt_pk_fp8_f32(clip(v.x), clip(v.y), 0, false);
-      pk = __builtin_amdgcn_cvt_pk_fp8_f32(clip(v.z), clip(v.w), pk, true);
+      // the hardware conversion (OCP formats, round to nearest even, gradual underflow) on
+      // values already clipped to the format's range gives the codes of the software one
+      int pk;
+      if constexpr (FMT == 0) {
+        pk = __builtin_amdgcn_cvt_pk_fp8_f32(clip(v.x), clip(v.y), 0, false);
+        pk = __builtin_amdgcn_cvt_pk_fp8_f32(clip(v.z), clip(v.w), pk, true);
+      } else {
+        pk = __builtin_amdgcn_cvt_pk_bf8_f32(clip(v.x), clip(v.y), 0, false);
+        pk = __builtin_amdgcn_cvt_pk_bf8_f32(clip(v.z), clip(v.w), pk, true);
+      }
       w[c] = (uint32_t)pk;
     }
     reinterpret_cast<uint4*>(codes)[g] = make_uint4(w[0], w[1], w[2], w[3]);
@@ -410,6 +437,7 @@ __global__ __launch_bounds__(256) void quantize_i8_cols_vec_kernel(const float* 
   }
 }
 
+template <int FMT = 0>
 int quantize_e4m3_dev(const float* x, int64_t n, float scale, void* codes, float* scale_out_dev, hipStream_t s) {
   if (n <= 0 || !x || !codes) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
@@ -425,7 +453,7 @@ int quantize_e4m3_dev(const float* x, int64_t n, float scale, void* codes, float
     // 8 ns each: two workgroups per CU, not sixteen)
     hipLaunchKernelGGL(absmax_kernel, dim3(std::min(blocks, 512)), dim3(256), 0, s, x, (long)n, amax);
   }
-  hipLaunchKernelGGL(quantize_e4m3_kernel, dim3(blocks), dim3(256), 0, s, x, (long)n, scale, amax,
+  hipLaunchKernelGGL((quantize_f8_kernel<FMT>), dim3(blocks), dim3(256), 0, s, x, (long)n, scale, amax,
                      static_cast<uint8_t*>(codes), scale_out_dev);
   return launch_status();
 }
@@ -691,6 +719,22 @@ int gemm8_host(const void* A, const void* B, const float* rs, const float* cs, f
   return kOk;
 }
 
+template <int FMT>
+int quantize_f8_host(const float* x, int64_t n, float scale, void* codes, float* scale_out) {
+  if (n <= 0 || !x || !codes) return kBadShape;
+  if (probe_device() != kOk) return kNoDevice;
+  DeviceScope scope;
+  float* dx = static_cast<float*>(scope.alloc((size_t)n * 4, x));
+  void* dc = scope.alloc((size_t)n);
+  float* ds = static_cast<float*>(scope.alloc(4));
+  if (scope.failed()) return kDeviceFailed;
+  int rc = quantize_e4m3_dev<FMT>(dx, n, scale, dc, ds, nullptr);
+  if (rc != kOk) return rc;
+  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
+  if (!scope.download(codes, dc, (size_t)n)) return kDeviceFailed;
+  if (scale_out && !scope.download(scale_out, ds, 4)) return kDeviceFailed;
+  return kOk;
+}
 }  // namespace
 }  // namespace tsr950
 
@@ -712,6 +756,15 @@ int tessera_gfx950_gemm_e4m3_bf16(const void* A, const void* B, float scale_a, f
 int tessera_gfx950_gemm_e4m3_f32(const void* A, const void* B, float scale_a, float scale_b, void* D, int M,
                                  int N, int K) {
   return gemm8_host<FP8, EPI8_SCALED_F32>(A, B, nullptr, nullptr, scale_a, scale_b, D, nullptr, M, N, K);
+}
+
+int tessera_gfx950_gemm_e5m2_bf16(const void* A, const void* B, float scale_a, float scale_b, void* D, int M,
+                                  int N, int K) {
+  return gemm8_host<BF8, EPI8_SCALED_BF16>(A, B, nullptr, nullptr, scale_a, scale_b, D, nullptr, M, N, K);
+}
+int tessera_gfx950_gemm_e5m2_f32(const void* A, const void* B, float scale_a, float scale_b, void* D, int M,
+                                 int N, int K) {
+  return gemm8_host<BF8, EPI8_SCALED_F32>(A, B, nullptr, nullptr, scale_a, scale_b, D, nullptr, M, N, K);
 }
 
 int tessera_gfx950_gemm_i8_i32_dev(const void* A, const void* B, void* C, int M, int N, int K, void* stream) {
@@ -739,9 +792,26 @@ int tessera_gfx950_gemm_e4m3_f32_dev(const void* A, const void* B, float scale_a
   return gemm8_dev<FP8, EPI8_SCALED_F32>(p, as_stream(stream));
 }
 
+int tessera_gfx950_gemm_e5m2_bf16_dev(const void* A, const void* B, float scale_a, float scale_b, void* D,
+                                      int M, int N, int K, void* stream) {
+  Gemm8Params p = make_params(A, B, D, M, N, K);
+  p.scale_a = scale_a; p.scale_b = scale_b;
+  return gemm8_dev<BF8, EPI8_SCALED_BF16>(p, as_stream(stream));
+}
+int tessera_gfx950_gemm_e5m2_f32_dev(const void* A, const void* B, float scale_a, float scale_b, void* D,
+                                     int M, int N, int K, void* stream) {
+  Gemm8Params p = make_params(A, B, D, M, N, K);
+  p.scale_a = scale_a; p.scale_b = scale_b;
+  return gemm8_dev<BF8, EPI8_SCALED_F32>(p, as_stream(stream));
+}
+
 int tessera_gfx950_quantize_e4m3_f32_dev(const float* x, int64_t n, float scale, void* codes,
                                          float* scale_out_dev, void* stream) {
-  return quantize_e4m3_dev(x, n, scale, codes, scale_out_dev, as_stream(stream));
+  return quantize_e4m3_dev<0>(x, n, scale, codes, scale_out_dev, as_stream(stream));
+}
+int tessera_gfx950_quantize_e5m2_f32_dev(const float* x, int64_t n, float scale, void* codes,
+                                         float* scale_out_dev, void* stream) {
+  return quantize_e4m3_dev<1>(x, n, scale, codes, scale_out_dev, as_stream(stream));
 }
 int tessera_gfx950_quantize_i8_f32_dev(const float* x, int M, int N, int axis, void* q, float* scales,
                                        void* stream) {
@@ -818,19 +888,10 @@ int tessera_gfx950_fpquant_f32(const float* x, int64_t n, float max_normal, int 
 }
 
 int tessera_gfx950_quantize_e4m3_f32(const float* x, int64_t n, float scale, void* codes, float* scale_out) {
-  if (n <= 0 || !x || !codes) return kBadShape;
-  if (probe_device() != kOk) return kNoDevice;
-  DeviceScope scope;
-  float* dx = static_cast<float*>(scope.alloc((size_t)n * 4, x));
-  void* dc = scope.alloc((size_t)n);
-  float* ds = static_cast<float*>(scope.alloc(4));
-  if (scope.failed()) return kDeviceFailed;
-  int rc = quantize_e4m3_dev(dx, n, scale, dc, ds, nullptr);
-  if (rc != kOk) return rc;
-  if (hipDeviceSynchronize() != hipSuccess) return kDeviceFailed;
-  if (!scope.download(codes, dc, (size_t)n)) return kDeviceFailed;
-  if (scale_out && !scope.download(scale_out, ds, 4)) return kDeviceFailed;
-  return kOk;
+  return quantize_f8_host<0>(x, n, scale, codes, scale_out);
+}
+int tessera_gfx950_quantize_e5m2_f32(const float* x, int64_t n, float scale, void* codes, float* scale_out) {
+  return quantize_f8_host<1>(x, n, scale, codes, scale_out);
 }
 
 int tessera_gfx950_quantize_i8_tensor_f32(const float* x, int64_t n, float scale, void* q, float* scale_out) {

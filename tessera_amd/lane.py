@@ -86,7 +86,9 @@ _SIGNATURES = {
     "tessera_gfx950_gemm_i8_i32": _GEMM,
     "tessera_gfx950_gemm_w8a8_f32": [_c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int],
     "tessera_gfx950_gemm_e4m3_bf16": [_c_vp, _c_vp, _c_f, _c_f, _c_vp, _c_int, _c_int, _c_int],
+    "tessera_gfx950_gemm_e5m2_bf16": [_c_vp, _c_vp, _c_f, _c_f, _c_vp, _c_int, _c_int, _c_int],
     "tessera_gfx950_gemm_e4m3_f32": [_c_vp, _c_vp, _c_f, _c_f, _c_vp, _c_int, _c_int, _c_int],
+    "tessera_gfx950_gemm_e5m2_f32": [_c_vp, _c_vp, _c_f, _c_f, _c_vp, _c_int, _c_int, _c_int],
     "tessera_gfx950_gemm_f16_dev": _GEMM + [_c_vp],
     "tessera_gfx950_gemm_bf16_dev": _GEMM + [_c_vp],
     "tessera_gfx950_gemm_f16_f16_dev": _GEMM + [_c_vp],
@@ -124,7 +126,9 @@ _SIGNATURES = {
     "tessera_gfx950_gemm_i8_i32_dev": _GEMM + [_c_vp],
     "tessera_gfx950_gemm_w8a8_f32_dev": [_c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_gemm_e4m3_bf16_dev": [_c_vp, _c_vp, _c_f, _c_f, _c_vp, _c_int, _c_int, _c_int, _c_vp],
+    "tessera_gfx950_gemm_e5m2_bf16_dev": [_c_vp, _c_vp, _c_f, _c_f, _c_vp, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_gemm_e4m3_f32_dev": [_c_vp, _c_vp, _c_f, _c_f, _c_vp, _c_int, _c_int, _c_int, _c_vp],
+    "tessera_gfx950_gemm_e5m2_f32_dev": [_c_vp, _c_vp, _c_f, _c_f, _c_vp, _c_int, _c_int, _c_int, _c_vp],
     "tessera_gfx950_stream_release": [_c_vp],
     "tessera_gfx950_gemm_bf16_bench": [_c_int, _c_int, _c_int, _c_int, _P(ctypes.c_double)],
     "tessera_gfx950_gemm_f16_bench": [_c_int] * 6 + [_P(ctypes.c_double)],
@@ -133,8 +137,10 @@ _SIGNATURES = {
     "tessera_gfx950_mfma_probe_bf16_dev": [_c_vp, _c_int, _c_vp, _P(ctypes.c_double), _c_vp],
     "tessera_gfx950_mfma_probe_dev": [_c_int, _c_vp, _c_int, _c_vp, _P(ctypes.c_double), _c_vp],
     "tessera_gfx950_quantize_e4m3_f32": [_c_vp, _c_i64, _c_f, _c_vp, _P(_c_f)],
+    "tessera_gfx950_quantize_e5m2_f32": [_c_vp, _c_i64, _c_f, _c_vp, _P(_c_f)],
     "tessera_gfx950_quantize_i8_f32": [_c_vp, _c_int, _c_int, _c_int, _c_vp, _c_vp],
     "tessera_gfx950_quantize_e4m3_f32_dev": [_c_vp, _c_i64, _c_f, _c_vp, _c_vp, _c_vp],
+    "tessera_gfx950_quantize_e5m2_f32_dev": [_c_vp, _c_i64, _c_f, _c_vp, _c_vp, _c_vp],
     "tessera_gfx950_quantize_i8_f32_dev": [_c_vp, _c_int, _c_int, _c_int, _c_vp, _c_vp, _c_vp],
     "tessera_gfx950_flash_attn_f16": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int],
     "tessera_gfx950_flash_attn_bf16": [_c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int],

@@ -1198,12 +1198,24 @@ def e4m3_table() -> np.ndarray:
     return _E4M3_TABLE
 
 
-def quantize_fp8_codes(x, *, scale=None):
-    """Per-tensor e4m3 quantisation on the device → ``(codes uint8, scale f32)``."""
+def e5m2_table() -> np.ndarray:
+    """The 256 OCP e5m2 code values as f32 (a code is the upper byte of an IEEE half)."""
+    return (np.arange(256, dtype=np.uint16) << 8).view(np.float16).astype(np.float32)
+
+
+def _fp8_format(format: str) -> str:
+    if format not in ("e4m3", "e5m2"):
+        raise ValueError(f"format must be 'e4m3' or 'e5m2'; got {format!r}")
+    return format
+
+
+def quantize_fp8_codes(x, *, scale=None, format: str = "e4m3"):
+    """Per-tensor fp8 quantisation on the device → ``(codes uint8, scale f32)``; ``format``
+    ``"e4m3"`` or ``"e5m2"`` (the operand formats of :func:`gemm_fp8`)."""
     xa = np.ascontiguousarray(_unbox(x), np.float32)
     codes = np.empty(xa.shape, np.uint8)
     s_out = ctypes.c_float(0)
-    rc = _lane.load().tessera_gfx950_quantize_e4m3_f32(
+    rc = getattr(_lane.load(), f"tessera_gfx950_quantize_{_fp8_format(format)}_f32")(
         xa.ctypes.data, xa.size, float(scale) if scale is not None else 0.0, codes.ctypes.data,
         ctypes.byref(s_out))
     _lane.check(rc, "quantize_fp8")
@@ -1216,8 +1228,10 @@ def quantize_fp8(x, *, format: str = "e4m3", scale=None):
     return _quantize_per_tensor(x, format, ("e4m3", "e5m2"), scale)
 
 
-def gemm_fp8(a_codes, b_codes, scale_a, scale_b, *, out: str = "bf16"):
-    """``f32acc(Aq . Bq) * scale_a * scale_b`` over e4m3 codes; bf16 or f32 result."""
+def gemm_fp8(a_codes, b_codes, scale_a, scale_b, *, out: str = "bf16", format: str = "e4m3"):
+    """``f32acc(Aq . Bq) * scale_a * scale_b`` over fp8 codes (both operands ``format``:
+    ``"e4m3"`` or ``"e5m2"``); bf16 or f32 result."""
+    fmt = _fp8_format(format)
     a = np.ascontiguousarray(a_codes, np.uint8)
     b = np.ascontiguousarray(b_codes, np.uint8)
     if a.ndim != 2 or b.ndim != 2 or a.shape[1] != b.shape[0]:
@@ -1226,10 +1240,10 @@ def gemm_fp8(a_codes, b_codes, scale_a, scale_b, *, out: str = "bf16"):
     N = b.shape[1]
     if out == "bf16":
         d = np.empty((M, N), np.uint16)
-        fn = _lane.load().tessera_gfx950_gemm_e4m3_bf16
+        fn = getattr(_lane.load(), f"tessera_gfx950_gemm_{fmt}_bf16")
     elif out == "f32":
         d = np.empty((M, N), np.float32)
-        fn = _lane.load().tessera_gfx950_gemm_e4m3_f32
+        fn = getattr(_lane.load(), f"tessera_gfx950_gemm_{fmt}_f32")
     else:
         raise ValueError("out must be 'bf16' or 'f32'")
     _lane.check(fn(a.ctypes.data, b.ctypes.data, float(scale_a), float(scale_b), d.ctypes.data, M, N, K), "gemm_fp8")

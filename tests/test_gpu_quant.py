@@ -483,3 +483,52 @@ def test_quantised_grouped_gemm_inside_the_reference_budgets(lane, quant, bound)
     got = ops.grouped_gemm(x, w, gs, quant=quant, out="f32")
     rel = np.linalg.norm(got - ref) / (np.linalg.norm(ref) + 1e-9)
     assert rel < bound, f"{quant}: {rel:.4f}"
+
+
+def test_e5m2_quantiser_matches_oracle(lane):
+    """e5m2 codes: scale and codes bit for bit on random data, every grid point a fixed point, saturation
+    at +-57344, every midpoint between neighbours and its two f32 neighbours (ties to even), through
+    the 16-wide hardware-conversion path and the element tail alike."""
+    rng = np.random.default_rng(14)
+    x = (rng.standard_normal(1 << 16) * np.exp(rng.standard_normal(1 << 16) * 3)).astype(np.float32)
+    x[:64] = np.linspace(-1e-6, 1e-6, 64, dtype=np.float32)
+    codes, scale = ops.quantize_fp8_codes(x, format="e5m2")
+    ocodes, ogrid, oscale = orc.quantize_fp8_e5m2(x)
+    table = orc.e5m2_decode_table()
+    assert scale == oscale and np.array_equal(table[codes], ogrid)          # (-0 and +0 are two codes of one value)
+    assert np.array_equal(ops.e5m2_table(), table, equal_nan=True)
+    finite = np.isfinite(table)
+    c2, _ = ops.quantize_fp8_codes(table[finite], scale=1.0, format="e5m2")
+    assert np.array_equal(table[c2], table[finite])
+    c3, _ = ops.quantize_fp8_codes(np.array([1e9, -1e9, 60000.0, 0.0], np.float32), scale=1.0, format="e5m2")
+    assert list(c3) == [0x7B, 0xFB, 0x7B, 0x00]
+    grid = np.sort(np.unique(np.abs(table[finite]))).astype(np.float32)
+    mid = ((grid[:-1].astype(np.float64) + grid[1:].astype(np.float64)) / 2).astype(np.float32)
+    probe = np.concatenate([mid, np.nextafter(mid, np.float32(np.inf)), np.nextafter(mid, np.float32(-np.inf))])
+    probe = np.concatenate([probe, -probe])
+    for xs in (probe, probe[:13]):
+        got, _ = ops.quantize_fp8_codes(xs, scale=1.0, format="e5m2")
+        assert np.array_equal(table[got], orc.fpquant_grid(xs, 57344.0, 2, -14))
+    with pytest.raises(ValueError):
+        ops.quantize_fp8_codes(x, format="e3m4")
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (256, 512, 1024), (130, 272, 208), (9, 21, 13), (300, 1024, 8192),
+                                   (1, 8192, 8192), (48, 272, 2112), (1024, 2048, 1024), (517, 1003, 771)])
+def test_fp8_e5m2_gemm(lane, M, N, K):
+    """The e5m2 operand format on every 8-bit kernel (both tile heights, K split, streaming, per-element,
+    repitched) against the oracle's f64 product of the decoded codes."""
+    rng = np.random.default_rng(60 + M)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    ac, _, sa = orc.quantize_fp8_e5m2(A)
+    bc, _, sb = orc.quantize_fp8_e5m2(B)
+    ref = orc.gemm_fp8_codes(ac, bc, sa, sb, "e5m2")
+    got32 = ops.gemm_fp8(ac, bc, sa, sb, out="f32", format="e5m2")
+    assert orc.max_rel_err(got32, ref) <= 2e-3
+    if K >= 1024:      # two mantissa bits: the format's own error against the unquantised product
+        assert orc.max_rel_err(got32, A.astype(np.float64) @ B.astype(np.float64)) <= 1e-1
+    got16 = ops.gemm_fp8(ac, bc, sa, sb, out="bf16", format="e5m2")
+    assert np.array_equal(got16.to_float32(), orc.round_to_storage(got32, "bf16"))
+    with pytest.raises(ValueError):
+        ops.gemm_fp8(ac, bc, sa, sb, format="e2m5")

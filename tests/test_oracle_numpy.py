@@ -502,3 +502,23 @@ def test_per_tensor_int8_closed_forms():
     assert list(q) == [0, 2, 2, 0, -2, 127, -127]
     q, s = orc.quantize_int8_tensor(np.zeros(5, np.float32))
     assert s == np.float32(1.0) and not q.any()
+
+
+def test_e5m2_tables_against_the_library_and_the_format():
+    """The e5m2 decode table against torch.float8_e5m2 for all 256 codes and against the half-precision
+    identity; encode(decode(c)) = c on every finite code; the grid function lands on table values only."""
+    import torch
+    t = orc.e5m2_decode_table()
+    lib = torch.arange(256, dtype=torch.uint8).view(torch.float8_e5m2).to(torch.float32).numpy()
+    assert np.array_equal(t, lib, equal_nan=True)
+    assert np.array_equal(t, (np.arange(256, dtype=np.uint16) << 8).view(np.float16).astype(np.float32), equal_nan=True)
+    finite = np.isfinite(t)
+    codes = np.arange(256, dtype=np.uint8)[finite]
+    back = orc.e5m2_encode(t[finite])
+    assert np.array_equal(back & 0x7F, codes & 0x7F) and np.array_equal(t[back], t[codes])
+    rng = np.random.default_rng(9)
+    x = (rng.standard_normal(4000) * np.exp(rng.standard_normal(4000) * 4)).astype(np.float32)
+    c, grid, s = orc.quantize_fp8_e5m2(x)
+    assert np.array_equal(t[c], grid) and np.all(np.abs(grid) <= 57344)
+    want = torch.from_numpy(np.clip(x / s, -57344, 57344)).to(torch.float8_e5m2).to(torch.float32).numpy()
+    assert np.array_equal(grid, want)                    # the library's own rounding of the same scaled values
