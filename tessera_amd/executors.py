@@ -312,7 +312,7 @@ def execute_gfx950_moe_transport(artifact: RuntimeArtifact, args: Any):
 
 
 def execute_gfx950_quant_gemm(artifact: RuntimeArtifact, args: Any):
-    """``tessera.fp8_gemm``: operands (a_codes, b_codes), kwargs scale_a/scale_b/out;
+    """``tessera.fp8_gemm``: operands (a_codes, b_codes), kwargs scale_a/scale_b/out/format;
     ``tessera.w8a8_gemm``: operands (x_q, w_q, a_scale, w_scale)."""
     md = artifact.metadata or {}
     op = _single_op(artifact, ("tessera.fp8_gemm", "tessera.w8a8_gemm"), "gfx950_quant_gemm")
@@ -323,7 +323,8 @@ def execute_gfx950_quant_gemm(artifact: RuntimeArtifact, args: Any):
         if len(names) != 2:
             raise ValueError("fp8_gemm requires two operands")
         return _ops.gemm_fp8(values[names[0]], values[names[1]], float(kwargs.get("scale_a", 1.0)),
-                             float(kwargs.get("scale_b", 1.0)), out=str(kwargs.get("out", "bf16")))
+                             float(kwargs.get("scale_b", 1.0)), out=str(kwargs.get("out", "bf16")),
+                             format=str(kwargs.get("format", "e4m3")))
     if len(names) != 4:
         raise ValueError("w8a8_gemm requires x_q, w_q, a_scale, w_scale")
     return _ops.w8a8_gemm(*(values[n] for n in names))
