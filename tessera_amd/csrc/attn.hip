@@ -54,9 +54,7 @@ int launch_flash(const FlashParams& p, hipStream_t s) {
                                   : dim3(p.B * p.Hq, qblocks * q.nsplit, 1);
     hipLaunchKernelGGL(kern, grid, dim3(G::THREADS), G::SMEM, s, q);
     if (int rc = launch_status(); rc != kOk) return rc;
-    const long quads = (long)rows * (p.D / 4);
-    hipLaunchKernelGGL((flash_decode_merge_kernel<T>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p,
-                       static_cast<const float*>(q.O), static_cast<const float*>(q.LSE), q.nsplit);
+    launch_flash_merge<T>(p, static_cast<const float*>(q.O), static_cast<const float*>(q.LSE), q.nsplit, s);
     return launch_status();
   }
   const dim3 grid = xcd_grouped ? dim3(8 * p.ratio, qblocks, p.B * p.Hkv / 8) : dim3(p.B * p.Hq, qblocks, 1);
@@ -116,9 +114,7 @@ int launch_decode(const FlashParams& p, hipStream_t s) {
   }
   hipLaunchKernelGGL(kern, dim3(kvheads, nsplit), dim3(G::THREADS), G::SMEM, s, dp);
   if (int rc = launch_status(); rc != kOk || nsplit == 1) return rc;
-  const long quads = (long)p.B * p.Hq * p.Sq * (DP / 4);
-  hipLaunchKernelGGL((flash_decode_merge_kernel<T>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p,
-                     dp.part_o, dp.part_lse, nsplit);
+  launch_flash_merge<T>(p, dp.part_o, dp.part_lse, nsplit, s);
   return launch_status();
 }
 // (up to 32 rows per KV head at D = 256, 64 at D = 128, 128 at D = 64: one, two or four query

@@ -339,4 +339,103 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const FlashPara
   if (p.LSE && d == 0) p.LSE[row] = wsum > 0.f ? mx + __logf(wsum) : -INFINITY;
 }
 
+// The same merge with one workgroup per row, for many splits (a long single sequence: few rows, up to 512
+// splits): the thread-per-four-columns form above walks the splits one dependent memory round trip after
+// another.  Here the row's LSE values go through LDS, the weights are formed once, the 256 threads share
+// the splits among 256 / (D / 4) groups with all their loads independent, and the groups' sums are added
+// in group order.  Every order of summation is fixed, so the result does not depend on scheduling.
+constexpr int kMergeMaxSplits = 512;
+template <class T>
+__global__ __launch_bounds__(256) void flash_decode_merge_rows_kernel(const FlashParams p, const float* __restrict__ part_o,
+                                                                      const float* __restrict__ part_lse, int nsplit) {
+  __shared__ float sh_w[kMergeMaxSplits];
+  __shared__ float4 sh_acc[256];
+  __shared__ float sh_red[8];
+  const int D = p.D, per_row = D / 4, G = 256 / per_row;
+  const long total_rows = (long)p.B * p.Hq * p.Sq;
+  const long row = blockIdx.x;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  float mx = -INFINITY;
+  for (int s = t; s < nsplit; s += 256) {
+    const float l = part_lse[(long)s * total_rows + row];
+    sh_w[s] = l;
+    mx = fmaxf(mx, l);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  if (lane == 0) sh_red[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(sh_red[0], sh_red[1]), fmaxf(sh_red[2], sh_red[3]));
+  for (int s = t; s < nsplit; s += 256) sh_w[s] = mx > -INFINITY ? __expf(sh_w[s] - mx) : 0.f;
+  __syncthreads();
+  if (wave == 0) {                                     // the sum of the weights: lane order, then a fixed tree
+    float ws = 0.f;
+    for (int s = lane; s < nsplit; s += 64) ws += sh_w[s];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ws += __shfl_xor(ws, o, 64);
+    if (lane == 0) sh_red[4] = ws;
+  }
+  const int g = t / per_row, c = t - g * per_row;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (g < G) {
+    const float* src = part_o + row * D + 4 * c;
+    const long step = total_rows * D;
+    int s = g;
+    for (; s + 3 * G < nsplit; s += 4 * G) {
+      const float4 v0 = *reinterpret_cast<const float4*>(src + (long)s * step);
+      const float4 v1 = *reinterpret_cast<const float4*>(src + (long)(s + G) * step);
+      const float4 v2 = *reinterpret_cast<const float4*>(src + (long)(s + 2 * G) * step);
+      const float4 v3 = *reinterpret_cast<const float4*>(src + (long)(s + 3 * G) * step);
+      const float w0 = sh_w[s], w1 = sh_w[s + G], w2 = sh_w[s + 2 * G], w3 = sh_w[s + 3 * G];
+      acc.x += w0 * v0.x; acc.y += w0 * v0.y; acc.z += w0 * v0.z; acc.w += w0 * v0.w;
+      acc.x += w1 * v1.x; acc.y += w1 * v1.y; acc.z += w1 * v1.z; acc.w += w1 * v1.w;
+      acc.x += w2 * v2.x; acc.y += w2 * v2.y; acc.z += w2 * v2.z; acc.w += w2 * v2.w;
+      acc.x += w3 * v3.x; acc.y += w3 * v3.y; acc.z += w3 * v3.z; acc.w += w3 * v3.w;
+    }
+    for (; s < nsplit; s += G) {
+      const float4 v = *reinterpret_cast<const float4*>(src + (long)s * step);
+      const float w = sh_w[s];
+      acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
+    }
+  }
+  sh_acc[t] = acc;
+  __syncthreads();
+  if (g != 0) return;
+  for (int gg = 1; gg < G; ++gg) {
+    const float4 v = sh_acc[gg * per_row + c];
+    acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+  }
+  const float wsum = sh_red[4];
+  const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
+  acc.x *= inv; acc.y *= inv; acc.z *= inv; acc.w *= inv;
+  const int d = 4 * c;
+  const int q = (int)(row % p.Sq);
+  const int hq = (int)((row / p.Sq) % p.Hq);
+  const int b = (int)(row / ((long)p.Sq * p.Hq));
+  const long o_at = b * p.os.batch + hq * p.os.head + (long)q * p.os.row + d;
+  if (p.out_storage) {
+    uint2 pk;
+    pk.x = pack2<T>(acc.x, acc.y);
+    pk.y = pack2<T>(acc.z, acc.w);
+    *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.O) + o_at) = pk;
+  } else {
+    *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.O) + o_at) = acc;
+  }
+  if (p.LSE && c == 0) p.LSE[row] = wsum > 0.f ? mx + __logf(wsum) : -INFINITY;
+}
+
+// Launches the merge of `nsplit` partials: a workgroup per row from 8 splits on while the rows are few
+// (with many rows the thread-per-four-columns form has the parallelism to hide its round trips).
+template <class T>
+inline void launch_flash_merge(const FlashParams& p, const float* part_o, const float* part_lse, int nsplit, hipStream_t s) {
+  const long rows = (long)p.B * p.Hq * p.Sq;
+  if (nsplit >= 8 && nsplit <= kMergeMaxSplits && rows <= 4096) {
+    hipLaunchKernelGGL((flash_decode_merge_rows_kernel<T>), dim3((unsigned)rows), dim3(256), 0, s, p, part_o, part_lse, nsplit);
+    return;
+  }
+  const long quads = rows * (p.D / 4);
+  hipLaunchKernelGGL((flash_decode_merge_kernel<T>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, p, part_o,
+                     part_lse, nsplit);
+}
+
 }  // namespace tsr950
