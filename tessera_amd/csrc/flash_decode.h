@@ -310,16 +310,33 @@ __global__ __launch_bounds__(256) void flash_decode_merge_kernel(const FlashPara
   if (idx >= total_rows * per_row) return;
   const long row = idx / per_row;
   const int d = (int)(idx - row * per_row) * 4;
+  // (four splits fetched together in both passes: every one of these loads is a trip to memory)
   float mx = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, part_lse[(long)s * total_rows + row]);
+  for (int s0 = 0; s0 < nsplit; s0 += 4) {
+    float l[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) l[u] = s0 + u < nsplit ? part_lse[(long)(s0 + u) * total_rows + row] : -INFINITY;
+    mx = fmaxf(fmaxf(mx, fmaxf(l[0], l[1])), fmaxf(l[2], l[3]));
+  }
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   float wsum = 0.f;
   if (mx > -INFINITY) {
-    for (int s = 0; s < nsplit; ++s) {
-      const float w = __expf(part_lse[(long)s * total_rows + row] - mx);
-      const float4 v = *reinterpret_cast<const float4*>(part_o + ((long)s * total_rows + row) * D + d);
-      acc.x += w * v.x; acc.y += w * v.y; acc.z += w * v.z; acc.w += w * v.w;
-      wsum += w;
+    for (int s0 = 0; s0 < nsplit; s0 += 4) {
+      float l[4];
+      float4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const bool on = s0 + u < nsplit;
+        l[u] = on ? part_lse[(long)(s0 + u) * total_rows + row] : -INFINITY;
+        v[u] = on ? *reinterpret_cast<const float4*>(part_o + ((long)(s0 + u) * total_rows + row) * D + d)
+                  : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {                    // split order
+        const float w = __expf(l[u] - mx);             // (exp(-inf) = 0 for the splits past the end)
+        acc.x += w * v[u].x; acc.y += w * v[u].y; acc.z += w * v[u].z; acc.w += w * v[u].w;
+        wsum += w;
+      }
     }
   }
   const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;

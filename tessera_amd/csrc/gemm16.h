@@ -780,9 +780,15 @@ __global__ __launch_bounds__(256) void gemm16_rest_sum_kernel(const float* __res
   const long tile_elems = 256 * 256;
   const float* src = ws + (long)blockIdx.y * tile_elems + row * 256 + col;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int z = 0; z < splits; ++z) {
-    const float4 v = *reinterpret_cast<const float4*>(src + (long)z * gridDim.y * tile_elems);
-    acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+  // (four slices fetched together: every one of these loads is a trip to memory)
+  for (int z0 = 0; z0 < splits; z0 += 4) {
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      v[u] = z0 + u < splits ? *reinterpret_cast<const float4*>(src + (long)(z0 + u) * gridDim.y * tile_elems)
+                             : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) { acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w; }   // slice order
   }
   if (bias) {
     const float4 bv = *reinterpret_cast<const float4*>(bias + n);

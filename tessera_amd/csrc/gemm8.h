@@ -449,10 +449,17 @@ __global__ __launch_bounds__(256) void gemm8_split_sum_kernel(const void* __rest
   const long o = (long)m * p.N + n, mn = (long)p.M * p.N;
   float v[4];
   if constexpr (IS_I8) {
+    // (the partials of four slices are fetched together: they were written by other XCDs, so every
+    // one of these loads pays a trip to memory)
     int4 acc = make_int4(0, 0, 0, 0);
-    for (int z = 0; z < splits; ++z) {
-      const int4 a = *reinterpret_cast<const int4*>(reinterpret_cast<const int32_t*>(part) + z * mn + o);
-      acc.x += a.x; acc.y += a.y; acc.z += a.z; acc.w += a.w;
+    for (int z0 = 0; z0 < splits; z0 += 4) {
+      int4 a[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        a[u] = z0 + u < splits ? *reinterpret_cast<const int4*>(reinterpret_cast<const int32_t*>(part) + (z0 + u) * mn + o)
+                               : make_int4(0, 0, 0, 0);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) { acc.x += a[u].x; acc.y += a[u].y; acc.z += a[u].z; acc.w += a[u].w; }
     }
     if constexpr (EPI == EPI8_I32) {
       *reinterpret_cast<int4*>(reinterpret_cast<int32_t*>(p.D) + o) = acc;
@@ -466,9 +473,14 @@ __global__ __launch_bounds__(256) void gemm8_split_sum_kernel(const void* __rest
     }
   } else {
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int z = 0; z < splits; ++z) {
-      const float4 a = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(part) + z * mn + o);
-      acc.x += a.x; acc.y += a.y; acc.z += a.z; acc.w += a.w;
+    for (int z0 = 0; z0 < splits; z0 += 4) {
+      float4 a[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        a[u] = z0 + u < splits ? *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(part) + (z0 + u) * mn + o)
+                               : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) { acc.x += a[u].x; acc.y += a[u].y; acc.z += a[u].z; acc.w += a[u].w; }   // slice order
     }
     v[0] = (acc.x * p.scale_a) * p.scale_b; v[1] = (acc.y * p.scale_a) * p.scale_b;
     v[2] = (acc.z * p.scale_a) * p.scale_b; v[3] = (acc.w * p.scale_a) * p.scale_b;
