@@ -71,7 +71,7 @@ def _ramp(lane, launch):
     run at the GEMM's lower clock: such rows read a few percent slow)."""
     if not _RAMP["foreign"]:
         t0 = time.perf_counter()
-        while time.perf_counter() - t0 < RAMP_SECONDS:
+        while time.perf_counter() - t0 < _RAMP.get("seconds", RAMP_SECONDS):
             for _ in range(4):
                 launch()
             lane.synchronize()
@@ -84,7 +84,7 @@ def _ramp(lane, launch):
     a, b, d, n = _RAMP["bufs"]
     fn = lane.load().tessera_gfx950_gemm_bf16_dev
     t0 = time.perf_counter()
-    while time.perf_counter() - t0 < RAMP_SECONDS:
+    while time.perf_counter() - t0 < _RAMP.get("seconds", RAMP_SECONDS):
         for _ in range(8):
             lane.check(fn(a.ptr, b.ptr, d.ptr, n, n, n, None), "ramp")
         lane.synchronize()
@@ -349,7 +349,8 @@ def bench_quant(lane, steps, warmup, check=True):
             turn[0] += 1
             lane.check(lib.tessera_gfx950_gemm_w8a8_f32_dev(xq.ptr, wcopies[turn[0] & 3].ptr, rs.ptr, cs.ptr, dd.ptr, None,
                                                             Md, N, K, None), "gemm_w8a8")
-        _, ev = _timed(lane, dec, max(steps, 50), warmup)
+        # (a short run — the counter passes of the profiles use --steps 3 — stays short)
+        _, ev = _timed(lane, dec, max(steps, 50) if steps >= 10 else steps, warmup)
         dbytes = 1.0 * K * N + Md * K + 4.0 * Md * N
         out[f"gemm_w8a8_decode_M{Md}_8192x8192"] = {"ms": ev, "gbs": dbytes / ev / 1e6,
                                                     "frac_hbm_peak": dbytes / ev / 1e6 / PEAK_HBM_GBS, "weights_cycled": 4}
@@ -900,6 +901,9 @@ def main() -> int:
                                                  "(for a profiler run with one clean row per workload)")
     ap.add_argument("--profile", action="store_true",
                     help="ramp the clocks with a kernel no workload times (clean per-kernel rows under a profiler)")
+    ap.add_argument("--ramp-seconds", type=float, default=RAMP_SECONDS,
+                    help="length of the untimed clock ramp before every timed region (a counter pass of a profiler "
+                         "records every launch: a shorter ramp keeps its output small)")
     ap.add_argument("--no-vendor", action="store_true", help="skip the vendor-library GEMM leg (a PyTorch child process)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a 1 GiB copy kernel (counter calibration for profiled runs)")
@@ -920,6 +924,7 @@ def main() -> int:
         return 3
 
     _RAMP["foreign"] = bool(args.profile)
+    _RAMP["seconds"] = max(0.0, float(args.ramp_seconds))
     if args.no_clock or args.profile:
         _OPTS["ceiling_seconds"] = 0.0
     if args.clocks:
