@@ -612,7 +612,8 @@ int tessera_gfx950_moe_swiglu_block_bf16_dev(const void* x, const void* wg, cons
 /* The same block reading its input through the dispatch map: row m of the block's
  * input is x[token_of_slot[m]], x the unpermuted bf16 [T,K] activation, so
  * moe_dispatch (python/tessera/stdlib/moe.py:117-125) needs no pass and no x_perm
- * buffer of its own.  token_of_slot: device int32[S] with values in [0, T);
+ * buffer of its own.  token_of_slot: device int32[S] with values in [0, T) (not read, and
+ * may be NULL, when S == 0);
  * T * K * 2 must not exceed 2 GiB - 17 (the range of the buffer load that fetches a
  * token row: rows past it would read as zeros), else rc 1. */
 int tessera_gfx950_moe_swiglu_block_gather_bf16_dev(const void* x, const int32_t* token_of_slot,

@@ -1288,7 +1288,7 @@ int tessera_gfx950_moe_swiglu_block_gather_bf16_dev(const void* x, const int32_t
                                                     const void* wu, const void* wd, const int32_t* offsets, void* y,
                                                     void* hidden, int T, int S, int K, int F, int N, int E,
                                                     void* stream) {
-  if (!token_of_slot) return kBadShape;
+  if (S > 0 && !token_of_slot) return kBadShape;       // (no slots: no map to read)
   return swiglu_dev(x, wg, wu, wd, offsets, y, hidden, S, K, F, N, E, as_stream(stream), token_of_slot, T);
 }
 

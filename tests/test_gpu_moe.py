@@ -287,6 +287,23 @@ def test_swiglu_block_reading_through_the_dispatch_map(lane, T, K, F, N, E, k):
         b.close()
 
 
+def test_swiglu_block_with_no_slots_is_a_no_op(lane):
+    """No slots (every token dropped, or an empty batch): the block entries return success without
+    reading the activation, the dispatch map or the output — null pointers included."""
+    K, F, N, E = 64, 128, 64, 4
+    w = [lane.DeviceBuffer.from_host(np.zeros((E, a, b), np.uint16)) for a, b in ((K, F), (K, F), (F, N))]
+    doff = lane.DeviceBuffer.from_host(np.zeros(E + 1, np.int32))
+    lib = lane.load()
+    lane.check(lib.tessera_gfx950_moe_swiglu_block_bf16_dev(None, w[0].ptr, w[1].ptr, w[2].ptr, doff.ptr, None, None,
+                                                            0, K, F, N, E, None), "swiglu block, no slots")
+    lane.check(lib.tessera_gfx950_moe_swiglu_block_gather_bf16_dev(None, None, w[0].ptr, w[1].ptr, w[2].ptr, doff.ptr,
+                                                                   None, None, 5, 0, K, F, N, E, None),
+               "gathering swiglu block, no slots")
+    lane.synchronize()
+    for b in w + [doff]:
+        b.close()
+
+
 def test_grouped_gemm_fp8_quant(lane):
     """quant="fp8_e4m3": per-tensor e4m3 for x and for every expert's weight, then the
     grouped product (compiler/grouped_layout.py:353-392).  Checked against the oracle's
