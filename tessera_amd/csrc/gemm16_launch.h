@@ -235,8 +235,9 @@ inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
     const long tiles = t128 ? tiles128 : (long)ceil_div(M, 64) * ceil_div(N, 64);
     splits = (int)std::max<long>(1, std::min<long>((kSplitTargetWgs + tiles - 1) / tiles, K / 512));
     // the f32 partials are written and read once per split (8 M N splits bytes against
-    // 2 K N bytes of B): beyond two splits keep that under about 0.4 of the weight traffic
-    splits = (int)std::min<long>(splits, std::max<long>(2, K / (10L * M)));
+    // 2 K (M + N) bytes of operands: B dominates under few rows, A over few columns): beyond two
+    // splits keep that under about 0.4 of the operand traffic
+    splits = (int)std::min<long>(splits, std::max<long>(2, (long)K * (M + N) / (10L * M * N)));
     while (splits > 1 && K % (splits * G16_BK) != 0) --splits;
   }
   return {t128 ? 128 : 64, splits, false};
