@@ -179,6 +179,14 @@ inline double est_split_sum_us(long mn, int splits) {
 }
 
 inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
+  if (batch == 1 && M <= kWeightStreamMaxM && N >= 128) {
+    // Few rows under a very wide weight matrix (a vocabulary projection, a fused up projection):
+    // tiles enough for three quarters of the compute units without a K split, which would add a
+    // pass over the partials and little parallelism.  The wider tile reads 512 contiguous bytes
+    // of a row of B instead of 256 and streams faster once it, too, fills the chip.
+    if ((long)ceil_div(M, 128) * ceil_div(N, 256) >= 192) return {256, 1, false, 1, 128};
+    if ((long)ceil_div(M, 128) * ceil_div(N, 128) >= 192) return {128, 1, false};
+  }
   if (batch == 1 && M <= kSkinnyMaxM && K % 32 == 0 && K >= 512) {
     // one workgroup per 64-column strip and K split; about one workgroup per CU, and
     // at least two 32-row slices for each of a workgroup's 8 waves

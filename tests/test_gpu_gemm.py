@@ -227,6 +227,33 @@ def test_skinny_gemm(lane, M, N, K, st):
     assert np.array_equal(ops.gemm(a, b, out="f32"), got)               # fixed summation order
 
 
+# Few rows under a very wide weight matrix (a vocabulary projection): tiles enough for the chip
+# without a K split, 128 x 256 tiles from 192 of them on, 128 x 128 below; and the opposite
+# shape, many rows over one narrow column of tiles (a router's logits), which splits K by the
+# traffic of A.  (M, N, K, workgroup tile the launcher reports, K splits)
+WIDE_AND_TALL = [(1, 49152, 256, (128, 256, 64), 1), (8, 50048, 96, (128, 256, 64), 1),
+                 (33, 24576, 320, (128, 128, 64), 1), (128, 24584, 64, (128, 128, 64), 1),
+                 (8192, 64, 4096, (64, 64, 64), 4), (5000, 8, 2048, (64, 64, 64), 4)]
+
+
+@pytest.mark.parametrize("M,N,K,tile,splits", WIDE_AND_TALL)
+@pytest.mark.parametrize("st", ["bf16", "f16"])
+def test_wide_weight_and_tall_products(lane, M, N, K, tile, splits, st):
+    from tessera_amd.schedule import select_gfx950_gemm_schedule as sel
+    sch = sel(M, N, K, dtype=st)
+    assert (sch.workgroup_tile, sch.split_k) == (tile, splits)
+    A = _rand((M, K), 1.0, 31)
+    B = _rand((K, N), 1.0 / np.sqrt(K), 32)
+    ref = orc.gemm_f64(A, B, st)
+    a = b16.from_float32(A) if st == "bf16" else A.astype(np.float16)
+    b = b16.from_float32(B) if st == "bf16" else B.astype(np.float16)
+    got = ops.gemm(a, b, out="f32")
+    assert orc.max_rel_err(got, ref) <= 1e-5
+    stored = ops.gemm(a, b)
+    sf = stored.to_float32() if st == "bf16" else stored.astype(np.float32)
+    assert np.array_equal(sf, orc.round_to_storage(got, st))
+
+
 def test_full_size_bf16_gemm_properties(lane):
     """8192^3 is too large for a CPU product inside the test budget; check
     size-independent properties instead: linearity in A and agreement with
