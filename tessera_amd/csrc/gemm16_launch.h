@@ -163,12 +163,14 @@ inline double est_tiles256_us(long tiles, int ksteps) {
   if (rem) t += 9.6 + ksteps * (1.09 + 0.34 * std::min(1.0, std::max(0.0, (rem - 144) / 112.0)));
   return t;
 }
-// (a 128 x 256 tile: 7 us and 0.60 us per step, 0.82 with every compute unit busy — per FLOP a fifth
-// slower than the 256 x 256 tile, but twice as many tiles to fill the chip with)
+// (a 128 x 256 tile: 7 us and 0.60 us per step up to about 96 tiles at a time, 0.82 with every
+// compute unit busy over several rounds — per FLOP a fifth slower than the 256 x 256 tile, but
+// twice as many tiles to fill the chip with; a single partial round of 160 to 255 tiles measured
+// 0.83 to 0.93 per step)
 inline double est_tiles128x256_us(long tiles, int ksteps) {
   const long full = tiles / 256, rem = tiles % 256;
   double t = (double)full * (7.0 + ksteps * 0.82);
-  if (rem) t += 7.0 + ksteps * (0.60 + 0.22 * std::min(1.0, std::max(0.0, (rem - 144) / 112.0)));
+  if (rem) t += 7.0 + ksteps * (0.60 + 0.28 * std::min(1.0, std::max(0.0, (rem - 96) / 64.0)));
   return t;
 }
 inline double est_tiles128_us(long tiles, int ksteps) {
@@ -207,7 +209,9 @@ inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
     };
     consider(128, 1, est_tiles128_us(tiles128, ksteps));
     {
-      const double us = est_tiles128x256_us((long)ceil_div(M, 128) * ceil_div(N, 256) * batch, ksteps);
+      // (its estimate is the least certain of the three — the per-step figure moved by 13 % between
+      // shapes of equal tile count — so it has to win by a margin)
+      const double us = 1.06 * est_tiles128x256_us((long)ceil_div(M, 128) * ceil_div(N, 256) * batch, ksteps);
       if (us < best_us) { best_us = us; best = Gemm16Schedule{256, 1, false, 1, 128}; }
     }
     if (batch == 1) {
