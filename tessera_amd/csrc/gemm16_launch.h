@@ -180,6 +180,28 @@ inline double est_split_sum_us(long mn, int splits) {
   return splits > 1 ? 2.0 + (double)mn * (4.0 * splits + 2.0) / 4.4e6 : 0.0;
 }
 
+// Time estimate (microseconds) for 33 to 128 rows against a weight matrix that streams from HBM,
+// fitted (13 % rms) to timings of forced (tile, split) pairs on this part over 19 weight shapes from
+// 2048 x 7168 to 32768 x 4096 with the weights cycled through copies: a launch cost, then the larger
+// of the busiest compute unit's K steps (its first workgroup at `step`, every further one sharing
+// the unit at `shared` per step) and the time to stream the tile columns of B at `tbs` TB/s, which
+// takes about 185 workgroups in flight to reach; a split adds 3.4 us and 1.6 us per million
+// partial sums.
+struct FewRowTile { int tile_m, tile_n; double launch, step, shared, tbs; };
+constexpr FewRowTile kFewRowTiles[3] = {{64, 64, 0.26, 0.514, 0.256, 5.39},
+                                        {128, 128, 2.31, 0.345, 0.728, 5.46},
+                                        {128, 256, 3.97, 0.693, 1.582, 7.01}};
+inline double est_few_rows_us(const FewRowTile& t, int M, int N, int K, int splits) {
+  const long wgs = (long)ceil_div(M, t.tile_m) * ceil_div(N, t.tile_n) * splits;
+  const double steps = (double)K / G16_BK / splits;
+  const double busiest = (double)((wgs + 255) / 256);
+  const double compute = steps * (t.step + t.shared * (busiest - 1.0));
+  const double bytes = 2.0 * K * ceil_div(N, t.tile_n) * t.tile_n;
+  const double stream = bytes / (t.tbs * 1e6 * std::min(1.0, wgs / 185.0));
+  const double sum = splits > 1 ? 3.4 + (double)M * N * splits * 1.6e-6 : 0.0;
+  return t.launch + std::max(compute, stream) + sum;
+}
+
 inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
   if (batch == 1 && M <= kWeightStreamMaxM && N >= 128) {
     // Few rows under a very wide weight matrix (a vocabulary projection, a fused up projection):
@@ -195,6 +217,22 @@ inline Gemm16Schedule select_gemm16_schedule(int M, int N, int K, int batch) {
     const int strips = ceil_div(N, 64);
     int splits = std::max(1, std::min((256 + strips / 2) / strips, K / 512));
     return {64, splits, true};
+  }
+  if (batch == 1 && M > 32 && M <= kWeightStreamMaxM && N >= 2048 && K >= 1024) {
+    // the cheapest of the three small tiles with K in 1 to 16 parts, by the estimate above (below
+    // 33 rows the rule further down is as good as the estimate: 1 % apart over the same shapes)
+    Gemm16Schedule best{128, 1, false};
+    double best_us = 1e30;
+    for (const FewRowTile& t : kFewRowTiles)
+      for (int splits : {1, 2, 3, 4, 6, 8, 12, 16}) {
+        if (K % (splits * G16_BK) != 0 || K / splits < 512) continue;
+        const double us = est_few_rows_us(t, M, N, K, splits);
+        if (us < best_us) {
+          best_us = us;
+          best = t.tile_n == 256 ? Gemm16Schedule{256, splits, false, 1, 128} : Gemm16Schedule{t.tile_m, splits, false};
+        }
+      }
+    return best;
   }
   const long tiles256 = (long)ceil_div(M, 256) * ceil_div(N, 256) * batch;
   const long tiles128 = (long)ceil_div(M, 128) * ceil_div(N, 128) * batch;
@@ -393,7 +431,7 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
   if constexpr (EPI != EPI_F32) {
     if (fused) return kBadShape;
   }
-  if (sch.tile == 256 && sch.tile_m == 128) {
+  if (sch.tile == 256 && sch.tile_m == 128 && sch.split_k == 1) {
     if constexpr (EPI == EPI_F32) {
       if (fused) return launch_gemm16_tile<T, 128, 256, 2, 2, EPI_F32_FUSED, false, kBigTileMfma>(p, s);
     }
@@ -438,7 +476,8 @@ int launch_gemm16(Gemm16Params p, hipStream_t s) {
         q.K = p.K;
         rc = launch_gemm16_skinny<T, EPI_F32>(q, ceil_div(ceil_div(p.K, splits), 32) * 32, splits, s);
       } else {
-        rc = sch.tile == 256 ? launch_gemm16_tile<T, 256, 256, 2, 2, EPI_F32, false, kBigTileMfma>(q, s)
+        rc = sch.tile == 256 && sch.tile_m == 128 ? launch_gemm16_tile<T, 128, 256, 2, 2, EPI_F32, false, kBigTileMfma>(q, s)
+             : sch.tile == 256 ? launch_gemm16_tile<T, 256, 256, 2, 2, EPI_F32, false, kBigTileMfma>(q, s)
              : t128      ? launch_gemm16_tile<T, 128, 128, 2, 2, EPI_F32, false>(q, s)
                          : launch_gemm16_tile<T, 64, 64, 2, 2, EPI_F32, false>(q, s);
       }

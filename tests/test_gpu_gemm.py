@@ -233,7 +233,10 @@ def test_skinny_gemm(lane, M, N, K, st):
 # traffic of A.  (M, N, K, workgroup tile the launcher reports, K splits)
 WIDE_AND_TALL = [(1, 49152, 256, (128, 256, 64), 1), (8, 50048, 96, (128, 256, 64), 1),
                  (33, 24576, 320, (128, 128, 64), 1), (128, 24584, 64, (128, 128, 64), 1),
-                 (8192, 64, 4096, (64, 64, 64), 4), (5000, 8, 2048, (64, 64, 64), 4)]
+                 (8192, 64, 4096, (64, 64, 64), 4), (5000, 8, 2048, (64, 64, 64), 4),
+                 # 33 to 128 rows: tile and split by the fitted estimate, the 128 x 256 tile with K splits among them
+                 (128, 10240, 8192, (128, 256, 64), 4), (64, 14336, 4096, (128, 256, 64), 4),
+                 (100, 5120, 5120, (128, 128, 64), 4), (48, 2048, 7168, (64, 64, 64), 8)]
 
 
 @pytest.mark.parametrize("M,N,K,tile,splits", WIDE_AND_TALL)
