@@ -633,7 +633,10 @@ __device__ __forceinline__ void gemm16_tile(const Gemm16Params& p, char* smem, c
   }
 }
 
-template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32>
+// MID (grouped 256-row tiles only): a last row tile of 65 to 128 rows runs on the 128-row tile
+// body.  A separate instantiation, for launches whose groups average at most a tile of rows: the
+// kernel that serves large groups keeps its two bodies.
+template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32, bool MID = false>
 __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Params p) {
   constexpr bool SWIGLU = (EPI == EPI_SWIGLU16 || EPI == EPI_GATED_F32);
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -731,6 +734,12 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm16_kernel(const Gemm16Par
     if (m_end - m_begin <= 64) {
       // (paced when full tiles of the same group and column run beside it; 16-wide step only)
       gemm16_tile<T, 64, BN, 1, 4, EPI, GROUPED, MS>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db, MS == 16 && tm > 0);
+      return;
+    }
+    // (up to 128 rows left — a group of about a hundred rows, a chunk of a thousand tokens over
+    // 64 experts — the 128-row tile: half the matrix work)
+    if (MID && m_end - m_begin <= 128) {
+      gemm16_tile<T, 128, BN, 2, 2, EPI, GROUPED, MS>(p, smem, m_begin, m_end, tn, Ab, Bb, B2b, Db);
       return;
     }
   }

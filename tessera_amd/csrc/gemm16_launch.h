@@ -71,10 +71,10 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 // wg_limit > 0: only the first wg_limit workgroups of a dense product's tile order are launched
 // (the caller serves the remaining tiles itself).
-template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32>
+template <class T, int BM, int BN, int WM, int WN, int EPI, bool GROUPED, int MS = 32, bool MID = false>
 int launch_gemm16_tile(Gemm16Params p, hipStream_t s, int wg_limit = 0) {
   using S = Gemm16Smem<BM, BN>;
-  auto kern = gemm16_kernel<T, BM, BN, WM, WN, EPI, GROUPED, MS>;
+  auto kern = gemm16_kernel<T, BM, BN, WM, WN, EPI, GROUPED, MS, MID>;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [&] {
@@ -572,11 +572,16 @@ int launch_gemm16_grouped(Gemm16Params p, hipStream_t s) {
     hipLaunchKernelGGL((gemm16_grouped_generic_kernel<T, EPI>), grid, block, 0, s, p);
     return launch_status();
   }
+  // groups that average at most a tile of rows (a chunk of a thousand tokens over 64 experts): the
+  // instantiation whose last row tile also comes in a 128-row form
+  const bool mid = (long)p.M <= 256L * p.groups;
   if constexpr (EPI == EPI_SWIGLU16) {
+    if (mid) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true, kGroupedTileMfma, true>(p, s);
     return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true, kGroupedTileMfma>(p, s);
   } else {
-    if ((long)p.M >= 64L * p.groups) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true, kGroupedTileMfma>(p, s);
-    return launch_gemm16_tile<T, 128, 128, 2, 2, EPI, true>(p, s);
+    if ((long)p.M < 64L * p.groups) return launch_gemm16_tile<T, 128, 128, 2, 2, EPI, true>(p, s);
+    if (mid) return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true, kGroupedTileMfma, true>(p, s);
+    return launch_gemm16_tile<T, 256, 256, 2, 2, EPI, true, kGroupedTileMfma>(p, s);
   }
 }
 
