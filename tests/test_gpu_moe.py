@@ -179,6 +179,8 @@ def test_dispatch_and_combine(lane):
     ([3, 5], 24, 40),
     # last row tiles of 64 / 65 rows: either side of the short last-tile form
     ([64, 65, 320, 321, 0, 256], 200, 328),
+    # groups of about a tile of rows: last tiles of 65 to 128 rows take the 128-row form, 129 the full one
+    ([128, 129, 127, 66, 384, 385, 0, 100], 264, 520),
 ])
 def test_grouped_gemm(lane, sizes, K, N):
     E, T = len(sizes), int(sum(sizes))
@@ -250,6 +252,7 @@ def _swiglu_inputs(sizes, K, F, N, seed):
     ([9, 200], 64, 1408, 320),
     ([3, 5, 0], 24, 40, 56),
     ([64, 65, 320, 321, 0, 256], 200, 328, 136),
+    ([128, 129, 127, 66, 384, 385, 0, 100], 264, 520, 200),
 ])
 def test_moe_swiglu_block(lane, sizes, K, F, N):
     x, wg, wu, wd = _swiglu_inputs(sizes, K, F, N, 5)
