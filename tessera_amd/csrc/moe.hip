@@ -322,7 +322,7 @@ int route_launch(const float* scores, int T, int E, int k, int normalize, int ca
 
 int route_dev(const float* scores, int T, int E, int k, int normalize, int capacity, int32_t* token_of_slot,
               int32_t* expert_of_slot, float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
-              int32_t* num_slots, hipStream_t s) {
+              int32_t* num_slots, hipStream_t s, const PlanOutputs& plan = PlanOutputs{}) {
   if (bad_route(scores, T, E, k, token_of_slot, expert_of_slot, combine_weights, group_sizes, group_offsets))
     return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
@@ -332,7 +332,7 @@ int route_dev(const float* scores, int T, int E, int k, int normalize, int capac
   char* ws = static_cast<char*>(stream_workspace(s, route_workspace_bytes(T * k, E)));
   if (!ws) return kDeviceFailed;
   return route_launch(scores, T, E, k, normalize, capacity, kRouterSoftmaxAll, token_of_slot, expert_of_slot,
-                      combine_weights, group_sizes, group_offsets, num_slots, ws, s);
+                      combine_weights, group_sizes, group_offsets, num_slots, ws, s, plan);
 }
 
 // route_top_k (or a given selection) + the packing plan with its token-major outputs.
@@ -429,7 +429,14 @@ __global__ __launch_bounds__(1024) void combine_scan_kernel(int32_t* cnt, int T,
   const int lo = min((int)threadIdx.x * per, T), hi = min(lo + per, T);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int sum = 0;
-  for (int i = lo; i < hi; ++i) sum += cnt[i];
+  // (eight counts per round trip here as well: the loop is not unrolled on its own)
+  for (int i0 = lo; i0 < hi; i0 += 8) {
+    int v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = i0 + u < hi ? cnt[i0 + u] : 0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) sum += v[u];
+  }
   // inclusive scan of the 1024 partial sums: inside each wave by shuffles, then over the
   // 16 wave totals (two barriers in all)
   int incl = sum;
@@ -484,26 +491,36 @@ __device__ __forceinline__ float add_rounded_product(float acc, float v, float w
 // or 4 f32 columns), so a slot row is read with 16-byte loads; needs N a multiple of
 // the run and 16-byte aligned rows.  The sum over a token's slots runs in ascending
 // slot order for every column either way.
+// `ranked` > 0: the token's slots are not taken from the lists but from the routing's own
+// token-major table, list[t ranked + j] = packed position of the token's j-th choice or -1 for a
+// dropped one (ranked <= 256); off is not read.
 template <class YT, bool VEC>
 __global__ __launch_bounds__(256) void combine_kernel(const YT* y, const float* w, const int32_t* off,
-                                                      const int32_t* list, float* out, int N) {
+                                                      const int32_t* list, float* out, int N, int ranked) {
   constexpr int kMaxSorted = 256;
   constexpr int RUN = VEC ? 16 / (int)sizeof(YT) : 1;
   __shared__ int sorted[kMaxSorted];
   __shared__ float sw[kMaxSorted];
   const int t = blockIdx.x;
-  const int lo = off[t], hi = off[t + 1];
-  const int len = hi - lo;
+  const int lo = ranked > 0 ? t * ranked : off[t], hi = ranked > 0 ? lo + ranked : off[t + 1];
+  int len = hi - lo;
   const bool small = len <= kMaxSorted;
   if (small) {
     // rank of every slot id inside the token's list -> ascending order in LDS
+    int kept = 0;
+    for (int i = 0; i < len; ++i) kept += list[lo + i] >= 0;
     for (int j = threadIdx.x; j < len; j += 256) {
       const int sl = list[lo + j];
+      if (sl < 0) continue;
       int rank = 0;
-      for (int i = 0; i < len; ++i) rank += list[lo + i] < sl;
+      for (int i = 0; i < len; ++i) {
+        const int other = list[lo + i];
+        rank += other >= 0 && other < sl;
+      }
       sorted[rank] = sl;
       sw[rank] = w[sl];
     }
+    len = kept;
     __syncthreads();
   }
   for (int n = threadIdx.x * RUN; n < N; n += 256 * RUN) {
@@ -630,11 +647,21 @@ int unpack_combine_dev(const void* y, const int32_t* inverse_perm, const float* 
   return launch_status();
 }
 
+// `positions` (with k = `ranked`): the routing's token-major table of packed positions; the
+// per-token lists are then not built.
 template <class YT>
 int combine_dev(const void* y, const int32_t* token_of_slot, const float* w, float* out, int T, int S, int N,
-                hipStream_t s, const int32_t* n_dev = nullptr) {
+                hipStream_t s, const int32_t* n_dev = nullptr, const int32_t* positions = nullptr, int ranked = 0) {
   if (T <= 0 || S < 0 || N <= 0 || !out || (S > 0 && (!y || !token_of_slot || !w))) return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
+  if (positions && ranked > 0 && ranked <= 256) {
+    const bool vec = N % (16 / (int)sizeof(YT)) == 0 && aligned16(y) && aligned16(out);
+    if (vec)
+      hipLaunchKernelGGL((combine_kernel<YT, true>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, nullptr, positions, out, N, ranked);
+    else
+      hipLaunchKernelGGL((combine_kernel<YT, false>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, nullptr, positions, out, N, ranked);
+    return launch_status();
+  }
   // the per-token slot lists live in the stream's own workspace (the combine kernel below
   // is their last reader; work on one stream runs in order)
   const size_t tok_bytes = ((size_t)(T + 1) * 4 + 255) & ~(size_t)255;
@@ -649,9 +676,9 @@ int combine_dev(const void* y, const int32_t* token_of_slot, const float* w, flo
   if (S > 0) hipLaunchKernelGGL(combine_fill_kernel, dim3(ceil_div(S, 256)), dim3(256), 0, s, token_of_slot, S, T, off, cnt, list, n_dev);
   const bool vec = N % (16 / (int)sizeof(YT)) == 0 && aligned16(y) && aligned16(out);
   if (vec)
-    hipLaunchKernelGGL((combine_kernel<YT, true>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, off, list, out, N);
+    hipLaunchKernelGGL((combine_kernel<YT, true>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, off, list, out, N, 0);
   else
-    hipLaunchKernelGGL((combine_kernel<YT, false>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, off, list, out, N);
+    hipLaunchKernelGGL((combine_kernel<YT, false>), dim3(T), dim3(256), 0, s, static_cast<const YT*>(y), w, off, list, out, N, 0);
   return launch_status();
 }
 
@@ -780,7 +807,7 @@ inline size_t round256(size_t b) { return (b + 255) & ~(size_t)255; }
 // Device scratch of the whole layer: router scores (bf16) and logits (f32), the hidden
 // activation h [T k, F] and the expert output y [T k, N] (both bf16).
 struct LayerScratch {
-  size_t scores, logits, hidden, y, total;
+  size_t scores, logits, hidden, y, positions, total;
 };
 LayerScratch layer_scratch(int T, int F, int N, int E, int k) {
   LayerScratch w{};
@@ -789,7 +816,8 @@ LayerScratch layer_scratch(int T, int F, int N, int E, int k) {
   w.logits = w.scores + round256((size_t)T * E * 2);
   w.hidden = w.logits + round256((size_t)T * E * 4);
   w.y = w.hidden + round256(S * F * 2);
-  w.total = w.y + round256(S * N * 2);
+  w.positions = w.y + round256(S * N * 2);      // token-major packed positions, for the combine
+  w.total = w.positions + round256(S * 4);
   return w;
 }
 
@@ -834,13 +862,18 @@ int moe_layer_dev(const void* x, const void* w_router, const float* router_logit
                        reinterpret_cast<const uint16_t*>(ws + w.scores), reinterpret_cast<float*>(ws + w.logits), n);
     logits = reinterpret_cast<const float*>(ws + w.logits);
   }
+  // (the placement pass also leaves each token's packed positions, so the combine need not
+  // rebuild per-token slot lists from token_of_slot)
+  PlanOutputs plan;
+  plan.inverse_perm = reinterpret_cast<int32_t*>(ws + w.positions);
   int rc = route_dev(logits, T, E, k, normalize, capacity, token_of_slot, expert_of_slot, combine_weights,
-                     group_sizes, group_offsets, num_slots, s);
+                     group_sizes, group_offsets, num_slots, s, plan);
   if (rc != kOk) return rc;
   const int S = T * k;
   rc = swiglu_dev(x, wg, wu, wd, group_offsets, ws + w.y, ws + w.hidden, S, H, F, N, E, s, token_of_slot, T);
   if (rc != kOk) return rc;
-  return combine_dev<uint16_t>(ws + w.y, token_of_slot, combine_weights, out, T, S, N, s, num_slots);
+  return combine_dev<uint16_t>(ws + w.y, token_of_slot, combine_weights, out, T, S, N, s, num_slots,
+                               plan.inverse_perm, k);
 }
 
 // Host-pointer form of the layer: upload, run moe_layer_dev, download.
