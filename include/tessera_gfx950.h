@@ -644,7 +644,8 @@ int tessera_gfx950_moe_layer_router_bf16(const void* x, const void* w_router, co
  * execution the device-operand lease of python/tessera/runtime.py:1549-1614 exists for.
  * All pointers are device memory.  workspace: at least
  * tessera_gfx950_moe_layer_workspace_bytes(...) bytes, 16-byte aligned (router scores and
- * logits, the hidden activation [T k, F] and the expert output [T k, N]).  The six
+ * logits, the hidden activation [T k, F], the expert output [T k, N] and each token's packed
+ * slot positions [T k]).  The six
  * metadata outputs are required (later stages read them): token_of_slot /
  * expert_of_slot / combine_weights hold T*k entries of which the first *num_slots are
  * valid.  T * H * 2 must stay inside the 2 GiB buffer range (see the gather block above). */
