@@ -90,6 +90,23 @@ def test_int8_every_kernel_against_one_big_weight(lane, M):
     assert np.array_equal(acc.astype(np.int64).sum(0), xq.astype(np.int64).sum(0) @ wq.astype(np.int64))
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 12288, 12288), (256, 8192, 8192), (48, 18432, 6144), (512, 8192, 8192)])
+def test_int8_schedules_the_fitted_estimate_picks(lane, M, N, K):
+    """16 to 1024 rows under a wide weight matrix: where the fitted estimate promises a clear gain the
+    launcher leaves its rule (128-row tiles with 2 to 4 K parts, also in place of the streaming kernel).
+    Sampled rows exact, column sums of the whole result in exact integer arithmetic."""
+    from tessera_amd.schedule import select_gfx950_gemm_schedule as sel
+    sch = sel(M, N, K, dtype="int8")
+    assert sch.workgroup_tile == (128, 256, 128) and sch.split_k in (2, 3, 4)
+    rng = np.random.default_rng(M + N)
+    xq = rng.integers(-127, 128, (M, K)).astype(np.int8)
+    wq = rng.integers(-127, 128, (K, N)).astype(np.int8)
+    acc = ops.gemm_i8(xq, wq)
+    rows = rng.choice(M, 8, replace=False)
+    assert np.array_equal(acc[rows], orc.gemm_i8_i32(xq[rows], wq))
+    assert np.array_equal(acc.astype(np.int64).sum(0), xq.astype(np.int64).sum(0) @ wq.astype(np.int64))
+
+
 def test_w8a8_headline_shape_properties(lane):
     """M=4096, N=K=8192: accumulators checked exactly on sampled rows/columns."""
     M, N, K = 4096, 8192, 8192
