@@ -34,7 +34,7 @@ inline double est_tiles8_us(int bm, long tiles, int ksteps) {
 // weights cycled through copies) under 16 to 1024 rows: a launch cost, then the larger of the busiest
 // compute unit's K steps (its first workgroup at `step`, every further one sharing the unit at
 // `shared` per step) and the time to stream the tile columns of B at `tbs` TB/s, which takes about
-// 155 workgroups in flight to reach and is stretched by a last, partly filled round; the sum over
+// 155 workgroups in flight to reach (256 for the streaming kernel) and is stretched by a last, partly filled round; the sum over
 // K parts (always there behind the streaming kernel) adds 2 us and 1.4 us per million partials.
 struct Gemm8Fit { double launch, step, shared, tbs; };
 constexpr Gemm8Fit kGemm8Fit[3] = {{5.23, 0.731, 1.265, 5.44},     // the streaming kernel (a step = one 64-row slice of a wave)
@@ -50,7 +50,12 @@ inline double est_gemm8_fit_us(int kind, int M, int N, int K, int splits) {
   const double busiest = (double)((wgs + 255) / 256);
   const double compute = steps * (f.step + f.shared * (busiest - 1.0));
   const double bytes = (double)K * cols * (kind == 0 ? 128 : 256);
-  const double stream = bytes / (f.tbs * 1e6 * std::min(1.0, wgs / 155.0)) * (wgs > 256 ? busiest * 256.0 / wgs : 1.0);
+  // (the fit put the rate's saturation at 155 workgroups for all three; the streaming kernel, one
+  // workgroup per compute unit, is set to 256: the fit's largest misses were its runs at 144 workgroups,
+  // measured a third slower than estimated, and over the fit's shapes the choices at 16 and 32 rows come
+  // out 5 % faster with it)
+  const double sat = kind == 0 ? 256.0 : 155.0;
+  const double stream = bytes / (f.tbs * 1e6 * std::min(1.0, wgs / sat)) * (wgs > 256 ? busiest * 256.0 / wgs : 1.0);
   const double sum = (splits > 1 || kind == 0) ? 2.06 + (double)M * N * splits * 1.43e-6 : 0.0;
   return f.launch + std::max(compute, stream) + sum;
 }
