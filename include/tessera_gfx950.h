@@ -49,8 +49,10 @@
  * recorded kernels hold the workspace's address.  Replay such a graph on the stream it was
  * captured on (launched elsewhere it shares that stream's workspace with eager calls on it
  * and races with them), and do not release the stream's workspace while the graph is in
- * use.  tessera_gfx950_moe_layer_bf16_dev takes a caller-owned workspace instead and has
- * neither restriction.  Any entry point (tessera_gfx950_probe is the cheapest) must have
+ * use.  tessera_gfx950_moe_layer_bf16_dev takes a caller-owned workspace instead: given the
+ * router logits it uses no memory of the library's and has neither restriction (given a router
+ * weight, the router product is a GEMM like any other and may split K through the stream's
+ * workspace).  Any entry point (tessera_gfx950_probe is the cheapest) must have
  * been called once before the first capture: the first call initialises the device.
  */
 #ifndef TESSERA_GFX950_H

@@ -322,7 +322,7 @@ int route_launch(const float* scores, int T, int E, int k, int normalize, int ca
 
 int route_dev(const float* scores, int T, int E, int k, int normalize, int capacity, int32_t* token_of_slot,
               int32_t* expert_of_slot, float* combine_weights, int32_t* group_sizes, int32_t* group_offsets,
-              int32_t* num_slots, hipStream_t s, const PlanOutputs& plan = PlanOutputs{}) {
+              int32_t* num_slots, hipStream_t s) {
   if (bad_route(scores, T, E, k, token_of_slot, expert_of_slot, combine_weights, group_sizes, group_offsets))
     return kBadShape;
   if (probe_device() != kOk) return kNoDevice;
@@ -332,7 +332,7 @@ int route_dev(const float* scores, int T, int E, int k, int normalize, int capac
   char* ws = static_cast<char*>(stream_workspace(s, route_workspace_bytes(T * k, E)));
   if (!ws) return kDeviceFailed;
   return route_launch(scores, T, E, k, normalize, capacity, kRouterSoftmaxAll, token_of_slot, expert_of_slot,
-                      combine_weights, group_sizes, group_offsets, num_slots, ws, s, plan);
+                      combine_weights, group_sizes, group_offsets, num_slots, ws, s);
 }
 
 // route_top_k (or a given selection) + the packing plan with its token-major outputs.
@@ -807,7 +807,7 @@ inline size_t round256(size_t b) { return (b + 255) & ~(size_t)255; }
 // Device scratch of the whole layer: router scores (bf16) and logits (f32), the hidden
 // activation h [T k, F] and the expert output y [T k, N] (both bf16).
 struct LayerScratch {
-  size_t scores, logits, hidden, y, positions, total;
+  size_t scores, logits, hidden, y, positions, route, total;
 };
 LayerScratch layer_scratch(int T, int F, int N, int E, int k) {
   LayerScratch w{};
@@ -817,7 +817,8 @@ LayerScratch layer_scratch(int T, int F, int N, int E, int k) {
   w.hidden = w.logits + round256((size_t)T * E * 4);
   w.y = w.hidden + round256(S * F * 2);
   w.positions = w.y + round256(S * N * 2);      // token-major packed positions, for the combine
-  w.total = w.positions + round256(S * 4);
+  w.route = w.positions + round256(S * 4);      // the routing kernels' temporaries
+  w.total = w.route + round256(route_workspace_bytes((int)S, E));
   return w;
 }
 
@@ -866,8 +867,12 @@ int moe_layer_dev(const void* x, const void* w_router, const float* router_logit
   // rebuild per-token slot lists from token_of_slot)
   PlanOutputs plan;
   plan.inverse_perm = reinterpret_cast<int32_t*>(ws + w.positions);
-  int rc = route_dev(logits, T, E, k, normalize, capacity, token_of_slot, expert_of_slot, combine_weights,
-                     group_sizes, group_offsets, num_slots, s, plan);
+  // (the routing temporaries, too, come from the caller's workspace: with the logits given the
+  // layer touches no memory of the library's)
+  if (bad_route(logits, T, E, k, token_of_slot, expert_of_slot, combine_weights, group_sizes, group_offsets))
+    return kBadShape;
+  int rc = route_launch(logits, T, E, k, normalize, capacity, kRouterSoftmaxAll, token_of_slot, expert_of_slot,
+                        combine_weights, group_sizes, group_offsets, num_slots, ws + w.route, s, plan);
   if (rc != kOk) return rc;
   const int S = T * k;
   rc = swiglu_dev(x, wg, wu, wd, group_offsets, ws + w.y, ws + w.hidden, S, H, F, N, E, s, token_of_slot, T);

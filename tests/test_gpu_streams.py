@@ -314,3 +314,65 @@ def test_dev_entry_points_under_stream_capture(lane, hip):
             L.hipGraphDestroy(graph)
         hip.sync(s)
         hip.destroy(s)
+
+
+def test_layer_with_logits_given_captures_on_a_fresh_stream(lane, hip):
+    """The whole-layer entry with the router logits given takes every temporary from the caller's
+    workspace: it records into a capture on a stream that has run nothing eagerly (no workspace of the
+    library's to size), and the replays equal the eager result of another stream bit for bit."""
+    L = hip.lib
+    L.hipStreamBeginCapture.argtypes = [ctypes.c_void_p, ctypes.c_int]
+    L.hipStreamEndCapture.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]
+    L.hipGraphInstantiate.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_void_p,
+                                      ctypes.c_void_p, ctypes.c_size_t]
+    L.hipGraphLaunch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    L.hipGraphExecDestroy.argtypes = [ctypes.c_void_p]
+    L.hipGraphDestroy.argtypes = [ctypes.c_void_p]
+    lib = lane.load()
+    assert lib.tessera_gfx950_probe() == 0                     # the device is initialised before any capture
+    rng = np.random.default_rng(71)
+    T, H, F, E, k = 260, 128, 192, 8, 2
+    bits = lambda a: np.asarray(b16.from_float32(a.astype(np.float32)), np.uint16)
+    x = lane.DeviceBuffer.from_host(bits(rng.standard_normal((T, H))))
+    lg = lane.DeviceBuffer.from_host(rng.standard_normal((T, E)).astype(np.float32))
+    wg, wu = (lane.DeviceBuffer.from_host(bits(rng.standard_normal((E, H, F)) / 12)) for _ in range(2))
+    wd = lane.DeviceBuffer.from_host(bits(rng.standard_normal((E, F, H)) / 14))
+    need = ctypes.c_size_t(0)
+    lane.check(lib.tessera_gfx950_moe_layer_workspace_bytes(T, H, F, H, E, k, ctypes.byref(need)), "workspace")
+    ws, out = lane.DeviceBuffer(need.value), lane.DeviceBuffer(T * H * 4)
+    S = T * k
+    plan = [lane.DeviceBuffer(S * 4), lane.DeviceBuffer(S * 4), lane.DeviceBuffer(S * 4), lane.DeviceBuffer(E * 4),
+            lane.DeviceBuffer((E + 1) * 4), lane.DeviceBuffer(4)]
+
+    def enqueue(s):
+        lane.check(lib.tessera_gfx950_moe_layer_bf16_dev(
+            x.ptr, None, lg.ptr, wg.ptr, wu.ptr, wd.ptr, out.ptr, ws.ptr, need.value, T, H, F, H, E, k, 1, 0,
+            *(b.ptr for b in plan), s), "moe_layer")
+
+    eager, fresh = hip.stream(), hip.stream()
+    graph, exe = ctypes.c_void_p(), ctypes.c_void_p()
+    try:
+        enqueue(eager)
+        hip.sync(eager)
+        want = out.download((T, H), np.float32)
+        assert np.isfinite(want).all() and np.abs(want).max() > 0
+        assert L.hipStreamBeginCapture(fresh, 0) == 0
+        enqueue(fresh)
+        assert L.hipStreamEndCapture(fresh, ctypes.byref(graph)) == 0 and graph.value
+        assert L.hipGraphInstantiate(ctypes.byref(exe), graph, None, None, 0) == 0
+        for replay in range(3):
+            for buf in (out, ws, *plan):
+                buf.zero()
+            assert L.hipGraphLaunch(exe, fresh) == 0
+            hip.sync(fresh)
+            assert np.array_equal(out.download((T, H), np.float32), want), replay
+    finally:
+        if exe.value:
+            L.hipGraphExecDestroy(exe)
+        if graph.value:
+            L.hipGraphDestroy(graph)
+        for s in (eager, fresh):
+            hip.sync(s)
+            hip.destroy(s)
+        for b in (x, lg, wg, wu, wd, ws, out, *plan):
+            b.close()
